@@ -1,0 +1,57 @@
+#!/usr/bin/env python3
+"""Regenerate tests/golden/*.json from the reference's own operator tests.
+
+Each reference test file is compiled in place (never copied) against this
+repository's tim::vx headers and host-side front end, with a recording
+Executor and a recording stand-in for the gtest macros (capture/). Running the
+result executes every TEST body: the reference's helpers quantize the inline
+vectors exactly as they would for the vendor simulator, and every
+EXPECT_EQ / ArraysMatch becomes one JSON case holding the graph, the input and
+constant data and the expected output with its tolerance.
+
+Needs /root/reference (present only in the build container); the committed
+JSON files are what the test-suite reads.
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+REPO = os.path.dirname(os.path.dirname(HERE))
+REF = os.environ.get("TVX_REFERENCE", "/root/reference")
+PKG = os.path.join(REPO, "tim-vx_amd")
+
+SOURCES = {
+    "conv2d": "src/tim/vx/ops/conv2d_test.cc",
+    "depthwise_conv": "src/tim/vx/ops/depthwiseConv_test.cc",
+    "fullyconnected": "src/tim/vx/ops/fullyconnected_test.cc",
+    "max_pool": "src/tim/vx/ops/max_pool_test.cc",
+    "avg_pool": "src/tim/vx/ops/avg_pool_test.cc",
+}
+
+
+def main():
+    build = os.path.join(HERE, "capture", "_build")
+    os.makedirs(build, exist_ok=True)
+    common = [
+        "g++", "-std=c++17", "-O1", "-w",
+        "-I", os.path.join(HERE, "capture"),
+        "-I", os.path.join(PKG, "include"),
+        "-I", os.path.join(PKG, "src"),
+        "-I", REF,
+        '-DTVX_REF_TEST_UTILS="%s"' % os.path.join(REF, "src/tim/vx/test_utils.h"),
+    ]
+    host = [os.path.join(PKG, "src", f) for f in ("frontend.cc", "graph_passes.cc")]
+    for name, rel in SOURCES.items():
+        exe = os.path.join(build, "capture_" + name)
+        cmd = common + [os.path.join(REF, rel),
+                        os.path.join(HERE, "capture", "capture_main.cc")] + host + ["-o", exe]
+        print("building", name, flush=True)
+        subprocess.check_call(cmd)
+        out = os.path.join(HERE, name + ".json")
+        subprocess.check_call([exe, out])
+        print("wrote", out, os.path.getsize(out), "bytes", flush=True)
+
+
+if __name__ == "__main__":
+    sys.exit(main())

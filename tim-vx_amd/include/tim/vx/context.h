@@ -1,0 +1,2 @@
+#pragma once
+#include "tim/vx/detail/core_api.h"
