@@ -1,0 +1,196 @@
+/*
+ * tvx_hip.h - C ABI between a TIM-VX graph runtime and the MI355X (gfx950)
+ * kernels of the quantized convolution path.
+ *
+ * In the reference this seam is the OpenVX NN extension that ovxlib calls into
+ * the closed Vivante driver. Each entry point below names the driver call it
+ * stands in for. Like a vx_node, an operator is created once (weights are
+ * re-packed, requantization tables are built, a kernel variant is chosen -
+ * the work the driver does in vxVerifyGraph) and then run any number of times
+ * (vxProcessGraph).
+ *
+ * Conventions: plain C, POD structs, device memory is passed as raw pointers,
+ * `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ * Every function returns TVX_OK (0) or a negative tvx_status; tvx_last_error()
+ * gives a text for the calling thread's last failure. *_run() only enqueues
+ * work; the caller synchronizes. Nothing here allocates per run.
+ *
+ * Tensor layouts (dim 0 fastest, as everywhere in TIM-VX): activations WHCN,
+ * convolution weights WHIcOc, depthwise weights {Kw, Kh, Ic*multiplier, 1},
+ * fully-connected input {K, M}, weight {K, N}, output {N, M}.
+ */
+#ifndef TVX_HIP_H_
+#define TVX_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum tvx_status {
+  TVX_OK = 0,
+  TVX_E_INVALID = -1,     /* bad argument / inconsistent descriptor */
+  TVX_E_UNSUPPORTED = -2, /* valid request this library has no kernel for */
+  TVX_E_DEVICE = -3,      /* HIP runtime failure, no usable GPU */
+  TVX_E_NOMEM = -4
+} tvx_status;
+
+typedef enum tvx_dtype { TVX_U8 = 0, TVX_I8 = 1, TVX_F16 = 2, TVX_F32 = 3 } tvx_dtype;
+
+/* Activation fused into the producing operator's epilogue
+ * (stands in for the driver-side conv+relu fusion done inside vxVerifyGraph). */
+typedef enum tvx_activation { TVX_ACT_NONE = 0, TVX_ACT_RELU = 1, TVX_ACT_RELU6 = 2 } tvx_activation;
+
+/* vx_nn_pooling_type: include/VX/vx_khr_nn.h (VX_NN_POOLING_MAX/AVG/AVG_ANDROID);
+ * numbering follows tim::vx::PoolType (include/tim/vx/types.h:62). */
+typedef enum tvx_pool_type { TVX_POOL_MAX = 0, TVX_POOL_AVG = 1, TVX_POOL_L2 = 2, TVX_POOL_AVG_ANDROID = 3 } tvx_pool_type;
+
+typedef struct tvx_op tvx_op; /* opaque operator (the vx_node analogue) */
+
+/* ---- library / device ---------------------------------------------------- */
+const char* tvx_version(void);
+const char* tvx_last_error(void);
+const char* tvx_status_string(int status);
+/* Number of usable GPUs; 0 when there is none (never an error). */
+int tvx_device_count(void);
+
+/* Device memory and streams for runtimes that do not bring their own
+ * (replaces the driver-owned tensor storage behind vxCreateTensor /
+ * vxCopyTensorPatch: src/tim/vx/tensor.cc:154-228). */
+int tvx_malloc(void** dev_ptr, size_t bytes);
+int tvx_free(void* dev_ptr);
+int tvx_memcpy_h2d(void* dst_dev, const void* src_host, size_t bytes, void* stream);
+int tvx_memcpy_d2h(void* dst_host, const void* src_dev, size_t bytes, void* stream);
+int tvx_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* stream);
+int tvx_stream_create(void** stream);
+int tvx_stream_destroy(void* stream);
+int tvx_stream_synchronize(void* stream);
+
+/* ---- requantization (host side, no GPU needed) ---------------------------- */
+/* real multiplier m (= s_in * s_w / s_out in double) -> mult * 2^-shift with
+ * mult in [2^30, 2^31). The kernels apply it as one round-half-to-even right
+ * shift of the 64-bit product acc * mult. */
+int tvx_quantize_multiplier(double m, int32_t* mult, int32_t* shift);
+/* The same fixed-point requantization the kernels' epilogues use, on the host:
+ * round_half_even(acc * mult / 2^shift). */
+int64_t tvx_requantize(int32_t acc, int32_t mult, int32_t shift);
+
+/* ---- Conv2d (dense, 1x1, depthwise) --------------------------------------- */
+/* Replaces vxConvolutionLayer(graph, inputs, weights, biases,
+ * vx_nn_convolution_params_ext2_t{padding l/r/t/b, dilation, stride,
+ * depth_multiplier, overflow/rounding policy}, outputs)
+ * (prebuilt-sdk/x86_64_linux/include/VX/vx_khr_nn.h:738-824,835-873), as called
+ * from src/tim/vx/internal/src/kernel/vx/convolutional.c:504-582. */
+typedef struct tvx_conv2d_desc {
+  uint32_t in_w, in_h, in_c, batch;
+  uint32_t k_w, k_h;
+  uint32_t out_w, out_h, out_c;
+  uint32_t stride_w, stride_h;
+  uint32_t dilation_w, dilation_h; /* >= 1 */
+  uint32_t pad_left, pad_top;      /* right/bottom follow from out_w/out_h */
+  int32_t multiplier;              /* 0 = dense; > 0 = depthwise, oc = ic*multiplier + j */
+  int32_t in_dtype, w_dtype, out_dtype; /* tvx_dtype */
+  float in_scale;
+  int32_t in_zp;
+  float w_scale;  /* per-tensor weight quantization ...                      */
+  int32_t w_zp;
+  const float* w_scales; /* ... or per-output-channel scales (host, out_c entries, zero point 0) */
+  float out_scale;
+  int32_t out_zp;
+  int32_t activation; /* tvx_activation */
+} tvx_conv2d_desc;
+
+/* weights_host: WHIcOc image of the constant weights, or NULL when the weights
+ * are a run-time tensor (then pass them to tvx_op_run as `in1`).
+ * bias_host: int32 (quantized) or float (floating point) [out_c], or NULL. */
+int tvx_conv2d_create(const tvx_conv2d_desc* desc, const void* weights_host,
+                      const void* bias_host, tvx_op** op);
+
+/* ---- FullyConnected ------------------------------------------------------- */
+/* Replaces vxFullyConnectedLayer (vx_khr_nn.h:875-915) as called from
+ * src/tim/vx/internal/src/ops/vsi_nn_op_fullconnect2.c:118-126:
+ * out[m*N + n] = requant(sum_k (x[m*K+k]-zx)(w[n*K+k]-zw[n]) + bias[n]). */
+typedef struct tvx_fc_desc {
+  uint32_t m, k, n;
+  int32_t in_dtype, w_dtype, out_dtype;
+  float in_scale;
+  int32_t in_zp;
+  float w_scale;
+  int32_t w_zp;
+  const float* w_scales; /* per output feature (host, n entries) or NULL */
+  float out_scale;
+  int32_t out_zp;
+  int32_t activation;
+} tvx_fc_desc;
+
+int tvx_fully_connected_create(const tvx_fc_desc* desc, const void* weights_host,
+                               const void* bias_host, tvx_op** op);
+
+/* ---- Pool2d ---------------------------------------------------------------- */
+/* Replaces vxPoolingLayer2(graph, input, vx_nn_pooling_params_ext_t, output)
+ * (vx_khr_nn.h:1696-1744) as called from
+ * src/tim/vx/internal/src/ops/vsi_nn_op_pool.c:144-150. */
+typedef struct tvx_pool2d_desc {
+  uint32_t in_w, in_h, channels, batch;
+  uint32_t out_w, out_h;
+  uint32_t k_w, k_h, stride_w, stride_h, pad_left, pad_top;
+  int32_t pool_type; /* tvx_pool_type */
+  int32_t dtype;     /* input and output */
+  float in_scale;
+  int32_t in_zp;
+  float out_scale;
+  int32_t out_zp;
+} tvx_pool2d_desc;
+
+int tvx_pool2d_create(const tvx_pool2d_desc* desc, tvx_op** op);
+
+/* ---- element-wise ---------------------------------------------------------- */
+/* Standalone ReLU / ReLU6: replaces vxActivationLayer(RELU / RELU6)
+ * (src/tim/vx/internal/src/ops/vsi_nn_op_relu.c:48-55,
+ *  src/tim/vx/internal/src/kernel/vx/eltwise_unary_vx.c:333-352). */
+typedef struct tvx_eltwise_desc {
+  uint64_t count;
+  int32_t dtype;
+  int32_t activation; /* activation op: which clamp */
+  float a_scale;
+  int32_t a_zp;
+  float b_scale; /* second operand (Add only) */
+  int32_t b_zp;
+  float out_scale;
+  int32_t out_zp;
+} tvx_eltwise_desc;
+
+int tvx_activation_create(const tvx_eltwise_desc* desc, tvx_op** op);
+/* Same-shape Add: replaces vxTensorAddNode
+ * (src/tim/vx/internal/src/kernel/vx/eltwise_vx.c:56-67). */
+int tvx_add_create(const tvx_eltwise_desc* desc, tvx_op** op);
+
+/* Softmax over dim 0 of a {channels, rows} view, fp32 output: replaces
+ * vxSoftmaxLayer2 (src/tim/vx/internal/src/kernel/vx/softmax_vx.c:88). */
+typedef struct tvx_softmax_desc {
+  uint32_t channels;
+  uint64_t rows;
+  float beta;
+  int32_t in_dtype;
+  float in_scale;
+  int32_t in_zp;
+} tvx_softmax_desc;
+
+int tvx_softmax_create(const tvx_softmax_desc* desc, tvx_op** op);
+
+/* ---- running / inspecting operators ---------------------------------------- */
+/* Enqueue one execution (the per-node share of vxProcessGraph).
+ * in0: activation; in1: run-time weights (conv / FC created without constant
+ * weights) or the second Add operand, else NULL; out: result. All device
+ * pointers, sized by the operator's descriptor. */
+int tvx_op_run(tvx_op* op, const void* in0, const void* in1, void* out, void* stream);
+/* Name of the kernel variant chosen at creation, e.g. "conv2d_generic". */
+const char* tvx_op_kernel_name(const tvx_op* op);
+void tvx_op_destroy(tvx_op* op);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TVX_HIP_H_ */

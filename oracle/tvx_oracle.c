@@ -105,11 +105,8 @@ void tvxo_quantize_multiplier(double m, int32_t* mult, int32_t* shift) {
 /* round_half_even(acc * mult / 2^shift), as a 64-bit integer */
 int64_t tvxo_requant(int32_t acc, int32_t mult, int32_t shift) {
   int64_t p = (int64_t)acc * (int64_t)mult;
-  if (shift <= 0) {
-    int s = -shift;
-    if (s > 31) s = 31;
-    return p * ((int64_t)1 << s); /* |p| < 2^62: callers clamp right after */
-  }
+  /* multiplier >= 2^30: any non-zero accumulator saturates every 8-bit output */
+  if (shift <= 0) return p > 0 ? ((int64_t)1 << 40) : (p < 0 ? -((int64_t)1 << 40) : 0);
   if (shift > 62) return 0;
   int64_t fl = p >> shift; /* arithmetic: floor */
   int64_t rem = p & (((int64_t)1 << shift) - 1);

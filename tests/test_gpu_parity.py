@@ -1,0 +1,172 @@
+"""Seeded random operators: HIP C ABI vs the CPU oracle, bit-exact for integer
+tensors, rel 1e-2 for floating point (the tolerance the path's contract states)."""
+import numpy as np
+import pytest
+
+import tvx_case as TC
+
+pytestmark = pytest.mark.gpu
+
+FLOAT_RTOL = 1e-2
+
+
+def rand_q(rng, shape, dtype):
+    if dtype == 0:
+        return rng.integers(0, 256, shape).astype(np.uint8)
+    return rng.integers(-128, 128, shape).astype(np.int8)
+
+
+def conv_case(rng, *, n, c, h, w, oc, kh, kw, stride, dil, pad, mult, mode):
+    """mode: 'u8' (per-tensor), 'i8pc' (int8 per-channel), 'u8pc' (u8 act, i8 pc weights), 'f32', 'f16'."""
+    icg = 1 if mult > 0 else c
+    if mult > 0:
+        oc = c * mult
+    out_w = (w + pad[0] + pad[1] - ((kw - 1) * dil[0] + 1)) // stride[0] + 1
+    out_h = (h + pad[2] + pad[3] - ((kh - 1) * dil[1] + 1)) // stride[1] + 1
+    kws = dict(in_shape=[w, h, c, n], w_shape=[kw, kh, icg, oc], out_shape=[out_w, out_h, oc, n],
+               stride=stride, dilation=dil, pad_left=pad[0], pad_top=pad[2], multiplier=mult)
+    if mode in ("f32", "f16"):
+        npd = np.float32 if mode == "f32" else np.float16
+        dt = 3 if mode == "f32" else 2
+        x = rng.standard_normal(n * c * h * w).astype(npd)
+        wt = (rng.standard_normal(oc * icg * kh * kw) * 0.2).astype(npd)
+        b = rng.standard_normal(oc).astype(np.float32)
+        kws.update(in_dtype=dt, w_dtype=dt, out_dtype=dt)
+        return x, wt, b, kws
+    in_dt = 0 if mode.startswith("u8") else 1
+    w_dt = 0 if mode == "u8" else 1
+    x = rand_q(rng, n * c * h * w, in_dt)
+    wt = rand_q(rng, oc * icg * kh * kw, w_dt)
+    b = rng.integers(-4096, 4097, oc).astype(np.int32)
+    zx = 128 if in_dt == 0 else int(rng.integers(-10, 10))
+    kmacs = icg * kh * kw
+    s_out = float(np.float32(0.05 * 0.01 * 40 * np.sqrt(kmacs)))
+    if mode == "u8":
+        wq = (0.01, 120, None)
+    else:
+        wq = (1.0, 0, np.exp(rng.uniform(np.log(0.002), np.log(0.05), oc)).astype(np.float32))
+    kws.update(in_dtype=in_dt, w_dtype=w_dt, out_dtype=in_dt, in_q=(0.05, zx), w_q=wq,
+               out_q=(s_out, 3 if in_dt == 0 else -3))
+    return x, wt, b, kws
+
+
+CONV_GRID = [
+    dict(n=2, c=8, h=9, w=11, oc=6, kh=3, kw=3, stride=[1, 1], dil=[1, 1], pad=[1, 1, 1, 1], mult=0),
+    dict(n=1, c=3, h=17, w=15, oc=16, kh=3, kw=3, stride=[2, 2], dil=[1, 1], pad=[0, 1, 0, 1], mult=0),
+    dict(n=3, c=16, h=7, w=7, oc=32, kh=1, kw=1, stride=[1, 1], dil=[1, 1], pad=[0, 0, 0, 0], mult=0),
+    dict(n=2, c=5, h=12, w=10, oc=4, kh=5, kw=3, stride=[1, 2], dil=[2, 1], pad=[2, 2, 3, 3], mult=0),
+    dict(n=2, c=6, h=10, w=10, oc=0, kh=3, kw=3, stride=[1, 1], dil=[1, 1], pad=[1, 1, 1, 1], mult=1),
+    dict(n=1, c=4, h=9, w=13, oc=0, kh=3, kw=3, stride=[2, 2], dil=[1, 1], pad=[1, 1, 1, 1], mult=2),
+]
+
+
+@pytest.mark.parametrize("mode", ["u8", "i8pc", "u8pc", "f32", "f16"])
+@pytest.mark.parametrize("gi", range(len(CONV_GRID)))
+@pytest.mark.parametrize("act", [0, 2])
+def test_conv2d_random(oracle, gi, mode, act):
+    rng = np.random.default_rng(1000 + gi * 10 + act)
+    x, w, b, kws = conv_case(rng, mode=mode, **CONV_GRID[gi])
+    want = oracle.conv2d(x, w, b, act=act, **kws)
+    got = TC.gpu_conv2d(x, w, b, act=act, **kws)
+    if mode in ("f32", "f16"):
+        assert np.allclose(got.astype(np.float32), want.astype(np.float32), rtol=FLOAT_RTOL, atol=2e-2)
+    else:
+        assert np.array_equal(got, want)
+        assert len(np.unique(want)) > 4  # the case exercises more than saturation
+
+
+def test_conv2d_without_bias_and_runtime_weights(oracle):
+    rng = np.random.default_rng(5)
+    x, w, b, kws = conv_case(rng, mode="u8", **CONV_GRID[0])
+    want = oracle.conv2d(x, w, None, **kws)
+    assert np.array_equal(TC.gpu_conv2d(x, w, None, **kws), want)
+    assert np.array_equal(TC.gpu_conv2d(x, w, None, const_weights=False, **kws), want)
+
+
+@pytest.mark.parametrize("mode", ["u8", "i8pc", "u8pc", "f32", "f16"])
+@pytest.mark.parametrize("shape", [(5, 37, 11), (64, 256, 48), (1, 800, 500), (33, 130, 70)])
+def test_fully_connected_random(oracle, mode, shape):
+    m, k, n = shape
+    rng = np.random.default_rng(m * 7 + k)
+    if mode in ("f32", "f16"):
+        npd, dt = (np.float32, 3) if mode == "f32" else (np.float16, 2)
+        x = rng.standard_normal(m * k).astype(npd)
+        w = (rng.standard_normal(n * k) * 0.02).astype(npd)
+        b = rng.standard_normal(n).astype(np.float32)
+        kws = dict(m=m, k=k, n=n, in_dtype=dt, w_dtype=dt, out_dtype=dt)
+        want = oracle.fully_connected(x, w, b, **kws)
+        got = TC.gpu_fully_connected(x, w, b, **kws)
+        assert np.allclose(got.astype(np.float32), want.astype(np.float32), rtol=FLOAT_RTOL, atol=2e-2)
+        return
+    in_dt = 0 if mode.startswith("u8") else 1
+    w_dt = 0 if mode == "u8" else 1
+    x, w = rand_q(rng, m * k, in_dt), rand_q(rng, n * k, w_dt)
+    b = rng.integers(-16384, 16385, n).astype(np.int32)
+    wq = (0.01, 120, None) if mode == "u8" else \
+        (1.0, 0, np.exp(rng.uniform(np.log(0.001), np.log(0.02), n)).astype(np.float32))
+    kws = dict(m=m, k=k, n=n, in_dtype=in_dt, w_dtype=w_dt, out_dtype=in_dt,
+               in_q=(0.02, 128 if in_dt == 0 else 0), w_q=wq,
+               out_q=(float(np.float32(0.02 * 0.01 * 40 * np.sqrt(k))), 5 if in_dt == 0 else 0))
+    for act in (0, 1):
+        want = oracle.fully_connected(x, w, b, act=act, **kws)
+        got = TC.gpu_fully_connected(x, w, b, act=act, **kws)
+        assert np.array_equal(got, want)
+    assert len(np.unique(want)) > 4
+
+
+POOLS = [
+    dict(in_shape=[24, 24, 20, 3], ksize=[2, 2], stride=[2, 2], pad=[0, 0, 0, 0]),
+    dict(in_shape=[7, 7, 64, 2], ksize=[7, 7], stride=[7, 7], pad=[0, 0, 0, 0]),
+    dict(in_shape=[13, 9, 5, 2], ksize=[3, 3], stride=[2, 2], pad=[1, 1, 0, 1]),
+    dict(in_shape=[10, 10, 3, 1], ksize=[3, 2], stride=[1, 3], pad=[1, 0, 1, 1]),
+]
+
+
+@pytest.mark.parametrize("dtype", [0, 1, 2, 3])
+@pytest.mark.parametrize("ptype", [0, 1, 3])
+@pytest.mark.parametrize("pi", range(len(POOLS)))
+def test_pool2d_random(oracle, pi, ptype, dtype):
+    p = POOLS[pi]
+    rng = np.random.default_rng(pi * 100 + ptype * 10 + dtype)
+    w, h, c, n = p["in_shape"]
+    out_w = (w + p["pad"][0] + p["pad"][1] - p["ksize"][0]) // p["stride"][0] + 1
+    out_h = (h + p["pad"][2] + p["pad"][3] - p["ksize"][1]) // p["stride"][1] + 1
+    kws = dict(in_shape=p["in_shape"], out_shape=[out_w, out_h, c, n], ksize=p["ksize"],
+               stride=p["stride"], pad_left=p["pad"][0], pad_top=p["pad"][2], pool_type=ptype, dtype=dtype)
+    if dtype < 2:
+        x = rand_q(rng, w * h * c * n, dtype)
+        for in_q, out_q in (((0.1, 7), (0.1, 7)), ((0.1, 7), (0.07, -2 if dtype else 9))):
+            want = oracle.pool2d(x, in_q=in_q, out_q=out_q, **kws)
+            got = TC.gpu_pool2d(x, in_q=in_q, out_q=out_q, **kws)
+            assert np.array_equal(got, want)
+    else:
+        x = rng.standard_normal(w * h * c * n).astype(np.float32 if dtype == 3 else np.float16)
+        want = oracle.pool2d(x, **kws)
+        got = TC.gpu_pool2d(x, **kws)
+        assert np.allclose(got.astype(np.float32), want.astype(np.float32), rtol=FLOAT_RTOL, atol=1e-3)
+
+
+@pytest.mark.parametrize("dtype", [0, 1])
+def test_eltwise_quantized(oracle, dtype):
+    rng = np.random.default_rng(dtype)
+    a, b = rand_q(rng, 100003, dtype), rand_q(rng, 100003, dtype)
+    za, zb, zo = (120, 110, 128) if dtype == 0 else (3, -4, 5)
+    for act in (1, 2):
+        for out_q in ((0.05, za), (0.031, zo)):
+            want = oracle.activation(act, dtype, a, (0.05, za), out_q)
+            assert np.array_equal(TC.gpu_activation(act, dtype, a, (0.05, za), out_q), want)
+    want = oracle.add(dtype, a, (0.03, za), b, (0.05, zb), (0.07, zo))
+    assert np.array_equal(TC.gpu_add(dtype, a, (0.03, za), b, (0.05, zb), (0.07, zo)), want)
+    sm_want = oracle.softmax(dtype, a[:100000], 10, 1.0, (0.1, za))
+    sm_got = TC.gpu_softmax(dtype, a[:100000], 10, 1.0, (0.1, za))
+    assert np.allclose(sm_got, sm_want, rtol=1e-4, atol=1e-7)
+
+
+def test_eltwise_float(oracle):
+    rng = np.random.default_rng(3)
+    a = (rng.standard_normal(5000) * 4).astype(np.float32)
+    b = rng.standard_normal(5000).astype(np.float32)
+    assert np.array_equal(TC.gpu_activation(2, 3, a, (1.0, 0), (1.0, 0)), np.clip(a, 0, 6))
+    assert np.array_equal(TC.gpu_add(3, a, (1.0, 0), b, (1.0, 0), (1.0, 0)), a + b)
+    h = a.astype(np.float16)
+    assert np.array_equal(TC.gpu_activation(1, 2, h, (1.0, 0), (1.0, 0)), np.maximum(h, 0))

@@ -1,0 +1,198 @@
+"""Independent checks that pin what the golden vectors leave open: the fixed-point
+requantization against exact rational arithmetic, ties, and the conv / FC / pool
+restatement against brute-force numpy on random tensors."""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+
+def rne_fraction(fr):
+    fl = fr.numerator // fr.denominator
+    rem = fr - fl
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1):
+        fl += 1
+    return fl
+
+
+def test_quantize_multiplier_is_within_2_pow_minus_31(oracle):
+    rng = np.random.default_rng(1)
+    for m in list(10.0 ** rng.uniform(-9, 2, 300)) + [0.25, 0.5, 1.0, 2.0, 3.0, 4.0, 1.0058823529]:
+        mult, shift = oracle.quantize_multiplier(float(m))
+        assert 2 ** 30 <= mult < 2 ** 31
+        approx = Fraction(mult, 2 ** shift) if shift >= 0 else Fraction(mult * 2 ** (-shift))
+        assert abs(approx / Fraction(float(m)) - 1) <= Fraction(1, 2 ** 31)
+
+
+def test_requant_is_exact_rne_of_the_fixed_point_product(oracle):
+    rng = np.random.default_rng(2)
+    for _ in range(2000):
+        acc = int(rng.integers(-2 ** 31, 2 ** 31))
+        mult = int(rng.integers(2 ** 30, 2 ** 31))
+        shift = int(rng.integers(1, 63))
+        assert oracle.requant(acc, mult, shift) == rne_fraction(Fraction(acc * mult, 2 ** shift))
+
+
+def test_requant_ties_go_to_even(oracle):
+    # M = 0.5 exactly: odd accumulators land on .5
+    mult, shift = oracle.quantize_multiplier(0.5)
+    got = [oracle.requant(a, mult, shift) for a in (-5, -3, -1, 1, 3, 5, 7)]
+    assert got == [-2, -2, 0, 0, 2, 2, 4]
+    # powers of two are exact
+    for m in (0.25, 1.0, 2.0, 4.0):
+        mult, shift = oracle.quantize_multiplier(m)
+        for a in (-1000, -7, 0, 4, 12345):
+            assert oracle.requant(a, mult, shift) == rne_fraction(Fraction(a) * Fraction(m))
+
+
+def brute_conv(x, w, bias, stride, dil, pad_l, pad_t, out_w, out_h, multiplier):
+    """x [N,C,H,W], w [Oc,Icg,Kh,Kw] integer arrays -> int64 accumulators [N,Oc,Ho,Wo]."""
+    n, c, h, wd = x.shape
+    oc, icg, kh, kw = w.shape
+    acc = np.zeros((n, oc, out_h, out_w), dtype=np.int64)
+    for o in range(oc):
+        for ci in range(icg):
+            ic = (o // multiplier) if multiplier > 0 else ci
+            for ky in range(kh):
+                for kx in range(kw):
+                    for oh in range(out_h):
+                        ih = oh * stride[1] - pad_t + ky * dil[1]
+                        if ih < 0 or ih >= h:
+                            continue
+                        for ow in range(out_w):
+                            iw = ow * stride[0] - pad_l + kx * dil[0]
+                            if iw < 0 or iw >= wd:
+                                continue
+                            acc[:, o, oh, ow] += x[:, ic, ih, iw] * w[o, ci, ky, kx]
+    if bias is not None:
+        acc += bias[None, :, None, None]
+    return acc
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_conv_restatement_vs_bruteforce(oracle, seed):
+    rng = np.random.default_rng(100 + seed)
+    u8 = seed % 2 == 0
+    depthwise = seed % 3 == 2
+    n, c, h, wd = 2, 4, int(rng.integers(5, 9)), int(rng.integers(5, 9))
+    kh, kw = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+    stride = [int(rng.integers(1, 3)), int(rng.integers(1, 3))]
+    dil = [int(rng.integers(1, 3)), int(rng.integers(1, 3))]
+    pad_l, pad_t = int(rng.integers(0, 3)), int(rng.integers(0, 3))
+    mult = 2 if depthwise else 0
+    oc = c * mult if depthwise else 5
+    icg = 1 if depthwise else c
+    out_w = (wd + 2 * pad_l - ((kw - 1) * dil[0] + 1)) // stride[0] + 1
+    out_h = (h + 2 * pad_t - ((kh - 1) * dil[1] + 1)) // stride[1] + 1
+    if u8:
+        x = rng.integers(0, 256, (n, c, h, wd)).astype(np.uint8)
+        w = rng.integers(0, 256, (oc, icg, kh, kw)).astype(np.uint8)
+        zx, zw, zo = 128, 120, 3
+        w_scales = None
+        in_dt = w_dt = oracle.U8
+    else:
+        x = rng.integers(-128, 128, (n, c, h, wd)).astype(np.int8)
+        w = rng.integers(-128, 128, (oc, icg, kh, kw)).astype(np.int8)
+        zx, zw, zo = -5, 0, -7
+        w_scales = np.exp(rng.uniform(np.log(0.002), np.log(0.05), oc)).astype(np.float32)
+        in_dt = w_dt = oracle.I8
+    bias = rng.integers(-4096, 4097, oc).astype(np.int32)
+    s_in, s_w, s_out = np.float32(0.05), np.float32(0.01), np.float32(0.11)
+    acc = brute_conv(x.astype(np.int64) - zx, w.astype(np.int64) - zw, bias.astype(np.int64),
+                     stride, dil, pad_l, pad_t, out_w, out_h, mult)
+    qmin, qmax = (0, 255) if u8 else (-128, 127)
+    want = np.zeros_like(acc)
+    for o in range(oc):
+        sw = float(w_scales[o]) if w_scales is not None else float(s_w)
+        m, sh = oracle.quantize_multiplier(float(s_in) * sw / float(s_out))
+        flat = [min(qmax, max(qmin, rne_fraction(Fraction(int(a) * m, 2 ** sh)) + zo))
+                for a in acc[:, o].ravel()]
+        want[:, o] = np.asarray(flat).reshape(acc[:, o].shape)
+    got = oracle.conv2d(x.ravel(), w.ravel(), bias, in_shape=[wd, h, c, n], w_shape=[kw, kh, icg, oc],
+                        out_shape=[out_w, out_h, oc, n], stride=stride, dilation=dil, pad_left=pad_l,
+                        pad_top=pad_t, multiplier=mult, in_dtype=in_dt, w_dtype=w_dt, out_dtype=in_dt,
+                        in_q=(float(s_in), zx), w_q=(float(s_w), zw, w_scales), out_q=(float(s_out), zo))
+    assert np.array_equal(got.astype(np.int64), want.ravel())
+
+
+def test_conv_matches_torch_conv2d_on_dequantized_integers(oracle):
+    # textbook reduction: the int32 accumulator equals F.conv2d on (x - zx), (w - zw)
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(7)
+    n, c, h, wd, oc, k = 2, 8, 9, 10, 6, 3
+    x = rng.integers(0, 256, (n, c, h, wd)).astype(np.uint8)
+    w = rng.integers(0, 256, (oc, c, k, k)).astype(np.uint8)
+    bias = rng.integers(-500, 500, oc).astype(np.int32)
+    zx, zw = 128, 120
+    acc = F.conv2d(torch.from_numpy(x.astype(np.float64) - zx), torch.from_numpy(w.astype(np.float64) - zw),
+                   torch.from_numpy(bias.astype(np.float64)), stride=1, padding=1).numpy()
+    # scale chosen so requant is the identity: out = acc (then clamp)
+    got = oracle.conv2d(x.ravel(), w.ravel(), bias, in_shape=[wd, h, c, n], w_shape=[k, k, c, oc],
+                        out_shape=[wd, h, oc, n], stride=[1, 1], dilation=[1, 1], pad_left=1, pad_top=1,
+                        multiplier=0, in_dtype=oracle.U8, w_dtype=oracle.U8, out_dtype=oracle.U8,
+                        in_q=(1.0, zx), w_q=(2.0 ** -12, zw, None), out_q=(1.0, 100))
+    want = np.clip(np.array([rne_fraction(Fraction(int(a), 4096)) for a in acc.ravel()]) + 100, 0, 255)
+    assert np.array_equal(got.astype(np.int64), want)
+
+
+def test_fc_restatement_vs_numpy(oracle):
+    rng = np.random.default_rng(11)
+    m, k, n = 7, 33, 9
+    x = rng.integers(-128, 128, (m, k)).astype(np.int8)
+    w = rng.integers(-128, 128, (n, k)).astype(np.int8)
+    bias = rng.integers(-16384, 16385, n).astype(np.int32)
+    ws = np.exp(rng.uniform(np.log(0.001), np.log(0.02), n)).astype(np.float32)
+    s_in, s_out, zx, zo = np.float32(0.02), np.float32(0.05), 3, -4
+    acc = (x.astype(np.int64) - zx) @ w.astype(np.int64).T + bias
+    want = np.zeros((m, n), dtype=np.int64)
+    for j in range(n):
+        mu, sh = oracle.quantize_multiplier(float(s_in) * float(ws[j]) / float(s_out))
+        want[:, j] = [min(127, max(-128, rne_fraction(Fraction(int(a) * mu, 2 ** sh)) + zo)) for a in acc[:, j]]
+    got = oracle.fully_connected(x.ravel(), w.ravel(), bias, m=m, k=k, n=n, in_dtype=oracle.I8,
+                                 w_dtype=oracle.I8, out_dtype=oracle.I8, in_q=(float(s_in), zx),
+                                 w_q=(1.0, 0, ws), out_q=(float(s_out), zo))
+    assert np.array_equal(got.astype(np.int64), want.ravel())
+
+
+def test_fused_relu6_equals_conv_then_relu6_when_quant_is_shared(oracle):
+    rng = np.random.default_rng(13)
+    n, c, h, wd, oc = 1, 8, 6, 6, 4
+    x = rng.integers(0, 256, (n, c, h, wd)).astype(np.uint8)
+    w = rng.integers(0, 256, (oc, c, 3, 3)).astype(np.uint8)
+    bias = rng.integers(-4096, 4097, oc).astype(np.int32)
+    kw = dict(in_shape=[wd, h, c, n], w_shape=[3, 3, c, oc], out_shape=[wd, h, oc, n], stride=[1, 1],
+              dilation=[1, 1], pad_left=1, pad_top=1, multiplier=0, in_dtype=oracle.U8,
+              w_dtype=oracle.U8, out_dtype=oracle.U8, in_q=(0.05, 128), w_q=(0.01, 120, None),
+              out_q=(0.1, 0))
+    fused = oracle.conv2d(x.ravel(), w.ravel(), bias, act=oracle.ACT_RELU6, **kw)
+    plain = oracle.conv2d(x.ravel(), w.ravel(), bias, **kw)
+    two_step = oracle.activation(oracle.ACT_RELU6, oracle.U8, plain, (0.1, 0), (0.1, 0))
+    assert np.array_equal(fused, two_step)
+    assert fused.max() <= 60
+
+
+def test_pool_avg_divisors(oracle):
+    # AVG divides by the window area, AVG_ANDROID by the in-bounds count
+    x = np.arange(1, 10, dtype=np.float32)
+    kw = dict(in_shape=[3, 3, 1, 1], out_shape=[2, 2, 1, 1], ksize=[2, 2], stride=[2, 2],
+              pad_left=0, pad_top=0, dtype=oracle.F32)
+    avg = oracle.pool2d(x, pool_type=oracle.POOL["AVG"], **kw)
+    android = oracle.pool2d(x, pool_type=oracle.POOL["AVG_ANDROID"], **kw)
+    assert np.allclose(avg, [(1 + 2 + 4 + 5) / 4, (3 + 6) / 4, (7 + 8) / 4, 9 / 4])
+    assert np.allclose(android, [(1 + 2 + 4 + 5) / 4, (3 + 6) / 2, (7 + 8) / 2, 9])
+
+
+def test_quantized_add_and_softmax(oracle):
+    rng = np.random.default_rng(17)
+    a = rng.integers(0, 256, 1000).astype(np.uint8)
+    b = rng.integers(0, 256, 1000).astype(np.uint8)
+    got = oracle.add(oracle.U8, a, (0.03, 120), b, (0.05, 110), (0.07, 128))
+    real = (a.astype(np.float64) - 120) * 0.03 + (b.astype(np.float64) - 110) * 0.05
+    want = np.clip(np.rint(real / 0.07) + 128, 0, 255)
+    assert np.max(np.abs(got.astype(np.float64) - want)) <= 1  # float32 scales vs exact decimals
+    x = rng.integers(0, 256, 40).astype(np.uint8)
+    sm = oracle.softmax(oracle.U8, x, 10, 1.0, (0.1, 128))
+    ref = np.exp((x.reshape(4, 10).astype(np.float64) - 128) * np.float32(0.1))
+    ref /= ref.sum(axis=1, keepdims=True)
+    assert np.allclose(sm.reshape(4, 10), ref, rtol=1e-5, atol=1e-7)

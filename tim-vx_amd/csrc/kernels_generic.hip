@@ -1,0 +1,572 @@
+// Generic kernels: one thread per output element, any shape / stride /
+// dilation / padding / multiplier, every supported dtype. They are the
+// variant of last resort and the on-GPU cross-check for the tuned variants.
+#include "variants.h"
+
+namespace tvx {
+namespace {
+
+template <int DT> struct Elem;
+template <> struct Elem<TVX_U8> { using type = uint8_t; };
+template <> struct Elem<TVX_I8> { using type = int8_t; };
+template <> struct Elem<TVX_F16> { using type = __half; };
+template <> struct Elem<TVX_F32> { using type = float; };
+
+__device__ __forceinline__ float ToFloat(float v) { return v; }
+__device__ __forceinline__ float ToFloat(__half v) { return __half2float(v); }
+__device__ __forceinline__ void FromFloat(float v, float* o) { *o = v; }
+__device__ __forceinline__ void FromFloat(float v, __half* o) { *o = __float2half_rn(v); }
+
+__device__ __forceinline__ float ApplyAct(float v, int act) {
+  if (act == TVX_ACT_RELU || act == TVX_ACT_RELU6) v = v < 0.f ? 0.f : v;
+  if (act == TVX_ACT_RELU6) v = v > 6.f ? 6.f : v;
+  return v;
+}
+
+constexpr int kBlock = 256;
+inline unsigned Blocks(uint64_t n) { return static_cast<unsigned>((n + kBlock - 1) / kBlock); }
+
+// ---------------------------------------------------------------------------
+// Conv2d
+// ---------------------------------------------------------------------------
+struct ConvArgs {
+  int in_w, in_h, in_c, batch, k_w, k_h, out_w, out_h, out_c;
+  int stride_w, stride_h, dil_w, dil_h, pad_left, pad_top, multiplier;
+  int in_zp, w_zp, out_zp, lo, hi, act;
+};
+
+template <typename XT, typename WT>
+__global__ void __launch_bounds__(kBlock)
+ConvQuantKernel(ConvArgs a, const XT* __restrict__ x, const WT* __restrict__ w,
+                const int32_t* __restrict__ bias, const int32_t* __restrict__ mult,
+                const int32_t* __restrict__ shift, XT* __restrict__ y, uint64_t total) {
+  const uint64_t idx = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (idx >= total) return;
+  const int ow = idx % a.out_w;
+  const int oh = (idx / a.out_w) % a.out_h;
+  const int oc = (idx / (static_cast<uint64_t>(a.out_w) * a.out_h)) % a.out_c;
+  const int n = idx / (static_cast<uint64_t>(a.out_w) * a.out_h * a.out_c);
+  const int ic_per_oc = a.multiplier > 0 ? 1 : a.in_c;
+  const int ic0 = a.multiplier > 0 ? oc / a.multiplier : 0;
+  int32_t acc = 0;
+  for (int ci = 0; ci < ic_per_oc; ++ci) {
+    const XT* xp = x + (static_cast<uint64_t>(n) * a.in_c + ic0 + ci) * a.in_h * a.in_w;
+    const WT* wp = w + (static_cast<uint64_t>(oc) * ic_per_oc + ci) * a.k_h * a.k_w;
+    for (int ky = 0; ky < a.k_h; ++ky) {
+      const int ih = oh * a.stride_h - a.pad_top + ky * a.dil_h;
+      if (ih < 0 || ih >= a.in_h) continue;
+      for (int kx = 0; kx < a.k_w; ++kx) {
+        const int iw = ow * a.stride_w - a.pad_left + kx * a.dil_w;
+        if (iw < 0 || iw >= a.in_w) continue;
+        acc += (static_cast<int32_t>(xp[ih * a.in_w + iw]) - a.in_zp) *
+               (static_cast<int32_t>(wp[ky * a.k_w + kx]) - a.w_zp);
+      }
+    }
+  }
+  if (bias) acc += bias[oc];
+  y[idx] = static_cast<XT>(RequantClamp(acc, mult[oc], shift[oc], a.out_zp, a.lo, a.hi));
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock)
+ConvFloatKernel(ConvArgs a, const T* __restrict__ x, const T* __restrict__ w,
+                const float* __restrict__ bias, T* __restrict__ y, uint64_t total) {
+  const uint64_t idx = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (idx >= total) return;
+  const int ow = idx % a.out_w;
+  const int oh = (idx / a.out_w) % a.out_h;
+  const int oc = (idx / (static_cast<uint64_t>(a.out_w) * a.out_h)) % a.out_c;
+  const int n = idx / (static_cast<uint64_t>(a.out_w) * a.out_h * a.out_c);
+  const int ic_per_oc = a.multiplier > 0 ? 1 : a.in_c;
+  const int ic0 = a.multiplier > 0 ? oc / a.multiplier : 0;
+  float acc = 0.f;
+  for (int ci = 0; ci < ic_per_oc; ++ci) {
+    const T* xp = x + (static_cast<uint64_t>(n) * a.in_c + ic0 + ci) * a.in_h * a.in_w;
+    const T* wp = w + (static_cast<uint64_t>(oc) * ic_per_oc + ci) * a.k_h * a.k_w;
+    for (int ky = 0; ky < a.k_h; ++ky) {
+      const int ih = oh * a.stride_h - a.pad_top + ky * a.dil_h;
+      if (ih < 0 || ih >= a.in_h) continue;
+      for (int kx = 0; kx < a.k_w; ++kx) {
+        const int iw = ow * a.stride_w - a.pad_left + kx * a.dil_w;
+        if (iw < 0 || iw >= a.in_w) continue;
+        acc += ToFloat(xp[ih * a.in_w + iw]) * ToFloat(wp[ky * a.k_w + kx]);
+      }
+    }
+  }
+  if (bias) acc += bias[oc];
+  FromFloat(ApplyAct(acc, a.act), &y[idx]);
+}
+
+int ConvGenericRun(tvx_op* op, const void* in0, const void* in1, void* out, hipStream_t st) {
+  const tvx_conv2d_desc& d = op->conv;
+  ConvArgs a{static_cast<int>(d.in_w), static_cast<int>(d.in_h), static_cast<int>(d.in_c),
+             static_cast<int>(d.batch), static_cast<int>(d.k_w), static_cast<int>(d.k_h),
+             static_cast<int>(d.out_w), static_cast<int>(d.out_h), static_cast<int>(d.out_c),
+             static_cast<int>(d.stride_w), static_cast<int>(d.stride_h),
+             static_cast<int>(d.dilation_w), static_cast<int>(d.dilation_h),
+             static_cast<int>(d.pad_left), static_cast<int>(d.pad_top), d.multiplier,
+             d.in_zp, op->w_zp, d.out_zp, op->act_lo, op->act_hi, d.activation};
+  const void* w = op->has_const_weights ? op->weights.ptr : in1;
+  const uint64_t total = static_cast<uint64_t>(d.out_w) * d.out_h * d.out_c * d.batch;
+  const dim3 grid(Blocks(total)), block(kBlock);
+  const int32_t* bias_i = op->bias.as<int32_t>();
+  const int32_t *mu = op->mult.as<int32_t>(), *sh = op->shift.as<int32_t>();
+  if (d.in_dtype == TVX_U8 && d.w_dtype == TVX_U8) {
+    hipLaunchKernelGGL((ConvQuantKernel<uint8_t, uint8_t>), grid, block, 0, st, a,
+                       static_cast<const uint8_t*>(in0), static_cast<const uint8_t*>(w), bias_i,
+                       mu, sh, static_cast<uint8_t*>(out), total);
+  } else if (d.in_dtype == TVX_U8 && d.w_dtype == TVX_I8) {
+    hipLaunchKernelGGL((ConvQuantKernel<uint8_t, int8_t>), grid, block, 0, st, a,
+                       static_cast<const uint8_t*>(in0), static_cast<const int8_t*>(w), bias_i, mu,
+                       sh, static_cast<uint8_t*>(out), total);
+  } else if (d.in_dtype == TVX_I8) {
+    hipLaunchKernelGGL((ConvQuantKernel<int8_t, int8_t>), grid, block, 0, st, a,
+                       static_cast<const int8_t*>(in0), static_cast<const int8_t*>(w), bias_i, mu,
+                       sh, static_cast<int8_t*>(out), total);
+  } else if (d.in_dtype == TVX_F32) {
+    hipLaunchKernelGGL((ConvFloatKernel<float>), grid, block, 0, st, a,
+                       static_cast<const float*>(in0), static_cast<const float*>(w),
+                       op->bias.as<float>(), static_cast<float*>(out), total);
+  } else {
+    hipLaunchKernelGGL((ConvFloatKernel<__half>), grid, block, 0, st, a,
+                       static_cast<const __half*>(in0), static_cast<const __half*>(w),
+                       op->bias.as<float>(), static_cast<__half*>(out), total);
+  }
+  TVX_HIP_CHECK(hipGetLastError());
+  return TVX_OK;
+}
+
+// ---------------------------------------------------------------------------
+// FullyConnected
+// ---------------------------------------------------------------------------
+struct FcArgs {
+  int m, k, n, in_zp, w_zp, out_zp, lo, hi, act;
+};
+
+template <typename XT, typename WT>
+__global__ void __launch_bounds__(kBlock)
+FcQuantKernel(FcArgs a, const XT* __restrict__ x, const WT* __restrict__ w,
+              const int32_t* __restrict__ bias, const int32_t* __restrict__ mult,
+              const int32_t* __restrict__ shift, XT* __restrict__ y, uint64_t total) {
+  const uint64_t idx = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (idx >= total) return;
+  const int n = idx % a.n;
+  const uint64_t m = idx / a.n;
+  const XT* xp = x + m * a.k;
+  const WT* wp = w + static_cast<uint64_t>(n) * a.k;
+  int32_t acc = 0;
+  for (int k = 0; k < a.k; ++k)
+    acc += (static_cast<int32_t>(xp[k]) - a.in_zp) * (static_cast<int32_t>(wp[k]) - a.w_zp);
+  if (bias) acc += bias[n];
+  y[idx] = static_cast<XT>(RequantClamp(acc, mult[n], shift[n], a.out_zp, a.lo, a.hi));
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock)
+FcFloatKernel(FcArgs a, const T* __restrict__ x, const T* __restrict__ w,
+              const float* __restrict__ bias, T* __restrict__ y, uint64_t total) {
+  const uint64_t idx = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (idx >= total) return;
+  const int n = idx % a.n;
+  const uint64_t m = idx / a.n;
+  const T* xp = x + m * a.k;
+  const T* wp = w + static_cast<uint64_t>(n) * a.k;
+  float acc = 0.f;
+  for (int k = 0; k < a.k; ++k) acc += ToFloat(xp[k]) * ToFloat(wp[k]);
+  if (bias) acc += bias[n];
+  FromFloat(ApplyAct(acc, a.act), &y[idx]);
+}
+
+int FcGenericRun(tvx_op* op, const void* in0, const void* in1, void* out, hipStream_t st) {
+  const tvx_fc_desc& d = op->fc;
+  FcArgs a{static_cast<int>(d.m), static_cast<int>(d.k), static_cast<int>(d.n), d.in_zp, op->w_zp,
+           d.out_zp, op->act_lo, op->act_hi, d.activation};
+  const void* w = op->has_const_weights ? op->weights.ptr : in1;
+  const uint64_t total = static_cast<uint64_t>(d.m) * d.n;
+  const dim3 grid(Blocks(total)), block(kBlock);
+  const int32_t* bias_i = op->bias.as<int32_t>();
+  const int32_t *mu = op->mult.as<int32_t>(), *sh = op->shift.as<int32_t>();
+  if (d.in_dtype == TVX_U8 && d.w_dtype == TVX_U8) {
+    hipLaunchKernelGGL((FcQuantKernel<uint8_t, uint8_t>), grid, block, 0, st, a,
+                       static_cast<const uint8_t*>(in0), static_cast<const uint8_t*>(w), bias_i,
+                       mu, sh, static_cast<uint8_t*>(out), total);
+  } else if (d.in_dtype == TVX_U8 && d.w_dtype == TVX_I8) {
+    hipLaunchKernelGGL((FcQuantKernel<uint8_t, int8_t>), grid, block, 0, st, a,
+                       static_cast<const uint8_t*>(in0), static_cast<const int8_t*>(w), bias_i, mu,
+                       sh, static_cast<uint8_t*>(out), total);
+  } else if (d.in_dtype == TVX_I8) {
+    hipLaunchKernelGGL((FcQuantKernel<int8_t, int8_t>), grid, block, 0, st, a,
+                       static_cast<const int8_t*>(in0), static_cast<const int8_t*>(w), bias_i, mu,
+                       sh, static_cast<int8_t*>(out), total);
+  } else if (d.in_dtype == TVX_F32) {
+    hipLaunchKernelGGL((FcFloatKernel<float>), grid, block, 0, st, a,
+                       static_cast<const float*>(in0), static_cast<const float*>(w),
+                       op->bias.as<float>(), static_cast<float*>(out), total);
+  } else {
+    hipLaunchKernelGGL((FcFloatKernel<__half>), grid, block, 0, st, a,
+                       static_cast<const __half*>(in0), static_cast<const __half*>(w),
+                       op->bias.as<float>(), static_cast<__half*>(out), total);
+  }
+  TVX_HIP_CHECK(hipGetLastError());
+  return TVX_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Pool2d
+// ---------------------------------------------------------------------------
+struct PoolArgs {
+  int in_w, in_h, out_w, out_h, k_w, k_h, stride_w, stride_h, pad_left, pad_top, type;
+  int in_zp, out_zp, qmin, qmax, mult, shift;
+  double ratio;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock)
+PoolQuantKernel(PoolArgs a, const T* __restrict__ x, T* __restrict__ y, uint64_t total) {
+  const uint64_t idx = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (idx >= total) return;
+  const int ow = idx % a.out_w;
+  const int oh = (idx / a.out_w) % a.out_h;
+  const uint64_t plane = idx / (static_cast<uint64_t>(a.out_w) * a.out_h);
+  const T* xp = x + plane * a.in_w * a.in_h;
+  int cnt = 0, vmax = INT32_MIN;
+  int64_t sum = 0;
+  for (int ky = 0; ky < a.k_h; ++ky) {
+    const int ih = oh * a.stride_h - a.pad_top + ky;
+    if (ih < 0 || ih >= a.in_h) continue;
+    for (int kx = 0; kx < a.k_w; ++kx) {
+      const int iw = ow * a.stride_w - a.pad_left + kx;
+      if (iw < 0 || iw >= a.in_w) continue;
+      const int v = static_cast<int>(xp[ih * a.in_w + iw]) - a.in_zp;
+      ++cnt;
+      sum += v;
+      vmax = v > vmax ? v : vmax;
+    }
+  }
+  int64_t r = 0;
+  if (a.type == TVX_POOL_MAX) {
+    if (cnt) r = RequantRne(vmax, a.mult, a.shift);
+  } else {
+    const int div = a.type == TVX_POOL_AVG ? a.k_w * a.k_h : cnt;
+    if (div) r = static_cast<int64_t>(rint(static_cast<double>(sum) * a.ratio / static_cast<double>(div)));
+  }
+  r += a.out_zp;
+  r = r < a.qmin ? a.qmin : (r > a.qmax ? a.qmax : r);
+  y[idx] = static_cast<T>(r);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock)
+PoolFloatKernel(PoolArgs a, const T* __restrict__ x, T* __restrict__ y, uint64_t total) {
+  const uint64_t idx = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (idx >= total) return;
+  const int ow = idx % a.out_w;
+  const int oh = (idx / a.out_w) % a.out_h;
+  const uint64_t plane = idx / (static_cast<uint64_t>(a.out_w) * a.out_h);
+  const T* xp = x + plane * a.in_w * a.in_h;
+  int cnt = 0;
+  float vmax = -INFINITY, sum = 0.f;
+  for (int ky = 0; ky < a.k_h; ++ky) {
+    const int ih = oh * a.stride_h - a.pad_top + ky;
+    if (ih < 0 || ih >= a.in_h) continue;
+    for (int kx = 0; kx < a.k_w; ++kx) {
+      const int iw = ow * a.stride_w - a.pad_left + kx;
+      if (iw < 0 || iw >= a.in_w) continue;
+      const float v = ToFloat(xp[ih * a.in_w + iw]);
+      ++cnt;
+      sum += v;
+      vmax = v > vmax ? v : vmax;
+    }
+  }
+  float r;
+  if (a.type == TVX_POOL_MAX) {
+    r = cnt ? vmax : 0.f;
+  } else {
+    const int div = a.type == TVX_POOL_AVG ? a.k_w * a.k_h : cnt;
+    r = div ? sum / static_cast<float>(div) : 0.f;
+  }
+  FromFloat(r, &y[idx]);
+}
+
+int PoolGenericRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
+  const tvx_pool2d_desc& d = op->pool;
+  PoolArgs a{static_cast<int>(d.in_w), static_cast<int>(d.in_h), static_cast<int>(d.out_w),
+             static_cast<int>(d.out_h), static_cast<int>(d.k_w), static_cast<int>(d.k_h),
+             static_cast<int>(d.stride_w), static_cast<int>(d.stride_h),
+             static_cast<int>(d.pad_left), static_cast<int>(d.pad_top), d.pool_type,
+             d.in_zp, d.out_zp, d.dtype == TVX_U8 ? 0 : -128, d.dtype == TVX_U8 ? 255 : 127,
+             op->geo[0], op->geo[1],
+             op->quantized ? static_cast<double>(d.in_scale) / static_cast<double>(d.out_scale) : 1.0};
+  const uint64_t total = static_cast<uint64_t>(d.out_w) * d.out_h * d.channels * d.batch;
+  const dim3 grid(Blocks(total)), block(kBlock);
+  switch (d.dtype) {
+    case TVX_U8:
+      hipLaunchKernelGGL((PoolQuantKernel<uint8_t>), grid, block, 0, st, a,
+                         static_cast<const uint8_t*>(in0), static_cast<uint8_t*>(out), total);
+      break;
+    case TVX_I8:
+      hipLaunchKernelGGL((PoolQuantKernel<int8_t>), grid, block, 0, st, a,
+                         static_cast<const int8_t*>(in0), static_cast<int8_t*>(out), total);
+      break;
+    case TVX_F32:
+      hipLaunchKernelGGL((PoolFloatKernel<float>), grid, block, 0, st, a,
+                         static_cast<const float*>(in0), static_cast<float*>(out), total);
+      break;
+    default:
+      hipLaunchKernelGGL((PoolFloatKernel<__half>), grid, block, 0, st, a,
+                         static_cast<const __half*>(in0), static_cast<__half*>(out), total);
+  }
+  TVX_HIP_CHECK(hipGetLastError());
+  return TVX_OK;
+}
+
+// ---------------------------------------------------------------------------
+// element-wise
+// ---------------------------------------------------------------------------
+struct EltArgs {
+  int a_zp, b_zp, out_zp, lo, hi, mult, shift, act;
+  double ra, rb;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock)
+ActQuantKernel(EltArgs a, const T* __restrict__ x, T* __restrict__ y, uint64_t total) {
+  const uint64_t idx = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (idx >= total) return;
+  y[idx] = static_cast<T>(
+      RequantClamp(static_cast<int32_t>(x[idx]) - a.a_zp, a.mult, a.shift, a.out_zp, a.lo, a.hi));
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock)
+ActFloatKernel(EltArgs a, const T* __restrict__ x, T* __restrict__ y, uint64_t total) {
+  const uint64_t idx = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (idx >= total) return;
+  FromFloat(ApplyAct(ToFloat(x[idx]), a.act), &y[idx]);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock)
+AddQuantKernel(EltArgs a, const T* __restrict__ x, const T* __restrict__ z, T* __restrict__ y,
+               uint64_t total) {
+  const uint64_t idx = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (idx >= total) return;
+  // rne(fma(a - za, sa/so, (b - zb) * (sb/so))) in double: one defined order.
+  const double tb = __dmul_rn(static_cast<double>(static_cast<int32_t>(z[idx]) - a.b_zp), a.rb);
+  const double t = fma(static_cast<double>(static_cast<int32_t>(x[idx]) - a.a_zp), a.ra, tb);
+  int64_t r = static_cast<int64_t>(rint(t)) + a.out_zp;
+  r = r < a.lo ? a.lo : (r > a.hi ? a.hi : r);
+  y[idx] = static_cast<T>(r);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock)
+AddFloatKernel(const T* __restrict__ x, const T* __restrict__ z, T* __restrict__ y, uint64_t total) {
+  const uint64_t idx = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (idx >= total) return;
+  FromFloat(ToFloat(x[idx]) + ToFloat(z[idx]), &y[idx]);
+}
+
+EltArgs MakeEltArgs(const tvx_op* op) {
+  const tvx_eltwise_desc& d = op->elt;
+  EltArgs a{};
+  a.a_zp = d.a_zp;
+  a.b_zp = d.b_zp;
+  a.out_zp = d.out_zp;
+  a.lo = op->act_lo;
+  a.hi = op->act_hi;
+  a.mult = op->geo[0];
+  a.shift = op->geo[1];
+  a.act = d.activation;
+  if (op->quantized) {
+    a.ra = static_cast<double>(d.a_scale) / static_cast<double>(d.out_scale);
+    a.rb = static_cast<double>(d.b_scale) / static_cast<double>(d.out_scale);
+  }
+  return a;
+}
+
+int ActivationRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
+  const EltArgs a = MakeEltArgs(op);
+  const uint64_t total = op->elt.count;
+  if (!total) return TVX_OK;
+  const dim3 grid(Blocks(total)), block(kBlock);
+  switch (op->elt.dtype) {
+    case TVX_U8:
+      hipLaunchKernelGGL((ActQuantKernel<uint8_t>), grid, block, 0, st, a,
+                         static_cast<const uint8_t*>(in0), static_cast<uint8_t*>(out), total);
+      break;
+    case TVX_I8:
+      hipLaunchKernelGGL((ActQuantKernel<int8_t>), grid, block, 0, st, a,
+                         static_cast<const int8_t*>(in0), static_cast<int8_t*>(out), total);
+      break;
+    case TVX_F32:
+      hipLaunchKernelGGL((ActFloatKernel<float>), grid, block, 0, st, a,
+                         static_cast<const float*>(in0), static_cast<float*>(out), total);
+      break;
+    default:
+      hipLaunchKernelGGL((ActFloatKernel<__half>), grid, block, 0, st, a,
+                         static_cast<const __half*>(in0), static_cast<__half*>(out), total);
+  }
+  TVX_HIP_CHECK(hipGetLastError());
+  return TVX_OK;
+}
+
+int AddRun(tvx_op* op, const void* in0, const void* in1, void* out, hipStream_t st) {
+  const EltArgs a = MakeEltArgs(op);
+  const uint64_t total = op->elt.count;
+  if (!total) return TVX_OK;
+  const dim3 grid(Blocks(total)), block(kBlock);
+  switch (op->elt.dtype) {
+    case TVX_U8:
+      hipLaunchKernelGGL((AddQuantKernel<uint8_t>), grid, block, 0, st, a,
+                         static_cast<const uint8_t*>(in0), static_cast<const uint8_t*>(in1),
+                         static_cast<uint8_t*>(out), total);
+      break;
+    case TVX_I8:
+      hipLaunchKernelGGL((AddQuantKernel<int8_t>), grid, block, 0, st, a,
+                         static_cast<const int8_t*>(in0), static_cast<const int8_t*>(in1),
+                         static_cast<int8_t*>(out), total);
+      break;
+    case TVX_F32:
+      hipLaunchKernelGGL((AddFloatKernel<float>), grid, block, 0, st,
+                         static_cast<const float*>(in0), static_cast<const float*>(in1),
+                         static_cast<float*>(out), total);
+      break;
+    default:
+      hipLaunchKernelGGL((AddFloatKernel<__half>), grid, block, 0, st,
+                         static_cast<const __half*>(in0), static_cast<const __half*>(in1),
+                         static_cast<__half*>(out), total);
+  }
+  TVX_HIP_CHECK(hipGetLastError());
+  return TVX_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Softmax: one thread per row (rows are short: class counts)
+// ---------------------------------------------------------------------------
+template <typename T, bool QUANT>
+__global__ void __launch_bounds__(kBlock)
+SoftmaxKernel(int c, uint64_t rows, float beta, float scale, int zp, const T* __restrict__ x,
+              float* __restrict__ y) {
+  const uint64_t r = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (r >= rows) return;
+  const T* xp = x + r * c;
+  float* yp = y + r * c;
+  float mx = -INFINITY;
+  for (int i = 0; i < c; ++i) {
+    float v;
+    if constexpr (QUANT) v = scale * static_cast<float>(static_cast<int>(xp[i]) - zp);
+    else v = ToFloat(xp[i]);
+    yp[i] = v;
+    mx = v > mx ? v : mx;
+  }
+  float sum = 0.f;
+  for (int i = 0; i < c; ++i) {
+    const float e = expf(beta * (yp[i] - mx));
+    yp[i] = e;
+    sum += e;
+  }
+  for (int i = 0; i < c; ++i) yp[i] = yp[i] / sum;
+}
+
+int SoftmaxRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
+  const tvx_softmax_desc& d = op->sm;
+  if (!d.rows) return TVX_OK;
+  const dim3 grid(Blocks(d.rows)), block(kBlock);
+  float* y = static_cast<float*>(out);
+  const int c = static_cast<int>(d.channels);
+  switch (d.in_dtype) {
+    case TVX_U8:
+      hipLaunchKernelGGL((SoftmaxKernel<uint8_t, true>), grid, block, 0, st, c, d.rows, d.beta,
+                         d.in_scale, d.in_zp, static_cast<const uint8_t*>(in0), y);
+      break;
+    case TVX_I8:
+      hipLaunchKernelGGL((SoftmaxKernel<int8_t, true>), grid, block, 0, st, c, d.rows, d.beta,
+                         d.in_scale, d.in_zp, static_cast<const int8_t*>(in0), y);
+      break;
+    case TVX_F32:
+      hipLaunchKernelGGL((SoftmaxKernel<float, false>), grid, block, 0, st, c, d.rows, d.beta, 1.f,
+                         0, static_cast<const float*>(in0), y);
+      break;
+    default:
+      hipLaunchKernelGGL((SoftmaxKernel<__half, false>), grid, block, 0, st, c, d.rows, d.beta, 1.f,
+                         0, static_cast<const __half*>(in0), y);
+  }
+  TVX_HIP_CHECK(hipGetLastError());
+  return TVX_OK;
+}
+
+int UploadWeightsAndBias(tvx_op* op, const void* w, size_t w_bytes, const void* b, size_t b_bytes) {
+  int s = TVX_OK;
+  if (w) s = op->weights.Upload(w, w_bytes);
+  if (s == TVX_OK && b) s = op->bias.Upload(b, b_bytes);
+  return s;
+}
+
+}  // namespace
+
+int ConvGenericSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w, const void* b) {
+  const uint64_t ic_per_oc = d->multiplier > 0 ? 1 : d->in_c;
+  const size_t w_bytes = static_cast<size_t>(d->k_w) * d->k_h * ic_per_oc * d->out_c * DtypeBytes(d->w_dtype);
+  int s = UploadWeightsAndBias(op, w, w_bytes, b, static_cast<size_t>(d->out_c) * 4);
+  if (s != TVX_OK) return s;
+  op->run = ConvGenericRun;
+  op->kernel_name = "conv2d_generic";
+  return TVX_OK;
+}
+
+int FcGenericSetup(tvx_op* op, const tvx_fc_desc* d, const void* w, const void* b) {
+  const size_t w_bytes = static_cast<size_t>(d->k) * d->n * DtypeBytes(d->w_dtype);
+  int s = UploadWeightsAndBias(op, w, w_bytes, b, static_cast<size_t>(d->n) * 4);
+  if (s != TVX_OK) return s;
+  op->run = FcGenericRun;
+  op->kernel_name = "fc_generic";
+  return TVX_OK;
+}
+
+static int ScalarRequant(tvx_op* op, float in_scale, float out_scale) {
+  std::vector<int32_t> mult, shift;
+  int s = BuildRequantTables(1, in_scale, 1.0f, nullptr, out_scale, &mult, &shift);
+  if (s != TVX_OK) return s;
+  op->geo[0] = mult[0];
+  op->geo[1] = shift[0];
+  return TVX_OK;
+}
+
+int PoolGenericSetup(tvx_op* op) {
+  if (op->quantized) {
+    int s = ScalarRequant(op, op->pool.in_scale, op->pool.out_scale);
+    if (s != TVX_OK) return s;
+  }
+  op->run = PoolGenericRun;
+  op->kernel_name = "pool2d_generic";
+  return TVX_OK;
+}
+
+int ActivationSetup(tvx_op* op) {
+  if (op->quantized) {
+    int s = ScalarRequant(op, op->elt.a_scale, op->elt.out_scale);
+    if (s != TVX_OK) return s;
+    ActRange(op->elt.dtype, op->elt.out_scale, op->elt.out_zp, op->elt.activation, &op->act_lo,
+             &op->act_hi);
+  }
+  op->run = ActivationRun;
+  op->kernel_name = "activation_generic";
+  return TVX_OK;
+}
+
+int AddSetup(tvx_op* op) {
+  if (op->quantized)
+    ActRange(op->elt.dtype, op->elt.out_scale, op->elt.out_zp, TVX_ACT_NONE, &op->act_lo, &op->act_hi);
+  op->run = AddRun;
+  op->kernel_name = "add_generic";
+  return TVX_OK;
+}
+
+int SoftmaxSetup(tvx_op* op) {
+  op->run = SoftmaxRun;
+  op->kernel_name = "softmax_generic";
+  return TVX_OK;
+}
+
+}  // namespace tvx

@@ -1,0 +1,388 @@
+// C ABI of include/tvx_hip.h: library/device helpers, descriptor validation,
+// requantization tables, and the walk over kernel variants that picks the
+// first one claiming an operator (the counterpart of ovxlib's
+// vsi_nn_kernel_selector priority walk, src/tim/vx/internal/src/kernel/vsi_nn_kernel.c:1178-1299).
+#include <cmath>
+#include <cstring>
+#include <new>
+
+#include "tvx_internal.h"
+#include "variants.h"
+
+namespace tvx {
+
+static thread_local char g_error[512] = "";
+
+int SetError(int status, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return status;
+}
+
+int DeviceBuffer::Alloc(size_t n) {
+  if (ptr) { (void)hipFree(ptr); ptr = nullptr; }
+  bytes = n;
+  if (n == 0) return TVX_OK;
+  TVX_HIP_CHECK(hipMalloc(&ptr, n));
+  return TVX_OK;
+}
+
+int DeviceBuffer::Upload(const void* host, size_t n) {
+  int s = Alloc(n);
+  if (s != TVX_OK) return s;
+  if (n) TVX_HIP_CHECK(hipMemcpy(ptr, host, n, hipMemcpyHostToDevice));
+  return TVX_OK;
+}
+
+static void QuantizeMultiplier(double m, int32_t* mult, int32_t* shift) {
+  if (!(m > 0.0) || !std::isfinite(m)) {
+    *mult = 0;
+    *shift = 1;
+    return;
+  }
+  int e = 0;
+  const double q = std::frexp(m, &e);
+  int64_t qi = std::llround(q * 2147483648.0);
+  if (qi == (int64_t{1} << 31)) {
+    qi >>= 1;
+    ++e;
+  }
+  *mult = static_cast<int32_t>(qi);
+  *shift = 31 - e;
+}
+
+int BuildRequantTables(uint32_t channels, float in_scale, float w_scale,
+                       const float* w_scales, float out_scale,
+                       std::vector<int32_t>* mult, std::vector<int32_t>* shift) {
+  mult->resize(channels);
+  shift->resize(channels);
+  if (!(out_scale > 0.f) || !(in_scale > 0.f))
+    return SetError(TVX_E_INVALID, "scales must be positive (in %g, out %g)", in_scale, out_scale);
+  for (uint32_t c = 0; c < channels; ++c) {
+    const double ws = w_scales ? static_cast<double>(w_scales[c]) : static_cast<double>(w_scale);
+    if (!(ws > 0.0)) return SetError(TVX_E_INVALID, "weight scale of channel %u is %g", c, ws);
+    int32_t m, s;
+    QuantizeMultiplier(static_cast<double>(in_scale) * ws / static_cast<double>(out_scale), &m, &s);
+    if (s < 1)
+      return SetError(TVX_E_UNSUPPORTED, "requantization multiplier of channel %u is >= 2^30", c);
+    if (s > 62) {  // underflows to 0 for every int32 accumulator
+      m = 0;
+      s = 1;
+    }
+    (*mult)[c] = m;
+    (*shift)[c] = s;
+  }
+  return TVX_OK;
+}
+
+void ActRange(int out_dtype, float out_scale, int32_t out_zp, int act, int32_t* lo, int32_t* hi) {
+  *lo = out_dtype == TVX_U8 ? 0 : -128;
+  *hi = out_dtype == TVX_U8 ? 255 : 127;
+  if (act == TVX_ACT_RELU || act == TVX_ACT_RELU6) {
+    if (out_zp > *lo) *lo = out_zp;
+  }
+  if (act == TVX_ACT_RELU6) {
+    const double six = std::nearbyint(6.0 / static_cast<double>(out_scale));
+    if (six < 1e9) {
+      const int64_t top = static_cast<int64_t>(out_zp) + static_cast<int64_t>(six);
+      if (top < *hi) *hi = static_cast<int32_t>(top);
+    }
+  }
+  if (*lo > *hi) *lo = *hi;
+}
+
+static bool ValidDtype(int d) { return d >= TVX_U8 && d <= TVX_F32; }
+
+static int CheckOperandTypes(int in, int w, int out, const char* what) {
+  if (!ValidDtype(in) || !ValidDtype(w) || !ValidDtype(out))
+    return SetError(TVX_E_INVALID, "%s: unknown dtype", what);
+  if (IsQuant(in)) {
+    // u8 x u8, i8 x i8, and either activation with int8 per-channel weights
+    if (!IsQuant(w) || !IsQuant(out) || out != in)
+      return SetError(TVX_E_UNSUPPORTED, "%s: dtype combination in=%d w=%d out=%d", what, in, w, out);
+    if (in == TVX_I8 && w == TVX_U8)
+      return SetError(TVX_E_UNSUPPORTED, "%s: int8 activations with uint8 weights", what);
+  } else if (w != in || out != in) {
+    return SetError(TVX_E_UNSUPPORTED, "%s: dtype combination in=%d w=%d out=%d", what, in, w, out);
+  }
+  return TVX_OK;
+}
+
+}  // namespace tvx
+
+using namespace tvx;
+
+extern "C" {
+
+const char* tvx_version(void) { return "tvx-hip 0.1 (gfx950)"; }
+const char* tvx_last_error(void) { return g_error; }
+
+const char* tvx_status_string(int status) {
+  switch (status) {
+    case TVX_OK: return "ok";
+    case TVX_E_INVALID: return "invalid argument";
+    case TVX_E_UNSUPPORTED: return "unsupported";
+    case TVX_E_DEVICE: return "device error";
+    case TVX_E_NOMEM: return "out of memory";
+  }
+  return "unknown status";
+}
+
+int tvx_device_count(void) {
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return n;
+}
+
+int tvx_malloc(void** dev_ptr, size_t bytes) {
+  if (!dev_ptr) return SetError(TVX_E_INVALID, "tvx_malloc: null result pointer");
+  *dev_ptr = nullptr;
+  if (bytes == 0) return TVX_OK;
+  hipError_t e = hipMalloc(dev_ptr, bytes);
+  if (e == hipErrorOutOfMemory) return SetError(TVX_E_NOMEM, "hipMalloc(%zu) out of memory", bytes);
+  if (e != hipSuccess) return SetError(TVX_E_DEVICE, "hipMalloc(%zu): %s", bytes, hipGetErrorString(e));
+  return TVX_OK;
+}
+
+int tvx_free(void* dev_ptr) {
+  if (dev_ptr) TVX_HIP_CHECK(hipFree(dev_ptr));
+  return TVX_OK;
+}
+
+int tvx_memcpy_h2d(void* dst, const void* src, size_t bytes, void* stream) {
+  if (bytes == 0) return TVX_OK;
+  if (!dst || !src) return SetError(TVX_E_INVALID, "tvx_memcpy_h2d: null pointer");
+  TVX_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, static_cast<hipStream_t>(stream)));
+  return TVX_OK;
+}
+
+int tvx_memcpy_d2h(void* dst, const void* src, size_t bytes, void* stream) {
+  if (bytes == 0) return TVX_OK;
+  if (!dst || !src) return SetError(TVX_E_INVALID, "tvx_memcpy_d2h: null pointer");
+  TVX_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, static_cast<hipStream_t>(stream)));
+  return TVX_OK;
+}
+
+int tvx_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream) {
+  if (bytes == 0) return TVX_OK;
+  if (!dst || !src) return SetError(TVX_E_INVALID, "tvx_memcpy_d2d: null pointer");
+  TVX_HIP_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)));
+  return TVX_OK;
+}
+
+int tvx_stream_create(void** stream) {
+  if (!stream) return SetError(TVX_E_INVALID, "tvx_stream_create: null result pointer");
+  hipStream_t s = nullptr;
+  TVX_HIP_CHECK(hipStreamCreate(&s));  // default priority
+  *stream = s;
+  return TVX_OK;
+}
+
+int tvx_stream_destroy(void* stream) {
+  if (stream) TVX_HIP_CHECK(hipStreamDestroy(static_cast<hipStream_t>(stream)));
+  return TVX_OK;
+}
+
+int tvx_stream_synchronize(void* stream) {
+  TVX_HIP_CHECK(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  return TVX_OK;
+}
+
+int tvx_quantize_multiplier(double m, int32_t* mult, int32_t* shift) {
+  if (!mult || !shift) return SetError(TVX_E_INVALID, "tvx_quantize_multiplier: null pointer");
+  QuantizeMultiplier(m, mult, shift);
+  return TVX_OK;
+}
+
+int64_t tvx_requantize(int32_t acc, int32_t mult, int32_t shift) {
+  const int64_t p = static_cast<int64_t>(acc) * static_cast<int64_t>(mult);
+  if (shift < 1) return p > 0 ? (int64_t{1} << 40) : (p < 0 ? -(int64_t{1} << 40) : 0);
+  if (shift > 62) return 0;
+  int64_t fl = p >> shift;
+  const int64_t rem = p & ((int64_t{1} << shift) - 1);
+  const int64_t half = int64_t{1} << (shift - 1);
+  if (rem > half || (rem == half && (fl & 1))) ++fl;
+  return fl;
+}
+
+static int NoGpu() {
+  if (tvx_device_count() <= 0)
+    return SetError(TVX_E_DEVICE, "no HIP device: this library has no CPU path");
+  return TVX_OK;
+}
+
+int tvx_conv2d_create(const tvx_conv2d_desc* d, const void* weights_host,
+                      const void* bias_host, tvx_op** out) {
+  if (!d || !out) return SetError(TVX_E_INVALID, "tvx_conv2d_create: null argument");
+  *out = nullptr;
+  if (!d->in_w || !d->in_h || !d->in_c || !d->batch || !d->k_w || !d->k_h || !d->out_w ||
+      !d->out_h || !d->out_c || !d->stride_w || !d->stride_h || !d->dilation_w || !d->dilation_h)
+    return SetError(TVX_E_INVALID, "tvx_conv2d_create: zero extent, stride or dilation");
+  if (d->multiplier < 0) return SetError(TVX_E_INVALID, "tvx_conv2d_create: negative multiplier");
+  if (d->multiplier > 0 && d->out_c != d->in_c * static_cast<uint32_t>(d->multiplier))
+    return SetError(TVX_E_INVALID, "tvx_conv2d_create: depthwise out_c %u != in_c %u * multiplier %d",
+                    d->out_c, d->in_c, d->multiplier);
+  // the last window row/column must start inside the padded input
+  if (static_cast<uint64_t>(d->out_w - 1) * d->stride_w >= static_cast<uint64_t>(d->in_w) + d->pad_left ||
+      static_cast<uint64_t>(d->out_h - 1) * d->stride_h >= static_cast<uint64_t>(d->in_h) + d->pad_top)
+    return SetError(TVX_E_INVALID, "tvx_conv2d_create: output extent reaches past the input");
+  int s = CheckOperandTypes(d->in_dtype, d->w_dtype, d->out_dtype, "tvx_conv2d_create");
+  if (s != TVX_OK) return s;
+  if ((s = NoGpu()) != TVX_OK) return s;
+
+  tvx_op* op = new (std::nothrow) tvx_op();
+  if (!op) return SetError(TVX_E_NOMEM, "tvx_conv2d_create: host allocation failed");
+  op->kind = OP_CONV2D;
+  op->conv = *d;
+  op->conv.w_scales = nullptr;  // host pointer is not kept
+  op->quantized = IsQuant(d->in_dtype);
+  op->has_const_weights = weights_host != nullptr;
+  op->w_zp = d->w_scales ? 0 : d->w_zp;
+  if (op->quantized) {
+    std::vector<int32_t>&mult = op->h_mult, &shift = op->h_shift;
+    s = BuildRequantTables(d->out_c, d->in_scale, d->w_scale, d->w_scales, d->out_scale, &mult, &shift);
+    if (s == TVX_OK) s = op->mult.Upload(mult.data(), mult.size() * 4);
+    if (s == TVX_OK) s = op->shift.Upload(shift.data(), shift.size() * 4);
+    ActRange(d->out_dtype, d->out_scale, d->out_zp, d->activation, &op->act_lo, &op->act_hi);
+    if (s != TVX_OK) { delete op; return s; }
+  }
+  s = TVX_E_UNSUPPORTED;
+  for (ConvSetupFn fn : ConvVariants()) {
+    s = fn(op, d, weights_host, bias_host);
+    if (s != TVX_E_UNSUPPORTED) break;
+  }
+  if (s != TVX_OK) { delete op; return s; }
+  *out = op;
+  return TVX_OK;
+}
+
+int tvx_fully_connected_create(const tvx_fc_desc* d, const void* weights_host,
+                               const void* bias_host, tvx_op** out) {
+  if (!d || !out) return SetError(TVX_E_INVALID, "tvx_fully_connected_create: null argument");
+  *out = nullptr;
+  if (!d->m || !d->k || !d->n) return SetError(TVX_E_INVALID, "tvx_fully_connected_create: zero extent");
+  int s = CheckOperandTypes(d->in_dtype, d->w_dtype, d->out_dtype, "tvx_fully_connected_create");
+  if (s != TVX_OK) return s;
+  if ((s = NoGpu()) != TVX_OK) return s;
+  tvx_op* op = new (std::nothrow) tvx_op();
+  if (!op) return SetError(TVX_E_NOMEM, "tvx_fully_connected_create: host allocation failed");
+  op->kind = OP_FC;
+  op->fc = *d;
+  op->fc.w_scales = nullptr;
+  op->quantized = IsQuant(d->in_dtype);
+  op->has_const_weights = weights_host != nullptr;
+  op->w_zp = d->w_scales ? 0 : d->w_zp;
+  if (op->quantized) {
+    std::vector<int32_t>&mult = op->h_mult, &shift = op->h_shift;
+    s = BuildRequantTables(d->n, d->in_scale, d->w_scale, d->w_scales, d->out_scale, &mult, &shift);
+    if (s == TVX_OK) s = op->mult.Upload(mult.data(), mult.size() * 4);
+    if (s == TVX_OK) s = op->shift.Upload(shift.data(), shift.size() * 4);
+    ActRange(d->out_dtype, d->out_scale, d->out_zp, d->activation, &op->act_lo, &op->act_hi);
+    if (s != TVX_OK) { delete op; return s; }
+  }
+  s = TVX_E_UNSUPPORTED;
+  for (FcSetupFn fn : FcVariants()) {
+    s = fn(op, d, weights_host, bias_host);
+    if (s != TVX_E_UNSUPPORTED) break;
+  }
+  if (s != TVX_OK) { delete op; return s; }
+  *out = op;
+  return TVX_OK;
+}
+
+int tvx_pool2d_create(const tvx_pool2d_desc* d, tvx_op** out) {
+  if (!d || !out) return SetError(TVX_E_INVALID, "tvx_pool2d_create: null argument");
+  *out = nullptr;
+  if (!d->in_w || !d->in_h || !d->channels || !d->batch || !d->out_w || !d->out_h || !d->k_w ||
+      !d->k_h || !d->stride_w || !d->stride_h)
+    return SetError(TVX_E_INVALID, "tvx_pool2d_create: zero extent or stride");
+  if (!ValidDtype(d->dtype)) return SetError(TVX_E_INVALID, "tvx_pool2d_create: unknown dtype");
+  if (d->pool_type != TVX_POOL_MAX && d->pool_type != TVX_POOL_AVG && d->pool_type != TVX_POOL_AVG_ANDROID)
+    return SetError(TVX_E_UNSUPPORTED, "tvx_pool2d_create: pool type %d", d->pool_type);
+  int s = NoGpu();
+  if (s != TVX_OK) return s;
+  tvx_op* op = new (std::nothrow) tvx_op();
+  if (!op) return SetError(TVX_E_NOMEM, "tvx_pool2d_create: host allocation failed");
+  op->kind = OP_POOL2D;
+  op->pool = *d;
+  op->quantized = IsQuant(d->dtype);
+  if (op->quantized && (!(d->in_scale > 0.f) || !(d->out_scale > 0.f))) {
+    delete op;
+    return SetError(TVX_E_INVALID, "tvx_pool2d_create: scales must be positive");
+  }
+  s = TVX_E_UNSUPPORTED;
+  for (SimpleSetupFn fn : PoolVariants()) {
+    s = fn(op);
+    if (s != TVX_E_UNSUPPORTED) break;
+  }
+  if (s != TVX_OK) { delete op; return s; }
+  *out = op;
+  return TVX_OK;
+}
+
+static int CreateSimple(int kind, const tvx_eltwise_desc* d, tvx_op** out, int (*setup)(tvx_op*),
+                        const char* what) {
+  if (!d || !out) return SetError(TVX_E_INVALID, "%s: null argument", what);
+  *out = nullptr;
+  if (!ValidDtype(d->dtype)) return SetError(TVX_E_INVALID, "%s: unknown dtype", what);
+  if (IsQuant(d->dtype) && (!(d->a_scale > 0.f) || !(d->out_scale > 0.f) ||
+                            (kind == OP_ADD && !(d->b_scale > 0.f))))
+    return SetError(TVX_E_INVALID, "%s: scales must be positive", what);
+  int s = NoGpu();
+  if (s != TVX_OK) return s;
+  tvx_op* op = new (std::nothrow) tvx_op();
+  if (!op) return SetError(TVX_E_NOMEM, "%s: host allocation failed", what);
+  op->kind = kind;
+  op->elt = *d;
+  op->quantized = IsQuant(d->dtype);
+  s = setup(op);
+  if (s != TVX_OK) { delete op; return s; }
+  *out = op;
+  return TVX_OK;
+}
+
+int tvx_activation_create(const tvx_eltwise_desc* d, tvx_op** out) {
+  return CreateSimple(OP_ACTIVATION, d, out, ActivationSetup, "tvx_activation_create");
+}
+
+int tvx_add_create(const tvx_eltwise_desc* d, tvx_op** out) {
+  return CreateSimple(OP_ADD, d, out, AddSetup, "tvx_add_create");
+}
+
+int tvx_softmax_create(const tvx_softmax_desc* d, tvx_op** out) {
+  if (!d || !out) return SetError(TVX_E_INVALID, "tvx_softmax_create: null argument");
+  *out = nullptr;
+  if (!d->channels) return SetError(TVX_E_INVALID, "tvx_softmax_create: zero channels");
+  if (!ValidDtype(d->in_dtype)) return SetError(TVX_E_INVALID, "tvx_softmax_create: unknown dtype");
+  int s = NoGpu();
+  if (s != TVX_OK) return s;
+  tvx_op* op = new (std::nothrow) tvx_op();
+  if (!op) return SetError(TVX_E_NOMEM, "tvx_softmax_create: host allocation failed");
+  op->kind = OP_SOFTMAX;
+  op->sm = *d;
+  op->quantized = IsQuant(d->in_dtype);
+  s = SoftmaxSetup(op);
+  if (s != TVX_OK) { delete op; return s; }
+  *out = op;
+  return TVX_OK;
+}
+
+int tvx_op_run(tvx_op* op, const void* in0, const void* in1, void* out_ptr, void* stream) {
+  if (!op || !op->run) return SetError(TVX_E_INVALID, "tvx_op_run: null operator");
+  if (!in0 || !out_ptr) return SetError(TVX_E_INVALID, "tvx_op_run: null tensor pointer");
+  if ((op->kind == OP_CONV2D || op->kind == OP_FC) && !op->has_const_weights && !in1)
+    return SetError(TVX_E_INVALID, "tvx_op_run: operator was created without weights, pass them as in1");
+  if (op->kind == OP_ADD && !in1) return SetError(TVX_E_INVALID, "tvx_op_run: Add needs two operands");
+  return op->run(op, in0, in1, out_ptr, static_cast<hipStream_t>(stream));
+}
+
+const char* tvx_op_kernel_name(const tvx_op* op) { return op ? op->kernel_name : ""; }
+
+void tvx_op_destroy(tvx_op* op) { delete op; }
+
+}  // extern "C"

@@ -1,0 +1,110 @@
+// Shared declarations of the HIP side: the operator object behind tvx_op,
+// error reporting, and the device-side requantization every epilogue uses.
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <vector>
+
+#include "tvx_hip.h"
+
+namespace tvx {
+
+int SetError(int status, const char* fmt, ...);
+
+#define TVX_HIP_CHECK(expr)                                                     \
+  do {                                                                          \
+    hipError_t e_ = (expr);                                                     \
+    if (e_ != hipSuccess)                                                       \
+      return ::tvx::SetError(TVX_E_DEVICE, "%s failed: %s (%s:%d)", #expr,      \
+                             hipGetErrorString(e_), __FILE__, __LINE__);        \
+  } while (0)
+
+enum OpKind { OP_CONV2D = 1, OP_FC, OP_POOL2D, OP_ACTIVATION, OP_ADD, OP_SOFTMAX };
+
+// Device buffer owned by an operator, released in its destructor.
+struct DeviceBuffer {
+  void* ptr = nullptr;
+  size_t bytes = 0;
+  ~DeviceBuffer() { if (ptr) (void)hipFree(ptr); }
+  DeviceBuffer() = default;
+  DeviceBuffer(const DeviceBuffer&) = delete;
+  DeviceBuffer& operator=(const DeviceBuffer&) = delete;
+  int Upload(const void* host, size_t n);
+  int Alloc(size_t n);
+  template <typename T> T* as() const { return static_cast<T*>(ptr); }
+};
+
+}  // namespace tvx
+
+// The object behind the opaque handle. One `run` function per kernel variant.
+struct tvx_op {
+  int kind = 0;
+  const char* kernel_name = "";
+  int (*run)(tvx_op*, const void* in0, const void* in1, void* out, hipStream_t) = nullptr;
+
+  tvx_conv2d_desc conv{};
+  tvx_fc_desc fc{};
+  tvx_pool2d_desc pool{};
+  tvx_eltwise_desc elt{};
+  tvx_softmax_desc sm{};
+
+  bool quantized = false;
+  bool has_const_weights = false;
+  int32_t act_lo = 0, act_hi = 0;  // output clamp incl. fused activation
+  int32_t w_zp = 0;                // 0 for per-channel weights
+
+  tvx::DeviceBuffer weights;  // as given (WHIcOc / {K,N})
+  tvx::DeviceBuffer packed;   // variant-specific re-packed weights
+  tvx::DeviceBuffer bias;     // int32 or float [oc]
+  tvx::DeviceBuffer mult;     // int32 [oc]
+  tvx::DeviceBuffer shift;    // int32 [oc]
+  tvx::DeviceBuffer aux;      // variant-specific tables (e.g. folded bias)
+  std::vector<int32_t> h_mult, h_shift;  // host copies of mult / shift
+
+  // variant-specific launch geometry
+  int32_t geo[8] = {0};
+};
+
+namespace tvx {
+
+// ---- device-side arithmetic -------------------------------------------------
+
+// round_half_even(acc * mult / 2^shift); shift in [1, 62] (host guarantees it,
+// larger shifts are delivered as mult = 0).
+__device__ __forceinline__ int64_t RequantRne(int32_t acc, int32_t mult, int32_t shift) {
+  const int64_t p = static_cast<int64_t>(acc) * static_cast<int64_t>(mult);
+  int64_t fl = p >> shift;
+  const int64_t rem = p & ((int64_t{1} << shift) - 1);
+  const int64_t half = int64_t{1} << (shift - 1);
+  if (rem > half || (rem == half && (fl & 1))) ++fl;
+  return fl;
+}
+
+__device__ __forceinline__ int32_t RequantClamp(int32_t acc, int32_t mult, int32_t shift,
+                                                int32_t zp, int32_t lo, int32_t hi) {
+  int64_t r = RequantRne(acc, mult, shift) + zp;
+  r = r < lo ? lo : (r > hi ? hi : r);
+  return static_cast<int32_t>(r);
+}
+
+// ---- host helpers ------------------------------------------------------------
+// Per-output-channel requantization tables (mult/shift) for a conv / FC.
+int BuildRequantTables(uint32_t channels, float in_scale, float w_scale,
+                       const float* w_scales, float out_scale,
+                       std::vector<int32_t>* mult, std::vector<int32_t>* shift);
+void ActRange(int out_dtype, float out_scale, int32_t out_zp, int act, int32_t* lo, int32_t* hi);
+inline bool IsQuant(int dtype) { return dtype == TVX_U8 || dtype == TVX_I8; }
+inline size_t DtypeBytes(int dtype) {
+  return dtype == TVX_F32 ? 4 : (dtype == TVX_F16 ? 2 : 1);
+}
+
+int ActivationSetup(tvx_op* op);
+int AddSetup(tvx_op* op);
+int SoftmaxSetup(tvx_op* op);
+
+}  // namespace tvx

@@ -1,0 +1,30 @@
+// Registry of kernel variants. Each setup function inspects the operator at
+// creation and either claims it (TVX_OK: packs weights, fills op->run and
+// op->kernel_name), declines (TVX_E_UNSUPPORTED: the next variant is asked),
+// or fails (any other status aborts creation). Lists are ordered fastest
+// first; the generic variant at the end accepts everything the descriptor
+// checks let through.
+#pragma once
+
+#include <vector>
+
+#include "tvx_internal.h"
+
+namespace tvx {
+
+typedef int (*ConvSetupFn)(tvx_op*, const tvx_conv2d_desc*, const void* weights_host,
+                           const void* bias_host);
+typedef int (*FcSetupFn)(tvx_op*, const tvx_fc_desc*, const void* weights_host,
+                         const void* bias_host);
+typedef int (*SimpleSetupFn)(tvx_op*);
+
+const std::vector<ConvSetupFn>& ConvVariants();
+const std::vector<FcSetupFn>& FcVariants();
+const std::vector<SimpleSetupFn>& PoolVariants();
+
+// generic (kernels_generic.hip)
+int ConvGenericSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
+int FcGenericSetup(tvx_op*, const tvx_fc_desc*, const void*, const void*);
+int PoolGenericSetup(tvx_op*);
+
+}  // namespace tvx

@@ -1,0 +1,21 @@
+// Priority order of the kernel variants (fastest first, generic last).
+#include "variants.h"
+
+namespace tvx {
+
+const std::vector<ConvSetupFn>& ConvVariants() {
+  static const std::vector<ConvSetupFn> v = {ConvGenericSetup};
+  return v;
+}
+
+const std::vector<FcSetupFn>& FcVariants() {
+  static const std::vector<FcSetupFn> v = {FcGenericSetup};
+  return v;
+}
+
+const std::vector<SimpleSetupFn>& PoolVariants() {
+  static const std::vector<SimpleSetupFn> v = {PoolGenericSetup};
+  return v;
+}
+
+}  // namespace tvx
