@@ -1,0 +1,189 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized convolution hot path on one MI355X.
+
+A step = one pass of the hot path over one batch of synthetic input that is
+already resident in HBM. The headline workload is BASELINE.json's configs[1]:
+one uint8 per-tensor Conv2d 3x3 64->64 on 56x56 at batch 32, SAME padding, fused
+ReLU6. Prints ONE JSON line (metric: int8 conv TOPS) carrying the dominant
+kernel's roofline and a CPU baseline timed on the host cores; `extra` holds the
+same measurements for the other single-operator configurations.
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+REPO = os.path.dirname(os.path.abspath(__file__))
+for p in (REPO, os.path.join(REPO, "oracle"), os.path.join(REPO, "tests")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, 5.0 POP/s
+PEAK_HBM_GBS = 8000.0     # HBM3E, 8 TB/s
+SEED = 0x71
+
+
+def conv_cfg2(T, rng):
+    n, c, h, w, oc = 32, 64, 56, 56, 64
+    x = rng.integers(0, 256, n * c * h * w, dtype=np.uint8)
+    wt = rng.integers(0, 256, oc * c * 9, dtype=np.uint8)
+    b = rng.integers(-4096, 4097, oc).astype(np.int32)
+    d = T.Conv2dDesc()
+    d.in_w, d.in_h, d.in_c, d.batch = w, h, c, n
+    d.k_w = d.k_h = 3
+    d.out_w, d.out_h, d.out_c = w, h, oc
+    d.stride_w = d.stride_h = d.dilation_w = d.dilation_h = 1
+    d.pad_left = d.pad_top = 1
+    d.in_dtype = d.w_dtype = d.out_dtype = T.U8
+    d.in_scale, d.in_zp, d.w_scale, d.w_zp = 0.05, 128, 0.01, 120
+    d.out_scale, d.out_zp, d.activation = 0.1, 0, T.ACT_RELU6
+    op = T.conv2d_create(d, wt, b)
+    macs = n * h * w * oc * c * 9
+    algo_bytes = x.size + n * oc * h * w + wt.size + 4 * oc
+    oracle_kws = dict(in_shape=[w, h, c, n], w_shape=[3, 3, c, oc], out_shape=[w, h, oc, n],
+                      stride=[1, 1], dilation=[1, 1], pad_left=1, pad_top=1, multiplier=0,
+                      in_dtype=0, w_dtype=0, out_dtype=0, in_q=(0.05, 128), w_q=(0.01, 120, None),
+                      out_q=(0.1, 0), act=2)
+    return dict(name="conv2d_u8_3x3_64to64_56x56_b32_same_relu6", op=op, inputs=(x,), out_elems=n * oc * h * w,
+                out_dtype=np.uint8, ops=2 * macs, algo_bytes=algo_bytes, bound="mfma",
+                oracle=("conv2d", (x, wt, b), oracle_kws, n))
+
+
+def fc_cfg5(T, rng):
+    m, k, n = 8192, 4096, 4096
+    x = rng.integers(-128, 128, m * k, dtype=np.int8)
+    wt = rng.integers(-128, 128, n * k, dtype=np.int8)
+    b = rng.integers(-16384, 16385, n).astype(np.int32)
+    ws = np.exp(rng.uniform(np.log(0.001), np.log(0.02), n)).astype(np.float32)
+    d = T.FcDesc()
+    d.m, d.k, d.n = m, k, n
+    d.in_dtype = d.w_dtype = d.out_dtype = T.I8
+    d.in_scale, d.in_zp = 0.02, 0
+    import ctypes as C
+    d.w_scales = ws.ctypes.data_as(C.POINTER(C.c_float))
+    d.out_scale, d.out_zp = 0.05, 0
+    op = T.fully_connected_create(d, wt, b)
+    return dict(name="fc_i8_per_channel_m8192_k4096_n4096", op=op, inputs=(x,), out_elems=m * n,
+                out_dtype=np.int8, ops=2 * m * k * n, algo_bytes=m * k + n * k + m * n + 4 * n,
+                bound="mfma", oracle=None)
+
+
+def time_workload(wl, steps, warmup):
+    """Returns (wall ms per step over exactly `steps` steps, mean per-launch kernel ms)."""
+    import torch
+    stream = torch.cuda.current_stream()
+    dev_in = [torch.from_numpy(a).cuda() for a in wl["inputs"]]
+    tdt = {np.uint8: torch.uint8, np.int8: torch.int8}[wl["out_dtype"]]
+    out = torch.empty(wl["out_elems"], dtype=tdt, device="cuda")
+    op = wl["op"]
+    in1 = dev_in[1] if len(dev_in) > 1 else None
+    for _ in range(warmup):
+        op.run(dev_in[0], in1, out, stream.cuda_stream)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        op.run(dev_in[0], in1, out, stream.cuda_stream)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    # per-launch duration: HIP events recorded on the launch stream around every launch
+    pairs = []
+    for _ in range(steps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        op.run(dev_in[0], in1, out, stream.cuda_stream)
+        e1.record(stream)
+        pairs.append((e0, e1))
+    torch.cuda.synchronize()
+    kernel_ms = float(np.mean([a.elapsed_time(b) for a, b in pairs]))
+    wl["device_out"] = out
+    return wall_ms, kernel_ms
+
+
+def roofline(wl, kernel_ms, traffic=None):
+    if wl["bound"] == "mfma":
+        achieved = wl["ops"] / (kernel_ms * 1e-3) / 1e12
+        return dict(bound="mfma", achieved=round(achieved, 3), peak=PEAK_INT8_TOPS, unit="TOP/s",
+                    frac=round(achieved / PEAK_INT8_TOPS, 5), traffic=traffic)
+    achieved = wl["algo_bytes"] / (kernel_ms * 1e-3) / 1e9
+    return dict(bound="hbm", achieved=round(achieved, 2), peak=PEAK_HBM_GBS, unit="GB/s",
+                frac=round(achieved / PEAK_HBM_GBS, 5), traffic=traffic)
+
+
+def cpu_baseline(wl, gpu_out):
+    """The CPU restatement (oracle, OpenMP) on a bounded sample of the same workload:
+    the first `sample_n` images of the batch; also re-checks the GPU result on them."""
+    import tvx_oracle as O
+    kind, arrays, kws, batch = wl["oracle"]
+    sample_n = 4
+    x, wt, b = arrays
+    per_img = x.size // batch
+    kws = dict(kws)
+    kws["in_shape"] = kws["in_shape"][:3] + [sample_n]
+    kws["out_shape"] = kws["out_shape"][:3] + [sample_n]
+    xs = np.ascontiguousarray(x[:per_img * sample_n])
+    O.conv2d(xs[:per_img], wt, b, **dict(kws, in_shape=kws["in_shape"][:3] + [1],
+                                        out_shape=kws["out_shape"][:3] + [1]))  # warm-up
+    t0 = time.perf_counter()
+    ref = O.conv2d(xs, wt, b, **kws)
+    dt = time.perf_counter() - t0
+    ok = bool(np.array_equal(ref, gpu_out[:ref.size]))
+    tops = wl["ops"] * sample_n / batch / dt / 1e12
+    return dict(value=round(tops, 5), unit="TOPS", cores=O.lib().tvxo_num_threads(), kind="port",
+                sample="first %d of %d images of the same conv, CPU restatement (not the vendor simulator), "
+                       "OpenMP, %.2f s; GPU output equal on the sample: %s" % (sample_n, batch, dt, ok)), ok
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-extra", action="store_true", help="skip the non-headline workloads")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU: the hot path has no CPU fallback")
+    T = importlib.import_module("tim-vx_amd")
+    rng = np.random.default_rng(SEED)
+
+    wl = conv_cfg2(T, rng)
+    wall_ms, kernel_ms = time_workload(wl, args.steps, args.warmup)
+    gpu_out = wl["device_out"].cpu().numpy()
+    cpu, parity_ok = cpu_baseline(wl, gpu_out)
+    traffic = None
+    tpath = os.path.join(REPO, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        traffic = json.load(open(tpath)).get(wl["op"].kernel_name)
+    line = {
+        "metric": "int8 conv TOPS", "value": round(wl["ops"] / (wall_ms * 1e-3) / 1e12, 3), "unit": "TOPS",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8",
+        "data": "synthetic",
+        "config": {"workload": wl["name"], "kernel": wl["op"].kernel_name, "batch": 32,
+                   "parity_vs_oracle_on_sample": parity_ok},
+        "roofline": dict(roofline(wl, kernel_ms, traffic), kernel=wl["op"].kernel_name,
+                         kernel_ms=round(kernel_ms, 5)),
+        "cpu_baseline": cpu,
+    }
+    if not args.no_extra:
+        extra = {}
+        for make in (fc_cfg5,):
+            w2 = make(T, rng)
+            steps2 = max(5, min(args.steps, 50))
+            wall2, k2 = time_workload(w2, steps2, min(args.warmup, 5))
+            extra[w2["name"]] = dict(kernel=w2["op"].kernel_name, ms_per_step=round(wall2, 5),
+                                     tops=round(w2["ops"] / (wall2 * 1e-3) / 1e12, 2),
+                                     gbs=round(w2["algo_bytes"] / (wall2 * 1e-3) / 1e9, 1),
+                                     roofline=dict(roofline(w2, k2), kernel_ms=round(k2, 5)))
+        line["extra"] = extra
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

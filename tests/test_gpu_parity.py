@@ -170,3 +170,46 @@ def test_eltwise_float(oracle):
     assert np.array_equal(TC.gpu_add(3, a, (1.0, 0), b, (1.0, 0), (1.0, 0)), a + b)
     h = a.astype(np.float16)
     assert np.array_equal(TC.gpu_activation(1, 2, h, (1.0, 0), (1.0, 0)), np.maximum(h, 0))
+
+
+@pytest.mark.parametrize("mode", ["u8", "i8pc", "u8pc"])
+@pytest.mark.parametrize("shape", [(300, 512, 272), (257, 144, 513), (2, 1280, 1000)])
+def test_fully_connected_mfma_edges(oracle, mode, shape):
+    """Tile edges of the MFMA variant: M, N not multiples of the 256-tile, K of the 128-step."""
+    m, k, n = shape
+    rng = np.random.default_rng(m + k + n)
+    in_dt = 0 if mode.startswith("u8") else 1
+    w_dt = 0 if mode == "u8" else 1
+    x, w = rand_q(rng, m * k, in_dt), rand_q(rng, n * k, w_dt)
+    b = rng.integers(-16384, 16385, n).astype(np.int32)
+    wq = (0.01, 117, None) if mode == "u8" else \
+        (1.0, 0, np.exp(rng.uniform(np.log(0.001), np.log(0.02), n)).astype(np.float32))
+    kws = dict(m=m, k=k, n=n, in_dtype=in_dt, w_dtype=w_dt, out_dtype=in_dt,
+               in_q=(0.02, 131 if in_dt == 0 else -2), w_q=wq,
+               out_q=(float(np.float32(0.02 * 0.01 * 40 * np.sqrt(k))), 5 if in_dt == 0 else 0))
+    want = oracle.fully_connected(x, w, b, **kws)
+    got = TC.gpu_fully_connected(x, w, b, want_kernel="fc_mfma_i8_256x256x128", **kws)
+    assert np.array_equal(got, want)
+    assert len(np.unique(want)) > 4
+
+
+def test_fully_connected_full_size_int8_per_channel(oracle):
+    """M=8192, K=4096, N=4096 int8 per-channel: the whole problem on the GPU, a
+    seeded sample of 48 rows recomputed by the oracle, plus linearity in the bias."""
+    m, k, n = 8192, 4096, 4096
+    rng = np.random.default_rng(0x75)
+    x = rng.integers(-128, 128, m * k, dtype=np.int8)
+    w = rng.integers(-128, 128, n * k, dtype=np.int8)
+    b = rng.integers(-16384, 16385, n).astype(np.int32)
+    ws = np.exp(rng.uniform(np.log(0.001), np.log(0.02), n)).astype(np.float32)
+    kws = dict(k=k, n=n, in_dtype=1, w_dtype=1, out_dtype=1, in_q=(0.02, 0), w_q=(1.0, 0, ws),
+               out_q=(0.05, 0))
+    got = TC.gpu_fully_connected(x, w, b, m=m, want_kernel="fc_mfma_i8_256x256x128", **kws).reshape(m, n)
+    rows = np.sort(rng.choice(m, 48, replace=False))
+    want = oracle.fully_connected(np.ascontiguousarray(x.reshape(m, k)[rows]).ravel(), w, b, m=len(rows), **kws)
+    assert np.array_equal(got[rows], want.reshape(len(rows), n))
+    assert len(np.unique(got)) > 100
+    # rows are independent: permuting input rows permutes output rows
+    perm = rng.permutation(m)
+    got_p = TC.gpu_fully_connected(np.ascontiguousarray(x.reshape(m, k)[perm]).ravel(), w, b, m=m, **kws)
+    assert np.array_equal(got_p.reshape(m, n), got[perm])

@@ -22,6 +22,9 @@ const std::vector<ConvSetupFn>& ConvVariants();
 const std::vector<FcSetupFn>& FcVariants();
 const std::vector<SimpleSetupFn>& PoolVariants();
 
+// int8 MFMA fully-connected (fc_mfma_i8.hip)
+int FcMfmaSetup(tvx_op*, const tvx_fc_desc*, const void*, const void*);
+
 // generic (kernels_generic.hip)
 int ConvGenericSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 int FcGenericSetup(tvx_op*, const tvx_fc_desc*, const void*, const void*);

@@ -9,7 +9,7 @@ const std::vector<ConvSetupFn>& ConvVariants() {
 }
 
 const std::vector<FcSetupFn>& FcVariants() {
-  static const std::vector<FcSetupFn> v = {FcGenericSetup};
+  static const std::vector<FcSetupFn> v = {FcMfmaSetup, FcGenericSetup};
   return v;
 }
 
