@@ -118,23 +118,25 @@ def cpu_baseline(wl, gpu_out):
     the first `sample_n` images of the batch; also re-checks the GPU result on them."""
     import tvx_oracle as O
     kind, arrays, kws, batch = wl["oracle"]
-    sample_n = 4
+    sample_n = batch  # the whole batch, repeated until about 10 s of CPU time have passed
     x, wt, b = arrays
     per_img = x.size // batch
     kws = dict(kws)
-    kws["in_shape"] = kws["in_shape"][:3] + [sample_n]
-    kws["out_shape"] = kws["out_shape"][:3] + [sample_n]
-    xs = np.ascontiguousarray(x[:per_img * sample_n])
-    O.conv2d(xs[:per_img], wt, b, **dict(kws, in_shape=kws["in_shape"][:3] + [1],
-                                        out_shape=kws["out_shape"][:3] + [1]))  # warm-up
-    t0 = time.perf_counter()
-    ref = O.conv2d(xs, wt, b, **kws)
-    dt = time.perf_counter() - t0
+    O.conv2d(np.ascontiguousarray(x[:per_img]), wt, b,
+             **dict(kws, in_shape=kws["in_shape"][:3] + [1], out_shape=kws["out_shape"][:3] + [1]))  # warm-up
+    reps, dt = 0, 0.0
+    while dt < 10.0 and reps < 50:
+        t0 = time.perf_counter()
+        ref = O.conv2d(x, wt, b, **kws)
+        dt += time.perf_counter() - t0
+        reps += 1
+    dt /= reps
     ok = bool(np.array_equal(ref, gpu_out[:ref.size]))
     tops = wl["ops"] * sample_n / batch / dt / 1e12
     return dict(value=round(tops, 5), unit="TOPS", cores=O.lib().tvxo_num_threads(), kind="port",
-                sample="first %d of %d images of the same conv, CPU restatement (not the vendor simulator), "
-                       "OpenMP, %.2f s; GPU output equal on the sample: %s" % (sample_n, batch, dt, ok)), ok
+                sample="the same %d-image conv, %d repetitions of %.3f s each; CPU restatement in C with OpenMP "
+                       "(not the vendor simulator, which cannot run here); GPU output equal to it: %s"
+                       % (batch, reps, dt, ok)), ok
 
 
 def main():

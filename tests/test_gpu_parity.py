@@ -213,3 +213,44 @@ def test_fully_connected_full_size_int8_per_channel(oracle):
     perm = rng.permutation(m)
     got_p = TC.gpu_fully_connected(np.ascontiguousarray(x.reshape(m, k)[perm]).ravel(), w, b, m=m, **kws)
     assert np.array_equal(got_p.reshape(m, n), got[perm])
+
+
+def test_conv2d_cfg2_full_size(oracle):
+    """uint8 3x3 64->64 on 56x56x64 at batch 32, SAME, fused ReLU6: whole output vs the oracle."""
+    rng = np.random.default_rng(0x72)
+    n, c, h, w, oc = 32, 64, 56, 56, 64
+    x = rng.integers(0, 256, n * c * h * w, dtype=np.uint8)
+    wt = rng.integers(0, 256, oc * c * 9, dtype=np.uint8)
+    b = rng.integers(-4096, 4097, oc).astype(np.int32)
+    kws = dict(in_shape=[w, h, c, n], w_shape=[3, 3, c, oc], out_shape=[w, h, oc, n], stride=[1, 1],
+               dilation=[1, 1], pad_left=1, pad_top=1, multiplier=0, in_dtype=0, w_dtype=0, out_dtype=0,
+               in_q=(0.05, 128), w_q=(0.01, 120, None), out_q=(0.1, 0), act=2)
+    want = oracle.conv2d(x, wt, b, **kws)
+    got = TC.gpu_conv2d(x, wt, b, want_kernel="conv2d_igemm_i8", **kws)
+    assert np.array_equal(got, want)
+    assert got.max() == 60 and len(np.unique(got)) == 61  # ReLU6 at scale 0.1: q in [0, 60]
+
+
+IGEMM_GRID = [
+    # (n, c, h, w, oc, kh, kw, stride, dil, pad[l,r,t,b])
+    (2, 32, 28, 28, 64, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),
+    (1, 3, 32, 32, 32, 3, 3, [2, 2], [1, 1], [0, 1, 0, 1]),
+    (2, 16, 14, 14, 96, 1, 1, [1, 1], [1, 1], [0, 0, 0, 0]),
+    (1, 64, 9, 7, 40, 3, 3, [1, 1], [2, 2], [2, 2, 2, 2]),
+    (1, 20, 8, 8, 50, 5, 5, [1, 1], [1, 1], [0, 0, 0, 0]),
+    (3, 64, 7, 7, 160, 3, 3, [2, 1], [1, 1], [1, 1, 1, 1]),
+    (1, 24, 13, 20, 144, 1, 1, [1, 1], [1, 1], [0, 0, 0, 0]),
+]
+
+
+@pytest.mark.parametrize("mode", ["u8", "i8pc", "u8pc"])
+@pytest.mark.parametrize("gi", range(len(IGEMM_GRID)))
+def test_conv2d_igemm_shapes(oracle, gi, mode):
+    n, c, h, w, oc, kh, kw, stride, dil, pad = IGEMM_GRID[gi]
+    rng = np.random.default_rng(2000 + gi)
+    x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=oc, kh=kh, kw=kw, stride=stride, dil=dil,
+                              pad=pad, mult=0, mode=mode)
+    want = oracle.conv2d(x, wt, b, act=1, **kws)
+    got = TC.gpu_conv2d(x, wt, b, act=1, want_kernel="conv2d_igemm_i8", **kws)
+    assert np.array_equal(got, want)
+    assert len(np.unique(want)) > 4

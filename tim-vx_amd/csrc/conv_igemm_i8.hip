@@ -1,0 +1,565 @@
+// Dense quantized Conv2d as an implicit GEMM on the int8 matrix cores.
+//
+// GEMM view: rows = output pixels of one image, columns = output channels,
+// reduction = (ky, kx, c) with the channel fastest. Activations arrive WHCN
+// (W fastest, channel planes H*W apart) but v_mfma_i32_32x32x32_i8 wants 16
+// consecutive reduction bytes per lane, so the workgroup first builds a
+// channel-innermost halo tile of its input window in LDS (4 x 4 byte
+// transposes in registers on the way in, all global loads of a thread in
+// flight at once). Out-of-image positions of the tile hold the input zero
+// point, so every window sums over all taps and the zero-point expansion
+//   sum (x - zx)(w - zw) = sum xs ws - zws * Sx - zxs * Sw + K zxs zws
+// needs one per-pixel sum Sx (taken with v_dot4 from the fragments already in
+// registers) and per-channel constants folded into the bias at creation.
+// The MFMA A operand of tap (ky, kx) is read straight out of the halo tile -
+// no im2col copy exists anywhere. The packed weights of the channel block are
+// DMA-ed global -> LDS (no registers) while the halo tile is being built and
+// stay there for the whole tile.
+//
+// Epilogue: requantize with 32-bit arithmetic where the shifts allow it, pack
+// four pixels per dword, stage [oc][pixel] in LDS, copy out as contiguous
+// runs of the WHCN output.
+#include <algorithm>
+
+#include "variants.h"
+
+namespace tvx {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int kThreads = 256;
+constexpr int kMaxPtw = 2;     // 32-pixel MFMA tiles per wavefront (tile <= 256 pixels)
+constexpr int kLoadBatch = 8;  // halo units a thread keeps in flight
+
+// requantization flavours of the epilogue
+constexpr int kRqGeneric = 0;    // any shift: 64-bit product
+constexpr int kRqFast = 1;       // all shifts >= 33: high half of the product + tie fix-up
+constexpr int kRqFastNoTie = 2;  // additionally no accumulator can land on a tie
+
+struct ConvArgs {
+  const uint8_t* x;
+  const int8_t* w;       // packed [oc_alloc][kstride]
+  uint8_t* y;
+  const int32_t* biasf;  // bias + per-channel zero-point terms
+  const v4i* rq;         // per channel {mult, shift | t, half, lowmask}
+  int C, H, W, OC, OH, OW;
+  int kh, kw, sh, sw, dh, dw, pad_t, pad_l;
+  int cp, cpc;           // channels padded to 16, and 16-byte chunks per pixel
+  int ksteps, kstride;
+  int P, PT, tiles_per_image, oct;
+  int iht, iwt;          // halo tile extent
+  int swz_shift, swz_mask;
+  int xor_mask;          // 0x80808080 for uint8 activations, else 0
+  int pad_fill;          // input zero point (int8 domain) in all four bytes
+  int zws, out_zp, lo, hi;
+  int out_stride;        // epilogue staging row stride in bytes (odd number of dwords)
+  int w_chunks;          // 16-byte chunks of one channel block's weights
+  uint32_t magic_c4n, magic_w4n;  // ceil(2^32 / d) for the loader's index split (0: d == 1)
+  int off_w, off_halo, off_sx;    // LDS carve-up
+};
+
+__device__ __forceinline__ int FastDiv(int u, uint32_t magic) {
+  return magic ? static_cast<int>(__umulhi(static_cast<uint32_t>(u), magic)) : u;
+}
+
+__device__ __forceinline__ int HaloOffset(const ConvArgs& a, int hp, int c) {
+  const int cc = c >> 4;
+  const int sw = (hp >> a.swz_shift) & a.swz_mask;
+  return hp * a.cp + (((cc ^ sw) << 4) | (c & 15));
+}
+
+__device__ __forceinline__ int ChannelFill(const ConvArgs& a, int c) {
+  // zero-point bytes for real channels, zero for the padding up to 16
+  const int n = a.C - c;  // real channels left in this group of four
+  if (n >= 4) return a.pad_fill;
+  if (n <= 0) return 0;
+  return a.pad_fill & ((1 << (8 * n)) - 1);
+}
+
+// Position of one lane's 16-byte chunk in the (ky, kx, chunk) reduction order.
+struct ChunkIter {
+  int cc, kx, ky;
+};
+
+template <int RQ>
+__device__ __forceinline__ int Requant8(int v, const v4i& q, int zp, int lo, int hi) {
+  if (RQ == kRqGeneric) return RequantClamp(v, q[0], q[1], zp, lo, hi);
+  // shift = 32 + t, t >= 1: the low half of the product only matters on exact ties
+  const int h = __mulhi(v, q[0]);
+  int r = (h + q[2]) >> q[1];
+  if (RQ == kRqFast) {
+    const bool tie = ((h & (2 * q[2] - 1)) == q[2]) && ((v & q[3]) == 0);
+    if (tie && (r & 1)) --r;
+  }
+  r += zp;
+  return r < lo ? lo : (r > hi ? hi : r);
+}
+
+template <int OT, int RQ>
+__global__ void __launch_bounds__(kThreads) ConvIgemmKernel(ConvArgs a) {
+  extern __shared__ __attribute__((aligned(16))) int8_t lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tile = blockIdx.x % a.tiles_per_image;
+  const int n = blockIdx.x / a.tiles_per_image;
+  const int oc0 = blockIdx.y * a.oct;
+  const int hw = a.OH * a.OW;
+  const int p0 = tile * a.P;
+  const int p_end = min(p0 + a.P, hw);
+  const int r0 = p0 / a.OW;
+  const int r1 = (p_end - 1) / a.OW;
+  const int ih0 = r0 * a.sh - a.pad_t;
+  const int rows_needed = (r1 - r0) * a.sh + (a.kh - 1) * a.dh + 1;
+
+  int8_t* w_lds = lds + a.off_w;
+  int8_t* halo = lds + a.off_halo;
+  int* sx_lds = reinterpret_cast<int*>(lds + a.off_sx);
+
+  // ---- weights of this channel block: global -> LDS DMA, 1 KiB per wave instruction
+  {
+    const int8_t* src = a.w + static_cast<size_t>(oc0) * a.kstride;
+    for (int i = wave * 64; i < a.w_chunks; i += kThreads) {
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)(src + static_cast<size_t>(i + lane) * 16),
+          (__attribute__((address_space(3))) void*)(w_lds + i * 16), 16, 0, 0);
+    }
+  }
+  // ---- halo tile -------------------------------------------------------------
+  const size_t plane = static_cast<size_t>(a.H) * a.W;
+  const uint8_t* xin = a.x + static_cast<size_t>(n) * a.C * plane;
+  const int c4n = a.cp / 4;
+  if ((a.W & 3) == 0) {
+    // unit = (halo row, 4 input columns, 4 channels); lanes run over channel groups first
+    const int w4n = a.W / 4;
+    const int units = rows_needed * w4n * c4n;
+    for (int base = 0; base < units; base += kThreads * kLoadBatch) {
+      int d[kLoadBatch][4];
+#pragma unroll
+      for (int b = 0; b < kLoadBatch; ++b) {
+        const int u = base + b * kThreads + tid;
+        d[b][0] = d[b][1] = d[b][2] = d[b][3] = 0;
+        if (u < units) {
+          const int q1 = FastDiv(u, a.magic_c4n);
+          const int c = (u - q1 * c4n) * 4;
+          const int hr = FastDiv(q1, a.magic_w4n);
+          const int w4 = q1 - hr * w4n;
+          const int ih = ih0 + hr;
+          if (ih >= 0 && ih < a.H) {
+            const uint8_t* src = xin + c * plane + static_cast<size_t>(ih) * a.W + w4 * 4;
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              if (c + j < a.C) d[b][j] = *reinterpret_cast<const int*>(src + j * plane) ^ a.xor_mask;
+          } else {
+            // a row above / below the image: the zero point in every real channel
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+              if (c + j < a.C) d[b][j] = a.pad_fill;
+          }
+        }
+      }
+#pragma unroll
+      for (int b = 0; b < kLoadBatch; ++b) {
+        const int u = base + b * kThreads + tid;
+        if (u < units) {
+          const int q1 = FastDiv(u, a.magic_c4n);
+          const int c = (u - q1 * c4n) * 4;
+          const int hr = FastDiv(q1, a.magic_w4n);
+          const int w4 = q1 - hr * w4n;
+          // 4 x 4 byte transpose: d[j] = 4 pixels of channel c+j  ->  px[i] = 4 channels of pixel i
+          const int lo01 = __builtin_amdgcn_perm(d[b][1], d[b][0], 0x05010400);
+          const int hi01 = __builtin_amdgcn_perm(d[b][1], d[b][0], 0x07030602);
+          const int lo23 = __builtin_amdgcn_perm(d[b][3], d[b][2], 0x05010400);
+          const int hi23 = __builtin_amdgcn_perm(d[b][3], d[b][2], 0x07030602);
+          int px[4];
+          px[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100);
+          px[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302);
+          px[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100);
+          px[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302);
+          const int hc = a.pad_l + w4 * 4;
+          const int hp = hr * a.iwt + hc;
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (hc + i < a.iwt) *reinterpret_cast<int*>(halo + HaloOffset(a, hp + i, c)) = px[i];
+        }
+      }
+    }
+  } else {
+    // general width: one (halo row, column, 4 channels) dword at a time
+    const int units = rows_needed * a.W * c4n;
+    for (int u = tid; u < units; u += kThreads) {
+      const int c4 = u % c4n;
+      const int iw = (u / c4n) % a.W;
+      const int hr = u / (c4n * a.W);
+      if (a.pad_l + iw >= a.iwt) continue;
+      const int ih = ih0 + hr;
+      const int c = c4 * 4;
+      int v = ChannelFill(a, c);
+      if (ih >= 0 && ih < a.H) {
+        v = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          if (c + j >= a.C) continue;
+          const int b = xin[(c + j) * plane + static_cast<size_t>(ih) * a.W + iw] ^ (a.xor_mask & 0xff);
+          v |= b << (8 * j);
+        }
+      }
+      *reinterpret_cast<int*>(halo + HaloOffset(a, hr * a.iwt + a.pad_l + iw, c)) = v;
+    }
+  }
+  // left / right padding columns
+  {
+    const int right0 = a.pad_l + a.W;
+    const int pad_cols = a.pad_l + max(a.iwt - right0, 0);
+    const int units = rows_needed * pad_cols * c4n;
+    for (int u = tid; u < units; u += kThreads) {
+      const int c4 = u % c4n;
+      const int pc = (u / c4n) % pad_cols;
+      const int hr = u / (c4n * pad_cols);
+      const int hc = pc < a.pad_l ? pc : right0 + (pc - a.pad_l);
+      *reinterpret_cast<int*>(halo + HaloOffset(a, hr * a.iwt + hc, c4 * 4)) = ChannelFill(a, c4 * 4);
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the weight DMA has landed
+  __syncthreads();
+
+  // ---- main loop ---------------------------------------------------------------
+  const int frag_row = lane & 31, frag_half = lane >> 5;
+  int hp_base[kMaxPtw];
+  int n_ptw = 0;
+#pragma unroll
+  for (int i = 0; i < kMaxPtw; ++i) {
+    const int pt = wave + 4 * i;
+    hp_base[i] = 0;
+    if (pt < a.PT) {
+      n_ptw = i + 1;
+      int p = p0 + pt * 32 + frag_row;
+      p = min(p, hw - 1);
+      const int oh = p / a.OW, ow = p - oh * a.OW;
+      hp_base[i] = (oh - r0) * a.sh * a.iwt + ow * a.sw;
+    }
+  }
+  v16i acc[kMaxPtw][OT];
+#pragma unroll
+  for (int i = 0; i < kMaxPtw; ++i)
+#pragma unroll
+    for (int j = 0; j < OT; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+  int sx[kMaxPtw] = {0, 0};
+
+  // Every wavefront runs the same instruction stream: a wavefront whose second
+  // pixel tile lies beyond the workgroup's tile computes it anyway (on pixel 0)
+  // and drops the result, and the padding chunk of an odd chunk count is read
+  // from a valid address and zeroed, so no MFMA sits under divergent control flow.
+  {
+    const int row_step = a.dh * a.iwt;
+    ChunkIter it;
+    if (a.cpc == 1) { it.cc = 0; it.kx = frag_half; it.ky = 0; }
+    else { it.cc = frag_half; it.kx = 0; it.ky = 0; }
+    while (it.kx >= a.kw) { it.kx -= a.kw; ++it.ky; }
+    const int8_t* w_row = w_lds + frag_row * a.kstride + frag_half * 16;
+
+    auto load_a = [&](v4i* fa) {
+      const bool valid = it.ky < a.kh;
+      const int tap_hp = valid ? it.ky * row_step + it.kx * a.dw : 0;
+      const int cc = valid ? it.cc : 0;
+#pragma unroll
+      for (int i = 0; i < kMaxPtw; ++i) {
+        const int hp = hp_base[i] + tap_hp;
+        const int swz = (hp >> a.swz_shift) & a.swz_mask;
+        const v4i v = *reinterpret_cast<const v4i*>(halo + hp * a.cp + ((cc ^ swz) << 4));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) fa[i][e] = valid ? v[e] : 0;
+      }
+    };
+    auto load_b = [&](v4i* fb, int ks) {
+      // one k-step past the end reads bytes that exist in LDS and are never used
+#pragma unroll
+      for (int j = 0; j < OT; ++j)
+        fb[j] = *reinterpret_cast<const v4i*>(w_row + j * 32 * a.kstride + ks * 32);
+    };
+    auto advance = [&]() {
+      it.cc += 2;
+#pragma unroll
+      for (int rep = 0; rep < 2; ++rep) {
+        const bool wrap = it.cc >= a.cpc;
+        it.cc -= wrap ? a.cpc : 0;
+        it.kx += wrap ? 1 : 0;
+        const bool row = it.kx >= a.kw;
+        it.kx = row ? 0 : it.kx;
+        it.ky += row ? 1 : 0;
+      }
+    };
+    auto step = [&](const v4i* fa, const v4i* fb) {
+#pragma unroll
+      for (int i = 0; i < kMaxPtw; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) sx[i] = __builtin_amdgcn_sdot4(fa[i][q], 0x01010101, sx[i], false);
+#pragma unroll
+      for (int j = 0; j < OT; ++j)
+#pragma unroll
+        for (int i = 0; i < kMaxPtw; ++i)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    };
+
+    v4i fa0[kMaxPtw], fb0[OT], fa1[kMaxPtw], fb1[OT];
+    load_a(fa0);
+    load_b(fb0, 0);
+    int ks = 0;
+    for (; ks + 1 < a.ksteps; ks += 2) {
+      advance();
+      load_a(fa1);
+      load_b(fb1, ks + 1);
+      step(fa0, fb0);
+      advance();
+      load_a(fa0);
+      load_b(fb0, ks + 2);
+      step(fa1, fb1);
+    }
+    if (ks < a.ksteps) step(fa0, fb0);
+  }
+
+  // ---- epilogue ----------------------------------------------------------------
+#pragma unroll
+  for (int i = 0; i < kMaxPtw; ++i) {
+    sx[i] += __shfl_xor(sx[i], 32);
+    if (i < n_ptw && frag_half == 0) sx_lds[(wave + 4 * i) * 32 + frag_row] = sx[i];
+  }
+  __syncthreads();  // everyone is done reading weights and halo; sx_lds is visible
+  int8_t* out_tile = lds + a.off_w;  // [oct][out_stride], aliases weights + halo
+#pragma unroll
+  for (int j = 0; j < OT; ++j) {
+    const int ocl = j * 32 + frag_row;
+    const int oc = oc0 + ocl;  // tables are allocated up to the padded channel count
+    const int bias = a.biasf[oc];
+    const v4i q = a.rq[oc];
+#pragma unroll
+    for (int i = 0; i < kMaxPtw; ++i) {
+      if (i >= n_ptw) continue;
+      const int pt = wave + 4 * i;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int pl = pt * 32 + 8 * g + 4 * frag_half;
+        const v4i s4 = *reinterpret_cast<const v4i*>(sx_lds + pl);
+        uint32_t packed = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int v = acc[i][j][g * 4 + e] + bias - a.zws * s4[e];
+          packed |= static_cast<uint32_t>(Requant8<RQ>(v, q, a.out_zp, a.lo, a.hi) & 0xff) << (8 * e);
+        }
+        *reinterpret_cast<uint32_t*>(out_tile + ocl * a.out_stride + pl) = packed;
+      }
+    }
+  }
+  __syncthreads();
+  const int valid = p_end - p0;
+  const int oc_n = min(a.oct, a.OC - oc0);
+  uint8_t* ybase = a.y + (static_cast<size_t>(n) * a.OC + oc0) * hw + p0;
+  if ((hw & 3) == 0) {
+    const int per_row = valid >> 2;  // p0 and hw are multiples of 4: whole dwords
+    for (int o = wave; o < oc_n; o += 4)
+      for (int dwi = lane; dwi < per_row; dwi += 64)
+        *reinterpret_cast<uint32_t*>(ybase + static_cast<size_t>(o) * hw + dwi * 4) =
+            *reinterpret_cast<const uint32_t*>(out_tile + o * a.out_stride + dwi * 4);
+  } else {
+    for (int o = wave; o < oc_n; o += 4)
+      for (int pi = lane; pi < valid; pi += 64)
+        ybase[static_cast<size_t>(o) * hw + pi] = static_cast<uint8_t>(out_tile[o * a.out_stride + pi]);
+  }
+}
+
+struct Plan {
+  ConvArgs a;
+  int lds_bytes;
+  int ot, rq;
+  dim3 grid;
+};
+
+template <int OT>
+void LaunchRq(const Plan* plan, const ConvArgs& a, hipStream_t st) {
+  const dim3 block(kThreads);
+  if (plan->rq == kRqFastNoTie)
+    hipLaunchKernelGGL((ConvIgemmKernel<OT, kRqFastNoTie>), plan->grid, block, plan->lds_bytes, st, a);
+  else if (plan->rq == kRqFast)
+    hipLaunchKernelGGL((ConvIgemmKernel<OT, kRqFast>), plan->grid, block, plan->lds_bytes, st, a);
+  else
+    hipLaunchKernelGGL((ConvIgemmKernel<OT, kRqGeneric>), plan->grid, block, plan->lds_bytes, st, a);
+}
+
+int ConvIgemmRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
+  const Plan* plan = reinterpret_cast<const Plan*>(op->host_blob.data());
+  ConvArgs a = plan->a;
+  a.x = static_cast<const uint8_t*>(in0);
+  a.y = static_cast<uint8_t*>(out);
+  if (plan->ot == 1) LaunchRq<1>(plan, a, st);
+  else if (plan->ot == 2) LaunchRq<2>(plan, a, st);
+  else LaunchRq<4>(plan, a, st);
+  TVX_HIP_CHECK(hipGetLastError());
+  return TVX_OK;
+}
+
+int RoundUp(int v, int m) { return (v + m - 1) / m * m; }
+
+uint32_t Magic(int d) {
+  return d <= 1 ? 0u : static_cast<uint32_t>(((uint64_t{1} << 32) + d - 1) / d);
+}
+
+template <int OT, int RQ>
+hipError_t AllowLds(int bytes) {
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(&ConvIgemmKernel<OT, RQ>),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
+}  // namespace
+
+// Claims dense quantized convolutions with constant weights whose weight block
+// and halo tile fit the CU's LDS.
+int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const void* bias_host) {
+  if (!op->quantized || !w_host || d->multiplier != 0) return TVX_E_UNSUPPORTED;
+  ConvArgs a{};
+  a.C = d->in_c; a.H = d->in_h; a.W = d->in_w; a.OC = d->out_c; a.OH = d->out_h; a.OW = d->out_w;
+  a.kh = d->k_h; a.kw = d->k_w; a.sh = d->stride_h; a.sw = d->stride_w;
+  a.dh = d->dilation_h; a.dw = d->dilation_w; a.pad_t = d->pad_top; a.pad_l = d->pad_left;
+  a.cp = RoundUp(a.C, 16);
+  a.cpc = a.cp / 16;
+  const int taps = a.kh * a.kw;
+  const int kchunks = taps * a.cpc;
+  a.ksteps = (kchunks + 1) / 2;
+  a.kstride = a.ksteps * 32 + 16;
+  const int oc_pad = RoundUp(a.OC, 32);
+  const int ot = oc_pad <= 32 ? 1 : (oc_pad <= 64 ? 2 : 4);
+  a.oct = 32 * ot;
+  const int oc_blocks = (oc_pad + a.oct - 1) / a.oct;
+  const int oc_alloc = oc_blocks * a.oct;
+  // pixel tile: the multiple of 32 (<= 256) wasting the fewest MFMA rows
+  const int hw = a.OH * a.OW;
+  int best_p = 32;
+  double best_eff = 0;
+  for (int p = 256; p >= 32; p -= 32) {
+    const int tiles = (hw + p - 1) / p;
+    const double eff = static_cast<double>(hw) / (static_cast<double>(tiles) * p);
+    if (eff > best_eff + 1e-9) { best_eff = eff; best_p = p; }
+  }
+  a.P = best_p;
+  a.PT = a.P / 32;
+  a.tiles_per_image = (hw + a.P - 1) / a.P;
+  // halo extent: the most output rows any tile touches
+  int max_rows = 1;
+  for (int t = 0; t < a.tiles_per_image; ++t) {
+    const int p0 = t * a.P, pe = std::min(p0 + a.P, hw);
+    max_rows = std::max(max_rows, (pe - 1) / a.OW - p0 / a.OW + 1);
+  }
+  a.iht = (max_rows - 1) * a.sh + (a.kh - 1) * a.dh + 1;
+  a.iwt = std::max((a.OW - 1) * a.sw + (a.kw - 1) * a.dw + 1, 1);
+  // 16-byte chunks of a pixel are XOR-swizzled with the pixel index so that the
+  // 32 rows of a fragment read spread over all bank groups (power-of-two chunk counts)
+  if (a.cpc == 2) { a.swz_shift = 2; a.swz_mask = 1; }
+  else if (a.cpc == 4) { a.swz_shift = 1; a.swz_mask = 3; }
+  else if (a.cpc >= 8 && (a.cpc & (a.cpc - 1)) == 0) { a.swz_shift = 0; a.swz_mask = 7; }
+  else { a.swz_shift = 0; a.swz_mask = 0; }
+  const bool x_u8 = d->in_dtype == TVX_U8, w_u8 = d->w_dtype == TVX_U8;
+  const int zxs = d->in_zp - (x_u8 ? 128 : 0);
+  const int zws = op->w_zp - (w_u8 ? 128 : 0);
+  if (zxs < -128 || zxs > 127) return TVX_E_UNSUPPORTED;  // zero point outside the tensor's range
+  a.xor_mask = x_u8 ? static_cast<int>(0x80808080u) : 0;
+  a.pad_fill = static_cast<int>(static_cast<uint32_t>(zxs & 0xff) * 0x01010101u);
+  a.zws = zws;
+  a.out_zp = d->out_zp; a.lo = op->act_lo; a.hi = op->act_hi;
+  a.out_stride = ((a.P / 4) | 1) * 4;
+  a.magic_c4n = Magic(a.cp / 4);
+  a.magic_w4n = Magic(std::max(a.W / 4, 1));
+  // LDS carve-up: the per-pixel sums first; the weight + halo region behind them
+  // is reused as the epilogue's staging tile
+  const int w_bytes = RoundUp(a.oct * a.kstride, 1024);  // whole 1 KiB DMA bursts
+  a.w_chunks = w_bytes / 16;
+  const int halo_bytes = RoundUp(a.iht * a.iwt * a.cp + 16, 16);
+  const int sx_bytes = a.P * 4;
+  a.off_sx = 0;
+  a.off_w = sx_bytes;
+  a.off_halo = a.off_w + w_bytes;
+  const int out_bytes = a.oct * a.out_stride;
+  const int lds_bytes = a.off_w + std::max(w_bytes + halo_bytes, RoundUp(out_bytes, 16));
+  if (lds_bytes > 150 * 1024) return TVX_E_UNSUPPORTED;
+  // the loader's index split is exact while units * divisor < 2^32
+  if (static_cast<uint64_t>(a.iht) * a.W * a.cp >= (1ull << 24)) return TVX_E_UNSUPPORTED;
+  if (static_cast<uint64_t>(d->batch) * a.tiles_per_image > 0x7fffffffull) return TVX_E_UNSUPPORTED;
+
+  // ---- pack weights [oc][(ky,kx,c)] int8 with zero padding, fold constants -------
+  // slack behind the last block: its DMA reads whole 1 KiB bursts
+  std::vector<int8_t> packed(static_cast<size_t>(oc_alloc) * a.kstride + 1024, 0);
+  std::vector<int32_t> biasf(oc_alloc, 0);
+  const uint8_t* src = static_cast<const uint8_t*>(w_host);
+  const int32_t* b = static_cast<const int32_t*>(bias_host);
+  for (int oc = 0; oc < a.OC; ++oc) {
+    int64_t sw = 0;
+    for (int t = 0; t < taps; ++t)
+      for (int c = 0; c < a.C; ++c) {
+        const uint8_t raw = src[(static_cast<size_t>(oc) * a.C + c) * taps + t];
+        const int8_t v = static_cast<int8_t>(w_u8 ? raw ^ 0x80 : raw);
+        packed[static_cast<size_t>(oc) * a.kstride + (t * a.cpc + c / 16) * 16 + c % 16] = v;
+        sw += v;
+      }
+    const int64_t v = (b ? b[oc] : 0) - static_cast<int64_t>(zxs) * sw +
+                      static_cast<int64_t>(taps) * a.C * zxs * zws;
+    biasf[oc] = static_cast<int32_t>(static_cast<uint32_t>(v));
+  }
+  // ---- requantization tables: 32-bit arithmetic when every shift is >= 33 -------
+  int rq = kRqFastNoTie;
+  for (int oc = 0; oc < a.OC; ++oc) {
+    const int32_t m = op->h_mult[oc], s = op->h_shift[oc];
+    if (m == 0) continue;
+    if (s < 33) { rq = kRqGeneric; break; }
+    // a tie needs an accumulator v with v * m = 2^(s-1) (mod 2^s): ctz(v) = s - 1 - ctz(m) <= 31
+    if (__builtin_ctz(static_cast<uint32_t>(m)) >= s - 32) rq = kRqFast;
+  }
+  std::vector<int32_t> rqt(static_cast<size_t>(oc_alloc) * 4, 0);
+  for (int oc = 0; oc < oc_alloc; ++oc) {
+    int32_t m = oc < a.OC ? op->h_mult[oc] : 0, s = oc < a.OC ? op->h_shift[oc] : 33;
+    if (m == 0) s = 33;
+    int32_t* q = &rqt[static_cast<size_t>(oc) * 4];
+    q[0] = m;
+    if (rq == kRqGeneric) {
+      q[1] = s;
+    } else {
+      const int t = s - 32;
+      const int ctz = m ? __builtin_ctz(static_cast<uint32_t>(m)) : 0;
+      q[1] = t;
+      q[2] = 1 << (t - 1);
+      q[3] = ctz == 0 ? -1 : static_cast<int32_t>((uint32_t{1} << (32 - ctz)) - 1);
+    }
+  }
+  int s = op->packed.Upload(packed.data(), packed.size());
+  if (s == TVX_OK) s = op->aux.Upload(biasf.data(), biasf.size() * 4);
+  if (s == TVX_OK) s = op->aux2.Upload(rqt.data(), rqt.size() * 4);
+  if (s != TVX_OK) return s;
+  a.w = op->packed.as<int8_t>();
+  a.biasf = op->aux.as<int32_t>();
+  a.rq = op->aux2.as<v4i>();
+
+  hipError_t e = hipSuccess;
+  if (ot == 1) {
+    e = rq == kRqGeneric ? AllowLds<1, kRqGeneric>(lds_bytes)
+        : (rq == kRqFast ? AllowLds<1, kRqFast>(lds_bytes) : AllowLds<1, kRqFastNoTie>(lds_bytes));
+  } else if (ot == 2) {
+    e = rq == kRqGeneric ? AllowLds<2, kRqGeneric>(lds_bytes)
+        : (rq == kRqFast ? AllowLds<2, kRqFast>(lds_bytes) : AllowLds<2, kRqFastNoTie>(lds_bytes));
+  } else {
+    e = rq == kRqGeneric ? AllowLds<4, kRqGeneric>(lds_bytes)
+        : (rq == kRqFast ? AllowLds<4, kRqFast>(lds_bytes) : AllowLds<4, kRqFastNoTie>(lds_bytes));
+  }
+  if (e != hipSuccess)
+    return SetError(TVX_E_DEVICE, "hipFuncSetAttribute(dynamic LDS %d): %s", lds_bytes, hipGetErrorString(e));
+  Plan plan;
+  plan.a = a;
+  plan.lds_bytes = lds_bytes;
+  plan.ot = ot;
+  plan.rq = rq;
+  plan.grid = dim3(static_cast<unsigned>(d->batch * a.tiles_per_image), static_cast<unsigned>(oc_blocks));
+  op->host_blob.assign(reinterpret_cast<const uint8_t*>(&plan), reinterpret_cast<const uint8_t*>(&plan) + sizeof(plan));
+  op->run = ConvIgemmRun;
+  op->kernel_name = "conv2d_igemm_i8";
+  return TVX_OK;
+}
+
+}  // namespace tvx

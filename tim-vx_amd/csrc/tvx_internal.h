@@ -64,7 +64,9 @@ struct tvx_op {
   tvx::DeviceBuffer mult;     // int32 [oc]
   tvx::DeviceBuffer shift;    // int32 [oc]
   tvx::DeviceBuffer aux;      // variant-specific tables (e.g. folded bias)
+  tvx::DeviceBuffer aux2;     // variant-specific tables (e.g. requantization records)
   std::vector<int32_t> h_mult, h_shift;  // host copies of mult / shift
+  std::vector<uint8_t> host_blob;        // variant-specific launch plan
 
   // variant-specific launch geometry
   int32_t geo[8] = {0};

@@ -25,6 +25,9 @@ const std::vector<SimpleSetupFn>& PoolVariants();
 // int8 MFMA fully-connected (fc_mfma_i8.hip)
 int FcMfmaSetup(tvx_op*, const tvx_fc_desc*, const void*, const void*);
 
+// int8 MFMA implicit-GEMM convolution (conv_igemm_i8.hip)
+int ConvIgemmSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
+
 // generic (kernels_generic.hip)
 int ConvGenericSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 int FcGenericSetup(tvx_op*, const tvx_fc_desc*, const void*, const void*);
