@@ -44,20 +44,21 @@ struct ConvArgs {
   uint8_t* y;
   const int32_t* biasf;  // bias + per-channel zero-point terms
   const v4i* rq;         // per channel {mult, shift | t, half, lowmask}
+  const int2* tapt;      // per (k-step, fragment half): {halo byte offset of the chunk, dot4 multiplier}
   int C, H, W, OC, OH, OW;
   int kh, kw, sh, sw, dh, dw, pad_t, pad_l;
   int cp, cpc;           // channels padded to 16, and 16-byte chunks per pixel
   int ksteps, kstride;
   int P, PT, tiles_per_image, oct;
   int iht, iwt;          // halo tile extent
-  int swz_shift, swz_mask;
+  int pix_stride;        // bytes per halo pixel: cp, plus 16 when cp/16 is even (bank spread)
   int xor_mask;          // 0x80808080 for uint8 activations, else 0
   int pad_fill;          // input zero point (int8 domain) in all four bytes
   int zws, out_zp, lo, hi;
   int out_stride;        // epilogue staging row stride in bytes (odd number of dwords)
   int w_chunks;          // 16-byte chunks of one channel block's weights
-  uint32_t magic_c4n, magic_w4n;  // ceil(2^32 / d) for the loader's index split (0: d == 1)
-  int off_w, off_halo, off_sx;    // LDS carve-up
+  int w4_blocks;         // ceil(W / 64): blocks of 16 four-column patches per channel row
+  int off_w, off_halo, off_sx, off_tap;  // LDS carve-up
 };
 
 __device__ __forceinline__ int FastDiv(int u, uint32_t magic) {
@@ -65,9 +66,7 @@ __device__ __forceinline__ int FastDiv(int u, uint32_t magic) {
 }
 
 __device__ __forceinline__ int HaloOffset(const ConvArgs& a, int hp, int c) {
-  const int cc = c >> 4;
-  const int sw = (hp >> a.swz_shift) & a.swz_mask;
-  return hp * a.cp + (((cc ^ sw) << 4) | (c & 15));
+  return hp * a.pix_stride + c;
 }
 
 __device__ __forceinline__ int ChannelFill(const ConvArgs& a, int c) {
@@ -78,23 +77,20 @@ __device__ __forceinline__ int ChannelFill(const ConvArgs& a, int c) {
   return a.pad_fill & ((1 << (8 * n)) - 1);
 }
 
-// Position of one lane's 16-byte chunk in the (ky, kx, chunk) reduction order.
-struct ChunkIter {
-  int cc, kx, ky;
-};
-
 template <int RQ>
 __device__ __forceinline__ int Requant8(int v, const v4i& q, int zp, int lo, int hi) {
   if (RQ == kRqGeneric) return RequantClamp(v, q[0], q[1], zp, lo, hi);
-  // shift = 32 + t, t >= 1: the low half of the product only matters on exact ties
+  // shift = 32 + t, t >= 1: only the high half of the product is needed, the low
+  // half matters on exact ties alone. q[2] = 2^(t-1) + (zp << t) rounds half up
+  // and adds the output zero point in one step.
   const int h = __mulhi(v, q[0]);
   int r = (h + q[2]) >> q[1];
   if (RQ == kRqFast) {
-    const bool tie = ((h & (2 * q[2] - 1)) == q[2]) && ((v & q[3]) == 0);
-    if (tie && (r & 1)) --r;
+    const int half = 1 << (q[1] - 1);
+    const bool tie = ((h & (2 * half - 1)) == half) && ((v & q[3]) == 0);
+    if (tie && ((r - zp) & 1)) --r;
   }
-  r += zp;
-  return r < lo ? lo : (r > hi ? hi : r);
+  return max(lo, min(r, hi));
 }
 
 template <int OT, int RQ>
@@ -125,47 +121,63 @@ __global__ void __launch_bounds__(kThreads) ConvIgemmKernel(ConvArgs a) {
           (__attribute__((address_space(3))) void*)(w_lds + i * 16), 16, 0, 0);
     }
   }
+  // the reduction order as a table (built once per operator): no index math in the main loop
+  int2* tap_lds = reinterpret_cast<int2*>(lds + a.off_tap);
+  for (int i = tid; i < a.ksteps * 2 + 2; i += kThreads) tap_lds[i] = a.tapt[i];
   // ---- halo tile -------------------------------------------------------------
   const size_t plane = static_cast<size_t>(a.H) * a.W;
   const uint8_t* xin = a.x + static_cast<size_t>(n) * a.C * plane;
   const int c4n = a.cp / 4;
   if ((a.W & 3) == 0) {
-    // unit = (halo row, 4 input columns, 4 channels); lanes run over channel groups first
+    // A thread owns one (4 input columns, 4 channels) patch and walks the halo
+    // rows with it, kLoadBatch rows of loads in flight; lanes run over channel
+    // groups first so that a wavefront's LDS stores spread over the banks.
     const int w4n = a.W / 4;
-    const int units = rows_needed * w4n * c4n;
-    for (int base = 0; base < units; base += kThreads * kLoadBatch) {
-      int d[kLoadBatch][4];
+    const int patches = a.w4_blocks * ((c4n + 3) / 4) * 64;
+    const uint32_t plane32 = static_cast<uint32_t>(plane);
+    const int row_bytes = a.iwt * a.pix_stride;
+    for (int pi = tid; pi < patches; pi += kThreads) {
+      // patch index -> (column group, channel group): 16 consecutive lanes read 64
+      // contiguous bytes of one channel row, the next 16 lanes the next channel group
+      const int blk = pi >> 6, in_blk = pi & 63;
+      int w4 = (blk % a.w4_blocks) * 16 + (in_blk & 15);
+      int c4 = (blk / a.w4_blocks) * 4 + (in_blk >> 4);
+      if (w4 >= w4n || c4 >= c4n) continue;
+      const int c = c4 * 4;
+      const int hc = a.pad_l + w4 * 4;
+      // byte offsets of the patch's four channel rows inside this image (< 2^31)
+      uint32_t src_off[4];
+      int fill[4];
 #pragma unroll
-      for (int b = 0; b < kLoadBatch; ++b) {
-        const int u = base + b * kThreads + tid;
-        d[b][0] = d[b][1] = d[b][2] = d[b][3] = 0;
-        if (u < units) {
-          const int q1 = FastDiv(u, a.magic_c4n);
-          const int c = (u - q1 * c4n) * 4;
-          const int hr = FastDiv(q1, a.magic_w4n);
-          const int w4 = q1 - hr * w4n;
-          const int ih = ih0 + hr;
-          if (ih >= 0 && ih < a.H) {
-            const uint8_t* src = xin + c * plane + static_cast<size_t>(ih) * a.W + w4 * 4;
+      for (int j = 0; j < 4; ++j) {
+        const bool real = c + j < a.C;
+        src_off[j] = static_cast<uint32_t>(real ? c + j : 0) * plane32 + static_cast<uint32_t>(w4 * 4);
+        fill[j] = real ? a.pad_fill : 0;
+      }
+      const int xm = a.xor_mask;
+      int xmask[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-              if (c + j < a.C) d[b][j] = *reinterpret_cast<const int*>(src + j * plane) ^ a.xor_mask;
-          } else {
-            // a row above / below the image: the zero point in every real channel
+      for (int j = 0; j < 4; ++j) xmask[j] = c + j < a.C ? xm : 0;
+      const int dst0 = __mul24(hc, a.pix_stride) + c;
+      // columns of this patch that exist in the halo tile (stride > 1 may cut the right edge)
+      const int ncols = min(4, a.iwt - hc);
+      for (int hr0 = 0; hr0 < rows_needed; hr0 += kLoadBatch) {
+        int d[kLoadBatch][4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-              if (c + j < a.C) d[b][j] = a.pad_fill;
+        for (int b = 0; b < kLoadBatch; ++b) {
+          const int ih = ih0 + hr0 + b;
+          const bool inside = hr0 + b < rows_needed && ih >= 0 && ih < a.H;
+          const uint32_t row_off = __umul24(static_cast<uint32_t>(inside ? ih : 0), static_cast<uint32_t>(a.W));
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            // out-of-image rows load row 0 (in bounds) and are replaced by the zero point
+            const int v = *reinterpret_cast<const int*>(xin + (src_off[j] + row_off));
+            d[b][j] = inside ? (c + j < a.C ? v ^ xmask[j] : 0) : fill[j];
           }
         }
-      }
 #pragma unroll
-      for (int b = 0; b < kLoadBatch; ++b) {
-        const int u = base + b * kThreads + tid;
-        if (u < units) {
-          const int q1 = FastDiv(u, a.magic_c4n);
-          const int c = (u - q1 * c4n) * 4;
-          const int hr = FastDiv(q1, a.magic_w4n);
-          const int w4 = q1 - hr * w4n;
+        for (int b = 0; b < kLoadBatch; ++b) {
+          if (hr0 + b >= rows_needed) continue;
           // 4 x 4 byte transpose: d[j] = 4 pixels of channel c+j  ->  px[i] = 4 channels of pixel i
           const int lo01 = __builtin_amdgcn_perm(d[b][1], d[b][0], 0x05010400);
           const int hi01 = __builtin_amdgcn_perm(d[b][1], d[b][0], 0x07030602);
@@ -176,11 +188,10 @@ __global__ void __launch_bounds__(kThreads) ConvIgemmKernel(ConvArgs a) {
           px[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302);
           px[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100);
           px[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302);
-          const int hc = a.pad_l + w4 * 4;
-          const int hp = hr * a.iwt + hc;
+          int8_t* dst = halo + dst0 + __mul24(hr0 + b, row_bytes);
 #pragma unroll
           for (int i = 0; i < 4; ++i)
-            if (hc + i < a.iwt) *reinterpret_cast<int*>(halo + HaloOffset(a, hp + i, c)) = px[i];
+            if (i < ncols) *reinterpret_cast<int*>(dst + __mul24(i, a.pix_stride)) = px[i];
         }
       }
     }
@@ -207,17 +218,16 @@ __global__ void __launch_bounds__(kThreads) ConvIgemmKernel(ConvArgs a) {
       *reinterpret_cast<int*>(halo + HaloOffset(a, hr * a.iwt + a.pad_l + iw, c)) = v;
     }
   }
-  // left / right padding columns
+  // left / right padding columns: one (halo row, pad column) per step of a thread
   {
     const int right0 = a.pad_l + a.W;
     const int pad_cols = a.pad_l + max(a.iwt - right0, 0);
-    const int units = rows_needed * pad_cols * c4n;
-    for (int u = tid; u < units; u += kThreads) {
-      const int c4 = u % c4n;
-      const int pc = (u / c4n) % pad_cols;
-      const int hr = u / (c4n * pad_cols);
+    const int cells = rows_needed * pad_cols;
+    for (int cell = tid; cell < cells; cell += kThreads) {
+      const int hr = cell / pad_cols, pc = cell - hr * pad_cols;
       const int hc = pc < a.pad_l ? pc : right0 + (pc - a.pad_l);
-      *reinterpret_cast<int*>(halo + HaloOffset(a, hr * a.iwt + hc, c4 * 4)) = ChannelFill(a, c4 * 4);
+      int8_t* dst = halo + (hr * a.iwt + hc) * a.pix_stride;
+      for (int c = 0; c < a.cp; c += 4) *reinterpret_cast<int*>(dst + c) = ChannelFill(a, c);
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the weight DMA has landed
@@ -225,77 +235,55 @@ __global__ void __launch_bounds__(kThreads) ConvIgemmKernel(ConvArgs a) {
 
   // ---- main loop ---------------------------------------------------------------
   const int frag_row = lane & 31, frag_half = lane >> 5;
-  int hp_base[kMaxPtw];
+  int a_base[kMaxPtw];  // byte offset of each pixel's window origin in the halo tile (+ this lane's half)
   int n_ptw = 0;
 #pragma unroll
   for (int i = 0; i < kMaxPtw; ++i) {
     const int pt = wave + 4 * i;
-    hp_base[i] = 0;
+    a_base[i] = 0;
     if (pt < a.PT) {
       n_ptw = i + 1;
       int p = p0 + pt * 32 + frag_row;
       p = min(p, hw - 1);
       const int oh = p / a.OW, ow = p - oh * a.OW;
-      hp_base[i] = (oh - r0) * a.sh * a.iwt + ow * a.sw;
+      a_base[i] = ((oh - r0) * a.sh * a.iwt + ow * a.sw) * a.pix_stride;
     }
   }
+  // accumulators start at the folded bias of the lane's output channel
   v16i acc[kMaxPtw][OT];
 #pragma unroll
-  for (int i = 0; i < kMaxPtw; ++i)
+  for (int j = 0; j < OT; ++j) {
+    const int bias = a.biasf[oc0 + j * 32 + frag_row];  // tables cover the padded channel count
 #pragma unroll
-    for (int j = 0; j < OT; ++j)
+    for (int i = 0; i < kMaxPtw; ++i)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = bias;
+  }
   int sx[kMaxPtw] = {0, 0};
 
   // Every wavefront runs the same instruction stream: a wavefront whose second
   // pixel tile lies beyond the workgroup's tile computes it anyway (on pixel 0)
-  // and drops the result, and the padding chunk of an odd chunk count is read
-  // from a valid address and zeroed, so no MFMA sits under divergent control flow.
+  // and drops the result. A k-step's chunk position comes from the tap table; the
+  // padding chunk of an odd chunk count meets zero weights and carries a zero dot4
+  // multiplier, which keeps it out of the pixel sum.
   {
-    const int row_step = a.dh * a.iwt;
-    ChunkIter it;
-    if (a.cpc == 1) { it.cc = 0; it.kx = frag_half; it.ky = 0; }
-    else { it.cc = frag_half; it.kx = 0; it.ky = 0; }
-    while (it.kx >= a.kw) { it.kx -= a.kw; ++it.ky; }
     const int8_t* w_row = w_lds + frag_row * a.kstride + frag_half * 16;
+    const int2* my_tap = tap_lds + frag_half;
 
-    auto load_a = [&](v4i* fa) {
-      const bool valid = it.ky < a.kh;
-      const int tap_hp = valid ? it.ky * row_step + it.kx * a.dw : 0;
-      const int cc = valid ? it.cc : 0;
+    auto load_ab = [&](v4i* fa, v4i* fb, int ks, int2 t) {
 #pragma unroll
-      for (int i = 0; i < kMaxPtw; ++i) {
-        const int hp = hp_base[i] + tap_hp;
-        const int swz = (hp >> a.swz_shift) & a.swz_mask;
-        const v4i v = *reinterpret_cast<const v4i*>(halo + hp * a.cp + ((cc ^ swz) << 4));
-#pragma unroll
-        for (int e = 0; e < 4; ++e) fa[i][e] = valid ? v[e] : 0;
-      }
-    };
-    auto load_b = [&](v4i* fb, int ks) {
+      for (int i = 0; i < kMaxPtw; ++i)
+        fa[i] = *reinterpret_cast<const v4i*>(halo + a_base[i] + t.x);
       // one k-step past the end reads bytes that exist in LDS and are never used
 #pragma unroll
       for (int j = 0; j < OT; ++j)
         fb[j] = *reinterpret_cast<const v4i*>(w_row + j * 32 * a.kstride + ks * 32);
     };
-    auto advance = [&]() {
-      it.cc += 2;
-#pragma unroll
-      for (int rep = 0; rep < 2; ++rep) {
-        const bool wrap = it.cc >= a.cpc;
-        it.cc -= wrap ? a.cpc : 0;
-        it.kx += wrap ? 1 : 0;
-        const bool row = it.kx >= a.kw;
-        it.kx = row ? 0 : it.kx;
-        it.ky += row ? 1 : 0;
-      }
-    };
-    auto step = [&](const v4i* fa, const v4i* fb) {
+    auto step = [&](const v4i* fa, const v4i* fb, int ones) {
 #pragma unroll
       for (int i = 0; i < kMaxPtw; ++i)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) sx[i] = __builtin_amdgcn_sdot4(fa[i][q], 0x01010101, sx[i], false);
+        for (int q = 0; q < 4; ++q) sx[i] = __builtin_amdgcn_sdot4(fa[i][q], ones, sx[i], false);
 #pragma unroll
       for (int j = 0; j < OT; ++j)
 #pragma unroll
@@ -304,36 +292,34 @@ __global__ void __launch_bounds__(kThreads) ConvIgemmKernel(ConvArgs a) {
     };
 
     v4i fa0[kMaxPtw], fb0[OT], fa1[kMaxPtw], fb1[OT];
-    load_a(fa0);
-    load_b(fb0, 0);
+    int2 t0 = my_tap[0], t1 = my_tap[2];  // the table has one spare k-step at its end
+    load_ab(fa0, fb0, 0, t0);
     int ks = 0;
     for (; ks + 1 < a.ksteps; ks += 2) {
-      advance();
-      load_a(fa1);
-      load_b(fb1, ks + 1);
-      step(fa0, fb0);
-      advance();
-      load_a(fa0);
-      load_b(fb0, ks + 2);
-      step(fa1, fb1);
+      const int2 t2 = my_tap[(ks + 2) * 2];
+      load_ab(fa1, fb1, ks + 1, t1);
+      step(fa0, fb0, t0.y);
+      const int2 t3 = my_tap[(ks + 3) * 2];
+      load_ab(fa0, fb0, ks + 2, t2);
+      step(fa1, fb1, t1.y);
+      t0 = t2;
+      t1 = t3;
     }
-    if (ks < a.ksteps) step(fa0, fb0);
+    if (ks < a.ksteps) step(fa0, fb0, t0.y);
   }
 
   // ---- epilogue ----------------------------------------------------------------
 #pragma unroll
   for (int i = 0; i < kMaxPtw; ++i) {
     sx[i] += __shfl_xor(sx[i], 32);
-    if (i < n_ptw && frag_half == 0) sx_lds[(wave + 4 * i) * 32 + frag_row] = sx[i];
+    if (i < n_ptw && frag_half == 0) sx_lds[(wave + 4 * i) * 32 + frag_row] = a.zws * sx[i];
   }
   __syncthreads();  // everyone is done reading weights and halo; sx_lds is visible
   int8_t* out_tile = lds + a.off_w;  // [oct][out_stride], aliases weights + halo
 #pragma unroll
   for (int j = 0; j < OT; ++j) {
     const int ocl = j * 32 + frag_row;
-    const int oc = oc0 + ocl;  // tables are allocated up to the padded channel count
-    const int bias = a.biasf[oc];
-    const v4i q = a.rq[oc];
+    const v4i q = a.rq[oc0 + ocl];
 #pragma unroll
     for (int i = 0; i < kMaxPtw; ++i) {
       if (i >= n_ptw) continue;
@@ -345,7 +331,7 @@ __global__ void __launch_bounds__(kThreads) ConvIgemmKernel(ConvArgs a) {
         uint32_t packed = 0;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const int v = acc[i][j][g * 4 + e] + bias - a.zws * s4[e];
+          const int v = acc[i][j][g * 4 + e] - s4[e];
           packed |= static_cast<uint32_t>(Requant8<RQ>(v, q, a.out_zp, a.lo, a.hi) & 0xff) << (8 * e);
         }
         *reinterpret_cast<uint32_t*>(out_tile + ocl * a.out_stride + pl) = packed;
@@ -452,12 +438,9 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   }
   a.iht = (max_rows - 1) * a.sh + (a.kh - 1) * a.dh + 1;
   a.iwt = std::max((a.OW - 1) * a.sw + (a.kw - 1) * a.dw + 1, 1);
-  // 16-byte chunks of a pixel are XOR-swizzled with the pixel index so that the
-  // 32 rows of a fragment read spread over all bank groups (power-of-two chunk counts)
-  if (a.cpc == 2) { a.swz_shift = 2; a.swz_mask = 1; }
-  else if (a.cpc == 4) { a.swz_shift = 1; a.swz_mask = 3; }
-  else if (a.cpc >= 8 && (a.cpc & (a.cpc - 1)) == 0) { a.swz_shift = 0; a.swz_mask = 7; }
-  else { a.swz_shift = 0; a.swz_mask = 0; }
+  // Consecutive pixels of a fragment read must fall into different 16-byte bank
+  // groups: that holds when the pixel stride is an odd number of 16-byte chunks.
+  a.pix_stride = (a.cpc & 1) ? a.cp : a.cp + 16;
   const bool x_u8 = d->in_dtype == TVX_U8, w_u8 = d->w_dtype == TVX_U8;
   const int zxs = d->in_zp - (x_u8 ? 128 : 0);
   const int zws = op->w_zp - (w_u8 ? 128 : 0);
@@ -467,22 +450,28 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   a.zws = zws;
   a.out_zp = d->out_zp; a.lo = op->act_lo; a.hi = op->act_hi;
   a.out_stride = ((a.P / 4) | 1) * 4;
-  a.magic_c4n = Magic(a.cp / 4);
-  a.magic_w4n = Magic(std::max(a.W / 4, 1));
+  a.w4_blocks = (a.W / 4 + 15) / 16;
   // LDS carve-up: the per-pixel sums first; the weight + halo region behind them
   // is reused as the epilogue's staging tile
   const int w_bytes = RoundUp(a.oct * a.kstride, 1024);  // whole 1 KiB DMA bursts
   a.w_chunks = w_bytes / 16;
-  const int halo_bytes = RoundUp(a.iht * a.iwt * a.cp + 16, 16);
+  const int halo_bytes = RoundUp(a.iht * a.iwt * a.pix_stride + 16, 16);
   const int sx_bytes = a.P * 4;
+  const int tap_bytes = RoundUp((a.ksteps * 2 + 4) * 8, 16);
   a.off_sx = 0;
-  a.off_w = sx_bytes;
+  a.off_tap = sx_bytes;
+  a.off_w = sx_bytes + tap_bytes;
   a.off_halo = a.off_w + w_bytes;
   const int out_bytes = a.oct * a.out_stride;
   const int lds_bytes = a.off_w + std::max(w_bytes + halo_bytes, RoundUp(out_bytes, 16));
   if (lds_bytes > 150 * 1024) return TVX_E_UNSUPPORTED;
   // the loader's index split is exact while units * divisor < 2^32
-  if (static_cast<uint64_t>(a.iht) * a.W * a.cp >= (1ull << 24)) return TVX_E_UNSUPPORTED;
+  if (static_cast<uint64_t>(a.W) * a.cp >= (1ull << 24)) return TVX_E_UNSUPPORTED;
+  // the loader uses 24-bit multiplies and 32-bit offsets inside one image
+  if (static_cast<uint64_t>(a.H) * a.W >= (1ull << 24) ||
+      static_cast<uint64_t>(a.H) * a.W * a.C >= (1ull << 31) ||
+      static_cast<uint64_t>(a.iht) * a.iwt * a.pix_stride >= (1ull << 23))
+    return TVX_E_UNSUPPORTED;
   if (static_cast<uint64_t>(d->batch) * a.tiles_per_image > 0x7fffffffull) return TVX_E_UNSUPPORTED;
 
   // ---- pack weights [oc][(ky,kx,c)] int8 with zero padding, fold constants -------
@@ -509,7 +498,7 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   for (int oc = 0; oc < a.OC; ++oc) {
     const int32_t m = op->h_mult[oc], s = op->h_shift[oc];
     if (m == 0) continue;
-    if (s < 33) { rq = kRqGeneric; break; }
+    if (s < 33 || s - 32 > 20) { rq = kRqGeneric; break; }  // (zp << t) + 2^30 must fit int32
     // a tie needs an accumulator v with v * m = 2^(s-1) (mod 2^s): ctz(v) = s - 1 - ctz(m) <= 31
     if (__builtin_ctz(static_cast<uint32_t>(m)) >= s - 32) rq = kRqFast;
   }
@@ -525,17 +514,28 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
       const int t = s - 32;
       const int ctz = m ? __builtin_ctz(static_cast<uint32_t>(m)) : 0;
       q[1] = t;
-      q[2] = 1 << (t - 1);
+      q[2] = (1 << (t - 1)) + (d->out_zp << t);
       q[3] = ctz == 0 ? -1 : static_cast<int32_t>((uint32_t{1} << (32 - ctz)) - 1);
     }
   }
+  // tap table: chunk q = 2 * kstep + half of the (ky, kx, chunk) order; two spare
+  // k-steps at the end so that the loop's prefetch stays inside the table
+  std::vector<int32_t> tapt(static_cast<size_t>(a.ksteps + 2) * 4, 0);
+  for (int q = 0; q < kchunks; ++q) {
+    const int t = q / a.cpc, cc = q % a.cpc;
+    const int ky = t / a.kw, kx = t % a.kw;
+    tapt[q * 2] = (ky * a.dh * a.iwt + kx * a.dw) * a.pix_stride + cc * 16;
+    tapt[q * 2 + 1] = 0x01010101;
+  }
   int s = op->packed.Upload(packed.data(), packed.size());
+  if (s == TVX_OK) s = op->aux3.Upload(tapt.data(), tapt.size() * 4);
   if (s == TVX_OK) s = op->aux.Upload(biasf.data(), biasf.size() * 4);
   if (s == TVX_OK) s = op->aux2.Upload(rqt.data(), rqt.size() * 4);
   if (s != TVX_OK) return s;
   a.w = op->packed.as<int8_t>();
   a.biasf = op->aux.as<int32_t>();
   a.rq = op->aux2.as<v4i>();
+  a.tapt = op->aux3.as<int2>();
 
   hipError_t e = hipSuccess;
   if (ot == 1) {

@@ -65,6 +65,7 @@ struct tvx_op {
   tvx::DeviceBuffer shift;    // int32 [oc]
   tvx::DeviceBuffer aux;      // variant-specific tables (e.g. folded bias)
   tvx::DeviceBuffer aux2;     // variant-specific tables (e.g. requantization records)
+  tvx::DeviceBuffer aux3;     // variant-specific tables (e.g. reduction-order table)
   std::vector<int32_t> h_mult, h_shift;  // host copies of mult / shift
   std::vector<uint8_t> host_blob;        // variant-specific launch plan
 
