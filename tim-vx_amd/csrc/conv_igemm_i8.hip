@@ -33,11 +33,6 @@ constexpr int kThreads = 256;
 constexpr int kMaxPtw = 2;     // 32-pixel MFMA tiles per wavefront (tile <= 256 pixels)
 constexpr int kLoadBatch = 8;  // halo units a thread keeps in flight
 
-// requantization flavours of the epilogue
-constexpr int kRqGeneric = 0;    // any shift: 64-bit product
-constexpr int kRqFast = 1;       // all shifts >= 33: high half of the product + tie fix-up
-constexpr int kRqFastNoTie = 2;  // additionally no accumulator can land on a tie
-
 struct ConvArgs {
   const uint8_t* x;
   const int8_t* w;       // packed [oc_alloc][kstride]
@@ -75,22 +70,6 @@ __device__ __forceinline__ int ChannelFill(const ConvArgs& a, int c) {
   if (n >= 4) return a.pad_fill;
   if (n <= 0) return 0;
   return a.pad_fill & ((1 << (8 * n)) - 1);
-}
-
-template <int RQ>
-__device__ __forceinline__ int Requant8(int v, const v4i& q, int zp, int lo, int hi) {
-  if (RQ == kRqGeneric) return RequantClamp(v, q[0], q[1], zp, lo, hi);
-  // shift = 32 + t, t >= 1: only the high half of the product is needed, the low
-  // half matters on exact ties alone. q[2] = 2^(t-1) + (zp << t) rounds half up
-  // and adds the output zero point in one step.
-  const int h = __mulhi(v, q[0]);
-  int r = (h + q[2]) >> q[1];
-  if (RQ == kRqFast) {
-    const int half = 1 << (q[1] - 1);
-    const bool tie = ((h & (2 * half - 1)) == half) && ((v & q[3]) == 0);
-    if (tie && ((r - zp) & 1)) --r;
-  }
-  return max(lo, min(r, hi));
 }
 
 template <int OT, int RQ>
@@ -493,31 +472,9 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
                       static_cast<int64_t>(taps) * a.C * zxs * zws;
     biasf[oc] = static_cast<int32_t>(static_cast<uint32_t>(v));
   }
-  // ---- requantization tables: 32-bit arithmetic when every shift is >= 33 -------
-  int rq = kRqFastNoTie;
-  for (int oc = 0; oc < a.OC; ++oc) {
-    const int32_t m = op->h_mult[oc], s = op->h_shift[oc];
-    if (m == 0) continue;
-    if (s < 33 || s - 32 > 20) { rq = kRqGeneric; break; }  // (zp << t) + 2^30 must fit int32
-    // a tie needs an accumulator v with v * m = 2^(s-1) (mod 2^s): ctz(v) = s - 1 - ctz(m) <= 31
-    if (__builtin_ctz(static_cast<uint32_t>(m)) >= s - 32) rq = kRqFast;
-  }
-  std::vector<int32_t> rqt(static_cast<size_t>(oc_alloc) * 4, 0);
-  for (int oc = 0; oc < oc_alloc; ++oc) {
-    int32_t m = oc < a.OC ? op->h_mult[oc] : 0, s = oc < a.OC ? op->h_shift[oc] : 33;
-    if (m == 0) s = 33;
-    int32_t* q = &rqt[static_cast<size_t>(oc) * 4];
-    q[0] = m;
-    if (rq == kRqGeneric) {
-      q[1] = s;
-    } else {
-      const int t = s - 32;
-      const int ctz = m ? __builtin_ctz(static_cast<uint32_t>(m)) : 0;
-      q[1] = t;
-      q[2] = (1 << (t - 1)) + (d->out_zp << t);
-      q[3] = ctz == 0 ? -1 : static_cast<int32_t>((uint32_t{1} << (32 - ctz)) - 1);
-    }
-  }
+  // ---- requantization records: 32-bit arithmetic when every shift allows it -------
+  std::vector<int32_t> rqt;
+  const int rq = BuildRequantRecords(op->h_mult, op->h_shift, a.OC, oc_alloc, d->out_zp, &rqt);
   // tap table: chunk q = 2 * kstep + half of the (ky, kx, chunk) order; two spare
   // k-steps at the end so that the loop's prefetch stays inside the table
   std::vector<int32_t> tapt(static_cast<size_t>(a.ksteps + 2) * 4, 0);

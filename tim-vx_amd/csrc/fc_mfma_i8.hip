@@ -5,9 +5,11 @@
 // Tiling: one 256-thread workgroup (4 wavefronts, 2 x 2) owns a TM x TN = 256 x 256
 // output tile and walks K in steps of 128 bytes; each wavefront accumulates a
 // 128 x 128 sub-tile as 4 x 4 MFMA tiles (256 accumulator registers per lane).
-// Global -> registers -> LDS, double buffered (2 x 64 KiB of the CU's 160 KiB);
-// rows are 128 B in LDS and their 16 B chunks are XOR-swizzled with the row
-// number so that the 32 lanes of a fragment read hit 8 different bank groups.
+// Operand tiles go global -> LDS by DMA (no registers), double buffered (2 x 64
+// KiB of the CU's 160 KiB); rows are 128 B in LDS and their 16 B chunks are
+// XOR-swizzled with the row number so that the 32 lanes of a fragment read hit
+// 8 different bank groups. Fragments of the next 32-byte k-step are fetched
+// while the 16 MFMAs of the current one run.
 //
 // The MFMA "A" operand is the weight fragment and "B" the activation fragment,
 // so a lane ends up with one activation row m and, per accumulator quad, four
@@ -35,19 +37,16 @@ struct FcArgs {
   const int8_t* w;      // [N][K] int8 (uint8 weights are re-biased when packed)
   int8_t* y;            // [M][N]
   const int32_t* biasf; // [N] bias + per-feature zero-point terms
-  const int32_t* mult;  // [N]
-  const int32_t* shift; // [N]
+  const tvx_v4i* rq;    // [N padded to the tile] requantization records
+  const int8_t* zeros;  // 128 x 0x00 then 128 x 0x80: source of reduction chunks past K
   int M, N, K;
   int zws;              // weight zero point in the int8 domain (0 for per-channel)
   int out_zp, lo, hi;
   int tiles_m, tiles_n;
 };
 
-__device__ __forceinline__ int SwizzledOffset(int row, int chunk) {
-  return row * TK + ((chunk ^ (row & 7)) << 4);
-}
 
-template <bool X_U8, bool ROWSUM>
+template <bool X_U8, bool ROWSUM, int RQ>
 __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   const int tid = threadIdx.x;
@@ -60,41 +59,44 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   int tile = blockIdx.x;
   const int total = a.tiles_m * a.tiles_n;
   if ((total & 7) == 0) tile = (tile & 7) * (total >> 3) + (tile >> 3);
-  // inside a run, walk 8 tiles along n before stepping m
   const int tn_idx = tile % a.tiles_n, tm_idx = tile / a.tiles_n;
   const int m0 = tm_idx * TM, n0 = tn_idx * TN;
 
-  // ---- global -> register staging: thread t carries chunk (t % 8) of rows t/8 + 32 i
-  const int ld_chunk = tid & 7;
-  const int ld_row = tid >> 3;
-  v4i stage_x[8], stage_w[8];
-
-  auto load_global = [&](int k0) {
-    const int kc = k0 + ld_chunk * 16;
-    const bool k_ok = kc < a.K;
+  // ---- global -> LDS DMA ------------------------------------------------------
+  // One wave instruction moves 64 x 16 bytes into 1 KiB of consecutive LDS: 8
+  // rows x 128 bytes of an operand tile. The XOR swizzle of the LDS layout is
+  // applied on the source side: lane l fetches chunk (l & 7) ^ (l >> 3) of row
+  // l >> 3, a permutation inside one 128-byte line. A wavefront moves rows
+  // [64 w, 64 w + 64) of both operands per k-tile (16 instructions).
+  const int dma_row = lane >> 3;
+  uint32_t off_x[8], off_w[8];  // byte offsets from the tensor bases (tensors are < 4 GiB)
+  int dma_chunk[2];             // source chunk of this lane for even / odd instructions
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int r = ld_row + 32 * i;
-      v4i vx = {0, 0, 0, 0}, vw = {0, 0, 0, 0};
-      if (k_ok && m0 + r < a.M) {
-        vx = *reinterpret_cast<const v4i*>(a.x + static_cast<size_t>(m0 + r) * a.K + kc);
-        if (X_U8) vx ^= static_cast<int>(0x80808080);
-      }
-      if (k_ok && n0 + r < a.N)
-        vw = *reinterpret_cast<const v4i*>(a.w + static_cast<size_t>(n0 + r) * a.K + kc);
-      stage_x[i] = vx;
-      stage_w[i] = vw;
-    }
-  };
-  auto store_lds = [&](int stage) {
-    int8_t* xs = lds + stage * 2 * kTileBytes;
+  for (int i = 0; i < 8; ++i) {
+    const int r = wave * 64 + i * 8 + dma_row;
+    // LDS slot (row r, position lane & 7) holds chunk (lane & 7) ^ ((r >> 1) & 7) of the row
+    const int chunk = (lane & 7) ^ ((r >> 1) & 7);
+    dma_chunk[i & 1] = chunk;
+    const int xm = min(m0 + r, a.M - 1), wr = min(n0 + r, a.N - 1);  // rows past the edge are computed and dropped
+    off_x[i] = static_cast<uint32_t>(xm) * static_cast<uint32_t>(a.K) + chunk * 16;
+    off_w[i] = static_cast<uint32_t>(wr) * static_cast<uint32_t>(a.K) + chunk * 16;
+  }
+  const bool k_tail = (a.K % TK) != 0;
+  auto dma_tile = [&](int kt, int stage) {
+    int8_t* xs = lds + stage * 2 * kTileBytes + wave * 64 * TK;
     int8_t* ws = xs + kTileBytes;
+    const int k0 = kt * TK;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const int r = ld_row + 32 * i;
-      const int off = SwizzledOffset(r, ld_chunk);
-      *reinterpret_cast<v4i*>(xs + off) = stage_x[i];
-      *reinterpret_cast<v4i*>(ws + off) = stage_w[i];
+      const bool past = k_tail && k0 + dma_chunk[i & 1] * 16 >= a.K;  // only in the last k-tile
+      // reduction bytes past K: zero for the weights, the int8-domain zero (0x80 before
+      // the re-bias of uint8 activations) for the activations
+      const int8_t* px = past ? a.zeros + (X_U8 ? 128 : 0) : a.x + (off_x[i] + k0);
+      const int8_t* pw = past ? a.zeros : a.w + (off_w[i] + k0);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)px,
+                                       (__attribute__((address_space(3))) void*)(xs + i * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)pw,
+                                       (__attribute__((address_space(3))) void*)(ws + i * 1024), 16, 0, 0);
     }
   };
 
@@ -109,42 +111,71 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
 
   const int frag_row = lane & 31;   // row inside a 32-row MFMA tile
   const int frag_half = lane >> 5;  // which 16-byte half of a 32-byte k-step
+  // byte offsets of this lane's fragment rows; the swizzle term depends on kk only
+  const int x_row_off = (wm * 128 + frag_row) * TK, w_row_off = (wn * 128 + frag_row) * TK;
+  const int row7 = (frag_row >> 1) & 7;  // fragment tiles start at multiples of 32 rows
 
+  auto load_frags = [&](const int8_t* xs, const int8_t* ws, int kk, v4i* fx, v4i* fw) {
+    const int sw = (((kk * 2 + frag_half) ^ row7) << 4);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      fx[t] = *reinterpret_cast<const v4i*>(xs + x_row_off + t * 32 * TK + sw);
+      fw[t] = *reinterpret_cast<const v4i*>(ws + w_row_off + t * 32 * TK + sw);
+    }
+  };
+  auto mma = [&](v4i* fx, const v4i* fw) {
+    if (X_U8) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) fx[t] ^= static_cast<int>(0x80808080);
+    }
+    if (ROWSUM) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          rowsum[t] = __builtin_amdgcn_sdot4(fx[t][q], 0x01010101, rowsum[t], false);
+    }
+#pragma unroll
+    for (int tn = 0; tn < 4; ++tn)
+#pragma unroll
+      for (int tm = 0; tm < 4; ++tm)
+        acc[tn][tm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[tn], fx[tm], acc[tn][tm], 0, 0, 0);
+  };
+
+  // Steady state of one k-tile (four 32-byte k-steps, 16 MFMAs each): the
+  // fragments of step kk + 1 are fetched while step kk multiplies; the barrier
+  // that publishes the next tile's DMA sits before the last step, so that the
+  // first fragments of the next tile are already on their way while it runs, and
+  // the DMA of the tile after next starts as soon as the barrier has freed this stage.
   const int k_tiles = (a.K + TK - 1) / TK;
-  load_global(0);
-  store_lds(0);
+  dma_tile(0, 0);
+  if (k_tiles > 1) dma_tile(1, 1);
+  if (k_tiles > 1) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");  // tile 0 landed (16 newer DMAs may be in flight)
+  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-
+  v4i fx0[4], fw0[4], fx1[4], fw1[4];
+  load_frags(lds, lds + kTileBytes, 0, fx0, fw0);
   for (int kt = 0; kt < k_tiles; ++kt) {
     const int stage = kt & 1;
-    if (kt + 1 < k_tiles) load_global((kt + 1) * TK);
     const int8_t* xs = lds + stage * 2 * kTileBytes;
     const int8_t* ws = xs + kTileBytes;
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      const int chunk = kk * 2 + frag_half;
-      v4i fx[4], fw[4];
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        fx[t] = *reinterpret_cast<const v4i*>(xs + SwizzledOffset(wm * 128 + t * 32 + frag_row, chunk));
-        fw[t] = *reinterpret_cast<const v4i*>(ws + SwizzledOffset(wn * 128 + t * 32 + frag_row, chunk));
-      }
-      if (ROWSUM) {
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-#pragma unroll
-          for (int q = 0; q < 4; ++q)
-            rowsum[t] = __builtin_amdgcn_sdot4(fx[t][q], 0x01010101, rowsum[t], false);
-      }
-#pragma unroll
-      for (int tn = 0; tn < 4; ++tn)
-#pragma unroll
-        for (int tm = 0; tm < 4; ++tm)
-          acc[tn][tm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[tn], fx[tm], acc[tn][tm], 0, 0, 0);
-    }
-    if (kt + 1 < k_tiles) store_lds(stage ^ 1);
+    load_frags(xs, ws, 1, fx1, fw1);
+    mma(fx0, fw0);
+    load_frags(xs, ws, 2, fx0, fw0);
+    mma(fx1, fw1);
+    load_frags(xs, ws, 3, fx1, fw1);
+    mma(fx0, fw0);
+    // all my reads of this stage are done and the next tile's DMA has landed
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
+    if (kt + 2 < k_tiles) dma_tile(kt + 2, stage);
+    if (kt + 1 < k_tiles) {
+      const int8_t* nx = lds + (stage ^ 1) * 2 * kTileBytes;
+      load_frags(nx, nx + kTileBytes, 0, fx0, fw0);
+    }
+    mma(fx1, fw1);
   }
+  __syncthreads();  // the epilogue reuses the LDS
 
   // ---- epilogue: requantize, stage the int8 tile in LDS, store 16-byte rows ----
   if (ROWSUM) {
@@ -159,13 +190,13 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
       // accumulator rows 8g + 4*(lane/32) + 0..3 of this MFMA tile = 4 consecutive features
       const int nl = wn * 128 + tn * 32 + 8 * g + 4 * frag_half;
       const int n = n0 + nl;
-      int b4[4], m4[4], s4[4];
+      // records and folded bias are allocated up to the padded feature count
+      int b4[4];
+      tvx_v4i q4[4];
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int nn = n + q < a.N ? n + q : a.N - 1;
-        b4[q] = a.biasf[nn];
-        m4[q] = a.mult[nn];
-        s4[q] = a.shift[nn];
+        b4[q] = a.biasf[n + q];
+        q4[q] = a.rq[n + q];
       }
 #pragma unroll
       for (int tm = 0; tm < 4; ++tm) {
@@ -175,7 +206,7 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
         for (int q = 0; q < 4; ++q) {
           int v = acc[tn][tm][g * 4 + q] + b4[q];
           if (ROWSUM) v -= a.zws * rowsum[tm];
-          const int r = RequantClamp(v, m4[q], s4[q], a.out_zp, a.lo, a.hi);
+          const int r = Requant8<RQ>(v, q4[q], a.out_zp, a.lo, a.hi);
           packed |= static_cast<uint32_t>(r & 0xff) << (8 * q);
         }
         *reinterpret_cast<uint32_t*>(out_tile + ml * kOutStride + nl) = packed;
@@ -199,6 +230,25 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   }
 }
 
+template <bool X_U8, bool ROWSUM>
+void LaunchRq(int rq, dim3 grid, hipStream_t st, const FcArgs& a) {
+  const dim3 block(kThreads);
+  if (rq == kRqFastNoTie)
+    hipLaunchKernelGGL((FcMfmaKernel<X_U8, ROWSUM, kRqFastNoTie>), grid, block, kLdsBytes, st, a);
+  else if (rq == kRqFast)
+    hipLaunchKernelGGL((FcMfmaKernel<X_U8, ROWSUM, kRqFast>), grid, block, kLdsBytes, st, a);
+  else
+    hipLaunchKernelGGL((FcMfmaKernel<X_U8, ROWSUM, kRqGeneric>), grid, block, kLdsBytes, st, a);
+}
+
+template <bool X_U8, bool ROWSUM>
+hipError_t AllowLds(int rq) {
+  const void* f = rq == kRqFastNoTie ? reinterpret_cast<const void*>(&FcMfmaKernel<X_U8, ROWSUM, kRqFastNoTie>)
+                  : (rq == kRqFast ? reinterpret_cast<const void*>(&FcMfmaKernel<X_U8, ROWSUM, kRqFast>)
+                                   : reinterpret_cast<const void*>(&FcMfmaKernel<X_U8, ROWSUM, kRqGeneric>));
+  return hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+}
+
 int FcMfmaRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
   const tvx_fc_desc& d = op->fc;
   FcArgs a;
@@ -206,8 +256,8 @@ int FcMfmaRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t s
   a.w = op->packed.as<int8_t>();
   a.y = static_cast<int8_t*>(out);
   a.biasf = op->aux.as<int32_t>();
-  a.mult = op->mult.as<int32_t>();
-  a.shift = op->shift.as<int32_t>();
+  a.rq = op->aux2.as<tvx_v4i>();
+  a.zeros = op->aux3.as<int8_t>();
   a.M = static_cast<int>(d.m);
   a.N = static_cast<int>(d.n);
   a.K = static_cast<int>(d.k);
@@ -217,12 +267,13 @@ int FcMfmaRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t s
   a.hi = op->act_hi;
   a.tiles_m = (a.M + TM - 1) / TM;
   a.tiles_n = (a.N + TN - 1) / TN;
-  const dim3 grid(a.tiles_m * a.tiles_n), block(kThreads);
+  const dim3 grid(a.tiles_m * a.tiles_n);
   const bool x_u8 = d.in_dtype == TVX_U8, rowsum = a.zws != 0;
-  if (x_u8 && rowsum) hipLaunchKernelGGL((FcMfmaKernel<true, true>), grid, block, kLdsBytes, st, a);
-  else if (x_u8) hipLaunchKernelGGL((FcMfmaKernel<true, false>), grid, block, kLdsBytes, st, a);
-  else if (rowsum) hipLaunchKernelGGL((FcMfmaKernel<false, true>), grid, block, kLdsBytes, st, a);
-  else hipLaunchKernelGGL((FcMfmaKernel<false, false>), grid, block, kLdsBytes, st, a);
+  const int rq = op->geo[1];
+  if (x_u8 && rowsum) LaunchRq<true, true>(rq, grid, st, a);
+  else if (x_u8) LaunchRq<true, false>(rq, grid, st, a);
+  else if (rowsum) LaunchRq<false, true>(rq, grid, st, a);
+  else LaunchRq<false, false>(rq, grid, st, a);
   TVX_HIP_CHECK(hipGetLastError());
   return TVX_OK;
 }
@@ -234,6 +285,8 @@ int FcMfmaRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t s
 int FcMfmaSetup(tvx_op* op, const tvx_fc_desc* d, const void* w_host, const void* bias_host) {
   if (!op->quantized || !w_host || (d->k & 15) != 0) return TVX_E_UNSUPPORTED;
   if (static_cast<uint64_t>(d->m) * d->n >= (1ull << 31) || d->k > (1u << 24)) return TVX_E_UNSUPPORTED;
+  if (static_cast<uint64_t>(d->m) * d->k >= (1ull << 32) || static_cast<uint64_t>(d->n) * d->k >= (1ull << 32))
+    return TVX_E_UNSUPPORTED;  // the operand DMA addresses rows with 32-bit offsets
   const size_t wn = static_cast<size_t>(d->n) * d->k;
   const bool w_u8 = d->w_dtype == TVX_U8;
   // int8-domain operands: uint8 tensors are shifted by 128, zero points follow
@@ -242,7 +295,8 @@ int FcMfmaSetup(tvx_op* op, const tvx_fc_desc* d, const void* w_host, const void
   std::vector<int8_t> ws(wn);
   const uint8_t* src = static_cast<const uint8_t*>(w_host);
   for (size_t i = 0; i < wn; ++i) ws[i] = static_cast<int8_t>(w_u8 ? src[i] ^ 0x80 : src[i]);
-  std::vector<int32_t> biasf(d->n);
+  const uint32_t n_alloc = (d->n + TN - 1) / TN * TN;
+  std::vector<int32_t> biasf(n_alloc, 0);
   const int32_t* b = static_cast<const int32_t*>(bias_host);
   for (uint32_t n = 0; n < d->n; ++n) {
     int64_t sw = 0;
@@ -252,24 +306,23 @@ int FcMfmaSetup(tvx_op* op, const tvx_fc_desc* d, const void* w_host, const void
                       static_cast<int64_t>(d->k) * zxs * zws;
     biasf[n] = static_cast<int32_t>(static_cast<uint32_t>(v));  // int32 accumulators wrap
   }
+  std::vector<int32_t> rqt;
+  const int rq = BuildRequantRecords(op->h_mult, op->h_shift, static_cast<int>(d->n),
+                                     static_cast<int>(n_alloc), d->out_zp, &rqt);
   int s = op->packed.Upload(ws.data(), wn);
   if (s == TVX_OK) s = op->aux.Upload(biasf.data(), biasf.size() * 4);
+  if (s == TVX_OK) s = op->aux2.Upload(rqt.data(), rqt.size() * 4);
+  std::vector<int8_t> zeros(256, 0);
+  for (int i = 128; i < 256; ++i) zeros[i] = static_cast<int8_t>(-128);
+  if (s == TVX_OK) s = op->aux3.Upload(zeros.data(), zeros.size());
   if (s != TVX_OK) return s;
-  hipError_t e = hipSuccess;
-  e = hipFuncSetAttribute(reinterpret_cast<const void*>(&FcMfmaKernel<true, true>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-  if (e == hipSuccess)
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&FcMfmaKernel<true, false>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-  if (e == hipSuccess)
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&FcMfmaKernel<false, true>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-  if (e == hipSuccess)
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&FcMfmaKernel<false, false>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+  const bool x_u8 = d->in_dtype == TVX_U8, rowsum = zws != 0;
+  hipError_t e = x_u8 ? (rowsum ? AllowLds<true, true>(rq) : AllowLds<true, false>(rq))
+                      : (rowsum ? AllowLds<false, true>(rq) : AllowLds<false, false>(rq));
   if (e != hipSuccess)
     return SetError(TVX_E_DEVICE, "hipFuncSetAttribute(dynamic LDS %d): %s", kLdsBytes, hipGetErrorString(e));
   op->geo[0] = zws;
+  op->geo[1] = rq;
   op->run = FcMfmaRun;
   op->kernel_name = "fc_mfma_i8_256x256x128";
   return TVX_OK;

@@ -77,6 +77,36 @@ int BuildRequantTables(uint32_t channels, float in_scale, float w_scale,
   return TVX_OK;
 }
 
+int BuildRequantRecords(const std::vector<int32_t>& mult, const std::vector<int32_t>& shift,
+                        int channels, int alloc, int out_zp, std::vector<int32_t>* records) {
+  int rq = kRqFastNoTie;
+  for (int c = 0; c < channels; ++c) {
+    const int32_t m = mult[c], s = shift[c];
+    if (m == 0) continue;
+    // (zp << t) + 2^30 must stay inside int32
+    if (s < 33 || s - 32 > 20) { rq = kRqGeneric; break; }
+    // a tie needs an accumulator v with v * m = 2^(s-1) (mod 2^s): ctz(v) = s - 1 - ctz(m) <= 31
+    if (__builtin_ctz(static_cast<uint32_t>(m)) >= s - 32) rq = kRqFast;
+  }
+  records->assign(static_cast<size_t>(alloc) * 4, 0);
+  for (int c = 0; c < alloc; ++c) {
+    int32_t m = c < channels ? mult[c] : 0, s = c < channels ? shift[c] : 33;
+    if (m == 0) s = 33;
+    int32_t* q = &(*records)[static_cast<size_t>(c) * 4];
+    q[0] = m;
+    if (rq == kRqGeneric) {
+      q[1] = s;
+    } else {
+      const int t = s - 32;
+      const int ctz = m ? __builtin_ctz(static_cast<uint32_t>(m)) : 0;
+      q[1] = t;
+      q[2] = (1 << (t - 1)) + (out_zp << t);
+      q[3] = ctz == 0 ? -1 : static_cast<int32_t>((uint32_t{1} << (32 - ctz)) - 1);
+    }
+  }
+  return rq;
+}
+
 void ActRange(int out_dtype, float out_scale, int32_t out_zp, int act, int32_t* lo, int32_t* hi) {
   *lo = out_dtype == TVX_U8 ? 0 : -128;
   *hi = out_dtype == TVX_U8 ? 255 : 127;

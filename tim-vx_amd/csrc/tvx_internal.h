@@ -95,7 +95,36 @@ __device__ __forceinline__ int32_t RequantClamp(int32_t acc, int32_t mult, int32
   return static_cast<int32_t>(r);
 }
 
+// ---- 32-bit requantization for MFMA epilogues ----------------------------------
+// When every channel's shift is 32 + t with 1 <= t <= 20, round_half_even(acc * mult
+// / 2^shift) + zp only needs the high half of the product: r = (hi + 2^(t-1) +
+// (zp << t)) >> t rounds half up and adds the zero point; the low half matters on
+// exact ties alone, which are fixed up (or proven impossible at creation).
+// Record per channel: {mult, t (or the full shift in generic mode), rounding
+// constant, mask of the accumulator bits that decide whether the low half is 0}.
+typedef int tvx_v4i __attribute__((ext_vector_type(4)));
+constexpr int kRqGeneric = 0;    // any shift: 64-bit product
+constexpr int kRqFast = 1;       // high half of the product + tie fix-up
+constexpr int kRqFastNoTie = 2;  // additionally no accumulator can land on a tie
+
+template <int RQ>
+__device__ __forceinline__ int Requant8(int v, const tvx_v4i& q, int zp, int lo, int hi) {
+  if (RQ == kRqGeneric) return RequantClamp(v, q[0], q[1], zp, lo, hi);
+  const int h = __mulhi(v, q[0]);
+  int r = (h + q[2]) >> q[1];
+  if (RQ == kRqFast) {
+    const int half = 1 << (q[1] - 1);
+    const bool tie = ((h & (2 * half - 1)) == half) && ((v & q[3]) == 0);
+    if (tie && ((r - zp) & 1)) --r;
+  }
+  return max(lo, min(r, hi));
+}
+
 // ---- host helpers ------------------------------------------------------------
+// Builds the records above for `alloc` channels (the first `channels` from the
+// operator's mult/shift tables, the rest neutral) and returns the flavour.
+int BuildRequantRecords(const std::vector<int32_t>& mult, const std::vector<int32_t>& shift,
+                        int channels, int alloc, int out_zp, std::vector<int32_t>* records);
 // Per-output-channel requantization tables (mult/shift) for a conv / FC.
 int BuildRequantTables(uint32_t channels, float in_scale, float w_scale,
                        const float* w_scales, float out_scale,
