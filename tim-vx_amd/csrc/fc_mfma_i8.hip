@@ -82,22 +82,22 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
     off_w[i] = static_cast<uint32_t>(wr) * static_cast<uint32_t>(a.K) + chunk * 16;
   }
   const bool k_tail = (a.K % TK) != 0;
-  auto dma_tile = [&](int kt, int stage) {
-    int8_t* xs = lds + stage * 2 * kTileBytes + wave * 64 * TK;
-    int8_t* ws = xs + kTileBytes;
+  // piece 2 i moves 8 rows of X, piece 2 i + 1 the same rows of W
+  auto dma_piece = [&](int kt, int stage, int piece) {
+    const int i = piece >> 1;
+    int8_t* dst = lds + stage * 2 * kTileBytes + wave * 64 * TK + i * 1024 + ((piece & 1) ? kTileBytes : 0);
     const int k0 = kt * TK;
+    const bool past = k_tail && k0 + dma_chunk[i & 1] * 16 >= a.K;  // only in the last k-tile
+    // reduction bytes past K: zero for the weights, the int8-domain zero (0x80 before
+    // the re-bias of uint8 activations) for the activations
+    const int8_t* src = (piece & 1) ? (past ? a.zeros : a.w + (off_w[i] + k0))
+                                    : (past ? a.zeros + (X_U8 ? 128 : 0) : a.x + (off_x[i] + k0));
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                     (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+  };
+  auto dma_tile = [&](int kt, int stage) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const bool past = k_tail && k0 + dma_chunk[i & 1] * 16 >= a.K;  // only in the last k-tile
-      // reduction bytes past K: zero for the weights, the int8-domain zero (0x80 before
-      // the re-bias of uint8 activations) for the activations
-      const int8_t* px = past ? a.zeros + (X_U8 ? 128 : 0) : a.x + (off_x[i] + k0);
-      const int8_t* pw = past ? a.zeros : a.w + (off_w[i] + k0);
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)px,
-                                       (__attribute__((address_space(3))) void*)(xs + i * 1024), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)pw,
-                                       (__attribute__((address_space(3))) void*)(ws + i * 1024), 16, 0, 0);
-    }
+    for (int piece = 0; piece < 16; ++piece) dma_piece(kt, stage, piece);
   };
 
   v16i acc[4][4];  // [tn][tm]
@@ -115,15 +115,33 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   const int x_row_off = (wm * 128 + frag_row) * TK, w_row_off = (wn * 128 + frag_row) * TK;
   const int row7 = (frag_row >> 1) & 7;  // fragment tiles start at multiples of 32 rows
 
-  auto load_frags = [&](const int8_t* xs, const int8_t* ws, int kk, v4i* fx, v4i* fw) {
-    const int sw = (((kk * 2 + frag_half) ^ row7) << 4);
+  // Fragment fetches are issued as inline assembly and waited for with explicit
+  // s_waitcnt: the compiler's own wait insertion treats fragments carried across
+  // the loop back-edge conservatively (waits for every LDS operation in flight),
+  // which would serialize the fetch of step kk + 1 with the MFMAs of step kk.
+  const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<size_t>(lds));
+  uint32_t frag_x[4], frag_w[4];  // per k-step: LDS address of this lane's first X / W fragment
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      fx[t] = *reinterpret_cast<const v4i*>(xs + x_row_off + t * 32 * TK + sw);
-      fw[t] = *reinterpret_cast<const v4i*>(ws + w_row_off + t * 32 * TK + sw);
-    }
+  for (int kk = 0; kk < 4; ++kk) {
+    const int sw = (((kk * 2 + frag_half) ^ row7) << 4);
+    frag_x[kk] = lds_base + x_row_off + sw;
+    frag_w[kk] = lds_base + kTileBytes + w_row_off + sw;
+  }
+#define TVX_DS_READ(dst, addr, off) \
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
+  auto load_frags = [&](uint32_t stage_off, int kk, v4i* fx, v4i* fw) {
+    const uint32_t ax = frag_x[kk] + stage_off, aw = frag_w[kk] + stage_off;
+    TVX_DS_READ(fx[0], ax, 0);
+    TVX_DS_READ(fw[0], aw, 0);
+    TVX_DS_READ(fx[1], ax, 32 * TK);
+    TVX_DS_READ(fw[1], aw, 32 * TK);
+    TVX_DS_READ(fx[2], ax, 64 * TK);
+    TVX_DS_READ(fw[2], aw, 64 * TK);
+    TVX_DS_READ(fx[3], ax, 96 * TK);
+    TVX_DS_READ(fw[3], aw, 96 * TK);
   };
-  auto mma = [&](v4i* fx, const v4i* fw) {
+#undef TVX_DS_READ
+  auto prep = [&](v4i* fx) {
     if (X_U8) {
 #pragma unroll
       for (int t = 0; t < 4; ++t) fx[t] ^= static_cast<int>(0x80808080);
@@ -135,11 +153,28 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
         for (int q = 0; q < 4; ++q)
           rowsum[t] = __builtin_amdgcn_sdot4(fx[t][q], 0x01010101, rowsum[t], false);
     }
+  };
+  auto mma = [&](v4i* fx, const v4i* fw) {
+    prep(fx);
 #pragma unroll
     for (int tn = 0; tn < 4; ++tn)
 #pragma unroll
       for (int tm = 0; tm < 4; ++tm)
         acc[tn][tm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[tn], fx[tm], acc[tn][tm], 0, 0, 0);
+  };
+  // the same 16 MFMAs with one DMA instruction of a later tile issued behind each:
+  // a wavefront that issues its DMA back to back sits in the memory pipeline's
+  // issue queue while its matrix core idles
+  auto mma_dma = [&](v4i* fx, const v4i* fw, int dma_kt, int dma_stage) {
+    prep(fx);
+#pragma unroll
+    for (int tn = 0; tn < 4; ++tn)
+#pragma unroll
+      for (int tm = 0; tm < 4; ++tm) {
+        acc[tn][tm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[tn], fx[tm], acc[tn][tm], 0, 0, 0);
+        dma_piece(dma_kt, dma_stage, tn * 4 + tm);
+        __builtin_amdgcn_sched_barrier(0);
+      }
   };
 
   // Steady state of one k-tile (four 32-byte k-steps, 16 MFMAs each): the
@@ -148,33 +183,44 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   // first fragments of the next tile are already on their way while it runs, and
   // the DMA of the tile after next starts as soon as the barrier has freed this stage.
   const int k_tiles = (a.K + TK - 1) / TK;
+  // The loop body is branch-free: past the last tile it re-fetches the last tile
+  // into the stage nobody reads any more, which keeps the hardware wait counters
+  // exact (a conditional block in the loop makes the compiler wait for everything).
+  const int last_tile = k_tiles - 1;
   dma_tile(0, 0);
-  if (k_tiles > 1) dma_tile(1, 1);
-  if (k_tiles > 1) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");  // tile 0 landed (16 newer DMAs may be in flight)
-  else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  dma_tile(min(1, last_tile), 1);
+  asm volatile("s_waitcnt vmcnt(16)" ::: "memory");  // tile 0 landed (16 newer DMAs may be in flight)
   __syncthreads();
   v4i fx0[4], fw0[4], fx1[4], fw1[4];
-  load_frags(lds, lds + kTileBytes, 0, fx0, fw0);
+  load_frags(0, 0, fx0, fw0);
   for (int kt = 0; kt < k_tiles; ++kt) {
     const int stage = kt & 1;
-    const int8_t* xs = lds + stage * 2 * kTileBytes;
-    const int8_t* ws = xs + kTileBytes;
-    load_frags(xs, ws, 1, fx1, fw1);
+    const uint32_t so = stage * 2 * kTileBytes, so_next = (stage ^ 1) * 2 * kTileBytes;
+    // "wait until at most 8 LDS reads are in flight" = the older fragment set has arrived
+    load_frags(so, 1, fx1, fw1);
+    asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
     mma(fx0, fw0);
-    load_frags(xs, ws, 2, fx0, fw0);
+    __builtin_amdgcn_sched_barrier(0);
+    load_frags(so, 2, fx0, fw0);
+    asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
     mma(fx1, fw1);
-    load_frags(xs, ws, 3, fx1, fw1);
+    __builtin_amdgcn_sched_barrier(0);
+    load_frags(so, 3, fx1, fw1);
+    asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
     mma(fx0, fw0);
+    __builtin_amdgcn_sched_barrier(0);
     // all my reads of this stage are done and the next tile's DMA has landed
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
-    if (kt + 2 < k_tiles) dma_tile(kt + 2, stage);
-    if (kt + 1 < k_tiles) {
-      const int8_t* nx = lds + (stage ^ 1) * 2 * kTileBytes;
-      load_frags(nx, nx + kTileBytes, 0, fx0, fw0);
-    }
-    mma(fx1, fw1);
+    load_frags(so_next, 0, fx0, fw0);
+    __builtin_amdgcn_sched_barrier(0);
+    mma_dma(fx1, fw1, min(kt + 2, last_tile), stage);
+    __builtin_amdgcn_sched_barrier(0);
   }
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // no DMA may land in the epilogue's staging tile
   __syncthreads();  // the epilogue reuses the LDS
 
   // ---- epilogue: requantize, stage the int8 tile in LDS, store 16-byte rows ----
