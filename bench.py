@@ -72,6 +72,52 @@ def fc_cfg5(T, rng):
                 bound="mfma", oracle=None)
 
 
+def dw_cfg3a(T, rng):
+    n, c, h, w = 32, 32, 112, 112
+    x = rng.integers(-128, 128, n * c * h * w, dtype=np.int8)
+    wt = rng.integers(-128, 128, c * 9, dtype=np.int8)
+    b = rng.integers(-4096, 4097, c).astype(np.int32)
+    ws = np.exp(rng.uniform(np.log(0.002), np.log(0.05), c)).astype(np.float32)
+    import ctypes as C
+    d = T.Conv2dDesc()
+    d.in_w, d.in_h, d.in_c, d.batch = w, h, c, n
+    d.k_w = d.k_h = 3
+    d.out_w, d.out_h, d.out_c = w, h, c
+    d.stride_w = d.stride_h = d.dilation_w = d.dilation_h = 1
+    d.pad_left = d.pad_top = 1
+    d.multiplier = 1
+    d.in_dtype = d.w_dtype = d.out_dtype = T.I8
+    d.in_scale, d.in_zp = 0.03, 0
+    d.w_scales = ws.ctypes.data_as(C.POINTER(C.c_float))
+    d.out_scale, d.out_zp = 0.08, 0
+    op = T.conv2d_create(d, wt, b)
+    return dict(name="depthwise3x3_i8_per_channel_112x112x32_b32", op=op, inputs=(x,), out_elems=x.size,
+                out_dtype=np.int8, ops=2 * x.size * 9, algo_bytes=2 * x.size + wt.size + 4 * c,
+                bound="hbm", oracle=None)
+
+
+def pw_cfg3b(T, rng):
+    n, c, h, w, oc = 32, 32, 112, 112, 64
+    x = rng.integers(-128, 128, n * c * h * w, dtype=np.int8)
+    wt = rng.integers(-128, 128, oc * c, dtype=np.int8)
+    b = rng.integers(-4096, 4097, oc).astype(np.int32)
+    ws = np.exp(rng.uniform(np.log(0.002), np.log(0.05), oc)).astype(np.float32)
+    import ctypes as C
+    d = T.Conv2dDesc()
+    d.in_w, d.in_h, d.in_c, d.batch = w, h, c, n
+    d.k_w = d.k_h = 1
+    d.out_w, d.out_h, d.out_c = w, h, oc
+    d.stride_w = d.stride_h = d.dilation_w = d.dilation_h = 1
+    d.in_dtype = d.w_dtype = d.out_dtype = T.I8
+    d.in_scale, d.in_zp = 0.08, 0
+    d.w_scales = ws.ctypes.data_as(C.POINTER(C.c_float))
+    d.out_scale, d.out_zp, d.activation = 0.05, 0, T.ACT_RELU6
+    op = T.conv2d_create(d, wt, b)
+    return dict(name="pointwise1x1_i8_per_channel_32to64_112x112_b32_relu6", op=op, inputs=(x,),
+                out_elems=n * oc * h * w, out_dtype=np.int8, ops=2 * n * h * w * c * oc,
+                algo_bytes=x.size + n * oc * h * w + wt.size + 4 * oc, bound="hbm", oracle=None)
+
+
 def time_workload(wl, steps, warmup):
     """Returns (wall ms per step over exactly `steps` steps, mean per-launch kernel ms)."""
     import torch
@@ -175,7 +221,7 @@ def main():
     }
     if not args.no_extra:
         extra = {}
-        for make in (fc_cfg5,):
+        for make in (fc_cfg5, dw_cfg3a, pw_cfg3b):
             w2 = make(T, rng)
             steps2 = max(5, min(args.steps, 50))
             wall2, k2 = time_workload(w2, steps2, min(args.warmup, 5))

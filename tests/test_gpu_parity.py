@@ -254,3 +254,57 @@ def test_conv2d_igemm_shapes(oracle, gi, mode):
     got = TC.gpu_conv2d(x, wt, b, act=1, want_kernel="conv2d_igemm_i8", **kws)
     assert np.array_equal(got, want)
     assert len(np.unique(want)) > 4
+
+
+DW_GRID = [
+    # (n, c, h, w, stride, pad[l,r,t,b])
+    (2, 8, 16, 16, 1, [1, 1, 1, 1]),
+    (1, 5, 9, 12, 1, [1, 1, 1, 1]),
+    (3, 4, 17, 20, 2, [0, 1, 0, 1]),
+    (2, 6, 16, 24, 2, [1, 1, 1, 1]),
+    (1, 3, 10, 8, 1, [0, 0, 0, 0]),
+    (1, 7, 33, 40, 1, [1, 1, 2, 2]),
+]
+
+
+@pytest.mark.parametrize("mode", ["u8", "i8pc", "u8pc"])
+@pytest.mark.parametrize("gi", range(len(DW_GRID)))
+def test_depthwise3x3_shapes(oracle, gi, mode):
+    n, c, h, w, s, pad = DW_GRID[gi]
+    rng = np.random.default_rng(3000 + gi)
+    x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=0, kh=3, kw=3, stride=[s, s], dil=[1, 1],
+                              pad=pad, mult=1, mode=mode)
+    fast = kws["out_shape"][0] % 4 == 0
+    for act in (0, 2):
+        want = oracle.conv2d(x, wt, b, act=act, **kws)
+        got = TC.gpu_conv2d(x, wt, b, act=act, want_kernel="dwconv3x3_i8" if fast else "conv2d_generic", **kws)
+        assert np.array_equal(got, want)
+    assert len(np.unique(want)) > 4
+
+
+def test_depthwise_then_pointwise_full_size(oracle):
+    """int8 per-channel block: depthwise 3x3 on 112x112x32 at batch 32, then pointwise 1x1 32->64
+    with fused ReLU6; both stages whole-tensor against the oracle."""
+    rng = np.random.default_rng(0x73)
+    n, c, h, w, oc = 32, 32, 112, 112, 64
+    x = rng.integers(-128, 128, n * c * h * w, dtype=np.int8)
+    wd = rng.integers(-128, 128, c * 9, dtype=np.int8)
+    bd = rng.integers(-4096, 4097, c).astype(np.int32)
+    sd = np.exp(rng.uniform(np.log(0.002), np.log(0.05), c)).astype(np.float32)
+    kd = dict(in_shape=[w, h, c, n], w_shape=[3, 3, c, 1], out_shape=[w, h, c, n], stride=[1, 1],
+              dilation=[1, 1], pad_left=1, pad_top=1, multiplier=1, in_dtype=1, w_dtype=1, out_dtype=1,
+              in_q=(0.03, 0), w_q=(1.0, 0, sd), out_q=(0.08, 0))
+    mid_want = oracle.conv2d(x, wd, bd, **kd)
+    mid = TC.gpu_conv2d(x, wd, bd, want_kernel="dwconv3x3_i8", **kd)
+    assert np.array_equal(mid, mid_want)
+    assert len(np.unique(mid)) > 100
+    wp = rng.integers(-128, 128, oc * c, dtype=np.int8)
+    bp = rng.integers(-4096, 4097, oc).astype(np.int32)
+    sp = np.exp(rng.uniform(np.log(0.002), np.log(0.05), oc)).astype(np.float32)
+    kp = dict(in_shape=[w, h, c, n], w_shape=[1, 1, c, oc], out_shape=[w, h, oc, n], stride=[1, 1],
+              dilation=[1, 1], pad_left=0, pad_top=0, multiplier=0, in_dtype=1, w_dtype=1, out_dtype=1,
+              in_q=(0.08, 0), w_q=(1.0, 0, sp), out_q=(0.05, 0), act=2)
+    out_want = oracle.conv2d(mid, wp, bp, **kp)
+    out = TC.gpu_conv2d(mid, wp, bp, want_kernel="conv2d_igemm_i8", **kp)
+    assert np.array_equal(out, out_want)
+    assert out.min() == 0 and out.max() == 120  # ReLU6 at scale 0.05

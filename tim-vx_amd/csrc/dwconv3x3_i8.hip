@@ -1,0 +1,219 @@
+// Depthwise 3x3 quantized convolution (multiplier 1) in WHCN: every (image,
+// channel) plane is an independent 2-D stencil, so the kernel streams planes
+// through registers at memory speed and never touches the matrix cores.
+//
+// A thread owns a 4-column x 4-row patch of one plane's output; it issues all
+// loads of the input rows behind the patch up front: per row the dword(s) under
+// its columns plus one dword on each side (neighbouring threads load the same
+// lines: L1 hits), cuts the four 3-byte windows out of them with v_alignbyte and
+// feeds each window to three v_dot4 (one per kernel row, weights of a kernel row
+// packed in one register). Rows above / below the image and columns left / right
+// of it read as the input zero point, so the zero-point expansion
+//   sum (x - zx)(w - zw) = sum xs ws - zws * Sx - zxs * Sw + 9 zxs zws
+// only needs the window sum Sx when the weight zero point is non-zero (one
+// more v_dot4 with ones per window and kernel row); the channel constants are
+// folded into the bias at creation. Requantization is the exact fixed-point
+// one of the other kernels; four results are packed into one dword store.
+#include <algorithm>
+
+#include "variants.h"
+
+namespace tvx {
+namespace {
+
+constexpr int kThreads = 256;
+
+struct DwArgs {
+  const uint8_t* x;
+  uint8_t* y;
+  const int32_t* wpk;    // per channel: 3 dwords, kernel row ky = bytes (w[ky][0], w[ky][1], w[ky][2], 0) int8
+  const int32_t* biasf;  // per channel: bias - zxs * Sw + 9 zxs zws
+  const tvx_v4i* rq;     // per channel requantization record
+  int C, H, W, OH, OW;
+  int pad_t, pad_l;
+  int ow4;               // output dwords per row
+  int rg_per_block;      // row groups (of kRowsPerThread output rows) per workgroup
+  int xor_mask, pad_fill, zws, out_zp, lo, hi;
+};
+
+// bytes [idx, idx + 4) of the little-endian byte array formed by arr[0], arr[1], ...
+template <int IDX, int N>
+__device__ __forceinline__ int Window(const int (&arr)[N]) {
+  constexpr int d = IDX / 4, sh = IDX % 4;
+  static_assert(d + (sh ? 1 : 0) < N, "window outside the loaded dwords");
+  if (sh == 0) return arr[d];
+  return __builtin_amdgcn_alignbyte(arr[d + 1], arr[d], sh);
+}
+
+constexpr int kRowsPerThread = 4;  // output rows a thread produces
+
+// S = stride (1 or 2, both directions), PL = left padding (0 or 1)
+template <int S, int PL, bool BOXSUM, int RQ>
+__global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
+  const int plane = blockIdx.x;
+  const int c = plane % a.C;
+  const int tid = threadIdx.x;
+  const int rgl = tid / a.ow4;
+  const int w4 = tid - rgl * a.ow4;
+  const int oh0 = (blockIdx.y * a.rg_per_block + rgl) * kRowsPerThread;
+  if (rgl >= a.rg_per_block || oh0 >= a.OH) return;
+
+  const uint8_t* xp = a.x + static_cast<size_t>(plane) * a.H * a.W;
+  uint8_t* yp = a.y + static_cast<size_t>(plane) * a.OH * a.OW;
+  const int wk0 = a.wpk[c * 3 + 0], wk1 = a.wpk[c * 3 + 1], wk2 = a.wpk[c * 3 + 2];
+  const int bias = a.biasf[c];
+  const tvx_v4i q = a.rq[c];
+  const int in_dwords = a.W / 4;
+
+  // input dwords under this thread's four outputs: S of them, starting at S * w4;
+  // the byte array of a row is {left neighbour, own dwords, right neighbour}
+  constexpr int kOwn = S;
+  constexpr int kRows = S * (kRowsPerThread - 1) + 3;  // input rows behind the thread's output rows
+  const int d0 = S * w4;
+  const int ih0 = oh0 * S - a.pad_t;
+
+  // all loads of the thread are issued before the first use
+  int raw[kRows][kOwn + 2];
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) {
+    const int ih = ih0 + r;
+    const bool inside = ih >= 0 && ih < a.H;
+    const int* row = reinterpret_cast<const int*>(xp + static_cast<size_t>(inside ? ih : 0) * a.W);
+#pragma unroll
+    for (int i = 0; i < kOwn + 2; ++i) {
+      const int d = d0 - 1 + i;
+      const bool ok = inside && d >= 0 && d < in_dwords;
+      const int v = row[ok ? d : 0];
+      raw[r][i] = ok ? v ^ a.xor_mask : a.pad_fill;
+    }
+  }
+  int win[kRows][4];
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) {
+    // output i of this thread reads input bytes [S i - PL, S i - PL + 3) of its own span
+    win[r][0] = Window<4 + S * 0 - PL>(raw[r]);
+    win[r][1] = Window<4 + S * 1 - PL>(raw[r]);
+    win[r][2] = Window<4 + S * 2 - PL>(raw[r]);
+    win[r][3] = Window<4 + S * 3 - PL>(raw[r]);
+  }
+#pragma unroll
+  for (int o = 0; o < kRowsPerThread; ++o) {
+    if (oh0 + o >= a.OH) break;
+    uint32_t packed = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int acc = bias;
+      acc = __builtin_amdgcn_sdot4(win[S * o][i], wk0, acc, false);
+      acc = __builtin_amdgcn_sdot4(win[S * o + 1][i], wk1, acc, false);
+      acc = __builtin_amdgcn_sdot4(win[S * o + 2][i], wk2, acc, false);
+      if (BOXSUM) {
+        int sx = __builtin_amdgcn_sdot4(win[S * o][i], 0x00010101, 0, false);
+        sx = __builtin_amdgcn_sdot4(win[S * o + 1][i], 0x00010101, sx, false);
+        sx = __builtin_amdgcn_sdot4(win[S * o + 2][i], 0x00010101, sx, false);
+        acc -= a.zws * sx;
+      }
+      packed |= static_cast<uint32_t>(Requant8<RQ>(acc, q, a.out_zp, a.lo, a.hi) & 0xff) << (8 * i);
+    }
+    *reinterpret_cast<uint32_t*>(yp + static_cast<size_t>(oh0 + o) * a.OW + w4 * 4) = packed;
+  }
+}
+
+struct Plan {
+  DwArgs a;
+  int stride, pad_l, boxsum, rq;
+  dim3 grid;
+};
+
+template <int S, int PL, bool BOXSUM>
+void LaunchRq(const Plan* p, const DwArgs& a, hipStream_t st) {
+  const dim3 block(kThreads);
+  if (p->rq == kRqFastNoTie) hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqFastNoTie>), p->grid, block, 0, st, a);
+  else if (p->rq == kRqFast) hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqFast>), p->grid, block, 0, st, a);
+  else hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqGeneric>), p->grid, block, 0, st, a);
+}
+
+template <int S, int PL>
+void LaunchBox(const Plan* p, const DwArgs& a, hipStream_t st) {
+  if (p->boxsum) LaunchRq<S, PL, true>(p, a, st);
+  else LaunchRq<S, PL, false>(p, a, st);
+}
+
+int DwRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
+  const Plan* p = reinterpret_cast<const Plan*>(op->host_blob.data());
+  DwArgs a = p->a;
+  a.x = static_cast<const uint8_t*>(in0);
+  a.y = static_cast<uint8_t*>(out);
+  if (p->stride == 1) {
+    if (p->pad_l) LaunchBox<1, 1>(p, a, st); else LaunchBox<1, 0>(p, a, st);
+  } else {
+    if (p->pad_l) LaunchBox<2, 1>(p, a, st); else LaunchBox<2, 0>(p, a, st);
+  }
+  TVX_HIP_CHECK(hipGetLastError());
+  return TVX_OK;
+}
+
+}  // namespace
+
+// Claims quantized depthwise 3x3, multiplier 1, dilation 1, stride 1 or 2 (both
+// directions), constant weights, row lengths that are multiples of four.
+int DwConv3x3Setup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const void* bias_host) {
+  if (!op->quantized || !w_host || d->multiplier != 1) return TVX_E_UNSUPPORTED;
+  if (d->k_w != 3 || d->k_h != 3 || d->dilation_w != 1 || d->dilation_h != 1) return TVX_E_UNSUPPORTED;
+  if (d->stride_w != d->stride_h || (d->stride_w != 1 && d->stride_w != 2)) return TVX_E_UNSUPPORTED;
+  if (d->pad_left > 1 || (d->in_w & 3) || (d->out_w & 3)) return TVX_E_UNSUPPORTED;
+  const int S = d->stride_w;
+  const int ow4 = d->out_w / 4;
+  if (ow4 > kThreads) return TVX_E_UNSUPPORTED;
+  // every output's window must end inside {own dwords, right neighbour}
+  if (static_cast<uint32_t>((d->out_w - 1) * S + 2) >= d->in_w + d->pad_left + 4) return TVX_E_UNSUPPORTED;
+  const bool x_u8 = d->in_dtype == TVX_U8, w_u8 = d->w_dtype == TVX_U8;
+  const int zxs = d->in_zp - (x_u8 ? 128 : 0);
+  const int zws = op->w_zp - (w_u8 ? 128 : 0);
+  if (zxs < -128 || zxs > 127) return TVX_E_UNSUPPORTED;
+  const int C = d->in_c;
+  std::vector<int32_t> wpk(static_cast<size_t>(C) * 3), biasf(C);
+  const uint8_t* src = static_cast<const uint8_t*>(w_host);
+  const int32_t* b = static_cast<const int32_t*>(bias_host);
+  for (int c = 0; c < C; ++c) {
+    int64_t sw = 0;
+    for (int ky = 0; ky < 3; ++ky) {
+      uint32_t pk = 0;
+      for (int kx = 0; kx < 3; ++kx) {
+        const uint8_t raw = src[static_cast<size_t>(c) * 9 + ky * 3 + kx];
+        const int8_t v = static_cast<int8_t>(w_u8 ? raw ^ 0x80 : raw);
+        pk |= static_cast<uint32_t>(static_cast<uint8_t>(v)) << (8 * kx);
+        sw += v;
+      }
+      wpk[static_cast<size_t>(c) * 3 + ky] = static_cast<int32_t>(pk);
+    }
+    const int64_t v = (b ? b[c] : 0) - static_cast<int64_t>(zxs) * sw + 9ll * zxs * zws;
+    biasf[c] = static_cast<int32_t>(static_cast<uint32_t>(v));
+  }
+  std::vector<int32_t> rqt;
+  const int rq = BuildRequantRecords(op->h_mult, op->h_shift, C, C, d->out_zp, &rqt);
+  int s = op->packed.Upload(wpk.data(), wpk.size() * 4);
+  if (s == TVX_OK) s = op->aux.Upload(biasf.data(), biasf.size() * 4);
+  if (s == TVX_OK) s = op->aux2.Upload(rqt.data(), rqt.size() * 4);
+  if (s != TVX_OK) return s;
+  Plan p{};
+  DwArgs& a = p.a;
+  a.wpk = op->packed.as<int32_t>();
+  a.biasf = op->aux.as<int32_t>();
+  a.rq = op->aux2.as<tvx_v4i>();
+  a.C = C; a.H = d->in_h; a.W = d->in_w; a.OH = d->out_h; a.OW = d->out_w;
+  a.pad_t = d->pad_top; a.pad_l = d->pad_left;
+  a.ow4 = ow4;
+  a.rg_per_block = std::max(1, kThreads / ow4);
+  const int row_groups = (static_cast<int>(d->out_h) + kRowsPerThread - 1) / kRowsPerThread;
+  a.xor_mask = x_u8 ? static_cast<int>(0x80808080u) : 0;
+  a.pad_fill = static_cast<int>(static_cast<uint32_t>(zxs & 0xff) * 0x01010101u);
+  a.zws = zws; a.out_zp = d->out_zp; a.lo = op->act_lo; a.hi = op->act_hi;
+  p.stride = S; p.pad_l = d->pad_left; p.boxsum = zws != 0; p.rq = rq;
+  p.grid = dim3(d->batch * C, (row_groups + a.rg_per_block - 1) / a.rg_per_block);
+  op->host_blob.assign(reinterpret_cast<const uint8_t*>(&p), reinterpret_cast<const uint8_t*>(&p) + sizeof(p));
+  op->run = DwRun;
+  op->kernel_name = "dwconv3x3_i8";
+  return TVX_OK;
+}
+
+}  // namespace tvx

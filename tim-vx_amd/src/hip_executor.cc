@@ -1,0 +1,364 @@
+// Executor of a compiled tim::vx graph on the GPU, reaching it only through the
+// C ABI of include/tvx_hip.h (this file needs no HIP header).
+//
+// Realize() is the counterpart of vsi_nn_SetupGraph's compute_node pass plus
+// vxVerifyGraph (src/tim/vx/internal/src/vsi_nn_graph.c:389-467,1591-1603): every
+// operator becomes one tvx_op (the vx_node analogue), constants are uploaded and
+// re-packed, and Conv2d / FullyConnected followed by Relu / Relu6 through a
+// single-consumer TRANSIENT tensor with the same quantization are fused into the
+// producer's epilogue - the fusion the closed driver performs itself.
+// Execute() is vsi_nn_RunGraph -> vxProcessGraph (vsi_nn_graph.c:1605-1639):
+// inputs go host -> device, operators run in order on one stream, outputs come
+// back, and the call returns when everything is visible to the host.
+#include <cmath>
+#include <cstring>
+#include <map>
+
+#include "runtime.h"
+#include "tvx_hip.h"
+
+namespace tim {
+namespace vx {
+namespace {
+
+int DtypeCode(DataType t) {
+  switch (t) {
+    case DataType::UINT8: return TVX_U8;
+    case DataType::INT8: return TVX_I8;
+    case DataType::FLOAT16: return TVX_F16;
+    case DataType::FLOAT32: return TVX_F32;
+    default: return -1;
+  }
+}
+
+float ScaleOf(const TensorSpec& s) {
+  return s.quantization_.Scales().empty() ? 1.0f : s.quantization_.Scales()[0];
+}
+int32_t ZpOf(const TensorSpec& s) {
+  return s.quantization_.ZeroPoints().empty() ? 0 : s.quantization_.ZeroPoints()[0];
+}
+bool IsQuantSpec(const TensorSpec& s) {
+  return s.datatype_ == DataType::UINT8 || s.datatype_ == DataType::INT8;
+}
+
+struct Step {
+  tvx_op* op = nullptr;
+  TensorImpl* in0 = nullptr;
+  TensorImpl* in1 = nullptr;  // run-time weights / second Add operand
+  TensorImpl* out = nullptr;
+  std::string name;
+};
+
+class HipExecutor : public Executor {
+ public:
+  ~HipExecutor() override {
+    for (auto& s : steps_) tvx_op_destroy(s.op);
+    for (auto& kv : owned_) tvx_free(kv.second);
+    if (stream_) tvx_stream_destroy(stream_);
+  }
+
+  bool Realize(GraphImpl* graph) override {
+    if (tvx_device_count() <= 0) {
+      VSILOGE("no GPU: this runtime has no CPU execution path");
+      return false;
+    }
+    if (tvx_stream_create(&stream_) != TVX_OK) return Fail("stream");
+    // ---- activation fusion plan ------------------------------------------------
+    std::map<Operation*, Operation*> fused_act;  // producer -> activation folded into it
+    std::map<Operation*, bool> skipped;
+    for (Operation* op : graph->sorted_ops_) {
+      OpImpl* im = op->impl().get();
+      if (im->kind_ != OpKind::CONV2D && im->kind_ != OpKind::FCL) continue;
+      auto mid = im->outputs_tensor_[0];
+      if (!(mid->GetSpec().attr_ & TensorAttribute::TRANSIENT)) continue;
+      auto consumers = graph->GetConsumersOp(mid);
+      if (consumers.size() != 1) continue;
+      OpImpl* act = consumers[0]->impl().get();
+      if (act->kind_ != OpKind::RELU && act->kind_ != OpKind::RELU6) continue;
+      const TensorSpec &ms = mid->GetSpec(), &os = act->outputs_tensor_[0]->GetSpec();
+      if (ms.datatype_ != os.datatype_) continue;
+      if (IsQuantSpec(ms) && (ScaleOf(ms) != ScaleOf(os) || ZpOf(ms) != ZpOf(os))) continue;
+      fused_act[op] = consumers[0].get();
+      skipped[consumers[0].get()] = true;
+    }
+    // ---- device storage: one buffer per tensor, Reshape outputs alias their input --
+    for (Operation* op : graph->sorted_ops_) {
+      OpImpl* im = op->impl().get();
+      for (auto& t : im->inputs_tensor_)
+        if (!t->IsPlaceHolder() && !EnsureBuffer(static_cast<TensorImpl*>(t.get()))) return false;
+      if (im->kind_ == OpKind::RESHAPE) {
+        dev_[static_cast<TensorImpl*>(im->outputs_tensor_[0].get())] =
+            dev_[static_cast<TensorImpl*>(im->inputs_tensor_[0].get())];
+        continue;
+      }
+      for (auto& t : im->outputs_tensor_)
+        if (!EnsureBuffer(static_cast<TensorImpl*>(t.get()))) return false;
+    }
+    // ---- operators ---------------------------------------------------------------
+    for (Operation* op : graph->sorted_ops_) {
+      if (skipped.count(op)) continue;
+      OpImpl* im = op->impl().get();
+      if (im->attrs_.overflow != OverflowPolicy::SATURATE || im->attrs_.rounding != RoundingPolicy::RTNE) {
+        VSILOGE("%s: only SATURATE + RTNE rounding policy is implemented", OpKindName(im->kind_));
+        return false;
+      }
+      int act = TVX_ACT_NONE;
+      TensorImpl* out = static_cast<TensorImpl*>(im->outputs_tensor_[0].get());
+      auto f = fused_act.find(op);
+      if (f != fused_act.end()) {
+        OpImpl* a = f->second->impl().get();
+        act = a->kind_ == OpKind::RELU ? TVX_ACT_RELU : TVX_ACT_RELU6;
+        out = static_cast<TensorImpl*>(a->outputs_tensor_[0].get());
+      }
+      bool ok = true;
+      switch (im->kind_) {
+        case OpKind::CONV2D: ok = AddConv(im, out, act); break;
+        case OpKind::FCL: ok = AddFc(im, out, act); break;
+        case OpKind::POOL: ok = AddPool(im, out); break;
+        case OpKind::RELU: ok = AddActivation(im, out, TVX_ACT_RELU); break;
+        case OpKind::RELU6: ok = AddActivation(im, out, TVX_ACT_RELU6); break;
+        case OpKind::ADD: ok = AddAdd(im, out); break;
+        case OpKind::SOFTMAX: ok = AddSoftmax(im, out); break;
+        case OpKind::RESHAPE: break;  // aliased
+      }
+      if (!ok) return false;
+    }
+    // constants that are read at run time (weights bound as non-constant tensors are
+    // uploaded in Execute); constant activations are uploaded once here
+    for (auto& kv : dev_) {
+      TensorImpl* t = kv.first;
+      if (t->IsConstTensor() && t->HostData() && owned_.count(t)) {
+        if (tvx_memcpy_h2d(kv.second, t->HostData(), t->HostBytes(), stream_) != TVX_OK) return Fail("upload");
+        t->host_dirty_ = false;
+      }
+    }
+    return tvx_stream_synchronize(stream_) == TVX_OK || Fail("sync");
+  }
+
+  bool Execute(GraphImpl* graph) override {
+    // host -> device: every host-visible non-output tensor whose host image changed
+    for (auto& kv : dev_) {
+      TensorImpl* t = kv.first;
+      if (!owned_.count(t) || (t->spec_.attr_ & TensorAttribute::OUTPUT)) continue;
+      if (t->host_dirty_ && t->HostData()) {
+        if (tvx_memcpy_h2d(kv.second, t->HostData(), t->HostBytes(), stream_) != TVX_OK) return Fail("input upload");
+        t->host_dirty_ = false;
+      }
+    }
+    for (auto& s : steps_) {
+      const int st = tvx_op_run(s.op, dev_[s.in0], s.in1 ? dev_[s.in1] : nullptr, dev_[s.out], stream_);
+      if (st != TVX_OK) {
+        VSILOGE("%s failed: %s", s.name.c_str(), tvx_last_error());
+        return false;
+      }
+    }
+    for (auto& t : graph->outputs_tensor_) {
+      TensorImpl* ti = static_cast<TensorImpl*>(t.get());
+      auto it = dev_.find(ti);
+      if (it == dev_.end()) continue;  // an OUTPUT tensor no operator writes
+      ti->EnsureHostBuffer();
+      if (tvx_memcpy_d2h(ti->HostData(), it->second, ti->HostBytes(), stream_) != TVX_OK) return Fail("output download");
+    }
+    return tvx_stream_synchronize(stream_) == TVX_OK || Fail("sync");
+  }
+
+ private:
+  bool Fail(const char* what) {
+    VSILOGE("%s: %s", what, tvx_last_error());
+    return false;
+  }
+
+  bool EnsureBuffer(TensorImpl* t) {
+    if (dev_.count(t)) return true;
+    void* p = nullptr;
+    if (tvx_malloc(&p, t->HostBytes() ? t->HostBytes() : 16) != TVX_OK) return Fail("device allocation");
+    dev_[t] = p;
+    owned_[t] = p;
+    return true;
+  }
+
+  void Push(tvx_op* op, OpImpl* im, TensorImpl* in0, TensorImpl* in1, TensorImpl* out) {
+    Step s;
+    s.op = op;
+    s.in0 = in0;
+    s.in1 = in1;
+    s.out = out;
+    s.name = std::string(OpKindName(im->kind_)) + " (" + tvx_op_kernel_name(op) + ")";
+    VSILOGI("uid %u -> %s", im->uid_, s.name.c_str());
+    steps_.push_back(s);
+  }
+
+  // Weight quantization -> descriptor fields; per-channel scales stay alive in `scales`.
+  static void WeightQuant(const TensorSpec& w, float* scale, int32_t* zp, const float** scales) {
+    *scales = nullptr;
+    *scale = 1.0f;
+    *zp = 0;
+    if (w.quantization_.Type() == QuantType::SYMMETRIC_PER_CHANNEL) {
+      *scales = w.quantization_.Scales().data();
+    } else if (w.quantization_.Type() == QuantType::ASYMMETRIC) {
+      *scale = ScaleOf(w);
+      *zp = ZpOf(w);
+    }
+  }
+
+  bool AddConv(OpImpl* im, TensorImpl* out, int act) {
+    TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
+    TensorImpl* w = static_cast<TensorImpl*>(im->inputs_tensor_[1].get());
+    TensorImpl* b = im->inputs_tensor_.size() > 2 && !im->inputs_tensor_[2]->IsPlaceHolder()
+                        ? static_cast<TensorImpl*>(im->inputs_tensor_[2].get()) : nullptr;
+    const OpAttrs& a = im->attrs_;
+    const ShapeType &xs = x->spec_.shape_, &ws = w->spec_.shape_, &os = out->spec_.shape_;
+    tvx_conv2d_desc d{};
+    d.in_w = xs[0]; d.in_h = xs[1]; d.in_c = xs[2]; d.batch = xs[3];
+    d.k_w = ws[0]; d.k_h = ws[1];
+    d.out_w = os[0]; d.out_h = os[1]; d.out_c = os[2];
+    d.stride_w = a.stride[0]; d.stride_h = a.stride[1];
+    d.dilation_w = a.dilation[0]; d.dilation_h = a.dilation[1];
+    d.pad_left = a.pad[0]; d.pad_top = a.pad[2];
+    d.multiplier = a.multiplier;
+    d.in_dtype = DtypeCode(x->spec_.datatype_);
+    d.w_dtype = DtypeCode(w->spec_.datatype_);
+    d.out_dtype = DtypeCode(out->spec_.datatype_);
+    d.in_scale = ScaleOf(x->spec_); d.in_zp = ZpOf(x->spec_);
+    WeightQuant(w->spec_, &d.w_scale, &d.w_zp, &d.w_scales);
+    d.out_scale = ScaleOf(out->spec_); d.out_zp = ZpOf(out->spec_);
+    d.activation = act;
+    if (b && !b->IsConstTensor()) {
+      VSILOGE("CONV2D: a run-time bias tensor is not supported");
+      return false;
+    }
+    const bool const_w = w->IsConstTensor() && w->HostData();
+    tvx_op* op = nullptr;
+    if (tvx_conv2d_create(&d, const_w ? w->HostData() : nullptr, b ? b->HostData() : nullptr, &op) != TVX_OK)
+      return Fail("tvx_conv2d_create");
+    Push(op, im, x, const_w ? nullptr : w, out);
+    return true;
+  }
+
+  bool AddFc(OpImpl* im, TensorImpl* out, int act) {
+    TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
+    TensorImpl* w = static_cast<TensorImpl*>(im->inputs_tensor_[1].get());
+    TensorImpl* b = im->inputs_tensor_.size() > 2 && !im->inputs_tensor_[2]->IsPlaceHolder()
+                        ? static_cast<TensorImpl*>(im->inputs_tensor_[2].get()) : nullptr;
+    const ShapeType& xs = x->spec_.shape_;
+    uint64_t k = 1, m = 1;
+    for (uint32_t i = 0; i <= im->attrs_.axis; ++i) k *= xs[i];
+    for (size_t i = im->attrs_.axis + 1; i < xs.size(); ++i) m *= xs[i];
+    tvx_fc_desc d{};
+    d.m = static_cast<uint32_t>(m);
+    d.k = static_cast<uint32_t>(k);
+    d.n = w->spec_.shape_.back();
+    d.in_dtype = DtypeCode(x->spec_.datatype_);
+    d.w_dtype = DtypeCode(w->spec_.datatype_);
+    d.out_dtype = DtypeCode(out->spec_.datatype_);
+    d.in_scale = ScaleOf(x->spec_); d.in_zp = ZpOf(x->spec_);
+    WeightQuant(w->spec_, &d.w_scale, &d.w_zp, &d.w_scales);
+    d.out_scale = ScaleOf(out->spec_); d.out_zp = ZpOf(out->spec_);
+    d.activation = act;
+    if (b && !b->IsConstTensor()) {
+      VSILOGE("FCL: a run-time bias tensor is not supported");
+      return false;
+    }
+    const bool const_w = w->IsConstTensor() && w->HostData();
+    tvx_op* op = nullptr;
+    if (tvx_fully_connected_create(&d, const_w ? w->HostData() : nullptr, b ? b->HostData() : nullptr, &op) != TVX_OK)
+      return Fail("tvx_fully_connected_create");
+    Push(op, im, x, const_w ? nullptr : w, out);
+    return true;
+  }
+
+  bool AddPool(OpImpl* im, TensorImpl* out) {
+    TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
+    const OpAttrs& a = im->attrs_;
+    const ShapeType &xs = x->spec_.shape_, &os = out->spec_.shape_;
+    tvx_pool2d_desc d{};
+    if (a.pool_1d) {  // {W, C, N} viewed as {W, 1, C, N}
+      d.in_w = xs[0]; d.in_h = 1; d.channels = xs[1]; d.batch = xs[2];
+      d.out_w = os[0]; d.out_h = 1;
+    } else {
+      d.in_w = xs[0]; d.in_h = xs[1]; d.channels = xs[2]; d.batch = xs[3];
+      d.out_w = os[0]; d.out_h = os[1];
+    }
+    d.k_w = a.ksize[0]; d.k_h = a.pool_1d ? 1 : a.ksize[1];
+    d.stride_w = a.stride[0] ? a.stride[0] : 1;
+    d.stride_h = a.pool_1d ? 1 : (a.stride[1] ? a.stride[1] : 1);
+    d.pad_left = a.pad[0]; d.pad_top = a.pool_1d ? 0 : a.pad[2];
+    d.pool_type = static_cast<int>(a.pool_type);
+    d.dtype = DtypeCode(x->spec_.datatype_);
+    d.in_scale = ScaleOf(x->spec_); d.in_zp = ZpOf(x->spec_);
+    d.out_scale = ScaleOf(out->spec_); d.out_zp = ZpOf(out->spec_);
+    tvx_op* op = nullptr;
+    if (tvx_pool2d_create(&d, &op) != TVX_OK) return Fail("tvx_pool2d_create");
+    Push(op, im, x, nullptr, out);
+    return true;
+  }
+
+  bool AddActivation(OpImpl* im, TensorImpl* out, int act) {
+    TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
+    if (x->spec_.datatype_ != out->spec_.datatype_) {
+      VSILOGE("activation: input and output data types differ");
+      return false;
+    }
+    tvx_eltwise_desc d{};
+    d.count = static_cast<uint64_t>(x->spec_.GetElementNum());
+    d.dtype = DtypeCode(x->spec_.datatype_);
+    d.activation = act;
+    d.a_scale = ScaleOf(x->spec_); d.a_zp = ZpOf(x->spec_);
+    d.out_scale = ScaleOf(out->spec_); d.out_zp = ZpOf(out->spec_);
+    tvx_op* op = nullptr;
+    if (tvx_activation_create(&d, &op) != TVX_OK) return Fail("tvx_activation_create");
+    Push(op, im, x, nullptr, out);
+    return true;
+  }
+
+  bool AddAdd(OpImpl* im, TensorImpl* out) {
+    TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
+    TensorImpl* z = static_cast<TensorImpl*>(im->inputs_tensor_[1].get());
+    if (x->spec_.datatype_ != z->spec_.datatype_ || x->spec_.datatype_ != out->spec_.datatype_) {
+      VSILOGE("ADD: operand data types differ");
+      return false;
+    }
+    tvx_eltwise_desc d{};
+    d.count = static_cast<uint64_t>(x->spec_.GetElementNum());
+    d.dtype = DtypeCode(x->spec_.datatype_);
+    d.a_scale = ScaleOf(x->spec_); d.a_zp = ZpOf(x->spec_);
+    d.b_scale = ScaleOf(z->spec_); d.b_zp = ZpOf(z->spec_);
+    d.out_scale = ScaleOf(out->spec_); d.out_zp = ZpOf(out->spec_);
+    tvx_op* op = nullptr;
+    if (tvx_add_create(&d, &op) != TVX_OK) return Fail("tvx_add_create");
+    Push(op, im, x, z, out);
+    return true;
+  }
+
+  bool AddSoftmax(OpImpl* im, TensorImpl* out) {
+    TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
+    if (im->attrs_.sm_axis != 0 || out->spec_.datatype_ != DataType::FLOAT32) {
+      VSILOGE("SOFTMAX: only axis 0 with a FLOAT32 output is implemented");
+      return false;
+    }
+    tvx_softmax_desc d{};
+    d.channels = x->spec_.shape_[0];
+    d.rows = static_cast<uint64_t>(x->spec_.GetElementNum()) / d.channels;
+    d.beta = im->attrs_.beta;
+    d.in_dtype = DtypeCode(x->spec_.datatype_);
+    d.in_scale = ScaleOf(x->spec_); d.in_zp = ZpOf(x->spec_);
+    tvx_op* op = nullptr;
+    if (tvx_softmax_create(&d, &op) != TVX_OK) return Fail("tvx_softmax_create");
+    Push(op, im, x, nullptr, out);
+    return true;
+  }
+
+  void* stream_ = nullptr;
+  std::vector<Step> steps_;
+  std::map<TensorImpl*, void*> dev_;    // tensor -> device pointer (possibly an alias)
+  std::map<TensorImpl*, void*> owned_;  // tensors that own their buffer
+};
+
+}  // namespace
+
+std::unique_ptr<Executor> CreateExecutor() {
+  return std::unique_ptr<Executor>(new HipExecutor());
+}
+
+}  // namespace vx
+}  // namespace tim
