@@ -238,3 +238,65 @@ def run_case(case):
                       pad_top=a["pad"][2], pool_type=POOL[a["pool_type"]],
                       dtype=DTYPE_CODE[x["dtype"]], in_q=(s, z), out_q=(so, zo))
     raise NotImplementedError(op["kind"])
+
+
+def run_graph(graph, keep_all=False):
+    """Interpret a multi-operator graph description operator by operator (no fusion): every
+    operator's result is quantized to its own output tensor before the next one reads it,
+    which is what the reference's graph semantics prescribe (each vx node writes a tensor).
+    Tensors need resolved shapes and explicit pads. Returns the flat output array (or the
+    dict of all tensors' values)."""
+    ts = {t["id"]: t for t in graph["tensors"]}
+    val = {}
+    for t in graph["tensors"]:
+        if t["data"] is not None:
+            d = t["data"]
+            val[t["id"]] = (expand(d, t["dtype"]) if isinstance(d, (list, dict))
+                            else np.ascontiguousarray(np.asarray(d), dtype=NP_DTYPE[t["dtype"]]).reshape(-1))
+    for o in graph["ops"]:
+        a = o["attrs"]
+        ins = [ts[i] if i >= 0 else None for i in o["inputs"]]
+        out = ts[o["outputs"][0]]
+        k = o["kind"]
+        x = ins[0]
+        s, z, _ = _q(x["quant"])
+        so, zo, _ = _q(out["quant"])
+        xv = val[x["id"]]
+        if k == "CONV2D":
+            w = ins[1]
+            bias = val[ins[2]["id"]] if len(ins) > 2 and ins[2] is not None else None
+            y = conv2d(xv, val[w["id"]], bias, in_shape=x["shape"], w_shape=w["shape"],
+                       out_shape=out["shape"], stride=a["stride"], dilation=a["dilation"],
+                       pad_left=a["pad"][0], pad_top=a["pad"][2], multiplier=a["multiplier"],
+                       in_dtype=DTYPE_CODE[x["dtype"]], w_dtype=DTYPE_CODE[w["dtype"]],
+                       out_dtype=DTYPE_CODE[out["dtype"]], in_q=(s, z), w_q=_q(w["quant"]),
+                       out_q=(so, zo))
+        elif k == "FCL":
+            w = ins[1]
+            bias = val[ins[2]["id"]] if len(ins) > 2 and ins[2] is not None else None
+            kk = int(np.prod(x["shape"][:a["axis"] + 1]))
+            m = int(np.prod(x["shape"][a["axis"] + 1:]))
+            y = fully_connected(xv, val[w["id"]], bias, m=m, k=kk, n=w["shape"][-1],
+                                in_dtype=DTYPE_CODE[x["dtype"]], w_dtype=DTYPE_CODE[w["dtype"]],
+                                out_dtype=DTYPE_CODE[out["dtype"]], in_q=(s, z),
+                                w_q=_q(w["quant"]), out_q=(so, zo))
+        elif k == "POOL":
+            y = pool2d(xv, in_shape=pad4(x["shape"]), out_shape=pad4(out["shape"]),
+                       ksize=a["ksize"], stride=a["stride"], pad_left=a["pad"][0],
+                       pad_top=a["pad"][2], pool_type=POOL[a["pool_type"]],
+                       dtype=DTYPE_CODE[x["dtype"]], in_q=(s, z), out_q=(so, zo))
+        elif k in ("RELU", "RELU6"):
+            y = activation(ACT_RELU if k == "RELU" else ACT_RELU6, DTYPE_CODE[x["dtype"]], xv,
+                           (s, z), (so, zo))
+        elif k == "ADD":
+            b = ins[1]
+            sb, zb, _ = _q(b["quant"])
+            y = add(DTYPE_CODE[x["dtype"]], xv, (s, z), val[b["id"]], (sb, zb), (so, zo))
+        elif k == "SOFTMAX":
+            y = softmax(DTYPE_CODE[x["dtype"]], xv, x["shape"][0], a.get("beta", 1.0), (s, z))
+        elif k == "RESHAPE":
+            y = xv
+        else:
+            raise NotImplementedError(k)
+        val[out["id"]] = y
+    return val if keep_all else val[graph["output"]]

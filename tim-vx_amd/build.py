@@ -64,6 +64,11 @@ def build_runtime(verbose=False):
           "-I", os.path.join(REPO, "include")] + srcs +
          ["-L", os.path.join(PKG_DIR, "lib"), "-ltvx_hip", "-Wl,-rpath,$ORIGIN",
           "-o", os.path.join(PKG_DIR, "lib", "libtim-vx.so")], verbose)
+    # the graph-file runner: an application of the public API, linked like any other
+    _run(["g++", "-std=c++17", "-O2", "-Wall", "-I", os.path.join(PKG_DIR, "include"),
+          os.path.join(PKG_DIR, "src", "tools", "graph_runner.cc"),
+          "-L", os.path.join(PKG_DIR, "lib"), "-ltim-vx", "-ltvx_hip", "-Wl,-rpath,$ORIGIN",
+          "-o", os.path.join(PKG_DIR, "lib", "tvx_graph_runner")], verbose)
 
 
 def build_all(verbose=False):

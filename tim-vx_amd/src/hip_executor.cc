@@ -10,7 +10,9 @@
 // Execute() is vsi_nn_RunGraph -> vxProcessGraph (vsi_nn_graph.c:1605-1639):
 // inputs go host -> device, operators run in order on one stream, outputs come
 // back, and the call returns when everything is visible to the host.
+#include <chrono>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 
@@ -20,6 +22,8 @@
 namespace tim {
 namespace vx {
 namespace {
+
+double g_last_device_ms = 0.0;
 
 int DtypeCode(DataType t) {
   switch (t) {
@@ -145,12 +149,23 @@ class HipExecutor : public Executor {
         t->host_dirty_ = false;
       }
     }
+    // With TVX_RUNTIME_PROFILE set, the operator sequence is timed on its own
+    // (uploads drained first), for tools that report device time per Run().
+    std::chrono::steady_clock::time_point t0;
+    if (profile_) {
+      if (tvx_stream_synchronize(stream_) != TVX_OK) return Fail("sync");
+      t0 = std::chrono::steady_clock::now();
+    }
     for (auto& s : steps_) {
       const int st = tvx_op_run(s.op, dev_[s.in0], s.in1 ? dev_[s.in1] : nullptr, dev_[s.out], stream_);
       if (st != TVX_OK) {
         VSILOGE("%s failed: %s", s.name.c_str(), tvx_last_error());
         return false;
       }
+    }
+    if (profile_) {
+      if (tvx_stream_synchronize(stream_) != TVX_OK) return Fail("sync");
+      g_last_device_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
     }
     for (auto& t : graph->outputs_tensor_) {
       TensorImpl* ti = static_cast<TensorImpl*>(t.get());
@@ -349,6 +364,7 @@ class HipExecutor : public Executor {
   }
 
   void* stream_ = nullptr;
+  bool profile_ = std::getenv("TVX_RUNTIME_PROFILE") != nullptr;
   std::vector<Step> steps_;
   std::map<TensorImpl*, void*> dev_;    // tensor -> device pointer (possibly an alias)
   std::map<TensorImpl*, void*> owned_;  // tensors that own their buffer
@@ -362,3 +378,7 @@ std::unique_ptr<Executor> CreateExecutor() {
 
 }  // namespace vx
 }  // namespace tim
+
+// Milliseconds the operator sequence of the most recent Graph::Run() took on the
+// device (0 unless TVX_RUNTIME_PROFILE is set). No counterpart in the reference.
+extern "C" double tvx_runtime_last_device_ms(void) { return tim::vx::g_last_device_ms; }

@@ -1,0 +1,244 @@
+// tvx_graph_runner: builds graphs through the public tim::vx API from a plain-text
+// description, runs them, and writes what each graph produced.
+//
+//   tvx_graph_runner <graphs.txt> <blob.bin> <out.bin>
+//
+// graphs.txt, one record per line, fields separated by blanks:
+//   graph <name>
+//   t <id> <dtype> <attr> <rank> <dims..> <quant> <channel_dim> <ns> <scales..> <nz> <zps..> <off> <len>
+//       bytes [off, off+len) of blob.bin are the tensor's data; len 0 = no data.
+//       CONSTANT tensors get theirs at creation, INPUT tensors by CopyDataToTensor.
+//   op <KIND> <n_in> <ids..> <n_out> <ids..> <pad_type> <pl> <pr> <pt> <pb> <sw> <sh> <dw> <dh>
+//      <kw> <kh> <multiplier> <weights> <pool_type> <round_type> <pool_1d> <axis> <beta> <sm_axis>
+//      <n_shape> <shape..>
+//       id -1 = the graph's placeholder tensor (no bias)
+//   run <tensor id>           compile + run; append the tensor to out.bin
+//   bench <warmup> <iters>    time Graph::Run() (after a `run`)
+//   end
+// For every `run` one line goes to stdout: "ok <name> <offset> <bytes>" or
+// "fail <name> <stage>"; for every `bench`: "bench <name> <ms per Run> <ms per Run, device part>".
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <iostream>
+#include <map>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "tim/vx/context.h"
+#include "tim/vx/graph.h"
+#include "tim/vx/ops.h"
+#include "tim/vx/tensor.h"
+
+extern "C" double tvx_runtime_last_device_ms(void);
+
+using namespace tim::vx;
+
+namespace {
+
+DataType ParseDtype(const std::string& s) {
+  static const std::map<std::string, DataType> m = {
+      {"UINT8", DataType::UINT8},     {"INT8", DataType::INT8},       {"INT16", DataType::INT16},
+      {"INT32", DataType::INT32},     {"FLOAT16", DataType::FLOAT16}, {"FLOAT32", DataType::FLOAT32},
+      {"UINT32", DataType::UINT32},   {"BOOL8", DataType::BOOL8}};
+  auto it = m.find(s);
+  if (it == m.end()) { std::fprintf(stderr, "unknown dtype %s\n", s.c_str()); std::exit(2); }
+  return it->second;
+}
+TensorAttribute ParseAttr(const std::string& s) {
+  if (s == "CONSTANT") return TensorAttribute::CONSTANT;
+  if (s == "INPUT") return TensorAttribute::INPUT;
+  if (s == "OUTPUT") return TensorAttribute::OUTPUT;
+  if (s == "TRANSIENT") return TensorAttribute::TRANSIENT;
+  return TensorAttribute::VARIABLE;
+}
+QuantType ParseQuant(const std::string& s) {
+  if (s == "ASYMMETRIC") return QuantType::ASYMMETRIC;
+  if (s == "SYMMETRIC_PER_CHANNEL") return QuantType::SYMMETRIC_PER_CHANNEL;
+  if (s == "ASYMMETRIC_PER_CHANNEL") return QuantType::ASYMMETRIC_PER_CHANNEL;
+  if (s == "DYNAMIC_FIXED_POINT") return QuantType::DYNAMIC_FIXED_POINT;
+  return QuantType::NONE;
+}
+PadType ParsePad(const std::string& s) {
+  if (s == "VALID") return PadType::VALID;
+  if (s == "SAME") return PadType::SAME;
+  if (s == "NONE") return PadType::NONE;
+  return PadType::AUTO;
+}
+PoolType ParsePool(const std::string& s) {
+  if (s == "AVG") return PoolType::AVG;
+  if (s == "L2") return PoolType::L2;
+  if (s == "AVG_ANDROID") return PoolType::AVG_ANDROID;
+  return PoolType::MAX;
+}
+
+struct Pending {
+  std::shared_ptr<Tensor> tensor;
+  size_t off = 0, len = 0;
+  bool is_input = false;
+};
+
+}  // namespace
+
+int main(int argc, char** argv) {
+  if (argc != 4) {
+    std::fprintf(stderr, "usage: %s graphs.txt blob.bin out.bin\n", argv[0]);
+    return 2;
+  }
+  std::ifstream txt(argv[1]);
+  std::ifstream blobf(argv[2], std::ios::binary);
+  if (!txt || !blobf) { std::fprintf(stderr, "cannot open inputs\n"); return 2; }
+  std::vector<char> blob((std::istreambuf_iterator<char>(blobf)), std::istreambuf_iterator<char>());
+  FILE* out = std::fopen(argv[3], "wb");
+  if (!out) { std::fprintf(stderr, "cannot open %s\n", argv[3]); return 2; }
+  size_t out_off = 0;
+
+  setenv("TVX_RUNTIME_PROFILE", "1", 0);  // makes `bench` report the device part of Run()
+  auto context = Context::Create();
+  std::shared_ptr<Graph> graph;
+  std::map<int, Pending> tensors;
+  std::string name, line;
+  bool compiled = false, compile_ok = false;
+
+  while (std::getline(txt, line)) {
+    std::istringstream ss(line);
+    std::string rec;
+    if (!(ss >> rec)) continue;
+    if (rec == "graph") {
+      ss >> name;
+      graph = context->CreateGraph();
+      tensors.clear();
+      compiled = compile_ok = false;
+    } else if (rec == "t") {
+      int id, rank, chdim, ns, nz;
+      std::string dt, attr, qt;
+      ss >> id >> dt >> attr >> rank;
+      ShapeType shape(rank);
+      for (auto& d : shape) ss >> d;
+      ss >> qt >> chdim >> ns;
+      std::vector<float> scales(ns);
+      for (auto& s : scales) ss >> s;
+      ss >> nz;
+      std::vector<int32_t> zps(nz);
+      for (auto& z : zps) ss >> z;
+      Pending p;
+      ss >> p.off >> p.len;
+      if (p.off + p.len > blob.size()) { std::fprintf(stderr, "blob range\n"); return 2; }
+      const QuantType q = ParseQuant(qt);
+      Quantization quant = q == QuantType::NONE ? Quantization() : Quantization(q, chdim, scales, zps);
+      TensorSpec spec(ParseDtype(dt), shape, ParseAttr(attr), quant);
+      p.is_input = attr == "INPUT";
+      const bool at_create = p.len && !p.is_input;
+      p.tensor = graph->CreateTensor(spec, at_create ? blob.data() + p.off : nullptr);
+      tensors[id] = p;
+    } else if (rec == "op") {
+      std::string kind, pad_type, pool_type, round_type;
+      int n_in, n_out;
+      ss >> kind >> n_in;
+      std::vector<std::shared_ptr<Tensor>> ins, outs;
+      for (int i = 0; i < n_in; ++i) {
+        int id;
+        ss >> id;
+        ins.push_back(id < 0 ? graph->CreateTensorPlaceHolder() : tensors.at(id).tensor);
+      }
+      ss >> n_out;
+      for (int i = 0; i < n_out; ++i) {
+        int id;
+        ss >> id;
+        outs.push_back(tensors.at(id).tensor);
+      }
+      std::array<uint32_t, 4> pad;
+      std::array<uint32_t, 2> stride, dil, ksize;
+      int32_t multiplier, weights, pool_1d, axis, sm_axis, n_shape;
+      float beta;
+      ss >> pad_type >> pad[0] >> pad[1] >> pad[2] >> pad[3] >> stride[0] >> stride[1] >> dil[0] >> dil[1] >>
+          ksize[0] >> ksize[1] >> multiplier >> weights >> pool_type >> round_type >> pool_1d >> axis >> beta >>
+          sm_axis >> n_shape;
+      std::vector<uint32_t> new_shape(n_shape);
+      for (auto& d : new_shape) ss >> d;
+      if (!ss) { std::fprintf(stderr, "malformed op record in %s\n", name.c_str()); return 2; }
+      const RoundType rnd = round_type == "CEILING" ? RoundType::CEILING : RoundType::FLOOR;
+      std::shared_ptr<Operation> op;
+      if (kind == "CONV2D") {
+        op = graph->CreateOperation<ops::Conv2d>(weights, ParsePad(pad_type), ksize, stride, dil, pad, multiplier);
+      } else if (kind == "FCL") {
+        op = graph->CreateOperation<ops::FullyConnected>(static_cast<uint32_t>(axis), static_cast<uint32_t>(weights));
+      } else if (kind == "POOL") {
+        if (pool_1d) {
+          op = graph->CreateOperation<ops::Pool1d>(ParsePool(pool_type), std::array<uint32_t, 2>{pad[0], pad[1]},
+                                                   ksize[0], stride[0], rnd);
+        } else if (ParsePad(pad_type) == PadType::AUTO) {
+          op = graph->CreateOperation<ops::Pool2d>(ParsePool(pool_type), pad, ksize, stride, rnd);
+        } else {
+          op = graph->CreateOperation<ops::Pool2d>(ParsePool(pool_type), ParsePad(pad_type), ksize, stride, rnd);
+        }
+      } else if (kind == "RELU") {
+        op = graph->CreateOperation<ops::Relu>();
+      } else if (kind == "RELU6") {
+        op = graph->CreateOperation<ops::Relu6>();
+      } else if (kind == "ADD") {
+        op = graph->CreateOperation<ops::Add>();
+      } else if (kind == "SOFTMAX") {
+        op = graph->CreateOperation<ops::Softmax>(beta, sm_axis);
+      } else if (kind == "RESHAPE") {
+        op = graph->CreateOperation<ops::Reshape>(new_shape);
+      } else {
+        std::fprintf(stderr, "unknown op kind %s\n", kind.c_str());
+        return 2;
+      }
+      op->BindInputs(ins).BindOutputs(outs);
+    } else if (rec == "run") {
+      int id;
+      ss >> id;
+      if (!compiled) {
+        compile_ok = graph->Compile();
+        compiled = true;
+      }
+      const char* stage = nullptr;
+      if (!compile_ok) stage = "compile";
+      if (!stage)
+        for (auto& kv : tensors)
+          if (kv.second.is_input && kv.second.len &&
+              !kv.second.tensor->CopyDataToTensor(blob.data() + kv.second.off, static_cast<uint32_t>(kv.second.len)))
+            stage = "copy_in";
+      if (!stage && !graph->Run()) stage = "run";
+      std::vector<char> result;
+      if (!stage) {
+        auto& t = tensors.at(id).tensor;
+        result.resize(t->GetSpec().GetByteSize());
+        if (!t->CopyDataFromTensor(result.data())) stage = "copy_out";
+      }
+      if (stage) {
+        std::printf("fail %s %s\n", name.c_str(), stage);
+      } else {
+        std::fwrite(result.data(), 1, result.size(), out);
+        std::printf("ok %s %zu %zu\n", name.c_str(), out_off, result.size());
+        out_off += result.size();
+      }
+      std::fflush(stdout);
+    } else if (rec == "bench") {
+      int warmup, iters;
+      ss >> warmup >> iters;
+      if (!compile_ok) { std::printf("fail %s bench\n", name.c_str()); continue; }
+      for (int i = 0; i < warmup; ++i) graph->Run();
+      double dev_ms = 0;
+      auto t0 = std::chrono::steady_clock::now();
+      for (int i = 0; i < iters; ++i) {
+        graph->Run();
+        dev_ms += tvx_runtime_last_device_ms();
+      }
+      auto t1 = std::chrono::steady_clock::now();
+      std::printf("bench %s %.6f %.6f\n", name.c_str(),
+                  std::chrono::duration<double, std::milli>(t1 - t0).count() / iters, dev_ms / iters);
+      std::fflush(stdout);
+    } else if (rec == "end") {
+      graph.reset();
+      tensors.clear();
+    }
+  }
+  std::fclose(out);
+  return 0;
+}
