@@ -185,6 +185,31 @@ def cpu_baseline(wl, gpu_out):
                        % (batch, reps, dt, ok)), ok
 
 
+def network_extras(steps, warmup):
+    """LeNet (the reference's CPU-runnable sample) and MobileNetV2 at batch 64 through the
+    tim::vx C++ API: images/s per Graph::Run(), whole call (host copies of the graph's input
+    and output included) and operator sequence alone."""
+    import tempfile
+    GF = importlib.import_module("tim-vx_amd.graphfile")
+    G = importlib.import_module("tim-vx_amd.graphs")
+    z = np.load(os.path.join(REPO, "tests", "golden", "lenet_asymu8.npz"))
+    nets = [("lenet_asymu8_b1", G.lenet_asymu8(z["weights"], z["input"], batch=1), 1),
+            ("mobilenet_v2_u8_b64_224", G.mobilenet_v2(batch=64, res=224), 64)]
+    out = {}
+    with tempfile.TemporaryDirectory() as d:
+        _, info, _ = GF.run_graphs([g for _, g, _ in nets], d, bench=(warmup, steps))
+    for name, g, batch in nets:
+        i = info.get(g["test"], {})
+        if "run_ms" not in i:
+            out[name] = {"error": i.get("fail", "no timing")}
+            continue
+        out[name] = {"images_per_s": round(batch / (i["run_ms"] * 1e-3), 1),
+                     "images_per_s_device": round(batch / (i["device_ms"] * 1e-3), 1),
+                     "run_ms": round(i["run_ms"], 4), "device_ms": round(i["device_ms"], 4),
+                     "tops_device": round(2 * G.mac_count(g) / (i["device_ms"] * 1e-3) / 1e12, 2)}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -229,6 +254,7 @@ def main():
                                      tops=round(w2["ops"] / (wall2 * 1e-3) / 1e12, 2),
                                      gbs=round(w2["algo_bytes"] / (wall2 * 1e-3) / 1e9, 1),
                                      roofline=dict(roofline(w2, k2), kernel_ms=round(k2, 5)))
+        extra.update(network_extras(max(5, min(args.steps, 30)), 3))
         line["extra"] = extra
     print(json.dumps(line))
 

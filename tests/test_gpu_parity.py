@@ -251,8 +251,38 @@ def test_conv2d_igemm_shapes(oracle, gi, mode):
     x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=oc, kh=kh, kw=kw, stride=stride, dil=dil,
                               pad=pad, mult=0, mode=mode)
     want = oracle.conv2d(x, wt, b, act=1, **kws)
-    got = TC.gpu_conv2d(x, wt, b, act=1, want_kernel="conv2d_igemm_i8", **kws)
+    pointwise = kh == 1 and kw == 1 and stride == [1, 1] and pad == [0, 0, 0, 0]
+    got = TC.gpu_conv2d(x, wt, b, act=1, want_kernel="pwconv_i8" if pointwise else "conv2d_igemm_i8", **kws)
     assert np.array_equal(got, want)
+    assert len(np.unique(want)) > 4
+
+
+PW_GRID = [
+    # (n, c, h, w, oc): 1x1 stride 1; HW % 16 == 0, % 4 == 0 and odd sizes; channel tails;
+    # few and many output tiles; a tile that straddles images
+    (2, 32, 16, 16, 64),
+    (3, 16, 14, 14, 96),
+    (5, 24, 7, 7, 144),
+    (2, 96, 14, 14, 576),
+    (3, 960, 7, 7, 320),
+    (1, 5, 3, 5, 7),
+    (2, 576, 14, 14, 96),
+    (1, 40, 20, 13, 33),
+    (2, 130, 6, 6, 200),
+]
+
+
+@pytest.mark.parametrize("mode", ["u8", "i8pc", "u8pc"])
+@pytest.mark.parametrize("gi", range(len(PW_GRID)))
+def test_pointwise_conv_shapes(oracle, gi, mode):
+    n, c, h, w, oc = PW_GRID[gi]
+    rng = np.random.default_rng(4000 + gi)
+    x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=oc, kh=1, kw=1, stride=[1, 1], dil=[1, 1],
+                              pad=[0, 0, 0, 0], mult=0, mode=mode)
+    for act in (0, 2):
+        want = oracle.conv2d(x, wt, b, act=act, **kws)
+        got = TC.gpu_conv2d(x, wt, b, act=act, want_kernel="pwconv_i8", **kws)
+        assert np.array_equal(got, want), int((got != want).sum())
     assert len(np.unique(want)) > 4
 
 
@@ -305,6 +335,6 @@ def test_depthwise_then_pointwise_full_size(oracle):
               dilation=[1, 1], pad_left=0, pad_top=0, multiplier=0, in_dtype=1, w_dtype=1, out_dtype=1,
               in_q=(0.08, 0), w_q=(1.0, 0, sp), out_q=(0.05, 0), act=2)
     out_want = oracle.conv2d(mid, wp, bp, **kp)
-    out = TC.gpu_conv2d(mid, wp, bp, want_kernel="conv2d_igemm_i8", **kp)
+    out = TC.gpu_conv2d(mid, wp, bp, want_kernel="pwconv_i8", **kp)
     assert np.array_equal(out, out_want)
     assert out.min() == 0 and out.max() == 120  # ReLU6 at scale 0.05

@@ -28,6 +28,9 @@ int FcMfmaSetup(tvx_op*, const tvx_fc_desc*, const void*, const void*);
 // int8 MFMA implicit-GEMM convolution (conv_igemm_i8.hip)
 int ConvIgemmSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 
+// pointwise (1x1) convolution with the whole channel depth of a pixel tile in LDS (pwconv_i8.hip)
+int PwConvSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
+
 // depthwise 3x3 stencil (dwconv3x3_i8.hip)
 int DwConv3x3Setup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 
