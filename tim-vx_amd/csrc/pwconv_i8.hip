@@ -16,8 +16,8 @@
 //     (1 KiB contiguous per wavefront load, prefetched two steps ahead across tile
 //     boundaries); they are small and live in L2.
 // Zero points: sum (x - zx)(w - zw) = sum xs ws - zws Sx - zxs Sw + C zxs zws with
-// xs, ws the operands moved to the signed int8 domain; Sx per pixel comes from
-// v_dot4 on the fragments, the per-channel constants are folded into the bias.
+// xs, ws the operands moved to the signed int8 domain; the Sx term is one more MFMA
+// against a constant fragment, the per-channel constants are folded into the bias.
 #include <algorithm>
 
 #include "variants.h"
@@ -28,12 +28,9 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-constexpr int kThreads = 256;
 constexpr int kPix = 128;          // flat pixels per workgroup
-constexpr int kPixTiles = kPix / 32;
 constexpr int kStageStride = 136;  // bytes per staged output row: 34 dwords spread 32 rows over all banks
 constexpr int kStageBytes = 32 * kStageStride;
-constexpr int kWaveLds = kStageBytes + kPix * 4;  // staging patch + per-pixel sums
 
 struct PwArgs {
   const uint8_t* x;
@@ -49,7 +46,8 @@ struct PwArgs {
   int oc_tiles;          // ceil(OC / 32)
   int tiles_per_wg;      // output tiles one workgroup walks (grid.y covers the rest)
   int xor_mask;          // 0x80808080 for uint8 activations
-  int zws, out_zp, lo, hi;
+  int neg_zws4;          // -(weight zero point, int8 domain) in all four bytes
+  int out_zp, lo, hi;
 };
 
 // 4 dwords = 4 channels x 4 pixels (pixel in the byte lanes) -> 4 dwords = 4 pixels x 4 channels.
@@ -64,17 +62,24 @@ __device__ __forceinline__ void Transpose4x4(const uint32_t in[4], uint32_t out[
   out[3] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x07060302);
 }
 
-// GRAN: pixels that are guaranteed to stay inside one image and to be aligned:
-// 16 (HW % 16 == 0), 4 (HW % 4 == 0) or 1.
-template <int GRAN, bool SX, int RQ>
-__global__ void __launch_bounds__(kThreads) PwConvKernel(PwArgs a) {
+// NW: wavefronts per workgroup (1: every wavefront is on its own - shallow inputs whose
+//     tile is a few KiB, many tiles in flight per CU; 4: the tile is built cooperatively).
+// PT: 32-pixel MFMA tiles per work item; an item is (output tile, 32*PT-pixel part), so
+//     that a workgroup with fewer output tiles than wavefronts still keeps all of them busy.
+// GRAN: pixels guaranteed to stay inside one image and to be aligned: 16, 4 or 1.
+// ZP: the weights have a zero point (int8 domain): its term -zws * sum_c xs is taken by a
+//     second MFMA against a constant fragment - the matrix cores idle here anyway.
+template <int NW, int PT, int GRAN, bool ZP, int RQ>
+__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4, 8))) PwConvKernel(PwArgs a) {
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
+  constexpr int kThreads = 64 * NW;
+  constexpr int kParts = 4 / PT;      // pixel parts per output tile
+  constexpr int kRowBytes = 32 * PT;  // staged bytes per output row
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave = NW == 1 ? 0 : __builtin_amdgcn_readfirstlane(tid >> 6);
   const long long q_base = static_cast<long long>(blockIdx.x) * kPix;
   int8_t* xl = lds;
-  int8_t* stage = lds + kPix * a.pix_stride + wave * kWaveLds;
-  int* sx_lds = reinterpret_cast<int*>(stage + kStageBytes);
+  int8_t* stage = lds + kPix * a.pix_stride + wave * kStageBytes;
 
   // ---- activations of the 128 pixels, all channels: global (pixel-innermost) -> LDS
   if (GRAN >= 4) {
@@ -84,7 +89,7 @@ __global__ void __launch_bounds__(kThreads) PwConvKernel(PwArgs a) {
     const long long n = live ? q0 / a.HW : 0;
     const int p = live ? static_cast<int>(q0 - n * a.HW) : 0;
     const uint8_t* src = a.x + (static_cast<size_t>(n) * a.C) * a.HW + p;
-    for (int cg = cg0; cg < a.cp / 16; cg += 8) {
+    for (int cg = cg0; cg < a.cp / 16; cg += 2 * NW) {
       uint32_t raw[16];
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
@@ -104,99 +109,93 @@ __global__ void __launch_bounds__(kThreads) PwConvKernel(PwArgs a) {
       }
     }
   } else {
-    const int px = tid & 127, cg0 = tid >> 7;
-    const long long q0 = q_base + px;
-    const bool live = q0 < a.Q;
-    const long long n = live ? q0 / a.HW : 0;
-    const int p = live ? static_cast<int>(q0 - n * a.HW) : 0;
-    const uint8_t* src = a.x + (static_cast<size_t>(n) * a.C) * a.HW + p;
-    for (int cg = cg0; cg < a.cp / 16; cg += 2) {
-      uint32_t w[4] = {0, 0, 0, 0};
+    for (int px = tid & 127; px < kPix; px += (NW == 1 ? 64 : 128)) {
+      const int cg0 = NW == 1 ? 0 : tid >> 7;
+      const long long q0 = q_base + px;
+      const bool live = q0 < a.Q;
+      const long long n = live ? q0 / a.HW : 0;
+      const int p = live ? static_cast<int>(q0 - n * a.HW) : 0;
+      const uint8_t* src = a.x + (static_cast<size_t>(n) * a.C) * a.HW + p;
+      for (int cg = cg0; cg < a.cp / 16; cg += (NW == 1 ? 1 : 2)) {
+        uint32_t w[4] = {0, 0, 0, 0};
 #pragma unroll
-      for (int j = 0; j < 16; ++j) {
-        const int c = cg * 16 + j;
-        const uint32_t b = (live && c < a.C) ? (src[static_cast<size_t>(c) * a.HW] ^ (a.xor_mask & 0xff)) : 0u;
-        w[j >> 2] |= b << (8 * (j & 3));
+        for (int j = 0; j < 16; ++j) {
+          const int c = cg * 16 + j;
+          const uint32_t b = (live && c < a.C) ? (src[static_cast<size_t>(c) * a.HW] ^ (a.xor_mask & 0xff)) : 0u;
+          w[j >> 2] |= b << (8 * (j & 3));
+        }
+        v4i v = {static_cast<int>(w[0]), static_cast<int>(w[1]), static_cast<int>(w[2]), static_cast<int>(w[3])};
+        *reinterpret_cast<v4i*>(xl + px * a.pix_stride + cg * 16) = v;
       }
-      v4i v = {static_cast<int>(w[0]), static_cast<int>(w[1]), static_cast<int>(w[2]), static_cast<int>(w[3])};
-      *reinterpret_cast<v4i*>(xl + px * a.pix_stride + cg * 16) = v;
     }
   }
 
+  // ---- work items of this wavefront: (output tile, pixel part) ---------------------------
+  const int t_begin = blockIdx.y * a.tiles_per_wg;
+  const int t_end = min(t_begin + a.tiles_per_wg, a.oc_tiles);
+  // wavefront w takes items w, w + NW, ...; with kParts | NW its pixel part never changes
+  const int part = wave % kParts;
+  const int tile_step = NW / kParts > 0 ? NW / kParts : 1;
+  const int tile0 = t_begin + wave / kParts;
+  const int n_tiles = tile0 < t_end ? (t_end - tile0 + tile_step - 1) / tile_step : 0;
+  if (NW > 1) __syncthreads();  // the input tile is complete; nothing below needs the other wavefronts
+  if (n_tiles <= 0) return;
+
   // ---- where this lane's output groups live (the same for every output tile) -----
-  // Copy-out mapping: GRAN 16: lane -> (row lane/8 + 8 i, 16-pixel chunk lane%8);
-  // GRAN 4: lane -> (row lane/32 + 2 i, dword lane%32); GRAN 1: lane -> pixels lane, lane+64.
-  constexpr int kGroups = GRAN == 1 ? 2 : 1;
+  // Copy-out mapping of a staged row of kRowBytes pixels: GRAN 16: lane -> 16-pixel chunk
+  // lane % (kRowBytes/16); GRAN 4: dword lane % (kRowBytes/4); GRAN 1: pixel lane % kRowBytes (+64).
+  constexpr int kPerRow = GRAN == 16 ? kRowBytes / 16 : (GRAN == 4 ? kRowBytes / 4 : (kRowBytes < 64 ? kRowBytes : 64));
+  constexpr int kGroups = (GRAN == 1 && kRowBytes > 64) ? 2 : 1;
+  constexpr int kRowsPerIter = 64 / kPerRow;
+  const int px_in_row = (lane % kPerRow) * GRAN;
   size_t out_off[kGroups];
   bool out_live[kGroups];
 #pragma unroll
   for (int g = 0; g < kGroups; ++g) {
-    const int px = GRAN == 16 ? (lane & 7) * 16 : (GRAN == 4 ? (lane & 31) * 4 : lane + 64 * g);
-    const long long q0 = q_base + px;
+    const long long q0 = q_base + part * kRowBytes + px_in_row + 64 * g;
     out_live[g] = q0 < a.Q;
     const long long n = out_live[g] ? q0 / a.HW : 0;
     out_off[g] = static_cast<size_t>(n) * a.OC * a.HW + static_cast<size_t>(q0 - n * a.HW);
   }
 
-  // ---- output tiles of this wavefront ------------------------------------------------
-  const int t_begin = blockIdx.y * a.tiles_per_wg;
-  const int t_end = min(t_begin + a.tiles_per_wg, a.oc_tiles);
-  const int n_tiles = (t_end - t_begin - wave + 3) / 4;  // tiles t_begin + wave + 4 j
-  __syncthreads();  // the input tile is complete; nothing below needs the other wavefronts
-  if (n_tiles <= 0) return;
-
   const int frag_row = lane & 31, frag_half = lane >> 5;
-  const int8_t* xa = xl + frag_row * a.pix_stride + frag_half * 16;
+  const int8_t* xa = xl + (part * kRowBytes + frag_row) * a.pix_stride + frag_half * 16;
   const int total = n_tiles * a.ksteps;
 
   // weight fragment stream, in consumption order
-  int pf_tile = t_begin + wave, pf_ks = 0, pf_left = total;
+  int pf_tile = tile0, pf_ks = 0, pf_left = total;
   auto next_frag = [&]() -> v4i {
     const v4i f = a.wpk[(static_cast<size_t>(pf_tile) * a.ksteps + pf_ks) * 64 + lane];
     if (--pf_left > 0) {  // past the end: keep re-reading the last fragment
-      if (++pf_ks == a.ksteps) { pf_ks = 0; pf_tile += 4; }
+      if (++pf_ks == a.ksteps) { pf_ks = 0; pf_tile += tile_step; }
     }
     return f;
   };
 
-  v16i acc[kPixTiles];
-  int sx[kPixTiles] = {0, 0, 0, 0};
-  int tile = t_begin + wave, ks = 0;
-  bool first = true;
+  v16i acc[PT];
+  int tile = tile0, ks = 0;
   auto init_acc = [&]() {
     const int b = a.biasf[tile * 32 + frag_row];
 #pragma unroll
-    for (int i = 0; i < kPixTiles; ++i)
+    for (int i = 0; i < PT; ++i)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][r] = b;
   };
+  const v4i fz = {a.neg_zws4, a.neg_zws4, a.neg_zws4, a.neg_zws4};
 
   auto epilogue = [&]() {
-    if (SX && first) {
-#pragma unroll
-      for (int i = 0; i < kPixTiles; ++i) {
-        sx[i] += __shfl_xor(sx[i], 32);
-        if (frag_half == 0) sx_lds[i * 32 + frag_row] = a.zws * sx[i];
-      }
-    }
-    first = false;
-    __builtin_amdgcn_wave_barrier();
     const int oc = tile * 32 + frag_row;
     const v4i q = a.rq[oc];
+    const int lo = a.lo, hi = a.hi;
 #pragma unroll
-    for (int i = 0; i < kPixTiles; ++i)
+    for (int i = 0; i < PT; ++i)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int pl = i * 32 + 8 * g + 4 * frag_half;
-        v4i s4 = {0, 0, 0, 0};
-        if (SX) s4 = *reinterpret_cast<const v4i*>(sx_lds + pl);
-        uint32_t packed = 0;
+        int v[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int v = acc[i][g * 4 + e] - s4[e];
-          packed |= static_cast<uint32_t>(Requant8<RQ>(v, q, a.out_zp, a.lo, a.hi) & 0xff) << (8 * e);
-        }
-        *reinterpret_cast<uint32_t*>(stage + frag_row * kStageStride + pl) = packed;
+        for (int e = 0; e < 4; ++e) v[e] = Requant8<RQ>(acc[i][g * 4 + e], q, a.out_zp, lo, hi);
+        *reinterpret_cast<uint32_t*>(stage + frag_row * kStageStride + pl) = PackBytes(v[0], v[1], v[2], v[3]);
       }
     __builtin_amdgcn_wave_barrier();
     // copy-out: rows of the staging patch -> WHCN output
@@ -204,52 +203,48 @@ __global__ void __launch_bounds__(kThreads) PwConvKernel(PwArgs a) {
     uint8_t* ybase = a.y + static_cast<size_t>(tile) * 32 * a.HW;
     if (GRAN == 16) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int row = (lane >> 3) + 8 * i;
-        const int8_t* s = stage + row * kStageStride + (lane & 7) * 16;
-        const uint2 lo = *reinterpret_cast<const uint2*>(s);
-        const uint2 hi = *reinterpret_cast<const uint2*>(s + 8);
+      for (int i = 0; i < 32 / kRowsPerIter; ++i) {
+        const int row = lane / kPerRow + kRowsPerIter * i;
+        const int8_t* s = stage + row * kStageStride + px_in_row;
+        const uint2 lo8 = *reinterpret_cast<const uint2*>(s);
+        const uint2 hi8 = *reinterpret_cast<const uint2*>(s + 8);
         if (row < rows && out_live[0])
           *reinterpret_cast<uint4*>(ybase + out_off[0] + static_cast<size_t>(row) * a.HW) =
-              make_uint4(lo.x, lo.y, hi.x, hi.y);
+              make_uint4(lo8.x, lo8.y, hi8.x, hi8.y);
       }
     } else if (GRAN == 4) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int row = (lane >> 5) + 2 * i;
-        const uint32_t v = *reinterpret_cast<const uint32_t*>(stage + row * kStageStride + (lane & 31) * 4);
+      for (int i = 0; i < 32 / kRowsPerIter; ++i) {
+        const int row = lane / kPerRow + kRowsPerIter * i;
+        const uint32_t v = *reinterpret_cast<const uint32_t*>(stage + row * kStageStride + px_in_row);
         if (row < rows && out_live[0])
           *reinterpret_cast<uint32_t*>(ybase + out_off[0] + static_cast<size_t>(row) * a.HW) = v;
       }
     } else {
-      for (int row = 0; row < rows; ++row)
+      for (int row = lane / kPerRow; row < rows; row += kRowsPerIter)
 #pragma unroll
         for (int g = 0; g < kGroups; ++g)
           if (out_live[g])
             ybase[out_off[g] + static_cast<size_t>(row) * a.HW] =
-                static_cast<uint8_t>(stage[row * kStageStride + lane + 64 * g]);
+                static_cast<uint8_t>(stage[row * kStageStride + px_in_row + 64 * g]);
     }
     __builtin_amdgcn_wave_barrier();
   };
 
   auto step = [&](const v4i& fw) {
-    v4i fx[kPixTiles];
+    v4i fx[PT];
 #pragma unroll
-    for (int i = 0; i < kPixTiles; ++i)
+    for (int i = 0; i < PT; ++i)
       fx[i] = *reinterpret_cast<const v4i*>(xa + i * 32 * a.pix_stride + ks * 32);
-    if (SX && first) {
 #pragma unroll
-      for (int i = 0; i < kPixTiles; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) sx[i] = __builtin_amdgcn_sdot4(fx[i][j], 0x01010101, sx[i], false);
-    }
-#pragma unroll
-    for (int i = 0; i < kPixTiles; ++i)
+    for (int i = 0; i < PT; ++i) {
       acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fx[i], fw, acc[i], 0, 0, 0);
+      if (ZP) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fx[i], fz, acc[i], 0, 0, 0);
+    }
     if (++ks == a.ksteps) {
       epilogue();
       ks = 0;
-      tile += 4;
+      tile += tile_step;
       if (tile < t_end) init_acc();
     }
   };
@@ -271,39 +266,48 @@ __global__ void __launch_bounds__(kThreads) PwConvKernel(PwArgs a) {
 
 struct Plan {
   PwArgs a;
-  int lds_bytes, gran, sx, rq;
+  int lds_bytes, nw, pt, gran, zp, rq;
   dim3 grid;
 };
 
-template <int GRAN, bool SX, int RQ>
+template <int NW, int PT, int GRAN, bool ZP, int RQ>
 int Launch(const Plan* plan, const PwArgs& a, hipStream_t st, bool configure) {
   if (configure) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&PwConvKernel<GRAN, SX, RQ>),
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&PwConvKernel<NW, PT, GRAN, ZP, RQ>),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, plan->lds_bytes);
     if (e != hipSuccess)
       return SetError(TVX_E_DEVICE, "hipFuncSetAttribute(dynamic LDS %d): %s", plan->lds_bytes, hipGetErrorString(e));
     return TVX_OK;
   }
-  hipLaunchKernelGGL((PwConvKernel<GRAN, SX, RQ>), plan->grid, dim3(kThreads), plan->lds_bytes, st, a);
+  hipLaunchKernelGGL((PwConvKernel<NW, PT, GRAN, ZP, RQ>), plan->grid, dim3(64 * NW), plan->lds_bytes, st, a);
   return TVX_OK;
 }
 
-template <int GRAN, bool SX>
+template <int NW, int PT, int GRAN, bool ZP>
 int DispatchRq(const Plan* plan, const PwArgs& a, hipStream_t st, bool configure) {
-  if (plan->rq == kRqFastNoTie) return Launch<GRAN, SX, kRqFastNoTie>(plan, a, st, configure);
-  if (plan->rq == kRqFast) return Launch<GRAN, SX, kRqFast>(plan, a, st, configure);
-  return Launch<GRAN, SX, kRqGeneric>(plan, a, st, configure);
+  if (plan->rq == kRqFastNoTie) return Launch<NW, PT, GRAN, ZP, kRqFastNoTie>(plan, a, st, configure);
+  if (plan->rq == kRqFast) return Launch<NW, PT, GRAN, ZP, kRqFast>(plan, a, st, configure);
+  return Launch<NW, PT, GRAN, ZP, kRqGeneric>(plan, a, st, configure);
 }
 
-template <int GRAN>
-int DispatchSx(const Plan* plan, const PwArgs& a, hipStream_t st, bool configure) {
-  return plan->sx ? DispatchRq<GRAN, true>(plan, a, st, configure) : DispatchRq<GRAN, false>(plan, a, st, configure);
+template <int NW, int PT, int GRAN>
+int DispatchZp(const Plan* plan, const PwArgs& a, hipStream_t st, bool configure) {
+  return plan->zp ? DispatchRq<NW, PT, GRAN, true>(plan, a, st, configure)
+                  : DispatchRq<NW, PT, GRAN, false>(plan, a, st, configure);
+}
+
+template <int NW, int PT>
+int DispatchGran(const Plan* plan, const PwArgs& a, hipStream_t st, bool configure) {
+  if (plan->gran == 16) return DispatchZp<NW, PT, 16>(plan, a, st, configure);
+  if (plan->gran == 4) return DispatchZp<NW, PT, 4>(plan, a, st, configure);
+  return DispatchZp<NW, PT, 1>(plan, a, st, configure);
 }
 
 int Dispatch(const Plan* plan, const PwArgs& a, hipStream_t st, bool configure) {
-  if (plan->gran == 16) return DispatchSx<16>(plan, a, st, configure);
-  if (plan->gran == 4) return DispatchSx<4>(plan, a, st, configure);
-  return DispatchSx<1>(plan, a, st, configure);
+  if (plan->nw == 1) return DispatchGran<1, 4>(plan, a, st, configure);
+  if (plan->pt == 4) return DispatchGran<4, 4>(plan, a, st, configure);
+  if (plan->pt == 2) return DispatchGran<4, 2>(plan, a, st, configure);
+  return DispatchGran<4, 1>(plan, a, st, configure);
 }
 
 int PwConvRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
@@ -341,7 +345,9 @@ int PwConvSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const 
   a.ksteps = a.cp / 32;
   a.pix_stride = a.cp + 16;
   a.oc_tiles = (a.OC + 31) / 32;
-  const int lds_bytes = kPix * a.pix_stride + 4 * kWaveLds;
+  // a shallow input (tile of a few KiB): one wavefront per workgroup, many tiles in flight
+  const int nw = kPix * a.pix_stride <= 20 * 1024 ? 1 : 4;
+  const int lds_bytes = kPix * a.pix_stride + nw * kStageBytes;
   if (lds_bytes > 160 * 1024) return TVX_E_UNSUPPORTED;
   const long long gx = (a.Q + kPix - 1) / kPix;
   if (gx > 0x7fffffffll) return TVX_E_UNSUPPORTED;
@@ -349,17 +355,20 @@ int PwConvSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const 
   const int zxs = d->in_zp - (x_u8 ? 128 : 0);
   const int zws = op->w_zp - (w_u8 ? 128 : 0);
   if (zxs < -128 || zxs > 127) return TVX_E_UNSUPPORTED;  // zero point outside the tensor's range
+  if (zws < -127 || zws > 127) return TVX_E_UNSUPPORTED;  // -zws must be an int8
   a.xor_mask = x_u8 ? static_cast<int>(0x80808080u) : 0;
-  a.zws = zws;
+  a.neg_zws4 = static_cast<int>(static_cast<uint32_t>((-zws) & 0xff) * 0x01010101u);
   a.out_zp = d->out_zp;
   a.lo = op->act_lo;
   a.hi = op->act_hi;
   // few pixel tiles: spread the output tiles over grid.y (in units of one tile per
   // wavefront) until the launch has a few workgroups per CU
-  const int quads = (a.oc_tiles + 3) / 4;
+  const int quads = (a.oc_tiles + nw - 1) / nw;
   int gy = static_cast<int>(std::min<long long>(quads, std::max<long long>(1, 1024 / gx)));
-  a.tiles_per_wg = ((quads + gy - 1) / gy) * 4;
+  a.tiles_per_wg = std::min(((quads + gy - 1) / gy) * nw, a.oc_tiles);
   gy = (a.oc_tiles + a.tiles_per_wg - 1) / a.tiles_per_wg;
+  // fewer output tiles than wavefronts: split the pixels of a tile over wavefronts instead
+  const int pt = nw == 1 ? 4 : (a.tiles_per_wg >= 4 ? 4 : (a.tiles_per_wg >= 2 ? 2 : 1));
 
   // ---- weights in fragment order, constants folded into the bias -------------------
   const int oc_alloc = a.oc_tiles * 32;
@@ -393,8 +402,10 @@ int PwConvSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const 
   Plan plan;
   plan.a = a;
   plan.lds_bytes = lds_bytes;
+  plan.nw = nw;
+  plan.pt = pt;
   plan.gran = (a.HW % 16 == 0) ? 16 : ((a.HW % 4 == 0) ? 4 : 1);
-  plan.sx = zws != 0;
+  plan.zp = zws != 0;
   plan.rq = rq;
   plan.grid = dim3(static_cast<unsigned>(gx), static_cast<unsigned>(gy));
   s = Dispatch(&plan, a, nullptr, true);

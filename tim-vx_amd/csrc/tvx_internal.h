@@ -107,6 +107,20 @@ constexpr int kRqGeneric = 0;    // any shift: 64-bit product
 constexpr int kRqFast = 1;       // high half of the product + tie fix-up
 constexpr int kRqFastNoTie = 2;  // additionally no accumulator can land on a tie
 
+// clamp(v, lo, hi) for lo <= hi in one instruction
+__device__ __forceinline__ int Med3(int v, int lo, int hi) {
+  int r;
+  asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "v"(lo), "v"(hi));
+  return r;
+}
+
+// The low bytes of four ints as one dword (a in byte 0).
+__device__ __forceinline__ uint32_t PackBytes(int a, int b, int c, int d) {
+  const uint32_t ab = __builtin_amdgcn_perm(static_cast<uint32_t>(b), static_cast<uint32_t>(a), 0x0c0c0400);
+  const uint32_t cd = __builtin_amdgcn_perm(static_cast<uint32_t>(d), static_cast<uint32_t>(c), 0x0c0c0400);
+  return __builtin_amdgcn_perm(cd, ab, 0x05040100);
+}
+
 template <int RQ>
 __device__ __forceinline__ int Requant8(int v, const tvx_v4i& q, int zp, int lo, int hi) {
   if (RQ == kRqGeneric) return RequantClamp(v, q[0], q[1], zp, lo, hi);
@@ -117,7 +131,7 @@ __device__ __forceinline__ int Requant8(int v, const tvx_v4i& q, int zp, int lo,
     const bool tie = ((h & (2 * half - 1)) == half) && ((v & q[3]) == 0);
     if (tie && ((r - zp) & 1)) --r;
   }
-  return max(lo, min(r, hi));
+  return Med3(r, lo, hi);
 }
 
 // ---- host helpers ------------------------------------------------------------
