@@ -119,7 +119,7 @@ def pw_cfg3b(T, rng):
 
 
 def time_workload(wl, steps, warmup):
-    """Returns (wall ms per step over exactly `steps` steps, mean per-launch kernel ms)."""
+    """Returns (wall ms per step over exactly `steps` steps, mean kernel ms per launch)."""
     import torch
     stream = torch.cuda.current_stream()
     dev_in = [torch.from_numpy(a).cuda() for a in wl["inputs"]]
@@ -130,21 +130,19 @@ def time_workload(wl, steps, warmup):
     for _ in range(warmup):
         op.run(dev_in[0], in1, out, stream.cuda_stream)
     torch.cuda.synchronize()
+    # The timed region: exactly `steps` launches, one kernel each, back to back on one
+    # stream. Wall clock brackets it with synchronisation on both sides; a HIP event pair
+    # recorded on the launch stream brackets the same region for the kernel's average
+    # launch duration (per-launch event pairs would add their own ~2 us to each sample).
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    e0.record(stream)
     for _ in range(steps):
         op.run(dev_in[0], in1, out, stream.cuda_stream)
+    e1.record(stream)
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    # per-launch duration: HIP events recorded on the launch stream around every launch
-    pairs = []
-    for _ in range(steps):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record(stream)
-        op.run(dev_in[0], in1, out, stream.cuda_stream)
-        e1.record(stream)
-        pairs.append((e0, e1))
-    torch.cuda.synchronize()
-    kernel_ms = float(np.mean([a.elapsed_time(b) for a, b in pairs]))
+    kernel_ms = e0.elapsed_time(e1) / steps
     wl["device_out"] = out
     return wall_ms, kernel_ms
 
@@ -216,12 +214,22 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extra", action="store_true", help="skip the non-headline workloads")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run only a plain 256 MiB device copy, 10 times (scales the HBM byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
     import torch
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU: the hot path has no CPU fallback")
+    if args.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(3)
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes": 256 << 20, "repeats": 10}))
+        return
     T = importlib.import_module("tim-vx_amd")
     rng = np.random.default_rng(SEED)
 
@@ -232,7 +240,7 @@ def main():
     traffic = None
     tpath = os.path.join(REPO, "profiles", "traffic.json")
     if os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get(wl["op"].kernel_name)
+        traffic = json.load(open(tpath)).get(wl["op"].kernel_name, {}).get("bytes_per_launch")
     line = {
         "metric": "int8 conv TOPS", "value": round(wl["ops"] / (wall_ms * 1e-3) / 1e12, 3), "unit": "TOPS",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 5),
