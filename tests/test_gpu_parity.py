@@ -272,10 +272,15 @@ PW_GRID = [
 ]
 
 
+@pytest.mark.parametrize("shape", [None, "128,1", "128,4", "32,1", "32,4"])
 @pytest.mark.parametrize("mode", ["u8", "i8pc", "u8pc"])
 @pytest.mark.parametrize("gi", range(len(PW_GRID)))
-def test_pointwise_conv_shapes(oracle, gi, mode):
+def test_pointwise_conv_shapes(oracle, gi, mode, shape, monkeypatch):
+    """Every workgroup shape of the kernel (pixels per workgroup, wavefronts) on every case,
+    not only the one the heuristic would pick."""
     n, c, h, w, oc = PW_GRID[gi]
+    if shape is not None:
+        monkeypatch.setenv("TVX_PWCONV_SHAPE", shape)
     rng = np.random.default_rng(4000 + gi)
     x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=oc, kh=1, kw=1, stride=[1, 1], dil=[1, 1],
                               pad=[0, 0, 0, 0], mult=0, mode=mode)

@@ -19,6 +19,8 @@
 // xs, ws the operands moved to the signed int8 domain; the Sx term is one more MFMA
 // against a constant fragment, the per-channel constants are folded into the bias.
 #include <algorithm>
+#include <cstdio>
+#include <cstdlib>
 
 #include "variants.h"
 
@@ -28,7 +30,6 @@ namespace {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-constexpr int kPix = 128;          // flat pixels per workgroup
 constexpr int kStageStride = 136;  // bytes per staged output row: 34 dwords spread 32 rows over all banks
 constexpr int kStageBytes = 32 * kStageStride;
 
@@ -62,6 +63,8 @@ __device__ __forceinline__ void Transpose4x4(const uint32_t in[4], uint32_t out[
   out[3] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x07060302);
 }
 
+// KP: flat pixels per workgroup: 128, or 32 when the whole batch has few pixels and more,
+//     smaller workgroups are needed to fill the chip.
 // NW: wavefronts per workgroup (1: every wavefront is on its own - shallow inputs whose
 //     tile is a few KiB, many tiles in flight per CU; 4: the tile is built cooperatively).
 // PT: 32-pixel MFMA tiles per work item; an item is (output tile, 32*PT-pixel part), so
@@ -69,11 +72,12 @@ __device__ __forceinline__ void Transpose4x4(const uint32_t in[4], uint32_t out[
 // GRAN: pixels guaranteed to stay inside one image and to be aligned: 16, 4 or 1.
 // ZP: the weights have a zero point (int8 domain): its term -zws * sum_c xs is taken by a
 //     second MFMA against a constant fragment - the matrix cores idle here anyway.
-template <int NW, int PT, int GRAN, bool ZP, int RQ>
+template <int KP, int NW, int PT, int GRAN, bool ZP, int RQ>
 __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4, 8))) PwConvKernel(PwArgs a) {
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   constexpr int kThreads = 64 * NW;
-  constexpr int kParts = 4 / PT;      // pixel parts per output tile
+  constexpr int kPix = KP;
+  constexpr int kParts = KP / (32 * PT);  // pixel parts per output tile
   constexpr int kRowBytes = 32 * PT;  // staged bytes per output row
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = NW == 1 ? 0 : __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -83,13 +87,14 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
 
   // ---- activations of the 128 pixels, all channels: global (pixel-innermost) -> LDS
   if (GRAN >= 4) {
-    const int pq = tid & 31, cg0 = tid >> 5;  // 4-pixel group, first 16-channel group
+    constexpr int kQuads = KP / 4;
+    const int pq = tid % kQuads, cg0 = tid / kQuads;  // 4-pixel group, first 16-channel group
     const long long q0 = q_base + pq * 4;
     const bool live = q0 < a.Q;
     const long long n = live ? q0 / a.HW : 0;
     const int p = live ? static_cast<int>(q0 - n * a.HW) : 0;
     const uint8_t* src = a.x + (static_cast<size_t>(n) * a.C) * a.HW + p;
-    for (int cg = cg0; cg < a.cp / 16; cg += 2 * NW) {
+    for (int cg = cg0; cg < a.cp / 16; cg += kThreads / kQuads) {
       uint32_t raw[16];
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
@@ -109,14 +114,16 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
       }
     }
   } else {
-    for (int px = tid & 127; px < kPix; px += (NW == 1 ? 64 : 128)) {
-      const int cg0 = NW == 1 ? 0 : tid >> 7;
+    constexpr int kPxStep = kThreads < KP ? kThreads : KP;  // pixels covered per pass
+    constexpr int kCgStep = kThreads / kPxStep;
+    for (int px = tid % kPxStep; px < kPix; px += kPxStep) {
+      const int cg0 = tid / kPxStep;
       const long long q0 = q_base + px;
       const bool live = q0 < a.Q;
       const long long n = live ? q0 / a.HW : 0;
       const int p = live ? static_cast<int>(q0 - n * a.HW) : 0;
       const uint8_t* src = a.x + (static_cast<size_t>(n) * a.C) * a.HW + p;
-      for (int cg = cg0; cg < a.cp / 16; cg += (NW == 1 ? 1 : 2)) {
+      for (int cg = cg0; cg < a.cp / 16; cg += kCgStep) {
         uint32_t w[4] = {0, 0, 0, 0};
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
@@ -135,7 +142,7 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
   const int t_end = min(t_begin + a.tiles_per_wg, a.oc_tiles);
   // wavefront w takes items w, w + NW, ...; with kParts | NW its pixel part never changes
   const int part = wave % kParts;
-  const int tile_step = NW / kParts > 0 ? NW / kParts : 1;
+  constexpr int tile_step = NW / kParts > 0 ? NW / kParts : 1;
   const int tile0 = t_begin + wave / kParts;
   const int n_tiles = tile0 < t_end ? (t_end - tile0 + tile_step - 1) / tile_step : 0;
   if (NW > 1) __syncthreads();  // the input tile is complete; nothing below needs the other wavefronts
@@ -266,48 +273,52 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
 
 struct Plan {
   PwArgs a;
-  int lds_bytes, nw, pt, gran, zp, rq;
+  int lds_bytes, kp, nw, pt, gran, zp, rq;
   dim3 grid;
 };
 
-template <int NW, int PT, int GRAN, bool ZP, int RQ>
+template <int KP, int NW, int PT, int GRAN, bool ZP, int RQ>
 int Launch(const Plan* plan, const PwArgs& a, hipStream_t st, bool configure) {
   if (configure) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&PwConvKernel<NW, PT, GRAN, ZP, RQ>),
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&PwConvKernel<KP, NW, PT, GRAN, ZP, RQ>),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, plan->lds_bytes);
     if (e != hipSuccess)
       return SetError(TVX_E_DEVICE, "hipFuncSetAttribute(dynamic LDS %d): %s", plan->lds_bytes, hipGetErrorString(e));
     return TVX_OK;
   }
-  hipLaunchKernelGGL((PwConvKernel<NW, PT, GRAN, ZP, RQ>), plan->grid, dim3(64 * NW), plan->lds_bytes, st, a);
+  hipLaunchKernelGGL((PwConvKernel<KP, NW, PT, GRAN, ZP, RQ>), plan->grid, dim3(64 * NW), plan->lds_bytes, st, a);
   return TVX_OK;
 }
 
-template <int NW, int PT, int GRAN, bool ZP>
+template <int KP, int NW, int PT, int GRAN, bool ZP>
 int DispatchRq(const Plan* plan, const PwArgs& a, hipStream_t st, bool configure) {
-  if (plan->rq == kRqFastNoTie) return Launch<NW, PT, GRAN, ZP, kRqFastNoTie>(plan, a, st, configure);
-  if (plan->rq == kRqFast) return Launch<NW, PT, GRAN, ZP, kRqFast>(plan, a, st, configure);
-  return Launch<NW, PT, GRAN, ZP, kRqGeneric>(plan, a, st, configure);
+  if (plan->rq == kRqFastNoTie) return Launch<KP, NW, PT, GRAN, ZP, kRqFastNoTie>(plan, a, st, configure);
+  if (plan->rq == kRqFast) return Launch<KP, NW, PT, GRAN, ZP, kRqFast>(plan, a, st, configure);
+  return Launch<KP, NW, PT, GRAN, ZP, kRqGeneric>(plan, a, st, configure);
 }
 
-template <int NW, int PT, int GRAN>
+template <int KP, int NW, int PT, int GRAN>
 int DispatchZp(const Plan* plan, const PwArgs& a, hipStream_t st, bool configure) {
-  return plan->zp ? DispatchRq<NW, PT, GRAN, true>(plan, a, st, configure)
-                  : DispatchRq<NW, PT, GRAN, false>(plan, a, st, configure);
+  return plan->zp ? DispatchRq<KP, NW, PT, GRAN, true>(plan, a, st, configure)
+                  : DispatchRq<KP, NW, PT, GRAN, false>(plan, a, st, configure);
 }
 
-template <int NW, int PT>
+template <int KP, int NW, int PT>
 int DispatchGran(const Plan* plan, const PwArgs& a, hipStream_t st, bool configure) {
-  if (plan->gran == 16) return DispatchZp<NW, PT, 16>(plan, a, st, configure);
-  if (plan->gran == 4) return DispatchZp<NW, PT, 4>(plan, a, st, configure);
-  return DispatchZp<NW, PT, 1>(plan, a, st, configure);
+  if (plan->gran == 16) return DispatchZp<KP, NW, PT, 16>(plan, a, st, configure);
+  if (plan->gran == 4) return DispatchZp<KP, NW, PT, 4>(plan, a, st, configure);
+  return DispatchZp<KP, NW, PT, 1>(plan, a, st, configure);
 }
 
 int Dispatch(const Plan* plan, const PwArgs& a, hipStream_t st, bool configure) {
-  if (plan->nw == 1) return DispatchGran<1, 4>(plan, a, st, configure);
-  if (plan->pt == 4) return DispatchGran<4, 4>(plan, a, st, configure);
-  if (plan->pt == 2) return DispatchGran<4, 2>(plan, a, st, configure);
-  return DispatchGran<4, 1>(plan, a, st, configure);
+  if (plan->kp == 32) {
+    if (plan->nw == 1) return DispatchGran<32, 1, 1>(plan, a, st, configure);
+    return DispatchGran<32, 4, 1>(plan, a, st, configure);
+  }
+  if (plan->nw == 1) return DispatchGran<128, 1, 4>(plan, a, st, configure);
+  if (plan->pt == 4) return DispatchGran<128, 4, 4>(plan, a, st, configure);
+  if (plan->pt == 2) return DispatchGran<128, 4, 2>(plan, a, st, configure);
+  return DispatchGran<128, 4, 1>(plan, a, st, configure);
 }
 
 int PwConvRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
@@ -345,11 +356,18 @@ int PwConvSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const 
   a.ksteps = a.cp / 32;
   a.pix_stride = a.cp + 16;
   a.oc_tiles = (a.OC + 31) / 32;
-  // a shallow input (tile of a few KiB): one wavefront per workgroup, many tiles in flight
-  const int nw = kPix * a.pix_stride <= 20 * 1024 ? 1 : 4;
-  const int lds_bytes = kPix * a.pix_stride + nw * kStageBytes;
+  // few pixels in the whole batch: 32-pixel workgroups, four times as many
+  int kp = a.Q < 128 * 1024 ? 32 : 128;
+  // a shallow input (its tile is loaded in one or two passes by a single wavefront): one
+  // wavefront per workgroup, no barrier, many tiles in flight per CU
+  int nw = a.cp / 16 <= (kp == 128 ? 4 : 16) ? 1 : 4;
+  if (const char* f = getenv("TVX_PWCONV_SHAPE")) {  // tuning aid: "<pixels per workgroup>,<wavefronts>"
+    int fk = 0, fn = 0;
+    if (sscanf(f, "%d,%d", &fk, &fn) == 2 && (fk == 32 || fk == 128) && (fn == 1 || fn == 4)) { kp = fk; nw = fn; }
+  }
+  const int lds_bytes = kp * a.pix_stride + nw * kStageBytes;
   if (lds_bytes > 160 * 1024) return TVX_E_UNSUPPORTED;
-  const long long gx = (a.Q + kPix - 1) / kPix;
+  const long long gx = (a.Q + kp - 1) / kp;
   if (gx > 0x7fffffffll) return TVX_E_UNSUPPORTED;
   const bool x_u8 = d->in_dtype == TVX_U8, w_u8 = d->w_dtype == TVX_U8;
   const int zxs = d->in_zp - (x_u8 ? 128 : 0);
@@ -368,7 +386,7 @@ int PwConvSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const 
   a.tiles_per_wg = std::min(((quads + gy - 1) / gy) * nw, a.oc_tiles);
   gy = (a.oc_tiles + a.tiles_per_wg - 1) / a.tiles_per_wg;
   // fewer output tiles than wavefronts: split the pixels of a tile over wavefronts instead
-  const int pt = nw == 1 ? 4 : (a.tiles_per_wg >= 4 ? 4 : (a.tiles_per_wg >= 2 ? 2 : 1));
+  const int pt = kp == 32 ? 1 : (nw == 1 ? 4 : (a.tiles_per_wg >= 4 ? 4 : (a.tiles_per_wg >= 2 ? 2 : 1)));
 
   // ---- weights in fragment order, constants folded into the bias -------------------
   const int oc_alloc = a.oc_tiles * 32;
@@ -402,6 +420,7 @@ int PwConvSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const 
   Plan plan;
   plan.a = a;
   plan.lds_bytes = lds_bytes;
+  plan.kp = kp;
   plan.nw = nw;
   plan.pt = pt;
   plan.gran = (a.HW % 16 == 0) ? 16 : ((a.HW % 4 == 0) ? 4 : 1);
