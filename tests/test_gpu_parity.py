@@ -312,8 +312,35 @@ def test_depthwise3x3_shapes(oracle, gi, mode):
     fast = kws["out_shape"][0] % 4 == 0
     for act in (0, 2):
         want = oracle.conv2d(x, wt, b, act=act, **kws)
-        got = TC.gpu_conv2d(x, wt, b, act=act, want_kernel="dwconv3x3_i8" if fast else "conv2d_generic", **kws)
+        got = TC.gpu_conv2d(x, wt, b, act=act, want_kernel="dwconv3x3_i8" if fast else "dwconv_planes_i8", **kws)
         assert np.array_equal(got, want)
+    assert len(np.unique(want)) > 4
+
+
+DWP_GRID = [
+    # (n, c, h, w, kh, kw, stride, dil, pad[l,r,t,b]): widths 14 / 7 / odd, 5x5 and 1x3 kernels,
+    # dilation, asymmetric padding, a plane count that leaves a ragged last workgroup
+    (4, 24, 14, 14, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),
+    (3, 40, 7, 7, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),
+    (2, 19, 14, 14, 3, 3, [2, 2], [1, 1], [0, 1, 0, 1]),
+    (1, 7, 9, 11, 5, 5, [1, 1], [1, 1], [2, 2, 2, 2]),
+    (2, 5, 13, 6, 3, 3, [1, 2], [2, 2], [2, 2, 2, 2]),
+    (1, 3, 5, 9, 1, 3, [1, 1], [1, 1], [1, 1, 0, 0]),
+    (70, 33, 7, 7, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),
+]
+
+
+@pytest.mark.parametrize("mode", ["u8", "i8pc", "u8pc"])
+@pytest.mark.parametrize("gi", range(len(DWP_GRID)))
+def test_depthwise_planes_shapes(oracle, gi, mode):
+    n, c, h, w, kh, kw, stride, dil, pad = DWP_GRID[gi]
+    rng = np.random.default_rng(5000 + gi)
+    x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=0, kh=kh, kw=kw, stride=stride, dil=dil,
+                              pad=pad, mult=1, mode=mode)
+    for act in (0, 2):
+        want = oracle.conv2d(x, wt, b, act=act, **kws)
+        got = TC.gpu_conv2d(x, wt, b, act=act, want_kernel="dwconv_planes_i8", **kws)
+        assert np.array_equal(got, want), int((got != want).sum())
     assert len(np.unique(want)) > 4
 
 

@@ -34,6 +34,9 @@ int PwConvSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 // depthwise 3x3 stencil (dwconv3x3_i8.hip)
 int DwConv3x3Setup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 
+// depthwise, any kernel / width, planes staged through LDS (dwconv_planes_i8.hip)
+int DwPlanesSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
+
 // generic (kernels_generic.hip)
 int ConvGenericSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 int FcGenericSetup(tvx_op*, const tvx_fc_desc*, const void*, const void*);
