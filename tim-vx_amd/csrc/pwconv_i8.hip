@@ -85,23 +85,86 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
   int8_t* xl = lds;
   int8_t* stage = lds + kPix * a.pix_stride + wave * kStageBytes;
 
+  // ---- work items of this wavefront: (output tile, pixel part) ---------------------------
+  const int t_begin = blockIdx.y * a.tiles_per_wg;
+  const int t_end = min(t_begin + a.tiles_per_wg, a.oc_tiles);
+  // wavefront w takes items w, w + NW, ...; with kParts | NW its pixel part never changes
+  const int part = wave % kParts;
+  constexpr int tile_step = NW / kParts > 0 ? NW / kParts : 1;
+  const int tile0 = t_begin + wave / kParts;
+  const int n_tiles = tile0 < t_end ? (t_end - tile0 + tile_step - 1) / tile_step : 0;
+
+  const int total = n_tiles * a.ksteps;
+
+  // weight fragment stream, in consumption order
+  int pf_tile = n_tiles > 0 ? tile0 : 0, pf_ks = 0, pf_left = total;
+  auto next_frag = [&]() -> v4i {
+    const v4i f = a.wpk[(static_cast<size_t>(pf_tile) * a.ksteps + pf_ks) * 64 + lane];
+    if (--pf_left > 0) {  // past the end: keep re-reading the last fragment
+      if (++pf_ks == a.ksteps) { pf_ks = 0; pf_tile += tile_step; }
+    }
+    return f;
+  };
+
+  // the first weight fragments travel while the input tile is being built
+  v4i f0 = next_frag();
+  v4i f1 = next_frag();
+
   // ---- activations of the 128 pixels, all channels: global (pixel-innermost) -> LDS
-  if (GRAN >= 4) {
+  {
+    // A thread takes a group of 4 consecutive flat pixels and 16 channels per pass: 16 dword
+    // loads in flight, 4x4 byte transposes, four 16-byte LDS stores. With GRAN 1 a group may
+    // start at any byte (the dword loads are then unaligned, which global memory allows) and
+    // may straddle two images or the end of the batch.
     constexpr int kQuads = KP / 4;
     const int pq = tid % kQuads, cg0 = tid / kQuads;  // 4-pixel group, first 16-channel group
     const long long q0 = q_base + pq * 4;
     const bool live = q0 < a.Q;
     const long long n = live ? q0 / a.HW : 0;
     const int p = live ? static_cast<int>(q0 - n * a.HW) : 0;
+    const bool whole = GRAN >= 4 ? live : (q0 + 3 < a.Q && p + 3 < a.HW);
     const uint8_t* src = a.x + (static_cast<size_t>(n) * a.C) * a.HW + p;
+    // GRAN 1, group straddling two images (or the end of the batch): its first k pixels end
+    // image n, the rest start image n + 1. Both parts are fetched as unaligned dwords - the
+    // second one shifted so that its bytes land in lanes k..3 - and merged with a byte mask.
+    // The bytes such a dword reads outside its own row belong to neighbouring rows of the
+    // tensor, except behind the very last row, which is therefore read byte by byte.
+    const int k_first = GRAN == 1 && live && !whole ? a.HW - p : 4;
+    const uint32_t mask_first = k_first >= 4 ? 0xffffffffu : ((1u << (8 * k_first)) - 1u);
+    const bool has_second = GRAN == 1 && live && !whole && q0 + k_first < a.Q;
+    const uint8_t* src2 = has_second ? a.x + (static_cast<size_t>(n + 1) * a.C) * a.HW - k_first : src;
+    const bool last_image = GRAN == 1 && live && !whole && (n + 1) * static_cast<long long>(a.HW) >= a.Q;
+    const bool any_split = GRAN == 1 && __any(live && !whole);
     for (int cg = cg0; cg < a.cp / 16; cg += kThreads / kQuads) {
       uint32_t raw[16];
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
         const int c = cg * 16 + j;
-        raw[j] = (live && c < a.C)
-                     ? *reinterpret_cast<const uint32_t*>(src + static_cast<size_t>(c) * a.HW) ^ a.xor_mask
-                     : 0u;
+        uint32_t v = 0;
+        if (live && c < a.C) {
+          const uint8_t* row = src + static_cast<size_t>(c) * a.HW;
+          if (GRAN >= 4) {
+            v = *reinterpret_cast<const uint32_t*>(row);
+          } else if (last_image && c == a.C - 1) {
+            for (int e = 0; e < k_first; ++e) v |= static_cast<uint32_t>(row[e]) << (8 * e);
+          } else {
+            __builtin_memcpy(&v, row, 4);
+          }
+          v ^= a.xor_mask;
+        }
+        raw[j] = v;
+      }
+      if (any_split) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          const int c = cg * 16 + j;
+          uint32_t v = 0;
+          if (has_second && c < a.C) {
+            __builtin_memcpy(&v, src2 + static_cast<size_t>(c) * a.HW, 4);
+            v ^= a.xor_mask;
+          }
+          raw[j] = (raw[j] & mask_first) | (v & ~mask_first);
+        }
       }
       uint32_t t[4][4];
 #pragma unroll
@@ -113,72 +176,39 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
         *reinterpret_cast<v4i*>(xl + (pq * 4 + e) * a.pix_stride + cg * 16) = v;
       }
     }
-  } else {
-    constexpr int kPxStep = kThreads < KP ? kThreads : KP;  // pixels covered per pass
-    constexpr int kCgStep = kThreads / kPxStep;
-    for (int px = tid % kPxStep; px < kPix; px += kPxStep) {
-      const int cg0 = tid / kPxStep;
-      const long long q0 = q_base + px;
-      const bool live = q0 < a.Q;
-      const long long n = live ? q0 / a.HW : 0;
-      const int p = live ? static_cast<int>(q0 - n * a.HW) : 0;
-      const uint8_t* src = a.x + (static_cast<size_t>(n) * a.C) * a.HW + p;
-      for (int cg = cg0; cg < a.cp / 16; cg += kCgStep) {
-        uint32_t w[4] = {0, 0, 0, 0};
-#pragma unroll
-        for (int j = 0; j < 16; ++j) {
-          const int c = cg * 16 + j;
-          const uint32_t b = (live && c < a.C) ? (src[static_cast<size_t>(c) * a.HW] ^ (a.xor_mask & 0xff)) : 0u;
-          w[j >> 2] |= b << (8 * (j & 3));
-        }
-        v4i v = {static_cast<int>(w[0]), static_cast<int>(w[1]), static_cast<int>(w[2]), static_cast<int>(w[3])};
-        *reinterpret_cast<v4i*>(xl + px * a.pix_stride + cg * 16) = v;
-      }
-    }
   }
 
-  // ---- work items of this wavefront: (output tile, pixel part) ---------------------------
-  const int t_begin = blockIdx.y * a.tiles_per_wg;
-  const int t_end = min(t_begin + a.tiles_per_wg, a.oc_tiles);
-  // wavefront w takes items w, w + NW, ...; with kParts | NW its pixel part never changes
-  const int part = wave % kParts;
-  constexpr int tile_step = NW / kParts > 0 ? NW / kParts : 1;
-  const int tile0 = t_begin + wave / kParts;
-  const int n_tiles = tile0 < t_end ? (t_end - tile0 + tile_step - 1) / tile_step : 0;
   if (NW > 1) __syncthreads();  // the input tile is complete; nothing below needs the other wavefronts
   if (n_tiles <= 0) return;
 
   // ---- where this lane's output groups live (the same for every output tile) -----
   // Copy-out mapping of a staged row of kRowBytes pixels: GRAN 16: lane -> 16-pixel chunk
-  // lane % (kRowBytes/16); GRAN 4: dword lane % (kRowBytes/4); GRAN 1: pixel lane % kRowBytes (+64).
-  constexpr int kPerRow = GRAN == 16 ? kRowBytes / 16 : (GRAN == 4 ? kRowBytes / 4 : (kRowBytes < 64 ? kRowBytes : 64));
-  constexpr int kGroups = (GRAN == 1 && kRowBytes > 64) ? 2 : 1;
+  // lane % (kRowBytes/16); GRAN 4 and 1: 4-pixel group lane % (kRowBytes/4), which with
+  // GRAN 1 may be unaligned or straddle two images (then stored byte by byte).
+  constexpr int kUnit = GRAN == 16 ? 16 : 4;
+  constexpr int kPerRow = kRowBytes / kUnit;
   constexpr int kRowsPerIter = 64 / kPerRow;
-  const int px_in_row = (lane % kPerRow) * GRAN;
-  size_t out_off[kGroups];
-  bool out_live[kGroups];
+  const int px_in_row = (lane % kPerRow) * kUnit;
+  const long long oq0 = q_base + part * kRowBytes + px_in_row;
+  const bool out_live = oq0 < a.Q;
+  const long long on = out_live ? oq0 / a.HW : 0;
+  const int op0 = out_live ? static_cast<int>(oq0 - on * a.HW) : 0;
+  const size_t out_off = static_cast<size_t>(on) * a.OC * a.HW + static_cast<size_t>(op0);
+  const bool out_whole = GRAN >= 4 ? out_live : (oq0 + 3 < a.Q && op0 + 3 < a.HW);
+  size_t out_px_off[4] = {0, 0, 0, 0};
+  bool out_px_live[4] = {false, false, false, false};
+  if (GRAN == 1 && out_live && !out_whole) {
 #pragma unroll
-  for (int g = 0; g < kGroups; ++g) {
-    const long long q0 = q_base + part * kRowBytes + px_in_row + 64 * g;
-    out_live[g] = q0 < a.Q;
-    const long long n = out_live[g] ? q0 / a.HW : 0;
-    out_off[g] = static_cast<size_t>(n) * a.OC * a.HW + static_cast<size_t>(q0 - n * a.HW);
+    for (int e = 0; e < 4; ++e) {
+      const long long qe = oq0 + e;
+      out_px_live[e] = qe < a.Q;
+      const long long ne = out_px_live[e] ? qe / a.HW : 0;
+      out_px_off[e] = static_cast<size_t>(ne) * a.OC * a.HW + static_cast<size_t>(qe - ne * a.HW);
+    }
   }
 
   const int frag_row = lane & 31, frag_half = lane >> 5;
   const int8_t* xa = xl + (part * kRowBytes + frag_row) * a.pix_stride + frag_half * 16;
-  const int total = n_tiles * a.ksteps;
-
-  // weight fragment stream, in consumption order
-  int pf_tile = tile0, pf_ks = 0, pf_left = total;
-  auto next_frag = [&]() -> v4i {
-    const v4i f = a.wpk[(static_cast<size_t>(pf_tile) * a.ksteps + pf_ks) * 64 + lane];
-    if (--pf_left > 0) {  // past the end: keep re-reading the last fragment
-      if (++pf_ks == a.ksteps) { pf_ks = 0; pf_tile += tile_step; }
-    }
-    return f;
-  };
-
   v16i acc[PT];
   int tile = tile0, ks = 0;
   auto init_acc = [&]() {
@@ -215,25 +245,26 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
         const int8_t* s = stage + row * kStageStride + px_in_row;
         const uint2 lo8 = *reinterpret_cast<const uint2*>(s);
         const uint2 hi8 = *reinterpret_cast<const uint2*>(s + 8);
-        if (row < rows && out_live[0])
-          *reinterpret_cast<uint4*>(ybase + out_off[0] + static_cast<size_t>(row) * a.HW) =
+        if (row < rows && out_live)
+          *reinterpret_cast<uint4*>(ybase + out_off + static_cast<size_t>(row) * a.HW) =
               make_uint4(lo8.x, lo8.y, hi8.x, hi8.y);
       }
-    } else if (GRAN == 4) {
+    } else {
 #pragma unroll
       for (int i = 0; i < 32 / kRowsPerIter; ++i) {
         const int row = lane / kPerRow + kRowsPerIter * i;
         const uint32_t v = *reinterpret_cast<const uint32_t*>(stage + row * kStageStride + px_in_row);
-        if (row < rows && out_live[0])
-          *reinterpret_cast<uint32_t*>(ybase + out_off[0] + static_cast<size_t>(row) * a.HW) = v;
-      }
-    } else {
-      for (int row = lane / kPerRow; row < rows; row += kRowsPerIter)
+        if (row < rows && out_whole) {
+          uint8_t* o = ybase + out_off + static_cast<size_t>(row) * a.HW;
+          if (GRAN == 4) *reinterpret_cast<uint32_t*>(o) = v;
+          else __builtin_memcpy(o, &v, 4);
+        } else if (GRAN == 1 && row < rows) {
 #pragma unroll
-        for (int g = 0; g < kGroups; ++g)
-          if (out_live[g])
-            ybase[out_off[g] + static_cast<size_t>(row) * a.HW] =
-                static_cast<uint8_t>(stage[row * kStageStride + px_in_row + 64 * g]);
+          for (int e = 0; e < 4; ++e)
+            if (out_px_live[e])
+              ybase[out_px_off[e] + static_cast<size_t>(row) * a.HW] = static_cast<uint8_t>(v >> (8 * e));
+        }
+      }
     }
     __builtin_amdgcn_wave_barrier();
   };
@@ -256,8 +287,6 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
     }
   };
 
-  v4i f0 = next_frag();
-  v4i f1 = next_frag();
   init_acc();
   for (int idx = 0; idx < total; idx += 2) {
     const v4i g0 = f0;
@@ -349,7 +378,7 @@ int PwConvSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const 
   a.C = d->in_c;
   a.OC = d->out_c;
   const uint64_t hw = static_cast<uint64_t>(d->in_w) * d->in_h;
-  if (hw >= (1ull << 30)) return TVX_E_UNSUPPORTED;
+  if (hw >= (1ull << 30) || hw < 4) return TVX_E_UNSUPPORTED;  // a 4-pixel group spans at most two images
   a.HW = static_cast<int>(hw);
   a.Q = static_cast<long long>(hw) * d->batch;
   a.cp = RoundUp(a.C, 32);
@@ -382,7 +411,11 @@ int PwConvSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const 
   // few pixel tiles: spread the output tiles over grid.y (in units of one tile per
   // wavefront) until the launch has a few workgroups per CU
   const int quads = (a.oc_tiles + nw - 1) / nw;
-  int gy = static_cast<int>(std::min<long long>(quads, std::max<long long>(1, 1024 / gx)));
+  // enough workgroups to give every SIMD several wavefronts; re-reading the small input
+  // tile per output-tile group is cheap next to walking many output tiles in sequence
+  long long want_wgs = nw == 1 ? 4096 : 2048;
+  if (const char* f = getenv("TVX_PWCONV_WGS")) want_wgs = std::max(1, atoi(f));  // tuning aid
+  int gy = static_cast<int>(std::min<long long>(quads, std::max<long long>(1, want_wgs / gx)));
   a.tiles_per_wg = std::min(((quads + gy - 1) / gy) * nw, a.oc_tiles);
   gy = (a.oc_tiles + a.tiles_per_wg - 1) / a.tiles_per_wg;
   // fewer output tiles than wavefronts: split the pixels of a tile over wavefronts instead
