@@ -240,6 +240,12 @@ IGEMM_GRID = [
     (1, 20, 8, 8, 50, 5, 5, [1, 1], [1, 1], [0, 0, 0, 0]),
     (3, 64, 7, 7, 160, 3, 3, [2, 1], [1, 1], [1, 1, 1, 1]),
     (1, 24, 13, 20, 144, 1, 1, [1, 1], [1, 1], [0, 0, 0, 0]),
+    # weights + halo beyond one LDS load: the reduction runs in channel groups
+    (1, 128, 14, 14, 160, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),
+    (2, 256, 7, 7, 64, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),
+    (1, 200, 9, 9, 40, 3, 3, [2, 2], [1, 1], [1, 1, 1, 1]),
+    (1, 96, 10, 12, 256, 5, 5, [1, 1], [1, 1], [2, 2, 2, 2]),
+    (1, 528, 6, 6, 32, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),
 ]
 
 

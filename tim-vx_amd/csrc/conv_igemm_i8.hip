@@ -42,7 +42,9 @@ struct ConvArgs {
   const int2* tapt;      // per (k-step, fragment half): {halo byte offset of the chunk, dot4 multiplier}
   int C, H, W, OC, OH, OW;
   int kh, kw, sh, sw, dh, dw, pad_t, pad_l;
-  int cp, cpc;           // channels padded to 16, and 16-byte chunks per pixel
+  int cp, cpc;           // channels of one reduction group padded to 16, and 16-byte chunks per pixel
+  int groups;            // reduction groups: the input channels are walked cp at a time
+  int w_group_stride;    // bytes between the packed weights of consecutive groups
   int ksteps, kstride;
   int P, PT, tiles_per_image, oct;
   int iht, iwt;          // halo tile extent
@@ -64,9 +66,9 @@ __device__ __forceinline__ int HaloOffset(const ConvArgs& a, int hp, int c) {
   return hp * a.pix_stride + c;
 }
 
-__device__ __forceinline__ int ChannelFill(const ConvArgs& a, int c) {
+__device__ __forceinline__ int ChannelFill(const ConvArgs& a, int c, int c_real) {
   // zero-point bytes for real channels, zero for the padding up to 16
-  const int n = a.C - c;  // real channels left in this group of four
+  const int n = c_real - c;  // real channels left in this group of four
   if (n >= 4) return a.pad_fill;
   if (n <= 0) return 0;
   return a.pad_fill & ((1 << (8 * n)) - 1);
@@ -91,127 +93,9 @@ __global__ void __launch_bounds__(kThreads) ConvIgemmKernel(ConvArgs a) {
   int8_t* halo = lds + a.off_halo;
   int* sx_lds = reinterpret_cast<int*>(lds + a.off_sx);
 
-  // ---- weights of this channel block: global -> LDS DMA, 1 KiB per wave instruction
-  {
-    const int8_t* src = a.w + static_cast<size_t>(oc0) * a.kstride;
-    for (int i = wave * 64; i < a.w_chunks; i += kThreads) {
-      __builtin_amdgcn_global_load_lds(
-          (const __attribute__((address_space(1))) void*)(src + static_cast<size_t>(i + lane) * 16),
-          (__attribute__((address_space(3))) void*)(w_lds + i * 16), 16, 0, 0);
-    }
-  }
   // the reduction order as a table (built once per operator): no index math in the main loop
   int2* tap_lds = reinterpret_cast<int2*>(lds + a.off_tap);
   for (int i = tid; i < a.ksteps * 2 + 2; i += kThreads) tap_lds[i] = a.tapt[i];
-  // ---- halo tile -------------------------------------------------------------
-  const size_t plane = static_cast<size_t>(a.H) * a.W;
-  const uint8_t* xin = a.x + static_cast<size_t>(n) * a.C * plane;
-  const int c4n = a.cp / 4;
-  if ((a.W & 3) == 0) {
-    // A thread owns one (4 input columns, 4 channels) patch and walks the halo
-    // rows with it, kLoadBatch rows of loads in flight; lanes run over channel
-    // groups first so that a wavefront's LDS stores spread over the banks.
-    const int w4n = a.W / 4;
-    const int patches = a.w4_blocks * ((c4n + 3) / 4) * 64;
-    const uint32_t plane32 = static_cast<uint32_t>(plane);
-    const int row_bytes = a.iwt * a.pix_stride;
-    for (int pi = tid; pi < patches; pi += kThreads) {
-      // patch index -> (column group, channel group): 16 consecutive lanes read 64
-      // contiguous bytes of one channel row, the next 16 lanes the next channel group
-      const int blk = pi >> 6, in_blk = pi & 63;
-      int w4 = (blk % a.w4_blocks) * 16 + (in_blk & 15);
-      int c4 = (blk / a.w4_blocks) * 4 + (in_blk >> 4);
-      if (w4 >= w4n || c4 >= c4n) continue;
-      const int c = c4 * 4;
-      const int hc = a.pad_l + w4 * 4;
-      // byte offsets of the patch's four channel rows inside this image (< 2^31)
-      uint32_t src_off[4];
-      int fill[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const bool real = c + j < a.C;
-        src_off[j] = static_cast<uint32_t>(real ? c + j : 0) * plane32 + static_cast<uint32_t>(w4 * 4);
-        fill[j] = real ? a.pad_fill : 0;
-      }
-      const int xm = a.xor_mask;
-      int xmask[4];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) xmask[j] = c + j < a.C ? xm : 0;
-      const int dst0 = __mul24(hc, a.pix_stride) + c;
-      // columns of this patch that exist in the halo tile (stride > 1 may cut the right edge)
-      const int ncols = min(4, a.iwt - hc);
-      for (int hr0 = 0; hr0 < rows_needed; hr0 += kLoadBatch) {
-        int d[kLoadBatch][4];
-#pragma unroll
-        for (int b = 0; b < kLoadBatch; ++b) {
-          const int ih = ih0 + hr0 + b;
-          const bool inside = hr0 + b < rows_needed && ih >= 0 && ih < a.H;
-          const uint32_t row_off = __umul24(static_cast<uint32_t>(inside ? ih : 0), static_cast<uint32_t>(a.W));
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            // out-of-image rows load row 0 (in bounds) and are replaced by the zero point
-            const int v = *reinterpret_cast<const int*>(xin + (src_off[j] + row_off));
-            d[b][j] = inside ? (c + j < a.C ? v ^ xmask[j] : 0) : fill[j];
-          }
-        }
-#pragma unroll
-        for (int b = 0; b < kLoadBatch; ++b) {
-          if (hr0 + b >= rows_needed) continue;
-          // 4 x 4 byte transpose: d[j] = 4 pixels of channel c+j  ->  px[i] = 4 channels of pixel i
-          const int lo01 = __builtin_amdgcn_perm(d[b][1], d[b][0], 0x05010400);
-          const int hi01 = __builtin_amdgcn_perm(d[b][1], d[b][0], 0x07030602);
-          const int lo23 = __builtin_amdgcn_perm(d[b][3], d[b][2], 0x05010400);
-          const int hi23 = __builtin_amdgcn_perm(d[b][3], d[b][2], 0x07030602);
-          int px[4];
-          px[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100);
-          px[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302);
-          px[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100);
-          px[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302);
-          int8_t* dst = halo + dst0 + __mul24(hr0 + b, row_bytes);
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            if (i < ncols) *reinterpret_cast<int*>(dst + __mul24(i, a.pix_stride)) = px[i];
-        }
-      }
-    }
-  } else {
-    // general width: one (halo row, column, 4 channels) dword at a time
-    const int units = rows_needed * a.W * c4n;
-    for (int u = tid; u < units; u += kThreads) {
-      const int c4 = u % c4n;
-      const int iw = (u / c4n) % a.W;
-      const int hr = u / (c4n * a.W);
-      if (a.pad_l + iw >= a.iwt) continue;
-      const int ih = ih0 + hr;
-      const int c = c4 * 4;
-      int v = ChannelFill(a, c);
-      if (ih >= 0 && ih < a.H) {
-        v = 0;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          if (c + j >= a.C) continue;
-          const int b = xin[(c + j) * plane + static_cast<size_t>(ih) * a.W + iw] ^ (a.xor_mask & 0xff);
-          v |= b << (8 * j);
-        }
-      }
-      *reinterpret_cast<int*>(halo + HaloOffset(a, hr * a.iwt + a.pad_l + iw, c)) = v;
-    }
-  }
-  // left / right padding columns: one (halo row, pad column) per step of a thread
-  {
-    const int right0 = a.pad_l + a.W;
-    const int pad_cols = a.pad_l + max(a.iwt - right0, 0);
-    const int cells = rows_needed * pad_cols;
-    for (int cell = tid; cell < cells; cell += kThreads) {
-      const int hr = cell / pad_cols, pc = cell - hr * pad_cols;
-      const int hc = pc < a.pad_l ? pc : right0 + (pc - a.pad_l);
-      int8_t* dst = halo + (hr * a.iwt + hc) * a.pix_stride;
-      for (int c = 0; c < a.cp; c += 4) *reinterpret_cast<int*>(dst + c) = ChannelFill(a, c);
-    }
-  }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the weight DMA has landed
-  __syncthreads();
-
   // ---- main loop ---------------------------------------------------------------
   const int frag_row = lane & 31, frag_half = lane >> 5;
   int a_base[kMaxPtw];  // byte offset of each pixel's window origin in the halo tile (+ this lane's half)
@@ -240,51 +124,176 @@ __global__ void __launch_bounds__(kThreads) ConvIgemmKernel(ConvArgs a) {
   }
   int sx[kMaxPtw] = {0, 0};
 
-  // Every wavefront runs the same instruction stream: a wavefront whose second
-  // pixel tile lies beyond the workgroup's tile computes it anyway (on pixel 0)
-  // and drops the result. A k-step's chunk position comes from the tap table; the
-  // padding chunk of an odd chunk count meets zero weights and carries a zero dot4
-  // multiplier, which keeps it out of the pixel sum.
-  {
-    const int8_t* w_row = w_lds + frag_row * a.kstride + frag_half * 16;
-    const int2* my_tap = tap_lds + frag_half;
-
-    auto load_ab = [&](v4i* fa, v4i* fb, int ks, int2 t) {
-#pragma unroll
-      for (int i = 0; i < kMaxPtw; ++i)
-        fa[i] = *reinterpret_cast<const v4i*>(halo + a_base[i] + t.x);
-      // one k-step past the end reads bytes that exist in LDS and are never used
-#pragma unroll
-      for (int j = 0; j < OT; ++j)
-        fb[j] = *reinterpret_cast<const v4i*>(w_row + j * 32 * a.kstride + ks * 32);
-    };
-    auto step = [&](const v4i* fa, const v4i* fb, int ones) {
-#pragma unroll
-      for (int i = 0; i < kMaxPtw; ++i)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) sx[i] = __builtin_amdgcn_sdot4(fa[i][q], ones, sx[i], false);
-#pragma unroll
-      for (int j = 0; j < OT; ++j)
-#pragma unroll
-        for (int i = 0; i < kMaxPtw; ++i)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
-    };
-
-    v4i fa0[kMaxPtw], fb0[OT], fa1[kMaxPtw], fb1[OT];
-    int2 t0 = my_tap[0], t1 = my_tap[2];  // the table has one spare k-step at its end
-    load_ab(fa0, fb0, 0, t0);
-    int ks = 0;
-    for (; ks + 1 < a.ksteps; ks += 2) {
-      const int2 t2 = my_tap[(ks + 2) * 2];
-      load_ab(fa1, fb1, ks + 1, t1);
-      step(fa0, fb0, t0.y);
-      const int2 t3 = my_tap[(ks + 3) * 2];
-      load_ab(fa0, fb0, ks + 2, t2);
-      step(fa1, fb1, t1.y);
-      t0 = t2;
-      t1 = t3;
+  // ---- reduction groups: (weights, halo tile) of cp input channels at a time ------------
+  for (int g = 0; g < a.groups; ++g) {
+    const int c_base = g * a.cp;
+    const int c_real = min(a.C - c_base, a.cp);
+    if (g > 0) __syncthreads();  // everyone is done with the previous group's tiles
+    // ---- weights of this channel block: global -> LDS DMA, 1 KiB per wave instruction
+    {
+      const int8_t* src = a.w + static_cast<size_t>(g) * a.w_group_stride + static_cast<size_t>(oc0) * a.kstride;
+      for (int i = wave * 64; i < a.w_chunks; i += kThreads) {
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(src + static_cast<size_t>(i + lane) * 16),
+            (__attribute__((address_space(3))) void*)(w_lds + i * 16), 16, 0, 0);
+      }
     }
-    if (ks < a.ksteps) step(fa0, fb0, t0.y);
+    // ---- halo tile -------------------------------------------------------------
+    const size_t plane = static_cast<size_t>(a.H) * a.W;
+    const uint8_t* xin = a.x + static_cast<size_t>(n) * a.C * plane;
+    const int c4n = a.cp / 4;
+    if ((a.W & 3) == 0) {
+      // A thread owns one (4 input columns, 4 channels) patch and walks the halo
+      // rows with it, kLoadBatch rows of loads in flight; lanes run over channel
+      // groups first so that a wavefront's LDS stores spread over the banks.
+      const int w4n = a.W / 4;
+      const int patches = a.w4_blocks * ((c4n + 3) / 4) * 64;
+      const uint32_t plane32 = static_cast<uint32_t>(plane);
+      const int row_bytes = a.iwt * a.pix_stride;
+      for (int pi = tid; pi < patches; pi += kThreads) {
+        // patch index -> (column group, channel group): 16 consecutive lanes read 64
+        // contiguous bytes of one channel row, the next 16 lanes the next channel group
+        const int blk = pi >> 6, in_blk = pi & 63;
+        int w4 = (blk % a.w4_blocks) * 16 + (in_blk & 15);
+        int c4 = (blk / a.w4_blocks) * 4 + (in_blk >> 4);
+        if (w4 >= w4n || c4 >= c4n) continue;
+        const int c = c4 * 4;
+        const int hc = a.pad_l + w4 * 4;
+        // byte offsets of the patch's four channel rows inside this image (< 2^31)
+        uint32_t src_off[4];
+        int fill[4];
+  #pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const bool real = c + j < c_real;
+          src_off[j] = static_cast<uint32_t>(real ? c_base + c + j : 0) * plane32 + static_cast<uint32_t>(w4 * 4);
+          fill[j] = real ? a.pad_fill : 0;
+        }
+        const int xm = a.xor_mask;
+        int xmask[4];
+  #pragma unroll
+        for (int j = 0; j < 4; ++j) xmask[j] = c + j < c_real ? xm : 0;
+        const int dst0 = __mul24(hc, a.pix_stride) + c;
+        // columns of this patch that exist in the halo tile (stride > 1 may cut the right edge)
+        const int ncols = min(4, a.iwt - hc);
+        for (int hr0 = 0; hr0 < rows_needed; hr0 += kLoadBatch) {
+          int d[kLoadBatch][4];
+  #pragma unroll
+          for (int b = 0; b < kLoadBatch; ++b) {
+            const int ih = ih0 + hr0 + b;
+            const bool inside = hr0 + b < rows_needed && ih >= 0 && ih < a.H;
+            const uint32_t row_off = __umul24(static_cast<uint32_t>(inside ? ih : 0), static_cast<uint32_t>(a.W));
+  #pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              // out-of-image rows load row 0 (in bounds) and are replaced by the zero point
+              const int v = *reinterpret_cast<const int*>(xin + (src_off[j] + row_off));
+              d[b][j] = inside ? (c + j < c_real ? v ^ xmask[j] : 0) : fill[j];
+            }
+          }
+  #pragma unroll
+          for (int b = 0; b < kLoadBatch; ++b) {
+            if (hr0 + b >= rows_needed) continue;
+            // 4 x 4 byte transpose: d[j] = 4 pixels of channel c+j  ->  px[i] = 4 channels of pixel i
+            const int lo01 = __builtin_amdgcn_perm(d[b][1], d[b][0], 0x05010400);
+            const int hi01 = __builtin_amdgcn_perm(d[b][1], d[b][0], 0x07030602);
+            const int lo23 = __builtin_amdgcn_perm(d[b][3], d[b][2], 0x05010400);
+            const int hi23 = __builtin_amdgcn_perm(d[b][3], d[b][2], 0x07030602);
+            int px[4];
+            px[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100);
+            px[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302);
+            px[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100);
+            px[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302);
+            int8_t* dst = halo + dst0 + __mul24(hr0 + b, row_bytes);
+  #pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (i < ncols) *reinterpret_cast<int*>(dst + __mul24(i, a.pix_stride)) = px[i];
+          }
+        }
+      }
+    } else {
+      // general width: one (halo row, column, 4 channels) dword at a time
+      const int units = rows_needed * a.W * c4n;
+      for (int u = tid; u < units; u += kThreads) {
+        const int c4 = u % c4n;
+        const int iw = (u / c4n) % a.W;
+        const int hr = u / (c4n * a.W);
+        if (a.pad_l + iw >= a.iwt) continue;
+        const int ih = ih0 + hr;
+        const int c = c4 * 4;
+        int v = ChannelFill(a, c, c_real);
+        if (ih >= 0 && ih < a.H) {
+          v = 0;
+  #pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            if (c + j >= c_real) continue;
+            const int b = xin[(c_base + c + j) * plane + static_cast<size_t>(ih) * a.W + iw] ^ (a.xor_mask & 0xff);
+            v |= b << (8 * j);
+          }
+        }
+        *reinterpret_cast<int*>(halo + HaloOffset(a, hr * a.iwt + a.pad_l + iw, c)) = v;
+      }
+    }
+    // left / right padding columns: one (halo row, pad column) per step of a thread
+    {
+      const int right0 = a.pad_l + a.W;
+      const int pad_cols = a.pad_l + max(a.iwt - right0, 0);
+      const int cells = rows_needed * pad_cols;
+      for (int cell = tid; cell < cells; cell += kThreads) {
+        const int hr = cell / pad_cols, pc = cell - hr * pad_cols;
+        const int hc = pc < a.pad_l ? pc : right0 + (pc - a.pad_l);
+        int8_t* dst = halo + (hr * a.iwt + hc) * a.pix_stride;
+        for (int c = 0; c < a.cp; c += 4) *reinterpret_cast<int*>(dst + c) = ChannelFill(a, c, c_real);
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the weight DMA has landed
+    __syncthreads();
+
+    // Every wavefront runs the same instruction stream: a wavefront whose second
+    // pixel tile lies beyond the workgroup's tile computes it anyway (on pixel 0)
+    // and drops the result. A k-step's chunk position comes from the tap table; the
+    // padding chunk of an odd chunk count meets zero weights and carries a zero dot4
+    // multiplier, which keeps it out of the pixel sum.
+    {
+      const int8_t* w_row = w_lds + frag_row * a.kstride + frag_half * 16;
+      const int2* my_tap = tap_lds + frag_half;
+
+      auto load_ab = [&](v4i* fa, v4i* fb, int ks, int2 t) {
+  #pragma unroll
+        for (int i = 0; i < kMaxPtw; ++i)
+          fa[i] = *reinterpret_cast<const v4i*>(halo + a_base[i] + t.x);
+        // one k-step past the end reads bytes that exist in LDS and are never used
+  #pragma unroll
+        for (int j = 0; j < OT; ++j)
+          fb[j] = *reinterpret_cast<const v4i*>(w_row + j * 32 * a.kstride + ks * 32);
+      };
+      auto step = [&](const v4i* fa, const v4i* fb, int ones) {
+  #pragma unroll
+        for (int i = 0; i < kMaxPtw; ++i)
+  #pragma unroll
+          for (int q = 0; q < 4; ++q) sx[i] = __builtin_amdgcn_sdot4(fa[i][q], ones, sx[i], false);
+  #pragma unroll
+        for (int j = 0; j < OT; ++j)
+  #pragma unroll
+          for (int i = 0; i < kMaxPtw; ++i)
+            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+      };
+
+      v4i fa0[kMaxPtw], fb0[OT], fa1[kMaxPtw], fb1[OT];
+      int2 t0 = my_tap[0], t1 = my_tap[2];  // the table has one spare k-step at its end
+      load_ab(fa0, fb0, 0, t0);
+      int ks = 0;
+      for (; ks + 1 < a.ksteps; ks += 2) {
+        const int2 t2 = my_tap[(ks + 2) * 2];
+        load_ab(fa1, fb1, ks + 1, t1);
+        step(fa0, fb0, t0.y);
+        const int2 t3 = my_tap[(ks + 3) * 2];
+        load_ab(fa0, fb0, ks + 2, t2);
+        step(fa1, fb1, t1.y);
+        t0 = t2;
+        t1 = t3;
+      }
+      if (ks < a.ksteps) step(fa0, fb0, t0.y);
+    }
+
   }
 
   // ---- epilogue ----------------------------------------------------------------
@@ -386,12 +395,7 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   a.C = d->in_c; a.H = d->in_h; a.W = d->in_w; a.OC = d->out_c; a.OH = d->out_h; a.OW = d->out_w;
   a.kh = d->k_h; a.kw = d->k_w; a.sh = d->stride_h; a.sw = d->stride_w;
   a.dh = d->dilation_h; a.dw = d->dilation_w; a.pad_t = d->pad_top; a.pad_l = d->pad_left;
-  a.cp = RoundUp(a.C, 16);
-  a.cpc = a.cp / 16;
   const int taps = a.kh * a.kw;
-  const int kchunks = taps * a.cpc;
-  a.ksteps = (kchunks + 1) / 2;
-  a.kstride = a.ksteps * 32 + 16;
   const int oc_pad = RoundUp(a.OC, 32);
   const int ot = oc_pad <= 32 ? 1 : (oc_pad <= 64 ? 2 : 4);
   a.oct = 32 * ot;
@@ -417,9 +421,6 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   }
   a.iht = (max_rows - 1) * a.sh + (a.kh - 1) * a.dh + 1;
   a.iwt = std::max((a.OW - 1) * a.sw + (a.kw - 1) * a.dw + 1, 1);
-  // Consecutive pixels of a fragment read must fall into different 16-byte bank
-  // groups: that holds when the pixel stride is an odd number of 16-byte chunks.
-  a.pix_stride = (a.cpc & 1) ? a.cp : a.cp + 16;
   const bool x_u8 = d->in_dtype == TVX_U8, w_u8 = d->w_dtype == TVX_U8;
   const int zxs = d->in_zp - (x_u8 ? 128 : 0);
   const int zws = op->w_zp - (w_u8 ? 128 : 0);
@@ -430,20 +431,47 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   a.out_zp = d->out_zp; a.lo = op->act_lo; a.hi = op->act_hi;
   a.out_stride = ((a.P / 4) | 1) * 4;
   a.w4_blocks = (a.W / 4 + 15) / 16;
-  // LDS carve-up: the per-pixel sums first; the weight + halo region behind them
-  // is reused as the epilogue's staging tile
-  const int w_bytes = RoundUp(a.oct * a.kstride, 1024);  // whole 1 KiB DMA bursts
-  a.w_chunks = w_bytes / 16;
-  const int halo_bytes = RoundUp(a.iht * a.iwt * a.pix_stride + 16, 16);
+  // Reduction groups: the weights of one output-channel block and the halo tile must sit in
+  // LDS together. All input channels at once when that fits next to a second workgroup on
+  // the CU; otherwise the largest channel group that does (the kernel then walks the groups,
+  // accumulating), and as a last resort whatever fits at all.
   const int sx_bytes = a.P * 4;
-  const int tap_bytes = RoundUp((a.ksteps * 2 + 4) * 8, 16);
-  a.off_sx = 0;
-  a.off_tap = sx_bytes;
-  a.off_w = sx_bytes + tap_bytes;
-  a.off_halo = a.off_w + w_bytes;
   const int out_bytes = a.oct * a.out_stride;
-  const int lds_bytes = a.off_w + std::max(w_bytes + halo_bytes, RoundUp(out_bytes, 16));
-  if (lds_bytes > 150 * 1024) return TVX_E_UNSUPPORTED;
+  int lds_bytes = 0, w_bytes = 0, kchunks = 0;
+  auto plan_group = [&](int cp) {
+    a.cp = cp;
+    a.cpc = cp / 16;
+    kchunks = taps * a.cpc;
+    a.ksteps = (kchunks + 1) / 2;
+    a.kstride = a.ksteps * 32 + 16;
+    // Consecutive pixels of a fragment read must fall into different 16-byte bank
+    // groups: that holds when the pixel stride is an odd number of 16-byte chunks.
+    a.pix_stride = (a.cpc & 1) ? a.cp : a.cp + 16;
+    w_bytes = RoundUp(a.oct * a.kstride, 1024);  // whole 1 KiB DMA bursts
+    a.w_chunks = w_bytes / 16;
+    const int halo_bytes = RoundUp(a.iht * a.iwt * a.pix_stride + 16, 16);
+    const int tap_bytes = RoundUp((a.ksteps * 2 + 4) * 8, 16);
+    // LDS carve-up: the per-pixel sums first; the weight + halo region behind them
+    // is reused as the epilogue's staging tile
+    a.off_sx = 0;
+    a.off_tap = sx_bytes;
+    a.off_w = sx_bytes + tap_bytes;
+    a.off_halo = a.off_w + w_bytes;
+    lds_bytes = a.off_w + std::max(w_bytes + halo_bytes, RoundUp(out_bytes, 16));
+    a.groups = (a.C + cp - 1) / cp;
+  };
+  const int c_pad = RoundUp(a.C, 16);
+  bool planned = false;
+  for (int limit : {76 * 1024, 150 * 1024}) {
+    for (int cp = c_pad; cp >= 16 && !planned; cp = cp > 256 ? 256 : cp / 2) {
+      const int c16 = RoundUp(cp, 16);
+      plan_group(c16);
+      if (lds_bytes <= limit) planned = true;
+    }
+    if (planned) break;
+  }
+  if (!planned) return TVX_E_UNSUPPORTED;
+  a.w_group_stride = oc_alloc * a.kstride + 1024;  // slack: the last block's DMA reads whole bursts
   // the loader's index split is exact while units * divisor < 2^32
   if (static_cast<uint64_t>(a.W) * a.cp >= (1ull << 24)) return TVX_E_UNSUPPORTED;
   // the loader uses 24-bit multiplies and 32-bit offsets inside one image
@@ -452,10 +480,10 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
       static_cast<uint64_t>(a.iht) * a.iwt * a.pix_stride >= (1ull << 23))
     return TVX_E_UNSUPPORTED;
   if (static_cast<uint64_t>(d->batch) * a.tiles_per_image > 0x7fffffffull) return TVX_E_UNSUPPORTED;
+  if (static_cast<uint64_t>(a.w_group_stride) * a.groups >= (1ull << 31)) return TVX_E_UNSUPPORTED;
 
-  // ---- pack weights [oc][(ky,kx,c)] int8 with zero padding, fold constants -------
-  // slack behind the last block: its DMA reads whole 1 KiB bursts
-  std::vector<int8_t> packed(static_cast<size_t>(oc_alloc) * a.kstride + 1024, 0);
+  // ---- pack weights [group][oc][(ky,kx,c)] int8 with zero padding, fold constants -------
+  std::vector<int8_t> packed(static_cast<size_t>(a.w_group_stride) * a.groups, 0);
   std::vector<int32_t> biasf(oc_alloc, 0);
   const uint8_t* src = static_cast<const uint8_t*>(w_host);
   const int32_t* b = static_cast<const int32_t*>(bias_host);
@@ -465,7 +493,9 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
       for (int c = 0; c < a.C; ++c) {
         const uint8_t raw = src[(static_cast<size_t>(oc) * a.C + c) * taps + t];
         const int8_t v = static_cast<int8_t>(w_u8 ? raw ^ 0x80 : raw);
-        packed[static_cast<size_t>(oc) * a.kstride + (t * a.cpc + c / 16) * 16 + c % 16] = v;
+        const int g = c / a.cp, cl = c % a.cp;
+        packed[static_cast<size_t>(g) * a.w_group_stride + static_cast<size_t>(oc) * a.kstride +
+               (t * a.cpc + cl / 16) * 16 + cl % 16] = v;
         sw += v;
       }
     const int64_t v = (b ? b[oc] : 0) - static_cast<int64_t>(zxs) * sw +
