@@ -23,6 +23,7 @@ for p in (REPO, os.path.join(REPO, "oracle"), os.path.join(REPO, "tests")):
         sys.path.insert(0, p)
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, 5.0 POP/s
+PEAK_F16_TFLOPS = 2500.0  # MI355X dense fp16 MFMA, 2.5 PFLOP/s
 PEAK_HBM_GBS = 8000.0     # HBM3E, 8 TB/s
 SEED = 0x71
 
@@ -70,6 +71,20 @@ def fc_cfg5(T, rng):
     return dict(name="fc_i8_per_channel_m8192_k4096_n4096", op=op, inputs=(x,), out_elems=m * n,
                 out_dtype=np.int8, ops=2 * m * k * n, algo_bytes=m * k + n * k + m * n + 4 * n,
                 bound="mfma", oracle=None)
+
+
+def fc_cfg5_f16(T, rng):
+    m, k, n = 8192, 4096, 4096
+    x = rng.standard_normal(m * k, dtype=np.float32).astype(np.float16)
+    wt = (rng.standard_normal(n * k, dtype=np.float32) * 0.02).astype(np.float16)
+    b = rng.standard_normal(n).astype(np.float32)
+    d = T.FcDesc()
+    d.m, d.k, d.n = m, k, n
+    d.in_dtype = d.w_dtype = d.out_dtype = T.F16
+    op = T.fully_connected_create(d, wt, b)
+    return dict(name="fc_f16_m8192_k4096_n4096", op=op, inputs=(x,), out_elems=m * n,
+                out_dtype=np.float16, ops=2 * m * k * n, algo_bytes=2 * (m * k + n * k + m * n) + 4 * n,
+                bound="mfma", peak=PEAK_F16_TFLOPS, oracle=None)
 
 
 def dw_cfg3a(T, rng):
@@ -123,7 +138,7 @@ def time_workload(wl, steps, warmup):
     import torch
     stream = torch.cuda.current_stream()
     dev_in = [torch.from_numpy(a).cuda() for a in wl["inputs"]]
-    tdt = {np.uint8: torch.uint8, np.int8: torch.int8}[wl["out_dtype"]]
+    tdt = {np.uint8: torch.uint8, np.int8: torch.int8, np.float16: torch.float16}[wl["out_dtype"]]
     out = torch.empty(wl["out_elems"], dtype=tdt, device="cuda")
     op = wl["op"]
     in1 = dev_in[1] if len(dev_in) > 1 else None
@@ -150,8 +165,9 @@ def time_workload(wl, steps, warmup):
 def roofline(wl, kernel_ms, traffic=None):
     if wl["bound"] == "mfma":
         achieved = wl["ops"] / (kernel_ms * 1e-3) / 1e12
-        return dict(bound="mfma", achieved=round(achieved, 3), peak=PEAK_INT8_TOPS, unit="TOP/s",
-                    frac=round(achieved / PEAK_INT8_TOPS, 5), traffic=traffic)
+        peak = wl.get("peak", PEAK_INT8_TOPS)
+        return dict(bound="mfma", achieved=round(achieved, 3), peak=peak,
+                    unit="TFLOP/s" if "peak" in wl else "TOP/s", frac=round(achieved / peak, 5), traffic=traffic)
     achieved = wl["algo_bytes"] / (kernel_ms * 1e-3) / 1e9
     return dict(bound="hbm", achieved=round(achieved, 2), peak=PEAK_HBM_GBS, unit="GB/s",
                 frac=round(achieved / PEAK_HBM_GBS, 5), traffic=traffic)
@@ -254,7 +270,7 @@ def main():
     }
     if not args.no_extra:
         extra = {}
-        for make in (fc_cfg5, dw_cfg3a, pw_cfg3b):
+        for make in (fc_cfg5, fc_cfg5_f16, dw_cfg3a, pw_cfg3b):
             w2 = make(T, rng)
             steps2 = max(5, min(args.steps, 50))
             wall2, k2 = time_workload(w2, steps2, min(args.warmup, 5))

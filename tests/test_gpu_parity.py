@@ -215,6 +215,41 @@ def test_fully_connected_full_size_int8_per_channel(oracle):
     assert np.array_equal(got_p.reshape(m, n), got[perm])
 
 
+@pytest.mark.parametrize("shape", [(300, 200, 260), (256, 64, 256), (1, 8, 3), (517, 1032, 40)])
+@pytest.mark.parametrize("act", [0, 1, 2])
+def test_fully_connected_float16_mfma_edges(oracle, shape, act):
+    """float16 FC on the matrix cores: ragged M / N tiles, K tails (K % 64 != 0), fused
+    ReLU / ReLU6. fp32 accumulation on both sides; tolerance 1e-2 relative."""
+    m, k, n = shape
+    rng = np.random.default_rng(m + k + n)
+    x = rng.standard_normal(m * k).astype(np.float16)
+    w = (rng.standard_normal(n * k) * 0.05).astype(np.float16)
+    b = rng.standard_normal(n).astype(np.float32)
+    kws = dict(m=m, k=k, n=n, in_dtype=2, w_dtype=2, out_dtype=2)
+    want = oracle.fully_connected(x, w, b, act=act, **kws)
+    got = TC.gpu_fully_connected(x, w, b, act=act, want_kernel="fc_mfma_f16_256x256x64", **kws)
+    assert np.allclose(got.astype(np.float32), want.astype(np.float32), rtol=1e-2, atol=1e-2)
+    if act == 2:
+        assert got.max() <= 6.0 and got.min() >= 0.0
+
+
+def test_fully_connected_full_size_float16(oracle):
+    """M=8192, K=4096, N=4096 float16 (inputs N(0,1), weights N(0,0.02)): the whole problem on
+    the GPU, a seeded sample of 32 rows recomputed by the oracle in fp32, within 1e-2."""
+    m, k, n = 8192, 4096, 4096
+    rng = np.random.default_rng(0x76)
+    x = rng.standard_normal(m * k, dtype=np.float32).astype(np.float16)
+    w = (rng.standard_normal(n * k, dtype=np.float32) * 0.02).astype(np.float16)
+    b = rng.standard_normal(n).astype(np.float32)
+    kws = dict(k=k, n=n, in_dtype=2, w_dtype=2, out_dtype=2)
+    got = TC.gpu_fully_connected(x, w, b, m=m, want_kernel="fc_mfma_f16_256x256x64", **kws).reshape(m, n)
+    rows = np.sort(rng.choice(m, 32, replace=False))
+    want = oracle.fully_connected(np.ascontiguousarray(x.reshape(m, k)[rows]).ravel(), w, b, m=len(rows), **kws)
+    want = want.reshape(len(rows), n).astype(np.float32)
+    assert np.allclose(got[rows].astype(np.float32), want, rtol=1e-2, atol=1e-2)
+    assert np.isfinite(got.astype(np.float32)).all()
+
+
 def test_conv2d_cfg2_full_size(oracle):
     """uint8 3x3 64->64 on 56x56x64 at batch 32, SAME, fused ReLU6: whole output vs the oracle."""
     rng = np.random.default_rng(0x72)

@@ -18,6 +18,15 @@
 //   sum (x - zx)(w - zw) = sum xs ws - zws * sum_k xs - zxs * sum_k ws + K zxs zws
 // (xs = x - 128 for uint8, zxs likewise) is per lane, with no exchange needed.
 // The per-feature terms are folded into the bias at creation.
+//
+// The float16 variant is the same kernel with the other matrix instruction:
+// v_mfma_f32_32x32x16_f16 also takes 16 operand bytes per lane (8 halves) and the
+// two lane halves also cover 32 bytes of a row, so tiles, DMA, swizzle and fragment
+// addresses are identical with K counted in bytes; accumulation is fp32, the
+// epilogue adds the fp32 bias, clamps for ReLU / ReLU6 and rounds to float16.
+#include <cstring>
+#include <type_traits>
+
 #include "variants.h"
 
 namespace tvx {
@@ -25,6 +34,8 @@ namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 constexpr int TM = 256, TN = 256, TK = 128;
 constexpr int kThreads = 256;
@@ -39,15 +50,25 @@ struct FcArgs {
   const int32_t* biasf; // [N] bias + per-feature zero-point terms
   const tvx_v4i* rq;    // [N padded to the tile] requantization records
   const int8_t* zeros;  // 128 x 0x00 then 128 x 0x80: source of reduction chunks past K
-  int M, N, K;
+  int M, N, K;          // K in bytes of a row (float16: twice the element count)
+  const float* biasf32; // float16 variant: [N padded to the tile] fp32 bias
+  float flo, fhi;       // float16 variant: activation clamp
   int zws;              // weight zero point in the int8 domain (0 for per-channel)
   int out_zp, lo, hi;
   int tiles_m, tiles_n;
 };
 
 
-template <bool X_U8, bool ROWSUM, int RQ>
+__device__ __forceinline__ v16i Mfma(const v4i& a, const v4i& b, const v16i& c) {
+  return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ v16f Mfma(const v4i& a, const v4i& b, const v16f& c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+}
+
+template <bool X_U8, bool ROWSUM, int RQ, bool F16 = false>
 __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
+  typedef typename std::conditional<F16, v16f, v16i>::type acc_t;
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -100,7 +121,7 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
     for (int piece = 0; piece < 16; ++piece) dma_piece(kt, stage, piece);
   };
 
-  v16i acc[4][4];  // [tn][tm]
+  acc_t acc[4][4];  // [tn][tm]
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -160,7 +181,7 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
     for (int tn = 0; tn < 4; ++tn)
 #pragma unroll
       for (int tm = 0; tm < 4; ++tm)
-        acc[tn][tm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[tn], fx[tm], acc[tn][tm], 0, 0, 0);
+        acc[tn][tm] = Mfma(fw[tn], fx[tm], acc[tn][tm]);
   };
   // the same 16 MFMAs with one DMA instruction of a later tile issued behind each:
   // a wavefront that issues its DMA back to back sits in the memory pipeline's
@@ -171,7 +192,7 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
     for (int tn = 0; tn < 4; ++tn)
 #pragma unroll
       for (int tm = 0; tm < 4; ++tm) {
-        acc[tn][tm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[tn], fx[tm], acc[tn][tm], 0, 0, 0);
+        acc[tn][tm] = Mfma(fw[tn], fx[tm], acc[tn][tm]);
         dma_piece(dma_kt, dma_stage, tn * 4 + tm);
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -223,55 +244,110 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // no DMA may land in the epilogue's staging tile
   __syncthreads();  // the epilogue reuses the LDS
 
-  // ---- epilogue: requantize, stage the int8 tile in LDS, store 16-byte rows ----
-  if (ROWSUM) {
+  // ---- epilogue ---------------------------------------------------------------
+  if constexpr (F16) {
+    // ---- epilogue, float16: bias, activation clamp, round; the 256 x 256 x 2-byte tile is
+    // staged in two rounds of 64 columns per wavefront column (64 KiB + padding each)
+    constexpr int kHalfStride = 128 * 2 + 16;  // bytes per staged row: 128 halves + padding
+    int8_t* out_tile = lds;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) rowsum[t] += __shfl_xor(rowsum[t], 32);
-  }
-  int8_t* out_tile = lds;  // TM rows x kOutStride bytes (the loop's last barrier freed the LDS)
+    for (int round = 0; round < 2; ++round) {
+      if (round) __syncthreads();
 #pragma unroll
-  for (int tn = 0; tn < 4; ++tn) {
+      for (int t2 = 0; t2 < 2; ++t2) {
+        const int tn = round * 2 + t2;
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      // accumulator rows 8g + 4*(lane/32) + 0..3 of this MFMA tile = 4 consecutive features
-      const int nl = wn * 128 + tn * 32 + 8 * g + 4 * frag_half;
-      const int n = n0 + nl;
-      // records and folded bias are allocated up to the padded feature count
-      int b4[4];
-      tvx_v4i q4[4];
+        for (int g = 0; g < 4; ++g) {
+          const int nw = tn * 32 + 8 * g + 4 * frag_half;  // column inside the wavefront's 128
+          const int n = n0 + wn * 128 + nw;
+          float b4[4];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        b4[q] = a.biasf[n + q];
-        q4[q] = a.rq[n + q];
-      }
+          for (int q = 0; q < 4; ++q) b4[q] = a.biasf32[n + q];
+          const int col = wn * 64 + t2 * 32 + 8 * g + 4 * frag_half;  // staged column (halves)
 #pragma unroll
-      for (int tm = 0; tm < 4; ++tm) {
-        const int ml = wm * 128 + tm * 32 + frag_row;
-        uint32_t packed = 0;
+          for (int tm = 0; tm < 4; ++tm) {
+            const int ml = wm * 128 + tm * 32 + frag_row;
+            _Float16 h[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          int v = acc[tn][tm][g * 4 + q] + b4[q];
-          if (ROWSUM) v -= a.zws * rowsum[tm];
-          const int r = Requant8<RQ>(v, q4[q], a.out_zp, a.lo, a.hi);
-          packed |= static_cast<uint32_t>(r & 0xff) << (8 * q);
+            for (int q = 0; q < 4; ++q) {
+              float v = acc[tn][tm][g * 4 + q] + b4[q];
+              v = fminf(fmaxf(v, a.flo), a.fhi);
+              h[q] = static_cast<_Float16>(v);
+            }
+            uint2 pk;
+            __builtin_memcpy(&pk, h, 8);
+            *reinterpret_cast<uint2*>(out_tile + ml * kHalfStride + col * 2) = pk;
+          }
         }
-        *reinterpret_cast<uint32_t*>(out_tile + ml * kOutStride + nl) = packed;
+      }
+      __syncthreads();
+      // staged columns [0, 64) belong to wn = 0, [64, 128) to wn = 1; 8 halves per 16-byte chunk
+      const bool vec_ok = (a.N & 7) == 0;
+      for (int c = tid; c < TM * 16; c += kThreads) {
+        const int ml = c >> 4, ch = c & 15;
+        const int wcol = ch >> 3, in_w = (ch & 7) * 8;
+        const int m = m0 + ml, n = n0 + wcol * 128 + round * 64 + in_w;
+        if (m >= a.M || n >= a.N) continue;
+        const int8_t* src = out_tile + ml * kHalfStride + (wcol * 64 + in_w) * 2;
+        int8_t* dst = a.y + (static_cast<size_t>(m) * a.N + n) * 2;
+        if (vec_ok) {
+          *reinterpret_cast<v4i*>(dst) = *reinterpret_cast<const v4i*>(src);
+        } else {
+          for (int q = 0; q < 8 && n + q < a.N; ++q)
+            reinterpret_cast<uint16_t*>(dst)[q] = reinterpret_cast<const uint16_t*>(src)[q];
+        }
       }
     }
-  }
-  __syncthreads();
-  const bool vec_ok = (a.N & 15) == 0;
-  for (int c = tid; c < TM * (TN / 16); c += kThreads) {
-    const int ml = c / (TN / 16), nc = (c % (TN / 16)) * 16;
-    const int m = m0 + ml, n = n0 + nc;
-    if (m >= a.M || n >= a.N) continue;
-    const v4i v = *reinterpret_cast<const v4i*>(out_tile + ml * kOutStride + nc);
-    int8_t* dst = a.y + static_cast<size_t>(m) * a.N + n;
-    if (vec_ok) {
-      *reinterpret_cast<v4i*>(dst) = v;
-    } else {
-      const int8_t* src = out_tile + ml * kOutStride + nc;
-      for (int q = 0; q < 16 && n + q < a.N; ++q) dst[q] = src[q];
+  } else {
+    if (ROWSUM) {
+  #pragma unroll
+      for (int t = 0; t < 4; ++t) rowsum[t] += __shfl_xor(rowsum[t], 32);
+    }
+    int8_t* out_tile = lds;  // TM rows x kOutStride bytes (the loop's last barrier freed the LDS)
+  #pragma unroll
+    for (int tn = 0; tn < 4; ++tn) {
+  #pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        // accumulator rows 8g + 4*(lane/32) + 0..3 of this MFMA tile = 4 consecutive features
+        const int nl = wn * 128 + tn * 32 + 8 * g + 4 * frag_half;
+        const int n = n0 + nl;
+        // records and folded bias are allocated up to the padded feature count
+        int b4[4];
+        tvx_v4i q4[4];
+  #pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          b4[q] = a.biasf[n + q];
+          q4[q] = a.rq[n + q];
+        }
+  #pragma unroll
+        for (int tm = 0; tm < 4; ++tm) {
+          const int ml = wm * 128 + tm * 32 + frag_row;
+          uint32_t packed = 0;
+  #pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            int v = acc[tn][tm][g * 4 + q] + b4[q];
+            if (ROWSUM) v -= a.zws * rowsum[tm];
+            const int r = Requant8<RQ>(v, q4[q], a.out_zp, a.lo, a.hi);
+            packed |= static_cast<uint32_t>(r & 0xff) << (8 * q);
+          }
+          *reinterpret_cast<uint32_t*>(out_tile + ml * kOutStride + nl) = packed;
+        }
+      }
+    }
+    __syncthreads();
+    const bool vec_ok = (a.N & 15) == 0;
+    for (int c = tid; c < TM * (TN / 16); c += kThreads) {
+      const int ml = c / (TN / 16), nc = (c % (TN / 16)) * 16;
+      const int m = m0 + ml, n = n0 + nc;
+      if (m >= a.M || n >= a.N) continue;
+      const v4i v = *reinterpret_cast<const v4i*>(out_tile + ml * kOutStride + nc);
+      int8_t* dst = a.y + static_cast<size_t>(m) * a.N + n;
+      if (vec_ok) {
+        *reinterpret_cast<v4i*>(dst) = v;
+      } else {
+        const int8_t* src = out_tile + ml * kOutStride + nc;
+        for (int q = 0; q < 16 && n + q < a.N; ++q) dst[q] = src[q];
+      }
     }
   }
 }
@@ -297,7 +373,7 @@ hipError_t AllowLds(int rq) {
 
 int FcMfmaRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
   const tvx_fc_desc& d = op->fc;
-  FcArgs a;
+  FcArgs a{};
   a.x = static_cast<const int8_t*>(in0);
   a.w = op->packed.as<int8_t>();
   a.y = static_cast<int8_t*>(out);
@@ -314,6 +390,15 @@ int FcMfmaRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t s
   a.tiles_m = (a.M + TM - 1) / TM;
   a.tiles_n = (a.N + TN - 1) / TN;
   const dim3 grid(a.tiles_m * a.tiles_n);
+  if (op->geo[2]) {  // float16
+    a.K = static_cast<int>(d.k) * 2;
+    a.biasf32 = op->aux.as<float>();
+    a.flo = d.activation == TVX_ACT_NONE ? -3.402823466e38f : 0.0f;
+    a.fhi = d.activation == TVX_ACT_RELU6 ? 6.0f : 3.402823466e38f;
+    hipLaunchKernelGGL((FcMfmaKernel<false, false, kRqGeneric, true>), grid, dim3(kThreads), kLdsBytes, st, a);
+    TVX_HIP_CHECK(hipGetLastError());
+    return TVX_OK;
+  }
   const bool x_u8 = d.in_dtype == TVX_U8, rowsum = a.zws != 0;
   const int rq = op->geo[1];
   if (x_u8 && rowsum) LaunchRq<true, true>(rq, grid, st, a);
@@ -326,9 +411,36 @@ int FcMfmaRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t s
 
 }  // namespace
 
-// Claims quantized FullyConnected with constant weights and K a multiple of 16
-// (every 16-byte operand chunk is then whole and aligned).
+// float16 x float16 -> float16 with constant weights and K a multiple of 8.
+static int FcMfmaSetupF16(tvx_op* op, const tvx_fc_desc* d, const void* w_host, const void* bias_host) {
+  if ((d->k & 7) != 0) return TVX_E_UNSUPPORTED;
+  if (static_cast<uint64_t>(d->m) * d->n >= (1ull << 30) || d->k > (1u << 23)) return TVX_E_UNSUPPORTED;
+  if (static_cast<uint64_t>(d->m) * d->k >= (1ull << 31) || static_cast<uint64_t>(d->n) * d->k >= (1ull << 31))
+    return TVX_E_UNSUPPORTED;  // the operand DMA addresses rows with 32-bit byte offsets
+  const uint32_t n_alloc = (d->n + TN - 1) / TN * TN;
+  std::vector<float> bias(n_alloc, 0.0f);
+  if (bias_host) std::memcpy(bias.data(), bias_host, sizeof(float) * d->n);
+  int s = op->packed.Upload(w_host, static_cast<size_t>(d->n) * d->k * 2);
+  if (s == TVX_OK) s = op->aux.Upload(bias.data(), bias.size() * 4);
+  std::vector<int8_t> zeros(256, 0);
+  if (s == TVX_OK) s = op->aux3.Upload(zeros.data(), zeros.size());
+  if (s != TVX_OK) return s;
+  const hipError_t e =
+      hipFuncSetAttribute(reinterpret_cast<const void*>(&FcMfmaKernel<false, false, kRqGeneric, true>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+  if (e != hipSuccess)
+    return SetError(TVX_E_DEVICE, "hipFuncSetAttribute(dynamic LDS %d): %s", kLdsBytes, hipGetErrorString(e));
+  op->geo[2] = 1;
+  op->run = FcMfmaRun;
+  op->kernel_name = "fc_mfma_f16_256x256x64";
+  return TVX_OK;
+}
+
+// Claims FullyConnected with constant weights: quantized with K a multiple of 16 (every
+// 16-byte operand chunk is then whole and aligned), or all-float16.
 int FcMfmaSetup(tvx_op* op, const tvx_fc_desc* d, const void* w_host, const void* bias_host) {
+  if (w_host && d->in_dtype == TVX_F16 && d->w_dtype == TVX_F16 && d->out_dtype == TVX_F16)
+    return FcMfmaSetupF16(op, d, w_host, bias_host);
   if (!op->quantized || !w_host || (d->k & 15) != 0) return TVX_E_UNSUPPORTED;
   if (static_cast<uint64_t>(d->m) * d->n >= (1ull << 31) || d->k > (1u << 24)) return TVX_E_UNSUPPORTED;
   if (static_cast<uint64_t>(d->m) * d->k >= (1ull << 32) || static_cast<uint64_t>(d->n) * d->k >= (1ull << 32))
