@@ -208,6 +208,7 @@ def network_extras(steps, warmup):
     G = importlib.import_module("tim-vx_amd.graphs")
     z = np.load(os.path.join(REPO, "tests", "golden", "lenet_asymu8.npz"))
     nets = [("lenet_asymu8_b1", G.lenet_asymu8(z["weights"], z["input"], batch=1), 1),
+            ("lenet_asymu8_b256", G.lenet_asymu8(z["weights"], z["input"], batch=256), 256),
             ("mobilenet_v2_u8_b64_224", G.mobilenet_v2(batch=64, res=224), 64)]
     out = {}
     with tempfile.TemporaryDirectory() as d:
