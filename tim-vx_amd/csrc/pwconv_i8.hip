@@ -73,7 +73,7 @@ __device__ __forceinline__ void Transpose4x4(const uint32_t in[4], uint32_t out[
 // ZP: the weights have a zero point (int8 domain): its term -zws * sum_c xs is taken by a
 //     second MFMA against a constant fragment - the matrix cores idle here anyway.
 template <int KP, int NW, int PT, int GRAN, bool ZP, int RQ>
-__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4, 8))) PwConvKernel(PwArgs a) {
+__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4, 4))) PwConvKernel(PwArgs a) {
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   constexpr int kThreads = 64 * NW;
   constexpr int kPix = KP;
@@ -94,21 +94,13 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
   const int tile0 = t_begin + wave / kParts;
   const int n_tiles = tile0 < t_end ? (t_end - tile0 + tile_step - 1) / tile_step : 0;
 
-  const int total = n_tiles * a.ksteps;
-
-  // weight fragment stream, in consumption order
-  int pf_tile = n_tiles > 0 ? tile0 : 0, pf_ks = 0, pf_left = total;
-  auto next_frag = [&]() -> v4i {
-    const v4i f = a.wpk[(static_cast<size_t>(pf_tile) * a.ksteps + pf_ks) * 64 + lane];
-    if (--pf_left > 0) {  // past the end: keep re-reading the last fragment
-      if (++pf_ks == a.ksteps) { pf_ks = 0; pf_tile += tile_step; }
-    }
-    return f;
-  };
-
-  // the first weight fragments travel while the input tile is being built
-  v4i f0 = next_frag();
-  v4i f1 = next_frag();
+  // Weight fragments stream global -> registers four k-steps ahead. The first four of a tile
+  // are requested before the previous tile's epilogue (for the first tile: before the input
+  // tile is built), so their latency hides behind work that does not need them.
+  auto frag_ptr = [&](int t, int k) { return a.wpk + (static_cast<size_t>(t) * a.ksteps + k) * 64 + lane; };
+  v4i nf[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) nf[j] = *frag_ptr(n_tiles > 0 ? tile0 : 0, min(j, a.ksteps - 1));
 
   // ---- activations of the 128 pixels, all channels: global (pixel-innermost) -> LDS
   {
@@ -133,36 +125,37 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
     const uint32_t mask_first = k_first >= 4 ? 0xffffffffu : ((1u << (8 * k_first)) - 1u);
     const bool has_second = GRAN == 1 && live && !whole && q0 + k_first < a.Q;
     const uint8_t* src2 = has_second ? a.x + (static_cast<size_t>(n + 1) * a.C) * a.HW - k_first : src;
+    // Every load below is unconditional - a load under a per-lane condition becomes a branch
+    // and a full wait, sixteen round trips instead of one: lanes and channels with nothing to
+    // fetch read a valid address (channel clamped, src at the tensor base) and are masked.
+    // The last row of the tensor must not be read past its end: there the dword is fetched
+    // 4 - k bytes early and shifted down.
     const bool last_image = GRAN == 1 && live && !whole && (n + 1) * static_cast<long long>(a.HW) >= a.Q;
+    const int back = last_image ? 4 - k_first : 0;
     const bool any_split = GRAN == 1 && __any(live && !whole);
     for (int cg = cg0; cg < a.cp / 16; cg += kThreads / kQuads) {
       uint32_t raw[16];
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
         const int c = cg * 16 + j;
-        uint32_t v = 0;
-        if (live && c < a.C) {
-          const uint8_t* row = src + static_cast<size_t>(c) * a.HW;
-          if (GRAN >= 4) {
-            v = *reinterpret_cast<const uint32_t*>(row);
-          } else if (last_image && c == a.C - 1) {
-            for (int e = 0; e < k_first; ++e) v |= static_cast<uint32_t>(row[e]) << (8 * e);
-          } else {
-            __builtin_memcpy(&v, row, 4);
-          }
-          v ^= a.xor_mask;
+        const uint8_t* row = src + static_cast<size_t>(min(c, a.C - 1)) * a.HW;
+        uint32_t v;
+        if (GRAN >= 4) {
+          v = *reinterpret_cast<const uint32_t*>(row);
+        } else {
+          const int bk = c == a.C - 1 ? back : 0;
+          __builtin_memcpy(&v, row - bk, 4);
+          v >>= 8 * bk;
         }
-        raw[j] = v;
+        raw[j] = (live && c < a.C) ? v ^ a.xor_mask : 0u;
       }
       if (any_split) {
 #pragma unroll
         for (int j = 0; j < 16; ++j) {
           const int c = cg * 16 + j;
-          uint32_t v = 0;
-          if (has_second && c < a.C) {
-            __builtin_memcpy(&v, src2 + static_cast<size_t>(c) * a.HW, 4);
-            v ^= a.xor_mask;
-          }
+          uint32_t v;
+          __builtin_memcpy(&v, src2 + static_cast<size_t>(min(c, a.C - 1)) * a.HW, 4);
+          v = (has_second && c < a.C) ? v ^ a.xor_mask : 0u;
           raw[j] = (raw[j] & mask_first) | (v & ~mask_first);
         }
       }
@@ -210,7 +203,7 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
   const int frag_row = lane & 31, frag_half = lane >> 5;
   const int8_t* xa = xl + (part * kRowBytes + frag_row) * a.pix_stride + frag_half * 16;
   v16i acc[PT];
-  int tile = tile0, ks = 0;
+  int tile = tile0;
   auto init_acc = [&]() {
     const int b = a.biasf[tile * 32 + frag_row];
 #pragma unroll
@@ -269,7 +262,7 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
     __builtin_amdgcn_wave_barrier();
   };
 
-  auto step = [&](const v4i& fw) {
+  auto step = [&](const v4i& fw, int ks) {
     v4i fx[PT];
 #pragma unroll
     for (int i = 0; i < PT; ++i)
@@ -279,24 +272,27 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
       acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fx[i], fw, acc[i], 0, 0, 0);
       if (ZP) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fx[i], fz, acc[i], 0, 0, 0);
     }
-    if (++ks == a.ksteps) {
-      epilogue();
-      ks = 0;
-      tile += tile_step;
-      if (tile < t_end) init_acc();
-    }
   };
 
-  init_acc();
-  for (int idx = 0; idx < total; idx += 2) {
-    const v4i g0 = f0;
-    f0 = next_frag();
-    step(g0);
-    if (idx + 1 < total) {
-      const v4i g1 = f1;
-      f1 = next_frag();
-      step(g1);
+  for (int ti = 0; ti < n_tiles; ++ti, tile += tile_step) {
+    init_acc();
+    v4i ring[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ring[j] = nf[j];
+    for (int k0 = 0; k0 < a.ksteps; k0 += 4) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        if (k0 + j < a.ksteps) {
+          const v4i g = ring[j];
+          if (k0 + j + 4 < a.ksteps) ring[j] = *frag_ptr(tile, k0 + j + 4);
+          step(g, k0 + j);
+        }
+      }
     }
+    const int next_tile = tile + tile_step < t_end ? tile + tile_step : tile;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) nf[j] = *frag_ptr(next_tile, min(j, a.ksteps - 1));
+    epilogue();
   }
 }
 
