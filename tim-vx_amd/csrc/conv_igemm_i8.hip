@@ -75,7 +75,7 @@ __device__ __forceinline__ int ChannelFill(const ConvArgs& a, int c, int c_real)
 }
 
 template <int OT, int RQ>
-__global__ void __launch_bounds__(kThreads) ConvIgemmKernel(ConvArgs a) {
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) ConvIgemmKernel(ConvArgs a) {
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int tile = blockIdx.x % a.tiles_per_image;
@@ -142,6 +142,9 @@ __global__ void __launch_bounds__(kThreads) ConvIgemmKernel(ConvArgs a) {
     const size_t plane = static_cast<size_t>(a.H) * a.W;
     const uint8_t* xin = a.x + static_cast<size_t>(n) * a.C * plane;
     const int c4n = a.cp / 4;
+    // 256 zero bytes: the slack behind the last group's packed weights
+    const uint8_t* zero_word =
+        reinterpret_cast<const uint8_t*>(a.w) + static_cast<size_t>(a.groups) * a.w_group_stride - 256;
     if ((a.W & 3) == 0) {
       // A thread owns one (4 input columns, 4 channels) patch and walks the halo
       // rows with it, kLoadBatch rows of loads in flight; lanes run over channel
@@ -160,36 +163,46 @@ __global__ void __launch_bounds__(kThreads) ConvIgemmKernel(ConvArgs a) {
         const int c = c4 * 4;
         const int hc = a.pad_l + w4 * 4;
         // byte offsets of the patch's four channel rows inside this image (< 2^31)
-        uint32_t src_off[4];
+        // Where each of the patch's four channel rows starts. A channel beyond the real ones
+        // reads a zero word behind the packed weights instead: the loaded value is then used
+        // as it is, with no select that the compiler could turn into a branch around the load.
+        const uint8_t* src_row[4];
+        uint32_t row_mul[4];
         int fill[4];
-  #pragma unroll
+#pragma unroll
         for (int j = 0; j < 4; ++j) {
           const bool real = c + j < c_real;
-          src_off[j] = static_cast<uint32_t>(real ? c_base + c + j : 0) * plane32 + static_cast<uint32_t>(w4 * 4);
+          src_row[j] = real ? xin + (static_cast<size_t>(c_base + c + j) * plane32 + static_cast<uint32_t>(w4 * 4))
+                            : zero_word;
+          row_mul[j] = real ? 1u : 0u;
           fill[j] = real ? a.pad_fill : 0;
         }
         const int xm = a.xor_mask;
         int xmask[4];
-  #pragma unroll
+#pragma unroll
         for (int j = 0; j < 4; ++j) xmask[j] = c + j < c_real ? xm : 0;
         const int dst0 = __mul24(hc, a.pix_stride) + c;
         // columns of this patch that exist in the halo tile (stride > 1 may cut the right edge)
         const int ncols = min(4, a.iwt - hc);
         for (int hr0 = 0; hr0 < rows_needed; hr0 += kLoadBatch) {
           int d[kLoadBatch][4];
-  #pragma unroll
+#pragma unroll
           for (int b = 0; b < kLoadBatch; ++b) {
             const int ih = ih0 + hr0 + b;
             const bool inside = hr0 + b < rows_needed && ih >= 0 && ih < a.H;
             const uint32_t row_off = __umul24(static_cast<uint32_t>(inside ? ih : 0), static_cast<uint32_t>(a.W));
-  #pragma unroll
+            const int keep = inside ? -1 : 0;
+#pragma unroll
             for (int j = 0; j < 4; ++j) {
-              // out-of-image rows load row 0 (in bounds) and are replaced by the zero point
-              const int v = *reinterpret_cast<const int*>(xin + (src_off[j] + row_off));
-              d[b][j] = inside ? (c + j < c_real ? v ^ xmask[j] : 0) : fill[j];
+              // out-of-image rows load row 0 (in bounds) and are replaced by the zero point; the
+              // replacement is a mask operation, not a select: a select on the wavefront-uniform
+              // `inside` would be turned into a branch around the load, and loads under branches
+              // are waited for one by one instead of travelling together
+              const int v = *reinterpret_cast<const int*>(src_row[j] + row_off * row_mul[j]);
+              d[b][j] = ((v ^ xmask[j]) & keep) | (fill[j] & ~keep);
             }
           }
-  #pragma unroll
+#pragma unroll
           for (int b = 0; b < kLoadBatch; ++b) {
             if (hr0 + b >= rows_needed) continue;
             // 4 x 4 byte transpose: d[j] = 4 pixels of channel c+j  ->  px[i] = 4 channels of pixel i
@@ -203,7 +216,7 @@ __global__ void __launch_bounds__(kThreads) ConvIgemmKernel(ConvArgs a) {
             px[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100);
             px[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302);
             int8_t* dst = halo + dst0 + __mul24(hr0 + b, row_bytes);
-  #pragma unroll
+#pragma unroll
             for (int i = 0; i < 4; ++i)
               if (i < ncols) *reinterpret_cast<int*>(dst + __mul24(i, a.pix_stride)) = px[i];
           }
@@ -222,7 +235,7 @@ __global__ void __launch_bounds__(kThreads) ConvIgemmKernel(ConvArgs a) {
         int v = ChannelFill(a, c, c_real);
         if (ih >= 0 && ih < a.H) {
           v = 0;
-  #pragma unroll
+#pragma unroll
           for (int j = 0; j < 4; ++j) {
             if (c + j >= c_real) continue;
             const int b = xin[(c_base + c + j) * plane + static_cast<size_t>(ih) * a.W + iw] ^ (a.xor_mask & 0xff);
@@ -257,22 +270,22 @@ __global__ void __launch_bounds__(kThreads) ConvIgemmKernel(ConvArgs a) {
       const int2* my_tap = tap_lds + frag_half;
 
       auto load_ab = [&](v4i* fa, v4i* fb, int ks, int2 t) {
-  #pragma unroll
+#pragma unroll
         for (int i = 0; i < kMaxPtw; ++i)
           fa[i] = *reinterpret_cast<const v4i*>(halo + a_base[i] + t.x);
         // one k-step past the end reads bytes that exist in LDS and are never used
-  #pragma unroll
+#pragma unroll
         for (int j = 0; j < OT; ++j)
           fb[j] = *reinterpret_cast<const v4i*>(w_row + j * 32 * a.kstride + ks * 32);
       };
       auto step = [&](const v4i* fa, const v4i* fb, int ones) {
-  #pragma unroll
+#pragma unroll
         for (int i = 0; i < kMaxPtw; ++i)
-  #pragma unroll
+#pragma unroll
           for (int q = 0; q < 4; ++q) sx[i] = __builtin_amdgcn_sdot4(fa[i][q], ones, sx[i], false);
-  #pragma unroll
+#pragma unroll
         for (int j = 0; j < OT; ++j)
-  #pragma unroll
+#pragma unroll
           for (int i = 0; i < kMaxPtw; ++i)
             acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
       };
