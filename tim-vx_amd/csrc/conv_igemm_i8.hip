@@ -317,6 +317,7 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2
   }
   __syncthreads();  // everyone is done reading weights and halo; sx_lds is visible
   int8_t* out_tile = lds + a.off_w;  // [oct][out_stride], aliases weights + halo
+  const int lo = a.lo, hi = a.hi;
 #pragma unroll
   for (int j = 0; j < OT; ++j) {
     const int ocl = j * 32 + frag_row;
@@ -329,13 +330,10 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2
       for (int g = 0; g < 4; ++g) {
         const int pl = pt * 32 + 8 * g + 4 * frag_half;
         const v4i s4 = *reinterpret_cast<const v4i*>(sx_lds + pl);
-        uint32_t packed = 0;
+        int r4[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int v = acc[i][j][g * 4 + e] - s4[e];
-          packed |= static_cast<uint32_t>(Requant8<RQ>(v, q, a.out_zp, a.lo, a.hi) & 0xff) << (8 * e);
-        }
-        *reinterpret_cast<uint32_t*>(out_tile + ocl * a.out_stride + pl) = packed;
+        for (int e = 0; e < 4; ++e) r4[e] = Requant8<RQ>(acc[i][j][g * 4 + e] - s4[e], q, a.out_zp, lo, hi);
+        *reinterpret_cast<uint32_t*>(out_tile + ocl * a.out_stride + pl) = PackBytes(r4[0], r4[1], r4[2], r4[3]);
       }
     }
   }
