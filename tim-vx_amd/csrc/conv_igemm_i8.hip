@@ -515,7 +515,8 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   }
   // ---- requantization records: 32-bit arithmetic when every shift allows it -------
   std::vector<int32_t> rqt;
-  const int rq = BuildRequantRecords(op->h_mult, op->h_shift, a.OC, oc_alloc, d->out_zp, &rqt);
+  const int rq = BuildRequantRecords(op->h_mult, op->h_shift, a.OC, oc_alloc, d->out_zp, &rqt,
+                                     AccumulatorBound(static_cast<uint64_t>(taps) * a.C, bias_host, a.OC));
   // tap table: chunk q = 2 * kstep + half of the (ky, kx, chunk) order; two spare
   // k-steps at the end so that the loop's prefetch stays inside the table
   std::vector<int32_t> tapt(static_cast<size_t>(a.ksteps + 2) * 4, 0);

@@ -3,16 +3,19 @@
 // through registers at memory speed and never touches the matrix cores.
 //
 // A thread owns a 4-column x 4-row patch of one plane's output; it issues all
-// loads of the input rows behind the patch up front: per row the dword(s) under
-// its columns plus one dword on each side (neighbouring threads load the same
-// lines: L1 hits), cuts the four 3-byte windows out of them with v_alignbyte and
-// feeds each window to three v_dot4 (one per kernel row, weights of a kernel row
-// packed in one register). Rows above / below the image and columns left / right
+// loads of the input rows behind the patch up front: per row only the dword(s)
+// under its own columns - the dword on either side comes from the neighbouring
+// lane by a wavefront shift (DPP), an image row occupying a power-of-two number
+// of lanes so that it never straddles two wavefronts. The thread cuts the four
+// 3-byte windows out of them with v_alignbyte and feeds each window to three
+// v_dot4 (one per kernel row, weights of a kernel row packed in one register). Rows above / below the image and columns left / right
 // of it read as the input zero point, so the zero-point expansion
 //   sum (x - zx)(w - zw) = sum xs ws - zws * Sx - zxs * Sw + 9 zxs zws
 // only needs the window sum Sx when the weight zero point is non-zero (one
-// more v_dot4 with ones per window and kernel row); the channel constants are
-// folded into the bias at creation. Requantization is the exact fixed-point
+// more v_dot4 with ones per window and kernel row) - and then only for the few
+// channels whose shifted weights ws - zws do not fit int8: for all others the
+// shifted weights are packed instead and the Sx term vanishes. The channel
+// constants are folded into the bias at creation. Requantization is the exact fixed-point
 // one of the other kernels; four results are packed into one dword store.
 #include <algorithm>
 
@@ -26,12 +29,14 @@ constexpr int kThreads = 256;
 struct DwArgs {
   const uint8_t* x;
   uint8_t* y;
-  const int32_t* wpk;    // per channel: 3 dwords, kernel row ky = bytes (w[ky][0], w[ky][1], w[ky][2], 0) int8
+  const int32_t* wpk;    // per channel: 4 dwords: kernel row ky = bytes (w[ky][0], w[ky][1], w[ky][2], 0) int8 for
+                         // ky = 0..2, then 1 when the channel needs the window sum (see the setup function)
   const int32_t* biasf;  // per channel: bias - zxs * Sw + 9 zxs zws
   const tvx_v4i* rq;     // per channel requantization record
   int C, H, W, OH, OW;
   int pad_t, pad_l;
   int ow4;               // output dwords per row
+  int lpr_shift;         // log2 of the lanes an image row occupies (>= ow4 lanes, the rest idle)
   int rg_per_block;      // row groups (of kRowsPerThread output rows) per workgroup
   int xor_mask, pad_fill, zws, out_zp, lo, hi;
 };
@@ -53,14 +58,16 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
   const int plane = blockIdx.x;
   const int c = plane % a.C;
   const int tid = threadIdx.x;
-  const int rgl = tid / a.ow4;
-  const int w4 = tid - rgl * a.ow4;
+  const int rgl = tid >> a.lpr_shift;
+  const int w4 = tid & ((1 << a.lpr_shift) - 1);
   const int oh0 = (blockIdx.y * a.rg_per_block + rgl) * kRowsPerThread;
-  if (rgl >= a.rg_per_block || oh0 >= a.OH) return;
+  if (oh0 >= a.OH) return;  // whole rows of lanes leave together: neighbours stay consistent
 
   const uint8_t* xp = a.x + static_cast<size_t>(plane) * a.H * a.W;
   uint8_t* yp = a.y + static_cast<size_t>(plane) * a.OH * a.OW;
-  const int wk0 = a.wpk[c * 3 + 0], wk1 = a.wpk[c * 3 + 1], wk2 = a.wpk[c * 3 + 2];
+  const int wk0 = a.wpk[c * 4 + 0], wk1 = a.wpk[c * 4 + 1], wk2 = a.wpk[c * 4 + 2];
+  // the channel is the same for the whole workgroup: a uniform branch, taken by few channels
+  const bool box = BOXSUM && __builtin_amdgcn_readfirstlane(a.wpk[c * 4 + 3]) != 0;
   const int bias = a.biasf[c];
   const tvx_v4i q = a.rq[c];
   const int in_dwords = a.W / 4;
@@ -71,21 +78,35 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
   constexpr int kRows = S * (kRowsPerThread - 1) + 3;  // input rows behind the thread's output rows
   const int d0 = S * w4;
   const int ih0 = oh0 * S - a.pad_t;
+  const bool has_left = w4 > 0;                      // else: left of the image
+  const bool has_right = d0 + kOwn < in_dwords;      // else: right of the image
 
-  // all loads of the thread are issued before the first use
+  // all loads of the thread are issued before the first use; a lane beyond the row's last
+  // output still fetches its dwords when they exist (its left neighbour needs them)
   int raw[kRows][kOwn + 2];
 #pragma unroll
   for (int r = 0; r < kRows; ++r) {
     const int ih = ih0 + r;
     const bool inside = ih >= 0 && ih < a.H;
     const int* row = reinterpret_cast<const int*>(xp + static_cast<size_t>(inside ? ih : 0) * a.W);
+    const int keep_row = inside ? -1 : 0;
 #pragma unroll
-    for (int i = 0; i < kOwn + 2; ++i) {
-      const int d = d0 - 1 + i;
-      const bool ok = inside && d >= 0 && d < in_dwords;
-      const int v = row[ok ? d : 0];
-      raw[r][i] = ok ? v ^ a.xor_mask : a.pad_fill;
+    for (int i = 0; i < kOwn; ++i) {
+      const int d = d0 + i;
+      const int keep = d < in_dwords ? keep_row : 0;
+      // mask arithmetic, not a select: a select on the loaded value would be compiled into a
+      // branch around the load, and then the loads would be waited for one at a time
+      const int v = row[min(d, in_dwords - 1)];
+      raw[r][1 + i] = ((v ^ a.xor_mask) & keep) | (a.pad_fill & ~keep);
     }
+  }
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) {
+    // lane l - 1 holds the dwords to the left, lane l + 1 those to the right (wave_shr:1, wave_shl:1)
+    const int l = __builtin_amdgcn_update_dpp(a.pad_fill, raw[r][kOwn], 0x138, 0xf, 0xf, false);
+    const int rr = __builtin_amdgcn_update_dpp(a.pad_fill, raw[r][1], 0x130, 0xf, 0xf, false);
+    raw[r][0] = has_left ? l : a.pad_fill;
+    raw[r][kOwn + 1] = has_right ? rr : a.pad_fill;
   }
   int win[kRows][4];
 #pragma unroll
@@ -96,6 +117,7 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
     win[r][2] = Window<4 + S * 2 - PL>(raw[r]);
     win[r][3] = Window<4 + S * 3 - PL>(raw[r]);
   }
+  if (w4 >= a.ow4) return;  // lanes that only fed their neighbour
 #pragma unroll
   for (int o = 0; o < kRowsPerThread; ++o) {
     if (oh0 + o >= a.OH) break;
@@ -106,7 +128,7 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
       acc = __builtin_amdgcn_sdot4(win[S * o][i], wk0, acc, false);
       acc = __builtin_amdgcn_sdot4(win[S * o + 1][i], wk1, acc, false);
       acc = __builtin_amdgcn_sdot4(win[S * o + 2][i], wk2, acc, false);
-      if (BOXSUM) {
+      if (BOXSUM && box) {
         int sx = __builtin_amdgcn_sdot4(win[S * o][i], 0x00010101, 0, false);
         sx = __builtin_amdgcn_sdot4(win[S * o + 1][i], 0x00010101, sx, false);
         sx = __builtin_amdgcn_sdot4(win[S * o + 2][i], 0x00010101, sx, false);
@@ -163,7 +185,12 @@ int DwConv3x3Setup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   if (d->pad_left > 1 || (d->in_w & 3) || (d->out_w & 3)) return TVX_E_UNSUPPORTED;
   const int S = d->stride_w;
   const int ow4 = d->out_w / 4;
-  if (ow4 > kThreads) return TVX_E_UNSUPPORTED;
+  // an image row takes a power-of-two number of lanes (at most a wavefront) that covers both its
+  // output dwords and its input dwords
+  const int in_dw = d->in_w / 4;
+  int lpr_shift = 0;
+  while ((1 << lpr_shift) < ow4 || S * (1 << lpr_shift) < in_dw) ++lpr_shift;
+  if (lpr_shift > 6) return TVX_E_UNSUPPORTED;
   // every output's window must end inside {own dwords, right neighbour}
   if (static_cast<uint32_t>((d->out_w - 1) * S + 2) >= d->in_w + d->pad_left + 4) return TVX_E_UNSUPPORTED;
   const bool x_u8 = d->in_dtype == TVX_U8, w_u8 = d->w_dtype == TVX_U8;
@@ -171,26 +198,38 @@ int DwConv3x3Setup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   const int zws = op->w_zp - (w_u8 ? 128 : 0);
   if (zxs < -128 || zxs > 127) return TVX_E_UNSUPPORTED;
   const int C = d->in_c;
-  std::vector<int32_t> wpk(static_cast<size_t>(C) * 3), biasf(C);
+  std::vector<int32_t> wpk(static_cast<size_t>(C) * 4), biasf(C);
   const uint8_t* src = static_cast<const uint8_t*>(w_host);
   const int32_t* b = static_cast<const int32_t*>(bias_host);
+  bool any_box = false;
   for (int c = 0; c < C; ++c) {
+    int ws[9];
+    bool fits = true;  // do the shifted weights ws - zws fit int8?
+    for (int t = 0; t < 9; ++t) {
+      const uint8_t raw = src[static_cast<size_t>(c) * 9 + t];
+      ws[t] = static_cast<int8_t>(w_u8 ? raw ^ 0x80 : raw);
+      if (ws[t] - zws < -128 || ws[t] - zws > 127) fits = false;
+    }
+    // sum (xs - zxs)(ws - zws): with wz = ws - zws it is sum xs wz - zxs sum wz; otherwise
+    // sum xs ws - zws Sx - zxs sum ws + 9 zxs zws with the window sum Sx taken in the kernel
     int64_t sw = 0;
     for (int ky = 0; ky < 3; ++ky) {
       uint32_t pk = 0;
       for (int kx = 0; kx < 3; ++kx) {
-        const uint8_t raw = src[static_cast<size_t>(c) * 9 + ky * 3 + kx];
-        const int8_t v = static_cast<int8_t>(w_u8 ? raw ^ 0x80 : raw);
-        pk |= static_cast<uint32_t>(static_cast<uint8_t>(v)) << (8 * kx);
+        const int v = fits ? ws[ky * 3 + kx] - zws : ws[ky * 3 + kx];
+        pk |= static_cast<uint32_t>(static_cast<uint8_t>(static_cast<int8_t>(v))) << (8 * kx);
         sw += v;
       }
-      wpk[static_cast<size_t>(c) * 3 + ky] = static_cast<int32_t>(pk);
+      wpk[static_cast<size_t>(c) * 4 + ky] = static_cast<int32_t>(pk);
     }
-    const int64_t v = (b ? b[c] : 0) - static_cast<int64_t>(zxs) * sw + 9ll * zxs * zws;
+    const bool box = !fits && zws != 0;
+    wpk[static_cast<size_t>(c) * 4 + 3] = box ? 1 : 0;
+    any_box |= box;
+    const int64_t v = (b ? b[c] : 0) - static_cast<int64_t>(zxs) * sw + (fits ? 0 : 9ll * zxs * zws);
     biasf[c] = static_cast<int32_t>(static_cast<uint32_t>(v));
   }
   std::vector<int32_t> rqt;
-  const int rq = BuildRequantRecords(op->h_mult, op->h_shift, C, C, d->out_zp, &rqt);
+  const int rq = BuildRequantRecords(op->h_mult, op->h_shift, C, C, d->out_zp, &rqt, AccumulatorBound(9, bias_host, C));
   int s = op->packed.Upload(wpk.data(), wpk.size() * 4);
   if (s == TVX_OK) s = op->aux.Upload(biasf.data(), biasf.size() * 4);
   if (s == TVX_OK) s = op->aux2.Upload(rqt.data(), rqt.size() * 4);
@@ -203,12 +242,13 @@ int DwConv3x3Setup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   a.C = C; a.H = d->in_h; a.W = d->in_w; a.OH = d->out_h; a.OW = d->out_w;
   a.pad_t = d->pad_top; a.pad_l = d->pad_left;
   a.ow4 = ow4;
-  a.rg_per_block = std::max(1, kThreads / ow4);
+  a.lpr_shift = lpr_shift;
+  a.rg_per_block = kThreads >> lpr_shift;
   const int row_groups = (static_cast<int>(d->out_h) + kRowsPerThread - 1) / kRowsPerThread;
   a.xor_mask = x_u8 ? static_cast<int>(0x80808080u) : 0;
   a.pad_fill = static_cast<int>(static_cast<uint32_t>(zxs & 0xff) * 0x01010101u);
   a.zws = zws; a.out_zp = d->out_zp; a.lo = op->act_lo; a.hi = op->act_hi;
-  p.stride = S; p.pad_l = d->pad_left; p.boxsum = zws != 0; p.rq = rq;
+  p.stride = S; p.pad_l = d->pad_left; p.boxsum = any_box; p.rq = rq;
   p.grid = dim3(d->batch * C, (row_groups + a.rg_per_block - 1) / a.rg_per_block);
   op->host_blob.assign(reinterpret_cast<const uint8_t*>(&p), reinterpret_cast<const uint8_t*>(&p) + sizeof(p));
   op->run = DwRun;

@@ -212,7 +212,7 @@ int DwPlanesSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, cons
     tab[static_cast<size_t>(c) * a.tab_stride + taps] = static_cast<int32_t>(static_cast<uint32_t>(v));
   }
   std::vector<int32_t> rqt;
-  p.rq = BuildRequantRecords(op->h_mult, op->h_shift, C, C, d->out_zp, &rqt);
+  p.rq = BuildRequantRecords(op->h_mult, op->h_shift, C, C, d->out_zp, &rqt, AccumulatorBound(taps, bias_host, C));
   int s = op->packed.Upload(tab.data(), tab.size() * 4);
   if (s == TVX_OK) s = op->aux2.Upload(rqt.data(), rqt.size() * 4);
   if (s != TVX_OK) return s;

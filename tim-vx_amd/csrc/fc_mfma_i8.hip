@@ -466,7 +466,8 @@ int FcMfmaSetup(tvx_op* op, const tvx_fc_desc* d, const void* w_host, const void
   }
   std::vector<int32_t> rqt;
   const int rq = BuildRequantRecords(op->h_mult, op->h_shift, static_cast<int>(d->n),
-                                     static_cast<int>(n_alloc), d->out_zp, &rqt);
+                                     static_cast<int>(n_alloc), d->out_zp, &rqt,
+                                     AccumulatorBound(d->k, bias_host, d->n));
   int s = op->packed.Upload(ws.data(), wn);
   if (s == TVX_OK) s = op->aux.Upload(biasf.data(), biasf.size() * 4);
   if (s == TVX_OK) s = op->aux2.Upload(rqt.data(), rqt.size() * 4);

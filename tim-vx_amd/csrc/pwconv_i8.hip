@@ -437,7 +437,8 @@ int PwConvSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const 
     biasf[oc] = static_cast<int32_t>(static_cast<uint32_t>(v));
   }
   std::vector<int32_t> rqt;
-  const int rq = BuildRequantRecords(op->h_mult, op->h_shift, a.OC, oc_alloc, d->out_zp, &rqt);
+  const int rq = BuildRequantRecords(op->h_mult, op->h_shift, a.OC, oc_alloc, d->out_zp, &rqt,
+                                     AccumulatorBound(a.C, bias_host, a.OC));
   int s = op->packed.Upload(packed.data(), packed.size());
   if (s == TVX_OK) s = op->aux.Upload(biasf.data(), biasf.size() * 4);
   if (s == TVX_OK) s = op->aux2.Upload(rqt.data(), rqt.size() * 4);

@@ -2,7 +2,9 @@
 // requantization tables, and the walk over kernel variants that picks the
 // first one claiming an operator (the counterpart of ovxlib's
 // vsi_nn_kernel_selector priority walk, src/tim/vx/internal/src/kernel/vsi_nn_kernel.c:1178-1299).
+#include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 
@@ -77,16 +79,30 @@ int BuildRequantTables(uint32_t channels, float in_scale, float w_scale,
   return TVX_OK;
 }
 
+int64_t AccumulatorBound(uint64_t reduction, const void* bias_host, uint32_t channels) {
+  // |sum (x - zx)(w - zw)| <= reduction * 255 * 255 for 8-bit operands
+  int64_t b = static_cast<int64_t>(reduction) * 255 * 255;
+  const int32_t* bias = static_cast<const int32_t*>(bias_host);
+  int64_t mx = 0;
+  for (uint32_t c = 0; bias && c < channels; ++c) mx = std::max<int64_t>(mx, std::llabs(static_cast<long long>(bias[c])));
+  return b + mx;
+}
+
 int BuildRequantRecords(const std::vector<int32_t>& mult, const std::vector<int32_t>& shift,
-                        int channels, int alloc, int out_zp, std::vector<int32_t>* records) {
+                        int channels, int alloc, int out_zp, std::vector<int32_t>* records,
+                        int64_t acc_bound) {
   int rq = kRqFastNoTie;
   for (int c = 0; c < channels; ++c) {
     const int32_t m = mult[c], s = shift[c];
     if (m == 0) continue;
     // (zp << t) + 2^30 must stay inside int32
     if (s < 33 || s - 32 > 20) { rq = kRqGeneric; break; }
-    // a tie needs an accumulator v with v * m = 2^(s-1) (mod 2^s): ctz(v) = s - 1 - ctz(m) <= 31
-    if (__builtin_ctz(static_cast<uint32_t>(m)) >= s - 32) rq = kRqFast;
+    // a tie needs an accumulator v with v * m = 2^(s-1) (mod 2^s): ctz(v) = s - 1 - ctz(m), which
+    // no 32-bit v has when that exceeds 31, and no accumulator of this operator has when
+    // 2^(s - 1 - ctz(m)) is beyond the largest magnitude it can reach
+    const int need = s - 1 - __builtin_ctz(static_cast<uint32_t>(m));
+    const bool reachable = need <= 31 && (acc_bound < 0 || (int64_t{1} << need) <= acc_bound);
+    if (reachable) rq = kRqFast;
   }
   records->assign(static_cast<size_t>(alloc) * 4, 0);
   for (int c = 0; c < alloc; ++c) {

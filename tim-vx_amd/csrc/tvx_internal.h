@@ -137,8 +137,13 @@ __device__ __forceinline__ int Requant8(int v, const tvx_v4i& q, int zp, int lo,
 // ---- host helpers ------------------------------------------------------------
 // Builds the records above for `alloc` channels (the first `channels` from the
 // operator's mult/shift tables, the rest neutral) and returns the flavour.
+// `acc_bound` (if >= 0) is the largest accumulator magnitude the operator can produce: ties
+// that would need a larger accumulator are ruled out.
 int BuildRequantRecords(const std::vector<int32_t>& mult, const std::vector<int32_t>& shift,
-                        int channels, int alloc, int out_zp, std::vector<int32_t>* records);
+                        int channels, int alloc, int out_zp, std::vector<int32_t>* records,
+                        int64_t acc_bound = -1);
+// reduction length * 255 * 255 + max |bias|: bound of sum (x - zx)(w - zw) + bias for 8-bit operands
+int64_t AccumulatorBound(uint64_t reduction, const void* bias_host, uint32_t channels);
 // Per-output-channel requantization tables (mult/shift) for a conv / FC.
 int BuildRequantTables(uint32_t channels, float in_scale, float w_scale,
                        const float* w_scales, float out_scale,
