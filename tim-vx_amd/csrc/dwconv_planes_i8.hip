@@ -1,16 +1,16 @@
 // Depthwise quantized convolution (multiplier 1) for small planes of any width.
 //
 // In WHCN every (image, channel) plane is contiguous, and so is a run of G
-// consecutive planes - input and output alike. A workgroup therefore copies the
-// G input planes into LDS as one linear, 16-byte-chunked stream (no row or
-// alignment structure needed: widths like 14 or 7 are as good as any), computes
-// the stencil out of LDS - a work item is four neighbouring outputs of one row,
-// sharing the loaded input columns - into an LDS image of the G output planes,
-// and copies that image out as another linear stream. Out-of-image taps read the
-// input zero point, so with wz = w - zw every output is
-//   bias - zx * sum(wz) + sum x * wz,
-// the first two terms folded at creation. Any kernel size, stride, dilation
-// and padding; 3x3 is unrolled.
+// consecutive planes - input and output alike. A workgroup therefore reads the
+// G input planes as one linear stream of aligned 16-byte chunks (no row or
+// alignment structure needed: widths like 14 or 7 are as good as any) and
+// scatters the bytes into LDS images of the planes that carry their padding
+// border, pre-filled with the input zero point: the stencil then runs without a
+// single bounds check. A work item is four neighbouring outputs of one row; for
+// 3x3 kernels of stride 1 or 2 they share the input columns they read. Results
+// go to an LDS image of the G output planes, which leaves as another linear
+// stream. With wz = w - zw every output is bias - zx * sum(wz) + sum x * wz, the
+// first two terms folded at creation and kept, with the taps, in LDS per plane.
 #include <algorithm>
 
 #include "variants.h"
@@ -32,26 +32,9 @@ struct DwpArgs {
   long long planes;    // batch * C
   int in_zp, out_zp, lo, hi;
   int ow4;             // work items per output row
+  int ph, pw;          // padded plane extent in LDS
+  int off_out, off_tab;  // LDS carve-up (bytes): output image, per-plane tables
 };
-
-// Linear copy of `len` bytes from global `src` into LDS so that byte i lands at
-// dst[(src & 15) + i]: whole aligned 16-byte chunks, except that a chunk reaching
-// past `limit` (the end of the tensor) is read byte by byte.
-__device__ __forceinline__ void CopyIn(const uint8_t* src, size_t len, const uint8_t* limit, uint8_t* dst, int tid) {
-  const uintptr_t s = reinterpret_cast<uintptr_t>(src);
-  const uint8_t* base = reinterpret_cast<const uint8_t*>(s & ~uintptr_t{15});
-  const int head = static_cast<int>(s & 15);
-  const int chunks = static_cast<int>((head + len + 15) / 16);
-  for (int i = tid; i < chunks; i += kThreads) {
-    const uint8_t* p = base + static_cast<size_t>(i) * 16;
-    if (p + 16 <= limit) {
-      *reinterpret_cast<uint4*>(dst + i * 16) = *reinterpret_cast<const uint4*>(p);
-    } else {
-      for (int b = 0; b < 16; ++b)
-        if (p + b < limit) dst[i * 16 + b] = p[b];
-    }
-  }
-}
 
 // Linear copy of `len` bytes from LDS (byte i at src[(dst & 15) + i]) to global `dst`.
 __device__ __forceinline__ void CopyOut(uint8_t* dst, size_t len, const uint8_t* src, int tid) {
@@ -70,25 +53,79 @@ __device__ __forceinline__ void CopyOut(uint8_t* dst, size_t len, const uint8_t*
   }
 }
 
-template <typename XT, bool K3, int RQ>
+// MODE 0: any kernel; 1: 3x3, stride 1, dilation 1; 2: 3x3, stride 2, dilation 1.
+template <typename XT, int MODE, int RQ>
 __global__ void __launch_bounds__(kThreads) DwPlanesKernel(DwpArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds_raw[];
   const int tid = threadIdx.x;
   const long long p0 = static_cast<long long>(blockIdx.x) * a.G;
   const int g_n = static_cast<int>(min(static_cast<long long>(a.G), a.planes - p0));
   const int hwi = a.H * a.W, hwo = a.OH * a.OW;
+  const int pplane = a.ph * a.pw;
   const uint8_t* src = a.x + static_cast<size_t>(p0) * hwi;
   uint8_t* dst = a.y + static_cast<size_t>(p0) * hwo;
-  const int in_head = static_cast<int>(reinterpret_cast<uintptr_t>(src) & 15);
-  const int out_head = static_cast<int>(reinterpret_cast<uintptr_t>(dst) & 15);
   uint8_t* in_lds = lds_raw;
-  uint8_t* out_lds = lds_raw + ((a.G * hwi + 15 + 16) & ~15);
-  CopyIn(src, static_cast<size_t>(g_n) * hwi, a.x + static_cast<size_t>(a.planes) * hwi, in_lds, tid);
-  __syncthreads();
-  const XT* xin = reinterpret_cast<const XT*>(in_lds + in_head);
-  uint8_t* yout = out_lds + out_head;
+  uint8_t* out_lds = lds_raw + a.off_out;
+  int* tab_lds = reinterpret_cast<int*>(lds_raw + a.off_tab);
+  const int taps = MODE ? 9 : a.kh * a.kw;
+  const int tstride = taps + 5;  // taps, folded bias, 4-dword requantization record
 
-  const int kh = K3 ? 3 : a.kh, kw = K3 ? 3 : a.kw;
+  // ---- padded planes <- zero point; per-plane tables ----------------------------------
+  {
+    const uint32_t z4 = static_cast<uint32_t>(a.in_zp & 0xff) * 0x01010101u;
+    const uint4 z16 = make_uint4(z4, z4, z4, z4);
+    for (int i = tid; i < a.off_out / 16; i += kThreads) reinterpret_cast<uint4*>(in_lds)[i] = z16;
+    for (int i = tid; i < g_n * tstride; i += kThreads) {
+      const int g = i / tstride, e = i - g * tstride;
+      const int c = static_cast<int>((p0 + g) % a.C);
+      tab_lds[i] = e <= taps ? a.tab[static_cast<size_t>(c) * a.tab_stride + e]
+                             : reinterpret_cast<const int*>(a.rq)[c * 4 + (e - taps - 1)];
+    }
+  }
+  __syncthreads();
+  // ---- input stream -> plane interiors ---------------------------------------------------
+  {
+    const uintptr_t sa = reinterpret_cast<uintptr_t>(src);
+    const uint8_t* base = reinterpret_cast<const uint8_t*>(sa & ~uintptr_t{15});
+    const int head = static_cast<int>(sa & 15);
+    const int len = g_n * hwi;
+    const int chunks = (head + len + 15) / 16;
+    const uint8_t* limit = a.x + static_cast<size_t>(a.planes) * hwi;
+    for (int i = tid; i < chunks; i += kThreads) {
+      const uint8_t* pch = base + static_cast<size_t>(i) * 16;
+      uint32_t w[4] = {0, 0, 0, 0};
+      if (pch + 16 <= limit) {
+        const uint4 v = *reinterpret_cast<const uint4*>(pch);
+        w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
+      } else {
+        for (int b = 0; b < 16; ++b)
+          if (pch + b < limit) w[b >> 2] |= static_cast<uint32_t>(pch[b]) << (8 * (b & 3));
+      }
+      // linear index of the chunk's first byte -> (plane, row, column), then walk
+      int li = i * 16 - head;
+      const int lj = max(li, 0);
+      int g = lj / hwi;
+      int rem = lj - g * hwi;
+      int iy = rem / a.W, ix = rem - iy * a.W;
+      uint8_t* o = in_lds + g * pplane + (iy + a.pad_t) * a.pw + a.pad_l + ix;
+#pragma unroll
+      for (int b = 0; b < 16; ++b, ++li) {
+        if (li < 0 || li >= len) continue;
+        *o = static_cast<uint8_t>(w[b >> 2] >> (8 * (b & 3)));
+        ++o;
+        if (++ix == a.W) {
+          ix = 0;
+          o += a.pw - a.W;
+          if (++iy == a.H) { iy = 0; o += pplane - a.H * a.pw; }
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- stencil ------------------------------------------------------------------------------
+  const int out_head = static_cast<int>(reinterpret_cast<uintptr_t>(dst) & 15);
+  uint8_t* yout = out_lds + out_head;
   const int items_per_plane = a.OH * a.ow4;
   const int items = g_n * items_per_plane;
   for (int it = tid; it < items; it += kThreads) {
@@ -96,40 +133,39 @@ __global__ void __launch_bounds__(kThreads) DwPlanesKernel(DwpArgs a) {
     const int r = it - g * items_per_plane;
     const int oy = r / a.ow4;
     const int ox0 = (r - oy * a.ow4) * 4;
-    const int c = static_cast<int>((p0 + g) % a.C);
-    const int32_t* t = a.tab + static_cast<size_t>(c) * a.tab_stride;
-    const int bias = t[kh * kw];
+    const int* t = tab_lds + g * tstride;
+    const int bias = t[taps];
     int acc[4] = {bias, bias, bias, bias};
-    const XT* plane = xin + g * hwi;
-    const int iy0 = oy * a.sh - a.pad_t;
-    const int ix0 = ox0 * a.sw - a.pad_l;
-    auto tap = [&](int ky, int kx) {
-      const int iy = iy0 + ky * a.dh;
-      const bool row_ok = iy >= 0 && iy < a.H;
-      const XT* row = plane + (row_ok ? iy : 0) * a.W;
-      const int wz = t[ky * kw + kx];
+    const XT* win = reinterpret_cast<const XT*>(in_lds) + g * pplane + (oy * a.sh) * a.pw + ox0 * a.sw;
+    if (MODE) {
+      constexpr int kCols = MODE == 1 ? 6 : 9;  // input columns behind four outputs
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int ix = ix0 + j * a.sw + kx * a.dw;
-        const bool ok = row_ok && ix >= 0 && ix < a.W;
-        const int xv = ok ? static_cast<int>(row[ok ? ix : 0]) : a.in_zp;
-        acc[j] += xv * wz;
+      for (int ky = 0; ky < 3; ++ky) {
+        int col[kCols];
+#pragma unroll
+        for (int j = 0; j < kCols; ++j) col[j] = static_cast<int>(win[ky * a.pw + j]);
+#pragma unroll
+        for (int kx = 0; kx < 3; ++kx) {
+          const int wz = t[ky * 3 + kx];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[j] += col[j * MODE + kx] * wz;
+        }
       }
-    };
-    if (K3) {
-#pragma unroll
-      for (int ky = 0; ky < 3; ++ky)
-#pragma unroll
-        for (int kx = 0; kx < 3; ++kx) tap(ky, kx);
     } else {
-      for (int ky = 0; ky < kh; ++ky)
-        for (int kx = 0; kx < kw; ++kx) tap(ky, kx);
+      for (int ky = 0; ky < a.kh; ++ky)
+        for (int kx = 0; kx < a.kw; ++kx) {
+          const int wz = t[ky * a.kw + kx];
+          const XT* px = win + (ky * a.dh) * a.pw + kx * a.dw;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) acc[j] += static_cast<int>(px[j * a.sw]) * wz;
+        }
     }
-    const tvx_v4i q = a.rq[c];
+    const tvx_v4i q = {t[taps + 1], t[taps + 2], t[taps + 3], t[taps + 4]};
     uint8_t* o = yout + g * hwo + oy * a.OW + ox0;
+    const int lo = a.lo, hi = a.hi;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      if (ox0 + j < a.OW) o[j] = static_cast<uint8_t>(Requant8<RQ>(acc[j], q, a.out_zp, a.lo, a.hi));
+      if (ox0 + j < a.OW) o[j] = static_cast<uint8_t>(Requant8<RQ>(acc[j], q, a.out_zp, lo, hi));
   }
   __syncthreads();
   CopyOut(dst, static_cast<size_t>(g_n) * hwo, out_lds, tid);
@@ -137,19 +173,26 @@ __global__ void __launch_bounds__(kThreads) DwPlanesKernel(DwpArgs a) {
 
 struct Plan {
   DwpArgs a;
-  int lds_bytes, x_u8, k3, rq;
+  int lds_bytes, x_u8, mode, rq;
   unsigned grid;
 };
 
-template <typename XT, bool K3>
+template <typename XT, int MODE>
 void LaunchRq(const Plan* p, const DwpArgs& a, hipStream_t st) {
   const dim3 grid(p->grid), block(kThreads);
   if (p->rq == kRqFastNoTie)
-    hipLaunchKernelGGL((DwPlanesKernel<XT, K3, kRqFastNoTie>), grid, block, p->lds_bytes, st, a);
+    hipLaunchKernelGGL((DwPlanesKernel<XT, MODE, kRqFastNoTie>), grid, block, p->lds_bytes, st, a);
   else if (p->rq == kRqFast)
-    hipLaunchKernelGGL((DwPlanesKernel<XT, K3, kRqFast>), grid, block, p->lds_bytes, st, a);
+    hipLaunchKernelGGL((DwPlanesKernel<XT, MODE, kRqFast>), grid, block, p->lds_bytes, st, a);
   else
-    hipLaunchKernelGGL((DwPlanesKernel<XT, K3, kRqGeneric>), grid, block, p->lds_bytes, st, a);
+    hipLaunchKernelGGL((DwPlanesKernel<XT, MODE, kRqGeneric>), grid, block, p->lds_bytes, st, a);
+}
+
+template <typename XT>
+void LaunchMode(const Plan* p, const DwpArgs& a, hipStream_t st) {
+  if (p->mode == 1) LaunchRq<XT, 1>(p, a, st);
+  else if (p->mode == 2) LaunchRq<XT, 2>(p, a, st);
+  else LaunchRq<XT, 0>(p, a, st);
 }
 
 int DwPlanesRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
@@ -159,11 +202,7 @@ int DwPlanesRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t
   a.y = static_cast<uint8_t*>(out);
   if ((reinterpret_cast<uintptr_t>(in0) | reinterpret_cast<uintptr_t>(out)) & 15)
     return SetError(TVX_E_INVALID, "dwconv_planes_i8: tensors must be 16-byte aligned");
-  if (p->x_u8) {
-    if (p->k3) LaunchRq<uint8_t, true>(p, a, st); else LaunchRq<uint8_t, false>(p, a, st);
-  } else {
-    if (p->k3) LaunchRq<int8_t, true>(p, a, st); else LaunchRq<int8_t, false>(p, a, st);
-  }
+  if (p->x_u8) LaunchMode<uint8_t>(p, a, st); else LaunchMode<int8_t>(p, a, st);
   TVX_HIP_CHECK(hipGetLastError());
   return TVX_OK;
 }
@@ -175,7 +214,7 @@ int DwPlanesRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t
 int DwPlanesSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const void* bias_host) {
   if (!op->quantized || !w_host || d->multiplier != 1) return TVX_E_UNSUPPORTED;
   const uint64_t hwi = static_cast<uint64_t>(d->in_w) * d->in_h, hwo = static_cast<uint64_t>(d->out_w) * d->out_h;
-  if (hwi == 0 || hwo == 0 || hwi + hwo > 40 * 1024) return TVX_E_UNSUPPORTED;
+  if (hwi == 0 || hwo == 0) return TVX_E_UNSUPPORTED;
   const int taps = d->k_w * d->k_h;
   if (taps > 121) return TVX_E_UNSUPPORTED;
   const int C = d->in_c;
@@ -189,13 +228,24 @@ int DwPlanesSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, cons
   a.planes = static_cast<long long>(d->batch) * C;
   a.in_zp = d->in_zp; a.out_zp = d->out_zp; a.lo = op->act_lo; a.hi = op->act_hi;
   a.ow4 = (a.OW + 3) / 4;
-  // planes per workgroup: about 8 KiB of input + output, but leave a few workgroups per CU
-  long long g = std::max<long long>(1, 8192 / static_cast<long long>(hwi + hwo));
+  // padded plane: every tap of every work item (four outputs, the last item of a row may
+  // overhang) reads inside it
+  const long long need_w = static_cast<long long>(a.ow4 * 4 - 1) * a.sw + static_cast<long long>(a.kw - 1) * a.dw + 1;
+  const long long need_h = static_cast<long long>(a.OH - 1) * a.sh + static_cast<long long>(a.kh - 1) * a.dh + 1;
+  const long long pw = std::max<long long>(need_w, a.pad_l + a.W), ph = std::max<long long>(need_h, a.pad_t + a.H);
+  if (pw * ph + static_cast<long long>(hwo) > 48 * 1024) return TVX_E_UNSUPPORTED;
+  a.pw = static_cast<int>(pw);
+  a.ph = static_cast<int>(ph);
+  // planes per workgroup: about 10 KiB of LDS images, but leave a few workgroups per CU
+  long long g = std::max<long long>(1, 10240 / (pw * ph + static_cast<long long>(hwo)));
   g = std::min<long long>(g, std::max<long long>(1, a.planes / 1024));
   a.G = static_cast<int>(std::min<long long>(g, 256));
   const long long grid = (a.planes + a.G - 1) / a.G;
   if (grid > 0x7fffffffll) return TVX_E_UNSUPPORTED;
-  p.lds_bytes = static_cast<int>(((a.G * hwi + 15 + 16) & ~15ull) + ((a.G * hwo + 15 + 16) & ~15ull));
+  a.off_out = static_cast<int>((a.G * pw * ph + 15) & ~15ll);
+  a.off_tab = a.off_out + static_cast<int>((a.G * hwo + 15 + 16) & ~15ull);
+  p.lds_bytes = a.off_tab + a.G * (taps + 5) * 4;
+  if (p.lds_bytes > 64 * 1024) return TVX_E_UNSUPPORTED;
   std::vector<int32_t> tab(static_cast<size_t>(C) * a.tab_stride);
   const uint8_t* src = static_cast<const uint8_t*>(w_host);
   const int32_t* b = static_cast<const int32_t*>(bias_host);
@@ -219,7 +269,9 @@ int DwPlanesSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, cons
   a.tab = op->packed.as<int32_t>();
   a.rq = op->aux2.as<tvx_v4i>();
   p.x_u8 = d->in_dtype == TVX_U8;
-  p.k3 = d->k_w == 3 && d->k_h == 3;
+  const bool k3 = d->k_w == 3 && d->k_h == 3 && d->dilation_w == 1 && d->dilation_h == 1 &&
+                  d->stride_w == d->stride_h;
+  p.mode = k3 && d->stride_w == 1 ? 1 : (k3 && d->stride_w == 2 ? 2 : 0);
   p.grid = static_cast<unsigned>(grid);
   op->host_blob.assign(reinterpret_cast<const uint8_t*>(&p), reinterpret_cast<const uint8_t*>(&p) + sizeof(p));
   op->run = DwPlanesRun;
