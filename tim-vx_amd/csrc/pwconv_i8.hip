@@ -13,8 +13,8 @@
 //     private LDS patch and writes them itself - no workgroup barrier after the
 //     input tile is built, and every global store is a complete cache line;
 //   * weights are pre-packed in MFMA fragment order and stream global -> registers
-//     (1 KiB contiguous per wavefront load, prefetched two steps ahead across tile
-//     boundaries); they are small and live in L2.
+//     (1 KiB contiguous per wavefront load, prefetched up to four steps ahead, the
+//     first ones of a tile during the previous tile's epilogue); they are small and live in L2.
 // Zero points: sum (x - zx)(w - zw) = sum xs ws - zws Sx - zxs Sw + C zxs zws with
 // xs, ws the operands moved to the signed int8 domain; the Sx term is one more MFMA
 // against a constant fragment, the per-channel constants are folded into the bias.
@@ -40,7 +40,7 @@ struct PwArgs {
   const int32_t* biasf;  // bias + per-channel zero-point terms
   const v4i* rq;         // per channel requantization record
   int C, OC, HW;
-  long long Q;           // batch * HW
+  int Q;                 // batch * HW (< 2^31 - 256: flat pixel indices are 32-bit)
   int cp;                // channels padded to 32
   int ksteps;            // cp / 32
   int pix_stride;        // LDS bytes per pixel: cp + 16 (an odd number of 16-byte chunks)
@@ -73,7 +73,7 @@ __device__ __forceinline__ void Transpose4x4(const uint32_t in[4], uint32_t out[
 // ZP: the weights have a zero point (int8 domain): its term -zws * sum_c xs is taken by a
 //     second MFMA against a constant fragment - the matrix cores idle here anyway.
 template <int KP, int NW, int PT, int GRAN, bool ZP, int RQ>
-__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4, 4))) PwConvKernel(PwArgs a) {
+__global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((PT == 4 && GRAN < 16) ? 3 : 4, (PT == 4 && GRAN < 16) ? 3 : 4))) PwConvKernel(PwArgs a) {
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   constexpr int kThreads = 64 * NW;
   constexpr int kPix = KP;
@@ -81,7 +81,7 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
   constexpr int kRowBytes = 32 * PT;  // staged bytes per output row
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = NW == 1 ? 0 : __builtin_amdgcn_readfirstlane(tid >> 6);
-  const long long q_base = static_cast<long long>(blockIdx.x) * kPix;
+  const int q_base = blockIdx.x * kPix;
   int8_t* xl = lds;
   int8_t* stage = lds + kPix * a.pix_stride + wave * kStageBytes;
 
@@ -98,9 +98,10 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
   // are requested before the previous tile's epilogue (for the first tile: before the input
   // tile is built), so their latency hides behind work that does not need them.
   auto frag_ptr = [&](int t, int k) { return a.wpk + (static_cast<size_t>(t) * a.ksteps + k) * 64 + lane; };
-  v4i nf[4];
+  constexpr int kRing = PT == 4 ? 2 : 4;  // fragments in flight; four pixel tiles leave room for two
+  v4i nf[kRing];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) nf[j] = *frag_ptr(n_tiles > 0 ? tile0 : 0, min(j, a.ksteps - 1));
+  for (int j = 0; j < kRing; ++j) nf[j] = *frag_ptr(n_tiles > 0 ? tile0 : 0, min(j, a.ksteps - 1));
 
   // ---- activations of the 128 pixels, all channels: global (pixel-innermost) -> LDS
   {
@@ -110,9 +111,9 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
     // may straddle two images or the end of the batch.
     constexpr int kQuads = KP / 4;
     const int pq = tid % kQuads, cg0 = tid / kQuads;  // 4-pixel group, first 16-channel group
-    const long long q0 = q_base + pq * 4;
+    const int q0 = q_base + pq * 4;
     const bool live = q0 < a.Q;
-    const long long n = live ? q0 / a.HW : 0;
+    const int n = live ? static_cast<int>(static_cast<uint32_t>(q0) / static_cast<uint32_t>(a.HW)) : 0;
     const int p = live ? static_cast<int>(q0 - n * a.HW) : 0;
     const bool whole = GRAN >= 4 ? live : (q0 + 3 < a.Q && p + 3 < a.HW);
     const uint8_t* src = a.x + (static_cast<size_t>(n) * a.C) * a.HW + p;
@@ -130,7 +131,7 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
     // fetch read a valid address (channel clamped, src at the tensor base) and are masked.
     // The last row of the tensor must not be read past its end: there the dword is fetched
     // 4 - k bytes early and shifted down.
-    const bool last_image = GRAN == 1 && live && !whole && (n + 1) * static_cast<long long>(a.HW) >= a.Q;
+    const bool last_image = GRAN == 1 && live && !whole && static_cast<long long>(n + 1) * a.HW >= a.Q;
     const int back = last_image ? 4 - k_first : 0;
     const bool any_split = GRAN == 1 && __any(live && !whole);
     for (int cg = cg0; cg < a.cp / 16; cg += kThreads / kQuads) {
@@ -182,9 +183,9 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
   constexpr int kPerRow = kRowBytes / kUnit;
   constexpr int kRowsPerIter = 64 / kPerRow;
   const int px_in_row = (lane % kPerRow) * kUnit;
-  const long long oq0 = q_base + part * kRowBytes + px_in_row;
+  const int oq0 = q_base + part * kRowBytes + px_in_row;
   const bool out_live = oq0 < a.Q;
-  const long long on = out_live ? oq0 / a.HW : 0;
+  const int on = out_live ? static_cast<int>(static_cast<uint32_t>(oq0) / static_cast<uint32_t>(a.HW)) : 0;
   const int op0 = out_live ? static_cast<int>(oq0 - on * a.HW) : 0;
   const size_t out_off = static_cast<size_t>(on) * a.OC * a.HW + static_cast<size_t>(op0);
   const bool out_whole = GRAN >= 4 ? out_live : (oq0 + 3 < a.Q && op0 + 3 < a.HW);
@@ -193,9 +194,9 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
   if (GRAN == 1 && out_live && !out_whole) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const long long qe = oq0 + e;
+      const int qe = oq0 + e;
       out_px_live[e] = qe < a.Q;
-      const long long ne = out_px_live[e] ? qe / a.HW : 0;
+      const int ne = out_px_live[e] ? static_cast<int>(static_cast<uint32_t>(qe) / static_cast<uint32_t>(a.HW)) : 0;
       out_px_off[e] = static_cast<size_t>(ne) * a.OC * a.HW + static_cast<size_t>(qe - ne * a.HW);
     }
   }
@@ -203,6 +204,17 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
   const int frag_row = lane & 31, frag_half = lane >> 5;
   const int8_t* xa = xl + (part * kRowBytes + frag_row) * a.pix_stride + frag_half * 16;
   v16i acc[PT];
+  // The zero-point term -zws * sum_c xs is the same for every output channel of a pixel. With
+  // at most two pixel tiles per item it gets accumulators of its own, filled while the first
+  // output tile is computed (an independent MFMA chain) and added to every tile's result.
+  constexpr bool kSplitZp = ZP && PT <= 2;
+  v16i accz[kSplitZp ? PT : 1];
+  if (kSplitZp) {
+#pragma unroll
+    for (int i = 0; i < PT; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) accz[i][r] = 0;
+  }
   int tile = tile0;
   auto init_acc = [&]() {
     const int b = a.biasf[tile * 32 + frag_row];
@@ -224,7 +236,8 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
         const int pl = i * 32 + 8 * g + 4 * frag_half;
         int v[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = Requant8<RQ>(acc[i][g * 4 + e], q, a.out_zp, lo, hi);
+        for (int e = 0; e < 4; ++e)
+          v[e] = Requant8<RQ>(acc[i][g * 4 + e] + (kSplitZp ? accz[i][g * 4 + e] : 0), q, a.out_zp, lo, hi);
         *reinterpret_cast<uint32_t*>(stage + frag_row * kStageStride + pl) = PackBytes(v[0], v[1], v[2], v[3]);
       }
     __builtin_amdgcn_wave_barrier();
@@ -262,7 +275,7 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
     __builtin_amdgcn_wave_barrier();
   };
 
-  auto step = [&](const v4i& fw, int ks) {
+  auto step = [&](const v4i& fw, int ks, bool first_tile) {
     v4i fx[PT];
 #pragma unroll
     for (int i = 0; i < PT; ++i)
@@ -270,28 +283,32 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(4,
 #pragma unroll
     for (int i = 0; i < PT; ++i) {
       acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fx[i], fw, acc[i], 0, 0, 0);
-      if (ZP) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fx[i], fz, acc[i], 0, 0, 0);
+      if (kSplitZp) {
+        if (first_tile) accz[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fx[i], fz, accz[i], 0, 0, 0);
+      } else if (ZP) {
+        acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fx[i], fz, acc[i], 0, 0, 0);
+      }
     }
   };
 
   for (int ti = 0; ti < n_tiles; ++ti, tile += tile_step) {
     init_acc();
-    v4i ring[4];
+    v4i ring[kRing];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) ring[j] = nf[j];
-    for (int k0 = 0; k0 < a.ksteps; k0 += 4) {
+    for (int j = 0; j < kRing; ++j) ring[j] = nf[j];
+    for (int k0 = 0; k0 < a.ksteps; k0 += kRing) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < kRing; ++j) {
         if (k0 + j < a.ksteps) {
           const v4i g = ring[j];
-          if (k0 + j + 4 < a.ksteps) ring[j] = *frag_ptr(tile, k0 + j + 4);
-          step(g, k0 + j);
+          if (k0 + j + kRing < a.ksteps) ring[j] = *frag_ptr(tile, k0 + j + kRing);
+          step(g, k0 + j, ti == 0);
         }
       }
     }
     const int next_tile = tile + tile_step < t_end ? tile + tile_step : tile;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) nf[j] = *frag_ptr(next_tile, min(j, a.ksteps - 1));
+    for (int j = 0; j < kRing; ++j) nf[j] = *frag_ptr(next_tile, min(j, a.ksteps - 1));
     epilogue();
   }
 }
@@ -376,7 +393,8 @@ int PwConvSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const 
   const uint64_t hw = static_cast<uint64_t>(d->in_w) * d->in_h;
   if (hw >= (1ull << 30) || hw < 4) return TVX_E_UNSUPPORTED;  // a 4-pixel group spans at most two images
   a.HW = static_cast<int>(hw);
-  a.Q = static_cast<long long>(hw) * d->batch;
+  if (hw * d->batch >= (1ull << 31) - 256) return TVX_E_UNSUPPORTED;
+  a.Q = static_cast<int>(hw * d->batch);
   a.cp = RoundUp(a.C, 32);
   a.ksteps = a.cp / 32;
   a.pix_stride = a.cp + 16;
@@ -392,7 +410,7 @@ int PwConvSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const 
   }
   const int lds_bytes = kp * a.pix_stride + nw * kStageBytes;
   if (lds_bytes > 160 * 1024) return TVX_E_UNSUPPORTED;
-  const long long gx = (a.Q + kp - 1) / kp;
+  const long long gx = (static_cast<long long>(a.Q) + kp - 1) / kp;
   if (gx > 0x7fffffffll) return TVX_E_UNSUPPORTED;
   const bool x_u8 = d->in_dtype == TVX_U8, w_u8 = d->w_dtype == TVX_U8;
   const int zxs = d->in_zp - (x_u8 ? 128 : 0);
