@@ -84,7 +84,7 @@ def test_conv2d_without_bias_and_runtime_weights(oracle):
 
 
 @pytest.mark.parametrize("mode", ["u8", "i8pc", "u8pc", "f32", "f16"])
-@pytest.mark.parametrize("shape", [(5, 37, 11), (64, 256, 48), (1, 800, 500), (33, 130, 70)])
+@pytest.mark.parametrize("shape", [(5, 37, 11), (64, 256, 48), (1, 800, 500), (33, 130, 70), (7, 500, 10), (3, 1283, 200)])
 def test_fully_connected_random(oracle, mode, shape):
     m, k, n = shape
     rng = np.random.default_rng(m * 7 + k)
@@ -173,7 +173,7 @@ def test_eltwise_float(oracle):
 
 
 @pytest.mark.parametrize("mode", ["u8", "i8pc", "u8pc"])
-@pytest.mark.parametrize("shape", [(300, 512, 272), (257, 144, 513), (2, 1280, 1000)])
+@pytest.mark.parametrize("shape", [(300, 512, 272), (257, 144, 513), (12, 1280, 1000)])
 def test_fully_connected_mfma_edges(oracle, mode, shape):
     """Tile edges of the MFMA variant: M, N not multiples of the 256-tile, K of the 128-step."""
     m, k, n = shape

@@ -442,6 +442,8 @@ int FcMfmaSetup(tvx_op* op, const tvx_fc_desc* d, const void* w_host, const void
   if (w_host && d->in_dtype == TVX_F16 && d->w_dtype == TVX_F16 && d->out_dtype == TVX_F16)
     return FcMfmaSetupF16(op, d, w_host, bias_host);
   if (!op->quantized || !w_host || (d->k & 15) != 0) return TVX_E_UNSUPPORTED;
+  // a handful of outputs does not fill one 256 x 256 tile: the wavefront-per-output kernel is quicker
+  if (static_cast<uint64_t>(d->m) * d->n <= 8192) return TVX_E_UNSUPPORTED;
   if (static_cast<uint64_t>(d->m) * d->n >= (1ull << 31) || d->k > (1u << 24)) return TVX_E_UNSUPPORTED;
   if (static_cast<uint64_t>(d->m) * d->k >= (1ull << 32) || static_cast<uint64_t>(d->n) * d->k >= (1ull << 32))
     return TVX_E_UNSUPPORTED;  // the operand DMA addresses rows with 32-bit offsets

@@ -161,6 +161,45 @@ FcQuantKernel(FcArgs a, const XT* __restrict__ x, const WT* __restrict__ w,
   y[idx] = static_cast<XT>(RequantClamp(acc, mult[n], shift[n], a.out_zp, a.lo, a.hi));
 }
 
+// One wavefront per output: the lanes stride over K four bytes at a time (consecutive lanes
+// read consecutive dwords of both rows) and the partial sums meet in a butterfly. For the
+// small FullyConnected layers at the end of a network - a few thousand outputs with a long
+// reduction - where one thread per output would walk its row alone.
+template <typename XT, typename WT>
+__global__ void __launch_bounds__(kBlock)
+FcQuantWaveKernel(FcArgs a, const XT* __restrict__ x, const WT* __restrict__ w,
+                  const int32_t* __restrict__ bias, const int32_t* __restrict__ mult,
+                  const int32_t* __restrict__ shift, XT* __restrict__ y, uint64_t total) {
+  const int lane = threadIdx.x & 63;
+  const uint64_t idx = static_cast<uint64_t>(blockIdx.x) * (kBlock / 64) + (threadIdx.x >> 6);
+  if (idx >= total) return;
+  const int n = idx % a.n;
+  const uint64_t m = idx / a.n;
+  const XT* xp = x + m * a.k;
+  const WT* wp = w + static_cast<uint64_t>(n) * a.k;
+  int32_t acc = 0;
+  const int k4 = a.k & ~3;
+  for (int k = lane * 4; k < k4; k += 256) {
+    uint32_t xv, wv;
+    __builtin_memcpy(&xv, xp + k, 4);  // rows start at any byte: unaligned dwords
+    __builtin_memcpy(&wv, wp + k, 4);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int32_t xe = static_cast<int32_t>(static_cast<XT>(xv >> (8 * b)));
+      const int32_t we = static_cast<int32_t>(static_cast<WT>(wv >> (8 * b)));
+      acc += (xe - a.in_zp) * (we - a.w_zp);
+    }
+  }
+  if (k4 + lane < a.k)
+    acc += (static_cast<int32_t>(xp[k4 + lane]) - a.in_zp) * (static_cast<int32_t>(wp[k4 + lane]) - a.w_zp);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+  if (lane == 0) {
+    if (bias) acc += bias[n];
+    y[idx] = static_cast<XT>(RequantClamp(acc, mult[n], shift[n], a.out_zp, a.lo, a.hi));
+  }
+}
+
 template <typename T>
 __global__ void __launch_bounds__(kBlock)
 FcFloatKernel(FcArgs a, const T* __restrict__ x, const T* __restrict__ w,
@@ -186,18 +225,36 @@ int FcGenericRun(tvx_op* op, const void* in0, const void* in1, void* out, hipStr
   const dim3 grid(Blocks(total)), block(kBlock);
   const int32_t* bias_i = op->bias.as<int32_t>();
   const int32_t *mu = op->mult.as<int32_t>(), *sh = op->shift.as<int32_t>();
+  // few outputs with a long reduction: a wavefront per output
+  const bool wave = total <= 16384 && d.k >= 128;
+  const dim3 wgrid(static_cast<unsigned>((total + kBlock / 64 - 1) / (kBlock / 64)));
   if (d.in_dtype == TVX_U8 && d.w_dtype == TVX_U8) {
-    hipLaunchKernelGGL((FcQuantKernel<uint8_t, uint8_t>), grid, block, 0, st, a,
-                       static_cast<const uint8_t*>(in0), static_cast<const uint8_t*>(w), bias_i,
-                       mu, sh, static_cast<uint8_t*>(out), total);
+    if (wave)
+      hipLaunchKernelGGL((FcQuantWaveKernel<uint8_t, uint8_t>), wgrid, block, 0, st, a,
+                         static_cast<const uint8_t*>(in0), static_cast<const uint8_t*>(w), bias_i,
+                         mu, sh, static_cast<uint8_t*>(out), total);
+    else
+      hipLaunchKernelGGL((FcQuantKernel<uint8_t, uint8_t>), grid, block, 0, st, a,
+                         static_cast<const uint8_t*>(in0), static_cast<const uint8_t*>(w), bias_i,
+                         mu, sh, static_cast<uint8_t*>(out), total);
   } else if (d.in_dtype == TVX_U8 && d.w_dtype == TVX_I8) {
-    hipLaunchKernelGGL((FcQuantKernel<uint8_t, int8_t>), grid, block, 0, st, a,
-                       static_cast<const uint8_t*>(in0), static_cast<const int8_t*>(w), bias_i, mu,
-                       sh, static_cast<uint8_t*>(out), total);
+    if (wave)
+      hipLaunchKernelGGL((FcQuantWaveKernel<uint8_t, int8_t>), wgrid, block, 0, st, a,
+                         static_cast<const uint8_t*>(in0), static_cast<const int8_t*>(w), bias_i, mu,
+                         sh, static_cast<uint8_t*>(out), total);
+    else
+      hipLaunchKernelGGL((FcQuantKernel<uint8_t, int8_t>), grid, block, 0, st, a,
+                         static_cast<const uint8_t*>(in0), static_cast<const int8_t*>(w), bias_i, mu,
+                         sh, static_cast<uint8_t*>(out), total);
   } else if (d.in_dtype == TVX_I8) {
-    hipLaunchKernelGGL((FcQuantKernel<int8_t, int8_t>), grid, block, 0, st, a,
-                       static_cast<const int8_t*>(in0), static_cast<const int8_t*>(w), bias_i, mu,
-                       sh, static_cast<int8_t*>(out), total);
+    if (wave)
+      hipLaunchKernelGGL((FcQuantWaveKernel<int8_t, int8_t>), wgrid, block, 0, st, a,
+                         static_cast<const int8_t*>(in0), static_cast<const int8_t*>(w), bias_i, mu,
+                         sh, static_cast<int8_t*>(out), total);
+    else
+      hipLaunchKernelGGL((FcQuantKernel<int8_t, int8_t>), grid, block, 0, st, a,
+                         static_cast<const int8_t*>(in0), static_cast<const int8_t*>(w), bias_i, mu,
+                         sh, static_cast<int8_t*>(out), total);
   } else if (d.in_dtype == TVX_F32) {
     hipLaunchKernelGGL((FcFloatKernel<float>), grid, block, 0, st, a,
                        static_cast<const float*>(in0), static_cast<const float*>(w),
