@@ -1,0 +1,142 @@
+"""Seeded differential sweep: random operator configurations, HIP result vs oracle, bit for bit.
+The shapes are drawn so that every kernel variant is reached many times (dense 3x3 / 5x5 /
+strided / dilated, pointwise with every pixel-count residue, depthwise on aligned and odd
+widths, FullyConnected around the tile and K-chunk edges, pooling of every type)."""
+import collections
+
+import numpy as np
+import pytest
+
+import tvx_case as TC
+from test_gpu_parity import conv_case, rand_q
+
+pytestmark = pytest.mark.gpu
+
+
+def _conv_config(rng):
+    kind = rng.choice(["dense", "pointwise", "depthwise", "depthwise_mobile"])
+    n = int(rng.integers(1, 4))
+    if kind == "depthwise_mobile":
+        # the MobileNet shape: 3x3, one stride for both axes, SAME padding, rows of whole dwords
+        st = int(rng.choice([1, 2]))
+        w, h = 4 * st * int(rng.integers(1, 9)), int(rng.integers(3, 24))
+        pl, pt = int(rng.integers(0, 2)), int(rng.integers(0, 2))
+        return dict(n=n, c=int(rng.integers(1, 70)), h=h, w=w, oc=0, kh=3, kw=3, stride=[st, st], dil=[1, 1],
+                    pad=[pl, 2 - pl if st == 1 else 1 - pl, pt, 1], mult=1)
+    if kind == "pointwise":
+        c, oc = int(rng.integers(1, 200)), int(rng.integers(1, 200))
+        h, w = int(rng.integers(1, 20)), int(rng.integers(2, 20))
+        if h * w < 4:
+            h = 2
+        return dict(n=n, c=c, h=h, w=w, oc=oc, kh=1, kw=1, stride=[1, 1], dil=[1, 1], pad=[0, 0, 0, 0], mult=0)
+    kh, kw = (int(rng.choice([1, 2, 3, 5])), int(rng.choice([1, 3, 5]))) if rng.random() < 0.3 else (3, 3)
+    s = [int(rng.choice([1, 1, 2])), int(rng.choice([1, 1, 2]))]
+    d = [int(rng.choice([1, 1, 1, 2])), int(rng.choice([1, 1, 1, 2]))]
+    # padding never exceeds the kernel's reach: every window touches the image
+    pad = [int(min(rng.integers(0, 3), (kw - 1) * d[0])) for _ in range(2)] + \
+          [int(min(rng.integers(0, 3), (kh - 1) * d[1])) for _ in range(2)]
+    h = int(rng.integers((kh - 1) * d[1] + 1, 24))
+    w = int(rng.choice([4, 8, 12, 16, 20, 28])) if rng.random() < 0.5 else int(rng.integers((kw - 1) * d[0] + 1, 24))
+    w = max(w, (kw - 1) * d[0] + 1)
+    if kind == "depthwise":
+        return dict(n=n, c=int(rng.integers(1, 40)), h=h, w=w, oc=0, kh=kh, kw=kw, stride=s, dil=d, pad=pad,
+                    mult=int(rng.choice([1, 1, 1, 2])))
+    return dict(n=n, c=int(rng.integers(1, 150)), h=h, w=w, oc=int(rng.integers(1, 150)), kh=kh, kw=kw,
+                stride=s, dil=d, pad=pad, mult=0)
+
+
+def test_conv2d_sweep(oracle, tvx):
+    rng = np.random.default_rng(0xC0)
+    seen = collections.Counter()
+    for i in range(240):
+        cfg = _conv_config(rng)
+        mode = str(rng.choice(["u8", "i8pc", "u8pc"]))
+        act = int(rng.integers(0, 3))
+        x, wt, b, kws = conv_case(rng, mode=mode, **cfg)
+        if min(kws["out_shape"][:2]) < 1:
+            continue
+        want = oracle.conv2d(x, wt, b, act=act, **kws)
+        d_kernel = []
+        got = _run_conv(tvx, x, wt, b, act, kws, d_kernel)
+        seen[d_kernel[0]] += 1
+        assert np.array_equal(got, want), (i, cfg, mode, act, d_kernel[0], int((got != want).sum()))
+    # the sweep is only worth its name if it reaches every convolution kernel
+    for k in ("conv2d_igemm_i8", "pwconv_i8", "dwconv3x3_i8", "dwconv_planes_i8", "conv2d_generic"):
+        assert seen[k] >= 5, seen
+
+
+def _run_conv(tvx, x, wt, b, act, kws, kernel_out):
+    """gpu_conv2d, also reporting which kernel ran."""
+    import ctypes as C
+    import torch
+    d = tvx.Conv2dDesc()
+    d.in_w, d.in_h, d.in_c, d.batch = kws["in_shape"]
+    d.k_w, d.k_h = kws["w_shape"][0], kws["w_shape"][1]
+    d.out_w, d.out_h, d.out_c = kws["out_shape"][:3]
+    d.stride_w, d.stride_h = kws["stride"]
+    d.dilation_w, d.dilation_h = kws["dilation"]
+    d.pad_left, d.pad_top, d.multiplier = kws["pad_left"], kws["pad_top"], kws["multiplier"]
+    d.in_dtype, d.w_dtype, d.out_dtype = kws["in_dtype"], kws["w_dtype"], kws["out_dtype"]
+    d.in_scale, d.in_zp = kws["in_q"]
+    d.w_scale, d.w_zp = kws["w_q"][0], kws["w_q"][1]
+    keep = None
+    if kws["w_q"][2] is not None:
+        keep = np.ascontiguousarray(kws["w_q"][2], dtype=np.float32)
+        d.w_scales = keep.ctypes.data_as(C.POINTER(C.c_float))
+    d.out_scale, d.out_zp = kws["out_q"]
+    d.activation = act
+    op = tvx.conv2d_create(d, wt, b)
+    kernel_out.append(op.kernel_name)
+    xd = TC.to_device(x)
+    yd = TC.device_out(int(np.prod(kws["out_shape"])), TC.NP_OF[kws["out_dtype"]])
+    op.run(xd, None, yd)
+    torch.cuda.synchronize()
+    out = yd.cpu().numpy()
+    op.close()
+    return out
+
+
+def test_fully_connected_sweep(oracle):
+    rng = np.random.default_rng(0xFC)
+    for i in range(60):
+        m = int(rng.choice([1, 2, 7, 33, 255, 256, 257, 300]))
+        k = int(rng.choice([16, 48, 112, 128, 144, 500, 512, 800, 1000]))
+        n = int(rng.choice([1, 10, 31, 64, 255, 256, 257, 500]))
+        mode = str(rng.choice(["u8", "i8pc", "u8pc"]))
+        in_dt = 0 if mode.startswith("u8") else 1
+        w_dt = 0 if mode == "u8" else 1
+        x, w = rand_q(rng, m * k, in_dt), rand_q(rng, n * k, w_dt)
+        b = rng.integers(-16384, 16385, n).astype(np.int32)
+        wq = (0.01, int(rng.integers(100, 157)), None) if mode == "u8" else \
+            (1.0, 0, np.exp(rng.uniform(np.log(0.001), np.log(0.02), n)).astype(np.float32))
+        kws = dict(m=m, k=k, n=n, in_dtype=in_dt, w_dtype=w_dt, out_dtype=in_dt,
+                   in_q=(0.02, int(rng.integers(100, 157)) if in_dt == 0 else int(rng.integers(-9, 10))), w_q=wq,
+                   out_q=(float(np.float32(0.02 * 0.01 * 40 * np.sqrt(k))), 5 if in_dt == 0 else -3))
+        act = int(rng.integers(0, 3))
+        want = oracle.fully_connected(x, w, b, act=act, **kws)
+        got = TC.gpu_fully_connected(x, w, b, act=act, **kws)
+        assert np.array_equal(got, want), (i, m, k, n, mode, act)
+
+
+def test_pool2d_sweep(oracle):
+    rng = np.random.default_rng(0xB0)
+    for i in range(80):
+        w, h = int(rng.integers(1, 30)), int(rng.integers(1, 30))
+        kw, kh = int(rng.integers(1, min(w, 7) + 1)), int(rng.integers(1, min(h, 7) + 1))
+        s = [int(rng.integers(1, 4)), int(rng.integers(1, 4))]
+        pad = [int(rng.integers(0, kw)), int(rng.integers(0, kw)), int(rng.integers(0, kh)), int(rng.integers(0, kh))]
+        c, n = int(rng.integers(1, 9)), int(rng.integers(1, 4))
+        out_w = (w + pad[0] + pad[1] - kw) // s[0] + 1
+        out_h = (h + pad[2] + pad[3] - kh) // s[1] + 1
+        if out_w < 1 or out_h < 1:
+            continue
+        dtype = int(rng.integers(0, 2))
+        ptype = int(rng.choice([0, 1, 3]))
+        kws = dict(in_shape=[w, h, c, n], out_shape=[out_w, out_h, c, n], ksize=[kw, kh], stride=s,
+                   pad_left=pad[0], pad_top=pad[2], pool_type=ptype, dtype=dtype)
+        x = rand_q(rng, w * h * c * n, dtype)
+        in_q = (0.1, 7)
+        out_q = (0.1, 7) if rng.random() < 0.5 else (0.07, 9 if dtype == 0 else -2)
+        want = oracle.pool2d(x, in_q=in_q, out_q=out_q, **kws)
+        got = TC.gpu_pool2d(x, in_q=in_q, out_q=out_q, **kws)
+        assert np.array_equal(got, want), (i, kws)
