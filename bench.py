@@ -280,6 +280,13 @@ def main():
                                      gbs=round(w2["algo_bytes"] / (wall2 * 1e-3) / 1e9, 1),
                                      roofline=dict(roofline(w2, k2), kernel_ms=round(k2, 5)))
         extra.update(network_extras(max(5, min(args.steps, 30)), 3))
+        # what this very device sustains with the simplest kernels: the int8 matrix cores on
+        # zeros (nominal clock) and on random bytes (the clock held under load), a streaming copy
+        extra["device_calibration"] = {
+            "mfma_i8_tops_zero_operands": round(T.calibrate_mfma_i8(False), 0),
+            "mfma_i8_tops_random_operands": round(T.calibrate_mfma_i8(True), 0),
+            "copy_read_plus_write_gbs": round(T.calibrate_copy(), 0),
+        }
         line["extra"] = extra
     print(json.dumps(line))
 

@@ -108,6 +108,8 @@ def lib():
         L.tvx_add_create.argtypes = [C.POINTER(EltwiseDesc), C.POINTER(vp)]
         L.tvx_softmax_create.argtypes = [C.POINTER(SoftmaxDesc), C.POINTER(vp)]
         L.tvx_op_run.argtypes = [vp, vp, vp, vp, vp]
+        L.tvx_calibrate_mfma_i8.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_double)]
+        L.tvx_calibrate_copy.argtypes = [C.c_size_t, C.c_int, C.POINTER(C.c_double)]
         L.tvx_op_destroy.argtypes = [vp]
         L.tvx_op_destroy.restype = None
         _lib = L
@@ -188,3 +190,18 @@ def softmax_create(desc):
     h = C.c_void_p()
     check(lib().tvx_softmax_create(C.byref(desc), C.byref(h)))
     return Op(h)
+
+
+def calibrate_mfma_i8(random_operands, launches=5):
+    """Sustained int8 matrix-core rate of this GPU in TOPS (zeros: nominal clock; random
+    operands: the clock held under the multipliers' switching power)."""
+    v = C.c_double()
+    check(lib().tvx_calibrate_mfma_i8(int(bool(random_operands)), launches, C.byref(v)))
+    return v.value
+
+
+def calibrate_copy(nbytes=256 << 20, launches=10):
+    """Read + write GB/s of a plain streaming device copy of `nbytes`."""
+    v = C.c_double()
+    check(lib().tvx_calibrate_copy(nbytes, launches, C.byref(v)))
+    return v.value

@@ -56,6 +56,7 @@ struct FcArgs {
   int zws;              // weight zero point in the int8 domain (0 for per-channel)
   int out_zp, lo, hi;
   int tiles_m, tiles_n;
+  int group_m;          // tile rows per panel of the tile order
 };
 
 
@@ -80,7 +81,15 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   int tile = blockIdx.x;
   const int total = a.tiles_m * a.tiles_n;
   if ((total & 7) == 0) tile = (tile & 7) * (total >> 3) + (tile >> 3);
-  const int tn_idx = tile % a.tiles_n, tm_idx = tile / a.tiles_n;
+  // Within that run, tiles go in panels of `group_m` tile rows, column by column: the
+  // workgroups running at the same time on an XCD then form a near-square block of tiles and
+  // share each operand panel between more of them (a 4 x 8 block re-reads 12 panels per
+  // k-tile for 32 tiles, a 2 x 16 block 18).
+  const int per_group = a.group_m * a.tiles_n;
+  const int first_m = (tile / per_group) * a.group_m;
+  const int gm = min(a.tiles_m - first_m, a.group_m);
+  const int in_group = tile % per_group;
+  const int tm_idx = first_m + in_group % gm, tn_idx = in_group / gm;
   const int m0 = tm_idx * TM, n0 = tn_idx * TN;
 
   // ---- global -> LDS DMA ------------------------------------------------------
@@ -389,6 +398,7 @@ int FcMfmaRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t s
   a.hi = op->act_hi;
   a.tiles_m = (a.M + TM - 1) / TM;
   a.tiles_n = (a.N + TN - 1) / TN;
+  a.group_m = 4;
   const dim3 grid(a.tiles_m * a.tiles_n);
   if (op->geo[2]) {  // float16
     a.K = static_cast<int>(d.k) * 2;
