@@ -368,6 +368,15 @@ DWP_GRID = [
     (2, 5, 13, 6, 3, 3, [1, 2], [2, 2], [2, 2, 2, 2]),
     (1, 3, 5, 9, 1, 3, [1, 1], [1, 1], [1, 1, 0, 0]),
     (70, 33, 7, 7, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),
+    # 3x3 dword form: left padding 0 / 2 / 3, widths 4 / 5 / 6 / 13, stride 2 on odd widths, rows
+    # of padding only at the top, more right padding than the kernel reaches
+    (3, 11, 6, 5, 3, 3, [1, 1], [1, 1], [0, 0, 0, 0]),
+    (2, 9, 8, 13, 3, 3, [1, 1], [1, 1], [2, 1, 2, 0]),
+    (2, 6, 5, 6, 3, 3, [1, 1], [1, 1], [3, 2, 1, 2]),
+    (5, 17, 13, 13, 3, 3, [2, 2], [1, 1], [1, 1, 1, 1]),
+    (3, 8, 9, 4, 3, 3, [2, 2], [1, 1], [0, 1, 1, 0]),
+    (2, 12, 7, 28, 3, 3, [1, 1], [1, 1], [2, 2, 1, 1]),
+    (64, 96, 14, 14, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),
 ]
 
 

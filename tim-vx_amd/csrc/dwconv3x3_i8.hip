@@ -176,6 +176,56 @@ int DwRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
 
 }  // namespace
 
+// Packs depthwise 3x3 weights for the signed dot4 stencils: per channel four dwords, the three
+// kernel rows (kx in bytes 0..2, byte 3 zero) and a correction word. With xs, ws the int8-domain
+// activations and weights and zxs, zws their zero points,
+//   sum (xs - zxs)(ws - zws) = sum xs wz - zxs sum wz            when wz = ws - zws fits int8,
+//                            = sum xs ws - zws Sx - zxs sum ws + 9 zxs zws   otherwise,
+// with the window sum Sx taken in the kernel. The correction word is 1 for channels in the second
+// form; with `all_or_none` every channel takes the second form as soon as one needs it (for
+// kernels that decide per operator, not per channel). The constant terms are folded into
+// `biasf`. Returns whether any channel needs the window sum.
+bool PackDepthwise3x3(int C, const void* w_host, bool w_u8, const void* bias_host, int zxs, int zws,
+                      bool all_or_none, std::vector<int32_t>* wpk_out, std::vector<int32_t>* biasf_out) {
+  std::vector<int32_t>& wpk = *wpk_out;
+  std::vector<int32_t>& biasf = *biasf_out;
+  wpk.assign(static_cast<size_t>(C) * 4, 0);
+  biasf.assign(C, 0);
+  const uint8_t* src = static_cast<const uint8_t*>(w_host);
+  const int32_t* b = static_cast<const int32_t*>(bias_host);
+  bool any_box = false, all_fit = true;
+  for (size_t i = 0; i < static_cast<size_t>(C) * 9; ++i) {
+    const int v = static_cast<int8_t>(w_u8 ? src[i] ^ 0x80 : src[i]);
+    if (v - zws < -128 || v - zws > 127) all_fit = false;
+  }
+  for (int c = 0; c < C; ++c) {
+    int ws[9];
+    bool fits = true;  // do the shifted weights ws - zws fit int8?
+    for (int t = 0; t < 9; ++t) {
+      const uint8_t raw = src[static_cast<size_t>(c) * 9 + t];
+      ws[t] = static_cast<int8_t>(w_u8 ? raw ^ 0x80 : raw);
+      if (ws[t] - zws < -128 || ws[t] - zws > 127) fits = false;
+    }
+    if (all_or_none) fits = all_fit;
+    int64_t sw = 0;
+    for (int ky = 0; ky < 3; ++ky) {
+      uint32_t pk = 0;
+      for (int kx = 0; kx < 3; ++kx) {
+        const int v = fits ? ws[ky * 3 + kx] - zws : ws[ky * 3 + kx];
+        pk |= static_cast<uint32_t>(static_cast<uint8_t>(static_cast<int8_t>(v))) << (8 * kx);
+        sw += v;
+      }
+      wpk[static_cast<size_t>(c) * 4 + ky] = static_cast<int32_t>(pk);
+    }
+    const bool box = !fits && zws != 0;
+    wpk[static_cast<size_t>(c) * 4 + 3] = box ? 1 : 0;
+    any_box |= box;
+    const int64_t v = (b ? b[c] : 0) - static_cast<int64_t>(zxs) * sw + (fits ? 0 : 9ll * zxs * zws);
+    biasf[c] = static_cast<int32_t>(static_cast<uint32_t>(v));
+  }
+  return any_box;
+}
+
 // Claims quantized depthwise 3x3, multiplier 1, dilation 1, stride 1 or 2 (both
 // directions), constant weights, row lengths that are multiples of four.
 int DwConv3x3Setup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const void* bias_host) {
@@ -198,36 +248,8 @@ int DwConv3x3Setup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   const int zws = op->w_zp - (w_u8 ? 128 : 0);
   if (zxs < -128 || zxs > 127) return TVX_E_UNSUPPORTED;
   const int C = d->in_c;
-  std::vector<int32_t> wpk(static_cast<size_t>(C) * 4), biasf(C);
-  const uint8_t* src = static_cast<const uint8_t*>(w_host);
-  const int32_t* b = static_cast<const int32_t*>(bias_host);
-  bool any_box = false;
-  for (int c = 0; c < C; ++c) {
-    int ws[9];
-    bool fits = true;  // do the shifted weights ws - zws fit int8?
-    for (int t = 0; t < 9; ++t) {
-      const uint8_t raw = src[static_cast<size_t>(c) * 9 + t];
-      ws[t] = static_cast<int8_t>(w_u8 ? raw ^ 0x80 : raw);
-      if (ws[t] - zws < -128 || ws[t] - zws > 127) fits = false;
-    }
-    // sum (xs - zxs)(ws - zws): with wz = ws - zws it is sum xs wz - zxs sum wz; otherwise
-    // sum xs ws - zws Sx - zxs sum ws + 9 zxs zws with the window sum Sx taken in the kernel
-    int64_t sw = 0;
-    for (int ky = 0; ky < 3; ++ky) {
-      uint32_t pk = 0;
-      for (int kx = 0; kx < 3; ++kx) {
-        const int v = fits ? ws[ky * 3 + kx] - zws : ws[ky * 3 + kx];
-        pk |= static_cast<uint32_t>(static_cast<uint8_t>(static_cast<int8_t>(v))) << (8 * kx);
-        sw += v;
-      }
-      wpk[static_cast<size_t>(c) * 4 + ky] = static_cast<int32_t>(pk);
-    }
-    const bool box = !fits && zws != 0;
-    wpk[static_cast<size_t>(c) * 4 + 3] = box ? 1 : 0;
-    any_box |= box;
-    const int64_t v = (b ? b[c] : 0) - static_cast<int64_t>(zxs) * sw + (fits ? 0 : 9ll * zxs * zws);
-    biasf[c] = static_cast<int32_t>(static_cast<uint32_t>(v));
-  }
+  std::vector<int32_t> wpk, biasf;
+  const bool any_box = PackDepthwise3x3(C, w_host, w_u8, bias_host, zxs, zws, false, &wpk, &biasf);
   std::vector<int32_t> rqt;
   const int rq = BuildRequantRecords(op->h_mult, op->h_shift, C, C, d->out_zp, &rqt, AccumulatorBound(9, bias_host, C));
   int s = op->packed.Upload(wpk.data(), wpk.size() * 4);

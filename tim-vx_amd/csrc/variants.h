@@ -36,6 +36,9 @@ int DwConv3x3Setup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 
 // depthwise, any kernel / width, planes staged through LDS (dwconv_planes_i8.hip)
 int DwPlanesSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
+// shared by the two depthwise 3x3 stencils (defined in dwconv3x3_i8.hip)
+bool PackDepthwise3x3(int C, const void* w_host, bool w_u8, const void* bias_host, int zxs, int zws,
+                      bool all_or_none, std::vector<int32_t>* wpk, std::vector<int32_t>* biasf);
 
 // generic (kernels_generic.hip)
 int ConvGenericSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
