@@ -37,7 +37,7 @@ struct DwArgs {
   int pad_t, pad_l;
   int ow4;               // output dwords per row
   int lpr_shift;         // log2 of the lanes an image row occupies (>= ow4 lanes, the rest idle)
-  int rg_per_block;      // row groups (of kRowsPerThread output rows) per workgroup
+  int rg_per_block;      // row groups (of RPT output rows) per workgroup
   int xor_mask, pad_fill, zws, out_zp, lo, hi;
 };
 
@@ -50,17 +50,17 @@ __device__ __forceinline__ int Window(const int (&arr)[N]) {
   return __builtin_amdgcn_alignbyte(arr[d + 1], arr[d], sh);
 }
 
-constexpr int kRowsPerThread = 4;  // output rows a thread produces
 
 // S = stride (1 or 2, both directions), PL = left padding (0 or 1)
-template <int S, int PL, bool BOXSUM, int RQ>
+// RPT: output rows a thread produces (more rows: fewer, fatter workgroups and fewer halo rows re-read)
+template <int S, int PL, bool BOXSUM, int RQ, int RPT>
 __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
   const int plane = blockIdx.x;
   const int c = plane % a.C;
   const int tid = threadIdx.x;
   const int rgl = tid >> a.lpr_shift;
   const int w4 = tid & ((1 << a.lpr_shift) - 1);
-  const int oh0 = (blockIdx.y * a.rg_per_block + rgl) * kRowsPerThread;
+  const int oh0 = (blockIdx.y * a.rg_per_block + rgl) * RPT;
   if (oh0 >= a.OH) return;  // whole rows of lanes leave together: neighbours stay consistent
 
   const uint8_t* xp = a.x + static_cast<size_t>(plane) * a.H * a.W;
@@ -75,7 +75,7 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
   // input dwords under this thread's four outputs: S of them, starting at S * w4;
   // the byte array of a row is {left neighbour, own dwords, right neighbour}
   constexpr int kOwn = S;
-  constexpr int kRows = S * (kRowsPerThread - 1) + 3;  // input rows behind the thread's output rows
+  constexpr int kRows = S * (RPT - 1) + 3;  // input rows behind the thread's output rows
   const int d0 = S * w4;
   const int ih0 = oh0 * S - a.pad_t;
   const bool has_left = w4 > 0;                      // else: left of the image
@@ -119,7 +119,7 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
   }
   if (w4 >= a.ow4) return;  // lanes that only fed their neighbour
 #pragma unroll
-  for (int o = 0; o < kRowsPerThread; ++o) {
+  for (int o = 0; o < RPT; ++o) {
     if (oh0 + o >= a.OH) break;
     uint32_t packed = 0;
 #pragma unroll
@@ -142,22 +142,28 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
 
 struct Plan {
   DwArgs a;
-  int stride, pad_l, boxsum, rq;
+  int stride, pad_l, boxsum, rq, rows_per_thread;
   dim3 grid;
 };
 
-template <int S, int PL, bool BOXSUM>
+template <int S, int PL, bool BOXSUM, int RPT>
 void LaunchRq(const Plan* p, const DwArgs& a, hipStream_t st) {
   const dim3 block(kThreads);
-  if (p->rq == kRqFastNoTie) hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqFastNoTie>), p->grid, block, 0, st, a);
-  else if (p->rq == kRqFast) hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqFast>), p->grid, block, 0, st, a);
-  else hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqGeneric>), p->grid, block, 0, st, a);
+  if (p->rq == kRqFastNoTie) hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqFastNoTie, RPT>), p->grid, block, 0, st, a);
+  else if (p->rq == kRqFast) hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqFast, RPT>), p->grid, block, 0, st, a);
+  else hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqGeneric, RPT>), p->grid, block, 0, st, a);
 }
 
 template <int S, int PL>
 void LaunchBox(const Plan* p, const DwArgs& a, hipStream_t st) {
-  if (p->boxsum) LaunchRq<S, PL, true>(p, a, st);
-  else LaunchRq<S, PL, false>(p, a, st);
+  // eight rows per thread only exist for stride 1 (chosen for tall planes)
+  if (S == 1 && p->rows_per_thread == 8) {
+    if (p->boxsum) LaunchRq<1, PL, true, 8>(p, a, st);
+    else LaunchRq<1, PL, false, 8>(p, a, st);
+  } else {
+    if (p->boxsum) LaunchRq<S, PL, true, 4>(p, a, st);
+    else LaunchRq<S, PL, false, 4>(p, a, st);
+  }
 }
 
 int DwRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
@@ -266,11 +272,14 @@ int DwConv3x3Setup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   a.ow4 = ow4;
   a.lpr_shift = lpr_shift;
   a.rg_per_block = kThreads >> lpr_shift;
-  const int row_groups = (static_cast<int>(d->out_h) + kRowsPerThread - 1) / kRowsPerThread;
+  // tall planes at stride 1: eight output rows per thread (a third of the workgroups to dispatch,
+  // ten input rows read for eight instead of six for four)
+  const int rpt = S == 1 && d->out_h >= 96 ? 8 : 4;
+  const int row_groups = (static_cast<int>(d->out_h) + rpt - 1) / rpt;
   a.xor_mask = x_u8 ? static_cast<int>(0x80808080u) : 0;
   a.pad_fill = static_cast<int>(static_cast<uint32_t>(zxs & 0xff) * 0x01010101u);
   a.zws = zws; a.out_zp = d->out_zp; a.lo = op->act_lo; a.hi = op->act_hi;
-  p.stride = S; p.pad_l = d->pad_left; p.boxsum = any_box; p.rq = rq;
+  p.stride = S; p.pad_l = d->pad_left; p.boxsum = any_box; p.rq = rq; p.rows_per_thread = rpt;
   p.grid = dim3(d->batch * C, (row_groups + a.rg_per_block - 1) / a.rg_per_block);
   op->host_blob.assign(reinterpret_cast<const uint8_t*>(&p), reinterpret_cast<const uint8_t*>(&p) + sizeof(p));
   op->run = DwRun;
