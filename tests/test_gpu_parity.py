@@ -172,10 +172,23 @@ def test_eltwise_float(oracle):
     assert np.array_equal(TC.gpu_activation(1, 2, h, (1.0, 0), (1.0, 0)), np.maximum(h, 0))
 
 
+FC_EDGE_SHAPES = [
+    # 256 x 256 tiles: M, N not multiples of the tile, K not of the 128-byte step
+    ((600, 512, 528), "fc_mfma_i8_256x256x128"), ((513, 144, 769), "fc_mfma_i8_256x256x128"),
+    # few outputs -> 16 x 16 tiles with the reduction split over four wavefronts: ragged M / N, N not a
+    # multiple of 4 (byte stores), K with a 16 / 32 / 48-byte tail and shorter than one 64-byte step,
+    # more k-steps than one batch of loads, the MobileNetV2 and LeNet classifier shapes
+    ((300, 512, 272), "fc_mfma_i8_16x16_splitk"), ((257, 144, 513), "fc_mfma_i8_16x16_splitk"),
+    ((12, 1280, 1000), "fc_mfma_i8_16x16_splitk"), ((64, 1280, 1000), "fc_mfma_i8_16x16_splitk"),
+    ((256, 800, 500), "fc_mfma_i8_16x16_splitk"), ((17, 48, 1001), "fc_mfma_i8_16x16_splitk"),
+    ((1000, 16, 9), "fc_mfma_i8_16x16_splitk"), ((33, 4112, 250), "fc_mfma_i8_16x16_splitk"),
+]
+
+
 @pytest.mark.parametrize("mode", ["u8", "i8pc", "u8pc"])
-@pytest.mark.parametrize("shape", [(300, 512, 272), (257, 144, 513), (12, 1280, 1000)])
-def test_fully_connected_mfma_edges(oracle, mode, shape):
-    """Tile edges of the MFMA variant: M, N not multiples of the 256-tile, K of the 128-step."""
+@pytest.mark.parametrize("shape,kernel", FC_EDGE_SHAPES)
+def test_fully_connected_mfma_edges(oracle, mode, shape, kernel):
+    """Tile and reduction edges of the two MFMA variants."""
     m, k, n = shape
     rng = np.random.default_rng(m + k + n)
     in_dt = 0 if mode.startswith("u8") else 1
@@ -187,9 +200,10 @@ def test_fully_connected_mfma_edges(oracle, mode, shape):
     kws = dict(m=m, k=k, n=n, in_dtype=in_dt, w_dtype=w_dt, out_dtype=in_dt,
                in_q=(0.02, 131 if in_dt == 0 else -2), w_q=wq,
                out_q=(float(np.float32(0.02 * 0.01 * 40 * np.sqrt(k))), 5 if in_dt == 0 else 0))
-    want = oracle.fully_connected(x, w, b, **kws)
-    got = TC.gpu_fully_connected(x, w, b, want_kernel="fc_mfma_i8_256x256x128", **kws)
-    assert np.array_equal(got, want)
+    for act in (0, 2):
+        want = oracle.fully_connected(x, w, b, act=act, **kws)
+        got = TC.gpu_fully_connected(x, w, b, act=act, want_kernel=kernel, **kws)
+        assert np.array_equal(got, want), int((got != want).sum())
     assert len(np.unique(want)) > 4
 
 

@@ -361,6 +361,99 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   }
 }
 
+
+// ---- few outputs: 16 x 16 tiles, the reduction split over the workgroup's wavefronts ---------
+// A layer like 64 x 1280 -> 1000 holds four 256 x 256 tiles - four workgroups on a chip of 256
+// CUs. Here a workgroup owns 16 x 16 outputs (v_mfma_i32_16x16x64_i8), its four wavefronts
+// take every fourth 64-byte k-step with operand fragments loaded straight from global memory
+// (eight k-steps in flight per wavefront, every load unconditional: positions past K read the
+// zero source, k-steps past the end re-read the last one and are dropped), the partial sums
+// meet in LDS and the first wavefront requantizes and stores. Same operands, tables and
+// arithmetic as the big kernel.
+constexpr int kSmallBatch = 8;
+
+template <bool X_U8, bool ROWSUM, int RQ>
+__global__ void __launch_bounds__(kThreads) FcSmallKernel(FcArgs a) {
+  __shared__ int red[4][4][64];
+  __shared__ int red_rs[4][64];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int tiles_n = (a.N + 15) / 16;
+  const int tn = blockIdx.x % tiles_n, tm = blockIdx.x / tiles_n;
+  const int n0 = tn * 16, m0 = tm * 16;
+  const int row = lane & 15, kq = lane >> 4;  // fragment row; 16-byte quarter of a 64-byte k-step
+  const int8_t* xrow = a.x + static_cast<size_t>(min(m0 + row, a.M - 1)) * a.K + kq * 16;
+  const int8_t* wrow = a.w + static_cast<size_t>(min(n0 + row, a.N - 1)) * a.K + kq * 16;
+  const int ksteps = (a.K + 63) / 64;
+  v4i acc = {0, 0, 0, 0};
+  int rowsum = 0;
+  for (int ks0 = wave; ks0 < ksteps; ks0 += 4 * kSmallBatch) {
+    v4i fx[kSmallBatch], fw[kSmallBatch];
+#pragma unroll
+    for (int b = 0; b < kSmallBatch; ++b) {
+      const int off = min(ks0 + 4 * b, ksteps - 1) * 64;
+      const bool past = off + kq * 16 >= a.K;  // only in the last k-step, when K is not a multiple of 64
+      // the address is selected, not the value: the load itself stays unconditional
+      const int8_t* px = past ? a.zeros + (X_U8 ? 128 : 0) : xrow + off;
+      const int8_t* pw = past ? a.zeros : wrow + off;
+      fx[b] = *reinterpret_cast<const v4i*>(px);
+      fw[b] = *reinterpret_cast<const v4i*>(pw);
+    }
+#pragma unroll
+    for (int b = 0; b < kSmallBatch; ++b) {
+      if (ks0 + 4 * b < ksteps) {  // uniform over the wavefront
+        if (X_U8) fx[b] ^= static_cast<int>(0x80808080);
+        if (ROWSUM) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) rowsum = __builtin_amdgcn_sdot4(fx[b][q], 0x01010101, rowsum, false);
+        }
+        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(fw[b], fx[b], acc, 0, 0, 0);
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) red[wave][r][lane] = acc[r];
+  if (ROWSUM) red_rs[wave][lane] = rowsum;
+  __syncthreads();
+  if (wave != 0) return;
+  // lane holds activation row m0 + lane % 16 and features n0 + 4 * (lane / 16) + 0..3
+  const int m = m0 + row, n = n0 + 4 * kq;
+  int rs = 0;
+  if (ROWSUM) {
+#pragma unroll
+    for (int w = 0; w < 4; ++w)
+#pragma unroll
+      for (int qq = 0; qq < 4; ++qq) rs += red_rs[w][qq * 16 + row];
+  }
+  int r4[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    int v = red[0][r][lane] + red[1][r][lane] + red[2][r][lane] + red[3][r][lane] + a.biasf[n + r];
+    if (ROWSUM) v -= a.zws * rs;
+    r4[r] = Requant8<RQ>(v, a.rq[n + r], a.out_zp, a.lo, a.hi);  // tables cover the padded feature count
+  }
+  if (m >= a.M || n >= a.N) return;
+  int8_t* dst = a.y + static_cast<size_t>(m) * a.N + n;
+  if ((a.N & 3) == 0) {
+    *reinterpret_cast<uint32_t*>(dst) = PackBytes(r4[0], r4[1], r4[2], r4[3]);
+  } else {
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      if (n + r < a.N) dst[r] = static_cast<int8_t>(r4[r]);
+  }
+}
+
+template <bool X_U8, bool ROWSUM>
+void LaunchSmallRq(int rq, dim3 grid, hipStream_t st, const FcArgs& a) {
+  const dim3 block(kThreads);
+  if (rq == kRqFastNoTie) hipLaunchKernelGGL((FcSmallKernel<X_U8, ROWSUM, kRqFastNoTie>), grid, block, 0, st, a);
+  else if (rq == kRqFast) hipLaunchKernelGGL((FcSmallKernel<X_U8, ROWSUM, kRqFast>), grid, block, 0, st, a);
+  else hipLaunchKernelGGL((FcSmallKernel<X_U8, ROWSUM, kRqGeneric>), grid, block, 0, st, a);
+}
+
+// Few enough outputs that 256 x 256 tiles would leave most of the chip idle.
+bool UseSmallTiles(const tvx_fc_desc& d) { return static_cast<uint64_t>(d.m) * d.n <= (1u << 18); }
+
 template <bool X_U8, bool ROWSUM>
 void LaunchRq(int rq, dim3 grid, hipStream_t st, const FcArgs& a) {
   const dim3 block(kThreads);
@@ -411,6 +504,15 @@ int FcMfmaRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t s
   }
   const bool x_u8 = d.in_dtype == TVX_U8, rowsum = a.zws != 0;
   const int rq = op->geo[1];
+  if (UseSmallTiles(d)) {
+    const dim3 small_grid(((a.M + 15) / 16) * ((a.N + 15) / 16));
+    if (x_u8 && rowsum) LaunchSmallRq<true, true>(rq, small_grid, st, a);
+    else if (x_u8) LaunchSmallRq<true, false>(rq, small_grid, st, a);
+    else if (rowsum) LaunchSmallRq<false, true>(rq, small_grid, st, a);
+    else LaunchSmallRq<false, false>(rq, small_grid, st, a);
+    TVX_HIP_CHECK(hipGetLastError());
+    return TVX_OK;
+  }
   if (x_u8 && rowsum) LaunchRq<true, true>(rq, grid, st, a);
   else if (x_u8) LaunchRq<true, false>(rq, grid, st, a);
   else if (rowsum) LaunchRq<false, true>(rq, grid, st, a);
@@ -495,7 +597,7 @@ int FcMfmaSetup(tvx_op* op, const tvx_fc_desc* d, const void* w_host, const void
   op->geo[0] = zws;
   op->geo[1] = rq;
   op->run = FcMfmaRun;
-  op->kernel_name = "fc_mfma_i8_256x256x128";
+  op->kernel_name = UseSmallTiles(*d) ? "fc_mfma_i8_16x16_splitk" : "fc_mfma_i8_256x256x128";
   return TVX_OK;
 }
 
