@@ -75,7 +75,7 @@ __device__ __forceinline__ int ChannelFill(const ConvArgs& a, int c, int c_real)
 }
 
 template <int OT, int RQ>
-__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) ConvIgemmKernel(ConvArgs a) {
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(OT == 1 ? 4 : 2, OT == 1 ? 4 : 2))) ConvIgemmKernel(ConvArgs a) {
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int tile = blockIdx.x % a.tiles_per_image;
