@@ -416,6 +416,34 @@ AddQuantKernel(EltArgs a, const T* __restrict__ x, const T* __restrict__ z, T* _
   y[idx] = static_cast<T>(r);
 }
 
+// The same arithmetic on 16 elements per thread (whole 16-byte chunks of both operands); the
+// ragged tail of the tensor goes to the one-element kernel above.
+template <typename T>
+__global__ void __launch_bounds__(kBlock)
+AddQuantVecKernel(EltArgs a, const uint4* __restrict__ x, const uint4* __restrict__ z, uint4* __restrict__ y,
+                  uint64_t chunks) {
+  const uint64_t idx = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (idx >= chunks) return;
+  const uint4 xv = x[idx], zv = z[idx];
+  const uint32_t xs[4] = {xv.x, xv.y, xv.z, xv.w}, zs[4] = {zv.x, zv.y, zv.z, zv.w};
+  uint32_t out[4];
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    int r4[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int xa = static_cast<int32_t>(static_cast<T>((xs[d] >> (8 * e)) & 0xff));
+      const int zb = static_cast<int32_t>(static_cast<T>((zs[d] >> (8 * e)) & 0xff));
+      const double tb = __dmul_rn(static_cast<double>(zb - a.b_zp), a.rb);
+      const double t = fma(static_cast<double>(xa - a.a_zp), a.ra, tb);
+      // |t| < 2^29 (8-bit operands, ratios bounded at creation): the 32-bit conversion is exact
+      r4[e] = Med3(static_cast<int>(rint(t)) + a.out_zp, a.lo, a.hi);
+    }
+    out[d] = PackBytes(r4[0], r4[1], r4[2], r4[3]);
+  }
+  y[idx] = make_uint4(out[0], out[1], out[2], out[3]);
+}
+
 template <typename T>
 __global__ void __launch_bounds__(kBlock)
 AddFloatKernel(const T* __restrict__ x, const T* __restrict__ z, T* __restrict__ y, uint64_t total) {
@@ -468,6 +496,28 @@ int ActivationRun(tvx_op* op, const void* in0, const void*, void* out, hipStream
   return TVX_OK;
 }
 
+// 16 elements per thread where all three tensors are 16-byte aligned and the ratios are small
+// enough for the 32-bit rounding conversion; the one-element kernel for the tail and otherwise.
+template <typename T>
+void AddQuantLaunch(const EltArgs& a, const void* in0, const void* in1, void* out, uint64_t total, bool small_ratios,
+                    hipStream_t st) {
+  const T* x = static_cast<const T*>(in0);
+  const T* z = static_cast<const T*>(in1);
+  T* y = static_cast<T*>(out);
+  uint64_t done = 0;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(in0) | reinterpret_cast<uintptr_t>(in1) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+  if (aligned && small_ratios && total >= 16) {
+    const uint64_t chunks = total / 16;
+    hipLaunchKernelGGL((AddQuantVecKernel<T>), dim3(Blocks(chunks)), dim3(kBlock), 0, st, a,
+                       reinterpret_cast<const uint4*>(x), reinterpret_cast<const uint4*>(z),
+                       reinterpret_cast<uint4*>(y), chunks);
+    done = chunks * 16;
+  }
+  if (done < total)
+    hipLaunchKernelGGL((AddQuantKernel<T>), dim3(Blocks(total - done)), dim3(kBlock), 0, st, a, x + done, z + done,
+                       y + done, total - done);
+}
+
 int AddRun(tvx_op* op, const void* in0, const void* in1, void* out, hipStream_t st) {
   const EltArgs a = MakeEltArgs(op);
   const uint64_t total = op->elt.count;
@@ -475,14 +525,10 @@ int AddRun(tvx_op* op, const void* in0, const void* in1, void* out, hipStream_t 
   const dim3 grid(Blocks(total)), block(kBlock);
   switch (op->elt.dtype) {
     case TVX_U8:
-      hipLaunchKernelGGL((AddQuantKernel<uint8_t>), grid, block, 0, st, a,
-                         static_cast<const uint8_t*>(in0), static_cast<const uint8_t*>(in1),
-                         static_cast<uint8_t*>(out), total);
+      AddQuantLaunch<uint8_t>(a, in0, in1, out, total, op->geo[2] != 0, st);
       break;
     case TVX_I8:
-      hipLaunchKernelGGL((AddQuantKernel<int8_t>), grid, block, 0, st, a,
-                         static_cast<const int8_t*>(in0), static_cast<const int8_t*>(in1),
-                         static_cast<int8_t*>(out), total);
+      AddQuantLaunch<int8_t>(a, in0, in1, out, total, op->geo[2] != 0, st);
       break;
     case TVX_F32:
       hipLaunchKernelGGL((AddFloatKernel<float>), grid, block, 0, st,
@@ -615,6 +661,10 @@ int ActivationSetup(tvx_op* op) {
 int AddSetup(tvx_op* op) {
   if (op->quantized)
     ActRange(op->elt.dtype, op->elt.out_scale, op->elt.out_zp, TVX_ACT_NONE, &op->act_lo, &op->act_hi);
+  // the 16-element kernel rounds through a 32-bit conversion: fine while |a ra + b rb| stays far below 2^31
+  const double ra = static_cast<double>(op->elt.a_scale) / static_cast<double>(op->elt.out_scale);
+  const double rb = static_cast<double>(op->elt.b_scale) / static_cast<double>(op->elt.out_scale);
+  op->geo[2] = op->quantized && ra < 1048576.0 && rb < 1048576.0 ? 1 : 0;
   op->run = AddRun;
   op->kernel_name = "add_generic";
   return TVX_OK;
