@@ -135,6 +135,37 @@ def test_lenet_sample_graph(tmp_path, oracle):
 
 
 @pytest.mark.gpu
+def test_repeated_runs_follow_the_inputs(tmp_path, oracle):
+    """Run() may be called again and again with the inputs re-filled in between
+    (src/tim/vx/graph.cc:378-391): six runs with the input alternating between two images,
+    host copies and synchronisations in between as an application would have them; every
+    run must equal the oracle's result for the image it was given."""
+    w, x = _lenet_data()
+    rng = np.random.default_rng(11)
+    other = rng.integers(0, 256, x.size, dtype=np.uint8)
+    g = GRAPHS.lenet_asymu8(w, x)
+    logits = copy.deepcopy(g)
+    logits["test"] = "lenet_logits_replay"
+    logits["ops"] = logits["ops"][:-1]
+    logits["tensors"] = logits["tensors"][:-1]
+    logits["tensors"][15]["attr"] = "OUTPUT"
+    logits["output"] = 15
+    in_id = next(t["id"] for t in logits["tensors"] if t["attr"] == "INPUT")
+    logits["reruns"] = [{in_id: other}, {in_id: x}, {in_id: other}, {in_id: other}, {in_id: x}]
+    want_x = oracle.run_graph(logits)
+    alt = copy.deepcopy(logits)
+    {t["id"]: t for t in alt["tensors"]}[in_id]["data"] = other
+    want_other = oracle.run_graph(alt)
+    assert not np.array_equal(want_x, want_other)
+    expect = [want_x, want_other, want_x, want_other, want_other, want_x]
+    res, info, log = GF.run_graphs([logits], str(tmp_path))
+    runs = [res[0]] + info["lenet_logits_replay"]["reruns"]
+    assert len(runs) == 6 and all(r is not None for r in runs), (info, log[-2000:])
+    for i, (got, want) in enumerate(zip(runs, expect)):
+        assert np.array_equal(got, want), i
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("batch,res", [(2, 224), (3, 96)])
 def test_mobilenet_v2_graph_bit_exact(tmp_path, oracle, batch, res):
     g = GRAPHS.mobilenet_v2(batch=batch, res=res, seed=batch)

@@ -83,6 +83,15 @@ def write_graphs(graphs, txt_path, blob_path, bench=None):
                       a["axis"], "%.9g" % a["beta"], a["sm_axis"], len(a["new_shape"])] + list(a["new_shape"])
                 txt.write(" ".join(str(x) for x in f) + "\n")
             txt.write("run %d\n" % g["output"])
+            # optional re-runs of the compiled graph with other input data: [{tensor id: array}, ...]
+            dtypes = {t["id"]: NP_DTYPE[t["dtype"]] for t in g["tensors"]}
+            for feeds in g.get("reruns", []):
+                for tid, data in feeds.items():
+                    raw = np.ascontiguousarray(np.asarray(data).astype(dtypes[tid], copy=False)).tobytes()
+                    txt.write("feed %d %d %d\n" % (tid, off, len(raw)))
+                    blob.write(raw)
+                    off += len(raw)
+                txt.write("run %d\n" % g["output"])
             if bench:
                 txt.write("bench %d %d\n" % bench)
             txt.write("end\n")
@@ -92,7 +101,9 @@ def run_graphs(graphs, workdir, bench=None, timeout=600, env=None):
     """Returns (outputs, info, log): per graph the flat output array (None where the runtime
     refused the graph, the stage then in info[name]["fail"]); with `bench`, info[name] holds
     the milliseconds per Graph::Run() as "run_ms" (whole call, host copies included) and
-    "device_ms" (the operator sequence alone); log is what the runtime wrote to stderr."""
+    "device_ms" (the operator sequence alone); a graph with "reruns" (a list of {input tensor
+    id: data}) is run again once per entry and info[name]["reruns"] lists those outputs; log is
+    what the runtime wrote to stderr."""
     if not os.path.exists(RUNNER):
         raise RuntimeError("%s is not built: run build.py" % RUNNER)
     os.makedirs(workdir, exist_ok=True)
@@ -121,11 +132,14 @@ def run_graphs(graphs, workdir, bench=None, timeout=600, env=None):
     for g in graphs:
         name = g["test"].replace(" ", "_")
         i = cursor.get(name, 0)
-        cursor[name] = i + 1
-        rec = by_name.get(name, [None] * (i + 1))[i]
-        if rec is None:
-            results.append(None)
-            continue
+        n_runs = 1 + len(g.get("reruns", []))
+        cursor[name] = i + n_runs
+        recs = by_name.get(name, [])[i:i + n_runs]
+        recs += [None] * (n_runs - len(recs))
         t = {t["id"]: t for t in g["tensors"]}[g["output"]]
-        results.append(np.frombuffer(raw[rec[0]:rec[0] + rec[1]], dtype=NP_DTYPE[t["dtype"]]).copy())
+        arrays = [None if r is None else np.frombuffer(raw[r[0]:r[0] + r[1]], dtype=NP_DTYPE[t["dtype"]]).copy()
+                  for r in recs]
+        results.append(arrays[0])
+        if n_runs > 1:
+            info.setdefault(name, {})["reruns"] = arrays[1:]
     return results, info, p.stderr

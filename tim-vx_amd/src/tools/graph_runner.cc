@@ -12,7 +12,8 @@
 //      <kw> <kh> <multiplier> <weights> <pool_type> <round_type> <pool_1d> <axis> <beta> <sm_axis>
 //      <n_shape> <shape..>
 //       id -1 = the graph's placeholder tensor (no bias)
-//   run <tensor id>           compile + run; append the tensor to out.bin
+//   run <tensor id>           compile (first time) + run; append the tensor to out.bin
+//   feed <tensor id> <off> <len>   an INPUT tensor takes these blob bytes from the next run on
 //   bench <warmup> <iters>    time Graph::Run() (after a `run`)
 //   end
 // For every `run` one line goes to stdout: "ok <name> <offset> <bytes>" or
@@ -219,6 +220,18 @@ int main(int argc, char** argv) {
         out_off += result.size();
       }
       std::fflush(stdout);
+    } else if (rec == "feed") {
+      // the input tensor takes other bytes of the blob from the next `run` on
+      int id;
+      size_t off, len;
+      ss >> id >> off >> len;
+      auto it = tensors.find(id);
+      if (it == tensors.end() || !it->second.is_input || off + len > blob.size()) {
+        std::fprintf(stderr, "bad feed record\n");
+        return 2;
+      }
+      it->second.off = off;
+      it->second.len = len;
     } else if (rec == "bench") {
       int warmup, iters;
       ss >> warmup >> iters;
