@@ -231,6 +231,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-extra", action="store_true", help="skip the non-headline workloads")
+    ap.add_argument("--no-networks", action="store_true",
+                    help="skip the LeNet / MobileNetV2 runs (child processes) and the device calibration")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain 256 MiB device copy, 10 times (scales the HBM byte counters)")
     args = ap.parse_args()
@@ -254,10 +256,17 @@ def main():
     wall_ms, kernel_ms = time_workload(wl, args.steps, args.warmup)
     gpu_out = wl["device_out"].cpu().numpy()
     cpu, parity_ok = cpu_baseline(wl, gpu_out)
-    traffic = None
+    # measured HBM bytes per launch (scaled FETCH_SIZE + WRITE_SIZE), kept per kernel and workload
+    tmap = {}
     tpath = os.path.join(REPO, "profiles", "traffic.json")
     if os.path.exists(tpath):
-        traffic = json.load(open(tpath)).get(wl["op"].kernel_name, {}).get("bytes_per_launch")
+        tmap = json.load(open(tpath))
+
+    def traffic_of(w):
+        rec = tmap.get(w["op"].kernel_name, {})
+        return rec.get("bytes_per_launch") if rec.get("workload") == w["name"] else None
+
+    traffic = traffic_of(wl)
     line = {
         "metric": "int8 conv TOPS", "value": round(wl["ops"] / (wall_ms * 1e-3) / 1e12, 3), "unit": "TOPS",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 5),
@@ -278,7 +287,11 @@ def main():
             extra[w2["name"]] = dict(kernel=w2["op"].kernel_name, ms_per_step=round(wall2, 5),
                                      tops=round(w2["ops"] / (wall2 * 1e-3) / 1e12, 2),
                                      gbs=round(w2["algo_bytes"] / (wall2 * 1e-3) / 1e9, 1),
-                                     roofline=dict(roofline(w2, k2), kernel_ms=round(k2, 5)))
+                                     roofline=dict(roofline(w2, k2, traffic_of(w2)), kernel_ms=round(k2, 5)))
+        if args.no_networks:
+            line["extra"] = extra
+            print(json.dumps(line))
+            return
         extra.update(network_extras(max(5, min(args.steps, 30)), 3))
         # what this very device sustains with the simplest kernels: the int8 matrix cores on
         # zeros (nominal clock) and on random bytes (the clock held under load), a streaming copy
