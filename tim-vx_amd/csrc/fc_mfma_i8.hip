@@ -2,14 +2,19 @@
 // Both operands are K-contiguous (an "NT" GEMM), which is exactly the operand
 // shape v_mfma_i32_32x32x32_i8 wants: every lane feeds 16 consecutive K bytes.
 //
-// Tiling: one 256-thread workgroup (4 wavefronts, 2 x 2) owns a TM x TN = 256 x 256
-// output tile and walks K in steps of 128 bytes; each wavefront accumulates a
-// 128 x 128 sub-tile as 4 x 4 MFMA tiles (256 accumulator registers per lane).
-// Operand tiles go global -> LDS by DMA (no registers), double buffered (2 x 64
-// KiB of the CU's 160 KiB); rows are 128 B in LDS and their 16 B chunks are
-// XOR-swizzled with the row number so that the 32 lanes of a fragment read hit
-// 8 different bank groups. Fragments of the next 32-byte k-step are fetched
-// while the 16 MFMAs of the current one run.
+// Tiling: one 256-thread workgroup (4 wavefronts) owns a TM x TN = 256 x 256 output tile
+// and walks K in steps of 128 bytes; wavefront w accumulates all 256 activation rows
+// against features [64 w, 64 w + 64) as 2 x 8 MFMA tiles (256 accumulator registers per
+// lane). The two operands take different roads. Activation tiles go global -> LDS by DMA
+// (no registers), four stages of 32 KiB; rows are 128 B in LDS and their 16 B chunks are
+// XOR-swizzled with the row number so that the 32 lanes of a fragment read hit 8 different
+// bank groups. The constant weights are packed at creation in MFMA-fragment order and go
+// global -> registers, three k-tiles deep, never through LDS: no wavefront needs another
+// one's weight fragments. Both prefetches run three k-tiles ahead, their instructions
+// spread evenly between the MFMAs (one every fourth). Measured on the 8192 x 4096 x 4096
+// layer: the k-loop takes the same time with and without the operand feed (it is bound by
+// the matrix cores, whose clock drops under random data, plus ~10 % for the barrier per
+// k-tile); prologue and epilogue of a tile cost ~9 us next to ~60 us of k-loop.
 //
 // The MFMA "A" operand is the weight fragment and "B" the activation fragment,
 // so a lane ends up with one activation row m and, per accumulator quad, four
@@ -39,8 +44,12 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 constexpr int TM = 256, TN = 256, TK = 128;
 constexpr int kThreads = 256;
-constexpr int kTileBytes = TM * TK;             // 32 KiB per operand tile
-constexpr int kLdsBytes = 4 * kTileBytes;       // X and W, two stages
+constexpr int kTileBytes = TM * TK;             // 32 KiB per activation tile
+constexpr int kStages = 4;                      // activation tiles in LDS (a power of two)
+constexpr int kTabOffset = kStages * kTileBytes;  // behind the stages: the tile's epilogue tables
+constexpr int kLdsBytes = kTabOffset + TN * 4 + TN * 16;  // folded bias (or fp32 bias), requantization records
+// k-tiles of the packed weights: whole rounds of three (the kernel's weight slots)
+__host__ __device__ constexpr int k_tiles_padded(int k_bytes) { return ((k_bytes + TK - 1) / TK + 2) / 3 * 3; }
 constexpr int kOutStride = TN + 16;             // epilogue staging row stride (bytes)
 
 struct FcArgs {
@@ -74,7 +83,6 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
 
   // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous
   // run of tiles so that neighbours in its L2 share operand panels.
@@ -92,212 +100,259 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   const int tm_idx = first_m + in_group % gm, tn_idx = in_group / gm;
   const int m0 = tm_idx * TM, n0 = tn_idx * TN;
 
-  // ---- global -> LDS DMA ------------------------------------------------------
+  // The epilogue's per-feature tables go to LDS now, one feature per thread: fetched in the
+  // epilogue they would cost a chain of dependent round trips per tile.
+  {
+    // (stored and read back through the same types: the tables are plain arrays to the compiler)
+    if constexpr (F16) {
+      reinterpret_cast<float*>(lds + kTabOffset)[tid] = a.biasf32[n0 + tid];
+    } else {
+      reinterpret_cast<int*>(lds + kTabOffset)[tid] = a.biasf[n0 + tid];  // tables are allocated up to the padded feature count
+      reinterpret_cast<tvx_v4i*>(lds + kTabOffset + TN * 4)[tid] = a.rq[n0 + tid];
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the in-flight counts below start from zero
+  }
+  // ---- activations: global -> LDS DMA ---------------------------------------------
   // One wave instruction moves 64 x 16 bytes into 1 KiB of consecutive LDS: 8
-  // rows x 128 bytes of an operand tile. The XOR swizzle of the LDS layout is
+  // rows x 128 bytes of the activation tile. The XOR swizzle of the LDS layout is
   // applied on the source side: lane l fetches chunk (l & 7) ^ (l >> 3) of row
   // l >> 3, a permutation inside one 128-byte line. A wavefront moves rows
-  // [64 w, 64 w + 64) of both operands per k-tile (16 instructions).
+  // [64 w, 64 w + 64) per k-tile (8 instructions).
   const int dma_row = lane >> 3;
-  uint32_t off_x[8], off_w[8];  // byte offsets from the tensor bases (tensors are < 4 GiB)
-  int dma_chunk[2];             // source chunk of this lane for even / odd instructions
+  uint32_t off_x[8];  // byte offsets from the tensor base (tensors are < 4 GiB)
+  int dma_chunk[2];   // source chunk of this lane for even / odd instructions
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const int r = wave * 64 + i * 8 + dma_row;
     // LDS slot (row r, position lane & 7) holds chunk (lane & 7) ^ ((r >> 1) & 7) of the row
     const int chunk = (lane & 7) ^ ((r >> 1) & 7);
     dma_chunk[i & 1] = chunk;
-    const int xm = min(m0 + r, a.M - 1), wr = min(n0 + r, a.N - 1);  // rows past the edge are computed and dropped
+    const int xm = min(m0 + r, a.M - 1);  // rows past the edge are computed and dropped
     off_x[i] = static_cast<uint32_t>(xm) * static_cast<uint32_t>(a.K) + chunk * 16;
-    off_w[i] = static_cast<uint32_t>(wr) * static_cast<uint32_t>(a.K) + chunk * 16;
   }
+  const int k_tiles = (a.K + TK - 1) / TK;
   const bool k_tail = (a.K % TK) != 0;
-  // piece 2 i moves 8 rows of X, piece 2 i + 1 the same rows of W
-  auto dma_piece = [&](int kt, int stage, int piece) {
-    const int i = piece >> 1;
-    int8_t* dst = lds + stage * 2 * kTileBytes + wave * 64 * TK + i * 1024 + ((piece & 1) ? kTileBytes : 0);
+  // piece i of k-tile kt into its stage; tiles past the last one and reduction bytes past K
+  // read the zero source (0x80 before the re-bias of uint8 activations) and meet zero weights
+  auto dma_piece = [&](int kt, int i) {
+    int8_t* dst = lds + (kt & (kStages - 1)) * kTileBytes + wave * 64 * TK + i * 1024;
     const int k0 = kt * TK;
-    const bool past = k_tail && k0 + dma_chunk[i & 1] * 16 >= a.K;  // only in the last k-tile
-    // reduction bytes past K: zero for the weights, the int8-domain zero (0x80 before
-    // the re-bias of uint8 activations) for the activations
-    const int8_t* src = (piece & 1) ? (past ? a.zeros : a.w + (off_w[i] + k0))
-                                    : (past ? a.zeros + (X_U8 ? 128 : 0) : a.x + (off_x[i] + k0));
+    // branch-free: the address is blended from the two candidates with a mask
+    const bool past = (kt >= k_tiles) | (k_tail & (k0 + dma_chunk[i & 1] * 16 >= a.K));
+    const uintptr_t real = reinterpret_cast<uintptr_t>(a.x) + (off_x[i] + static_cast<uint32_t>(k0));
+    const uintptr_t zero = reinterpret_cast<uintptr_t>(a.zeros) + (X_U8 ? 128 : 0);
+    const uintptr_t take_zero = past ? ~uintptr_t{0} : uintptr_t{0};
+    const int8_t* src = reinterpret_cast<const int8_t*>((zero & take_zero) | (real & ~take_zero));
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
                                      (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
   };
-  auto dma_tile = [&](int kt, int stage) {
-#pragma unroll
-    for (int piece = 0; piece < 16; ++piece) dma_piece(kt, stage, piece);
-  };
 
-  acc_t acc[4][4];  // [tn][tm]
+  // ---- weights: global -> registers, in fragment order -------------------------------
+  // The packed weights hold, per 32-feature block and 32-byte k-step, the 64 x 16 bytes of
+  // the MFMA operand in lane order: one fully coalesced 1 KiB load per fragment, no LDS.
+  // Wavefront w owns feature blocks 2 w and 2 w + 1 of the tile's eight and every
+  // activation row, so no fragment is fetched twice. Three k-tiles of fragments are
+  // resident; slot kt % 3 is refilled for k-tile kt + 3 as its k-steps retire.
+  const int8_t* wp[2];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int nb = 0; nb < 2; ++nb)
+    wp[nb] = a.w + (static_cast<size_t>(n0 / 32 + wave * 2 + nb) * (k_tiles_padded(a.K) * 4)) * 1024 + lane * 16;
+  v4i wr[3][8];  // [slot][nb * 4 + k-step]
+#define TVX_W_LOAD(dst, ptr, off) \
+  asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(dst) : "v"(ptr), "n"(off))
+  // fragment (nb, kk) of k-tile kt; k-tiles past the padded count do not exist: re-read the last
+  auto w_piece = [&](int kt, int nb, int kk, v4i& dst, int kt_max) {
+    const int8_t* ptr = wp[nb] + static_cast<size_t>(min(kt, kt_max)) * 4096;
+    if (kk == 0) TVX_W_LOAD(dst, ptr, 0);
+    else if (kk == 1) TVX_W_LOAD(dst, ptr, 1024);
+    else if (kk == 2) TVX_W_LOAD(dst, ptr, 2048);
+    else TVX_W_LOAD(dst, ptr, 3072);
+  };
+#undef TVX_W_LOAD
+
+  acc_t acc[2][8];  // [feature block][activation block]
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-  int rowsum[4] = {0, 0, 0, 0};
+  int rowsum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
 
   const int frag_row = lane & 31;   // row inside a 32-row MFMA tile
   const int frag_half = lane >> 5;  // which 16-byte half of a 32-byte k-step
-  // byte offsets of this lane's fragment rows; the swizzle term depends on kk only
-  const int x_row_off = (wm * 128 + frag_row) * TK, w_row_off = (wn * 128 + frag_row) * TK;
   const int row7 = (frag_row >> 1) & 7;  // fragment tiles start at multiples of 32 rows
 
-  // Fragment fetches are issued as inline assembly and waited for with explicit
-  // s_waitcnt: the compiler's own wait insertion treats fragments carried across
-  // the loop back-edge conservatively (waits for every LDS operation in flight),
-  // which would serialize the fetch of step kk + 1 with the MFMAs of step kk.
+  // Activation fragments are fetched by inline assembly and waited for with explicit
+  // s_waitcnt, like the weight fragments above: the compiler's own wait insertion treats
+  // values carried across the loop back-edge conservatively (it waits for everything in
+  // flight), which would serialize the fetches with the MFMAs.
   const uint32_t lds_base = static_cast<uint32_t>(reinterpret_cast<size_t>(lds));
-  uint32_t frag_x[4], frag_w[4];  // per k-step: LDS address of this lane's first X / W fragment
+  uint32_t frag_x[4];  // per k-step: LDS address of this lane's fragment in activation block 0, stage 0
 #pragma unroll
-  for (int kk = 0; kk < 4; ++kk) {
-    const int sw = (((kk * 2 + frag_half) ^ row7) << 4);
-    frag_x[kk] = lds_base + x_row_off + sw;
-    frag_w[kk] = lds_base + kTileBytes + w_row_off + sw;
-  }
+  for (int kk = 0; kk < 4; ++kk)
+    frag_x[kk] = lds_base + frag_row * TK + (((kk * 2 + frag_half) ^ row7) << 4);
 #define TVX_DS_READ(dst, addr, off) \
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
-  auto load_frags = [&](uint32_t stage_off, int kk, v4i* fx, v4i* fw) {
-    const uint32_t ax = frag_x[kk] + stage_off, aw = frag_w[kk] + stage_off;
+  auto load_frags = [&](int kt, int kk, v4i* fx) {
+    const uint32_t ax = frag_x[kk] + (kt & (kStages - 1)) * kTileBytes;
     TVX_DS_READ(fx[0], ax, 0);
-    TVX_DS_READ(fw[0], aw, 0);
     TVX_DS_READ(fx[1], ax, 32 * TK);
-    TVX_DS_READ(fw[1], aw, 32 * TK);
     TVX_DS_READ(fx[2], ax, 64 * TK);
-    TVX_DS_READ(fw[2], aw, 64 * TK);
     TVX_DS_READ(fx[3], ax, 96 * TK);
-    TVX_DS_READ(fw[3], aw, 96 * TK);
+    TVX_DS_READ(fx[4], ax, 128 * TK);
+    TVX_DS_READ(fx[5], ax, 160 * TK);
+    TVX_DS_READ(fx[6], ax, 192 * TK);
+    TVX_DS_READ(fx[7], ax, 224 * TK);
   };
 #undef TVX_DS_READ
-  auto prep = [&](v4i* fx) {
+  // One k-step: 16 MFMAs with the four memory operations of this k-step's share of the
+  // prefetch spread between them, one every fourth MFMA (issued in a burst they would queue
+  // up in the memory pipeline with the wavefront waiting behind them). The weight registers
+  // of this k-step are refilled (for k-tile kt + 3) only after the MFMAs that read them
+  // were issued.
+  auto k_step = [&](int kt, int kk, v4i* fx, v4i* w_slot, int kt_max) {
     if (X_U8) {
 #pragma unroll
-      for (int t = 0; t < 4; ++t) fx[t] ^= static_cast<int>(0x80808080);
+      for (int t = 0; t < 8; ++t) fx[t] ^= static_cast<int>(0x80808080);
     }
     if (ROWSUM) {
 #pragma unroll
-      for (int t = 0; t < 4; ++t)
+      for (int t = 0; t < 8; ++t)
 #pragma unroll
         for (int q = 0; q < 4; ++q)
           rowsum[t] = __builtin_amdgcn_sdot4(fx[t][q], 0x01010101, rowsum[t], false);
     }
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+#pragma unroll
+      for (int mb = 0; mb < 8; ++mb) {
+        acc[nb][mb] = Mfma(w_slot[nb * 4 + kk], fx[mb], acc[nb][mb]);
+        if (mb == 3) {
+          dma_piece(kt + 3, kk * 2 + nb);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if (mb == 7) {
+          __builtin_amdgcn_sched_barrier(0);
+          w_piece(kt + 3, nb, kk, w_slot[nb * 4 + kk], kt_max);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    }
   };
-  auto mma = [&](v4i* fx, const v4i* fw) {
-    prep(fx);
-#pragma unroll
-    for (int tn = 0; tn < 4; ++tn)
-#pragma unroll
-      for (int tm = 0; tm < 4; ++tm)
-        acc[tn][tm] = Mfma(fw[tn], fx[tm], acc[tn][tm]);
+  // k-tile kt with its weight slot: the fragments of k-step kk + 1 are fetched while step kk
+  // multiplies; the barrier that publishes the next k-tile sits before the last k-step, so
+  // that the first fragments of the next tile are on their way while it runs. Every k-tile
+  // issues 16 memory operations in the same order; "at most 28 in flight" at the barrier
+  // (12 of this k-tile, 16 of the one before) means that everything issued two k-tiles ago
+  // - the activations and weights of k-tile kt + 1 - has landed.
+  const int kt_max = k_tiles_padded(a.K) - 1;
+  v4i fxa[8], fxb[8];
+  auto k_tile = [&](int kt, v4i* w_slot) {
+    load_frags(kt, 1, fxb);
+    asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    k_step(kt, 0, fxa, w_slot, kt_max);
+    __builtin_amdgcn_sched_barrier(0);
+    load_frags(kt, 2, fxa);
+    asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    k_step(kt, 1, fxb, w_slot, kt_max);
+    __builtin_amdgcn_sched_barrier(0);
+    load_frags(kt, 3, fxb);
+    asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    k_step(kt, 2, fxa, w_slot, kt_max);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt vmcnt(28) lgkmcnt(0)" ::: "memory");
+    // the bare barrier: __syncthreads() adds a fence that waits for every memory operation in
+    // flight - the whole prefetch - at every k-tile
+    __builtin_amdgcn_s_barrier();
+    load_frags(kt + 1, 0, fxa);
+    __builtin_amdgcn_sched_barrier(0);
+    k_step(kt, 3, fxb, w_slot, kt_max);
+    __builtin_amdgcn_sched_barrier(0);
   };
-  // the same 16 MFMAs with one DMA instruction of a later tile issued behind each:
-  // a wavefront that issues its DMA back to back sits in the memory pipeline's
-  // issue queue while its matrix core idles
-  auto mma_dma = [&](v4i* fx, const v4i* fw, int dma_kt, int dma_stage) {
-    prep(fx);
+  // prologue: k-tiles 0, 1, 2 in the order every later k-tile uses (8 x (activation piece,
+  // weight fragment)), so that the in-flight counts line up from the first barrier on
 #pragma unroll
-    for (int tn = 0; tn < 4; ++tn)
+  for (int t = 0; t < 3; ++t)
 #pragma unroll
-      for (int tm = 0; tm < 4; ++tm) {
-        acc[tn][tm] = Mfma(fw[tn], fx[tm], acc[tn][tm]);
-        dma_piece(dma_kt, dma_stage, tn * 4 + tm);
+    for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+      for (int nb = 0; nb < 2; ++nb) {
+        dma_piece(t, kk * 2 + nb);
+        __builtin_amdgcn_sched_barrier(0);
+        w_piece(t, nb, kk, wr[t][nb * 4 + kk], kt_max);
         __builtin_amdgcn_sched_barrier(0);
       }
-  };
-
-  // Steady state of one k-tile (four 32-byte k-steps, 16 MFMAs each): the
-  // fragments of step kk + 1 are fetched while step kk multiplies; the barrier
-  // that publishes the next tile's DMA sits before the last step, so that the
-  // first fragments of the next tile are already on their way while it runs, and
-  // the DMA of the tile after next starts as soon as the barrier has freed this stage.
-  const int k_tiles = (a.K + TK - 1) / TK;
-  // The loop body is branch-free: past the last tile it re-fetches the last tile
-  // into the stage nobody reads any more, which keeps the hardware wait counters
-  // exact (a conditional block in the loop makes the compiler wait for everything).
-  const int last_tile = k_tiles - 1;
-  dma_tile(0, 0);
-  dma_tile(min(1, last_tile), 1);
-  asm volatile("s_waitcnt vmcnt(16)" ::: "memory");  // tile 0 landed (16 newer DMAs may be in flight)
-  __syncthreads();
-  v4i fx0[4], fw0[4], fx1[4], fw1[4];
-  load_frags(0, 0, fx0, fw0);
-  for (int kt = 0; kt < k_tiles; ++kt) {
-    const int stage = kt & 1;
-    const uint32_t so = stage * 2 * kTileBytes, so_next = (stage ^ 1) * 2 * kTileBytes;
-    // "wait until at most 8 LDS reads are in flight" = the older fragment set has arrived
-    load_frags(so, 1, fx1, fw1);
-    asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-    mma(fx0, fw0);
-    __builtin_amdgcn_sched_barrier(0);
-    load_frags(so, 2, fx0, fw0);
-    asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-    mma(fx1, fw1);
-    __builtin_amdgcn_sched_barrier(0);
-    load_frags(so, 3, fx1, fw1);
-    asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-    mma(fx0, fw0);
-    __builtin_amdgcn_sched_barrier(0);
-    // all my reads of this stage are done and the next tile's DMA has landed
-    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-    __syncthreads();
-    load_frags(so_next, 0, fx0, fw0);
-    __builtin_amdgcn_sched_barrier(0);
-    mma_dma(fx1, fw1, min(kt + 2, last_tile), stage);
-    __builtin_amdgcn_sched_barrier(0);
+  asm volatile("s_waitcnt vmcnt(32)" ::: "memory");  // k-tile 0 has landed
+  __builtin_amdgcn_s_barrier();
+  load_frags(0, 0, fxa);
+  // the loop runs whole rounds of three k-tiles (the weight slots are named registers); the
+  // packed weights are zero-padded to that count and the activations past K read zeros
+  for (int kt = 0; kt <= kt_max; kt += 3) {
+    k_tile(kt, wr[0]);
+    k_tile(kt + 1, wr[1]);
+    k_tile(kt + 2, wr[2]);
   }
-  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // no DMA may land in the epilogue's staging tile
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // nothing may land in the epilogue's staging tile
+  // The last round's prefetches target registers whose values nobody reads. To the compiler
+  // such registers are free the moment the fetch is "done" (it cannot see that the data is
+  // still on its way) and it would move epilogue arithmetic into them above the wait. Naming
+  // them as operands after the wait keeps them occupied until everything has landed.
+#define TVX_KEEP8(v) \
+  asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]))
+  TVX_KEEP8(wr[0]);
+  TVX_KEEP8(wr[1]);
+  TVX_KEEP8(wr[2]);
+  TVX_KEEP8(fxa);
+  TVX_KEEP8(fxb);
+#undef TVX_KEEP8
   __syncthreads();  // the epilogue reuses the LDS
 
   // ---- epilogue ---------------------------------------------------------------
+  // A lane holds activation row mb * 32 + lane % 32 and, per accumulator quad g, the four
+  // consecutive features 8 g + 4 (lane / 32) + 0..3 of its wavefront's blocks 2 w, 2 w + 1.
   if constexpr (F16) {
-    // ---- epilogue, float16: bias, activation clamp, round; the 256 x 256 x 2-byte tile is
-    // staged in two rounds of 64 columns per wavefront column (64 KiB + padding each)
+    // ---- float16: bias, activation clamp, round; the 256 x 256 x 2-byte tile is staged in
+    // two rounds, round r taking feature block r of every wavefront (128 columns, 64 KiB + padding)
     constexpr int kHalfStride = 128 * 2 + 16;  // bytes per staged row: 128 halves + padding
     int8_t* out_tile = lds;
 #pragma unroll
     for (int round = 0; round < 2; ++round) {
       if (round) __syncthreads();
 #pragma unroll
-      for (int t2 = 0; t2 < 2; ++t2) {
-        const int tn = round * 2 + t2;
+      for (int g = 0; g < 4; ++g) {
+        const int n = n0 + wave * 64 + round * 32 + 8 * g + 4 * frag_half;
+        float b4[4];
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int nw = tn * 32 + 8 * g + 4 * frag_half;  // column inside the wavefront's 128
-          const int n = n0 + wn * 128 + nw;
-          float b4[4];
+        for (int q = 0; q < 4; ++q) b4[q] = reinterpret_cast<const float*>(lds + kTabOffset)[n - n0 + q];
+        const int col = wave * 32 + 8 * g + 4 * frag_half;  // staged column (halves)
 #pragma unroll
-          for (int q = 0; q < 4; ++q) b4[q] = a.biasf32[n + q];
-          const int col = wn * 64 + t2 * 32 + 8 * g + 4 * frag_half;  // staged column (halves)
+        for (int mb = 0; mb < 8; ++mb) {
+          const int ml = mb * 32 + frag_row;
+          _Float16 h[4];
 #pragma unroll
-          for (int tm = 0; tm < 4; ++tm) {
-            const int ml = wm * 128 + tm * 32 + frag_row;
-            _Float16 h[4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              float v = acc[tn][tm][g * 4 + q] + b4[q];
-              v = fminf(fmaxf(v, a.flo), a.fhi);
-              h[q] = static_cast<_Float16>(v);
-            }
-            uint2 pk;
-            __builtin_memcpy(&pk, h, 8);
-            *reinterpret_cast<uint2*>(out_tile + ml * kHalfStride + col * 2) = pk;
+          for (int q = 0; q < 4; ++q) {
+            float v = acc[round][mb][g * 4 + q] + b4[q];
+            v = fminf(fmaxf(v, a.flo), a.fhi);
+            h[q] = static_cast<_Float16>(v);
           }
+          uint2 pk;
+          __builtin_memcpy(&pk, h, 8);
+          *reinterpret_cast<uint2*>(out_tile + ml * kHalfStride + col * 2) = pk;
         }
       }
       __syncthreads();
-      // staged columns [0, 64) belong to wn = 0, [64, 128) to wn = 1; 8 halves per 16-byte chunk
+      // staged columns [32 w, 32 w + 32) are features [64 w + 32 round, + 32) of the tile; 8 halves per chunk
       const bool vec_ok = (a.N & 7) == 0;
       for (int c = tid; c < TM * 16; c += kThreads) {
         const int ml = c >> 4, ch = c & 15;
-        const int wcol = ch >> 3, in_w = (ch & 7) * 8;
-        const int m = m0 + ml, n = n0 + wcol * 128 + round * 64 + in_w;
+        const int wcol = ch >> 2, in_w = (ch & 3) * 8;
+        const int m = m0 + ml, n = n0 + wcol * 64 + round * 32 + in_w;
         if (m >= a.M || n >= a.N) continue;
-        const int8_t* src = out_tile + ml * kHalfStride + (wcol * 64 + in_w) * 2;
+        const int8_t* src = out_tile + ml * kHalfStride + (wcol * 32 + in_w) * 2;
         int8_t* dst = a.y + (static_cast<size_t>(m) * a.N + n) * 2;
         if (vec_ok) {
           *reinterpret_cast<v4i*>(dst) = *reinterpret_cast<const v4i*>(src);
@@ -309,37 +364,33 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
     }
   } else {
     if (ROWSUM) {
-  #pragma unroll
-      for (int t = 0; t < 4; ++t) rowsum[t] += __shfl_xor(rowsum[t], 32);
+#pragma unroll
+      for (int t = 0; t < 8; ++t) rowsum[t] += __shfl_xor(rowsum[t], 32);
     }
     int8_t* out_tile = lds;  // TM rows x kOutStride bytes (the loop's last barrier freed the LDS)
-  #pragma unroll
-    for (int tn = 0; tn < 4; ++tn) {
-  #pragma unroll
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+#pragma unroll
       for (int g = 0; g < 4; ++g) {
-        // accumulator rows 8g + 4*(lane/32) + 0..3 of this MFMA tile = 4 consecutive features
-        const int nl = wn * 128 + tn * 32 + 8 * g + 4 * frag_half;
+        const int nl = wave * 64 + nb * 32 + 8 * g + 4 * frag_half;
         const int n = n0 + nl;
-        // records and folded bias are allocated up to the padded feature count
         int b4[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) b4[q] = reinterpret_cast<const int*>(lds + kTabOffset)[nl + q];
         tvx_v4i q4[4];
-  #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          b4[q] = a.biasf[n + q];
-          q4[q] = a.rq[n + q];
-        }
-  #pragma unroll
-        for (int tm = 0; tm < 4; ++tm) {
-          const int ml = wm * 128 + tm * 32 + frag_row;
-          uint32_t packed = 0;
-  #pragma unroll
+#pragma unroll
+        for (int q = 0; q < 4; ++q) q4[q] = reinterpret_cast<const tvx_v4i*>(lds + kTabOffset + TN * 4)[nl + q];
+#pragma unroll
+        for (int mb = 0; mb < 8; ++mb) {
+          const int ml = mb * 32 + frag_row;
+          int r4[4];
+#pragma unroll
           for (int q = 0; q < 4; ++q) {
-            int v = acc[tn][tm][g * 4 + q] + b4[q];
-            if (ROWSUM) v -= a.zws * rowsum[tm];
-            const int r = Requant8<RQ>(v, q4[q], a.out_zp, a.lo, a.hi);
-            packed |= static_cast<uint32_t>(r & 0xff) << (8 * q);
+            int v = acc[nb][mb][g * 4 + q] + b4[q];
+            if (ROWSUM) v -= a.zws * rowsum[mb];
+            r4[q] = Requant8<RQ>(v, q4[q], a.out_zp, a.lo, a.hi);
           }
-          *reinterpret_cast<uint32_t*>(out_tile + ml * kOutStride + nl) = packed;
+          *reinterpret_cast<uint32_t*>(out_tile + ml * kOutStride + nl) = PackBytes(r4[0], r4[1], r4[2], r4[3]);
         }
       }
     }
@@ -360,7 +411,6 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
     }
   }
 }
-
 
 // ---- few outputs: 16 x 16 tiles, the reduction split over the workgroup's wavefronts ---------
 // A layer like 64 x 1280 -> 1000 holds four 256 x 256 tiles - four workgroups on a chip of 256
@@ -523,6 +573,27 @@ int FcMfmaRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t s
 
 }  // namespace
 
+// Weights [N][k_bytes] (int8 domain or float16 bytes) -> MFMA-fragment order: for every block
+// of 32 features and every 32-byte k-step, 64 lanes x 16 bytes where lane l holds feature
+// 32 b + l % 32, bytes [32 ks + 16 (l / 32), + 16). Features are padded to the tile and the
+// reduction to whole rounds of three k-tiles, with zeros.
+static std::vector<int8_t> PackFragments(const int8_t* w, uint32_t n, uint32_t k_bytes) {
+  const size_t n_blocks = (n + TN - 1) / TN * (TN / 32);
+  const size_t ksteps = static_cast<size_t>(k_tiles_padded(static_cast<int>(k_bytes))) * 4;
+  std::vector<int8_t> out(n_blocks * ksteps * 1024, 0);
+  for (size_t b = 0; b < n_blocks; ++b)
+    for (int r = 0; r < 32; ++r) {
+      const size_t row = b * 32 + r;
+      if (row >= n) break;
+      const int8_t* src = w + row * k_bytes;
+      for (size_t c = 0; c * 16 < k_bytes; ++c) {  // 16-byte chunks of the row (k_bytes % 16 == 0)
+        const size_t ks = c >> 1, half = c & 1;
+        std::memcpy(&out[((b * ksteps + ks) * 64 + half * 32 + r) * 16], src + c * 16, 16);
+      }
+    }
+  return out;
+}
+
 // float16 x float16 -> float16 with constant weights and K a multiple of 8.
 static int FcMfmaSetupF16(tvx_op* op, const tvx_fc_desc* d, const void* w_host, const void* bias_host) {
   if ((d->k & 7) != 0) return TVX_E_UNSUPPORTED;
@@ -532,7 +603,8 @@ static int FcMfmaSetupF16(tvx_op* op, const tvx_fc_desc* d, const void* w_host, 
   const uint32_t n_alloc = (d->n + TN - 1) / TN * TN;
   std::vector<float> bias(n_alloc, 0.0f);
   if (bias_host) std::memcpy(bias.data(), bias_host, sizeof(float) * d->n);
-  int s = op->packed.Upload(w_host, static_cast<size_t>(d->n) * d->k * 2);
+  const std::vector<int8_t> frags = PackFragments(static_cast<const int8_t*>(w_host), d->n, d->k * 2);
+  int s = op->packed.Upload(frags.data(), frags.size());
   if (s == TVX_OK) s = op->aux.Upload(bias.data(), bias.size() * 4);
   std::vector<int8_t> zeros(256, 0);
   if (s == TVX_OK) s = op->aux3.Upload(zeros.data(), zeros.size());
@@ -582,7 +654,14 @@ int FcMfmaSetup(tvx_op* op, const tvx_fc_desc* d, const void* w_host, const void
   const int rq = BuildRequantRecords(op->h_mult, op->h_shift, static_cast<int>(d->n),
                                      static_cast<int>(n_alloc), d->out_zp, &rqt,
                                      AccumulatorBound(d->k, bias_host, d->n));
-  int s = op->packed.Upload(ws.data(), wn);
+  // the tiled kernel reads fragment order, the small-tile kernel plain rows
+  int s;
+  if (UseSmallTiles(*d)) {
+    s = op->packed.Upload(ws.data(), wn);
+  } else {
+    const std::vector<int8_t> frags = PackFragments(ws.data(), d->n, d->k);
+    s = op->packed.Upload(frags.data(), frags.size());
+  }
   if (s == TVX_OK) s = op->aux.Upload(biasf.data(), biasf.size() * 4);
   if (s == TVX_OK) s = op->aux2.Upload(rqt.data(), rqt.size() * 4);
   std::vector<int8_t> zeros(256, 0);
