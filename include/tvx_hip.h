@@ -100,6 +100,12 @@ typedef struct tvx_conv2d_desc {
   float out_scale;
   int32_t out_zp;
   int32_t activation; /* tvx_activation */
+  /* grouped convolution (vx_nn_convolution_params_ext2_t has no such field: the reference
+   * reaches it through its GROUPED_CONV2D operator, src/tim/vx/ops/groupedconv2d.cc): 0 or 1 =
+   * ordinary; g > 1 = output channels [j*out_c/g, (j+1)*out_c/g) read input channels
+   * [j*in_c/g, (j+1)*in_c/g) only and the weights are {k_w, k_h, in_c/g, out_c}. Needs
+   * multiplier == 0 and g dividing in_c and out_c. */
+  int32_t groups;
 } tvx_conv2d_desc;
 
 /* weights_host: WHIcOc image of the constant weights, or NULL when the weights

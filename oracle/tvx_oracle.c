@@ -173,11 +173,14 @@ typedef struct {
   float out_scale;
   int32_t out_zp;
   int32_t act;
+  int32_t groups; /* 0 or 1: ordinary; g > 1: grouped, weights {k_w, k_h, in_c/g, out_c} */
 } tvxo_conv_desc;
 
 /*
- * Conv2d, dense or depthwise (vxConvolutionLayer semantics,
- * vx_khr_nn.h:837-852; depthwise channel map vsi_nn_op_conv2d.c:275-278).
+ * Conv2d, dense, depthwise or grouped (vxConvolutionLayer semantics,
+ * vx_khr_nn.h:837-852; depthwise channel map vsi_nn_op_conv2d.c:275-278; grouped: output
+ * channel block j of out_c/g channels reads input channel block j of in_c/g channels, weights
+ * {k_w, k_h, in_c/g, out_c} - src/tim/vx/ops/groupedconv2d_test.cc:30-294 pins shapes and values).
  *   acc = sum (x - zx)(w - zw) + bias        (int32, wraps)
  *   y   = clamp(requant(acc) + zy)
  * Taps outside the input contribute nothing (padding with the real value 0).
@@ -187,14 +190,15 @@ void tvxo_conv2d(const tvxo_conv_desc* d, const void* x, const void* w,
                  const void* bias, void* y) {
   const int quant = d->in_dtype == TVXO_U8 || d->in_dtype == TVXO_I8;
   const int64_t in_plane = (int64_t)d->in_w * d->in_h, out_plane = (int64_t)d->out_w * d->out_h;
-  const int32_t ic_per_oc = d->multiplier > 0 ? 1 : d->in_c;
+  const int32_t groups = d->groups > 1 ? d->groups : 1;
+  const int32_t ic_per_oc = d->multiplier > 0 ? 1 : d->in_c / groups;
   int32_t lo = 0, hi = 0;
   if (quant) tvxo_act_range(d->out_dtype, d->out_scale, d->out_zp, d->act, &lo, &hi);
   const int64_t total = (int64_t)d->batch * d->out_c;
 #pragma omp parallel for schedule(static)
   for (int64_t job = 0; job < total; ++job) {
     const int32_t n = (int32_t)(job / d->out_c), oc = (int32_t)(job % d->out_c);
-    const int32_t ic0 = d->multiplier > 0 ? oc / d->multiplier : 0;
+    const int32_t ic0 = d->multiplier > 0 ? oc / d->multiplier : (oc / (d->out_c / groups)) * ic_per_oc;
     int32_t mult = 0, shift = 0;
     if (quant) {
       double ws = d->w_scales ? (double)d->w_scales[oc] : (double)d->w_scale;

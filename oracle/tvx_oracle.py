@@ -27,7 +27,7 @@ class ConvDesc(C.Structure):
         "in_dtype", "w_dtype", "out_dtype")] + [
         ("in_scale", C.c_float), ("in_zp", C.c_int32), ("w_scale", C.c_float),
         ("w_zp", C.c_int32), ("w_scales", C.POINTER(C.c_float)),
-        ("out_scale", C.c_float), ("out_zp", C.c_int32), ("act", C.c_int32)]
+        ("out_scale", C.c_float), ("out_zp", C.c_int32), ("act", C.c_int32), ("groups", C.c_int32)]
 
 
 class FcDesc(C.Structure):
@@ -101,9 +101,10 @@ def _q(quant):
 
 def conv2d(x, w, bias, *, in_shape, w_shape, out_shape, stride, dilation, pad_left, pad_top,
            multiplier, in_dtype, w_dtype, out_dtype, in_q=(1.0, 0), w_q=(1.0, 0, None),
-           out_q=(1.0, 0), act=ACT_NONE):
+           out_q=(1.0, 0), act=ACT_NONE, groups=0):
     """Shapes are WHCN / WHIcOc lists (dim 0 fastest); arrays are flat, C-contiguous."""
     d = ConvDesc()
+    d.groups = groups
     d.in_w, d.in_h, d.in_c, d.batch = in_shape
     d.k_w, d.k_h = w_shape[0], w_shape[1]
     d.out_w, d.out_h, d.out_c = out_shape[0], out_shape[1], out_shape[2]
@@ -213,7 +214,7 @@ def run_case(case):
         so, zo, _ = _q(out["quant"])
         return conv2d(arr[0], arr[1], bias, in_shape=x["shape"], w_shape=w["shape"],
                       out_shape=out["shape"], stride=a["stride"], dilation=a["dilation"],
-                      pad_left=a["pad"][0], pad_top=a["pad"][2], multiplier=a["multiplier"],
+                      pad_left=a["pad"][0], pad_top=a["pad"][2], multiplier=a["multiplier"], groups=a.get("groups", 0),
                       in_dtype=DTYPE_CODE[x["dtype"]], w_dtype=DTYPE_CODE[w["dtype"]],
                       out_dtype=DTYPE_CODE[out["dtype"]], in_q=(s, z), w_q=_q(w["quant"]),
                       out_q=(so, zo))
@@ -267,7 +268,7 @@ def run_graph(graph, keep_all=False):
             bias = val[ins[2]["id"]] if len(ins) > 2 and ins[2] is not None else None
             y = conv2d(xv, val[w["id"]], bias, in_shape=x["shape"], w_shape=w["shape"],
                        out_shape=out["shape"], stride=a["stride"], dilation=a["dilation"],
-                       pad_left=a["pad"][0], pad_top=a["pad"][2], multiplier=a["multiplier"],
+                       pad_left=a["pad"][0], pad_top=a["pad"][2], multiplier=a["multiplier"], groups=a.get("groups", 0),
                        in_dtype=DTYPE_CODE[x["dtype"]], w_dtype=DTYPE_CODE[w["dtype"]],
                        out_dtype=DTYPE_CODE[out["dtype"]], in_q=(s, z), w_q=_q(w["quant"]),
                        out_q=(so, zo))

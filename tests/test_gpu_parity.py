@@ -16,15 +16,17 @@ def rand_q(rng, shape, dtype):
     return rng.integers(-128, 128, shape).astype(np.int8)
 
 
-def conv_case(rng, *, n, c, h, w, oc, kh, kw, stride, dil, pad, mult, mode):
+def conv_case(rng, *, n, c, h, w, oc, kh, kw, stride, dil, pad, mult, mode, groups=0):
     """mode: 'u8' (per-tensor), 'i8pc' (int8 per-channel), 'u8pc' (u8 act, i8 pc weights), 'f32', 'f16'."""
-    icg = 1 if mult > 0 else c
+    icg = 1 if mult > 0 else c // max(groups, 1)
     if mult > 0:
         oc = c * mult
     out_w = (w + pad[0] + pad[1] - ((kw - 1) * dil[0] + 1)) // stride[0] + 1
     out_h = (h + pad[2] + pad[3] - ((kh - 1) * dil[1] + 1)) // stride[1] + 1
     kws = dict(in_shape=[w, h, c, n], w_shape=[kw, kh, icg, oc], out_shape=[out_w, out_h, oc, n],
                stride=stride, dilation=dil, pad_left=pad[0], pad_top=pad[2], multiplier=mult)
+    if groups:
+        kws["groups"] = groups
     if mode in ("f32", "f16"):
         npd = np.float32 if mode == "f32" else np.float16
         dt = 3 if mode == "f32" else 2
@@ -370,6 +372,40 @@ def test_depthwise3x3_shapes(oracle, gi, mode):
         got = TC.gpu_conv2d(x, wt, b, act=act, want_kernel="dwconv3x3_i8" if fast else "dwconv_planes_i8", **kws)
         assert np.array_equal(got, want)
     assert len(np.unique(want)) > 4
+
+
+GROUPED_GRID = [
+    # (n, c, oc, groups, h, w, k, stride, pad): the reference's shapes (groupedconv2d_test.cc) scaled up;
+    # groups == c is a depthwise convolution in disguise and must reach the depthwise kernels
+    (2, 6, 4, 2, 9, 9, 3, [1, 1], [0, 0, 0, 0], "conv2d_generic"),
+    (1, 12, 9, 3, 7, 10, 3, [2, 1], [1, 1, 1, 1], "conv2d_generic"),
+    (3, 8, 8, 4, 6, 6, 1, [1, 1], [0, 0, 0, 0], "conv2d_generic"),
+    (2, 16, 16, 16, 12, 12, 3, [1, 1], [1, 1, 1, 1], None),
+    (2, 6, 12, 6, 8, 8, 2, [2, 2], [0, 1, 0, 1], None),
+    (1, 5, 7, 1, 6, 6, 3, [1, 1], [1, 1, 1, 1], None),
+]
+
+
+@pytest.mark.parametrize("mode", ["u8", "i8pc", "u8pc", "f32", "f16"])
+@pytest.mark.parametrize("gi", range(len(GROUPED_GRID)))
+def test_grouped_conv2d(oracle, gi, mode):
+    n, c, oc, groups, h, w, k, stride, pad, kernel = GROUPED_GRID[gi]
+    rng = np.random.default_rng(7000 + gi)
+    x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=oc, kh=k, kw=k, stride=stride, dil=[1, 1],
+                              pad=pad, mult=0, mode=mode, groups=groups)
+    want = oracle.conv2d(x, wt, b, **kws)
+    quant = mode not in ("f32", "f16")
+    got = TC.gpu_conv2d(x, wt, b, want_kernel=kernel if quant else None, **kws)
+    if quant:
+        assert np.array_equal(got, want), int((got != want).sum())
+        assert len(np.unique(want)) > 4
+    else:
+        assert np.allclose(got.astype(np.float32), want.astype(np.float32), rtol=FLOAT_RTOL, atol=2e-2)
+    if groups == c and quant and oc == c and k == 3:
+        # the same numbers as the depthwise spelling of the operator
+        dw = dict(kws, multiplier=1)
+        dw.pop("groups")
+        assert np.array_equal(TC.gpu_conv2d(x, wt, b, **dw), got)
 
 
 DWP_GRID = [

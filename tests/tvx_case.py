@@ -10,7 +10,7 @@ import numpy as np
 import tvx_oracle as O
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-GOLDEN_FILES = ["conv2d", "depthwise_conv", "fullyconnected", "max_pool", "avg_pool"]
+GOLDEN_FILES = ["conv2d", "depthwise_conv", "grouped_conv2d", "fullyconnected", "max_pool", "avg_pool"]
 
 
 def load_cases(name):
@@ -72,9 +72,10 @@ def _wq(desc, w_q, keep):
 
 def gpu_conv2d(x, w, bias, *, in_shape, w_shape, out_shape, stride, dilation, pad_left, pad_top,
                multiplier, in_dtype, w_dtype, out_dtype, in_q=(1.0, 0), w_q=(1.0, 0, None),
-               out_q=(1.0, 0), act=0, const_weights=True, want_kernel=None):
+               out_q=(1.0, 0), act=0, const_weights=True, want_kernel=None, groups=0):
     T = tvx()
     d = T.Conv2dDesc()
+    d.groups = groups
     d.in_w, d.in_h, d.in_c, d.batch = in_shape
     d.k_w, d.k_h = w_shape[0], w_shape[1]
     d.out_w, d.out_h, d.out_c = out_shape[0], out_shape[1], out_shape[2]
@@ -213,7 +214,7 @@ def run_case_gpu(case):
         return gpu_conv2d(arr[0], arr[1], arr[2] if len(ins) > 2 else None, in_shape=x["shape"],
                           w_shape=w["shape"], out_shape=out["shape"], stride=a["stride"],
                           dilation=a["dilation"], pad_left=a["pad"][0], pad_top=a["pad"][2],
-                          multiplier=a["multiplier"], in_dtype=code[x["dtype"]],
+                          multiplier=a["multiplier"], groups=a.get("groups", 0), in_dtype=code[x["dtype"]],
                           w_dtype=code[w["dtype"]], out_dtype=code[out["dtype"]], in_q=(s, z),
                           w_q=O._q(w["quant"]), out_q=(so, zo),
                           const_weights=(w["attr"] == "CONSTANT"))

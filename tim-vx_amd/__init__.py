@@ -26,7 +26,7 @@ class Conv2dDesc(C.Structure):
         ("multiplier", C.c_int32), ("in_dtype", C.c_int32), ("w_dtype", C.c_int32),
         ("out_dtype", C.c_int32), ("in_scale", C.c_float), ("in_zp", C.c_int32),
         ("w_scale", C.c_float), ("w_zp", C.c_int32), ("w_scales", C.POINTER(C.c_float)),
-        ("out_scale", C.c_float), ("out_zp", C.c_int32), ("activation", C.c_int32)]
+        ("out_scale", C.c_float), ("out_zp", C.c_int32), ("activation", C.c_int32), ("groups", C.c_int32)]
 
 
 class FcDesc(C.Structure):

@@ -401,7 +401,7 @@ hipError_t AllowLds(int bytes) {
 // Claims dense quantized convolutions with constant weights whose weight block
 // and halo tile fit the CU's LDS.
 int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const void* bias_host) {
-  if (!op->quantized || !w_host || d->multiplier != 0) return TVX_E_UNSUPPORTED;
+  if (!op->quantized || !w_host || d->multiplier != 0 || d->groups > 1) return TVX_E_UNSUPPORTED;
   ConvArgs a{};
   a.C = d->in_c; a.H = d->in_h; a.W = d->in_w; a.OC = d->out_c; a.OH = d->out_h; a.OW = d->out_w;
   a.kh = d->k_h; a.kw = d->k_w; a.sh = d->stride_h; a.sw = d->stride_w;

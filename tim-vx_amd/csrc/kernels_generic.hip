@@ -33,7 +33,20 @@ struct ConvArgs {
   int in_w, in_h, in_c, batch, k_w, k_h, out_w, out_h, out_c;
   int stride_w, stride_h, dil_w, dil_h, pad_left, pad_top, multiplier;
   int in_zp, w_zp, out_zp, lo, hi, act;
+  int groups;  // >= 1
 };
+
+// Input channels one output channel reads, and the first of them: all of them (dense), one
+// (depthwise, oc = ic * multiplier + j) or the channels of its group.
+__device__ __forceinline__ void ChannelRange(const ConvArgs& a, int oc, int* ic_per_oc, int* ic0) {
+  if (a.multiplier > 0) {
+    *ic_per_oc = 1;
+    *ic0 = oc / a.multiplier;
+  } else {
+    *ic_per_oc = a.in_c / a.groups;
+    *ic0 = (oc / (a.out_c / a.groups)) * *ic_per_oc;
+  }
+}
 
 template <typename XT, typename WT>
 __global__ void __launch_bounds__(kBlock)
@@ -46,8 +59,8 @@ ConvQuantKernel(ConvArgs a, const XT* __restrict__ x, const WT* __restrict__ w,
   const int oh = (idx / a.out_w) % a.out_h;
   const int oc = (idx / (static_cast<uint64_t>(a.out_w) * a.out_h)) % a.out_c;
   const int n = idx / (static_cast<uint64_t>(a.out_w) * a.out_h * a.out_c);
-  const int ic_per_oc = a.multiplier > 0 ? 1 : a.in_c;
-  const int ic0 = a.multiplier > 0 ? oc / a.multiplier : 0;
+  int ic_per_oc, ic0;
+  ChannelRange(a, oc, &ic_per_oc, &ic0);
   int32_t acc = 0;
   for (int ci = 0; ci < ic_per_oc; ++ci) {
     const XT* xp = x + (static_cast<uint64_t>(n) * a.in_c + ic0 + ci) * a.in_h * a.in_w;
@@ -77,8 +90,8 @@ ConvFloatKernel(ConvArgs a, const T* __restrict__ x, const T* __restrict__ w,
   const int oh = (idx / a.out_w) % a.out_h;
   const int oc = (idx / (static_cast<uint64_t>(a.out_w) * a.out_h)) % a.out_c;
   const int n = idx / (static_cast<uint64_t>(a.out_w) * a.out_h * a.out_c);
-  const int ic_per_oc = a.multiplier > 0 ? 1 : a.in_c;
-  const int ic0 = a.multiplier > 0 ? oc / a.multiplier : 0;
+  int ic_per_oc, ic0;
+  ChannelRange(a, oc, &ic_per_oc, &ic0);
   float acc = 0.f;
   for (int ci = 0; ci < ic_per_oc; ++ci) {
     const T* xp = x + (static_cast<uint64_t>(n) * a.in_c + ic0 + ci) * a.in_h * a.in_w;
@@ -105,7 +118,7 @@ int ConvGenericRun(tvx_op* op, const void* in0, const void* in1, void* out, hipS
              static_cast<int>(d.stride_w), static_cast<int>(d.stride_h),
              static_cast<int>(d.dilation_w), static_cast<int>(d.dilation_h),
              static_cast<int>(d.pad_left), static_cast<int>(d.pad_top), d.multiplier,
-             d.in_zp, op->w_zp, d.out_zp, op->act_lo, op->act_hi, d.activation};
+             d.in_zp, op->w_zp, d.out_zp, op->act_lo, op->act_hi, d.activation, d.groups > 1 ? d.groups : 1};
   const void* w = op->has_const_weights ? op->weights.ptr : in1;
   const uint64_t total = static_cast<uint64_t>(d.out_w) * d.out_h * d.out_c * d.batch;
   const dim3 grid(Blocks(total)), block(kBlock);
@@ -609,7 +622,7 @@ int UploadWeightsAndBias(tvx_op* op, const void* w, size_t w_bytes, const void* 
 }  // namespace
 
 int ConvGenericSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w, const void* b) {
-  const uint64_t ic_per_oc = d->multiplier > 0 ? 1 : d->in_c;
+  const uint64_t ic_per_oc = d->multiplier > 0 ? 1 : d->in_c / (d->groups > 1 ? d->groups : 1);
   const size_t w_bytes = static_cast<size_t>(d->k_w) * d->k_h * ic_per_oc * d->out_c * DtypeBytes(d->w_dtype);
   int s = UploadWeightsAndBias(op, w, w_bytes, b, static_cast<size_t>(d->out_c) * 4);
   if (s != TVX_OK) return s;

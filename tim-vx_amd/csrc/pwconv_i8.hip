@@ -383,7 +383,7 @@ int RoundUp(int v, int m) { return (v + m - 1) / m * m; }
 // Claims dense quantized 1x1 convolutions with unit stride, no padding and constant
 // weights whose 128-pixel input tile fits the CU's LDS.
 int PwConvSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const void* bias_host) {
-  if (!op->quantized || !w_host || d->multiplier != 0) return TVX_E_UNSUPPORTED;
+  if (!op->quantized || !w_host || d->multiplier != 0 || d->groups > 1) return TVX_E_UNSUPPORTED;
   if (d->k_w != 1 || d->k_h != 1 || d->stride_w != 1 || d->stride_h != 1 || d->pad_left != 0 ||
       d->pad_top != 0 || d->out_w != d->in_w || d->out_h != d->in_h)
     return TVX_E_UNSUPPORTED;

@@ -270,6 +270,9 @@ int tvx_conv2d_create(const tvx_conv2d_desc* d, const void* weights_host,
       !d->out_h || !d->out_c || !d->stride_w || !d->stride_h || !d->dilation_w || !d->dilation_h)
     return SetError(TVX_E_INVALID, "tvx_conv2d_create: zero extent, stride or dilation");
   if (d->multiplier < 0) return SetError(TVX_E_INVALID, "tvx_conv2d_create: negative multiplier");
+  if (d->groups < 0 || (d->groups > 1 && (d->multiplier != 0 || d->in_c % d->groups || d->out_c % d->groups)))
+    return SetError(TVX_E_INVALID, "tvx_conv2d_create: %d groups do not divide in_c %u / out_c %u (or multiplier set)",
+                    d->groups, d->in_c, d->out_c);
   if (d->multiplier > 0 && d->out_c != d->in_c * static_cast<uint32_t>(d->multiplier))
     return SetError(TVX_E_INVALID, "tvx_conv2d_create: depthwise out_c %u != in_c %u * multiplier %d",
                     d->out_c, d->in_c, d->multiplier);
@@ -285,7 +288,16 @@ int tvx_conv2d_create(const tvx_conv2d_desc* d, const void* weights_host,
   if (!op) return SetError(TVX_E_NOMEM, "tvx_conv2d_create: host allocation failed");
   op->kind = OP_CONV2D;
   op->conv = *d;
-  op->conv.w_scales = nullptr;  // host pointer is not kept
+  // one input channel per group is a depthwise convolution in other words: same weight image
+  // ({k_w, k_h, 1, out_c} = {k_w, k_h, in_c * m, 1}), same channel map (oc / m), and the
+  // depthwise kernels apply
+  if (d->groups > 1 && static_cast<uint32_t>(d->groups) == d->in_c) {
+    op->conv.multiplier = static_cast<int32_t>(d->out_c / d->in_c);
+    op->conv.groups = 0;
+  }
+  const tvx_conv2d_desc norm = op->conv;
+  d = &norm;
+  op->conv.w_scales = nullptr;  // host pointer is not kept (`norm` still has it for the setup functions)
   op->quantized = IsQuant(d->in_dtype);
   op->has_const_weights = weights_host != nullptr;
   op->w_zp = d->w_scales ? 0 : d->w_zp;

@@ -60,6 +60,38 @@ class Conv2d : public BuiltinOp {
                            int32_t input_idx) override;
 };
 
+// Grouped 2-D convolution: output channel block j (Oc / groups channels) reads input
+// channel block j (Ic / groups channels); weight {Kw, Kh, Ic / groups, Oc}, optional bias {Oc}.
+// reference: include/tim/vx/ops/groupedconv2d.h:56-82, src/tim/vx/ops/groupedconv2d.cc
+class GroupedConv2d : public BuiltinOp {
+ public:
+  GroupedConv2d(Graph* graph, PadType padding, const std::array<uint32_t, 2>& strides,
+                const std::array<uint32_t, 2>& dilation, int32_t grouped_number,
+                DataLayout input_layout = DataLayout::WHCN,
+                DataLayout kernel_layout = DataLayout::WHIcOc);
+  GroupedConv2d(Graph* graph, const std::array<uint32_t, 4>& pad,
+                const std::array<uint32_t, 2>& strides,
+                const std::array<uint32_t, 2>& dilation, int32_t group_number,
+                DataLayout input_layout = DataLayout::WHCN,
+                DataLayout kernel_layout = DataLayout::WHIcOc);
+
+  DataLayout KernelDataLayout() { return kernel_layout_; }
+  std::shared_ptr<Operation> Clone(
+      std::shared_ptr<Graph>& graph) const override;
+
+ protected:
+  const PadType padding_;
+  const std::array<uint32_t, 2> strides_;
+  const std::array<uint32_t, 2> dilation_;
+  const std::array<uint32_t, 4> pad_;
+  const int32_t group_number_;
+  const DataLayout kernel_layout_;
+
+ private:
+  void OnBindInputPostProc(const std::shared_ptr<Tensor>& tensor,
+                           int32_t input_idx) override;
+};
+
 // out[n, m] = sum_k in[k, m] * w[k, n] + bias[n]; input dims 0..axis flatten
 // into k. reference: include/tim/vx/ops/fullyconnected.h:42-56
 class FullyConnected : public BuiltinOp {

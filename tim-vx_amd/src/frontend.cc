@@ -733,6 +733,55 @@ void Conv2d::OnBindInputPostProc(const std::shared_ptr<Tensor>& tensor, int32_t)
   PromoteHalfBias(this, impl_.get(), tensor);
 }
 
+// ---- GroupedConv2d ----------------------------------------------------------
+// The same operator kind as Conv2d with a group count (the reference has a kind of its own,
+// VSI_NN_OP_GROUPED_CONV2D, whose setup splits into per-group convolutions:
+// src/tim/vx/internal/src/ops/vsi_nn_op_grouped_conv2d.c).
+GroupedConv2d::GroupedConv2d(Graph* graph, PadType padding,
+                             const std::array<uint32_t, 2>& strides,
+                             const std::array<uint32_t, 2>& dilation, int32_t grouped_number,
+                             DataLayout input_layout, DataLayout kernel_layout)
+    : BuiltinOp(graph, K(OpKind::CONV2D), 0, 0, input_layout),
+      padding_(padding), strides_(strides), dilation_(dilation), pad_({0, 0, 0, 0}),
+      group_number_(grouped_number), kernel_layout_(kernel_layout) {
+  OpAttrs& a = impl_->attrs_;
+  a.pad_type = padding_ == PadType::NONE ? PadType::AUTO : padding_;
+  for (int i = 0; i < 2; ++i) {
+    a.stride[i] = strides_[i];
+    a.dilation[i] = dilation_[i];
+  }
+  a.groups = group_number_;
+}
+
+GroupedConv2d::GroupedConv2d(Graph* graph, const std::array<uint32_t, 4>& pad,
+                             const std::array<uint32_t, 2>& strides,
+                             const std::array<uint32_t, 2>& dilation, int32_t group_number,
+                             DataLayout input_layout, DataLayout kernel_layout)
+    : BuiltinOp(graph, K(OpKind::CONV2D), 0, 0, input_layout),
+      padding_(PadType::AUTO), strides_(strides), dilation_(dilation), pad_(pad),
+      group_number_(group_number), kernel_layout_(kernel_layout) {
+  OpAttrs& a = impl_->attrs_;
+  a.pad_type = PadType::AUTO;
+  for (int i = 0; i < 4; ++i) a.pad[i] = pad_[i];
+  for (int i = 0; i < 2; ++i) {
+    a.stride[i] = strides_[i];
+    a.dilation[i] = dilation_[i];
+  }
+  a.groups = group_number_;
+}
+
+std::shared_ptr<Operation> GroupedConv2d::Clone(std::shared_ptr<Graph>& graph) const {
+  if (padding_ != PadType::AUTO)
+    return graph->CreateOperation<GroupedConv2d>(padding_, strides_, dilation_, group_number_,
+                                                 impl_->layout_, kernel_layout_);
+  return graph->CreateOperation<GroupedConv2d>(pad_, strides_, dilation_, group_number_,
+                                               impl_->layout_, kernel_layout_);
+}
+
+void GroupedConv2d::OnBindInputPostProc(const std::shared_ptr<Tensor>& tensor, int32_t) {
+  PromoteHalfBias(this, impl_.get(), tensor);
+}
+
 // ---- FullyConnected -------------------------------------------------------
 FullyConnected::FullyConnected(Graph* graph, uint32_t axis)
     : FullyConnected(graph, axis, 0) {}

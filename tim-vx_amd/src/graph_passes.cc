@@ -172,6 +172,14 @@ bool SetupConv(OpImpl* op) {
       VSILOGE("depthwise weight must be {Kw, Kh, Ic*multiplier, 1}");
       return false;
     }
+  } else if (a.groups > 1) {
+    const uint32_t g = static_cast<uint32_t>(a.groups);
+    oc = ws[3];
+    if (xs[2] % g != 0 || oc % g != 0 || ws[2] != xs[2] / g) {
+      VSILOGE("GROUPED_CONV2D: %u groups need input C %u and weight Oc %u divisible and weight Ic %u == C / groups",
+              g, xs[2], oc, ws[2]);
+      return false;
+    }
   } else {
     oc = ws[3];
     if (ws[2] != xs[2]) {

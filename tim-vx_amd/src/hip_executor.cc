@@ -231,6 +231,7 @@ class HipExecutor : public Executor {
     d.dilation_w = a.dilation[0]; d.dilation_h = a.dilation[1];
     d.pad_left = a.pad[0]; d.pad_top = a.pad[2];
     d.multiplier = a.multiplier;
+    d.groups = a.groups;
     d.in_dtype = DtypeCode(x->spec_.datatype_);
     d.w_dtype = DtypeCode(w->spec_.datatype_);
     d.out_dtype = DtypeCode(out->spec_.datatype_);

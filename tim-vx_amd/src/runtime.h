@@ -46,6 +46,7 @@ struct OpAttrs {
   uint32_t dilation[2] = {1, 1};
   uint32_t ksize[2] = {0, 0};
   int32_t multiplier = 0;
+  int32_t groups = 0;  // GroupedConv2d: > 1
   uint32_t weights = 0;
   // pool
   PoolType pool_type = PoolType::MAX;
