@@ -99,6 +99,16 @@ def _q(quant):
     return 1.0, 0, None
 
 
+def _conv_shapes(a, x_shape, w_shape, out_shape):
+    """(in, weight, out) shapes in the 2-D operator's terms; Conv1d tensors {W, C, N} / {Kw, Ic, Oc}
+    are rows of height one."""
+    if a.get("conv_1d"):
+        return ([x_shape[0], 1, x_shape[1], x_shape[2]], [w_shape[0], 1, w_shape[1], w_shape[2]],
+                [out_shape[0], 1, out_shape[1], out_shape[2]])
+    return x_shape, w_shape, out_shape
+
+
+
 def conv2d(x, w, bias, *, in_shape, w_shape, out_shape, stride, dilation, pad_left, pad_top,
            multiplier, in_dtype, w_dtype, out_dtype, in_q=(1.0, 0), w_q=(1.0, 0, None),
            out_q=(1.0, 0), act=ACT_NONE, groups=0):
@@ -212,8 +222,9 @@ def run_case(case):
         bias = arr[2] if len(ins) > 2 else None
         s, z, _ = _q(x["quant"])
         so, zo, _ = _q(out["quant"])
-        return conv2d(arr[0], arr[1], bias, in_shape=x["shape"], w_shape=w["shape"],
-                      out_shape=out["shape"], stride=a["stride"], dilation=a["dilation"],
+        xs, wsh, osh = _conv_shapes(a, x["shape"], w["shape"], out["shape"])
+        return conv2d(arr[0], arr[1], bias, in_shape=xs, w_shape=wsh,
+                      out_shape=osh, stride=a["stride"], dilation=a["dilation"],
                       pad_left=a["pad"][0], pad_top=a["pad"][2], multiplier=a["multiplier"], groups=a.get("groups", 0),
                       in_dtype=DTYPE_CODE[x["dtype"]], w_dtype=DTYPE_CODE[w["dtype"]],
                       out_dtype=DTYPE_CODE[out["dtype"]], in_q=(s, z), w_q=_q(w["quant"]),
@@ -266,8 +277,9 @@ def run_graph(graph, keep_all=False):
         if k == "CONV2D":
             w = ins[1]
             bias = val[ins[2]["id"]] if len(ins) > 2 and ins[2] is not None else None
-            y = conv2d(xv, val[w["id"]], bias, in_shape=x["shape"], w_shape=w["shape"],
-                       out_shape=out["shape"], stride=a["stride"], dilation=a["dilation"],
+            xs, wsh, osh = _conv_shapes(a, x["shape"], w["shape"], out["shape"])
+            y = conv2d(xv, val[w["id"]], bias, in_shape=xs, w_shape=wsh,
+                       out_shape=osh, stride=a["stride"], dilation=a["dilation"],
                        pad_left=a["pad"][0], pad_top=a["pad"][2], multiplier=a["multiplier"], groups=a.get("groups", 0),
                        in_dtype=DTYPE_CODE[x["dtype"]], w_dtype=DTYPE_CODE[w["dtype"]],
                        out_dtype=DTYPE_CODE[out["dtype"]], in_q=(s, z), w_q=_q(w["quant"]),

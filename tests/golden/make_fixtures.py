@@ -25,6 +25,7 @@ SOURCES = {
     "conv2d": "src/tim/vx/ops/conv2d_test.cc",
     "depthwise_conv": "src/tim/vx/ops/depthwiseConv_test.cc",
     "grouped_conv2d": "src/tim/vx/ops/groupedconv2d_test.cc",
+    "conv1d": "src/tim/vx/ops/conv1d_test.cc",
     "fullyconnected": "src/tim/vx/ops/fullyconnected_test.cc",
     "max_pool": "src/tim/vx/ops/max_pool_test.cc",
     "avg_pool": "src/tim/vx/ops/avg_pool_test.cc",

@@ -9,15 +9,15 @@ CASES = TC.all_cases()
 
 
 def test_fixture_inventory():
-    # 24 conv2d tests (one of them loops over 66 input sizes), 16 depthwise, 3 grouped,
+    # 24 conv2d tests (one of them loops over 66 input sizes), 16 depthwise, 3 grouped, 3 one-dimensional,
     # 2 fully-connected, 3 max-pool, 8 avg-pool; the two int16 dynamic-fixed-point
     # conv tests of the reference are outside this path and not recorded.
     per_file = {}
     for n, c in CASES:
         per_file.setdefault(n, set()).add(c["test"])
     assert {k: len(v) for k, v in per_file.items()} == {
-        "conv2d": 24, "depthwise_conv": 16, "grouped_conv2d": 3, "fullyconnected": 2, "max_pool": 3, "avg_pool": 8}
-    assert len(CASES) == 121
+        "conv2d": 24, "depthwise_conv": 16, "grouped_conv2d": 3, "conv1d": 3, "fullyconnected": 2, "max_pool": 3, "avg_pool": 8}
+    assert len(CASES) == 124
 
 
 @pytest.mark.parametrize("item", CASES, ids=TC.case_id)
@@ -37,7 +37,8 @@ def test_declared_shapes_equal_inferred(oracle):
         t = {t["id"]: t for t in case["tensors"]}
         x, w, y = t[op["inputs"][0]], t[op["inputs"][1]], t[op["outputs"][0]]
         a = op["attrs"]
+        xs, ws, ys = oracle._conv_shapes(a, x["shape"], w["shape"], y["shape"])  # Conv1d: rows of height one
         for ax in (0, 1):
-            ke = (w["shape"][ax] - 1) * a["dilation"][ax] + 1
-            inferred = (x["shape"][ax] + a["pad"][2 * ax] + a["pad"][2 * ax + 1] - ke) // a["stride"][ax] + 1
-            assert y["shape"][ax] <= inferred
+            ke = (ws[ax] - 1) * a["dilation"][ax] + 1
+            inferred = (xs[ax] + a["pad"][2 * ax] + a["pad"][2 * ax + 1] - ke) // a["stride"][ax] + 1
+            assert ys[ax] <= inferred

@@ -60,6 +60,42 @@ class Conv2d : public BuiltinOp {
                            int32_t input_idx) override;
 };
 
+// 1-D convolution: activation {W, C, N}, weight {Kw, Ic, Oc} (depthwise: {Kw, 1, Ic*multiplier}),
+// optional bias {Oc}, output {W', Oc, N} - the 2-D operator on rows of height one.
+// reference: include/tim/vx/ops/conv1d.h:35-70, src/tim/vx/ops/conv1d.cc:34-84
+class Conv1d : public BuiltinOp {
+ public:
+  Conv1d(Graph* graph, PadType padding, uint32_t stride, uint32_t dilation, int32_t multiplier = 0,
+         DataLayout input_layout = DataLayout::WCN, DataLayout kernel_layout = DataLayout::WIcOc);
+  Conv1d(Graph* graph, const std::array<uint32_t, 2>& pad, uint32_t stride, uint32_t dilation,
+         int32_t multiplier = 0, DataLayout input_layout = DataLayout::WCN,
+         DataLayout kernel_layout = DataLayout::WIcOc);
+  Conv1d(Graph* graph, int32_t weights, PadType padding, uint32_t ksize, uint32_t stride,
+         uint32_t dilation, int32_t multiplier = 0, DataLayout input_layout = DataLayout::WCN,
+         DataLayout kernel_layout = DataLayout::WIcOc);
+  Conv1d(Graph* graph, int32_t weights, PadType padding, uint32_t ksize, uint32_t stride,
+         uint32_t dilation, const std::array<uint32_t, 2>& pad, int32_t multiplier = 0,
+         DataLayout input_layout = DataLayout::WCN, DataLayout kernel_layout = DataLayout::WIcOc);
+
+  DataLayout KernelDataLayout() { return kernel_layout_; }
+  std::shared_ptr<Operation> Clone(
+      std::shared_ptr<Graph>& graph) const override;
+
+ protected:
+  const uint32_t weights_;
+  const PadType padding_;
+  const uint32_t ksize_;
+  const uint32_t stride_;
+  const uint32_t dilation_;
+  const std::array<uint32_t, 2> pad_;
+  const int32_t multiplier_;
+  const DataLayout kernel_layout_;
+
+ private:
+  void OnBindInputPostProc(const std::shared_ptr<Tensor>& tensor,
+                           int32_t input_idx) override;
+};
+
 // Grouped 2-D convolution: output channel block j (Oc / groups channels) reads input
 // channel block j (Ic / groups channels); weight {Kw, Kh, Ic / groups, Oc}, optional bias {Oc}.
 // reference: include/tim/vx/ops/groupedconv2d.h:56-82, src/tim/vx/ops/groupedconv2d.cc

@@ -733,6 +733,47 @@ void Conv2d::OnBindInputPostProc(const std::shared_ptr<Tensor>& tensor, int32_t)
   PromoteHalfBias(this, impl_.get(), tensor);
 }
 
+// ---- Conv1d -----------------------------------------------------------------
+Conv1d::Conv1d(Graph* graph, PadType padding, uint32_t stride, uint32_t dilation,
+               int32_t multiplier, DataLayout input_layout, DataLayout kernel_layout)
+    : Conv1d(graph, 0, padding, 0, stride, dilation, {0, 0}, multiplier, input_layout, kernel_layout) {}
+
+Conv1d::Conv1d(Graph* graph, const std::array<uint32_t, 2>& pad, uint32_t stride, uint32_t dilation,
+               int32_t multiplier, DataLayout input_layout, DataLayout kernel_layout)
+    : Conv1d(graph, 0, PadType::AUTO, 0, stride, dilation, pad, multiplier, input_layout, kernel_layout) {}
+
+Conv1d::Conv1d(Graph* graph, int32_t weights, PadType padding, uint32_t ksize, uint32_t stride,
+               uint32_t dilation, int32_t multiplier, DataLayout input_layout, DataLayout kernel_layout)
+    : Conv1d(graph, weights, padding, ksize, stride, dilation, {0, 0}, multiplier, input_layout,
+             kernel_layout) {}
+
+Conv1d::Conv1d(Graph* graph, int32_t weights, PadType padding, uint32_t ksize, uint32_t stride,
+               uint32_t dilation, const std::array<uint32_t, 2>& pad, int32_t multiplier,
+               DataLayout input_layout, DataLayout kernel_layout)
+    : BuiltinOp(graph, K(OpKind::CONV2D), 0, 0, input_layout),
+      weights_(weights), padding_(padding), ksize_(ksize), stride_(stride), dilation_(dilation),
+      pad_(pad), multiplier_(multiplier), kernel_layout_(kernel_layout) {
+  OpAttrs& a = impl_->attrs_;
+  a.conv_1d = true;
+  a.pad_type = padding_ == PadType::NONE ? PadType::AUTO : padding_;
+  a.pad[0] = pad_[0];
+  a.pad[1] = pad_[1];
+  a.stride[0] = stride_;
+  a.stride[1] = 1;
+  a.dilation[0] = dilation_;
+  a.dilation[1] = 1;
+  a.multiplier = multiplier_;
+}
+
+std::shared_ptr<Operation> Conv1d::Clone(std::shared_ptr<Graph>& graph) const {
+  return graph->CreateOperation<Conv1d>(static_cast<int32_t>(weights_), padding_, ksize_, stride_,
+                                        dilation_, pad_, multiplier_, impl_->layout_, kernel_layout_);
+}
+
+void Conv1d::OnBindInputPostProc(const std::shared_ptr<Tensor>& tensor, int32_t) {
+  PromoteHalfBias(this, impl_.get(), tensor);
+}
+
 // ---- GroupedConv2d ----------------------------------------------------------
 // The same operator kind as Conv2d with a group count (the reference has a kind of its own,
 // VSI_NN_OP_GROUPED_CONV2D, whose setup splits into per-group convolutions:

@@ -141,12 +141,15 @@ bool SetupConv(OpImpl* op) {
   TensorImpl* b = op->inputs_tensor_.size() > 2 && !op->inputs_tensor_[2]->IsPlaceHolder()
                       ? Impl(op->inputs_tensor_[2]) : nullptr;
   TensorImpl* y = Impl(op->outputs_tensor_[0]);
-  if (op->layout_ != DataLayout::WHCN && op->layout_ != DataLayout::ANY) {
-    VSILOGE("CONV2D: only WHCN activations are supported");
+  const bool one_d = op->attrs_.conv_1d;
+  if (one_d ? (op->layout_ != DataLayout::WCN && op->layout_ != DataLayout::ANY)
+            : (op->layout_ != DataLayout::WHCN && op->layout_ != DataLayout::ANY)) {
+    VSILOGE("%s", one_d ? "CONV1D: only WCN activations are supported" : "CONV2D: only WHCN activations are supported");
     return false;
   }
-  if (x->spec_.shape_.size() != 4 || w->spec_.shape_.size() != 4) {
-    VSILOGE("CONV2D: input and weight must be 4-D");
+  if (one_d ? (x->spec_.shape_.size() != 3 || w->spec_.shape_.size() != 3)
+            : (x->spec_.shape_.size() != 4 || w->spec_.shape_.size() != 4)) {
+    VSILOGE("%s", one_d ? "CONV1D: input and weight must be 3-D" : "CONV2D: input and weight must be 4-D");
     return false;
   }
   if (!BiasScaleConsistent(x->spec_, w->spec_, b ? &b->spec_ : nullptr)) return false;
@@ -156,7 +159,18 @@ bool SetupConv(OpImpl* op) {
     return false;
   }
   OpAttrs& a = op->attrs_;
-  const ShapeType &xs = x->spec_.shape_, &ws = w->spec_.shape_;
+  // Conv1d: {W, C, N} x {Kw, Ic, Oc} is the 2-D operator on {W, 1, C, N} x {Kw, 1, Ic, Oc}; the
+  // depthwise weight {Kw, 1, Ic*m} is the 2-D depthwise weight {Kw, 1, Ic*m, 1}
+  // (src/tim/vx/internal/src/ops/vsi_nn_op_conv1d.c reshapes the same way)
+  ShapeType xs = x->spec_.shape_, ws = w->spec_.shape_;
+  if (one_d) {
+    xs = {xs[0], 1, xs[1], xs[2]};
+    ws = a.multiplier > 0 ? ShapeType{ws[0], 1, ws[2], 1} : ShapeType{ws[0], 1, ws[1], ws[2]};
+    if (a.multiplier > 0 && w->spec_.shape_[1] != 1) {
+      VSILOGE("CONV1D: depthwise weight must be {Kw, 1, Ic*multiplier}");
+      return false;
+    }
+  }
   for (int i = 0; i < 2; ++i)
     if (a.dilation[i] == 0) a.dilation[i] = 1;
   if (a.pad_type != PadType::AUTO) {
@@ -200,6 +214,7 @@ bool SetupConv(OpImpl* op) {
     VSILOGE("CONV2D: empty output");
     return false;
   }
+  if (one_d) return AssignShape(y, ShapeType{out[0], out[2], out[3]}, "CONV1D", 1);
   return AssignShape(y, out, "CONV2D", 2);
 }
 

@@ -222,7 +222,12 @@ class HipExecutor : public Executor {
     TensorImpl* b = im->inputs_tensor_.size() > 2 && !im->inputs_tensor_[2]->IsPlaceHolder()
                         ? static_cast<TensorImpl*>(im->inputs_tensor_[2].get()) : nullptr;
     const OpAttrs& a = im->attrs_;
-    const ShapeType &xs = x->spec_.shape_, &ws = w->spec_.shape_, &os = out->spec_.shape_;
+    ShapeType xs = x->spec_.shape_, ws = w->spec_.shape_, os = out->spec_.shape_;
+    if (a.conv_1d) {  // {W, C, N} tensors viewed as {W, 1, C, N}; only the kernel extents of `ws` are read
+      xs = {xs[0], 1, xs[1], xs[2]};
+      ws = {ws[0], 1, 0, 0};
+      os = {os[0], 1, os[1], os[2]};
+    }
     tvx_conv2d_desc d{};
     d.in_w = xs[0]; d.in_h = xs[1]; d.in_c = xs[2]; d.batch = xs[3];
     d.k_w = ws[0]; d.k_h = ws[1];

@@ -10,7 +10,7 @@
 //       CONSTANT tensors get theirs at creation, INPUT tensors by CopyDataToTensor.
 //   op <KIND> <n_in> <ids..> <n_out> <ids..> <pad_type> <pl> <pr> <pt> <pb> <sw> <sh> <dw> <dh>
 //      <kw> <kh> <multiplier> <weights> <pool_type> <round_type> <pool_1d> <axis> <beta> <sm_axis>
-//      <n_shape> <shape..> <groups>
+//      <n_shape> <shape..> <groups> <conv_1d>
 //       id -1 = the graph's placeholder tensor (no bias)
 //   run <tensor id>           compile (first time) + run; append the tensor to out.bin
 //   feed <tensor id> <off> <len>   an INPUT tensor takes these blob bytes from the next run on
@@ -160,12 +160,15 @@ int main(int argc, char** argv) {
           sm_axis >> n_shape;
       std::vector<uint32_t> new_shape(n_shape);
       for (auto& d : new_shape) ss >> d;
-      int32_t groups = 0;
-      ss >> groups;
+      int32_t groups = 0, conv_1d = 0;
+      ss >> groups >> conv_1d;
       if (!ss) { std::fprintf(stderr, "malformed op record in %s\n", name.c_str()); return 2; }
       const RoundType rnd = round_type == "CEILING" ? RoundType::CEILING : RoundType::FLOOR;
       std::shared_ptr<Operation> op;
-      if (kind == "CONV2D" && groups > 1) {
+      if (kind == "CONV2D" && conv_1d) {
+        op = graph->CreateOperation<ops::Conv1d>(weights, ParsePad(pad_type), ksize[0], stride[0], dil[0],
+                                                 std::array<uint32_t, 2>{pad[0], pad[1]}, multiplier);
+      } else if (kind == "CONV2D" && groups > 1) {
         if (ParsePad(pad_type) == PadType::AUTO)
           op = graph->CreateOperation<ops::GroupedConv2d>(pad, stride, dil, groups);
         else
