@@ -173,7 +173,8 @@ int tvx_activation_create(const tvx_eltwise_desc* desc, tvx_op** op);
  * (src/tim/vx/internal/src/kernel/vx/eltwise_vx.c:56-67). */
 int tvx_add_create(const tvx_eltwise_desc* desc, tvx_op** op);
 
-/* Softmax over dim 0 of a {channels, rows} view, fp32 output: replaces
+/* Softmax along one axis of a tensor viewed as {inner, channels, rows} (inner fastest: the
+ * product of the dimensions below the axis, 0 or 1 for axis 0), fp32 output: replaces
  * vxSoftmaxLayer2 (src/tim/vx/internal/src/kernel/vx/softmax_vx.c:88). */
 typedef struct tvx_softmax_desc {
   uint32_t channels;
@@ -182,6 +183,7 @@ typedef struct tvx_softmax_desc {
   int32_t in_dtype;
   float in_scale;
   int32_t in_zp;
+  uint64_t inner;
 } tvx_softmax_desc;
 
 int tvx_softmax_create(const tvx_softmax_desc* desc, tvx_op** op);

@@ -436,23 +436,29 @@ void tvxo_add(int dtype, int64_t count, const void* a, float a_scale, int32_t a_
  * (vxSoftmaxLayer2; src/tim/vx/internal/src/kernel/vx/softmax_vx.c:88):
  * dequantize, subtract the row maximum, exp(beta * v), normalize.
  */
-void tvxo_softmax(int dtype, int32_t c, int64_t rows, float beta, const void* x,
+void tvxo_softmax(int dtype, int32_t c, int64_t rows, int64_t inner, float beta, const void* x,
                   float in_scale, int32_t in_zp, float* y) {
+  /* the tensor is {inner, c, rows} with inner fastest: the axis' elements are `inner` apart
+   * (src/tim/vx/ops/softmax_test.cc:30-290 pins axes 0, 1 and 2 of 2-D and 3-D tensors) */
+  if (inner < 1) inner = 1;
   for (int64_t r = 0; r < rows; ++r) {
-    float mx = -INFINITY, sum = 0.f;
-    for (int32_t i = 0; i < c; ++i) {
-      int64_t idx = r * c + i;
-      float v = (dtype == TVXO_U8 || dtype == TVXO_I8) ? in_scale * (float)(load_q(x, dtype, idx) - in_zp)
-                                                     : load_f(x, dtype, idx);
-      y[idx] = v;
-      if (v > mx) mx = v;
+    for (int64_t in = 0; in < inner; ++in) {
+      const int64_t base = r * c * inner + in;
+      float mx = -INFINITY, sum = 0.f;
+      for (int32_t i = 0; i < c; ++i) {
+        int64_t idx = base + i * inner;
+        float v = (dtype == TVXO_U8 || dtype == TVXO_I8) ? in_scale * (float)(load_q(x, dtype, idx) - in_zp)
+                                                       : load_f(x, dtype, idx);
+        y[idx] = v;
+        if (v > mx) mx = v;
+      }
+      for (int32_t i = 0; i < c; ++i) {
+        float e = expf(beta * (y[base + i * inner] - mx));
+        y[base + i * inner] = e;
+        sum += e;
+      }
+      for (int32_t i = 0; i < c; ++i) y[base + i * inner] /= sum;
     }
-    for (int32_t i = 0; i < c; ++i) {
-      float e = expf(beta * (y[r * c + i] - mx));
-      y[r * c + i] = e;
-      sum += e;
-    }
-    for (int32_t i = 0; i < c; ++i) y[r * c + i] /= sum;
   }
 }
 

@@ -68,7 +68,7 @@ def lib():
                                          C.c_void_p, C.c_float, C.c_int32]
         _lib.tvxo_add.argtypes = [C.c_int, C.c_int64, C.c_void_p, C.c_float, C.c_int32, C.c_void_p,
                                   C.c_float, C.c_int32, C.c_void_p, C.c_float, C.c_int32]
-        _lib.tvxo_softmax.argtypes = [C.c_int, C.c_int32, C.c_int64, C.c_float, C.c_void_p, C.c_float,
+        _lib.tvxo_softmax.argtypes = [C.c_int, C.c_int32, C.c_int64, C.c_int64, C.c_float, C.c_void_p, C.c_float,
                                       C.c_int32, C.c_void_p]
         _lib.tvxo_conv2d.argtypes = [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         _lib.tvxo_fully_connected.argtypes = [C.POINTER(FcDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
@@ -186,9 +186,10 @@ def add(dtype, a, a_q, b, b_q, out_q):
     return y
 
 
-def softmax(dtype, x, c, beta, in_q):
+def softmax(dtype, x, c, beta, in_q, inner=1):
+    """Softmax along an axis of `c` elements that are `inner` apart (inner = product of the dimensions below it)."""
     y = np.zeros(x.size, dtype=np.float32)
-    lib().tvxo_softmax(dtype, c, x.size // c, beta, _ptr(x), in_q[0], in_q[1], _ptr(y))
+    lib().tvxo_softmax(dtype, c, x.size // (c * inner), inner, beta, _ptr(x), in_q[0], in_q[1], _ptr(y))
     return y
 
 
@@ -201,6 +202,12 @@ def expand(data, dtype_name):
     if isinstance(data, dict):
         return np.full(data["n"], data["fill"], dtype=npd)
     return np.asarray(data, dtype=npd)
+
+
+def _softmax_view(shape, axis):
+    """(elements along the axis, their distance) for a softmax along `axis` (dimension 0 is the fastest)."""
+    axis = axis % len(shape)
+    return shape[axis], int(np.prod(shape[:axis])) if axis else 1
 
 
 def pad4(shape):
@@ -249,6 +256,11 @@ def run_case(case):
                       ksize=a["ksize"], stride=a["stride"], pad_left=a["pad"][0],
                       pad_top=a["pad"][2], pool_type=POOL[a["pool_type"]],
                       dtype=DTYPE_CODE[x["dtype"]], in_q=(s, z), out_q=(so, zo))
+    if op["kind"] == "SOFTMAX":
+        x = ins[0]
+        s, z, _ = _q(x["quant"])
+        c, inner = _softmax_view(x["shape"], a.get("sm_axis", 0))
+        return softmax(DTYPE_CODE[x["dtype"]], arr[0], c, a.get("beta", 1.0), (s, z), inner)
     raise NotImplementedError(op["kind"])
 
 
@@ -306,7 +318,8 @@ def run_graph(graph, keep_all=False):
             sb, zb, _ = _q(b["quant"])
             y = add(DTYPE_CODE[x["dtype"]], xv, (s, z), val[b["id"]], (sb, zb), (so, zo))
         elif k == "SOFTMAX":
-            y = softmax(DTYPE_CODE[x["dtype"]], xv, x["shape"][0], a.get("beta", 1.0), (s, z))
+            c, inner = _softmax_view(x["shape"], a.get("sm_axis", 0))
+            y = softmax(DTYPE_CODE[x["dtype"]], xv, c, a.get("beta", 1.0), (s, z), inner)
         elif k == "RESHAPE":
             y = xv
         else:

@@ -29,6 +29,7 @@ SOURCES = {
     "fullyconnected": "src/tim/vx/ops/fullyconnected_test.cc",
     "max_pool": "src/tim/vx/ops/max_pool_test.cc",
     "avg_pool": "src/tim/vx/ops/avg_pool_test.cc",
+    "softmax": "src/tim/vx/ops/softmax_test.cc",
 }
 
 

@@ -53,7 +53,7 @@ class EltwiseDesc(C.Structure):
 
 class SoftmaxDesc(C.Structure):
     _fields_ = [("channels", C.c_uint32), ("rows", C.c_uint64), ("beta", C.c_float),
-                ("in_dtype", C.c_int32), ("in_scale", C.c_float), ("in_zp", C.c_int32)]
+                ("in_dtype", C.c_int32), ("in_scale", C.c_float), ("in_zp", C.c_int32), ("inner", C.c_uint64)]
 
 
 class TvxError(RuntimeError):

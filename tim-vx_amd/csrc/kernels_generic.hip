@@ -562,50 +562,53 @@ int AddRun(tvx_op* op, const void* in0, const void* in1, void* out, hipStream_t 
 // ---------------------------------------------------------------------------
 template <typename T, bool QUANT>
 __global__ void __launch_bounds__(kBlock)
-SoftmaxKernel(int c, uint64_t rows, float beta, float scale, int zp, const T* __restrict__ x,
+SoftmaxKernel(int c, uint64_t rows, uint64_t inner, float beta, float scale, int zp, const T* __restrict__ x,
               float* __restrict__ y) {
-  const uint64_t r = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
-  if (r >= rows) return;
-  const T* xp = x + r * c;
-  float* yp = y + r * c;
+  // one thread per (row, inner position); the c elements of its group are `inner` apart
+  const uint64_t t = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (t >= rows * inner) return;
+  const uint64_t base = (t / inner) * c * inner + t % inner;
+  const T* xp = x + base;
+  float* yp = y + base;
   float mx = -INFINITY;
   for (int i = 0; i < c; ++i) {
     float v;
-    if constexpr (QUANT) v = scale * static_cast<float>(static_cast<int>(xp[i]) - zp);
-    else v = ToFloat(xp[i]);
-    yp[i] = v;
+    if constexpr (QUANT) v = scale * static_cast<float>(static_cast<int>(xp[i * inner]) - zp);
+    else v = ToFloat(xp[i * inner]);
+    yp[i * inner] = v;
     mx = v > mx ? v : mx;
   }
   float sum = 0.f;
   for (int i = 0; i < c; ++i) {
-    const float e = expf(beta * (yp[i] - mx));
-    yp[i] = e;
+    const float e = expf(beta * (yp[i * inner] - mx));
+    yp[i * inner] = e;
     sum += e;
   }
-  for (int i = 0; i < c; ++i) yp[i] = yp[i] / sum;
+  for (int i = 0; i < c; ++i) yp[i * inner] = yp[i * inner] / sum;
 }
 
 int SoftmaxRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
   const tvx_softmax_desc& d = op->sm;
   if (!d.rows) return TVX_OK;
-  const dim3 grid(Blocks(d.rows)), block(kBlock);
+  const uint64_t inner = d.inner ? d.inner : 1;
+  const dim3 grid(Blocks(d.rows * inner)), block(kBlock);
   float* y = static_cast<float*>(out);
   const int c = static_cast<int>(d.channels);
   switch (d.in_dtype) {
     case TVX_U8:
-      hipLaunchKernelGGL((SoftmaxKernel<uint8_t, true>), grid, block, 0, st, c, d.rows, d.beta,
+      hipLaunchKernelGGL((SoftmaxKernel<uint8_t, true>), grid, block, 0, st, c, d.rows, inner, d.beta,
                          d.in_scale, d.in_zp, static_cast<const uint8_t*>(in0), y);
       break;
     case TVX_I8:
-      hipLaunchKernelGGL((SoftmaxKernel<int8_t, true>), grid, block, 0, st, c, d.rows, d.beta,
+      hipLaunchKernelGGL((SoftmaxKernel<int8_t, true>), grid, block, 0, st, c, d.rows, inner, d.beta,
                          d.in_scale, d.in_zp, static_cast<const int8_t*>(in0), y);
       break;
     case TVX_F32:
-      hipLaunchKernelGGL((SoftmaxKernel<float, false>), grid, block, 0, st, c, d.rows, d.beta, 1.f,
+      hipLaunchKernelGGL((SoftmaxKernel<float, false>), grid, block, 0, st, c, d.rows, inner, d.beta, 1.f,
                          0, static_cast<const float*>(in0), y);
       break;
     default:
-      hipLaunchKernelGGL((SoftmaxKernel<__half, false>), grid, block, 0, st, c, d.rows, d.beta, 1.f,
+      hipLaunchKernelGGL((SoftmaxKernel<__half, false>), grid, block, 0, st, c, d.rows, inner, d.beta, 1.f,
                          0, static_cast<const __half*>(in0), y);
   }
   TVX_HIP_CHECK(hipGetLastError());

@@ -353,13 +353,19 @@ class HipExecutor : public Executor {
 
   bool AddSoftmax(OpImpl* im, TensorImpl* out) {
     TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
-    if (im->attrs_.sm_axis != 0 || out->spec_.datatype_ != DataType::FLOAT32) {
-      VSILOGE("SOFTMAX: only axis 0 with a FLOAT32 output is implemented");
+    const ShapeType& xs = x->spec_.shape_;
+    const int32_t rank = static_cast<int32_t>(xs.size());
+    int32_t axis = im->attrs_.sm_axis;
+    if (axis < 0) axis += rank;  // negative axes count from the slowest dimension
+    if (axis < 0 || axis >= rank || out->spec_.datatype_ != DataType::FLOAT32) {
+      VSILOGE("SOFTMAX: axis %d of a rank-%d tensor with a FLOAT32 output is what is implemented", im->attrs_.sm_axis, rank);
       return false;
     }
     tvx_softmax_desc d{};
-    d.channels = x->spec_.shape_[0];
-    d.rows = static_cast<uint64_t>(x->spec_.GetElementNum()) / d.channels;
+    d.channels = xs[axis];
+    d.inner = 1;
+    for (int32_t i = 0; i < axis; ++i) d.inner *= xs[i];
+    d.rows = static_cast<uint64_t>(x->spec_.GetElementNum()) / (d.channels * d.inner);
     d.beta = im->attrs_.beta;
     d.in_dtype = DtypeCode(x->spec_.datatype_);
     d.in_scale = ScaleOf(x->spec_); d.in_zp = ZpOf(x->spec_);
