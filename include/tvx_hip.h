@@ -188,6 +188,20 @@ typedef struct tvx_softmax_desc {
 
 int tvx_softmax_create(const tvx_softmax_desc* desc, tvx_op** op);
 
+/* ---- Transpose (permute) ----------------------------------------------------- */
+/* Replaces the PERMUTE operator (src/tim/vx/ops/transpose.cc -> vxTensorPermuteNode):
+ * output dimension i is input dimension perm[i] (out.size[i] = in.size[perm[i]],
+ * src/tim/vx/internal/src/ops/vsi_nn_op_permute.c:219-230), dimension 0 fastest. Elements
+ * are moved as they are (any type of elem_bytes 1, 2 or 4). */
+typedef struct tvx_transpose_desc {
+  uint32_t rank;       /* 1..6 */
+  uint32_t in_dims[6];
+  uint32_t perm[6];
+  uint32_t elem_bytes;
+} tvx_transpose_desc;
+
+int tvx_transpose_create(const tvx_transpose_desc* desc, tvx_op** op);
+
 /* ---- running / inspecting operators ---------------------------------------- */
 /* Enqueue one execution (the per-node share of vxProcessGraph).
  * in0: activation; in1: run-time weights (conv / FC created without constant

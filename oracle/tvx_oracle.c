@@ -462,6 +462,34 @@ void tvxo_softmax(int dtype, int32_t c, int64_t rows, int64_t inner, float beta,
   }
 }
 
+/*
+ * Transpose (PERMUTE): output dimension i is input dimension perm[i], dimension 0 fastest
+ * (src/tim/vx/internal/src/ops/vsi_nn_op_permute.c:219-230 sizes the output as
+ * out.size[i] = in.size[perm[i]]; src/tim/vx/ops/transpose_test.cc:29-100). Elements are
+ * moved byte for byte. Written as a walk over INPUT coordinates that scatters, the reverse
+ * of the product's gather.
+ */
+void tvxo_transpose(int32_t rank, const uint32_t* in_dims, const uint32_t* perm, int32_t elem_bytes,
+                    const void* x, void* y) {
+  uint64_t out_stride_of_in[8], out_dims[8], total = 1, s = 1;
+  for (int32_t i = 0; i < rank; ++i) out_dims[i] = in_dims[perm[i]];
+  for (int32_t i = 0; i < rank; ++i) {
+    out_stride_of_in[perm[i]] = s; /* input dimension perm[i] is output dimension i */
+    s *= out_dims[i];
+    total *= in_dims[i];
+  }
+  uint32_t coord[8] = {0};
+  for (uint64_t idx = 0; idx < total; ++idx) {
+    uint64_t dst = 0;
+    for (int32_t i = 0; i < rank; ++i) dst += coord[i] * out_stride_of_in[i];
+    memcpy((char*)y + dst * elem_bytes, (const char*)x + idx * elem_bytes, (size_t)elem_bytes);
+    for (int32_t i = 0; i < rank; ++i) {
+      if (++coord[i] < in_dims[i]) break;
+      coord[i] = 0;
+    }
+  }
+}
+
 int tvxo_num_threads(void) {
 #ifdef _OPENMP
   return omp_get_max_threads();

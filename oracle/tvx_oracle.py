@@ -68,6 +68,9 @@ def lib():
                                          C.c_void_p, C.c_float, C.c_int32]
         _lib.tvxo_add.argtypes = [C.c_int, C.c_int64, C.c_void_p, C.c_float, C.c_int32, C.c_void_p,
                                   C.c_float, C.c_int32, C.c_void_p, C.c_float, C.c_int32]
+        _lib.tvxo_transpose.argtypes = [C.c_int32, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.c_int32,
+                                        C.c_void_p, C.c_void_p]
+        _lib.tvxo_transpose.restype = None
         _lib.tvxo_softmax.argtypes = [C.c_int, C.c_int32, C.c_int64, C.c_int64, C.c_float, C.c_void_p, C.c_float,
                                       C.c_int32, C.c_void_p]
         _lib.tvxo_conv2d.argtypes = [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
@@ -196,6 +199,16 @@ def softmax(dtype, x, c, beta, in_q, inner=1):
 # --------------------------------------------------------------------------
 # fixture cases
 # --------------------------------------------------------------------------
+def transpose(x, in_dims, perm):
+    """Output dimension i is input dimension perm[i] (dimension 0 fastest); x is the flat input."""
+    x = np.ascontiguousarray(x).reshape(-1)
+    y = np.empty_like(x)
+    dims = (C.c_uint32 * len(in_dims))(*in_dims)
+    pm = (C.c_uint32 * len(perm))(*perm)
+    lib().tvxo_transpose(len(in_dims), dims, pm, x.dtype.itemsize, _ptr(x), _ptr(y))
+    return y
+
+
 def expand(data, dtype_name):
     """Fixture 'data' field (list, or {'fill': v, 'n': count}) -> flat numpy array."""
     npd = NP_DTYPE[dtype_name]
@@ -261,6 +274,8 @@ def run_case(case):
         s, z, _ = _q(x["quant"])
         c, inner = _softmax_view(x["shape"], a.get("sm_axis", 0))
         return softmax(DTYPE_CODE[x["dtype"]], arr[0], c, a.get("beta", 1.0), (s, z), inner)
+    if op["kind"] == "TRANSPOSE":
+        return transpose(arr[0], ins[0]["shape"], a["perm"])
     raise NotImplementedError(op["kind"])
 
 
@@ -322,6 +337,8 @@ def run_graph(graph, keep_all=False):
             y = softmax(DTYPE_CODE[x["dtype"]], xv, c, a.get("beta", 1.0), (s, z), inner)
         elif k == "RESHAPE":
             y = xv
+        elif k == "TRANSPOSE":
+            y = transpose(xv, x["shape"], a["perm"])
         else:
             raise NotImplementedError(k)
         val[out["id"]] = y

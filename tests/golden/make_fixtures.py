@@ -30,6 +30,7 @@ SOURCES = {
     "max_pool": "src/tim/vx/ops/max_pool_test.cc",
     "avg_pool": "src/tim/vx/ops/avg_pool_test.cc",
     "softmax": "src/tim/vx/ops/softmax_test.cc",
+    "transpose": "src/tim/vx/ops/transpose_test.cc",
 }
 
 

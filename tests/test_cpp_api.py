@@ -135,6 +135,33 @@ def test_lenet_sample_graph(tmp_path, oracle):
 
 
 @pytest.mark.gpu
+def test_transpose_feeds_a_convolution(tmp_path, oracle):
+    """A channel-fastest {C, W, H, N} image brought to WHCN by Transpose{1, 2, 0, 3} (the permute
+    layout inference puts in front of an NHWC model, src/tim/transform/layout_inference.cc), then a
+    3x3 convolution; the output goes back to channel-fastest through Transpose{2, 0, 1, 3}."""
+    rng = np.random.default_rng(5)
+    c, w, h, n, oc = 8, 12, 10, 2, 16
+    q = GF.asym
+    x = rng.integers(0, 256, c * w * h * n, dtype=np.uint8)
+    wt = rng.integers(0, 256, 3 * 3 * c * oc, dtype=np.uint8)
+    bias = rng.integers(-500, 500, oc, dtype=np.int32)
+    T = GF.tensor
+    g = {"test": "transpose_conv_transpose", "output": 6, "tensors": [
+        T(0, "UINT8", "INPUT", [c, w, h, n], q(0.5, 128), x),
+        T(1, "UINT8", "TRANSIENT", [w, h, c, n], q(0.5, 128)),
+        T(2, "UINT8", "CONSTANT", [3, 3, c, oc], q(0.25, 120), wt),
+        T(3, "INT32", "CONSTANT", [oc], q(0.125, 0), bias),
+        T(4, "UINT8", "TRANSIENT", [w, h, oc, n], q(64.0, 100)),
+        T(6, "UINT8", "OUTPUT", [oc, w, h, n], q(64.0, 100))],
+        "ops": [GF.op("TRANSPOSE", [0], [1], perm=[1, 2, 0, 3]),
+                GF.op("CONV2D", [1, 2, 3], [4], pad_type="AUTO", pad=[1, 1, 1, 1], ksize=[3, 3], weights=oc),
+                GF.op("TRANSPOSE", [4], [6], perm=[2, 0, 1, 3])]}
+    res, info, log = GF.run_graphs([g], str(tmp_path))
+    assert res[0] is not None, (info, log[-2000:])
+    assert np.array_equal(res[0], oracle.run_graph(g))
+
+
+@pytest.mark.gpu
 def test_repeated_runs_follow_the_inputs(tmp_path, oracle):
     """Run() may be called again and again with the inputs re-filled in between
     (src/tim/vx/graph.cc:378-391): six runs with the input alternating between two images,

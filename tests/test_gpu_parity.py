@@ -470,3 +470,24 @@ def test_depthwise_then_pointwise_full_size(oracle):
     out = TC.gpu_conv2d(mid, wp, bp, want_kernel="pwconv_i8", **kp)
     assert np.array_equal(out, out_want)
     assert out.min() == 0 and out.max() == 120  # ReLU6 at scale 0.05
+
+
+@pytest.mark.parametrize("in_dims,perm", [
+    ((5, 3), (1, 0)), ((4, 3, 2), (2, 0, 1)), ((4, 3, 2), (1, 2, 0)), ((56, 56, 24, 3), (2, 0, 1, 3)),
+    ((24, 56, 56, 3), (1, 2, 0, 3)), ((7, 5, 3, 2), (0, 1, 2, 3)), ((3, 1, 4, 1, 5, 2), (5, 4, 3, 2, 1, 0)), ((6,), (0,))])
+def test_transpose(oracle, in_dims, perm):
+    # (2,0,1,3) / (1,2,0,3) are the WHCN <-> CWHN conversions layout inference inserts around NHWC models
+    for dt in (np.uint8, np.float16, np.int32):
+        x = ((np.arange(int(np.prod(in_dims))) * 7 + 3) % 60000).astype(np.uint32).astype(dt)
+        assert np.array_equal(TC.gpu_transpose(x, in_dims, perm), oracle.transpose(x, in_dims, perm))
+
+
+def test_transpose_rejects_bad_descriptors():
+    T = TC.tvx()
+    for rank, perm, eb in ((0, (0,), 1), (7, (0,) * 6, 1), (2, (0, 0), 1), (2, (0, 2), 1), (2, (1, 0), 3)):
+        d = T.TransposeDesc()
+        d.rank, d.elem_bytes = rank, eb
+        for i in range(min(rank, 6)):
+            d.in_dims[i], d.perm[i] = 2, perm[i]
+        with pytest.raises(T.TvxError):
+            T.transpose_create(d)

@@ -196,3 +196,30 @@ def test_quantized_add_and_softmax(oracle):
     ref = np.exp((x.reshape(4, 10).astype(np.float64) - 128) * np.float32(0.1))
     ref /= ref.sum(axis=1, keepdims=True)
     assert np.allclose(sm.reshape(4, 10), ref, rtol=1e-5, atol=1e-7)
+
+
+def _np_transpose(x, in_dims, perm):
+    # numpy's axes run slowest first, the tensors here fastest first: dimension d is numpy axis r-1-d.
+    r = len(in_dims)
+    a = x.reshape(tuple(reversed(in_dims)))
+    return np.transpose(a, axes=[r - 1 - perm[r - 1 - j] for j in range(r)]).reshape(-1)
+
+
+@pytest.mark.parametrize("in_dims,perm", [
+    ((5, 3), (1, 0)), ((4, 3, 2), (2, 0, 1)), ((4, 3, 2), (1, 2, 0)), ((7, 5, 3, 2), (2, 0, 1, 3)),
+    ((7, 5, 3, 2), (0, 1, 2, 3)), ((3, 1, 4, 1, 5), (4, 3, 2, 1, 0)), ((6,), (0,))])
+def test_transpose_restatement_vs_numpy(oracle, in_dims, perm):
+    # A non-involutive perm ((2,0,1) vs (1,2,0)) tells out[i] = in[perm[i]] from its inverse reading.
+    for dt in (np.uint8, np.float16, np.int32):
+        x = np.arange(int(np.prod(in_dims))).astype(dt)
+        got = oracle.transpose(x, in_dims, perm)
+        assert got.dtype == x.dtype
+        assert np.array_equal(got, _np_transpose(x, in_dims, perm))
+    # the extent rule of the reference: out.size[i] = in.size[perm[i]]; element at input coordinate c lands
+    # at output coordinate o with o[i] = c[perm[i]] -- checked by hand on one element of (4,3,2)/(2,0,1)
+    if in_dims == (4, 3, 2) and perm == (2, 0, 1):
+        x = np.arange(24, dtype=np.int32)
+        y = oracle.transpose(x, in_dims, perm)            # out dims (2, 4, 3)
+        c = (3, 1, 1)                                     # input offset 3 + 4*1 + 12*1 = 19
+        o = (c[2], c[0], c[1])                            # output offset 1 + 2*3 + 8*1 = 15
+        assert y[o[0] + 2 * o[1] + 8 * o[2]] == 19

@@ -10,7 +10,8 @@ import numpy as np
 import tvx_oracle as O
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-GOLDEN_FILES = ["conv2d", "depthwise_conv", "grouped_conv2d", "conv1d", "fullyconnected", "max_pool", "avg_pool", "softmax"]
+GOLDEN_FILES = ["conv2d", "depthwise_conv", "grouped_conv2d", "conv1d", "fullyconnected", "max_pool", "avg_pool", "softmax",
+                "transpose"]
 
 
 def load_cases(name):
@@ -204,6 +205,21 @@ def gpu_softmax(dtype, x, c, beta, in_q, inner=1):
     return yd.cpu().numpy()
 
 
+def gpu_transpose(x, in_dims, perm):
+    T = tvx()
+    d = T.TransposeDesc()
+    d.rank, d.elem_bytes = len(in_dims), x.dtype.itemsize
+    for i, (n, p) in enumerate(zip(in_dims, perm)):
+        d.in_dims[i], d.perm[i] = n, p
+    op = T.transpose_create(d)
+    import torch
+    xd = to_device(x)
+    yd = torch.empty_like(xd)
+    op.run(xd, None, yd)
+    torch.cuda.synchronize()
+    return yd.cpu().numpy()
+
+
 def run_case_gpu(case):
     """One-operator fixture graph through the C ABI; mirrors tvx_oracle.run_case."""
     tensors = {t["id"]: t for t in case["tensors"]}
@@ -248,4 +264,6 @@ def run_case_gpu(case):
         s, z, _ = O._q(x["quant"])
         c, inner = O._softmax_view(x["shape"], a.get("sm_axis", 0))
         return gpu_softmax(code[x["dtype"]], arr[0], c, a.get("beta", 1.0), (s, z), inner)
+    if op["kind"] == "TRANSPOSE":
+        return gpu_transpose(arr[0], ins[0]["shape"], a["perm"])
     raise NotImplementedError(op["kind"])

@@ -615,6 +615,56 @@ int SoftmaxRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t 
   return TVX_OK;
 }
 
+// ---------------------------------------------------------------------------
+// Transpose: one thread per output element; output dimension i walks input dimension perm[i]
+// ---------------------------------------------------------------------------
+struct TransposeArgs {
+  uint32_t rank;
+  uint32_t out_dims[6];
+  uint64_t in_stride[6];  // element stride of the input dimension each output dimension walks
+};
+
+template <typename T>
+__global__ void __launch_bounds__(kBlock)
+TransposeKernel(TransposeArgs a, const T* __restrict__ x, T* __restrict__ y, uint64_t total) {
+  const uint64_t idx = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (idx >= total) return;
+  uint64_t rest = idx, src = 0;
+  for (uint32_t i = 0; i < a.rank; ++i) {
+    const uint64_t c = rest % a.out_dims[i];
+    rest /= a.out_dims[i];
+    src += c * a.in_stride[i];
+  }
+  y[idx] = x[src];
+}
+
+int TransposeRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
+  const tvx_transpose_desc& d = op->tr;
+  TransposeArgs a{};
+  a.rank = d.rank;
+  uint64_t stride[6], total = 1;
+  for (uint32_t i = 0; i < d.rank; ++i) {
+    stride[i] = total;
+    total *= d.in_dims[i];
+  }
+  for (uint32_t i = 0; i < d.rank; ++i) {
+    a.out_dims[i] = d.in_dims[d.perm[i]];
+    a.in_stride[i] = stride[d.perm[i]];
+  }
+  const dim3 grid(Blocks(total)), block(kBlock);
+  if (d.elem_bytes == 1)
+    hipLaunchKernelGGL((TransposeKernel<uint8_t>), grid, block, 0, st, a, static_cast<const uint8_t*>(in0),
+                       static_cast<uint8_t*>(out), total);
+  else if (d.elem_bytes == 2)
+    hipLaunchKernelGGL((TransposeKernel<uint16_t>), grid, block, 0, st, a, static_cast<const uint16_t*>(in0),
+                       static_cast<uint16_t*>(out), total);
+  else
+    hipLaunchKernelGGL((TransposeKernel<uint32_t>), grid, block, 0, st, a, static_cast<const uint32_t*>(in0),
+                       static_cast<uint32_t*>(out), total);
+  TVX_HIP_CHECK(hipGetLastError());
+  return TVX_OK;
+}
+
 int UploadWeightsAndBias(tvx_op* op, const void* w, size_t w_bytes, const void* b, size_t b_bytes) {
   int s = TVX_OK;
   if (w) s = op->weights.Upload(w, w_bytes);
@@ -683,6 +733,12 @@ int AddSetup(tvx_op* op) {
   op->geo[2] = op->quantized && ra < 1048576.0 && rb < 1048576.0 ? 1 : 0;
   op->run = AddRun;
   op->kernel_name = "add_generic";
+  return TVX_OK;
+}
+
+int TransposeSetup(tvx_op* op) {
+  op->run = TransposeRun;
+  op->kernel_name = "transpose_generic";
   return TVX_OK;
 }
 

@@ -430,6 +430,31 @@ int tvx_softmax_create(const tvx_softmax_desc* d, tvx_op** out) {
   return TVX_OK;
 }
 
+int tvx_transpose_create(const tvx_transpose_desc* d, tvx_op** out) {
+  if (!d || !out) return SetError(TVX_E_INVALID, "tvx_transpose_create: null argument");
+  *out = nullptr;
+  if (d->rank < 1 || d->rank > 6) return SetError(TVX_E_INVALID, "tvx_transpose_create: rank %u not in 1..6", d->rank);
+  if (d->elem_bytes != 1 && d->elem_bytes != 2 && d->elem_bytes != 4)
+    return SetError(TVX_E_INVALID, "tvx_transpose_create: element size %u", d->elem_bytes);
+  uint32_t seen = 0;
+  for (uint32_t i = 0; i < d->rank; ++i) {
+    if (d->perm[i] >= d->rank || (seen >> d->perm[i] & 1u))
+      return SetError(TVX_E_INVALID, "tvx_transpose_create: perm is not a permutation of 0..%u", d->rank - 1);
+    seen |= 1u << d->perm[i];
+    if (!d->in_dims[i]) return SetError(TVX_E_INVALID, "tvx_transpose_create: zero extent");
+  }
+  int s = NoGpu();
+  if (s != TVX_OK) return s;
+  tvx_op* op = new (std::nothrow) tvx_op();
+  if (!op) return SetError(TVX_E_NOMEM, "tvx_transpose_create: host allocation failed");
+  op->kind = OP_TRANSPOSE;
+  op->tr = *d;
+  s = TransposeSetup(op);
+  if (s != TVX_OK) { delete op; return s; }
+  *out = op;
+  return TVX_OK;
+}
+
 int tvx_op_run(tvx_op* op, const void* in0, const void* in1, void* out_ptr, void* stream) {
   if (!op || !op->run) return SetError(TVX_E_INVALID, "tvx_op_run: null operator");
   if (!in0 || !out_ptr) return SetError(TVX_E_INVALID, "tvx_op_run: null tensor pointer");

@@ -257,6 +257,18 @@ class Reshape : public BuiltinOp {
   std::vector<uint32_t> size_;
 };
 
+// reference: include/tim/vx/ops/transpose.h
+// Output dimension i is input dimension perm[i], dimension 0 fastest.
+class Transpose : public BuiltinOp {
+ public:
+  Transpose(Graph* graph, const std::vector<uint32_t>& perm);
+  std::shared_ptr<Operation> Clone(
+      std::shared_ptr<Graph>& graph) const override;
+
+ protected:
+  std::vector<uint32_t> perm_;
+};
+
 }  // namespace ops
 }  // namespace vx
 }  // namespace tim

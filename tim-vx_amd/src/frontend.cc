@@ -35,6 +35,7 @@ const char* OpKindName(OpKind k) {
     case OpKind::ADD: return "ADD";
     case OpKind::SOFTMAX: return "SOFTMAX";
     case OpKind::RESHAPE: return "RESHAPE";
+    case OpKind::TRANSPOSE: return "TRANSPOSE";
   }
   return "?";
 }
@@ -991,6 +992,14 @@ Reshape::Reshape(Graph* graph, const std::vector<uint32_t>& target_shape)
 }
 std::shared_ptr<Operation> Reshape::Clone(std::shared_ptr<Graph>& graph) const {
   return graph->CreateOperation<Reshape>(size_);
+}
+
+Transpose::Transpose(Graph* graph, const std::vector<uint32_t>& perm)
+    : BuiltinOp(graph, K(OpKind::TRANSPOSE), 1, 1), perm_(perm) {
+  impl_->attrs_.perm = perm;
+}
+std::shared_ptr<Operation> Transpose::Clone(std::shared_ptr<Graph>& graph) const {
+  return graph->CreateOperation<Transpose>(perm_);
 }
 
 }  // namespace ops

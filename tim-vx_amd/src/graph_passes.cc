@@ -326,6 +326,37 @@ bool SetupReshape(OpImpl* op) {
   return AssignShape(Impl(op->outputs_tensor_[0]), op->attrs_.new_shape, "RESHAPE");
 }
 
+// reference: src/tim/vx/internal/src/ops/vsi_nn_op_permute.c:219-230 (out.size[i] = in.size[perm[i]])
+bool SetupTranspose(OpImpl* op) {
+  if (op->inputs_tensor_.size() != 1 || op->outputs_tensor_.size() != 1) {
+    VSILOGE("TRANSPOSE: wrong operand count");
+    return false;
+  }
+  TensorImpl* x = Impl(op->inputs_tensor_[0]);
+  TensorImpl* y = Impl(op->outputs_tensor_[0]);
+  const ShapeType& xs = x->spec_.shape_;
+  const std::vector<uint32_t>& perm = op->attrs_.perm;
+  if (perm.size() != xs.size() || xs.empty() || xs.size() > 6) {
+    VSILOGE("TRANSPOSE: perm of %zu entries for a rank-%zu input (ranks 1..6)", perm.size(), xs.size());
+    return false;
+  }
+  std::vector<bool> seen(xs.size(), false);
+  ShapeType out(xs.size());
+  for (size_t i = 0; i < perm.size(); ++i) {
+    if (perm[i] >= xs.size() || seen[perm[i]]) {
+      VSILOGE("TRANSPOSE: perm is not a permutation of the input's dimensions");
+      return false;
+    }
+    seen[perm[i]] = true;
+    out[i] = xs[perm[i]];
+  }
+  if (y->spec_.datatype_ != x->spec_.datatype_) {
+    VSILOGE("TRANSPOSE: output type differs from the input's");
+    return false;
+  }
+  return AssignShape(y, out, "TRANSPOSE");
+}
+
 }  // namespace
 
 bool GraphImpl::VerifyAndInfer() {
@@ -387,6 +418,7 @@ bool GraphImpl::VerifyAndInfer() {
       case OpKind::ADD: ok = SetupSameShape(im, "ADD", 2); break;
       case OpKind::SOFTMAX: ok = SetupSameShape(im, "SOFTMAX", 1); break;
       case OpKind::RESHAPE: ok = SetupReshape(im); break;
+      case OpKind::TRANSPOSE: ok = SetupTranspose(im); break;
     }
     if (!ok) {
       VSILOGE("setup of %s (uid %u) failed", OpKindName(im->kind_), im->uid_);

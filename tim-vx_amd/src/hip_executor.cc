@@ -124,6 +124,7 @@ class HipExecutor : public Executor {
         case OpKind::ADD: ok = AddAdd(im, out); break;
         case OpKind::SOFTMAX: ok = AddSoftmax(im, out); break;
         case OpKind::RESHAPE: break;  // aliased
+        case OpKind::TRANSPOSE: ok = AddTranspose(im, out); break;
       }
       if (!ok) return false;
     }
@@ -371,6 +372,21 @@ class HipExecutor : public Executor {
     d.in_scale = ScaleOf(x->spec_); d.in_zp = ZpOf(x->spec_);
     tvx_op* op = nullptr;
     if (tvx_softmax_create(&d, &op) != TVX_OK) return Fail("tvx_softmax_create");
+    Push(op, im, x, nullptr, out);
+    return true;
+  }
+
+  bool AddTranspose(OpImpl* im, TensorImpl* out) {
+    TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
+    tvx_transpose_desc d{};
+    d.rank = static_cast<uint32_t>(x->spec_.shape_.size());
+    for (uint32_t i = 0; i < d.rank; ++i) {
+      d.in_dims[i] = x->spec_.shape_[i];
+      d.perm[i] = im->attrs_.perm[i];
+    }
+    d.elem_bytes = static_cast<uint32_t>(x->spec_.GetElementByteSize());
+    tvx_op* op = nullptr;
+    if (tvx_transpose_create(&d, &op) != TVX_OK) return Fail("tvx_transpose_create");
     Push(op, im, x, nullptr, out);
     return true;
   }

@@ -32,7 +32,7 @@ int TvxLogThreshold();
 #define VSILOGD(...) TVX_LOG(::tim::vx::TVX_LOG_DEBUG, "D ", __VA_ARGS__)
 
 enum class OpKind : uint32_t {
-  CONV2D = 1, FCL, POOL, RELU, RELU6, ADD, SOFTMAX, RESHAPE
+  CONV2D = 1, FCL, POOL, RELU, RELU6, ADD, SOFTMAX, RESHAPE, TRANSPOSE
 };
 const char* OpKindName(OpKind k);
 
@@ -60,6 +60,8 @@ struct OpAttrs {
   int32_t sm_axis = 0;
   // reshape
   std::vector<uint32_t> new_shape;
+  // transpose
+  std::vector<uint32_t> perm;
   // rounding policy (Operation::SetRoundingPolicy)
   OverflowPolicy overflow = OverflowPolicy::SATURATE;
   RoundingPolicy rounding = RoundingPolicy::RTNE;

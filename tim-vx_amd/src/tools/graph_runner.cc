@@ -162,6 +162,10 @@ int main(int argc, char** argv) {
       for (auto& d : new_shape) ss >> d;
       int32_t groups = 0, conv_1d = 0;
       ss >> groups >> conv_1d;
+      int32_t n_perm = 0;
+      ss >> n_perm;
+      std::vector<uint32_t> perm(n_perm > 0 ? n_perm : 0);
+      for (auto& d : perm) ss >> d;
       if (!ss) { std::fprintf(stderr, "malformed op record in %s\n", name.c_str()); return 2; }
       const RoundType rnd = round_type == "CEILING" ? RoundType::CEILING : RoundType::FLOOR;
       std::shared_ptr<Operation> op;
@@ -196,6 +200,8 @@ int main(int argc, char** argv) {
         op = graph->CreateOperation<ops::Softmax>(beta, sm_axis);
       } else if (kind == "RESHAPE") {
         op = graph->CreateOperation<ops::Reshape>(new_shape);
+      } else if (kind == "TRANSPOSE") {
+        op = graph->CreateOperation<ops::Transpose>(perm);
       } else {
         std::fprintf(stderr, "unknown op kind %s\n", kind.c_str());
         return 2;
