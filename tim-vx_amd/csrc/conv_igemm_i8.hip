@@ -20,6 +20,7 @@
 // four pixels per dword, stage [oc][pixel] in LDS, copy out as contiguous
 // runs of the WHCN output.
 #include <algorithm>
+#include <type_traits>
 
 #include "variants.h"
 
@@ -31,7 +32,6 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int kThreads = 256;
 constexpr int kMaxPtw = 2;     // 32-pixel MFMA tiles per wavefront (tile <= 256 pixels)
-constexpr int kLoadBatch = 8;  // halo units a thread keeps in flight
 
 struct ConvArgs {
   const uint8_t* x;
@@ -55,7 +55,7 @@ struct ConvArgs {
   int out_stride;        // epilogue staging row stride in bytes (odd number of dwords)
   int w_chunks;          // 16-byte chunks of one channel block's weights
   int w4_blocks;         // ceil(W / 64): blocks of 16 four-column patches per channel row
-  int off_w, off_halo, off_sx, off_tap;  // LDS carve-up
+  int off_w, off_halo, off_sx, off_tap, off_rq, off_bias;  // LDS carve-up
 };
 
 __device__ __forceinline__ int FastDiv(int u, uint32_t magic) {
@@ -78,8 +78,16 @@ template <int OT, int RQ>
 __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(OT == 1 ? 4 : 2, OT == 1 ? 4 : 2))) ConvIgemmKernel(ConvArgs a) {
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int tile = blockIdx.x % a.tiles_per_image;
-  const int n = blockIdx.x / a.tiles_per_image;
+  // Workgroups go to the eight XCDs round-robin in launch order and each XCD has its own L2:
+  // renumber them so that an XCD gets a contiguous run of tiles. Neighbouring tiles of an image,
+  // whose halo rows overlap, then meet in one L2 instead of fetching the rows from HBM twice.
+  int bx = blockIdx.x;
+  if (gridDim.y == 1) {
+    const int per = gridDim.x >> 3, rem = gridDim.x & 7, xcd = bx & 7;
+    bx = xcd * per + min(xcd, rem) + (bx >> 3);
+  }
+  const int tile = bx % a.tiles_per_image;
+  const int n = bx / a.tiles_per_image;
   const int oc0 = blockIdx.y * a.oct;
   const int hw = a.OH * a.OW;
   const int p0 = tile * a.P;
@@ -93,9 +101,27 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(O
   int8_t* halo = lds + a.off_halo;
   int* sx_lds = reinterpret_cast<int*>(lds + a.off_sx);
 
-  // the reduction order as a table (built once per operator): no index math in the main loop
+  // The reduction order as a table (built once per operator: no index math in the main loop)
+  // and the epilogue's per-channel tables go global -> LDS by DMA here, ahead of the input
+  // loads, and are waited for together with the weights: no memory round trip of their own
+  // stands in front of the halo loads or at the head of the epilogue, and no register is held.
   int2* tap_lds = reinterpret_cast<int2*>(lds + a.off_tap);
-  for (int i = tid; i < a.ksteps * 2 + 2; i += kThreads) tap_lds[i] = a.tapt[i];
+  v4i* rq_lds = reinterpret_cast<v4i*>(lds + a.off_rq);
+  int* bias_lds = reinterpret_cast<int*>(lds + a.off_bias);
+  {
+    typedef const __attribute__((address_space(1))) void* gptr;
+    typedef __attribute__((address_space(3))) void* lptr;
+    const int tap_dwords = (a.ksteps * 2 + 2) * 2;
+    const int* tap_src = reinterpret_cast<const int*>(a.tapt);
+    for (int i = wave * 64; i < tap_dwords; i += kThreads)
+      if (i + lane < tap_dwords)
+        __builtin_amdgcn_global_load_lds((gptr)(tap_src + i + lane), (lptr)(reinterpret_cast<int*>(tap_lds) + i), 4, 0, 0);
+    for (int i = wave * 64; i < a.oct; i += kThreads)  // tables cover the padded channel count
+      if (i + lane < a.oct) {
+        __builtin_amdgcn_global_load_lds((gptr)(a.rq + oc0 + i + lane), (lptr)(rq_lds + i), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr)(a.biasf + oc0 + i + lane), (lptr)(bias_lds + i), 4, 0, 0);
+      }
+  }
   // ---- main loop ---------------------------------------------------------------
   const int frag_row = lane & 31, frag_half = lane >> 5;
   int a_base[kMaxPtw];  // byte offset of each pixel's window origin in the halo tile (+ this lane's half)
@@ -112,16 +138,14 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(O
       a_base[i] = ((oh - r0) * a.sh * a.iwt + ow * a.sw) * a.pix_stride;
     }
   }
-  // accumulators start at the folded bias of the lane's output channel
+  // accumulators start at zero; the folded bias is added in the epilogue
   v16i acc[kMaxPtw][OT];
 #pragma unroll
-  for (int j = 0; j < OT; ++j) {
-    const int bias = a.biasf[oc0 + j * 32 + frag_row];  // tables cover the padded channel count
+  for (int j = 0; j < OT; ++j)
 #pragma unroll
     for (int i = 0; i < kMaxPtw; ++i)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = bias;
-  }
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
   int sx[kMaxPtw] = {0, 0};
 
   // ---- reduction groups: (weights, halo tile) of cp input channels at a time ------------
@@ -147,7 +171,7 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(O
         reinterpret_cast<const uint8_t*>(a.w) + static_cast<size_t>(a.groups) * a.w_group_stride - 256;
     if ((a.W & 3) == 0) {
       // A thread owns one (4 input columns, 4 channels) patch and walks the halo
-      // rows with it, kLoadBatch rows of loads in flight; lanes run over channel
+      // rows with it, a batch of rows of loads in flight; lanes run over channel
       // groups first so that a wavefront's LDS stores spread over the banks.
       const int w4n = a.W / 4;
       const int patches = a.w4_blocks * ((c4n + 3) / 4) * 64;
@@ -184,26 +208,36 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(O
         const int dst0 = __mul24(hc, a.pix_stride) + c;
         // columns of this patch that exist in the halo tile (stride > 1 may cut the right edge)
         const int ncols = min(4, a.iwt - hc);
-        for (int hr0 = 0; hr0 < rows_needed; hr0 += kLoadBatch) {
-          int d[kLoadBatch][4];
+        // A batch of NB halo rows: all loads first, then masks, transposes and stores. The batch
+        // size follows the rows that are left (4, 6 or 8) so that few loads go to rows nobody needs.
+        auto batch = [&](auto nb_tag, int hr0) {
+          constexpr int NB = decltype(nb_tag)::value;
+          int d[NB][4];
+          // Out-of-image rows load row 0 (in bounds) and are replaced by the zero point; the
+          // replacement is a mask operation, not a select: a select on the wavefront-uniform
+          // `inside` would be turned into a branch around the load, and loads under branches
+          // are waited for one by one instead of travelling together. All loads of the batch are
+          // issued before any of them is used (the scheduling fence keeps the compiler from
+          // pulling uses, and with them waits, in between the loads).
 #pragma unroll
-          for (int b = 0; b < kLoadBatch; ++b) {
+          for (int b = 0; b < NB; ++b) {
             const int ih = ih0 + hr0 + b;
             const bool inside = hr0 + b < rows_needed && ih >= 0 && ih < a.H;
             const uint32_t row_off = __umul24(static_cast<uint32_t>(inside ? ih : 0), static_cast<uint32_t>(a.W));
+#pragma unroll
+            for (int j = 0; j < 4; ++j) d[b][j] = *reinterpret_cast<const int*>(src_row[j] + row_off * row_mul[j]);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int b = 0; b < NB; ++b) {
+            const int ih = ih0 + hr0 + b;
+            const bool inside = hr0 + b < rows_needed && ih >= 0 && ih < a.H;
             const int keep = inside ? -1 : 0;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              // out-of-image rows load row 0 (in bounds) and are replaced by the zero point; the
-              // replacement is a mask operation, not a select: a select on the wavefront-uniform
-              // `inside` would be turned into a branch around the load, and loads under branches
-              // are waited for one by one instead of travelling together
-              const int v = *reinterpret_cast<const int*>(src_row[j] + row_off * row_mul[j]);
-              d[b][j] = ((v ^ xmask[j]) & keep) | (fill[j] & ~keep);
-            }
+            for (int j = 0; j < 4; ++j) d[b][j] = ((d[b][j] ^ xmask[j]) & keep) | (fill[j] & ~keep);
           }
 #pragma unroll
-          for (int b = 0; b < kLoadBatch; ++b) {
+          for (int b = 0; b < NB; ++b) {
             if (hr0 + b >= rows_needed) continue;
             // 4 x 4 byte transpose: d[j] = 4 pixels of channel c+j  ->  px[i] = 4 channels of pixel i
             const int lo01 = __builtin_amdgcn_perm(d[b][1], d[b][0], 0x05010400);
@@ -219,6 +253,19 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(O
 #pragma unroll
             for (int i = 0; i < 4; ++i)
               if (i < ncols) *reinterpret_cast<int*>(dst + __mul24(i, a.pix_stride)) = px[i];
+          }
+        };
+        for (int hr0 = 0; hr0 < rows_needed;) {
+          const int left = rows_needed - hr0;
+          if (left > 6) {
+            batch(std::integral_constant<int, 8>{}, hr0);
+            hr0 += 8;
+          } else if (left > 4) {
+            batch(std::integral_constant<int, 6>{}, hr0);
+            hr0 += 6;
+          } else {
+            batch(std::integral_constant<int, 4>{}, hr0);
+            hr0 += 4;
           }
         }
       }
@@ -245,16 +292,18 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(O
         *reinterpret_cast<int*>(halo + HaloOffset(a, hr * a.iwt + a.pad_l + iw, c)) = v;
       }
     }
-    // left / right padding columns: one (halo row, pad column) per step of a thread
+    // left / right padding columns: one 16-channel chunk of a (halo row, pad column) per step of a thread
     {
       const int right0 = a.pad_l + a.W;
       const int pad_cols = a.pad_l + max(a.iwt - right0, 0);
-      const int cells = rows_needed * pad_cols;
-      for (int cell = tid; cell < cells; cell += kThreads) {
+      const int units = rows_needed * pad_cols * a.cpc;
+      for (int u = tid; u < units; u += kThreads) {
+        const int cell = u / a.cpc, c = (u - cell * a.cpc) * 16;
         const int hr = cell / pad_cols, pc = cell - hr * pad_cols;
         const int hc = pc < a.pad_l ? pc : right0 + (pc - a.pad_l);
-        int8_t* dst = halo + (hr * a.iwt + hc) * a.pix_stride;
-        for (int c = 0; c < a.cp; c += 4) *reinterpret_cast<int*>(dst + c) = ChannelFill(a, c, c_real);
+        *reinterpret_cast<v4i*>(halo + (hr * a.iwt + hc) * a.pix_stride + c) =
+            v4i{ChannelFill(a, c, c_real), ChannelFill(a, c + 4, c_real), ChannelFill(a, c + 8, c_real),
+                ChannelFill(a, c + 12, c_real)};
       }
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the weight DMA has landed
@@ -321,7 +370,8 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(O
 #pragma unroll
   for (int j = 0; j < OT; ++j) {
     const int ocl = j * 32 + frag_row;
-    const v4i q = a.rq[oc0 + ocl];
+    const v4i q = rq_lds[ocl];
+    const int bias = bias_lds[ocl];
 #pragma unroll
     for (int i = 0; i < kMaxPtw; ++i) {
       if (i >= n_ptw) continue;
@@ -332,7 +382,7 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(O
         const v4i s4 = *reinterpret_cast<const v4i*>(sx_lds + pl);
         int r4[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) r4[e] = Requant8<RQ>(acc[i][j][g * 4 + e] - s4[e], q, a.out_zp, lo, hi);
+        for (int e = 0; e < 4; ++e) r4[e] = Requant8<RQ>(acc[i][j][g * 4 + e] + (bias - s4[e]), q, a.out_zp, lo, hi);
         *reinterpret_cast<uint32_t*>(out_tile + ocl * a.out_stride + pl) = PackBytes(r4[0], r4[1], r4[2], r4[3]);
       }
     }
@@ -462,11 +512,14 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
     a.w_chunks = w_bytes / 16;
     const int halo_bytes = RoundUp(a.iht * a.iwt * a.pix_stride + 16, 16);
     const int tap_bytes = RoundUp((a.ksteps * 2 + 4) * 8, 16);
+    const int rq_bytes = a.oct * 16, bias_bytes = a.oct * 4;
     // LDS carve-up: the per-pixel sums first; the weight + halo region behind them
     // is reused as the epilogue's staging tile
     a.off_sx = 0;
     a.off_tap = sx_bytes;
-    a.off_w = sx_bytes + tap_bytes;
+    a.off_rq = a.off_tap + tap_bytes;
+    a.off_bias = a.off_rq + rq_bytes;
+    a.off_w = a.off_bias + bias_bytes;
     a.off_halo = a.off_w + w_bytes;
     lds_bytes = a.off_w + std::max(w_bytes + halo_bytes, RoundUp(out_bytes, 16));
     a.groups = (a.C + cp - 1) / cp;
