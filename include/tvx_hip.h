@@ -188,6 +188,24 @@ typedef struct tvx_softmax_desc {
 
 int tvx_softmax_create(const tvx_softmax_desc* desc, tvx_op** op);
 
+/* ---- DataConvert ------------------------------------------------------------------ */
+/* Replaces the DATACONVERT operator (src/tim/vx/ops/simple_operations.cc:39 -> vxTensorCopyNode /
+ * the conversions of src/tim/vx/internal/include/utils/vsi_nn_dtype_util_prv.h:228-266): every
+ * element goes to float32 ((q - zp) * scale, or the float value) and from there to the output
+ * type (rint(f / scale) + zp, saturated to the type's range; rounded to nearest even for
+ * float16). Any pair of the four tensor types. */
+typedef struct tvx_convert_desc {
+  uint64_t count;
+  int32_t in_dtype;
+  float in_scale;
+  int32_t in_zp;
+  int32_t out_dtype;
+  float out_scale;
+  int32_t out_zp;
+} tvx_convert_desc;
+
+int tvx_convert_create(const tvx_convert_desc* desc, tvx_op** op);
+
 /* ---- Transpose (permute) ----------------------------------------------------- */
 /* Replaces the PERMUTE operator (src/tim/vx/ops/transpose.cc -> vxTensorPermuteNode):
  * output dimension i is input dimension perm[i] (out.size[i] = in.size[perm[i]],

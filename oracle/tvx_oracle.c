@@ -463,6 +463,31 @@ void tvxo_softmax(int dtype, int32_t c, int64_t rows, int64_t inner, float beta,
 }
 
 /*
+ * DataConvert (VSI_NN_OP_DATACONVERT; src/tim/vx/ops/simple_operations.cc:39): every element
+ * goes through float32, as in ovxlib's type conversions
+ * (src/tim/vx/internal/include/utils/vsi_nn_dtype_util_prv.h:228-266):
+ *   f = (q - zp) * scale            for a quantized input, the value itself for a float one
+ *   q = sat(rint(f / scale) + zp)   for a quantized output (round half to even)
+ */
+void tvxo_convert(int in_dtype, int64_t count, const void* x, float in_scale, int32_t in_zp,
+                  int out_dtype, void* y, float out_scale, int32_t out_zp) {
+  const int in_q = in_dtype == TVXO_U8 || in_dtype == TVXO_I8;
+  const int out_q = out_dtype == TVXO_U8 || out_dtype == TVXO_I8;
+  const double qmin = out_dtype == TVXO_U8 ? 0 : -128, qmax = out_dtype == TVXO_U8 ? 255 : 127;
+  for (int64_t i = 0; i < count; ++i) {
+    const float f = in_q ? ((float)load_q(x, in_dtype, i) - (float)in_zp) * in_scale : load_f(x, in_dtype, i);
+    if (out_q) {
+      double r = (double)rintf(f / out_scale) + (double)out_zp;
+      r = r < qmin ? qmin : (r > qmax ? qmax : r);
+      if (r != r) r = qmin;
+      store_q(y, out_dtype, i, (int64_t)r);
+    } else {
+      store_f(y, out_dtype, i, f);
+    }
+  }
+}
+
+/*
  * Transpose (PERMUTE): output dimension i is input dimension perm[i], dimension 0 fastest
  * (src/tim/vx/internal/src/ops/vsi_nn_op_permute.c:219-230 sizes the output as
  * out.size[i] = in.size[perm[i]]; src/tim/vx/ops/transpose_test.cc:29-100). Elements are

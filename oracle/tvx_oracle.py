@@ -68,6 +68,9 @@ def lib():
                                          C.c_void_p, C.c_float, C.c_int32]
         _lib.tvxo_add.argtypes = [C.c_int, C.c_int64, C.c_void_p, C.c_float, C.c_int32, C.c_void_p,
                                   C.c_float, C.c_int32, C.c_void_p, C.c_float, C.c_int32]
+        _lib.tvxo_convert.argtypes = [C.c_int, C.c_int64, C.c_void_p, C.c_float, C.c_int32, C.c_int, C.c_void_p,
+                                      C.c_float, C.c_int32]
+        _lib.tvxo_convert.restype = None
         _lib.tvxo_transpose.argtypes = [C.c_int32, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32), C.c_int32,
                                         C.c_void_p, C.c_void_p]
         _lib.tvxo_transpose.restype = None
@@ -199,6 +202,17 @@ def softmax(dtype, x, c, beta, in_q, inner=1):
 # --------------------------------------------------------------------------
 # fixture cases
 # --------------------------------------------------------------------------
+NP_OF_CODE = {U8: np.uint8, I8: np.int8, F16: np.float16, F32: np.float32}
+
+
+def convert(x, in_dtype, in_q, out_dtype, out_q):
+    """DataConvert: element -> float32 -> output type (quantize / dequantize / requantize)."""
+    x = np.ascontiguousarray(x).reshape(-1)
+    y = np.zeros(x.size, dtype=NP_OF_CODE[out_dtype])
+    lib().tvxo_convert(in_dtype, x.size, _ptr(x), in_q[0], in_q[1], out_dtype, _ptr(y), out_q[0], out_q[1])
+    return y
+
+
 def transpose(x, in_dims, perm):
     """Output dimension i is input dimension perm[i] (dimension 0 fastest); x is the flat input."""
     x = np.ascontiguousarray(x).reshape(-1)
@@ -276,6 +290,10 @@ def run_case(case):
         return softmax(DTYPE_CODE[x["dtype"]], arr[0], c, a.get("beta", 1.0), (s, z), inner)
     if op["kind"] == "TRANSPOSE":
         return transpose(arr[0], ins[0]["shape"], a["perm"])
+    if op["kind"] == "DATACONVERT":
+        s, z, _ = _q(ins[0]["quant"])
+        so, zo, _ = _q(out["quant"])
+        return convert(arr[0], DTYPE_CODE[ins[0]["dtype"]], (s, z), DTYPE_CODE[out["dtype"]], (so, zo))
     raise NotImplementedError(op["kind"])
 
 
@@ -339,6 +357,8 @@ def run_graph(graph, keep_all=False):
             y = xv
         elif k == "TRANSPOSE":
             y = transpose(xv, x["shape"], a["perm"])
+        elif k == "DATACONVERT":
+            y = convert(xv, DTYPE_CODE[x["dtype"]], (s, z), DTYPE_CODE[out["dtype"]], (so, zo))
         else:
             raise NotImplementedError(k)
         val[out["id"]] = y

@@ -206,6 +206,19 @@ Sink Check(bool ok, const char* expr) {
   return Sink();
 }
 
+std::vector<double> g_near;
+void RecordGolden(const std::vector<double>& golden, double tol, const char* how);
+Sink RecordNear(double golden, double tol) {
+  g_near.push_back(golden);
+  // the graph is alive only inside the test body: emit as soon as every output element has its scalar
+  if (g_last_graph && !g_compile_failed && g_last_graph->outputs_tensor_.size() == 1 &&
+      static_cast<int64_t>(g_near.size()) == g_last_graph->outputs_tensor_[0]->GetSpec().GetElementNum()) {
+    RecordGolden(g_near, tol, "near");
+    g_near.clear();
+  }
+  return Sink();
+}
+
 void RecordGolden(const std::vector<double>& golden, double tol, const char* how) {
   if (!g_last_graph || g_compile_failed) {
     std::fprintf(stderr, "  [%s] no compiled graph: case skipped\n", g_current.c_str());
@@ -262,6 +275,7 @@ int main(int argc, char** argv) {
     g_case_in_test = 0;
     g_last_graph = nullptr;
     g_compile_failed = false;
+    tvxcap::g_near.clear();
     t.body();
     g_last_graph = nullptr;
     std::fprintf(stderr, "%s: %d case(s)\n", g_current.c_str(), g_case_in_test);

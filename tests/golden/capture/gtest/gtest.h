@@ -32,6 +32,9 @@ Sink RecordEq(const std::vector<T>& golden, const std::vector<T>&) {
 template <typename A, typename B>
 Sink RecordEq(const A&, const B&) { return Sink(); }
 Sink Check(bool ok, const char* expr);
+// EXPECT_NEAR(golden[i], output[i], tol) in a loop over the output: the scalars are gathered and
+// become one case when the test body ends, if there is one of them per output element.
+Sink RecordNear(double golden, double tol);
 }  // namespace tvxcap
 
 namespace testing {
@@ -56,5 +59,5 @@ inline Matcher<float> FloatNear(float, float) { return Matcher<float>(); }
 #define EXPECT_TRUE(x) ::tvxcap::Check(static_cast<bool>(x), #x)
 #define ASSERT_TRUE(x) ::tvxcap::Check(static_cast<bool>(x), #x)
 #define EXPECT_EQ(a, b) ::tvxcap::RecordEq((a), (b))
-#define EXPECT_NEAR(a, b, t) ::tvxcap::Sink()
+#define EXPECT_NEAR(a, b, t) ::tvxcap::RecordNear(static_cast<double>(a), static_cast<double>(static_cast<float>(t)))
 #define GTEST_SKIP() return

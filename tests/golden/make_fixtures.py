@@ -13,6 +13,7 @@ Needs /root/reference (present only in the build container); the committed
 JSON files are what the test-suite reads.
 """
 import os
+import re
 import subprocess
 import sys
 
@@ -31,7 +32,34 @@ SOURCES = {
     "avg_pool": "src/tim/vx/ops/avg_pool_test.cc",
     "softmax": "src/tim/vx/ops/softmax_test.cc",
     "transpose": "src/tim/vx/ops/transpose_test.cc",
+    # (file, test suite): only the TEST(suite, ...) bodies of a file that also tests operators outside this path
+    "dataconvert": ("src/tim/vx/ops/simple_operations_test.cc", "DataConvert"),
 }
+
+
+def select_suite(path, suite):
+    """The file's preprocessor lines plus the TEST(suite, ...) bodies, as text for the compiler's stdin
+    (nothing of the reference is written to disk)."""
+    text = open(path).read()
+    out = [l for l in text.splitlines() if l.startswith("#include")]
+    pos = 0
+    while True:
+        m = re.search(r"^TEST\(\s*%s\s*,[^)]*\)\s*\{" % re.escape(suite), text[pos:], re.M)
+        if not m:
+            break
+        start = pos + m.start()
+        depth, i = 0, pos + m.end() - 1
+        while True:
+            if text[i] == "{":
+                depth += 1
+            elif text[i] == "}":
+                depth -= 1
+                if depth == 0:
+                    break
+            i += 1
+        out.append(text[start:i + 1])
+        pos = i + 1
+    return "\n".join(out) + "\n"
 
 
 def main():
@@ -48,10 +76,14 @@ def main():
     host = [os.path.join(PKG, "src", f) for f in ("frontend.cc", "graph_passes.cc")]
     for name, rel in SOURCES.items():
         exe = os.path.join(build, "capture_" + name)
-        cmd = common + [os.path.join(REF, rel),
-                        os.path.join(HERE, "capture", "capture_main.cc")] + host + ["-o", exe]
+        rest = [os.path.join(HERE, "capture", "capture_main.cc")] + host + ["-o", exe]
         print("building", name, flush=True)
-        subprocess.check_call(cmd)
+        if isinstance(rel, tuple):
+            path = os.path.join(REF, rel[0])
+            cmd = common + ["-I", os.path.dirname(path), "-x", "c++", "-", "-x", "none"] + rest
+            subprocess.run(cmd, input=select_suite(path, rel[1]).encode(), check=True)
+        else:
+            subprocess.check_call(common + [os.path.join(REF, rel)] + rest)
         out = os.path.join(HERE, name + ".json")
         subprocess.check_call([exe, out])
         print("wrote", out, os.path.getsize(out), "bytes", flush=True)

@@ -491,3 +491,23 @@ def test_transpose_rejects_bad_descriptors():
             d.in_dims[i], d.perm[i] = 2, perm[i]
         with pytest.raises(T.TvxError):
             T.transpose_create(d)
+
+
+@pytest.mark.parametrize("in_dtype,out_dtype", [(i, o) for i in range(4) for o in range(4)])
+def test_dataconvert(oracle, in_dtype, out_dtype):
+    # every pair of the four tensor types, 100003 elements incl. ties, saturation and all 8-bit codes
+    rng = np.random.default_rng(in_dtype * 4 + out_dtype)
+    n = 100003
+    in_q = (0.037, 121 if in_dtype == 0 else -5) if in_dtype < 2 else (1.0, 0)
+    out_q = (0.052, 117 if out_dtype == 0 else 9) if out_dtype < 2 else (1.0, 0)
+    if in_dtype < 2:
+        x = rand_q(rng, n, in_dtype)
+    else:
+        x = (rng.standard_normal(n) * 4).astype(np.float32)
+        x[:64] = (np.arange(64) - 32) * np.float32(0.026)   # exact half-steps of the output scale
+        x[64:68] = [1e6, -1e6, 0.0, -0.0]
+        with np.errstate(over="ignore"):
+            x = x.astype(TC.NP_OF[in_dtype])   # 1e6 becomes inf in float16, on purpose
+    want = oracle.convert(x, in_dtype, in_q, out_dtype, out_q)
+    got = TC.gpu_convert(x, in_dtype, in_q, out_dtype, out_q)
+    assert np.array_equal(got.view(np.uint8), want.view(np.uint8))   # bit-exact, floats included

@@ -223,3 +223,26 @@ def test_transpose_restatement_vs_numpy(oracle, in_dims, perm):
         c = (3, 1, 1)                                     # input offset 3 + 4*1 + 12*1 = 19
         o = (c[2], c[0], c[1])                            # output offset 1 + 2*3 + 8*1 = 15
         assert y[o[0] + 2 * o[1] + 8 * o[2]] == 19
+
+
+def test_convert_restatement_vs_numpy(oracle):
+    # quantize: rint(f / scale) + zp with round-half-even and saturation (vsi_nn_dtype_util_prv.h:228-252)
+    f = np.array([0.0, 0.25, 0.75, 1.25, -0.25, -0.75, 63.0, 1000.0, -1000.0, 0.1, np.float32(0.3)], dtype=np.float32)
+    want = np.clip(np.rint(f / np.float32(0.5)) + 3, 0, 255).astype(np.uint8)          # numpy rint = half to even
+    assert list(want[:6]) == [3, 3, 5, 5, 3, 1]                                       # ties 0.5, 1.5, 2.5, -0.5, -1.5
+    assert np.array_equal(oracle.convert(f, 3, (1.0, 0), 0, (0.5, 3)), want)
+    want_i8 = np.clip(np.rint(f / np.float32(0.5)) - 3, -128, 127).astype(np.int8)
+    assert np.array_equal(oracle.convert(f, 3, (1.0, 0), 1, (0.5, -3)), want_i8)
+    # dequantize: (q - zp) * scale in float32, all 256 codes
+    q = np.arange(256, dtype=np.uint8)
+    got = oracle.convert(q, 0, (np.float32(0.0036), 7), 3, (1.0, 0))
+    assert np.array_equal(got, (q.astype(np.float32) - np.float32(7)) * np.float32(0.0036))
+    # requantize with equal scales is a shift of the zero point with saturation
+    assert np.array_equal(oracle.convert(q, 0, (0.25, 0), 0, (0.25, 10)), np.minimum(q.astype(np.int32) + 10, 255))
+    # uint8 <-> int8 with the zero point moved by 128 is the identity on the real values
+    i8 = oracle.convert(q, 0, (0.1, 128), 1, (0.1, 0))
+    assert np.array_equal(i8.astype(np.int32), q.astype(np.int32) - 128)
+    # float16 output rounds to nearest even like numpy's cast; float16 input widens exactly
+    h = oracle.convert(f, 3, (1.0, 0), 2, (1.0, 0))
+    assert np.array_equal(h.view(np.uint16), f.astype(np.float16).view(np.uint16))
+    assert np.array_equal(oracle.convert(h, 2, (1.0, 0), 3, (1.0, 0)), h.astype(np.float32))

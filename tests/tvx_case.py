@@ -11,7 +11,7 @@ import tvx_oracle as O
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 GOLDEN_FILES = ["conv2d", "depthwise_conv", "grouped_conv2d", "conv1d", "fullyconnected", "max_pool", "avg_pool", "softmax",
-                "transpose"]
+                "transpose", "dataconvert"]
 
 
 def load_cases(name):
@@ -205,6 +205,21 @@ def gpu_softmax(dtype, x, c, beta, in_q, inner=1):
     return yd.cpu().numpy()
 
 
+def gpu_convert(x, in_dtype, in_q, out_dtype, out_q):
+    T = tvx()
+    d = T.ConvertDesc()
+    d.count, d.in_dtype, d.out_dtype = x.size, in_dtype, out_dtype
+    d.in_scale, d.in_zp = in_q
+    d.out_scale, d.out_zp = out_q
+    op = T.convert_create(d)
+    import torch
+    xd = to_device(x)
+    yd = device_out(x.size, NP_OF[out_dtype])
+    op.run(xd, None, yd)
+    torch.cuda.synchronize()
+    return yd.cpu().numpy()
+
+
 def gpu_transpose(x, in_dims, perm):
     T = tvx()
     d = T.TransposeDesc()
@@ -266,4 +281,8 @@ def run_case_gpu(case):
         return gpu_softmax(code[x["dtype"]], arr[0], c, a.get("beta", 1.0), (s, z), inner)
     if op["kind"] == "TRANSPOSE":
         return gpu_transpose(arr[0], ins[0]["shape"], a["perm"])
+    if op["kind"] == "DATACONVERT":
+        s, z, _ = O._q(ins[0]["quant"])
+        so, zo, _ = O._q(out["quant"])
+        return gpu_convert(arr[0], code[ins[0]["dtype"]], (s, z), code[out["dtype"]], (so, zo))
     raise NotImplementedError(op["kind"])

@@ -56,6 +56,11 @@ class SoftmaxDesc(C.Structure):
                 ("in_dtype", C.c_int32), ("in_scale", C.c_float), ("in_zp", C.c_int32), ("inner", C.c_uint64)]
 
 
+class ConvertDesc(C.Structure):
+    _fields_ = [("count", C.c_uint64), ("in_dtype", C.c_int32), ("in_scale", C.c_float), ("in_zp", C.c_int32),
+                ("out_dtype", C.c_int32), ("out_scale", C.c_float), ("out_zp", C.c_int32)]
+
+
 class TransposeDesc(C.Structure):
     _fields_ = [("rank", C.c_uint32), ("in_dims", C.c_uint32 * 6), ("perm", C.c_uint32 * 6),
                 ("elem_bytes", C.c_uint32)]
@@ -112,6 +117,7 @@ def lib():
         L.tvx_activation_create.argtypes = [C.POINTER(EltwiseDesc), C.POINTER(vp)]
         L.tvx_add_create.argtypes = [C.POINTER(EltwiseDesc), C.POINTER(vp)]
         L.tvx_softmax_create.argtypes = [C.POINTER(SoftmaxDesc), C.POINTER(vp)]
+        L.tvx_convert_create.argtypes = [C.POINTER(ConvertDesc), C.POINTER(vp)]
         L.tvx_transpose_create.argtypes = [C.POINTER(TransposeDesc), C.POINTER(vp)]
         L.tvx_op_run.argtypes = [vp, vp, vp, vp, vp]
         L.tvx_calibrate_mfma_i8.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_double)]
@@ -195,6 +201,12 @@ def add_create(desc):
 def softmax_create(desc):
     h = C.c_void_p()
     check(lib().tvx_softmax_create(C.byref(desc), C.byref(h)))
+    return Op(h)
+
+
+def convert_create(desc):
+    h = C.c_void_p()
+    check(lib().tvx_convert_create(C.byref(desc), C.byref(h)))
     return Op(h)
 
 

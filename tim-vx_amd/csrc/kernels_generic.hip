@@ -1,6 +1,8 @@
 // Generic kernels: one thread per output element, any shape / stride /
 // dilation / padding / multiplier, every supported dtype. They are the
 // variant of last resort and the on-GPU cross-check for the tuned variants.
+#include <type_traits>
+
 #include "variants.h"
 
 namespace tvx {
@@ -665,6 +667,65 @@ int TransposeRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_
   return TVX_OK;
 }
 
+// ---------------------------------------------------------------------------
+// DataConvert: element -> float32 -> output type, one thread per element
+// ---------------------------------------------------------------------------
+struct ConvertArgs {
+  float in_scale, out_scale;
+  int in_zp, out_zp;
+};
+
+template <typename TI>
+__device__ __forceinline__ float ConvertLoad(const TI* x, uint64_t i, const ConvertArgs& a) {
+  if constexpr (std::is_same<TI, uint8_t>::value || std::is_same<TI, int8_t>::value)
+    return (static_cast<float>(static_cast<int>(x[i])) - static_cast<float>(a.in_zp)) * a.in_scale;
+  else
+    return ToFloat(x[i]);
+}
+
+template <typename TI, typename TO>
+__global__ void __launch_bounds__(kBlock)
+ConvertKernel(ConvertArgs a, const TI* __restrict__ x, TO* __restrict__ y, uint64_t total) {
+  const uint64_t idx = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
+  if (idx >= total) return;
+  const float f = ConvertLoad(x, idx, a);
+  if constexpr (std::is_same<TO, uint8_t>::value || std::is_same<TO, int8_t>::value) {
+    const float lo = std::is_same<TO, uint8_t>::value ? 0.f : -128.f, hi = std::is_same<TO, uint8_t>::value ? 255.f : 127.f;
+    // saturate in float (a NaN becomes the lower bound), then the conversion is exact
+    float r = rintf(__fdiv_rn(f, a.out_scale)) + static_cast<float>(a.out_zp);
+    r = fminf(fmaxf(r, lo), hi);
+    y[idx] = static_cast<TO>(static_cast<int>(r));
+  } else {
+    FromFloat(f, &y[idx]);
+  }
+}
+
+template <typename TI>
+void ConvertLaunchOut(const tvx_convert_desc& d, const ConvertArgs& a, const void* in0, void* out, hipStream_t st) {
+  const dim3 grid(Blocks(d.count)), block(kBlock);
+  const TI* x = static_cast<const TI*>(in0);
+  switch (d.out_dtype) {
+    case TVX_U8: hipLaunchKernelGGL((ConvertKernel<TI, uint8_t>), grid, block, 0, st, a, x, static_cast<uint8_t*>(out), d.count); break;
+    case TVX_I8: hipLaunchKernelGGL((ConvertKernel<TI, int8_t>), grid, block, 0, st, a, x, static_cast<int8_t*>(out), d.count); break;
+    case TVX_F16: hipLaunchKernelGGL((ConvertKernel<TI, __half>), grid, block, 0, st, a, x, static_cast<__half*>(out), d.count); break;
+    default: hipLaunchKernelGGL((ConvertKernel<TI, float>), grid, block, 0, st, a, x, static_cast<float*>(out), d.count); break;
+  }
+}
+
+int ConvertRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
+  const tvx_convert_desc& d = op->cv;
+  if (!d.count) return TVX_OK;
+  const ConvertArgs a{d.in_scale, d.out_scale, d.in_zp, d.out_zp};
+  switch (d.in_dtype) {
+    case TVX_U8: ConvertLaunchOut<uint8_t>(d, a, in0, out, st); break;
+    case TVX_I8: ConvertLaunchOut<int8_t>(d, a, in0, out, st); break;
+    case TVX_F16: ConvertLaunchOut<__half>(d, a, in0, out, st); break;
+    default: ConvertLaunchOut<float>(d, a, in0, out, st); break;
+  }
+  TVX_HIP_CHECK(hipGetLastError());
+  return TVX_OK;
+}
+
 int UploadWeightsAndBias(tvx_op* op, const void* w, size_t w_bytes, const void* b, size_t b_bytes) {
   int s = TVX_OK;
   if (w) s = op->weights.Upload(w, w_bytes);
@@ -733,6 +794,12 @@ int AddSetup(tvx_op* op) {
   op->geo[2] = op->quantized && ra < 1048576.0 && rb < 1048576.0 ? 1 : 0;
   op->run = AddRun;
   op->kernel_name = "add_generic";
+  return TVX_OK;
+}
+
+int ConvertSetup(tvx_op* op) {
+  op->run = ConvertRun;
+  op->kernel_name = "convert_generic";
   return TVX_OK;
 }
 

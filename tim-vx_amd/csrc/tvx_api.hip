@@ -430,6 +430,25 @@ int tvx_softmax_create(const tvx_softmax_desc* d, tvx_op** out) {
   return TVX_OK;
 }
 
+int tvx_convert_create(const tvx_convert_desc* d, tvx_op** out) {
+  if (!d || !out) return SetError(TVX_E_INVALID, "tvx_convert_create: null argument");
+  *out = nullptr;
+  if (!ValidDtype(d->in_dtype) || !ValidDtype(d->out_dtype))
+    return SetError(TVX_E_INVALID, "tvx_convert_create: unknown dtype");
+  if ((IsQuant(d->in_dtype) && !(d->in_scale > 0.f)) || (IsQuant(d->out_dtype) && !(d->out_scale > 0.f)))
+    return SetError(TVX_E_INVALID, "tvx_convert_create: a quantized tensor needs a positive scale");
+  int s = NoGpu();
+  if (s != TVX_OK) return s;
+  tvx_op* op = new (std::nothrow) tvx_op();
+  if (!op) return SetError(TVX_E_NOMEM, "tvx_convert_create: host allocation failed");
+  op->kind = OP_CONVERT;
+  op->cv = *d;
+  s = ConvertSetup(op);
+  if (s != TVX_OK) { delete op; return s; }
+  *out = op;
+  return TVX_OK;
+}
+
 int tvx_transpose_create(const tvx_transpose_desc* d, tvx_op** out) {
   if (!d || !out) return SetError(TVX_E_INVALID, "tvx_transpose_create: null argument");
   *out = nullptr;

@@ -24,7 +24,7 @@ int SetError(int status, const char* fmt, ...);
                              hipGetErrorString(e_), __FILE__, __LINE__);        \
   } while (0)
 
-enum OpKind { OP_CONV2D = 1, OP_FC, OP_POOL2D, OP_ACTIVATION, OP_ADD, OP_SOFTMAX, OP_TRANSPOSE };
+enum OpKind { OP_CONV2D = 1, OP_FC, OP_POOL2D, OP_ACTIVATION, OP_ADD, OP_SOFTMAX, OP_TRANSPOSE, OP_CONVERT };
 
 // Device buffer owned by an operator, released in its destructor.
 struct DeviceBuffer {
@@ -53,6 +53,7 @@ struct tvx_op {
   tvx_eltwise_desc elt{};
   tvx_softmax_desc sm{};
   tvx_transpose_desc tr{};
+  tvx_convert_desc cv{};
 
   bool quantized = false;
   bool has_const_weights = false;

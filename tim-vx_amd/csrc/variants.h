@@ -45,5 +45,6 @@ int ConvGenericSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 int FcGenericSetup(tvx_op*, const tvx_fc_desc*, const void*, const void*);
 int PoolGenericSetup(tvx_op*);
 int TransposeSetup(tvx_op*);
+int ConvertSetup(tvx_op*);
 
 }  // namespace tvx

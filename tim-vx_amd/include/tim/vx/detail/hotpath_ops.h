@@ -257,6 +257,15 @@ class Reshape : public BuiltinOp {
   std::vector<uint32_t> size_;
 };
 
+// reference: include/tim/vx/ops/simple_operations.h:118 (DataConvert only)
+// Converts between tensor types and quantizations: quantize, dequantize, requantize.
+class DataConvert : public BuiltinOp {
+ public:
+  DataConvert(Graph* graph);
+  std::shared_ptr<Operation> Clone(
+      std::shared_ptr<Graph>& graph) const override;
+};
+
 // reference: include/tim/vx/ops/transpose.h
 // Output dimension i is input dimension perm[i], dimension 0 fastest.
 class Transpose : public BuiltinOp {

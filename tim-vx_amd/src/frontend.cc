@@ -36,6 +36,7 @@ const char* OpKindName(OpKind k) {
     case OpKind::SOFTMAX: return "SOFTMAX";
     case OpKind::RESHAPE: return "RESHAPE";
     case OpKind::TRANSPOSE: return "TRANSPOSE";
+    case OpKind::DATACONVERT: return "DATACONVERT";
   }
   return "?";
 }
@@ -992,6 +993,11 @@ Reshape::Reshape(Graph* graph, const std::vector<uint32_t>& target_shape)
 }
 std::shared_ptr<Operation> Reshape::Clone(std::shared_ptr<Graph>& graph) const {
   return graph->CreateOperation<Reshape>(size_);
+}
+
+DataConvert::DataConvert(Graph* graph) : BuiltinOp(graph, K(OpKind::DATACONVERT), 1, 1) {}
+std::shared_ptr<Operation> DataConvert::Clone(std::shared_ptr<Graph>& graph) const {
+  return graph->CreateOperation<DataConvert>();
 }
 
 Transpose::Transpose(Graph* graph, const std::vector<uint32_t>& perm)

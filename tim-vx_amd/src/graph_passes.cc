@@ -419,6 +419,7 @@ bool GraphImpl::VerifyAndInfer() {
       case OpKind::SOFTMAX: ok = SetupSameShape(im, "SOFTMAX", 1); break;
       case OpKind::RESHAPE: ok = SetupReshape(im); break;
       case OpKind::TRANSPOSE: ok = SetupTranspose(im); break;
+      case OpKind::DATACONVERT: ok = SetupSameShape(im, "DATACONVERT", 1); break;
     }
     if (!ok) {
       VSILOGE("setup of %s (uid %u) failed", OpKindName(im->kind_), im->uid_);

@@ -125,6 +125,7 @@ class HipExecutor : public Executor {
         case OpKind::SOFTMAX: ok = AddSoftmax(im, out); break;
         case OpKind::RESHAPE: break;  // aliased
         case OpKind::TRANSPOSE: ok = AddTranspose(im, out); break;
+        case OpKind::DATACONVERT: ok = AddConvert(im, out); break;
       }
       if (!ok) return false;
     }
@@ -372,6 +373,23 @@ class HipExecutor : public Executor {
     d.in_scale = ScaleOf(x->spec_); d.in_zp = ZpOf(x->spec_);
     tvx_op* op = nullptr;
     if (tvx_softmax_create(&d, &op) != TVX_OK) return Fail("tvx_softmax_create");
+    Push(op, im, x, nullptr, out);
+    return true;
+  }
+
+  bool AddConvert(OpImpl* im, TensorImpl* out) {
+    TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
+    const int in_code = DtypeCode(x->spec_.datatype_), out_code = DtypeCode(out->spec_.datatype_);
+    if (in_code < 0 || out_code < 0) {
+      VSILOGE("DATACONVERT: UINT8, INT8, FLOAT16 and FLOAT32 tensors are what is implemented");
+      return false;
+    }
+    tvx_convert_desc d{};
+    d.count = static_cast<uint64_t>(x->spec_.GetElementNum());
+    d.in_dtype = in_code; d.in_scale = ScaleOf(x->spec_); d.in_zp = ZpOf(x->spec_);
+    d.out_dtype = out_code; d.out_scale = ScaleOf(out->spec_); d.out_zp = ZpOf(out->spec_);
+    tvx_op* op = nullptr;
+    if (tvx_convert_create(&d, &op) != TVX_OK) return Fail("tvx_convert_create");
     Push(op, im, x, nullptr, out);
     return true;
   }

@@ -32,7 +32,7 @@ int TvxLogThreshold();
 #define VSILOGD(...) TVX_LOG(::tim::vx::TVX_LOG_DEBUG, "D ", __VA_ARGS__)
 
 enum class OpKind : uint32_t {
-  CONV2D = 1, FCL, POOL, RELU, RELU6, ADD, SOFTMAX, RESHAPE, TRANSPOSE
+  CONV2D = 1, FCL, POOL, RELU, RELU6, ADD, SOFTMAX, RESHAPE, TRANSPOSE, DATACONVERT
 };
 const char* OpKindName(OpKind k);
 

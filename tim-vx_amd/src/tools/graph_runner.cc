@@ -200,6 +200,8 @@ int main(int argc, char** argv) {
         op = graph->CreateOperation<ops::Softmax>(beta, sm_axis);
       } else if (kind == "RESHAPE") {
         op = graph->CreateOperation<ops::Reshape>(new_shape);
+      } else if (kind == "DATACONVERT") {
+        op = graph->CreateOperation<ops::DataConvert>();
       } else if (kind == "TRANSPOSE") {
         op = graph->CreateOperation<ops::Transpose>(perm);
       } else {
