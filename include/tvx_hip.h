@@ -226,6 +226,12 @@ int tvx_transpose_create(const tvx_transpose_desc* desc, tvx_op** op);
  * weights) or the second Add operand, else NULL; out: result. All device
  * pointers, sized by the operator's descriptor. */
 int tvx_op_run(tvx_op* op, const void* in0, const void* in1, void* out, void* stream);
+/* The same with a third operand: the bias of a Conv2d / FullyConnected whose weights are given
+ * at run time too (created with weights_host == NULL and bias_host == NULL), int32 for quantized
+ * tensors, float32 otherwise. This is the reference's convolution whose weight and bias tensors
+ * are graph inputs (src/tim/transform/layout_inference_test.cc:65-121). in2 == NULL is
+ * tvx_op_run. */
+int tvx_op_run3(tvx_op* op, const void* in0, const void* in1, const void* in2, void* out, void* stream);
 /* Name of the kernel variant chosen at creation, e.g. "conv2d_generic". */
 const char* tvx_op_kernel_name(const tvx_op* op);
 void tvx_op_destroy(tvx_op* op);

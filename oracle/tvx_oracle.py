@@ -115,6 +115,33 @@ def _conv_shapes(a, x_shape, w_shape, out_shape):
 
 
 
+ACT_TO_WHCN = {"CWHN": [1, 2, 0, 3]}                      # activation layouts other than WHCN
+ACT_FROM_WHCN = {"CWHN": [2, 0, 1, 3]}
+KERNEL_TO_WHICOC = {"IcWHOc": [1, 2, 0, 3], "OcIcWH": [2, 3, 1, 0], "IcOcWH": [2, 3, 0, 1]}
+
+
+def _permuted(shape, perm):
+    return [shape[p] for p in perm]
+
+
+def _resolved_pad(a, in_shape, w_shape):
+    """Explicit {left, right, top, bottom} of a conv / pool: AUTO keeps the operator's own numbers,
+    VALID pads nothing, SAME makes out = ceil(in / stride) with the smaller half in front
+    (src/tim/vx/internal/src/utils/vsi_nn_util.c:221-235, 513-553)."""
+    if a["pad_type"] in ("AUTO", "NONE"):
+        return list(a["pad"])
+    if a["pad_type"] == "VALID":
+        return [0, 0, 0, 0]
+    pad = []
+    for ax in (0, 1):
+        dil = a["dilation"][ax] or 1
+        ke = (w_shape[ax] - 1) * dil + 1
+        out = -(-in_shape[ax] // a["stride"][ax])
+        total = max((out - 1) * a["stride"][ax] + ke - in_shape[ax], 0)
+        pad += [total // 2, total - total // 2]
+    return pad
+
+
 def conv2d(x, w, bias, *, in_shape, w_shape, out_shape, stride, dilation, pad_left, pad_top,
            multiplier, in_dtype, w_dtype, out_dtype, in_q=(1.0, 0), w_q=(1.0, 0, None),
            out_q=(1.0, 0), act=ACT_NONE, groups=0):
@@ -244,8 +271,9 @@ def pad4(shape):
 
 def run_case(case):
     """Run a one-operator fixture graph through the oracle; returns the flat output array."""
+    if case.get("layout_inference") or len(case["ops"]) > 1:
+        return run_graph(case)  # a source graph as the front end states it: layouts, unresolved pads
     tensors = {t["id"]: t for t in case["tensors"]}
-    assert len(case["ops"]) == 1, "fixtures hold single-operator graphs"
     op = case["ops"][0]
     a = op["attrs"]
     ins = [tensors[i] for i in op["inputs"]]
@@ -322,13 +350,25 @@ def run_graph(graph, keep_all=False):
         if k == "CONV2D":
             w = ins[1]
             bias = val[ins[2]["id"]] if len(ins) > 2 and ins[2] is not None else None
-            xs, wsh, osh = _conv_shapes(a, x["shape"], w["shape"], out["shape"])
-            y = conv2d(xv, val[w["id"]], bias, in_shape=xs, w_shape=wsh,
-                       out_shape=osh, stride=a["stride"], dilation=a["dilation"],
-                       pad_left=a["pad"][0], pad_top=a["pad"][2], multiplier=a["multiplier"], groups=a.get("groups", 0),
+            # operands in another layout are brought to WHCN / WHIcOc, the result is taken back
+            lay, klay = a.get("layout", "ANY"), a.get("kernel_layout", "ANY")
+            xshape, wshape, oshape, wv = x["shape"], w["shape"], out["shape"], val[w["id"]]
+            if lay in ACT_TO_WHCN:
+                xv = transpose(xv, xshape, ACT_TO_WHCN[lay])
+                xshape, oshape = _permuted(xshape, ACT_TO_WHCN[lay]), _permuted(oshape, ACT_TO_WHCN[lay])
+            if klay in KERNEL_TO_WHICOC:
+                wv = transpose(wv, wshape, KERNEL_TO_WHICOC[klay])
+                wshape = _permuted(wshape, KERNEL_TO_WHICOC[klay])
+            xs, wsh, osh = _conv_shapes(a, xshape, wshape, oshape)
+            pad = _resolved_pad(a, xs, wsh)
+            y = conv2d(xv, wv, bias, in_shape=xs, w_shape=wsh,
+                       out_shape=osh, stride=a["stride"], dilation=[d or 1 for d in a["dilation"]],
+                       pad_left=pad[0], pad_top=pad[2], multiplier=a["multiplier"], groups=a.get("groups", 0),
                        in_dtype=DTYPE_CODE[x["dtype"]], w_dtype=DTYPE_CODE[w["dtype"]],
                        out_dtype=DTYPE_CODE[out["dtype"]], in_q=(s, z), w_q=_q(w["quant"]),
                        out_q=(so, zo))
+            if lay in ACT_FROM_WHCN:
+                y = transpose(y, oshape, ACT_FROM_WHCN[lay])
         elif k == "FCL":
             w = ins[1]
             bias = val[ins[2]["id"]] if len(ins) > 2 and ins[2] is not None else None
@@ -339,10 +379,18 @@ def run_graph(graph, keep_all=False):
                                 out_dtype=DTYPE_CODE[out["dtype"]], in_q=(s, z),
                                 w_q=_q(w["quant"]), out_q=(so, zo))
         elif k == "POOL":
-            y = pool2d(xv, in_shape=pad4(x["shape"]), out_shape=pad4(out["shape"]),
-                       ksize=a["ksize"], stride=a["stride"], pad_left=a["pad"][0],
-                       pad_top=a["pad"][2], pool_type=POOL[a["pool_type"]],
+            lay = a.get("layout", "ANY")
+            xshape, oshape = x["shape"], out["shape"]
+            if lay in ACT_TO_WHCN:
+                xv = transpose(xv, xshape, ACT_TO_WHCN[lay])
+                xshape, oshape = _permuted(xshape, ACT_TO_WHCN[lay]), _permuted(oshape, ACT_TO_WHCN[lay])
+            pad = _resolved_pad(dict(a, dilation=[1, 1]), pad4(xshape), a["ksize"])
+            y = pool2d(xv, in_shape=pad4(xshape), out_shape=pad4(oshape),
+                       ksize=a["ksize"], stride=a["stride"], pad_left=pad[0],
+                       pad_top=pad[2], pool_type=POOL[a["pool_type"]],
                        dtype=DTYPE_CODE[x["dtype"]], in_q=(s, z), out_q=(so, zo))
+            if lay in ACT_FROM_WHCN:
+                y = transpose(y, oshape, ACT_FROM_WHCN[lay])
         elif k in ("RELU", "RELU6"):
             y = activation(ACT_RELU if k == "RELU" else ACT_RELU6, DTYPE_CODE[x["dtype"]], xv,
                            (s, z), (so, zo))

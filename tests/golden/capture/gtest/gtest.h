@@ -2,7 +2,9 @@
 // (tests/golden/make_fixtures.py). Instead of judging results it records the
 // expected vectors a test compares against, next to the graph the test built.
 #pragma once
+#include <cstddef>
 #include <cstdint>
+#include <cstring>
 #include <string>
 #include <type_traits>
 #include <vector>
@@ -29,12 +31,16 @@ Sink RecordEq(const std::vector<T>& golden, const std::vector<T>&) {
   RecordGolden(ToDouble(golden), 0.0, "eq");
   return Sink();
 }
+// shapes (EXPECT_EQ(tensor->GetShape(), expected_shape)) are not output vectors
+inline Sink RecordEq(const std::vector<uint32_t>&, const std::vector<uint32_t>&) { return Sink(); }
 template <typename A, typename B>
 Sink RecordEq(const A&, const B&) { return Sink(); }
 Sink Check(bool ok, const char* expr);
 // EXPECT_NEAR(golden[i], output[i], tol) in a loop over the output: the scalars are gathered and
 // become one case when the test body ends, if there is one of them per output element.
 Sink RecordNear(double golden, double tol);
+// memcmp(output, expected, bytes) == 0 inside EXPECT_TRUE: `expected` becomes the golden vector
+int RecordMem(const void* output, const void* expected, size_t bytes);
 }  // namespace tvxcap
 
 namespace testing {
@@ -60,4 +66,5 @@ inline Matcher<float> FloatNear(float, float) { return Matcher<float>(); }
 #define ASSERT_TRUE(x) ::tvxcap::Check(static_cast<bool>(x), #x)
 #define EXPECT_EQ(a, b) ::tvxcap::RecordEq((a), (b))
 #define EXPECT_NEAR(a, b, t) ::tvxcap::RecordNear(static_cast<double>(a), static_cast<double>(static_cast<float>(t)))
+#define memcmp(a, b, n) ::tvxcap::RecordMem((a), (b), (n))
 #define GTEST_SKIP() return

@@ -33,18 +33,21 @@ SOURCES = {
     "softmax": "src/tim/vx/ops/softmax_test.cc",
     "transpose": "src/tim/vx/ops/transpose_test.cc",
     # (file, test suite): only the TEST(suite, ...) bodies of a file that also tests operators outside this path
-    "dataconvert": ("src/tim/vx/ops/simple_operations_test.cc", "DataConvert"),
+    "dataconvert": ("src/tim/vx/ops/simple_operations_test.cc", ["DataConvert"]),
+    # the source graphs of the layout-inference tests that stay inside this path
+    "layout_inference": ("src/tim/transform/layout_inference_test.cc", ["LayoutInference", "GroupedConv2d", "FC"]),
 }
 
 
-def select_suite(path, suite):
-    """The file's preprocessor lines plus the TEST(suite, ...) bodies, as text for the compiler's stdin
-    (nothing of the reference is written to disk)."""
+def select_suite(path, suites):
+    """The file's preprocessor lines plus the TEST(suite, ...) bodies of the named suites, as text for the
+    compiler's stdin (nothing of the reference is written to disk)."""
+    suite = "|".join(re.escape(s) for s in suites)
     text = open(path).read()
     out = [l for l in text.splitlines() if l.startswith("#include")]
     pos = 0
     while True:
-        m = re.search(r"^TEST\(\s*%s\s*,[^)]*\)\s*\{" % re.escape(suite), text[pos:], re.M)
+        m = re.search(r"^TEST\(\s*(?:%s)\s*,[^)]*\)\s*\{" % suite, text[pos:], re.M)
         if not m:
             break
         start = pos + m.start()
@@ -65,25 +68,31 @@ def select_suite(path, suite):
 def main():
     build = os.path.join(HERE, "capture", "_build")
     os.makedirs(build, exist_ok=True)
-    common = [
-        "g++", "-std=c++17", "-O1", "-w",
-        "-I", os.path.join(HERE, "capture"),
-        "-I", os.path.join(PKG, "include"),
-        "-I", os.path.join(PKG, "src"),
-        "-I", REF,
-        '-DTVX_REF_TEST_UTILS="%s"' % os.path.join(REF, "src/tim/vx/test_utils.h"),
-    ]
-    host = [os.path.join(PKG, "src", f) for f in ("frontend.cc", "graph_passes.cc")]
+    cxx = ["g++", "-std=c++17", "-O1", "-w"]
+    product_inc = ["-I", os.path.join(PKG, "include"), "-I", os.path.join(PKG, "src")]
+    # the recording stand-ins (gtest, test_utils, the LayoutInference shim) shadow the real headers for the
+    # reference's test sources and the recorder only; the runtime's own sources are built without them
+    capture_inc = ["-I", os.path.join(HERE, "capture")] + product_inc + [
+        "-I", REF, '-DTVX_REF_TEST_UTILS="%s"' % os.path.join(REF, "src/tim/vx/test_utils.h")]
+    objs = []
+    for f in ("frontend.cc", "graph_passes.cc", "layout_inference.cc"):
+        obj = os.path.join(build, f.replace(".cc", ".o"))
+        subprocess.check_call(cxx + product_inc + ["-c", os.path.join(PKG, "src", f), "-o", obj])
+        objs.append(obj)
+    main_obj = os.path.join(build, "capture_main.o")
+    subprocess.check_call(cxx + capture_inc + ["-c", os.path.join(HERE, "capture", "capture_main.cc"), "-o", main_obj])
+    objs.append(main_obj)
     for name, rel in SOURCES.items():
         exe = os.path.join(build, "capture_" + name)
-        rest = [os.path.join(HERE, "capture", "capture_main.cc")] + host + ["-o", exe]
+        test_obj = os.path.join(build, "test_" + name + ".o")
         print("building", name, flush=True)
         if isinstance(rel, tuple):
             path = os.path.join(REF, rel[0])
-            cmd = common + ["-I", os.path.dirname(path), "-x", "c++", "-", "-x", "none"] + rest
+            cmd = cxx + capture_inc + ["-I", os.path.dirname(path), "-x", "c++", "-c", "-", "-o", test_obj]
             subprocess.run(cmd, input=select_suite(path, rel[1]).encode(), check=True)
         else:
-            subprocess.check_call(common + [os.path.join(REF, rel)] + rest)
+            subprocess.check_call(cxx + capture_inc + ["-c", os.path.join(REF, rel), "-o", test_obj])
+        subprocess.check_call(cxx + [test_obj] + objs + ["-o", exe])
         out = os.path.join(HERE, name + ".json")
         subprocess.check_call([exe, out])
         print("wrote", out, os.path.getsize(out), "bytes", flush=True)

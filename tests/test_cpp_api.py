@@ -162,6 +162,61 @@ def test_transpose_feeds_a_convolution(tmp_path, oracle):
 
 
 @pytest.mark.gpu
+def test_layout_inference_on_a_channel_fastest_network(tmp_path, oracle):
+    """What an NHWC front end hands over (src/tim/transform/layout_inference.cc): CWHN uint8
+    activations, IcWHOc kernels. conv3x3+relu6 -> depthwise3x3 -> 1x1 conv -> residual Add ->
+    avg pool -> Reshape -> FullyConnected -> Softmax. The rewritten graph must give what the
+    oracle computes operator by operator with explicit transposes around every CWHN operator;
+    at debug log level the plan shows one permute behind the input and one in front of Reshape."""
+    rng = np.random.default_rng(21)
+    c0, c1, w, h, n, classes = 8, 16, 12, 10, 2, 10
+    q, T, OP = GF.asym, GF.tensor, GF.op
+    u8 = lambda *s: rng.integers(0, 256, int(np.prod(s)), dtype=np.uint8)
+    cw = dict(layout="CWHN", kernel_layout="IcWHOc", pad_type="AUTO")
+    g = {"test": "nhwc_net", "output": 18, "layout_inference": True, "tensors": [
+        T(0, "UINT8", "INPUT", [c0, w, h, n], q(0.5, 128), u8(c0, w, h, n)),
+        T(1, "UINT8", "CONSTANT", [c0, 3, 3, c1], q(0.02, 120), u8(c0, 3, 3, c1)),
+        T(2, "INT32", "CONSTANT", [c1], q(0.01, 0), rng.integers(-500, 500, c1, dtype=np.int32)),
+        T(3, "UINT8", "TRANSIENT", [c1, w, h, n], q(4.0, 128)),
+        T(4, "UINT8", "CONSTANT", [c1, 3, 3, 1], q(0.03, 130), u8(c1, 3, 3, 1)),
+        T(5, "INT32", "CONSTANT", [c1], q(0.12, 0), rng.integers(-500, 500, c1, dtype=np.int32)),
+        T(6, "UINT8", "TRANSIENT", [c1, w, h, n], q(16.0, 110)),
+        T(7, "UINT8", "CONSTANT", [c1, 1, 1, c1], q(0.02, 125), u8(c1, 1, 1, c1)),
+        T(8, "INT32", "CONSTANT", [c1], q(0.32, 0), rng.integers(-500, 500, c1, dtype=np.int32)),
+        T(9, "UINT8", "TRANSIENT", [c1, w, h, n], q(60.0, 120)),
+        T(10, "UINT8", "TRANSIENT", [c1, w, h, n], q(64.0, 100)),
+        T(11, "UINT8", "TRANSIENT", [c1, w // 2, h // 2, n], q(64.0, 100)),
+        T(12, "UINT8", "TRANSIENT", [c1 * (w // 2) * (h // 2), n], q(64.0, 100)),
+        T(13, "UINT8", "CONSTANT", [c1 * (w // 2) * (h // 2), classes], q(1e-5, 128), u8(c1 * (w // 2) * (h // 2), classes)),
+        T(14, "INT32", "CONSTANT", [classes], q(0.00064, 0), rng.integers(-2000, 2000, classes, dtype=np.int32)),
+        T(15, "UINT8", "TRANSIENT", [classes, n], q(0.5, 128)),
+        T(18, "FLOAT32", "OUTPUT", [classes, n])],
+        "ops": [OP("CONV2D", [0, 1, 2], [3], pad=[1, 1, 1, 1], ksize=[3, 3], weights=c1, **cw),
+                OP("CONV2D", [3, 4, 5], [6], pad=[1, 1, 1, 1], ksize=[3, 3], weights=c1, multiplier=1, **cw),
+                OP("CONV2D", [6, 7, 8], [9], pad=[0, 0, 0, 0], ksize=[1, 1], weights=c1, **cw),
+                OP("ADD", [9, 3], [10]),
+                OP("POOL", [10], [11], pool_type="AVG", ksize=[2, 2], stride=[2, 2], pad=[0, 0, 0, 0], layout="CWHN", pad_type="AUTO"),
+                OP("RESHAPE", [11], [12], new_shape=[c1 * (w // 2) * (h // 2), n]),
+                OP("FCL", [12, 13, 14], [15], axis=0, weights=classes),
+                OP("SOFTMAX", [15], [18], beta=0.05, sm_axis=0)]}
+    res, info, log = GF.run_graphs([g], str(tmp_path), env={"VSI_NN_LOG_LEVEL": "3"})
+    assert res[0] is not None, (info, log[-3000:])
+    want = oracle.run_graph(g)
+    assert np.allclose(res[0], want, rtol=0, atol=1e-6), (res[0][:10], want[:10])
+    logits = copy.deepcopy(g)        # the uint8 logits bit for bit
+    logits["test"] = "nhwc_net_logits"
+    logits["ops"] = logits["ops"][:-1]
+    logits["tensors"] = logits["tensors"][:-1]
+    logits["tensors"][-1]["attr"] = "OUTPUT"
+    logits["output"] = 15
+    res2, info2, log2 = GF.run_graphs([logits], str(tmp_path), env={"VSI_NN_LOG_LEVEL": "3"})
+    assert res2[0] is not None, (info2, log2[-3000:])
+    assert np.array_equal(res2[0], oracle.run_graph(logits))
+    plan = [l for l in log2.splitlines() if "uid" in l and "->" in l]
+    assert sum("transpose" in l for l in plan) == 2, plan
+
+
+@pytest.mark.gpu
 def test_repeated_runs_follow_the_inputs(tmp_path, oracle):
     """Run() may be called again and again with the inputs re-filled in between
     (src/tim/vx/graph.cc:378-391): six runs with the input alternating between two images,

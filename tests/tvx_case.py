@@ -11,7 +11,7 @@ import tvx_oracle as O
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 GOLDEN_FILES = ["conv2d", "depthwise_conv", "grouped_conv2d", "conv1d", "fullyconnected", "max_pool", "avg_pool", "softmax",
-                "transpose", "dataconvert"]
+                "transpose", "dataconvert", "layout_inference"]
 
 
 def load_cases(name):

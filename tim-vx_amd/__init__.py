@@ -116,6 +116,7 @@ def lib():
         L.tvx_pool2d_create.argtypes = [C.POINTER(Pool2dDesc), C.POINTER(vp)]
         L.tvx_activation_create.argtypes = [C.POINTER(EltwiseDesc), C.POINTER(vp)]
         L.tvx_add_create.argtypes = [C.POINTER(EltwiseDesc), C.POINTER(vp)]
+        L.tvx_op_run3.argtypes = [vp, vp, vp, vp, vp, vp]
         L.tvx_softmax_create.argtypes = [C.POINTER(SoftmaxDesc), C.POINTER(vp)]
         L.tvx_convert_create.argtypes = [C.POINTER(ConvertDesc), C.POINTER(vp)]
         L.tvx_transpose_create.argtypes = [C.POINTER(TransposeDesc), C.POINTER(vp)]

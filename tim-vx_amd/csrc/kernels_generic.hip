@@ -124,7 +124,8 @@ int ConvGenericRun(tvx_op* op, const void* in0, const void* in1, void* out, hipS
   const void* w = op->has_const_weights ? op->weights.ptr : in1;
   const uint64_t total = static_cast<uint64_t>(d.out_w) * d.out_h * d.out_c * d.batch;
   const dim3 grid(Blocks(total)), block(kBlock);
-  const int32_t* bias_i = op->bias.as<int32_t>();
+  const int32_t* bias_i = op->bias_at_run ? static_cast<const int32_t*>(op->bias_at_run) : op->bias.as<int32_t>();
+  const float* bias_f = op->bias_at_run ? static_cast<const float*>(op->bias_at_run) : op->bias.as<float>();
   const int32_t *mu = op->mult.as<int32_t>(), *sh = op->shift.as<int32_t>();
   if (d.in_dtype == TVX_U8 && d.w_dtype == TVX_U8) {
     hipLaunchKernelGGL((ConvQuantKernel<uint8_t, uint8_t>), grid, block, 0, st, a,
@@ -141,11 +142,11 @@ int ConvGenericRun(tvx_op* op, const void* in0, const void* in1, void* out, hipS
   } else if (d.in_dtype == TVX_F32) {
     hipLaunchKernelGGL((ConvFloatKernel<float>), grid, block, 0, st, a,
                        static_cast<const float*>(in0), static_cast<const float*>(w),
-                       op->bias.as<float>(), static_cast<float*>(out), total);
+                       bias_f, static_cast<float*>(out), total);
   } else {
     hipLaunchKernelGGL((ConvFloatKernel<__half>), grid, block, 0, st, a,
                        static_cast<const __half*>(in0), static_cast<const __half*>(w),
-                       op->bias.as<float>(), static_cast<__half*>(out), total);
+                       bias_f, static_cast<__half*>(out), total);
   }
   TVX_HIP_CHECK(hipGetLastError());
   return TVX_OK;
@@ -238,7 +239,8 @@ int FcGenericRun(tvx_op* op, const void* in0, const void* in1, void* out, hipStr
   const void* w = op->has_const_weights ? op->weights.ptr : in1;
   const uint64_t total = static_cast<uint64_t>(d.m) * d.n;
   const dim3 grid(Blocks(total)), block(kBlock);
-  const int32_t* bias_i = op->bias.as<int32_t>();
+  const int32_t* bias_i = op->bias_at_run ? static_cast<const int32_t*>(op->bias_at_run) : op->bias.as<int32_t>();
+  const float* bias_f = op->bias_at_run ? static_cast<const float*>(op->bias_at_run) : op->bias.as<float>();
   const int32_t *mu = op->mult.as<int32_t>(), *sh = op->shift.as<int32_t>();
   // few outputs with a long reduction: a wavefront per output
   const bool wave = total <= 16384 && d.k >= 128;
@@ -273,11 +275,11 @@ int FcGenericRun(tvx_op* op, const void* in0, const void* in1, void* out, hipStr
   } else if (d.in_dtype == TVX_F32) {
     hipLaunchKernelGGL((FcFloatKernel<float>), grid, block, 0, st, a,
                        static_cast<const float*>(in0), static_cast<const float*>(w),
-                       op->bias.as<float>(), static_cast<float*>(out), total);
+                       bias_f, static_cast<float*>(out), total);
   } else {
     hipLaunchKernelGGL((FcFloatKernel<__half>), grid, block, 0, st, a,
                        static_cast<const __half*>(in0), static_cast<const __half*>(w),
-                       op->bias.as<float>(), static_cast<__half*>(out), total);
+                       bias_f, static_cast<__half*>(out), total);
   }
   TVX_HIP_CHECK(hipGetLastError());
   return TVX_OK;

@@ -483,6 +483,18 @@ int tvx_op_run(tvx_op* op, const void* in0, const void* in1, void* out_ptr, void
   return op->run(op, in0, in1, out_ptr, static_cast<hipStream_t>(stream));
 }
 
+int tvx_op_run3(tvx_op* op, const void* in0, const void* in1, const void* in2, void* out_ptr, void* stream) {
+  if (!in2) return tvx_op_run(op, in0, in1, out_ptr, stream);
+  if (!op || !op->run) return SetError(TVX_E_INVALID, "tvx_op_run3: null operator");
+  if ((op->kind != OP_CONV2D && op->kind != OP_FC) || op->has_const_weights || op->bias.ptr)
+    return SetError(TVX_E_UNSUPPORTED,
+                    "tvx_op_run3: a run-time bias goes with a Conv2d / FullyConnected created without weights and bias");
+  op->bias_at_run = in2;
+  const int s = tvx_op_run(op, in0, in1, out_ptr, stream);
+  op->bias_at_run = nullptr;
+  return s;
+}
+
 const char* tvx_op_kernel_name(const tvx_op* op) { return op ? op->kernel_name : ""; }
 
 void tvx_op_destroy(tvx_op* op) { delete op; }

@@ -46,6 +46,7 @@ struct tvx_op {
   int kind = 0;
   const char* kernel_name = "";
   int (*run)(tvx_op*, const void* in0, const void* in1, void* out, hipStream_t) = nullptr;
+  const void* bias_at_run = nullptr;  // set by tvx_op_run3 for the duration of one enqueue
 
   tvx_conv2d_desc conv{};
   tvx_fc_desc fc{};

@@ -707,6 +707,7 @@ Conv2d::Conv2d(Graph* graph, int32_t weights, PadType padding,
       dilation_(dilation), pad_(pad), multiplier_(multiplier),
       kernel_layout_(kernel_layout) {
   OpAttrs& a = impl_->attrs_;
+  a.kernel_layout = kernel_layout_;
   if (padding_ == PadType::NONE)
     VSILOGW("PadType::NONE is treated as AUTO (explicit pad)");
   a.pad_type = padding_ == PadType::NONE ? PadType::AUTO : padding_;
@@ -756,6 +757,7 @@ Conv1d::Conv1d(Graph* graph, int32_t weights, PadType padding, uint32_t ksize, u
       weights_(weights), padding_(padding), ksize_(ksize), stride_(stride), dilation_(dilation),
       pad_(pad), multiplier_(multiplier), kernel_layout_(kernel_layout) {
   OpAttrs& a = impl_->attrs_;
+  a.kernel_layout = kernel_layout_;
   a.conv_1d = true;
   a.pad_type = padding_ == PadType::NONE ? PadType::AUTO : padding_;
   a.pad[0] = pad_[0];
@@ -788,6 +790,7 @@ GroupedConv2d::GroupedConv2d(Graph* graph, PadType padding,
       padding_(padding), strides_(strides), dilation_(dilation), pad_({0, 0, 0, 0}),
       group_number_(grouped_number), kernel_layout_(kernel_layout) {
   OpAttrs& a = impl_->attrs_;
+  a.kernel_layout = kernel_layout_;
   a.pad_type = padding_ == PadType::NONE ? PadType::AUTO : padding_;
   for (int i = 0; i < 2; ++i) {
     a.stride[i] = strides_[i];
@@ -804,6 +807,7 @@ GroupedConv2d::GroupedConv2d(Graph* graph, const std::array<uint32_t, 4>& pad,
       padding_(PadType::AUTO), strides_(strides), dilation_(dilation), pad_(pad),
       group_number_(group_number), kernel_layout_(kernel_layout) {
   OpAttrs& a = impl_->attrs_;
+  a.kernel_layout = kernel_layout_;
   a.pad_type = PadType::AUTO;
   for (int i = 0; i < 4; ++i) a.pad[i] = pad_[i];
   for (int i = 0; i < 2; ++i) {

@@ -49,6 +49,7 @@ struct Step {
   tvx_op* op = nullptr;
   TensorImpl* in0 = nullptr;
   TensorImpl* in1 = nullptr;  // run-time weights / second Add operand
+  TensorImpl* in2 = nullptr;  // run-time bias
   TensorImpl* out = nullptr;
   std::string name;
 };
@@ -159,7 +160,8 @@ class HipExecutor : public Executor {
       t0 = std::chrono::steady_clock::now();
     }
     for (auto& s : steps_) {
-      const int st = tvx_op_run(s.op, dev_[s.in0], s.in1 ? dev_[s.in1] : nullptr, dev_[s.out], stream_);
+      const int st = tvx_op_run3(s.op, dev_[s.in0], s.in1 ? dev_[s.in1] : nullptr, s.in2 ? dev_[s.in2] : nullptr,
+                                 dev_[s.out], stream_);
       if (st != TVX_OK) {
         VSILOGE("%s failed: %s", s.name.c_str(), tvx_last_error());
         return false;
@@ -194,11 +196,12 @@ class HipExecutor : public Executor {
     return true;
   }
 
-  void Push(tvx_op* op, OpImpl* im, TensorImpl* in0, TensorImpl* in1, TensorImpl* out) {
+  void Push(tvx_op* op, OpImpl* im, TensorImpl* in0, TensorImpl* in1, TensorImpl* out, TensorImpl* in2 = nullptr) {
     Step s;
     s.op = op;
     s.in0 = in0;
     s.in1 = in1;
+    s.in2 = in2;
     s.out = out;
     s.name = std::string(OpKindName(im->kind_)) + " (" + tvx_op_kernel_name(op) + ")";
     VSILOGI("uid %u -> %s", im->uid_, s.name.c_str());
@@ -246,15 +249,14 @@ class HipExecutor : public Executor {
     WeightQuant(w->spec_, &d.w_scale, &d.w_zp, &d.w_scales);
     d.out_scale = ScaleOf(out->spec_); d.out_zp = ZpOf(out->spec_);
     d.activation = act;
-    if (b && !b->IsConstTensor()) {
-      VSILOGE("CONV2D: a run-time bias tensor is not supported");
-      return false;
-    }
-    const bool const_w = w->IsConstTensor() && w->HostData();
+    // a bias that is not a constant is read at run time, which the kernels with packed weights
+    // cannot do: weights and bias then both go in as operands of the generic kernel
+    const bool bias_at_run = b && !b->IsConstTensor();
+    const bool const_w = w->IsConstTensor() && w->HostData() && !bias_at_run;
     tvx_op* op = nullptr;
-    if (tvx_conv2d_create(&d, const_w ? w->HostData() : nullptr, b ? b->HostData() : nullptr, &op) != TVX_OK)
+    if (tvx_conv2d_create(&d, const_w ? w->HostData() : nullptr, b && !bias_at_run ? b->HostData() : nullptr, &op) != TVX_OK)
       return Fail("tvx_conv2d_create");
-    Push(op, im, x, const_w ? nullptr : w, out);
+    Push(op, im, x, const_w ? nullptr : w, out, bias_at_run ? b : nullptr);
     return true;
   }
 
@@ -278,15 +280,12 @@ class HipExecutor : public Executor {
     WeightQuant(w->spec_, &d.w_scale, &d.w_zp, &d.w_scales);
     d.out_scale = ScaleOf(out->spec_); d.out_zp = ZpOf(out->spec_);
     d.activation = act;
-    if (b && !b->IsConstTensor()) {
-      VSILOGE("FCL: a run-time bias tensor is not supported");
-      return false;
-    }
-    const bool const_w = w->IsConstTensor() && w->HostData();
+    const bool bias_at_run = b && !b->IsConstTensor();  // as for Conv2d
+    const bool const_w = w->IsConstTensor() && w->HostData() && !bias_at_run;
     tvx_op* op = nullptr;
-    if (tvx_fully_connected_create(&d, const_w ? w->HostData() : nullptr, b ? b->HostData() : nullptr, &op) != TVX_OK)
+    if (tvx_fully_connected_create(&d, const_w ? w->HostData() : nullptr, b && !bias_at_run ? b->HostData() : nullptr, &op) != TVX_OK)
       return Fail("tvx_fully_connected_create");
-    Push(op, im, x, const_w ? nullptr : w, out);
+    Push(op, im, x, const_w ? nullptr : w, out, bias_at_run ? b : nullptr);
     return true;
   }
 

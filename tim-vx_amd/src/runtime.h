@@ -47,6 +47,7 @@ struct OpAttrs {
   uint32_t ksize[2] = {0, 0};
   int32_t multiplier = 0;
   int32_t groups = 0;  // GroupedConv2d: > 1
+  DataLayout kernel_layout = DataLayout::WHIcOc;  // read by layout inference only
   bool conv_1d = false;  // Conv1d: {W, C, N} tensors, the 2-D operator on rows of height one
   uint32_t weights = 0;
   // pool

@@ -31,6 +31,7 @@
 
 #include "tim/vx/context.h"
 #include "tim/vx/graph.h"
+#include "tim/transform/layout_inference.h"
 #include "tim/vx/ops.h"
 #include "tim/vx/tensor.h"
 
@@ -69,6 +70,14 @@ PadType ParsePad(const std::string& s) {
   if (s == "NONE") return PadType::NONE;
   return PadType::AUTO;
 }
+DataLayout ParseLayout(const std::string& s, DataLayout fallback) {
+  static const std::map<std::string, DataLayout> m = {
+      {"WHCN", DataLayout::WHCN}, {"CWHN", DataLayout::CWHN}, {"IcWHOc", DataLayout::IcWHOc},
+      {"OcIcWH", DataLayout::OcIcWH}, {"IcOcWH", DataLayout::IcOcWH}, {"WHIcOc", DataLayout::WHIcOc},
+      {"WCN", DataLayout::WCN}, {"WIcOc", DataLayout::WIcOc}};
+  auto it = m.find(s);
+  return it == m.end() ? fallback : it->second;
+}
 PoolType ParsePool(const std::string& s) {
   if (s == "AVG") return PoolType::AVG;
   if (s == "L2") return PoolType::L2;
@@ -99,7 +108,7 @@ int main(int argc, char** argv) {
 
   setenv("TVX_RUNTIME_PROFILE", "1", 0);  // makes `bench` report the device part of Run()
   auto context = Context::Create();
-  std::shared_ptr<Graph> graph;
+  std::shared_ptr<Graph> graph, source_graph;
   std::map<int, Pending> tensors;
   std::string name, line;
   bool compiled = false, compile_ok = false;
@@ -166,7 +175,10 @@ int main(int argc, char** argv) {
       ss >> n_perm;
       std::vector<uint32_t> perm(n_perm > 0 ? n_perm : 0);
       for (auto& d : perm) ss >> d;
+      std::string layout_s = "ANY", klayout_s = "ANY";
+      ss >> layout_s >> klayout_s;
       if (!ss) { std::fprintf(stderr, "malformed op record in %s\n", name.c_str()); return 2; }
+      const DataLayout layout = ParseLayout(layout_s, DataLayout::WHCN), klayout = ParseLayout(klayout_s, DataLayout::WHIcOc);
       const RoundType rnd = round_type == "CEILING" ? RoundType::CEILING : RoundType::FLOOR;
       std::shared_ptr<Operation> op;
       if (kind == "CONV2D" && conv_1d) {
@@ -174,11 +186,11 @@ int main(int argc, char** argv) {
                                                  std::array<uint32_t, 2>{pad[0], pad[1]}, multiplier);
       } else if (kind == "CONV2D" && groups > 1) {
         if (ParsePad(pad_type) == PadType::AUTO)
-          op = graph->CreateOperation<ops::GroupedConv2d>(pad, stride, dil, groups);
+          op = graph->CreateOperation<ops::GroupedConv2d>(pad, stride, dil, groups, layout, klayout);
         else
-          op = graph->CreateOperation<ops::GroupedConv2d>(ParsePad(pad_type), stride, dil, groups);
+          op = graph->CreateOperation<ops::GroupedConv2d>(ParsePad(pad_type), stride, dil, groups, layout, klayout);
       } else if (kind == "CONV2D") {
-        op = graph->CreateOperation<ops::Conv2d>(weights, ParsePad(pad_type), ksize, stride, dil, pad, multiplier);
+        op = graph->CreateOperation<ops::Conv2d>(weights, ParsePad(pad_type), ksize, stride, dil, pad, multiplier, layout, klayout);
       } else if (kind == "FCL") {
         op = graph->CreateOperation<ops::FullyConnected>(static_cast<uint32_t>(axis), static_cast<uint32_t>(weights));
       } else if (kind == "POOL") {
@@ -186,9 +198,9 @@ int main(int argc, char** argv) {
           op = graph->CreateOperation<ops::Pool1d>(ParsePool(pool_type), std::array<uint32_t, 2>{pad[0], pad[1]},
                                                    ksize[0], stride[0], rnd);
         } else if (ParsePad(pad_type) == PadType::AUTO) {
-          op = graph->CreateOperation<ops::Pool2d>(ParsePool(pool_type), pad, ksize, stride, rnd);
+          op = graph->CreateOperation<ops::Pool2d>(ParsePool(pool_type), pad, ksize, stride, rnd, layout);
         } else {
-          op = graph->CreateOperation<ops::Pool2d>(ParsePool(pool_type), ParsePad(pad_type), ksize, stride, rnd);
+          op = graph->CreateOperation<ops::Pool2d>(ParsePool(pool_type), ParsePad(pad_type), ksize, stride, rnd, layout);
         }
       } else if (kind == "RELU") {
         op = graph->CreateOperation<ops::Relu>();
@@ -209,6 +221,16 @@ int main(int argc, char** argv) {
         return 2;
       }
       op->BindInputs(ins).BindOutputs(outs);
+    } else if (rec == "infer") {
+      // layout inference: the rewritten graph replaces the one built so far; INPUT / OUTPUT
+      // tensors are looked up through the map it returns
+      auto r = tim::transform::LayoutInference(graph, context);
+      for (auto& kv : tensors) {
+        auto it = r.second.find(kv.second.tensor);
+        if (it != r.second.end()) kv.second.tensor = it->second;
+      }
+      source_graph = graph;
+      graph = r.first;
     } else if (rec == "run") {
       int id;
       ss >> id;
@@ -267,6 +289,7 @@ int main(int argc, char** argv) {
       std::fflush(stdout);
     } else if (rec == "end") {
       graph.reset();
+      source_graph.reset();
       tensors.clear();
     }
   }
