@@ -188,6 +188,17 @@ typedef struct tvx_softmax_desc {
 
 int tvx_softmax_create(const tvx_softmax_desc* desc, tvx_op** op);
 
+/* ---- DeConv2d (transposed convolution) ----------------------------------------------- */
+/* Replaces vxDeconvolutionLayer (src/tim/vx/ops/deconv.cc:45-79,
+ * src/tim/vx/internal/src/ops/vsi_nn_op_deconvolution.c:217-218,398-497). Same descriptor as
+ * Conv2d, read the other way round: input pixel (ix, iy) adds in * w[kx, ky] to output pixel
+ * (ix * stride - pad_left + kx, iy * stride - pad_top + ky); weights {k_w, k_h, in_c / groups,
+ * out_c} as the reference's WHIcOc deconvolution kernel, {k_w, k_h, out_c, 1} with
+ * multiplier = 1 for the depthwise form (group == channels); dilation must be 1. The output
+ * extent is the caller's: (in - 1) * stride + k - pads + output_padding, or anything smaller. */
+int tvx_deconv2d_create(const tvx_conv2d_desc* desc, const void* weights_host, const void* bias_host,
+                        tvx_op** op);
+
 /* ---- DataConvert ------------------------------------------------------------------ */
 /* Replaces the DATACONVERT operator (src/tim/vx/ops/simple_operations.cc:39 -> vxTensorCopyNode /
  * the conversions of src/tim/vx/internal/include/utils/vsi_nn_dtype_util_prv.h:228-266): every

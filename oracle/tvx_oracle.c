@@ -245,6 +245,73 @@ void tvxo_conv2d(const tvxo_conv_desc* d, const void* x, const void* w,
   }
 }
 
+/*
+ * DeConv2d, the transposed convolution (vxDeconvolutionLayer; src/tim/vx/ops/deconv.cc:45-79,
+ * extent rule src/tim/vx/internal/src/ops/vsi_nn_op_deconvolution.c:217-218; values pinned by
+ * src/tim/vx/ops/deconv2d_test.cc:20-140: no kernel flip, out(0,0) = in(0,0) * w(0,0)).
+ * Written as the scatter it is defined by: input pixel (ix, iy) of channel ic adds
+ * (x - zx)(w[oc][ic][ky][kx] - zw) to output pixel (ix*stride - pad_left + kx, iy*stride - pad_top + ky);
+ * then bias, requantization and clamp as for Conv2d. Weights {k_w, k_h, in_c/groups, out_c};
+ * multiplier = 1 is the depthwise form ({k_w, k_h, c, 1}); dilation is not used.
+ */
+void tvxo_deconv2d(const tvxo_conv_desc* d, const void* x, const void* w, const void* bias, void* y) {
+  const int quant = d->in_dtype == TVXO_U8 || d->in_dtype == TVXO_I8;
+  const int64_t in_plane = (int64_t)d->in_w * d->in_h, out_plane = (int64_t)d->out_w * d->out_h;
+  const int32_t groups = d->groups > 1 ? d->groups : 1;
+  const int32_t ic_per_oc = d->multiplier > 0 ? 1 : d->in_c / groups;
+  int32_t lo = 0, hi = 0;
+  if (quant) tvxo_act_range(d->out_dtype, d->out_scale, d->out_zp, d->act, &lo, &hi);
+  const int64_t total = (int64_t)d->batch * d->out_c;
+#pragma omp parallel for schedule(static)
+  for (int64_t job = 0; job < total; ++job) {
+    const int32_t n = (int32_t)(job / d->out_c), oc = (int32_t)(job % d->out_c);
+    const int32_t ic0 = d->multiplier > 0 ? oc / d->multiplier : (oc / (d->out_c / groups)) * ic_per_oc;
+    const int32_t zw = d->w_scales ? 0 : d->w_zp;
+    int64_t* acc = (int64_t*)calloc((size_t)out_plane, sizeof(int64_t));
+    float* facc = (float*)calloc((size_t)out_plane, sizeof(float));
+    for (int32_t ci = 0; ci < ic_per_oc; ++ci) {
+      const int64_t xb = ((int64_t)n * d->in_c + ic0 + ci) * in_plane;
+      const int64_t wb = ((int64_t)oc * ic_per_oc + ci) * d->k_h * d->k_w;
+      for (int32_t iy = 0; iy < d->in_h; ++iy)
+        for (int32_t ix = 0; ix < d->in_w; ++ix)
+          for (int32_t ky = 0; ky < d->k_h; ++ky) {
+            const int32_t oy = iy * d->stride_h - d->pad_top + ky;
+            if (oy < 0 || oy >= d->out_h) continue;
+            for (int32_t kx = 0; kx < d->k_w; ++kx) {
+              const int32_t ox = ix * d->stride_w - d->pad_left + kx;
+              if (ox < 0 || ox >= d->out_w) continue;
+              const int64_t xi = xb + (int64_t)iy * d->in_w + ix, wi = wb + (int64_t)ky * d->k_w + kx;
+              if (quant)
+                acc[(int64_t)oy * d->out_w + ox] +=
+                    (int64_t)(load_q(x, d->in_dtype, xi) - d->in_zp) * (int64_t)(load_q(w, d->w_dtype, wi) - zw);
+              else
+                facc[(int64_t)oy * d->out_w + ox] += load_f(x, d->in_dtype, xi) * load_f(w, d->w_dtype, wi);
+            }
+          }
+    }
+    int32_t mult = 0, shift = 0;
+    if (quant) {
+      double ws = d->w_scales ? (double)d->w_scales[oc] : (double)d->w_scale;
+      tvxo_quantize_multiplier((double)d->in_scale * ws / (double)d->out_scale, &mult, &shift);
+    }
+    for (int64_t p = 0; p < out_plane; ++p) {
+      const int64_t yi = ((int64_t)n * d->out_c + oc) * out_plane + p;
+      if (quant) {
+        int64_t a = acc[p] + (bias ? ((const int32_t*)bias)[oc] : 0);
+        int64_t r = tvxo_requant((int32_t)(uint32_t)(uint64_t)a, mult, shift);
+        store_q(y, d->out_dtype, yi, clamp64(r + d->out_zp, lo, hi));
+      } else {
+        float f = facc[p] + (bias ? ((const float*)bias)[oc] : 0.f);
+        if (d->act == TVXO_ACT_RELU || d->act == TVXO_ACT_RELU6) f = f < 0.f ? 0.f : f;
+        if (d->act == TVXO_ACT_RELU6) f = f > 6.f ? 6.f : f;
+        store_f(y, d->out_dtype, yi, f);
+      }
+    }
+    free(acc);
+    free(facc);
+  }
+}
+
 typedef struct {
   int32_t m, k, n;
   int32_t in_dtype, w_dtype, out_dtype;

@@ -77,6 +77,7 @@ def lib():
         _lib.tvxo_softmax.argtypes = [C.c_int, C.c_int32, C.c_int64, C.c_int64, C.c_float, C.c_void_p, C.c_float,
                                       C.c_int32, C.c_void_p]
         _lib.tvxo_conv2d.argtypes = [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+        _lib.tvxo_deconv2d.argtypes = [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         _lib.tvxo_fully_connected.argtypes = [C.POINTER(FcDesc), C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         _lib.tvxo_pool2d.argtypes = [C.POINTER(PoolDesc), C.c_void_p, C.c_void_p]
     return _lib
@@ -144,8 +145,9 @@ def _resolved_pad(a, in_shape, w_shape):
 
 def conv2d(x, w, bias, *, in_shape, w_shape, out_shape, stride, dilation, pad_left, pad_top,
            multiplier, in_dtype, w_dtype, out_dtype, in_q=(1.0, 0), w_q=(1.0, 0, None),
-           out_q=(1.0, 0), act=ACT_NONE, groups=0):
-    """Shapes are WHCN / WHIcOc lists (dim 0 fastest); arrays are flat, C-contiguous."""
+           out_q=(1.0, 0), act=ACT_NONE, groups=0, transposed=False):
+    """Shapes are WHCN / WHIcOc lists (dim 0 fastest); arrays are flat, C-contiguous.
+    transposed: DeConv2d (same descriptor, read the other way round)."""
     d = ConvDesc()
     d.groups = groups
     d.in_w, d.in_h, d.in_c, d.batch = in_shape
@@ -165,7 +167,7 @@ def conv2d(x, w, bias, *, in_shape, w_shape, out_shape, stride, dilation, pad_le
     d.act = act
     np_out = {U8: np.uint8, I8: np.int8, F16: np.float16, F32: np.float32}[out_dtype]
     y = np.zeros(int(np.prod(out_shape)), dtype=np_out)
-    lib().tvxo_conv2d(C.byref(d), _ptr(x), _ptr(w), _ptr(bias), _ptr(y))
+    (lib().tvxo_deconv2d if transposed else lib().tvxo_conv2d)(C.byref(d), _ptr(x), _ptr(w), _ptr(bias), _ptr(y))
     return y
 
 
@@ -291,6 +293,15 @@ def run_case(case):
                       in_dtype=DTYPE_CODE[x["dtype"]], w_dtype=DTYPE_CODE[w["dtype"]],
                       out_dtype=DTYPE_CODE[out["dtype"]], in_q=(s, z), w_q=_q(w["quant"]),
                       out_q=(so, zo))
+    if op["kind"] == "DECONV2D":
+        x, w = ins[0], ins[1]
+        s, z, _ = _q(x["quant"])
+        so, zo, _ = _q(out["quant"])
+        return conv2d(arr[0], arr[1], arr[2] if len(ins) > 2 else None, in_shape=x["shape"], w_shape=w["shape"],
+                      out_shape=out["shape"], stride=a["stride"], dilation=[1, 1], pad_left=a["pad"][0],
+                      pad_top=a["pad"][2], multiplier=0, groups=a.get("groups", 0), in_dtype=DTYPE_CODE[x["dtype"]],
+                      w_dtype=DTYPE_CODE[w["dtype"]], out_dtype=DTYPE_CODE[out["dtype"]], in_q=(s, z),
+                      w_q=_q(w["quant"]), out_q=(so, zo), transposed=True)
     if op["kind"] == "FCL":
         x, w = ins[0], ins[1]
         bias = arr[2] if len(ins) > 2 else None

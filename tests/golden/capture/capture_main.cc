@@ -188,13 +188,13 @@ void EmitOp(OpImpl* op) {
                "], \"attrs\": {\"pad_type\": \"%s\", \"pad\": [%u,%u,%u,%u], "
                "\"stride\": [%u,%u], \"dilation\": [%u,%u], \"ksize\": [%u,%u], "
                "\"multiplier\": %d, \"weights\": %u, \"pool_type\": \"%s\", "
-               "\"round_type\": \"%s\", \"pool_1d\": %s, \"axis\": %u, \"groups\": %d, \"conv_1d\": %s, \"beta\": %.9g, \"sm_axis\": %d, \"layout\": \"%s\", \"kernel_layout\": \"%s\", \"perm\": [",
+               "\"round_type\": \"%s\", \"pool_1d\": %s, \"axis\": %u, \"groups\": %d, \"conv_1d\": %s, \"beta\": %.9g, \"sm_axis\": %d, \"layout\": \"%s\", \"kernel_layout\": \"%s\", \"output_padding\": [%u,%u], \"perm\": [",
                PadName(a.pad_type), a.pad[0], a.pad[1], a.pad[2], a.pad[3],
                a.stride[0], a.stride[1], a.dilation[0], a.dilation[1], a.ksize[0],
                a.ksize[1], a.multiplier, a.weights,
                pool_names[static_cast<int>(a.pool_type)],
                a.round_type == RoundType::CEILING ? "CEILING" : "FLOOR",
-               a.pool_1d ? "true" : "false", a.axis, a.groups, a.conv_1d ? "true" : "false", a.beta, a.sm_axis, LayoutName(op->layout_), LayoutName(a.kernel_layout));
+               a.pool_1d ? "true" : "false", a.axis, a.groups, a.conv_1d ? "true" : "false", a.beta, a.sm_axis, LayoutName(op->layout_), LayoutName(a.kernel_layout), a.output_padding[0], a.output_padding[1]);
   for (size_t i = 0; i < a.perm.size(); ++i) std::fprintf(g_out, "%s%u", i ? "," : "", a.perm[i]);
   std::fprintf(g_out, "]}}");
 }

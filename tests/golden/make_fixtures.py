@@ -32,6 +32,7 @@ SOURCES = {
     "avg_pool": "src/tim/vx/ops/avg_pool_test.cc",
     "softmax": "src/tim/vx/ops/softmax_test.cc",
     "transpose": "src/tim/vx/ops/transpose_test.cc",
+    "deconv2d": "src/tim/vx/ops/deconv2d_test.cc",
     # (file, test suite): only the TEST(suite, ...) bodies of a file that also tests operators outside this path
     "dataconvert": ("src/tim/vx/ops/simple_operations_test.cc", ["DataConvert"]),
     # the source graphs of the layout-inference tests that stay inside this path

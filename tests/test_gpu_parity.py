@@ -511,3 +511,39 @@ def test_dataconvert(oracle, in_dtype, out_dtype):
     want = oracle.convert(x, in_dtype, in_q, out_dtype, out_q)
     got = TC.gpu_convert(x, in_dtype, in_q, out_dtype, out_q)
     assert np.array_equal(got.view(np.uint8), want.view(np.uint8))   # bit-exact, floats included
+
+
+DECONV_GRID = [
+    # n, c, h, w, oc, kh, kw, stride, pad(l, t), output_padding, groups, mode
+    (2, 8, 7, 9, 12, 3, 3, (2, 2), (1, 1), (1, 1), 1, "u8"),        # the usual 2x upsampling
+    (1, 16, 14, 14, 16, 4, 4, (2, 2), (1, 1), (0, 0), 1, "i8pc"),
+    (3, 6, 5, 4, 6, 3, 3, (1, 1), (0, 0), (0, 0), 6, "u8"),          # depthwise form {Kw, Kh, C, 1}
+    (2, 6, 5, 4, 9, 2, 3, (3, 2), (0, 1), (2, 1), 3, "u8pc"),        # grouped, stride > kernel along W
+    (2, 5, 6, 6, 7, 3, 2, (2, 3), (2, 0), (1, 2), 1, "f32"),
+    (1, 4, 9, 8, 4, 5, 5, (2, 2), (2, 2), (1, 1), 1, "f16"),
+    (1, 3, 33, 31, 5, 3, 3, (2, 2), (1, 1), (1, 1), 1, "u8"),
+]
+
+
+@pytest.mark.parametrize("cfg", DECONV_GRID, ids=lambda c: "n%dc%d_%dx%d_oc%d_k%dx%d_s%s_p%s_op%s_g%d_%s" % (
+    c[0], c[1], c[2], c[3], c[4], c[5], c[6], "x".join(map(str, c[7])), "x".join(map(str, c[8])),
+    "x".join(map(str, c[9])), c[10], c[11]))
+def test_deconv2d(oracle, cfg):
+    n, c, h, w, oc, kh, kw, stride, pad, opad, groups, mode = cfg
+    rng = np.random.default_rng(DECONV_GRID.index(cfg) + 77)
+    ow = (w - 1) * stride[0] + kw - 2 * pad[0] + opad[0]
+    oh = (h - 1) * stride[1] + kh - 2 * pad[1] + opad[1]
+    depthwise = groups == c == oc
+    ws = [kw, kh, c, 1] if depthwise else [kw, kh, c // groups, oc]
+    x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=oc, kh=kh, kw=kw, stride=list(stride), dil=[1, 1],
+                              pad=[pad[0], pad[0], pad[1], pad[1]], mult=0, mode=mode, groups=groups)
+    kw_args = dict(kws)
+    kw_args.update(out_shape=[ow, oh, oc, n], w_shape=ws, groups=groups, transposed=True)
+    want = oracle.conv2d(x, wt, b, **kw_args)
+    for const_weights in (True, False):
+        got = TC.gpu_conv2d(x, wt, b, const_weights=const_weights, want_kernel="deconv2d_generic", **kw_args)
+        if mode in ("f32", "f16"):
+            assert np.allclose(got.astype(np.float32), want.astype(np.float32), rtol=1e-2, atol=1e-2)  # tolerance of the path
+        else:
+            assert np.array_equal(got, want)
+            assert 0.02 < np.mean((want > want.min()) & (want < want.max())), "saturated test data"

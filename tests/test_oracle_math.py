@@ -246,3 +246,84 @@ def test_convert_restatement_vs_numpy(oracle):
     h = oracle.convert(f, 3, (1.0, 0), 2, (1.0, 0))
     assert np.array_equal(h.view(np.uint16), f.astype(np.float16).view(np.uint16))
     assert np.array_equal(oracle.convert(h, 2, (1.0, 0), 3, (1.0, 0)), h.astype(np.float32))
+
+
+def _deconv_bruteforce(x, w, bias, xs, ws, os_, stride, pad, groups):
+    """Pure-Python gather form on integers: out(ox, oy) sums in(ix, iy) * w(kx, ky) over ix * s - pad + kx == ox."""
+    W, H, C, N = xs
+    KW, KH, ICG, OC = ws
+    OW, OH = os_[0], os_[1]
+    y = np.zeros((N, OC, OH, OW), dtype=np.int64)
+    xr = x.reshape(N, C, H, W).astype(np.int64)
+    wr = w.reshape(OC, ICG, KH, KW).astype(np.int64)
+    for n in range(N):
+        for oc in range(OC):
+            ic0 = (oc // (OC // groups)) * ICG
+            for oy in range(OH):
+                for ox in range(OW):
+                    acc = int(bias[oc]) if bias is not None else 0
+                    for ci in range(ICG):
+                        for ky in range(KH):
+                            ty = oy + pad[1] - ky
+                            if ty < 0 or ty % stride[1] or ty // stride[1] >= H:
+                                continue
+                            for kx in range(KW):
+                                tx = ox + pad[0] - kx
+                                if tx < 0 or tx % stride[0] or tx // stride[0] >= W:
+                                    continue
+                                acc += xr[n, ic0 + ci, ty // stride[1], tx // stride[0]] * wr[oc, ci, ky, kx]
+                    y[n, oc, oy, ox] = acc
+    return y.reshape(-1)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_deconv_restatement_vs_bruteforce_and_adjoint(oracle, seed):
+    rng = np.random.default_rng(100 + seed)
+    groups = [1, 1, 2, 1, 3, 1][seed]
+    icg, ocg = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+    C, OC = icg * groups, ocg * groups
+    W, H, N = int(rng.integers(2, 6)), int(rng.integers(2, 6)), int(rng.integers(1, 3))
+    KW, KH = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+    stride = [int(rng.integers(1, 4)), int(rng.integers(1, 4))]
+    pad = [int(rng.integers(0, KW)), int(rng.integers(0, KH))]
+    opad = [int(rng.integers(0, stride[0])), int(rng.integers(0, stride[1]))]
+    OW = (W - 1) * stride[0] + KW - pad[0] - int(rng.integers(0, 2)) + opad[0]
+    OH = (H - 1) * stride[1] + KH - pad[1] - int(rng.integers(0, 2)) + opad[1]
+    if OW < 1 or OH < 1:
+        pytest.skip("empty output")
+    xs, ws, os_ = [W, H, C, N], [KW, KH, icg, OC], [OW, OH, OC, N]
+    # (1) float32 operands holding small integers, unit scales: the oracle's scatter against a gather in Python
+    x = rng.integers(-5, 6, int(np.prod(xs))).astype(np.float32)
+    w = rng.integers(-4, 5, int(np.prod(ws))).astype(np.float32)
+    b = rng.integers(-9, 10, OC).astype(np.float32)
+    got = oracle.conv2d(x, w, b, in_shape=xs, w_shape=ws, out_shape=os_, stride=stride, dilation=[1, 1],
+                        pad_left=pad[0], pad_top=pad[1], multiplier=0, groups=groups, in_dtype=3, w_dtype=3,
+                        out_dtype=3, transposed=True)
+    want = _deconv_bruteforce(x, w, b, xs, ws, os_, stride, pad, groups)
+    assert np.array_equal(got.astype(np.int64), want)
+    # (2) adjoint of the (separately pinned) convolution: <conv(u), v> == <u, deconv(v)> when the extents are
+    # the exact ones; the convolution's weights are the same numbers with the channel roles swapped
+    if groups == 1 and opad == [0, 0]:
+        OWf, OHf = (W - 1) * stride[0] + KW - 2 * pad[0], (H - 1) * stride[1] + KH - 2 * pad[1]
+        if OWf >= KW and OHf >= KH and pad[0] < KW and pad[1] < KH and OWf > 0 and OHf > 0:
+            v = x                                             # deconv input  {W, H, C, N}
+            u = rng.integers(-5, 6, OWf * OHf * OC * N).astype(np.float32)   # conv input {OWf, OHf, OC, N}
+            dv = oracle.conv2d(v, w, None, in_shape=xs, w_shape=ws, out_shape=[OWf, OHf, OC, N], stride=stride,
+                               dilation=[1, 1], pad_left=pad[0], pad_top=pad[1], multiplier=0, in_dtype=3, w_dtype=3,
+                               out_dtype=3, transposed=True)
+            w_conv = np.ascontiguousarray(w.reshape(OC, icg, KH, KW).transpose(1, 0, 2, 3)).reshape(-1)  # [C][OC]
+            cu = oracle.conv2d(u, w_conv, None, in_shape=[OWf, OHf, OC, N], w_shape=[KW, KH, OC, C],
+                               out_shape=xs, stride=stride, dilation=[1, 1], pad_left=pad[0], pad_top=pad[1],
+                               multiplier=0, in_dtype=3, w_dtype=3, out_dtype=3)
+            assert float(np.dot(cu.astype(np.float64), v)) == float(np.dot(u, dv.astype(np.float64)))
+    # (3) quantized: requantization and zero points as for Conv2d, checked through the integer accumulators
+    xq = rng.integers(0, 256, int(np.prod(xs)), dtype=np.uint8)
+    wq = rng.integers(0, 256, int(np.prod(ws)), dtype=np.uint8)
+    bq = rng.integers(-300, 300, OC).astype(np.int32)
+    acc = _deconv_bruteforce(xq.astype(np.int64) - 121, wq.astype(np.int64) - 130, bq, xs, ws, os_, stride, pad, groups)
+    mult, shift = oracle.quantize_multiplier(0.5 * 0.25 / 37.0)
+    want_q = np.clip(np.array([oracle.requant(int(a), mult, shift) for a in acc]) + 100, 0, 255)
+    got_q = oracle.conv2d(xq, wq, bq, in_shape=xs, w_shape=ws, out_shape=os_, stride=stride, dilation=[1, 1],
+                          pad_left=pad[0], pad_top=pad[1], multiplier=0, groups=groups, in_dtype=0, w_dtype=0,
+                          out_dtype=0, in_q=(0.5, 121), w_q=(0.25, 130, None), out_q=(37.0, 100), transposed=True)
+    assert np.array_equal(got_q, want_q)

@@ -11,7 +11,8 @@ import tvx_oracle as O
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 GOLDEN_FILES = ["conv2d", "depthwise_conv", "grouped_conv2d", "conv1d", "fullyconnected", "max_pool", "avg_pool", "softmax",
-                "transpose", "dataconvert", "layout_inference"]
+                "transpose", "dataconvert", "layout_inference",
+                "deconv2d"]
 
 
 def load_cases(name):
@@ -79,7 +80,7 @@ def _wq(desc, w_q, keep):
 
 def gpu_conv2d(x, w, bias, *, in_shape, w_shape, out_shape, stride, dilation, pad_left, pad_top,
                multiplier, in_dtype, w_dtype, out_dtype, in_q=(1.0, 0), w_q=(1.0, 0, None),
-               out_q=(1.0, 0), act=0, const_weights=True, want_kernel=None, groups=0):
+               out_q=(1.0, 0), act=0, const_weights=True, want_kernel=None, groups=0, transposed=False):
     T = tvx()
     d = T.Conv2dDesc()
     d.groups = groups
@@ -95,7 +96,7 @@ def gpu_conv2d(x, w, bias, *, in_shape, w_shape, out_shape, stride, dilation, pa
     _wq(d, w_q, keep)
     d.out_scale, d.out_zp = out_q
     d.activation = act
-    op = T.conv2d_create(d, w if const_weights else None, bias)
+    op = (T.deconv2d_create if transposed else T.conv2d_create)(d, w if const_weights else None, bias)
     if want_kernel is not None:
         assert op.kernel_name == want_kernel, op.kernel_name
     import torch
@@ -256,6 +257,16 @@ def run_case_gpu(case):
                           w_dtype=code[w["dtype"]], out_dtype=code[out["dtype"]], in_q=(s, z),
                           w_q=O._q(w["quant"]), out_q=(so, zo),
                           const_weights=(w["attr"] == "CONSTANT"))
+    if op["kind"] == "DECONV2D":
+        x, w = ins[0], ins[1]
+        s, z, _ = O._q(x["quant"])
+        so, zo, _ = O._q(out["quant"])
+        return gpu_conv2d(arr[0], arr[1], arr[2] if len(ins) > 2 else None, in_shape=x["shape"], w_shape=w["shape"],
+                          out_shape=out["shape"], stride=a["stride"], dilation=[1, 1], pad_left=a["pad"][0],
+                          pad_top=a["pad"][2], multiplier=0, groups=a.get("groups", 0), in_dtype=code[x["dtype"]],
+                          w_dtype=code[w["dtype"]], out_dtype=code[out["dtype"]], in_q=(s, z),
+                          w_q=O._q(w["quant"]), out_q=(so, zo), const_weights=(w["attr"] == "CONSTANT"),
+                          transposed=True)
     if op["kind"] == "FCL":
         x, w = ins[0], ins[1]
         k = int(np.prod(x["shape"][:a["axis"] + 1]))

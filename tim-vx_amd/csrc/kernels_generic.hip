@@ -36,7 +36,22 @@ struct ConvArgs {
   int stride_w, stride_h, dil_w, dil_h, pad_left, pad_top, multiplier;
   int in_zp, w_zp, out_zp, lo, hi, act;
   int groups;  // >= 1
+  int transposed;  // DeConv2d: every input pixel scatters a window (gathered here per output)
 };
+
+// Input row (column) that kernel tap k of output row o reads, or -1. Convolution:
+// o * stride - pad + k * dil. Transposed convolution: the i with i * stride - pad + k = o.
+__device__ __forceinline__ int TapSource(const ConvArgs& a, int o, int k, int stride, int dil, int pad, int extent) {
+  int i;
+  if (a.transposed) {
+    const int t = o + pad - k;
+    if (t < 0 || t % stride) return -1;
+    i = t / stride;
+  } else {
+    i = o * stride - pad + k * dil;
+  }
+  return i >= 0 && i < extent ? i : -1;
+}
 
 // Input channels one output channel reads, and the first of them: all of them (dense), one
 // (depthwise, oc = ic * multiplier + j) or the channels of its group.
@@ -68,11 +83,11 @@ ConvQuantKernel(ConvArgs a, const XT* __restrict__ x, const WT* __restrict__ w,
     const XT* xp = x + (static_cast<uint64_t>(n) * a.in_c + ic0 + ci) * a.in_h * a.in_w;
     const WT* wp = w + (static_cast<uint64_t>(oc) * ic_per_oc + ci) * a.k_h * a.k_w;
     for (int ky = 0; ky < a.k_h; ++ky) {
-      const int ih = oh * a.stride_h - a.pad_top + ky * a.dil_h;
-      if (ih < 0 || ih >= a.in_h) continue;
+      const int ih = TapSource(a, oh, ky, a.stride_h, a.dil_h, a.pad_top, a.in_h);
+      if (ih < 0) continue;
       for (int kx = 0; kx < a.k_w; ++kx) {
-        const int iw = ow * a.stride_w - a.pad_left + kx * a.dil_w;
-        if (iw < 0 || iw >= a.in_w) continue;
+        const int iw = TapSource(a, ow, kx, a.stride_w, a.dil_w, a.pad_left, a.in_w);
+        if (iw < 0) continue;
         acc += (static_cast<int32_t>(xp[ih * a.in_w + iw]) - a.in_zp) *
                (static_cast<int32_t>(wp[ky * a.k_w + kx]) - a.w_zp);
       }
@@ -99,11 +114,11 @@ ConvFloatKernel(ConvArgs a, const T* __restrict__ x, const T* __restrict__ w,
     const T* xp = x + (static_cast<uint64_t>(n) * a.in_c + ic0 + ci) * a.in_h * a.in_w;
     const T* wp = w + (static_cast<uint64_t>(oc) * ic_per_oc + ci) * a.k_h * a.k_w;
     for (int ky = 0; ky < a.k_h; ++ky) {
-      const int ih = oh * a.stride_h - a.pad_top + ky * a.dil_h;
-      if (ih < 0 || ih >= a.in_h) continue;
+      const int ih = TapSource(a, oh, ky, a.stride_h, a.dil_h, a.pad_top, a.in_h);
+      if (ih < 0) continue;
       for (int kx = 0; kx < a.k_w; ++kx) {
-        const int iw = ow * a.stride_w - a.pad_left + kx * a.dil_w;
-        if (iw < 0 || iw >= a.in_w) continue;
+        const int iw = TapSource(a, ow, kx, a.stride_w, a.dil_w, a.pad_left, a.in_w);
+        if (iw < 0) continue;
         acc += ToFloat(xp[ih * a.in_w + iw]) * ToFloat(wp[ky * a.k_w + kx]);
       }
     }
@@ -120,7 +135,8 @@ int ConvGenericRun(tvx_op* op, const void* in0, const void* in1, void* out, hipS
              static_cast<int>(d.stride_w), static_cast<int>(d.stride_h),
              static_cast<int>(d.dilation_w), static_cast<int>(d.dilation_h),
              static_cast<int>(d.pad_left), static_cast<int>(d.pad_top), d.multiplier,
-             d.in_zp, op->w_zp, d.out_zp, op->act_lo, op->act_hi, d.activation, d.groups > 1 ? d.groups : 1};
+             d.in_zp, op->w_zp, d.out_zp, op->act_lo, op->act_hi, d.activation, d.groups > 1 ? d.groups : 1,
+             op->kind == OP_DECONV2D ? 1 : 0};
   const void* w = op->has_const_weights ? op->weights.ptr : in1;
   const uint64_t total = static_cast<uint64_t>(d.out_w) * d.out_h * d.out_c * d.batch;
   const dim3 grid(Blocks(total)), block(kBlock);
@@ -743,7 +759,7 @@ int ConvGenericSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w, const 
   int s = UploadWeightsAndBias(op, w, w_bytes, b, static_cast<size_t>(d->out_c) * 4);
   if (s != TVX_OK) return s;
   op->run = ConvGenericRun;
-  op->kernel_name = "conv2d_generic";
+  op->kernel_name = op->kind == OP_DECONV2D ? "deconv2d_generic" : "conv2d_generic";
   return TVX_OK;
 }
 

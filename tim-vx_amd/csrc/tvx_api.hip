@@ -319,6 +319,54 @@ int tvx_conv2d_create(const tvx_conv2d_desc* d, const void* weights_host,
   return TVX_OK;
 }
 
+int tvx_deconv2d_create(const tvx_conv2d_desc* d, const void* weights_host, const void* bias_host,
+                        tvx_op** out) {
+  if (!d || !out) return SetError(TVX_E_INVALID, "tvx_deconv2d_create: null argument");
+  *out = nullptr;
+  if (!d->in_w || !d->in_h || !d->in_c || !d->batch || !d->k_w || !d->k_h || !d->out_w || !d->out_h ||
+      !d->out_c || !d->stride_w || !d->stride_h)
+    return SetError(TVX_E_INVALID, "tvx_deconv2d_create: zero extent or stride");
+  if (d->dilation_w != 1 || d->dilation_h != 1)
+    return SetError(TVX_E_INVALID, "tvx_deconv2d_create: dilation must be 1");
+  if (d->multiplier != 0 && (d->multiplier != 1 || d->out_c != d->in_c))
+    return SetError(TVX_E_INVALID, "tvx_deconv2d_create: the depthwise form has multiplier 1 and out_c == in_c");
+  if (d->groups < 0 || (d->groups > 1 && (d->multiplier != 0 || d->in_c % d->groups || d->out_c % d->groups)))
+    return SetError(TVX_E_INVALID, "tvx_deconv2d_create: %d groups do not divide in_c %u / out_c %u (or multiplier set)",
+                    d->groups, d->in_c, d->out_c);
+  // no output pixel beyond what the last input pixel's window reaches
+  if (static_cast<uint64_t>(d->out_w) + d->pad_left > static_cast<uint64_t>(d->in_w - 1) * d->stride_w + d->k_w + d->stride_w - 1 ||
+      static_cast<uint64_t>(d->out_h) + d->pad_top > static_cast<uint64_t>(d->in_h - 1) * d->stride_h + d->k_h + d->stride_h - 1)
+    return SetError(TVX_E_INVALID, "tvx_deconv2d_create: output extent reaches past the last input window");
+  int s = CheckOperandTypes(d->in_dtype, d->w_dtype, d->out_dtype, "tvx_deconv2d_create");
+  if (s != TVX_OK) return s;
+  if ((s = NoGpu()) != TVX_OK) return s;
+  tvx_op* op = new (std::nothrow) tvx_op();
+  if (!op) return SetError(TVX_E_NOMEM, "tvx_deconv2d_create: host allocation failed");
+  op->kind = OP_DECONV2D;
+  op->conv = *d;
+  if (d->groups > 1 && static_cast<uint32_t>(d->groups) == d->in_c && d->out_c == d->in_c) {
+    op->conv.multiplier = 1;  // one channel per group: the depthwise form
+    op->conv.groups = 0;
+  }
+  const tvx_conv2d_desc norm = op->conv;
+  op->conv.w_scales = nullptr;
+  op->quantized = IsQuant(d->in_dtype);
+  op->has_const_weights = weights_host != nullptr;
+  op->w_zp = d->w_scales ? 0 : d->w_zp;
+  if (op->quantized) {
+    std::vector<int32_t>&mult = op->h_mult, &shift = op->h_shift;
+    s = BuildRequantTables(d->out_c, d->in_scale, d->w_scale, d->w_scales, d->out_scale, &mult, &shift);
+    if (s == TVX_OK) s = op->mult.Upload(mult.data(), mult.size() * 4);
+    if (s == TVX_OK) s = op->shift.Upload(shift.data(), shift.size() * 4);
+    ActRange(d->out_dtype, d->out_scale, d->out_zp, d->activation, &op->act_lo, &op->act_hi);
+    if (s != TVX_OK) { delete op; return s; }
+  }
+  s = ConvGenericSetup(op, &norm, weights_host, bias_host);
+  if (s != TVX_OK) { delete op; return s; }
+  *out = op;
+  return TVX_OK;
+}
+
 int tvx_fully_connected_create(const tvx_fc_desc* d, const void* weights_host,
                                const void* bias_host, tvx_op** out) {
   if (!d || !out) return SetError(TVX_E_INVALID, "tvx_fully_connected_create: null argument");
@@ -477,7 +525,7 @@ int tvx_transpose_create(const tvx_transpose_desc* d, tvx_op** out) {
 int tvx_op_run(tvx_op* op, const void* in0, const void* in1, void* out_ptr, void* stream) {
   if (!op || !op->run) return SetError(TVX_E_INVALID, "tvx_op_run: null operator");
   if (!in0 || !out_ptr) return SetError(TVX_E_INVALID, "tvx_op_run: null tensor pointer");
-  if ((op->kind == OP_CONV2D || op->kind == OP_FC) && !op->has_const_weights && !in1)
+  if ((op->kind == OP_CONV2D || op->kind == OP_DECONV2D || op->kind == OP_FC) && !op->has_const_weights && !in1)
     return SetError(TVX_E_INVALID, "tvx_op_run: operator was created without weights, pass them as in1");
   if (op->kind == OP_ADD && !in1) return SetError(TVX_E_INVALID, "tvx_op_run: Add needs two operands");
   return op->run(op, in0, in1, out_ptr, static_cast<hipStream_t>(stream));
@@ -486,7 +534,7 @@ int tvx_op_run(tvx_op* op, const void* in0, const void* in1, void* out_ptr, void
 int tvx_op_run3(tvx_op* op, const void* in0, const void* in1, const void* in2, void* out_ptr, void* stream) {
   if (!in2) return tvx_op_run(op, in0, in1, out_ptr, stream);
   if (!op || !op->run) return SetError(TVX_E_INVALID, "tvx_op_run3: null operator");
-  if ((op->kind != OP_CONV2D && op->kind != OP_FC) || op->has_const_weights || op->bias.ptr)
+  if ((op->kind != OP_CONV2D && op->kind != OP_DECONV2D && op->kind != OP_FC) || op->has_const_weights || op->bias.ptr)
     return SetError(TVX_E_UNSUPPORTED,
                     "tvx_op_run3: a run-time bias goes with a Conv2d / FullyConnected created without weights and bias");
   op->bias_at_run = in2;

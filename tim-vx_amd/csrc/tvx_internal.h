@@ -24,7 +24,7 @@ int SetError(int status, const char* fmt, ...);
                              hipGetErrorString(e_), __FILE__, __LINE__);        \
   } while (0)
 
-enum OpKind { OP_CONV2D = 1, OP_FC, OP_POOL2D, OP_ACTIVATION, OP_ADD, OP_SOFTMAX, OP_TRANSPOSE, OP_CONVERT };
+enum OpKind { OP_CONV2D = 1, OP_FC, OP_POOL2D, OP_ACTIVATION, OP_ADD, OP_SOFTMAX, OP_TRANSPOSE, OP_CONVERT, OP_DECONV2D };
 
 // Device buffer owned by an operator, released in its destructor.
 struct DeviceBuffer {

@@ -40,7 +40,7 @@ _DEFAULT_ATTRS = {"pad_type": "AUTO", "pad": [0, 0, 0, 0], "stride": [1, 1], "di
                   "ksize": [0, 0], "multiplier": 0, "weights": 0, "pool_type": "MAX",
                   "round_type": "FLOOR", "pool_1d": False, "axis": 0, "beta": 1.0, "sm_axis": 0,
                   "new_shape": [], "groups": 0, "conv_1d": False, "perm": [],
-                  "layout": "ANY", "kernel_layout": "ANY"}
+                  "layout": "ANY", "kernel_layout": "ANY", "output_padding": [0, 0]}
 
 
 def op(kind, inputs, outputs, **attrs):
@@ -82,7 +82,7 @@ def write_graphs(graphs, txt_path, blob_path, bench=None):
                 f += [a["pad_type"]] + list(a["pad"]) + list(a["stride"]) + list(a["dilation"]) + list(a["ksize"])
                 f += [a["multiplier"], a["weights"], a["pool_type"], a["round_type"], int(bool(a["pool_1d"])),
                       a["axis"], "%.9g" % a["beta"], a["sm_axis"], len(a["new_shape"])] + list(a["new_shape"]) + [a["groups"], int(bool(a["conv_1d"]))]
-                f += [len(a["perm"])] + list(a["perm"]) + [a["layout"], a["kernel_layout"]]
+                f += [len(a["perm"])] + list(a["perm"]) + [a["layout"], a["kernel_layout"]] + list(a["output_padding"])
                 txt.write(" ".join(str(x) for x in f) + "\n")
             if g.get("layout_inference"):
                 txt.write("infer\n")

@@ -257,6 +257,40 @@ class Reshape : public BuiltinOp {
   std::vector<uint32_t> size_;
 };
 
+// reference: include/tim/vx/ops/deconv.h:54-86
+// The transpose of Conv2d: weights {Kw, Kh, Ic, Oc}, or {Kw, Kh, C, 1} for the depthwise form
+// (group == channel count); out = (in - 1) * stride + k - pads + output_padding.
+class DeConv2d : public BuiltinOp {
+ public:
+  DeConv2d(Graph* graph, int32_t oc_count_, PadType pad_type,
+           const std::array<uint32_t, 2>& ksize,
+           const std::array<uint32_t, 2>& stride,
+           const std::array<uint32_t, 2>& output_padding,
+           DataLayout input_layout = DataLayout::WHCN,
+           DataLayout kernel_layout = DataLayout::WHIcOc);
+  DeConv2d(Graph* graph, int32_t oc_count_, PadType pad_type,
+           const std::array<uint32_t, 2>& ksize,
+           const std::array<uint32_t, 2>& stride,
+           const std::array<uint32_t, 2>& output_padding,
+           const std::array<uint32_t, 4>& pad, const uint32_t group = 1,
+           DataLayout input_layout = DataLayout::WHCN,
+           DataLayout kernel_layout = DataLayout::WHIcOc);
+  DataLayout KernelDataLayout() { return kernel_layout_; }
+  std::shared_ptr<Operation> Clone(
+      std::shared_ptr<Graph>& graph) const override;
+
+ protected:
+  void OnBindInputPostProc(const std::shared_ptr<Tensor>& tensor, int32_t input_idx) override;
+  const uint32_t oc_count_;
+  const PadType pad_type_;
+  const std::array<uint32_t, 2> ksize_;
+  const std::array<uint32_t, 2> stride_;
+  const std::array<uint32_t, 2> output_padding_;
+  const std::array<uint32_t, 4> pad_;
+  const uint32_t group_;
+  const DataLayout kernel_layout_;
+};
+
 // reference: include/tim/vx/ops/simple_operations.h:118 (DataConvert only)
 // Converts between tensor types and quantizations: quantize, dequantize, requantize.
 class DataConvert : public BuiltinOp {

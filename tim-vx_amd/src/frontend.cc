@@ -37,6 +37,7 @@ const char* OpKindName(OpKind k) {
     case OpKind::RESHAPE: return "RESHAPE";
     case OpKind::TRANSPOSE: return "TRANSPOSE";
     case OpKind::DATACONVERT: return "DATACONVERT";
+    case OpKind::DECONV2D: return "DECONV2D";
   }
   return "?";
 }
@@ -997,6 +998,44 @@ Reshape::Reshape(Graph* graph, const std::vector<uint32_t>& target_shape)
 }
 std::shared_ptr<Operation> Reshape::Clone(std::shared_ptr<Graph>& graph) const {
   return graph->CreateOperation<Reshape>(size_);
+}
+
+// ---- DeConv2d (reference: src/tim/vx/ops/deconv.cc:36-88) ------------------------------------
+DeConv2d::DeConv2d(Graph* graph, int32_t oc_count, PadType pad_type, const std::array<uint32_t, 2>& ksize,
+                   const std::array<uint32_t, 2>& stride, const std::array<uint32_t, 2>& output_padding,
+                   DataLayout input_layout, DataLayout kernel_layout)
+    : DeConv2d(graph, oc_count, pad_type, ksize, stride, output_padding, {0, 0, 0, 0}, 1, input_layout,
+               kernel_layout) {}
+
+DeConv2d::DeConv2d(Graph* graph, int32_t oc_count, PadType pad_type, const std::array<uint32_t, 2>& ksize,
+                   const std::array<uint32_t, 2>& stride, const std::array<uint32_t, 2>& output_padding,
+                   const std::array<uint32_t, 4>& pad, const uint32_t group, DataLayout input_layout,
+                   DataLayout kernel_layout)
+    : BuiltinOp(graph, K(OpKind::DECONV2D), 0, 0, input_layout),
+      oc_count_(oc_count), pad_type_(pad_type), ksize_(ksize), stride_(stride),
+      output_padding_(output_padding), pad_(pad), group_(group), kernel_layout_(kernel_layout) {
+  OpAttrs& a = impl_->attrs_;
+  a.kernel_layout = kernel_layout_;
+  // the pad type is carried along but the explicit pads are what sizes the output, as in the
+  // reference (vsi_nn_op_deconvolution.c:463-481)
+  a.pad_type = PadType::AUTO;
+  for (int i = 0; i < 4; ++i) a.pad[i] = pad_[i];
+  for (int i = 0; i < 2; ++i) {
+    a.stride[i] = stride_[i];
+    a.ksize[i] = ksize_[i];
+    a.output_padding[i] = output_padding_[i];
+  }
+  a.weights = oc_count_;
+  a.groups = static_cast<int32_t>(group_);
+}
+
+std::shared_ptr<Operation> DeConv2d::Clone(std::shared_ptr<Graph>& graph) const {
+  return graph->CreateOperation<DeConv2d>(static_cast<int32_t>(oc_count_), pad_type_, ksize_, stride_,
+                                          output_padding_, pad_, group_, impl_->layout_, kernel_layout_);
+}
+
+void DeConv2d::OnBindInputPostProc(const std::shared_ptr<Tensor>& tensor, int32_t) {
+  PromoteHalfBias(this, impl_.get(), tensor);
 }
 
 DataConvert::DataConvert(Graph* graph) : BuiltinOp(graph, K(OpKind::DATACONVERT), 1, 1) {}

@@ -218,6 +218,63 @@ bool SetupConv(OpImpl* op) {
   return AssignShape(y, out, "CONV2D", 2);
 }
 
+// reference: src/tim/vx/internal/src/ops/vsi_nn_op_deconvolution.c:217-218, 456-497
+bool SetupDeconv(OpImpl* op) {
+  if (op->inputs_tensor_.size() < 2 || op->outputs_tensor_.size() != 1) {
+    VSILOGE("DECONV2D needs {input, weight[, bias]} and one output");
+    return false;
+  }
+  TensorImpl *x = Impl(op->inputs_tensor_[0]), *w = Impl(op->inputs_tensor_[1]);
+  TensorImpl* b = op->inputs_tensor_.size() > 2 && !op->inputs_tensor_[2]->IsPlaceHolder()
+                      ? Impl(op->inputs_tensor_[2]) : nullptr;
+  TensorImpl* y = Impl(op->outputs_tensor_[0]);
+  if (op->layout_ != DataLayout::WHCN && op->layout_ != DataLayout::ANY) {
+    VSILOGE("DECONV2D: only WHCN activations are supported");
+    return false;
+  }
+  const ShapeType &xs = x->spec_.shape_, &ws = w->spec_.shape_;
+  if (xs.size() != 4 || ws.size() != 4) {
+    VSILOGE("DECONV2D: input and weight must be 4-D");
+    return false;
+  }
+  if (!BiasScaleConsistent(x->spec_, w->spec_, b ? &b->spec_ : nullptr)) return false;
+  if (!WeightPairSupported(x->spec_, w->spec_)) {
+    VSILOGE("Inputs/Outputs data type not support: %s x %s", DataTypeName(x->spec_.datatype_),
+            DataTypeName(w->spec_.datatype_));
+    return false;
+  }
+  OpAttrs& a = op->attrs_;
+  if (a.groups == 0) a.groups = 1;
+  const uint32_t g = static_cast<uint32_t>(a.groups);
+  uint32_t oc;
+  if (g > 1 && g == xs[2] && ws[3] == 1) {
+    oc = ws[2];  // depthwise form {Kw, Kh, C, 1}
+    if (oc != xs[2]) {
+      VSILOGE("DECONV2D: depthwise weight must be {Kw, Kh, C, 1} with C = input channels %u", xs[2]);
+      return false;
+    }
+  } else {
+    oc = ws[3];
+    if (xs[2] % g != 0 || oc % g != 0 || ws[2] != xs[2] / g) {
+      VSILOGE("DECONV2D: weight Ic %u != input C %u / group %u", ws[2], xs[2], g);
+      return false;
+    }
+  }
+  if (b && static_cast<uint32_t>(b->spec_.GetElementNum()) != oc) {
+    VSILOGE("DECONV2D: bias has %lld elements, expected %u", static_cast<long long>(b->spec_.GetElementNum()), oc);
+    return false;
+  }
+  a.ksize[0] = ws[0];
+  a.ksize[1] = ws[1];
+  const int64_t ow = (static_cast<int64_t>(xs[0]) - 1) * a.stride[0] + ws[0] - a.pad[0] - a.pad[1] + a.output_padding[0];
+  const int64_t oh = (static_cast<int64_t>(xs[1]) - 1) * a.stride[1] + ws[1] - a.pad[2] - a.pad[3] + a.output_padding[1];
+  if (ow <= 0 || oh <= 0 || !a.stride[0] || !a.stride[1]) {
+    VSILOGE("DECONV2D: empty output");
+    return false;
+  }
+  return AssignShape(y, ShapeType{static_cast<uint32_t>(ow), static_cast<uint32_t>(oh), oc, xs[3]}, "DECONV2D", 2);
+}
+
 bool SetupFcl(OpImpl* op) {
   if (op->inputs_tensor_.size() < 2 || op->outputs_tensor_.size() != 1) {
     VSILOGE("FCL needs {input, weight[, bias]} and one output");
@@ -420,6 +477,7 @@ bool GraphImpl::VerifyAndInfer() {
       case OpKind::RESHAPE: ok = SetupReshape(im); break;
       case OpKind::TRANSPOSE: ok = SetupTranspose(im); break;
       case OpKind::DATACONVERT: ok = SetupSameShape(im, "DATACONVERT", 1); break;
+      case OpKind::DECONV2D: ok = SetupDeconv(im); break;
     }
     if (!ok) {
       VSILOGE("setup of %s (uid %u) failed", OpKindName(im->kind_), im->uid_);

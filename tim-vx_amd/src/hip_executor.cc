@@ -127,6 +127,7 @@ class HipExecutor : public Executor {
         case OpKind::RESHAPE: break;  // aliased
         case OpKind::TRANSPOSE: ok = AddTranspose(im, out); break;
         case OpKind::DATACONVERT: ok = AddConvert(im, out); break;
+        case OpKind::DECONV2D: ok = AddConv(im, out, TVX_ACT_NONE, true); break;
       }
       if (!ok) return false;
     }
@@ -221,7 +222,7 @@ class HipExecutor : public Executor {
     }
   }
 
-  bool AddConv(OpImpl* im, TensorImpl* out, int act) {
+  bool AddConv(OpImpl* im, TensorImpl* out, int act, bool transposed = false) {
     TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
     TensorImpl* w = static_cast<TensorImpl*>(im->inputs_tensor_[1].get());
     TensorImpl* b = im->inputs_tensor_.size() > 2 && !im->inputs_tensor_[2]->IsPlaceHolder()
@@ -238,7 +239,7 @@ class HipExecutor : public Executor {
     d.k_w = ws[0]; d.k_h = ws[1];
     d.out_w = os[0]; d.out_h = os[1]; d.out_c = os[2];
     d.stride_w = a.stride[0]; d.stride_h = a.stride[1];
-    d.dilation_w = a.dilation[0]; d.dilation_h = a.dilation[1];
+    d.dilation_w = transposed ? 1 : a.dilation[0]; d.dilation_h = transposed ? 1 : a.dilation[1];
     d.pad_left = a.pad[0]; d.pad_top = a.pad[2];
     d.multiplier = a.multiplier;
     d.groups = a.groups;
@@ -254,8 +255,9 @@ class HipExecutor : public Executor {
     const bool bias_at_run = b && !b->IsConstTensor();
     const bool const_w = w->IsConstTensor() && w->HostData() && !bias_at_run;
     tvx_op* op = nullptr;
-    if (tvx_conv2d_create(&d, const_w ? w->HostData() : nullptr, b && !bias_at_run ? b->HostData() : nullptr, &op) != TVX_OK)
-      return Fail("tvx_conv2d_create");
+    if ((transposed ? tvx_deconv2d_create : tvx_conv2d_create)(&d, const_w ? w->HostData() : nullptr,
+                                                                 b && !bias_at_run ? b->HostData() : nullptr, &op) != TVX_OK)
+      return Fail(transposed ? "tvx_deconv2d_create" : "tvx_conv2d_create");
     Push(op, im, x, const_w ? nullptr : w, out, bias_at_run ? b : nullptr);
     return true;
   }

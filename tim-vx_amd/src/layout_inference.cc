@@ -263,6 +263,7 @@ struct Walk {
       }
       case OpKind::FCL:
       case OpKind::RESHAPE:
+      case OpKind::DECONV2D:  // taken in the source layout (WHCN is what it accepts)
       case OpKind::TRANSPOSE: {
         for (const auto& t : ins)
           new_ins.push_back(t->IsPlaceHolder() ? dst->CreateTensorPlaceHolder() : InLayout(t, Identity(RankOf(t))));

@@ -32,7 +32,7 @@ int TvxLogThreshold();
 #define VSILOGD(...) TVX_LOG(::tim::vx::TVX_LOG_DEBUG, "D ", __VA_ARGS__)
 
 enum class OpKind : uint32_t {
-  CONV2D = 1, FCL, POOL, RELU, RELU6, ADD, SOFTMAX, RESHAPE, TRANSPOSE, DATACONVERT
+  CONV2D = 1, FCL, POOL, RELU, RELU6, ADD, SOFTMAX, RESHAPE, TRANSPOSE, DATACONVERT, DECONV2D
 };
 const char* OpKindName(OpKind k);
 
@@ -48,6 +48,7 @@ struct OpAttrs {
   int32_t multiplier = 0;
   int32_t groups = 0;  // GroupedConv2d: > 1
   DataLayout kernel_layout = DataLayout::WHIcOc;  // read by layout inference only
+  uint32_t output_padding[2] = {0, 0};  // DeConv2d
   bool conv_1d = false;  // Conv1d: {W, C, N} tensors, the 2-D operator on rows of height one
   uint32_t weights = 0;
   // pool

@@ -177,6 +177,8 @@ int main(int argc, char** argv) {
       for (auto& d : perm) ss >> d;
       std::string layout_s = "ANY", klayout_s = "ANY";
       ss >> layout_s >> klayout_s;
+      std::array<uint32_t, 2> out_pad = {0, 0};
+      ss >> out_pad[0] >> out_pad[1];
       if (!ss) { std::fprintf(stderr, "malformed op record in %s\n", name.c_str()); return 2; }
       const DataLayout layout = ParseLayout(layout_s, DataLayout::WHCN), klayout = ParseLayout(klayout_s, DataLayout::WHIcOc);
       const RoundType rnd = round_type == "CEILING" ? RoundType::CEILING : RoundType::FLOOR;
@@ -212,6 +214,9 @@ int main(int argc, char** argv) {
         op = graph->CreateOperation<ops::Softmax>(beta, sm_axis);
       } else if (kind == "RESHAPE") {
         op = graph->CreateOperation<ops::Reshape>(new_shape);
+      } else if (kind == "DECONV2D") {
+        op = graph->CreateOperation<ops::DeConv2d>(weights, ParsePad(pad_type), ksize, stride, out_pad, pad,
+                                                   static_cast<uint32_t>(groups > 0 ? groups : 1), layout, klayout);
       } else if (kind == "DATACONVERT") {
         op = graph->CreateOperation<ops::DataConvert>();
       } else if (kind == "TRANSPOSE") {
