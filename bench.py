@@ -2,7 +2,7 @@
 """Benchmark of the quantized convolution hot path on one MI355X.
 
 A step = one pass of the hot path over one batch of synthetic input that is
-already resident in HBM. The headline workload is BASELINE.json's configs[1]:
+already resident in HBM. The headline workload is the configuration the metric is quoted on:
 one uint8 per-tensor Conv2d 3x3 64->64 on 56x56 at batch 32, SAME padding, fused
 ReLU6. Prints ONE JSON line (metric: int8 conv TOPS) carrying the dominant
 kernel's roofline and a CPU baseline timed on the host cores; `extra` holds the

@@ -217,11 +217,16 @@ def test_layout_inference_on_a_channel_fastest_network(tmp_path, oracle):
 
 
 @pytest.mark.gpu
-def test_repeated_runs_follow_the_inputs(tmp_path, oracle):
+@pytest.mark.parametrize("handles", [False, True], ids=["copies", "io_handles"])
+def test_repeated_runs_follow_the_inputs(tmp_path, oracle, handles):
     """Run() may be called again and again with the inputs re-filled in between
     (src/tim/vx/graph.cc:378-391): six runs with the input alternating between two images,
     host copies and synchronisations in between as an application would have them; every
-    run must equal the oracle's result for the image it was given."""
+    run must equal the oracle's result for the image it was given. With io_handles the graph's
+    input and output are Graph::CreateIOTensor tensors on buffers of the caller: filled in place
+    and handed over with FlushCacheForHandle, read in place after InvalidateCacheForHandle, and
+    every re-run brings a new input buffer in through SwapHandle (the old one, overwritten, must
+    not be read again) - the delegate's zero-copy protocol (include/tim/vx/tensor.h:154-166)."""
     w, x = _lenet_data()
     rng = np.random.default_rng(11)
     other = rng.integers(0, 256, x.size, dtype=np.uint8)
@@ -234,6 +239,7 @@ def test_repeated_runs_follow_the_inputs(tmp_path, oracle):
     logits["output"] = 15
     in_id = next(t["id"] for t in logits["tensors"] if t["attr"] == "INPUT")
     logits["reruns"] = [{in_id: other}, {in_id: x}, {in_id: other}, {in_id: other}, {in_id: x}]
+    logits["handles"] = handles
     want_x = oracle.run_graph(logits)
     alt = copy.deepcopy(logits)
     {t["id"]: t for t in alt["tensors"]}[in_id]["data"] = other

@@ -66,6 +66,8 @@ def write_graphs(graphs, txt_path, blob_path, bench=None):
     with open(txt_path, "w") as txt, open(blob_path, "wb") as blob:
         for g in graphs:
             txt.write("graph %s\n" % g["test"].replace(" ", "_"))
+            if g.get("handles"):
+                txt.write("handles\n")
             for t in g["tensors"]:
                 raw = tensor_bytes(t)
                 q = t["quant"]

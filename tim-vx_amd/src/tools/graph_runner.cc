@@ -18,6 +18,8 @@
 //   end
 // For every `run` one line goes to stdout: "ok <name> <offset> <bytes>" or
 // "fail <name> <stage>"; for every `bench`: "bench <name> <ms per Run> <ms per Run, device part>".
+#include <algorithm>
+#include <memory>
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
@@ -89,6 +91,10 @@ struct Pending {
   std::shared_ptr<Tensor> tensor;
   size_t off = 0, len = 0;
   bool is_input = false;
+  // `handles` graphs: the caller-owned buffer behind a CreateIOTensor tensor, and whether the next
+  // run must bring a fresh one in through SwapHandle
+  std::vector<char>* handle = nullptr;
+  bool swap_next = false;
 };
 
 }  // namespace
@@ -111,7 +117,8 @@ int main(int argc, char** argv) {
   std::shared_ptr<Graph> graph, source_graph;
   std::map<int, Pending> tensors;
   std::string name, line;
-  bool compiled = false, compile_ok = false;
+  bool compiled = false, compile_ok = false, use_handles = false;
+  std::vector<std::unique_ptr<std::vector<char>>> handle_bufs;
 
   while (std::getline(txt, line)) {
     std::istringstream ss(line);
@@ -122,6 +129,12 @@ int main(int argc, char** argv) {
       graph = context->CreateGraph();
       tensors.clear();
       compiled = compile_ok = false;
+      use_handles = false;
+      handle_bufs.clear();
+    } else if (rec == "handles") {
+      // graph inputs and outputs live in buffers of the caller (Graph::CreateIOTensor), are handed over
+      // with FlushCacheForHandle / InvalidateCacheForHandle and exchanged with SwapHandle between runs
+      use_handles = true;
     } else if (rec == "t") {
       int id, rank, chdim, ns, nz;
       std::string dt, attr, qt;
@@ -142,7 +155,13 @@ int main(int argc, char** argv) {
       TensorSpec spec(ParseDtype(dt), shape, ParseAttr(attr), quant);
       p.is_input = attr == "INPUT";
       const bool at_create = p.len && !p.is_input;
-      p.tensor = graph->CreateTensor(spec, at_create ? blob.data() + p.off : nullptr);
+      if (use_handles && (attr == "INPUT" || attr == "OUTPUT")) {
+        handle_bufs.emplace_back(new std::vector<char>(static_cast<size_t>(spec.GetByteSize())));
+        p.handle = handle_bufs.back().get();
+        p.tensor = graph->CreateIOTensor(spec, p.handle->data());
+      } else {
+        p.tensor = graph->CreateTensor(spec, at_create ? blob.data() + p.off : nullptr);
+      }
       tensors[id] = p;
     } else if (rec == "op") {
       std::string kind, pad_type, pool_type, round_type;
@@ -246,16 +265,37 @@ int main(int argc, char** argv) {
       const char* stage = nullptr;
       if (!compile_ok) stage = "compile";
       if (!stage)
-        for (auto& kv : tensors)
-          if (kv.second.is_input && kv.second.len &&
-              !kv.second.tensor->CopyDataToTensor(blob.data() + kv.second.off, static_cast<uint32_t>(kv.second.len)))
+        for (auto& kv : tensors) {
+          Pending& p = kv.second;
+          if (!p.is_input || !p.len) continue;
+          if (p.handle) {
+            if (p.swap_next) {  // a new buffer of the caller's takes the old one's place
+              handle_bufs.emplace_back(new std::vector<char>(p.handle->size()));
+              std::vector<char>* fresh = handle_bufs.back().get();
+              void* old = nullptr;
+              if (!p.tensor->SwapHandle(fresh->data(), false, &old) || old != p.handle->data()) stage = "swap_handle";
+              std::memset(p.handle->data(), 0xA5, p.handle->size());  // the old buffer must not be read again
+              p.handle = fresh;
+              p.swap_next = false;
+            }
+            std::memcpy(p.handle->data(), blob.data() + p.off, std::min(p.len, p.handle->size()));
+            if (!p.tensor->FlushCacheForHandle()) stage = "flush_handle";
+          } else if (!p.tensor->CopyDataToTensor(blob.data() + p.off, static_cast<uint32_t>(p.len))) {
             stage = "copy_in";
+          }
+        }
       if (!stage && !graph->Run()) stage = "run";
       std::vector<char> result;
       if (!stage) {
-        auto& t = tensors.at(id).tensor;
+        Pending& po = tensors.at(id);
+        auto& t = po.tensor;
         result.resize(t->GetSpec().GetByteSize());
-        if (!t->CopyDataFromTensor(result.data())) stage = "copy_out";
+        if (po.handle) {
+          if (!t->InvalidateCacheForHandle()) stage = "invalidate_handle";
+          else std::memcpy(result.data(), po.handle->data(), result.size());  // straight out of the caller's buffer
+        } else if (!t->CopyDataFromTensor(result.data())) {
+          stage = "copy_out";
+        }
       }
       if (stage) {
         std::printf("fail %s %s\n", name.c_str(), stage);
@@ -277,6 +317,7 @@ int main(int argc, char** argv) {
       }
       it->second.off = off;
       it->second.len = len;
+      it->second.swap_next = it->second.handle != nullptr;
     } else if (rec == "bench") {
       int warmup, iters;
       ss >> warmup >> iters;
