@@ -112,6 +112,26 @@ def test_every_reference_golden_through_the_cpp_api(tmp_path):
 
 
 @pytest.mark.gpu
+def test_every_reference_golden_through_the_platform_api(tmp_path):
+    """The same graphs as executables of the platform API (include/tim/vx/platform/platform.h:56-145,
+    samples/multi_device/multi_device_demo.cc:48-91): IDevice::Enumerate -> CreateExecutor ->
+    Compile(graph) -> AllocateTensor / SetInput / SetOutput -> Submit -> Trigger. The layout-inference
+    source graphs go in as they are: the executable resolves layouts when it rebuilds the graph."""
+    cases = _named_cases()
+    for c in cases:
+        c["platform"] = True
+        c["layout_inference"] = False
+    res, info, log = GF.run_graphs(cases, str(tmp_path))
+    bad = []
+    for c, out in zip(cases, res):
+        if out is None:
+            bad.append((c["test"], info.get(c["test"])))
+        elif not TC.matches(c, out):
+            bad.append((c["test"], out[:8], TC.golden_of(c)[:8]))
+    assert not bad, (bad[:5], log[-2000:])
+
+
+@pytest.mark.gpu
 def test_lenet_sample_graph(tmp_path, oracle):
     w, x = _lenet_data()
     g = GRAPHS.lenet_asymu8(w, x)
@@ -217,7 +237,7 @@ def test_layout_inference_on_a_channel_fastest_network(tmp_path, oracle):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("handles", [False, True], ids=["copies", "io_handles"])
+@pytest.mark.parametrize("handles", [False, True, "platform"], ids=["copies", "io_handles", "platform"])
 def test_repeated_runs_follow_the_inputs(tmp_path, oracle, handles):
     """Run() may be called again and again with the inputs re-filled in between
     (src/tim/vx/graph.cc:378-391): six runs with the input alternating between two images,
@@ -239,7 +259,8 @@ def test_repeated_runs_follow_the_inputs(tmp_path, oracle, handles):
     logits["output"] = 15
     in_id = next(t["id"] for t in logits["tensors"] if t["attr"] == "INPUT")
     logits["reruns"] = [{in_id: other}, {in_id: x}, {in_id: other}, {in_id: other}, {in_id: x}]
-    logits["handles"] = handles
+    logits["handles"] = handles is True
+    logits["platform"] = handles == "platform"   # re-submitted and triggered per run
     want_x = oracle.run_graph(logits)
     alt = copy.deepcopy(logits)
     {t["id"]: t for t in alt["tensors"]}[in_id]["data"] = other

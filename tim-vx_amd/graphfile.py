@@ -68,6 +68,8 @@ def write_graphs(graphs, txt_path, blob_path, bench=None):
             txt.write("graph %s\n" % g["test"].replace(" ", "_"))
             if g.get("handles"):
                 txt.write("handles\n")
+            if g.get("platform"):
+                txt.write("platform\n")
             for t in g["tensors"]:
                 raw = tensor_bytes(t)
                 q = t["quant"]

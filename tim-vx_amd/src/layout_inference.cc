@@ -290,13 +290,15 @@ std::shared_ptr<IPermuteVector> MakePermuteVector(const std::vector<uint32_t>& p
   return std::make_shared<PermuteVector>(perm);
 }
 
-std::pair<std::shared_ptr<vx::Graph>, std::map<std::shared_ptr<vx::Tensor>, std::shared_ptr<vx::Tensor>>>
-LayoutInference(const std::shared_ptr<vx::Graph>& src_graph, std::shared_ptr<vx::Context>& ctx,
-                std::map<std::shared_ptr<vx::Tensor>, std::shared_ptr<IPermuteVector>> tensor_pv_map) {
+// The walk itself, into a graph the caller made. io_map may arrive holding counterparts for some
+// of the source graph's INPUT / OUTPUT tensors (tensors of dst, with the source tensors' specs):
+// those are used instead of new ones. On return it holds all of them.
+bool RewriteInto(const std::shared_ptr<vx::Graph>& src_graph, const std::shared_ptr<vx::Graph>& dst_graph,
+                 const std::map<std::shared_ptr<vx::Tensor>, std::shared_ptr<IPermuteVector>>& tensor_pv_map,
+                 std::map<std::shared_ptr<vx::Tensor>, std::shared_ptr<vx::Tensor>>* io_map) {
   Walk w;
   w.src = src_graph;
-  w.dst = ctx->CreateGraph();
-  std::map<std::shared_ptr<Tensor>, std::shared_ptr<Tensor>> io_map;
+  w.dst = dst_graph;
   auto stated = [&](const std::shared_ptr<Tensor>& t) {
     auto it = tensor_pv_map.find(t);
     Perm p = it != tensor_pv_map.end() && it->second ? it->second->AsStdVec() : Identity(t->GetShape().size());
@@ -307,17 +309,18 @@ LayoutInference(const std::shared_ptr<vx::Graph>& src_graph, std::shared_ptr<vx:
     }
     return p;
   };
+  auto counterpart = [&](const std::shared_ptr<Tensor>& t) {
+    auto it = io_map->find(t);
+    if (it != io_map->end() && it->second) return it->second;
+    auto n = w.dst->CreateTensor(t->GetSpec());
+    (*io_map)[t] = n;
+    return n;
+  };
   for (const auto& t : src_graph->InputsTensor()) {
-    auto n = w.dst->CreateTensor(t->GetSpec());
-    w.mapped[t.get()] = n;
+    w.mapped[t.get()] = counterpart(t);
     w.pv[t.get()] = stated(t);
-    io_map[t] = n;
   }
-  for (const auto& t : src_graph->OutputsTensor()) {
-    auto n = w.dst->CreateTensor(t->GetSpec());
-    w.mapped[t.get()] = n;
-    io_map[t] = n;
-  }
+  for (const auto& t : src_graph->OutputsTensor()) w.mapped[t.get()] = counterpart(t);
   // dependency order: an operator is handled once every non-constant input has a counterpart
   std::deque<std::shared_ptr<Operation>> pending(src_graph->OpVector().begin(), src_graph->OpVector().end());
   std::set<Tensor*> produced;
@@ -342,8 +345,17 @@ LayoutInference(const std::shared_ptr<vx::Graph>& src_graph, std::shared_ptr<vx:
     VSILOGE("layout inference: %zu operators wait for tensors nothing produces", pending.size());
     w.ok = false;
   }
-  if (!w.ok) VSILOGE("layout inference failed; the returned graph is incomplete and will not compile");
-  return std::make_pair(w.dst, io_map);
+  if (!w.ok) VSILOGE("layout inference failed; the rewritten graph is incomplete and will not compile");
+  return w.ok;
+}
+
+std::pair<std::shared_ptr<vx::Graph>, std::map<std::shared_ptr<vx::Tensor>, std::shared_ptr<vx::Tensor>>>
+LayoutInference(const std::shared_ptr<vx::Graph>& src_graph, std::shared_ptr<vx::Context>& ctx,
+                std::map<std::shared_ptr<vx::Tensor>, std::shared_ptr<IPermuteVector>> tensor_pv_map) {
+  std::map<std::shared_ptr<Tensor>, std::shared_ptr<Tensor>> io_map;
+  auto dst = ctx->CreateGraph();
+  RewriteInto(src_graph, dst, tensor_pv_map, &io_map);
+  return std::make_pair(dst, io_map);
 }
 
 }  // namespace transform

@@ -236,3 +236,13 @@ const char* DataTypeName(DataType t);
 
 }  // namespace vx
 }  // namespace tim
+
+#include "tim/transform/layout_inference.h"
+namespace tim {
+namespace transform {
+// Rebuilds src_graph (layouts resolved) inside dst_graph; see layout_inference.cc.
+bool RewriteInto(const std::shared_ptr<vx::Graph>& src_graph, const std::shared_ptr<vx::Graph>& dst_graph,
+                 const std::map<std::shared_ptr<vx::Tensor>, std::shared_ptr<IPermuteVector>>& tensor_pv_map,
+                 std::map<std::shared_ptr<vx::Tensor>, std::shared_ptr<vx::Tensor>>* io_map);
+}  // namespace transform
+}  // namespace tim

@@ -35,6 +35,7 @@
 #include "tim/vx/graph.h"
 #include "tim/transform/layout_inference.h"
 #include "tim/vx/ops.h"
+#include "tim/vx/platform/platform.h"
 #include "tim/vx/tensor.h"
 
 extern "C" double tvx_runtime_last_device_ms(void);
@@ -95,6 +96,7 @@ struct Pending {
   // run must bring a fresh one in through SwapHandle
   std::vector<char>* handle = nullptr;
   bool swap_next = false;
+  std::shared_ptr<platform::ITensorHandle> th;  // `platform` graphs: the executable's handle for this tensor
 };
 
 }  // namespace
@@ -117,7 +119,9 @@ int main(int argc, char** argv) {
   std::shared_ptr<Graph> graph, source_graph;
   std::map<int, Pending> tensors;
   std::string name, line;
-  bool compiled = false, compile_ok = false, use_handles = false;
+  bool compiled = false, compile_ok = false, use_handles = false, use_platform = false;
+  std::shared_ptr<platform::IExecutor> executor;
+  std::shared_ptr<platform::IExecutable> executable;
   std::vector<std::unique_ptr<std::vector<char>>> handle_bufs;
 
   while (std::getline(txt, line)) {
@@ -131,6 +135,13 @@ int main(int argc, char** argv) {
       compiled = compile_ok = false;
       use_handles = false;
       handle_bufs.clear();
+      use_platform = false;
+      executable.reset();
+      executor.reset();
+    } else if (rec == "platform") {
+      // the graph runs as an executable of the platform API: device -> executor -> Compile(graph),
+      // tensor handles allocated by the executable for every graph input / output, Submit + Trigger
+      use_platform = true;
     } else if (rec == "handles") {
       // graph inputs and outputs live in buffers of the caller (Graph::CreateIOTensor), are handed over
       // with FlushCacheForHandle / InvalidateCacheForHandle and exchanged with SwapHandle between runs
@@ -258,6 +269,23 @@ int main(int argc, char** argv) {
     } else if (rec == "run") {
       int id;
       ss >> id;
+      if (!compiled && use_platform) {
+        compiled = true;
+        auto devices = platform::IDevice::Enumerate();
+        if (!devices.empty()) executor = devices[0]->CreateExecutor(0, -1, context);
+        if (executor) executable = platform::Compile(graph, executor);
+        if (executable) {
+          auto handle_for = [&](const std::shared_ptr<Tensor>& t) {
+            auto th = executable->AllocateTensor(t->GetSpec());
+            for (auto& kv : tensors)
+              if (kv.second.tensor == t) kv.second.th = th;
+            return th;
+          };
+          for (auto& t : graph->InputsTensor()) executable->SetInput(handle_for(t));
+          for (auto& t : graph->OutputsTensor()) executable->SetOutput(handle_for(t));
+          compile_ok = executable->Verify();
+        }
+      }
       if (!compiled) {
         compile_ok = graph->Compile();
         compiled = true;
@@ -268,7 +296,9 @@ int main(int argc, char** argv) {
         for (auto& kv : tensors) {
           Pending& p = kv.second;
           if (!p.is_input || !p.len) continue;
-          if (p.handle) {
+          if (use_platform) {
+            if (!p.th || !p.th->CopyDataToTensor(blob.data() + p.off, static_cast<uint32_t>(p.len))) stage = "copy_in";
+          } else if (p.handle) {
             if (p.swap_next) {  // a new buffer of the caller's takes the old one's place
               handle_bufs.emplace_back(new std::vector<char>(p.handle->size()));
               std::vector<char>* fresh = handle_bufs.back().get();
@@ -284,13 +314,15 @@ int main(int argc, char** argv) {
             stage = "copy_in";
           }
         }
-      if (!stage && !graph->Run()) stage = "run";
+      if (!stage && !(use_platform ? executable->Submit(executable) && executor->Trigger() : graph->Run())) stage = "run";
       std::vector<char> result;
       if (!stage) {
         Pending& po = tensors.at(id);
         auto& t = po.tensor;
         result.resize(t->GetSpec().GetByteSize());
-        if (po.handle) {
+        if (use_platform) {
+          if (!po.th || !po.th->CopyDataFromTensor(result.data())) stage = "copy_out";
+        } else if (po.handle) {
           if (!t->InvalidateCacheForHandle()) stage = "invalidate_handle";
           else std::memcpy(result.data(), po.handle->data(), result.size());  // straight out of the caller's buffer
         } else if (!t->CopyDataFromTensor(result.data())) {
