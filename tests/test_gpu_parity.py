@@ -547,3 +547,26 @@ def test_deconv2d(oracle, cfg):
         else:
             assert np.array_equal(got, want)
             assert 0.02 < np.mean((want > want.min()) & (want < want.max())), "saturated test data"
+
+
+IM2COL_GRID = [
+    # short windows (C * Kh * Kw <= 64, C not a multiple of 16): conv2d_im2col_i8
+    dict(n=3, c=3, h=33, w=31, oc=32, kh=3, kw=3, stride=[2, 2], dil=[1, 1], pad=[0, 1, 0, 1], mult=0),   # MobileNet conv1 form
+    dict(n=2, c=1, h=28, w=28, oc=20, kh=5, kw=5, stride=[1, 1], dil=[1, 1], pad=[0, 0, 0, 0], mult=0),   # LeNet conv1
+    dict(n=2, c=4, h=19, w=23, oc=50, kh=4, kw=4, stride=[1, 2], dil=[1, 1], pad=[2, 1, 1, 2], mult=0),   # K = 64 exactly
+    dict(n=1, c=7, h=20, w=20, oc=100, kh=3, kw=3, stride=[1, 1], dil=[2, 2], pad=[2, 2, 2, 2], mult=0),  # K = 63, dilated, 4 channel tiles
+    dict(n=5, c=2, h=9, w=7, oc=5, kh=1, kw=3, stride=[1, 1], dil=[1, 1], pad=[1, 1, 0, 0], mult=0),      # tiny, hw % 4 != 0
+    dict(n=2, c=3, h=64, w=64, oc=64, kh=3, kw=3, stride=[1, 1], dil=[1, 1], pad=[1, 1, 1, 1], mult=0),   # several workgroups per image
+]
+
+
+@pytest.mark.parametrize("mode", ["u8", "i8pc", "u8pc"])
+@pytest.mark.parametrize("gi", range(len(IM2COL_GRID)))
+def test_conv2d_im2col(oracle, gi, mode):
+    rng = np.random.default_rng(3000 + gi)
+    x, w, b, kws = conv_case(rng, mode=mode, **IM2COL_GRID[gi])
+    for act in (0, 2):
+        want = oracle.conv2d(x, w, b, act=act, **kws)
+        got = TC.gpu_conv2d(x, w, b, act=act, want_kernel="conv2d_im2col_i8", **kws)
+        assert np.array_equal(got, want), (gi, mode, act, np.flatnonzero(got != want)[:8])
+    assert 0.02 < np.mean((want > want.min()) & (want < want.max())), "saturated test data"

@@ -1,0 +1,299 @@
+// Quantized Conv2d with a short reduction (C * Kh * Kw <= 64) on the int8 matrix cores: the first
+// layers of image networks (3 x 3 x 3 = 27, 1 x 5 x 5 = 25). The implicit-GEMM kernel pads the
+// channels of every tap to 16 and would multiply mostly zeros there; here the whole window of an
+// output pixel - its (c, ky, kx) bytes, padded to 32 or 64 - is one row of the MFMA A operand.
+//
+// Workgroup = 256 output pixels of one image x all output channels (<= 128). Each thread
+// gathers the window of one pixel with byte loads (16 in flight, no branches: out-of-image taps
+// read a safe address and are replaced by the input zero point), keeps the window sum for the
+// zero-point expansion
+//   sum (x - zx)(w - zw) = sum xs ws - zws * Sx - zxs * Sw + K zxs zws
+// and stores the row to LDS. One or two v_mfma_i32_32x32x32_i8 steps per (pixel tile, channel
+// tile) follow; the epilogue is the implicit-GEMM kernel's: requantize, pack four pixels per
+// dword, stage [oc][pixel] in LDS, copy out as contiguous runs of the WHCN output.
+#include <algorithm>
+
+#include "variants.h"
+
+namespace tvx {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int kThreads = 256;
+constexpr int kPixels = 256;  // per workgroup: eight 32-pixel MFMA tiles, two per wavefront
+
+struct ImArgs {
+  const uint8_t* x;
+  const int8_t* w;       // packed [oct][row_stride] (the LDS image), reduction order (c, ky, kx), zero padded
+  uint8_t* y;
+  const int32_t* biasf;  // bias + per-channel zero-point terms
+  const v4i* rq;         // per channel {mult, shift | t, half, lowmask}
+  int C, H, W, OC, OH, OW;
+  int sh, sw, pad_t, pad_l;
+  int kp;                // reduction length padded to 32 or 64
+  int row_stride;        // bytes per LDS row of A and of the weights: kp + 16 (an odd number of 16-byte chunks)
+  int oct;               // output channels padded to 32
+  int xor_mask;          // 0x80 for uint8 activations, else 0
+  int pad_fill;          // input zero point in the int8 domain (one byte)
+  int zws, out_zp, lo, hi;
+  int out_stride;        // epilogue staging row stride in bytes (odd number of dwords)
+  int off_a, off_w, off_sx, off_rq, off_bias;  // LDS carve-up
+  // The window, one word per reduction index: c | dy << 8 | dx << 16 | 1 << 24, zero past the end.
+  // It travels in the kernel arguments so that the (wavefront-uniform) reads of it are scalar loads
+  // of memory nothing can write; a table in global memory is read per lane, one round trip a tap.
+  int taps[64];
+};
+
+template <int OT, int RQ>
+__global__ void __launch_bounds__(kThreads) ConvIm2colKernel(ImArgs a) {
+  extern __shared__ __attribute__((aligned(16))) int8_t lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n = blockIdx.y;
+  const int hw = a.OH * a.OW;
+  const int p0 = blockIdx.x * kPixels;
+  const int valid = min(kPixels, hw - p0);
+
+  int8_t* a_lds = lds + a.off_a;
+  int8_t* w_lds = lds + a.off_w;
+  int* sx_lds = reinterpret_cast<int*>(lds + a.off_sx);
+  v4i* rq_lds = reinterpret_cast<v4i*>(lds + a.off_rq);
+  int* bias_lds = reinterpret_cast<int*>(lds + a.off_bias);
+
+  // weights (already laid out as their LDS image) and the epilogue's tables: global -> LDS by DMA,
+  // waited for together with the window loads
+  {
+    typedef const __attribute__((address_space(1))) void* gptr;
+    typedef __attribute__((address_space(3))) void* lptr;
+    const int chunks = a.oct * a.row_stride >> 4;
+    for (int i = wave * 64; i < chunks; i += kThreads)
+      if (i + lane < chunks)
+        __builtin_amdgcn_global_load_lds((gptr)(a.w + static_cast<size_t>(i + lane) * 16), (lptr)(w_lds + i * 16), 16, 0, 0);
+    for (int i = wave * 64; i < a.oct; i += kThreads)
+      if (i + lane < a.oct) {
+        __builtin_amdgcn_global_load_lds((gptr)(a.rq + i + lane), (lptr)(rq_lds + i), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr)(a.biasf + i + lane), (lptr)(bias_lds + i), 4, 0, 0);
+      }
+  }
+
+  // ---- the window of this thread's pixel ------------------------------------------------
+  int sx = 0;
+  {
+    const int p = min(p0 + tid, hw - 1);  // threads past the end redo the last pixel; nobody reads their row
+    const int oh = p / a.OW, ow = p - oh * a.OW;
+    const int ih0 = oh * a.sh - a.pad_t, iw0 = ow * a.sw - a.pad_l;
+    const uint8_t* img = a.x + static_cast<size_t>(n) * a.C * a.H * a.W;
+    const int origin = ih0 * a.W + iw0;  // may be negative; only added to offsets of taps inside the image
+    const int plane = a.H * a.W;
+    for (int k0 = 0; k0 < a.kp; k0 += 16) {
+      int b[16];
+      bool inside[16], real[16];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const int t = a.taps[k0 + j];
+        const int c = t & 0xff, dy = (t >> 8) & 0xff, dx = (t >> 16) & 0xff;
+        real[j] = (t >> 24) != 0;
+        // bitwise, not short-circuit: no branch may stand between the loads
+        inside[j] = real[j] & (static_cast<unsigned>(ih0 + dy) < static_cast<unsigned>(a.H)) &
+                    (static_cast<unsigned>(iw0 + dx) < static_cast<unsigned>(a.W));
+        const int off = c * plane + dy * a.W + dx;  // scalar arithmetic
+        b[j] = img[static_cast<uint32_t>(inside[j] ? origin + off : 0)];  // uniform base + 32-bit lane offset
+      }
+      __builtin_amdgcn_sched_barrier(0);  // all sixteen loads travel together
+      int dw[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        int v = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int j = q * 4 + e;
+          const int byte = inside[j] ? (b[j] ^ a.xor_mask) : (real[j] ? a.pad_fill : 0);
+          v |= (byte & 0xff) << (8 * e);
+        }
+        dw[q] = v;
+        sx = __builtin_amdgcn_sdot4(v, 0x01010101, sx, false);
+      }
+      *reinterpret_cast<v4i*>(a_lds + tid * a.row_stride + k0) = v4i{dw[0], dw[1], dw[2], dw[3]};
+    }
+  }
+  sx_lds[tid] = a.zws * sx;
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the table DMA has landed
+  __syncthreads();
+
+  // ---- MFMA: wave w owns pixel tiles w and w + 4, all channel tiles ---------------------------
+  const int frag_row = lane & 31, frag_half = lane >> 5;
+  v16i acc[2][OT];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < OT; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+  for (int ks = 0; ks < a.kp; ks += 32) {
+    v4i fa[2], fb[OT];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      fa[i] = *reinterpret_cast<const v4i*>(a_lds + ((wave + 4 * i) * 32 + frag_row) * a.row_stride + ks + frag_half * 16);
+#pragma unroll
+    for (int j = 0; j < OT; ++j)
+      fb[j] = *reinterpret_cast<const v4i*>(w_lds + (j * 32 + frag_row) * a.row_stride + ks + frag_half * 16);
+#pragma unroll
+    for (int j = 0; j < OT; ++j)
+#pragma unroll
+      for (int i = 0; i < 2; ++i) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+  }
+  __syncthreads();  // everyone is done with the A rows and the weights: the staging tile takes their place
+
+  // ---- epilogue ---------------------------------------------------------------------------
+  int8_t* out_tile = lds + a.off_a;  // [oct][out_stride]
+  const int lo = a.lo, hi = a.hi;
+#pragma unroll
+  for (int j = 0; j < OT; ++j) {
+    const int ocl = j * 32 + frag_row;
+    const v4i q = rq_lds[ocl];
+    const int bias = bias_lds[ocl];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int pt = wave + 4 * i;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int pl = pt * 32 + 8 * g + 4 * frag_half;
+        const v4i s4 = *reinterpret_cast<const v4i*>(sx_lds + pl);
+        int r4[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r4[e] = Requant8<RQ>(acc[i][j][g * 4 + e] + (bias - s4[e]), q, a.out_zp, lo, hi);
+        *reinterpret_cast<uint32_t*>(out_tile + ocl * a.out_stride + pl) = PackBytes(r4[0], r4[1], r4[2], r4[3]);
+      }
+    }
+  }
+  __syncthreads();
+  uint8_t* ybase = a.y + static_cast<size_t>(n) * a.OC * hw + p0;
+  if ((hw & 3) == 0) {
+    const int per_row = valid >> 2;  // p0 and hw are multiples of 4: whole dwords
+    for (int o = wave; o < a.OC; o += 4)
+      for (int dwi = lane; dwi < per_row; dwi += 64)
+        *reinterpret_cast<uint32_t*>(ybase + static_cast<size_t>(o) * hw + dwi * 4) =
+            *reinterpret_cast<const uint32_t*>(out_tile + o * a.out_stride + dwi * 4);
+  } else {
+    for (int o = wave; o < a.OC; o += 4)
+      for (int pi = lane; pi < valid; pi += 64)
+        ybase[static_cast<size_t>(o) * hw + pi] = static_cast<uint8_t>(out_tile[o * a.out_stride + pi]);
+  }
+}
+
+struct Plan {
+  ImArgs a;
+  int lds_bytes;
+  int ot, rq;
+  dim3 grid;
+};
+
+template <int OT>
+void LaunchRq(const Plan* plan, const ImArgs& a, hipStream_t st) {
+  const dim3 block(kThreads);
+  if (plan->rq == kRqFastNoTie)
+    hipLaunchKernelGGL((ConvIm2colKernel<OT, kRqFastNoTie>), plan->grid, block, plan->lds_bytes, st, a);
+  else if (plan->rq == kRqFast)
+    hipLaunchKernelGGL((ConvIm2colKernel<OT, kRqFast>), plan->grid, block, plan->lds_bytes, st, a);
+  else
+    hipLaunchKernelGGL((ConvIm2colKernel<OT, kRqGeneric>), plan->grid, block, plan->lds_bytes, st, a);
+}
+
+int ConvIm2colRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
+  const Plan* plan = reinterpret_cast<const Plan*>(op->host_blob.data());
+  ImArgs a = plan->a;
+  a.x = static_cast<const uint8_t*>(in0);
+  a.y = static_cast<uint8_t*>(out);
+  if (plan->ot == 1) LaunchRq<1>(plan, a, st);
+  else if (plan->ot == 2) LaunchRq<2>(plan, a, st);
+  else LaunchRq<4>(plan, a, st);
+  TVX_HIP_CHECK(hipGetLastError());
+  return TVX_OK;
+}
+
+int RoundUp(int v, int m) { return (v + m - 1) / m * m; }
+
+}  // namespace
+
+// Claims dense quantized convolutions with constant weights whose whole window is at most 64
+// bytes and whose channel count the implicit-GEMM kernel would have to pad (C % 16 != 0).
+int ConvIm2colSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const void* bias_host) {
+  if (!op->quantized || !w_host || d->multiplier != 0 || d->groups > 1) return TVX_E_UNSUPPORTED;
+  const int taps = static_cast<int>(d->k_w * d->k_h);
+  const uint64_t k_real = static_cast<uint64_t>(d->in_c) * taps;
+  if (k_real > 64 || d->in_c % 16 == 0 || d->out_c > 128) return TVX_E_UNSUPPORTED;
+  if (static_cast<uint64_t>(d->in_c) * d->in_h * d->in_w >= (1ull << 31) || d->batch > 65535) return TVX_E_UNSUPPORTED;
+  ImArgs a{};
+  a.C = d->in_c; a.H = d->in_h; a.W = d->in_w; a.OC = d->out_c; a.OH = d->out_h; a.OW = d->out_w;
+  a.sh = d->stride_h; a.sw = d->stride_w; a.pad_t = d->pad_top; a.pad_l = d->pad_left;
+  const int K = static_cast<int>(k_real);
+  a.kp = K <= 32 ? 32 : 64;
+  a.row_stride = a.kp + 16;
+  const int ot = d->out_c <= 32 ? 1 : (d->out_c <= 64 ? 2 : 4);
+  a.oct = 32 * ot;
+  const bool x_u8 = d->in_dtype == TVX_U8, w_u8 = d->w_dtype == TVX_U8;
+  const int zxs = d->in_zp - (x_u8 ? 128 : 0);
+  const int zws = op->w_zp - (w_u8 ? 128 : 0);
+  if (zxs < -128 || zxs > 127) return TVX_E_UNSUPPORTED;  // zero point outside the tensor's range
+  a.xor_mask = x_u8 ? 0x80 : 0;
+  a.pad_fill = zxs & 0xff;
+  a.zws = zws;
+  a.out_zp = d->out_zp; a.lo = op->act_lo; a.hi = op->act_hi;
+  a.out_stride = ((kPixels / 4) | 1) * 4;
+  // LDS: window sums and tables first; A rows + weights behind them are reused as the staging tile
+  a.off_sx = 0;
+  a.off_rq = kPixels * 4;
+  a.off_bias = a.off_rq + a.oct * 16;
+  a.off_a = a.off_bias + a.oct * 4;
+  a.off_w = a.off_a + kPixels * a.row_stride;
+  const int lds_bytes = a.off_a + std::max(kPixels * a.row_stride + a.oct * a.row_stride, a.oct * a.out_stride);
+
+  // ---- pack weights [oc][(c, ky, kx)] int8 with zero padding, fold constants ---------------
+  std::vector<int8_t> packed(static_cast<size_t>(a.oct) * a.row_stride, 0);
+  std::vector<int32_t> biasf(a.oct, 0);
+  const uint8_t* src = static_cast<const uint8_t*>(w_host);
+  const int32_t* b = static_cast<const int32_t*>(bias_host);
+  for (int oc = 0; oc < a.OC; ++oc) {
+    int64_t sw = 0;
+    for (int k = 0; k < K; ++k) {  // the weight tensor's own order: [oc][c][ky][kx]
+      const uint8_t raw = src[static_cast<size_t>(oc) * K + k];
+      const int8_t v = static_cast<int8_t>(w_u8 ? raw ^ 0x80 : raw);
+      packed[static_cast<size_t>(oc) * a.row_stride + k] = v;
+      sw += v;
+    }
+    const int64_t v = (b ? b[oc] : 0) - static_cast<int64_t>(zxs) * sw + static_cast<int64_t>(K) * zxs * zws;
+    biasf[oc] = static_cast<int32_t>(static_cast<uint32_t>(v));
+  }
+  std::vector<int32_t> rqt;
+  const int rq = BuildRequantRecords(op->h_mult, op->h_shift, a.OC, a.oct, d->out_zp, &rqt,
+                                     AccumulatorBound(static_cast<uint64_t>(K), bias_host, a.OC));
+  if (d->k_h * d->dilation_h > 255 || d->k_w * d->dilation_w > 255) return TVX_E_UNSUPPORTED;  // dy, dx in a byte
+  for (int k = 0; k < K; ++k) {
+    const int c = k / taps, t = k % taps;
+    const int dy = (t / static_cast<int>(d->k_w)) * static_cast<int>(d->dilation_h);
+    const int dx = (t % static_cast<int>(d->k_w)) * static_cast<int>(d->dilation_w);
+    a.taps[k] = c | dy << 8 | dx << 16 | 1 << 24;
+  }
+  int s = op->packed.Upload(packed.data(), packed.size());
+  if (s == TVX_OK) s = op->aux.Upload(biasf.data(), biasf.size() * 4);
+  if (s == TVX_OK) s = op->aux2.Upload(rqt.data(), rqt.size() * 4);
+  if (s != TVX_OK) return s;
+  a.w = op->packed.as<int8_t>();
+  a.biasf = op->aux.as<int32_t>();
+  a.rq = op->aux2.as<v4i>();
+
+  Plan plan;
+  plan.a = a;
+  plan.lds_bytes = lds_bytes;
+  plan.ot = ot;
+  plan.rq = rq;
+  const int hw = a.OH * a.OW;
+  plan.grid = dim3(static_cast<unsigned>((hw + kPixels - 1) / kPixels), static_cast<unsigned>(d->batch));
+  op->host_blob.assign(reinterpret_cast<const uint8_t*>(&plan), reinterpret_cast<const uint8_t*>(&plan) + sizeof(plan));
+  op->run = ConvIm2colRun;
+  op->kernel_name = "conv2d_im2col_i8";
+  return TVX_OK;
+}
+
+}  // namespace tvx

@@ -27,6 +27,8 @@ int FcMfmaSetup(tvx_op*, const tvx_fc_desc*, const void*, const void*);
 
 // int8 MFMA implicit-GEMM convolution (conv_igemm_i8.hip)
 int ConvIgemmSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
+// Dense quantized conv whose whole window (C * Kh * Kw) is at most 64 bytes: im2col rows in LDS + MFMA.
+int ConvIm2colSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 
 // pointwise (1x1) convolution with the whole channel depth of a pixel tile in LDS (pwconv_i8.hip)
 int PwConvSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
