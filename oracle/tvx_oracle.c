@@ -9,7 +9,9 @@
  * 1739), whose binary is not part of the reference checkout. This file
  * restates the published semantics and is pinned by the reference's own
  * inline golden vectors (tests/golden/ *.json, recorded from
- * src/tim/vx/ops/{conv2d,depthwiseConv,fullyconnected,max_pool,avg_pool}_test.cc).
+ * src/tim/vx/ops/{conv2d,depthwiseConv,groupedconv2d,conv1d,deconv2d,fullyconnected,max_pool,
+ * avg_pool,softmax,transpose,simple_operations}_test.cc and
+ * src/tim/transform/layout_inference_test.cc).
  *
  * What the goldens pin: indexing, padding, stride, dilation, depthwise channel
  * mapping, zero-point handling, per-channel scales, saturation, pooling
@@ -19,7 +21,16 @@
  *     form: here a Q31 multiplier and a single round-half-to-even right shift
  *     of the 64-bit product;
  *   - quantized FullyConnected, ReLU/ReLU6, Add and quantized AVG rounding
- *     (the reference compares AVG with +-1 tolerance).
+ *     (the reference compares AVG with +-1 tolerance);
+ *   - DeConv2d with more than one channel per group: the reference's tests are
+ *     single-channel or depthwise, so the channel order of the {Kw, Kh, Ic, Oc}
+ *     weights follows include/tim/vx/ops/deconv.h:46-52 only;
+ *   - DataConvert on exact .5 ties (round-half-to-even of f / scale, as
+ *     vsi_nn_dtype_util_prv.h:228-252 computes it with the default rounding mode);
+ *   - Transpose: the reference's two tests move a {1, 3} vector and cannot tell a
+ *     permutation from its inverse; the direction follows the extent rule
+ *     out.size[i] = in.size[perm[i]] (vsi_nn_op_permute.c:219-230) and is checked
+ *     against numpy on non-involutive permutations.
  *
  * Layouts (dim 0 fastest): activations WHCN, weights WHIcOc, depthwise
  * weights {Kw,Kh,Ic*mult,1}, FC input {K,M}, weight {K,N}, output {N,M}
