@@ -188,6 +188,19 @@ typedef struct tvx_softmax_desc {
 
 int tvx_softmax_create(const tvx_softmax_desc* desc, tvx_op** op);
 
+/* ---- Conv2d + Add in one kernel -------------------------------------------------------- */
+/* A convolution whose result only feeds a same-shape Add (the residual connection of an inverted
+ * residual block): two nodes of the reference's graph (vxConvolutionLayer, then vxTensorAddNode:
+ * src/tim/vx/internal/src/kernel/vx/eltwise_vx.c:56-67) as one operator whose result is, bit for
+ * bit, what the two would give (the convolution's result quantized to its own output tensor
+ * first). `conv` describes the convolution as for tvx_conv2d_create, `add` the Add (dtype,
+ * a_* / b_* / out_* quantization; count and activation are ignored), conv_operand says which
+ * operand of the Add the convolution is (1 or 2); the other operand goes in as in1 of
+ * tvx_op_run. Returns TVX_E_UNSUPPORTED when no kernel fuses this convolution (the caller then
+ * creates the two operators). */
+int tvx_conv2d_add_create(const tvx_conv2d_desc* conv, const tvx_eltwise_desc* add, int conv_operand,
+                          const void* weights_host, const void* bias_host, tvx_op** op);
+
 /* ---- DeConv2d (transposed convolution) ----------------------------------------------- */
 /* Replaces vxDeconvolutionLayer (src/tim/vx/ops/deconv.cc:45-79,
  * src/tim/vx/internal/src/ops/vsi_nn_op_deconvolution.c:217-218,398-497). Same descriptor as

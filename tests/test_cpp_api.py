@@ -278,8 +278,11 @@ def test_repeated_runs_follow_the_inputs(tmp_path, oracle, handles):
 @pytest.mark.parametrize("batch,res", [(2, 224), (3, 96)])
 def test_mobilenet_v2_graph_bit_exact(tmp_path, oracle, batch, res):
     g = GRAPHS.mobilenet_v2(batch=batch, res=res, seed=batch)
-    out, info, log = GF.run_graphs([g], str(tmp_path))
+    out, info, log = GF.run_graphs([g], str(tmp_path), env={"VSI_NN_LOG_LEVEL": "3"})
     assert out[0] is not None, (info, log[-2000:])
     ref = oracle.run_graph(g)
     assert len(np.unique(ref)) > 30  # the synthetic network is not degenerate
     assert np.array_equal(out[0], ref), int((out[0] != ref).sum())
+    # the ten residual Adds ride on the projection convolutions in front of them: no Add kernel in the plan
+    plan = [l for l in log.splitlines() if "uid" in l and "->" in l]
+    assert sum("pwconv_add_i8" in l for l in plan) == 10 and not any("ADD" in l for l in plan), plan

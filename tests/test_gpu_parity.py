@@ -285,7 +285,7 @@ def test_conv2d_cfg2_full_size(oracle):
 IGEMM_GRID = [
     # (n, c, h, w, oc, kh, kw, stride, dil, pad[l,r,t,b])
     (2, 32, 28, 28, 64, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),
-    (1, 3, 32, 32, 32, 3, 3, [2, 2], [1, 1], [0, 1, 0, 1]),
+    (1, 12, 32, 32, 32, 3, 3, [2, 2], [1, 1], [0, 1, 0, 1]),   # channels padded to 16 (C = 3 would be im2col's)
     (2, 16, 14, 14, 96, 1, 1, [1, 1], [1, 1], [0, 0, 0, 0]),
     (1, 64, 9, 7, 40, 3, 3, [1, 1], [2, 2], [2, 2, 2, 2]),
     (1, 20, 8, 8, 50, 5, 5, [1, 1], [1, 1], [0, 0, 0, 0]),
@@ -570,3 +570,56 @@ def test_conv2d_im2col(oracle, gi, mode):
         got = TC.gpu_conv2d(x, w, b, act=act, want_kernel="conv2d_im2col_i8", **kws)
         assert np.array_equal(got, want), (gi, mode, act, np.flatnonzero(got != want)[:8])
     assert 0.02 < np.mean((want > want.min()) & (want < want.max())), "saturated test data"
+
+
+@pytest.mark.parametrize("side,n", [(16, 2), (14, 3), (7, 5), (5, 1)], ids=lambda v: str(v))   # hw % 16 == 0, % 4 == 0, odd
+@pytest.mark.parametrize("mode", ["u8", "i8pc"])
+@pytest.mark.parametrize("conv_operand", [1, 2])
+def test_pointwise_conv_with_fused_add(oracle, side, n, mode, conv_operand):
+    """tvx_conv2d_add_create against the two operators it stands for: the oracle's convolution, quantized to
+    the convolution's own output tensor, then the oracle's Add with the other operand."""
+    rng = np.random.default_rng(side * 10 + conv_operand)
+    c, oc = 48, 40
+    x, w, b, kws = conv_case(rng, n=n, c=c, h=side, w=side, oc=oc, kh=1, kw=1, stride=[1, 1], dil=[1, 1],
+                             pad=[0, 0, 0, 0], mult=0, mode=mode)
+    dt = kws["out_dtype"]
+    conv_q = kws["out_q"]
+    other = rand_q(rng, n * oc * side * side, dt)
+    other_q = (0.037, 121 if dt == 0 else -7)
+    sum_q = (float(np.float32(conv_q[0] * 1.3)), 119 if dt == 0 else 5)
+    t = oracle.conv2d(x, w, b, **kws)
+    a, aq, bb, bq = (t, conv_q, other, other_q) if conv_operand == 1 else (other, other_q, t, conv_q)
+    want = oracle.add(dt, a, aq, bb, bq, sum_q)
+    T = TC.tvx()
+    d = T.Conv2dDesc()
+    d.in_w, d.in_h, d.in_c, d.batch = kws["in_shape"]
+    d.k_w = d.k_h = 1
+    d.out_w, d.out_h, d.out_c = side, side, oc
+    d.stride_w = d.stride_h = d.dilation_w = d.dilation_h = 1
+    d.in_dtype, d.w_dtype, d.out_dtype = kws["in_dtype"], kws["w_dtype"], dt
+    d.in_scale, d.in_zp = kws["in_q"]
+    keep = []
+    TC._wq(d, kws["w_q"], keep)
+    d.out_scale, d.out_zp = conv_q
+    e = T.EltwiseDesc()
+    e.count, e.dtype = want.size, dt
+    e.a_scale, e.a_zp = aq
+    e.b_scale, e.b_zp = bq
+    e.out_scale, e.out_zp = sum_q
+    op = T.conv2d_add_create(d, e, conv_operand, w, b)
+    assert op.kernel_name == "pwconv_add_i8"
+    import torch
+    xd, od = TC.to_device(x), TC.to_device(other)
+    yd = TC.device_out(want.size, TC.NP_OF[dt])
+    op.run(xd, od, yd)
+    torch.cuda.synchronize()
+    got = yd.cpu().numpy()
+    assert np.array_equal(got, want), np.flatnonzero(got != want)[:8]
+    assert 0.05 < np.mean((want > want.min()) & (want < want.max()))
+    # a convolution no fused kernel takes: the caller is told so and creates the two operators
+    d.k_w = d.k_h = 3
+    d.pad_left = d.pad_top = 1
+    w3 = rand_q(rng, oc * c * 9, kws["w_dtype"])
+    with pytest.raises(T.TvxError) as err:
+        T.conv2d_add_create(d, e, conv_operand, w3, b)
+    assert err.value.status == T.E_UNSUPPORTED

@@ -112,6 +112,7 @@ def lib():
         L.tvx_requantize.restype = C.c_int64
         L.tvx_requantize.argtypes = [C.c_int32, C.c_int32, C.c_int32]
         L.tvx_conv2d_create.argtypes = [C.POINTER(Conv2dDesc), vp, vp, C.POINTER(vp)]
+        L.tvx_conv2d_add_create.argtypes = [C.POINTER(Conv2dDesc), C.POINTER(EltwiseDesc), C.c_int, vp, vp, C.POINTER(vp)]
         L.tvx_deconv2d_create.argtypes = [C.POINTER(Conv2dDesc), vp, vp, C.POINTER(vp)]
         L.tvx_fully_connected_create.argtypes = [C.POINTER(FcDesc), vp, vp, C.POINTER(vp)]
         L.tvx_pool2d_create.argtypes = [C.POINTER(Pool2dDesc), C.POINTER(vp)]
@@ -173,6 +174,13 @@ def conv2d_create(desc, weights=None, bias=None):
     """weights / bias: C-contiguous numpy arrays (host) or None."""
     h = C.c_void_p()
     check(lib().tvx_conv2d_create(C.byref(desc), _host_ptr(weights), _host_ptr(bias), C.byref(h)))
+    return Op(h)
+
+
+def conv2d_add_create(desc, add_desc, conv_operand, weights, bias=None):
+    h = C.c_void_p()
+    check(lib().tvx_conv2d_add_create(C.byref(desc), C.byref(add_desc), conv_operand, _host_ptr(weights),
+                                      _host_ptr(bias), C.byref(h)))
     return Op(h)
 
 

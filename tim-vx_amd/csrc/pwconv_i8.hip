@@ -49,7 +49,32 @@ struct PwArgs {
   int xor_mask;          // 0x80808080 for uint8 activations
   int neg_zws4;          // -(weight zero point, int8 domain) in all four bytes
   int out_zp, lo, hi;
+  // Fused residual Add (0 = off): the convolution's quantized output t meets a tensor r of the output's
+  // shape on the way out, y = clamp(rne(fma(a - za, ra, (b - zb) * rb)) + zo) in double, exactly the
+  // stand-alone Add on the tensor the convolution would have written. add_mode 1: a = t, b = r; 2: a = r, b = t.
+  const uint8_t* res;
+  double add_ra, add_rb;
+  int add_mode, add_signed;
+  int add_za, add_zb, add_zo, add_lo, add_hi;
 };
+
+// Four output bytes of the convolution and the four residual bytes at the same place -> four sums.
+__device__ __forceinline__ uint32_t AddResidual4(const PwArgs& a, uint32_t t4, uint32_t r4) {
+  int out[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    int t = (t4 >> (8 * e)) & 0xff, r = (r4 >> (8 * e)) & 0xff;
+    if (a.add_signed) {
+      t = static_cast<int8_t>(t);
+      r = static_cast<int8_t>(r);
+    }
+    const int av = a.add_mode == 1 ? t : r, bv = a.add_mode == 1 ? r : t;
+    const double tb = __dmul_rn(static_cast<double>(bv - a.add_zb), a.add_rb);
+    const double s = fma(static_cast<double>(av - a.add_za), a.add_ra, tb);
+    out[e] = Med3(static_cast<int>(rint(s)) + a.add_zo, a.add_lo, a.add_hi);
+  }
+  return PackBytes(out[0], out[1], out[2], out[3]);
+}
 
 // 4 dwords = 4 channels x 4 pixels (pixel in the byte lanes) -> 4 dwords = 4 pixels x 4 channels.
 __device__ __forceinline__ void Transpose4x4(const uint32_t in[4], uint32_t out[4]) {
@@ -243,7 +268,6 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((P
     __builtin_amdgcn_wave_barrier();
     // copy-out: rows of the staging patch -> WHCN output
     const int rows = min(32, a.OC - tile * 32);
-    uint8_t* ybase = a.y + static_cast<size_t>(tile) * 32 * a.HW;
     if (GRAN == 16) {
 #pragma unroll
       for (int i = 0; i < 32 / kRowsPerIter; ++i) {
@@ -251,24 +275,44 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((P
         const int8_t* s = stage + row * kStageStride + px_in_row;
         const uint2 lo8 = *reinterpret_cast<const uint2*>(s);
         const uint2 hi8 = *reinterpret_cast<const uint2*>(s + 8);
-        if (row < rows && out_live)
-          *reinterpret_cast<uint4*>(ybase + out_off + static_cast<size_t>(row) * a.HW) =
-              make_uint4(lo8.x, lo8.y, hi8.x, hi8.y);
+        if (row < rows && out_live) {
+          uint4 o = make_uint4(lo8.x, lo8.y, hi8.x, hi8.y);
+          const size_t at = static_cast<size_t>(tile) * 32 * a.HW + out_off + static_cast<size_t>(row) * a.HW;
+          if (a.add_mode) {
+            const uint4 r = *reinterpret_cast<const uint4*>(a.res + at);
+            o = make_uint4(AddResidual4(a, o.x, r.x), AddResidual4(a, o.y, r.y), AddResidual4(a, o.z, r.z),
+                           AddResidual4(a, o.w, r.w));
+          }
+          *reinterpret_cast<uint4*>(a.y + at) = o;
+        }
       }
     } else {
 #pragma unroll
       for (int i = 0; i < 32 / kRowsPerIter; ++i) {
         const int row = lane / kPerRow + kRowsPerIter * i;
-        const uint32_t v = *reinterpret_cast<const uint32_t*>(stage + row * kStageStride + px_in_row);
+        uint32_t v = *reinterpret_cast<const uint32_t*>(stage + row * kStageStride + px_in_row);
+        const size_t row_at = static_cast<size_t>(tile) * 32 * a.HW + static_cast<size_t>(row) * a.HW;
         if (row < rows && out_whole) {
-          uint8_t* o = ybase + out_off + static_cast<size_t>(row) * a.HW;
+          uint8_t* o = a.y + row_at + out_off;
+          if (a.add_mode) {
+            uint32_t r;
+            if (GRAN == 4) r = *reinterpret_cast<const uint32_t*>(a.res + row_at + out_off);
+            else __builtin_memcpy(&r, a.res + row_at + out_off, 4);
+            v = AddResidual4(a, v, r);
+          }
           if (GRAN == 4) *reinterpret_cast<uint32_t*>(o) = v;
           else __builtin_memcpy(o, &v, 4);
         } else if (GRAN == 1 && row < rows) {
+          if (a.add_mode) {
+            uint32_t r = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (out_px_live[e]) r |= static_cast<uint32_t>(a.res[row_at + out_px_off[e]]) << (8 * e);
+            v = AddResidual4(a, v, r);
+          }
 #pragma unroll
           for (int e = 0; e < 4; ++e)
-            if (out_px_live[e])
-              ybase[out_px_off[e] + static_cast<size_t>(row) * a.HW] = static_cast<uint8_t>(v >> (8 * e));
+            if (out_px_live[e]) a.y[row_at + out_px_off[e]] = static_cast<uint8_t>(v >> (8 * e));
         }
       }
     }
@@ -363,12 +407,14 @@ int Dispatch(const Plan* plan, const PwArgs& a, hipStream_t st, bool configure) 
   return DispatchGran<128, 4, 1>(plan, a, st, configure);
 }
 
-int PwConvRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
+int PwConvRun(tvx_op* op, const void* in0, const void* in1, void* out, hipStream_t st) {
   const Plan* plan = reinterpret_cast<const Plan*>(op->host_blob.data());
   PwArgs a = plan->a;
   a.x = static_cast<const uint8_t*>(in0);
   a.y = static_cast<uint8_t*>(out);
-  if ((reinterpret_cast<uintptr_t>(in0) | reinterpret_cast<uintptr_t>(out)) & (plan->gran - 1))
+  a.res = static_cast<const uint8_t*>(in1);
+  if (a.add_mode && !in1) return SetError(TVX_E_INVALID, "pwconv_i8: the fused Add needs its second operand as in1");
+  if ((reinterpret_cast<uintptr_t>(in0) | reinterpret_cast<uintptr_t>(out) | (a.add_mode ? reinterpret_cast<uintptr_t>(in1) : 0)) & (plan->gran - 1))
     return SetError(TVX_E_INVALID, "pwconv_i8: tensors must be %d-byte aligned", plan->gran);
   const int s = Dispatch(plan, a, st, false);
   if (s != TVX_OK) return s;
@@ -422,6 +468,21 @@ int PwConvSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const 
   a.out_zp = d->out_zp;
   a.lo = op->act_lo;
   a.hi = op->act_hi;
+  if (op->fused_add) {
+    const tvx_eltwise_desc& e = op->elt;  // a_* / b_* are the Add's first / second operand
+    const double ra = static_cast<double>(e.a_scale) / static_cast<double>(e.out_scale);
+    const double rb = static_cast<double>(e.b_scale) / static_cast<double>(e.out_scale);
+    // as for the stand-alone 16-element Add: the sum must stay far below 2^31 for the 32-bit conversion
+    if (!(ra < 1048576.0) || !(rb < 1048576.0)) return TVX_E_UNSUPPORTED;
+    a.add_mode = op->fused_add;
+    a.add_signed = d->out_dtype == TVX_I8;
+    a.add_ra = ra;
+    a.add_rb = rb;
+    a.add_za = e.a_zp;
+    a.add_zb = e.b_zp;
+    a.add_zo = e.out_zp;
+    ActRange(d->out_dtype, e.out_scale, e.out_zp, TVX_ACT_NONE, &a.add_lo, &a.add_hi);
+  }
   // few pixel tiles: spread the output tiles over grid.y (in units of one tile per
   // wavefront) until the launch has a few workgroups per CU
   const int quads = (a.oc_tiles + nw - 1) / nw;
@@ -479,7 +540,7 @@ int PwConvSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const 
   if (s != TVX_OK) return s;
   op->host_blob.assign(reinterpret_cast<const uint8_t*>(&plan), reinterpret_cast<const uint8_t*>(&plan) + sizeof(plan));
   op->run = PwConvRun;
-  op->kernel_name = "pwconv_i8";
+  op->kernel_name = op->fused_add ? "pwconv_add_i8" : "pwconv_i8";
   return TVX_OK;
 }
 

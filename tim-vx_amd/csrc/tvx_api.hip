@@ -319,6 +319,47 @@ int tvx_conv2d_create(const tvx_conv2d_desc* d, const void* weights_host,
   return TVX_OK;
 }
 
+int tvx_conv2d_add_create(const tvx_conv2d_desc* d, const tvx_eltwise_desc* add, int conv_operand,
+                          const void* weights_host, const void* bias_host, tvx_op** out) {
+  if (!d || !add || !out) return SetError(TVX_E_INVALID, "tvx_conv2d_add_create: null argument");
+  *out = nullptr;
+  if (conv_operand != 1 && conv_operand != 2)
+    return SetError(TVX_E_INVALID, "tvx_conv2d_add_create: conv_operand must be 1 or 2");
+  if (!IsQuant(d->in_dtype) || !IsQuant(d->out_dtype) || add->dtype != d->out_dtype || !weights_host ||
+      !(add->a_scale > 0.f) || !(add->b_scale > 0.f) || !(add->out_scale > 0.f))
+    return SetError(TVX_E_UNSUPPORTED, "tvx_conv2d_add_create: quantized tensors of one type and constant weights only");
+  // the convolution's own output quantization is the Add's for that operand
+  const float conv_scale = conv_operand == 1 ? add->a_scale : add->b_scale;
+  const int32_t conv_zp = conv_operand == 1 ? add->a_zp : add->b_zp;
+  if (conv_scale != d->out_scale || conv_zp != d->out_zp)
+    return SetError(TVX_E_INVALID, "tvx_conv2d_add_create: the Add's operand %d is not quantized like the convolution's output", conv_operand);
+  if (!d->in_w || !d->in_h || !d->in_c || !d->batch || !d->out_c)
+    return SetError(TVX_E_INVALID, "tvx_conv2d_add_create: zero extent");
+  int s = CheckOperandTypes(d->in_dtype, d->w_dtype, d->out_dtype, "tvx_conv2d_add_create");
+  if (s != TVX_OK) return s;
+  if ((s = NoGpu()) != TVX_OK) return s;
+  tvx_op* op = new (std::nothrow) tvx_op();
+  if (!op) return SetError(TVX_E_NOMEM, "tvx_conv2d_add_create: host allocation failed");
+  op->kind = OP_CONV2D;
+  op->conv = *d;
+  op->elt = *add;
+  op->fused_add = conv_operand;
+  const tvx_conv2d_desc norm = op->conv;
+  op->conv.w_scales = nullptr;
+  op->quantized = true;
+  op->has_const_weights = true;
+  op->w_zp = d->w_scales ? 0 : d->w_zp;
+  s = BuildRequantTables(d->out_c, d->in_scale, d->w_scale, d->w_scales, d->out_scale, &op->h_mult, &op->h_shift);
+  ActRange(d->out_dtype, d->out_scale, d->out_zp, d->activation, &op->act_lo, &op->act_hi);
+  if (s == TVX_OK) s = PwConvSetup(op, &norm, weights_host, bias_host);  // the kernel that has the fused form
+  if (s != TVX_OK) {
+    delete op;
+    return s == TVX_E_UNSUPPORTED ? SetError(TVX_E_UNSUPPORTED, "tvx_conv2d_add_create: no fused kernel for this convolution") : s;
+  }
+  *out = op;
+  return TVX_OK;
+}
+
 int tvx_deconv2d_create(const tvx_conv2d_desc* d, const void* weights_host, const void* bias_host,
                         tvx_op** out) {
   if (!d || !out) return SetError(TVX_E_INVALID, "tvx_deconv2d_create: null argument");
@@ -527,7 +568,7 @@ int tvx_op_run(tvx_op* op, const void* in0, const void* in1, void* out_ptr, void
   if (!in0 || !out_ptr) return SetError(TVX_E_INVALID, "tvx_op_run: null tensor pointer");
   if ((op->kind == OP_CONV2D || op->kind == OP_DECONV2D || op->kind == OP_FC) && !op->has_const_weights && !in1)
     return SetError(TVX_E_INVALID, "tvx_op_run: operator was created without weights, pass them as in1");
-  if (op->kind == OP_ADD && !in1) return SetError(TVX_E_INVALID, "tvx_op_run: Add needs two operands");
+  if ((op->kind == OP_ADD || op->fused_add) && !in1) return SetError(TVX_E_INVALID, "tvx_op_run: Add needs two operands");
   return op->run(op, in0, in1, out_ptr, static_cast<hipStream_t>(stream));
 }
 

@@ -47,6 +47,7 @@ struct tvx_op {
   const char* kernel_name = "";
   int (*run)(tvx_op*, const void* in0, const void* in1, void* out, hipStream_t) = nullptr;
   const void* bias_at_run = nullptr;  // set by tvx_op_run3 for the duration of one enqueue
+  int fused_add = 0;  // Conv2d + Add in one kernel: 1 = the convolution is the Add's first operand, 2 = its second (elt holds the Add)
 
   tvx_conv2d_desc conv{};
   tvx_fc_desc fc{};

@@ -86,6 +86,34 @@ class HipExecutor : public Executor {
       fused_act[op] = consumers[0].get();
       skipped[consumers[0].get()] = true;
     }
+    // ---- residual fusion plan: a convolution whose TRANSIENT result only feeds a same-type Add, the
+    // Add's other operand being there before the convolution runs, may become one operator
+    struct AddFusion { Operation* add; int conv_operand; };
+    std::map<Operation*, AddFusion> fused_add;  // convolution -> the Add folded into it
+    if (!std::getenv("TVX_NO_RESIDUAL_FUSION")) {  // tuning aid: keep the Adds as operators of their own
+      std::map<Tensor*, size_t> produced_at;  // position of the operator that writes a tensor
+      for (size_t i = 0; i < graph->sorted_ops_.size(); ++i)
+        for (auto& t : graph->sorted_ops_[i]->impl()->outputs_tensor_) produced_at[t.get()] = i;
+      for (size_t i = 0; i < graph->sorted_ops_.size(); ++i) {
+        Operation* add = graph->sorted_ops_[i];
+        OpImpl* aim = add->impl().get();
+        if (aim->kind_ != OpKind::ADD || aim->inputs_tensor_.size() != 2) continue;
+        for (int k = 0; k < 2; ++k) {
+          auto mid = aim->inputs_tensor_[k];
+          auto other = aim->inputs_tensor_[1 - k];
+          auto pit = produced_at.find(mid.get());
+          if (pit == produced_at.end() || !(mid->GetSpec().attr_ & TensorAttribute::TRANSIENT)) continue;
+          Operation* conv = graph->sorted_ops_[pit->second];
+          OpImpl* cim = conv->impl().get();
+          if (cim->kind_ != OpKind::CONV2D || cim->attrs_.conv_1d || fused_act.count(conv) || fused_add.count(conv)) continue;
+          if (graph->GetConsumersOp(mid).size() != 1 || mid == other) continue;
+          auto oit = produced_at.find(other.get());
+          if (oit != produced_at.end() && oit->second >= pit->second) continue;  // not there yet when the convolution runs
+          fused_add[conv] = AddFusion{add, k + 1};
+          break;
+        }
+      }
+    }
     // ---- device storage: one buffer per tensor, Reshape outputs alias their input --
     for (Operation* op : graph->sorted_ops_) {
       OpImpl* im = op->impl().get();
@@ -117,7 +145,16 @@ class HipExecutor : public Executor {
       }
       bool ok = true;
       switch (im->kind_) {
-        case OpKind::CONV2D: ok = AddConv(im, out, act); break;
+        case OpKind::CONV2D: {
+          auto fa = fused_add.find(op);
+          bool fused = false;
+          if (fa != fused_add.end()) {
+            ok = AddConv(im, out, act, false, fa->second.add->impl().get(), fa->second.conv_operand, &fused);
+            if (fused) skipped[fa->second.add] = true;
+          }
+          if (ok && !fused) ok = AddConv(im, out, act);
+          break;
+        }
         case OpKind::FCL: ok = AddFc(im, out, act); break;
         case OpKind::POOL: ok = AddPool(im, out); break;
         case OpKind::RELU: ok = AddActivation(im, out, TVX_ACT_RELU); break;
@@ -222,7 +259,11 @@ class HipExecutor : public Executor {
     }
   }
 
-  bool AddConv(OpImpl* im, TensorImpl* out, int act, bool transposed = false) {
+  // With add_im: tries the Conv2d + Add operator (conv_operand: which operand of the Add the convolution is);
+  // *fused says whether it exists for this convolution - if not, nothing has been added and the caller goes on
+  // with the two operators.
+  bool AddConv(OpImpl* im, TensorImpl* out, int act, bool transposed = false, OpImpl* add_im = nullptr,
+               int conv_operand = 0, bool* fused = nullptr) {
     TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
     TensorImpl* w = static_cast<TensorImpl*>(im->inputs_tensor_[1].get());
     TensorImpl* b = im->inputs_tensor_.size() > 2 && !im->inputs_tensor_[2]->IsPlaceHolder()
@@ -255,6 +296,27 @@ class HipExecutor : public Executor {
     const bool bias_at_run = b && !b->IsConstTensor();
     const bool const_w = w->IsConstTensor() && w->HostData() && !bias_at_run;
     tvx_op* op = nullptr;
+    if (add_im) {
+      *fused = false;
+      TensorImpl* a0 = static_cast<TensorImpl*>(add_im->inputs_tensor_[0].get());
+      TensorImpl* a1 = static_cast<TensorImpl*>(add_im->inputs_tensor_[1].get());
+      TensorImpl* sum = static_cast<TensorImpl*>(add_im->outputs_tensor_[0].get());
+      if (!const_w || a0->spec_.datatype_ != a1->spec_.datatype_ || a0->spec_.datatype_ != sum->spec_.datatype_ ||
+          a0->spec_.shape_ != a1->spec_.shape_)
+        return true;
+      tvx_eltwise_desc e{};
+      e.count = static_cast<uint64_t>(sum->spec_.GetElementNum());
+      e.dtype = DtypeCode(sum->spec_.datatype_);
+      e.a_scale = ScaleOf(a0->spec_); e.a_zp = ZpOf(a0->spec_);
+      e.b_scale = ScaleOf(a1->spec_); e.b_zp = ZpOf(a1->spec_);
+      e.out_scale = ScaleOf(sum->spec_); e.out_zp = ZpOf(sum->spec_);
+      const int st = tvx_conv2d_add_create(&d, &e, conv_operand, w->HostData(), b ? b->HostData() : nullptr, &op);
+      if (st == TVX_E_UNSUPPORTED) return true;
+      if (st != TVX_OK) return Fail("tvx_conv2d_add_create");
+      *fused = true;
+      Push(op, im, x, conv_operand == 1 ? a1 : a0, sum);
+      return true;
+    }
     if ((transposed ? tvx_deconv2d_create : tvx_conv2d_create)(&d, const_w ? w->HostData() : nullptr,
                                                                  b && !bias_at_run ? b->HostData() : nullptr, &op) != TVX_OK)
       return Fail(transposed ? "tvx_deconv2d_create" : "tvx_conv2d_create");
