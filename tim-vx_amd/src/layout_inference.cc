@@ -158,6 +158,11 @@ struct Walk {
     auto cur = mapped.at(t_src.get());
     const Perm& have = pv.at(t_src.get());
     if (have == want) return cur;
+    if (have.size() != want.size()) {
+      VSILOGE("layout inference: tensor %u has rank %zu where an operator expects rank %zu", t_src->GetId(), have.size(), want.size());
+      ok = false;
+      return nullptr;
+    }
     auto out = dst->CreateTensor(SpecFor(t_src, want, TensorAttribute::TRANSIENT));
     auto tr = dst->CreateOperation<vx::ops::Transpose>(Between(have, want));
     (*tr).BindInput(cur).BindOutput(out);
@@ -189,7 +194,13 @@ struct Walk {
     return inner;
   }
 
-  size_t RankOf(const std::shared_ptr<Tensor>& t) { return t->GetShape().size(); }
+  // TRANSIENT tensors are usually declared without a shape: their rank then comes from the permutation
+  // recorded for them when their producer was handled.
+  size_t RankOf(const std::shared_ptr<Tensor>& t) {
+    if (!t->GetShape().empty()) return t->GetShape().size();
+    auto it = pv.find(t.get());
+    return it != pv.end() ? it->second.size() : 0;
+  }
 
   void Handle(const std::shared_ptr<Operation>& op) {
     OpImpl* im = op->impl().get();
@@ -205,12 +216,11 @@ struct Walk {
     std::shared_ptr<Operation> clone;
     switch (im->kind_) {
       case OpKind::CONV2D: {
-        const size_t rank = RankOf(ins[0]);
+        const size_t rank = im->attrs_.conv_1d ? 3 : 4;
         const Perm act = im->attrs_.conv_1d ? Identity(rank) : ActivationLayout(im->layout_, rank);
         new_ins.push_back(InLayout(ins[0], act));
         if (ins.size() > 1)
-          new_ins.push_back(InLayout(ins[1], im->attrs_.conv_1d ? Identity(RankOf(ins[1]))
-                                                                : KernelLayout(im->attrs_.kernel_layout, RankOf(ins[1]))));
+          new_ins.push_back(InLayout(ins[1], im->attrs_.conv_1d ? Identity(3) : KernelLayout(im->attrs_.kernel_layout, 4)));
         for (size_t i = 2; i < ins.size(); ++i)
           new_ins.push_back(ins[i]->IsPlaceHolder() ? dst->CreateTensorPlaceHolder() : InLayout(ins[i], Identity(RankOf(ins[i]))));
         out_pv = act;
@@ -220,7 +230,7 @@ struct Walk {
         break;
       }
       case OpKind::POOL: {
-        const Perm act = im->attrs_.pool_1d ? Identity(RankOf(ins[0])) : ActivationLayout(im->layout_, RankOf(ins[0]));
+        const Perm act = im->attrs_.pool_1d ? Identity(3) : ActivationLayout(im->layout_, 4);
         new_ins.push_back(InLayout(ins[0], act));
         out_pv = act;
         clone = op->Clone(dst);
@@ -267,14 +277,21 @@ struct Walk {
       case OpKind::TRANSPOSE: {
         for (const auto& t : ins)
           new_ins.push_back(t->IsPlaceHolder() ? dst->CreateTensorPlaceHolder() : InLayout(t, Identity(RankOf(t))));
-        out_pv = Identity(RankOf(outs[0]));
+        const size_t out_rank = im->kind_ == OpKind::FCL ? 2
+                                : im->kind_ == OpKind::RESHAPE ? im->attrs_.new_shape.size()
+                                : im->kind_ == OpKind::TRANSPOSE ? im->attrs_.perm.size() : 4;
+        out_pv = Identity(out_rank);
         clone = op->Clone(dst);
         break;
       }
     }
     if (!ok || !clone) { ok = false; return; }
-    if (out_pv.empty() || (!outs[0]->GetShape().empty() && outs[0]->GetShape().size() != out_pv.size()))
-      out_pv = Identity(outs[0]->GetShape().size());
+    if (!outs[0]->GetShape().empty() && outs[0]->GetShape().size() != out_pv.size()) {
+      VSILOGE("layout inference: %s writes a rank-%zu tensor declared with rank %zu", vx::OpKindName(im->kind_),
+              out_pv.size(), outs[0]->GetShape().size());
+      ok = false;
+      return;
+    }
     auto out = OutLayout(outs[0], out_pv);
     for (auto& t : new_ins) {
       if (!t) { ok = false; return; }
