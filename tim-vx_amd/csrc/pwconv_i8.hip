@@ -251,6 +251,30 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((P
   const v4i fz = {a.neg_zws4, a.neg_zws4, a.neg_zws4, a.neg_zws4};
 
   auto epilogue = [&]() {
+    // Fused Add: the other operand's bytes for this lane's output groups are fetched first, so that
+    // the requantization below runs while they travel (a load next to the store that uses it would be
+    // a round trip per copy-out iteration: the compiler cannot move it above earlier stores).
+    constexpr int kIters = 32 / kRowsPerIter;
+    uint4 res16[GRAN == 16 ? kIters : 1];
+    uint32_t res4[GRAN == 16 ? 1 : kIters];
+    if (a.add_mode) {
+      const int rows_live = min(32, a.OC - tile * 32);
+#pragma unroll
+      for (int i = 0; i < kIters; ++i) {
+        const int row = lane / kPerRow + kRowsPerIter * i;
+        const size_t at = static_cast<size_t>(tile) * 32 * a.HW + out_off + static_cast<size_t>(row) * a.HW;
+        if (GRAN == 16) {
+          res16[i] = make_uint4(0, 0, 0, 0);
+          if (row < rows_live && out_live) res16[i] = *reinterpret_cast<const uint4*>(a.res + at);
+        } else {
+          res4[i] = 0;
+          if (row < rows_live && out_whole) {
+            if (GRAN == 4) res4[i] = *reinterpret_cast<const uint32_t*>(a.res + at);
+            else __builtin_memcpy(&res4[i], a.res + at, 4);
+          }
+        }
+      }
+    }
     const int oc = tile * 32 + frag_row;
     const v4i q = a.rq[oc];
     const int lo = a.lo, hi = a.hi;
@@ -279,7 +303,7 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((P
           uint4 o = make_uint4(lo8.x, lo8.y, hi8.x, hi8.y);
           const size_t at = static_cast<size_t>(tile) * 32 * a.HW + out_off + static_cast<size_t>(row) * a.HW;
           if (a.add_mode) {
-            const uint4 r = *reinterpret_cast<const uint4*>(a.res + at);
+            const uint4 r = res16[i];
             o = make_uint4(AddResidual4(a, o.x, r.x), AddResidual4(a, o.y, r.y), AddResidual4(a, o.z, r.z),
                            AddResidual4(a, o.w, r.w));
           }
@@ -294,12 +318,7 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((P
         const size_t row_at = static_cast<size_t>(tile) * 32 * a.HW + static_cast<size_t>(row) * a.HW;
         if (row < rows && out_whole) {
           uint8_t* o = a.y + row_at + out_off;
-          if (a.add_mode) {
-            uint32_t r;
-            if (GRAN == 4) r = *reinterpret_cast<const uint32_t*>(a.res + row_at + out_off);
-            else __builtin_memcpy(&r, a.res + row_at + out_off, 4);
-            v = AddResidual4(a, v, r);
-          }
+          if (a.add_mode) v = AddResidual4(a, v, res4[i]);
           if (GRAN == 4) *reinterpret_cast<uint32_t*>(o) = v;
           else __builtin_memcpy(o, &v, 4);
         } else if (GRAN == 1 && row < rows) {
