@@ -209,7 +209,10 @@ def network_extras(steps, warmup):
     z = np.load(os.path.join(REPO, "tests", "golden", "lenet_asymu8.npz"))
     nets = [("lenet_asymu8_b1", G.lenet_asymu8(z["weights"], z["input"], batch=1), 1),
             ("lenet_asymu8_b256", G.lenet_asymu8(z["weights"], z["input"], batch=256), 256),
-            ("mobilenet_v2_u8_b64_224", G.mobilenet_v2(batch=64, res=224), 64)]
+            ("mobilenet_v2_u8_b64_224", G.mobilenet_v2(batch=64, res=224), 64),
+            # the headline convolution as an application reaches it: through the C++ API, with the host copies
+            # of its input and output (run_ms is the PCIe-inclusive time, device_ms the operator alone)
+            ("conv3x3_u8_64to64_56x56_b32_cpp_api", G.conv3x3_same_relu6(), 32)]
     out = {}
     with tempfile.TemporaryDirectory() as d:
         _, info, _ = GF.run_graphs([g for _, g, _ in nets], d, bench=(warmup, steps))

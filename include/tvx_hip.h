@@ -61,6 +61,11 @@ int tvx_device_count(void);
  * vxCopyTensorPatch: src/tim/vx/tensor.cc:154-228). */
 int tvx_malloc(void** dev_ptr, size_t bytes);
 int tvx_free(void* dev_ptr);
+/* Page-locked host memory for tensors the application fills and reads (the host-visible buffers
+ * behind vsi_nn_AddTensorFromHandle, src/tim/vx/tensor.cc:415-437): copies from and to it run at
+ * the link's rate and without a staging copy. */
+int tvx_host_malloc(void** host_ptr, size_t bytes);
+int tvx_host_free(void* host_ptr);
 int tvx_memcpy_h2d(void* dst_dev, const void* src_host, size_t bytes, void* stream);
 int tvx_memcpy_d2h(void* dst_host, const void* src_dev, size_t bytes, void* stream);
 int tvx_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* stream);

@@ -623,3 +623,31 @@ def test_pointwise_conv_with_fused_add(oracle, side, n, mode, conv_operand):
     with pytest.raises(T.TvxError) as err:
         T.conv2d_add_create(d, e, conv_operand, w3, b)
     assert err.value.status == T.E_UNSUPPORTED
+
+
+def test_page_locked_host_memory_round_trip():
+    """tvx_host_malloc memory as source and target of the library's copies."""
+    import ctypes as C
+    T = TC.tvx()
+    L = T.lib()
+    vp = C.c_void_p
+    L.tvx_host_malloc.argtypes = [C.POINTER(vp), C.c_size_t]
+    L.tvx_host_free.argtypes = [vp]
+    L.tvx_malloc.argtypes = [C.POINTER(vp), C.c_size_t]
+    L.tvx_free.argtypes = [vp]
+    for f in (L.tvx_memcpy_h2d, L.tvx_memcpy_d2h):
+        f.argtypes = [vp, vp, C.c_size_t, vp]
+    L.tvx_stream_synchronize.argtypes = [vp]
+    n = 1 << 20
+    src, dst, dev = vp(), vp(), vp()
+    assert L.tvx_host_malloc(C.byref(src), n) == 0 and L.tvx_host_malloc(C.byref(dst), n) == 0
+    assert L.tvx_malloc(C.byref(dev), n) == 0
+    data = np.random.default_rng(5).integers(0, 256, n, dtype=np.uint8)
+    C.memmove(src, data.ctypes.data, n)
+    assert L.tvx_memcpy_h2d(dev, src, n, None) == 0 and L.tvx_memcpy_d2h(dst, dev, n, None) == 0
+    assert L.tvx_stream_synchronize(None) == 0
+    back = np.frombuffer((C.c_uint8 * n).from_address(dst.value), dtype=np.uint8)
+    assert np.array_equal(back, data)
+    assert L.tvx_host_free(src) == 0 and L.tvx_host_free(dst) == 0 and L.tvx_free(dev) == 0
+    empty = vp(1)
+    assert L.tvx_host_malloc(C.byref(empty), 0) == 0 and not empty.value

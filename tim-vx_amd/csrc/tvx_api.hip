@@ -195,6 +195,22 @@ int tvx_malloc(void** dev_ptr, size_t bytes) {
   return TVX_OK;
 }
 
+int tvx_host_malloc(void** host_ptr, size_t bytes) {
+  if (!host_ptr) return SetError(TVX_E_INVALID, "tvx_host_malloc: null result pointer");
+  *host_ptr = nullptr;
+  if (bytes == 0) return TVX_OK;
+  if (tvx_device_count() <= 0) return SetError(TVX_E_DEVICE, "no HIP device: page-locked memory needs one");
+  hipError_t e = hipHostMalloc(host_ptr, bytes, hipHostMallocDefault);
+  if (e == hipErrorOutOfMemory) return SetError(TVX_E_NOMEM, "hipHostMalloc(%zu) out of memory", bytes);
+  if (e != hipSuccess) return SetError(TVX_E_DEVICE, "hipHostMalloc(%zu): %s", bytes, hipGetErrorString(e));
+  return TVX_OK;
+}
+
+int tvx_host_free(void* host_ptr) {
+  if (host_ptr) TVX_HIP_CHECK(hipHostFree(host_ptr));
+  return TVX_OK;
+}
+
 int tvx_free(void* dev_ptr) {
   if (dev_ptr) TVX_HIP_CHECK(hipFree(dev_ptr));
   return TVX_OK;

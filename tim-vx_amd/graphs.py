@@ -167,6 +167,22 @@ def mobilenet_v2(batch=1, res=224, classes=1000, seed=0):
             "output": logits["id"]}
 
 
+def conv3x3_same_relu6(batch=32, channels=64, side=56, seed=0x71):
+    """One uint8 per-tensor 3x3 convolution with SAME padding and a Relu6 behind it (fused by the runtime):
+    the single-operator benchmark configuration as an application would build it."""
+    rng = np.random.default_rng(seed)
+    c, s, n = channels, side, batch
+    q = asym
+    return {"test": "conv3x3_u8_%dto%d_%dx%d_b%d" % (c, c, s, s, n), "output": 4, "tensors": [
+        tensor(0, "UINT8", "INPUT", [s, s, c, n], q(0.05, 128), rng.integers(0, 256, n * c * s * s, dtype=np.uint8)),
+        tensor(1, "UINT8", "CONSTANT", [3, 3, c, c], q(0.01, 120), rng.integers(0, 256, c * c * 9, dtype=np.uint8)),
+        tensor(2, "INT32", "CONSTANT", [c], q(0.0005, 0), rng.integers(-4096, 4097, c).astype(np.int32)),
+        tensor(3, "UINT8", "TRANSIENT", [s, s, c, n], q(0.1, 0)),
+        tensor(4, "UINT8", "OUTPUT", [s, s, c, n], q(0.1, 0))],
+        "ops": [op("CONV2D", [0, 1, 2], [3], pad_type="SAME", ksize=[3, 3], weights=c),
+                op("RELU6", [3], [4])]}
+
+
 def mac_count(graph):
     """Multiply-accumulates of every CONV2D / FCL of a graph description."""
     ts = {t["id"]: t for t in graph["tensors"]}

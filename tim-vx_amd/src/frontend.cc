@@ -204,7 +204,17 @@ TensorImpl::TensorImpl(GraphImpl* graph, const TensorSpec& spec,
   }
 }
 
-TensorImpl::~TensorImpl() {}
+void* (*g_host_alloc)(size_t bytes) = nullptr;
+void (*g_host_free)(void* p) = nullptr;
+
+TensorImpl::~TensorImpl() { ReleaseOwned(); }
+
+void TensorImpl::ReleaseOwned() {
+  if (owned_ && owned_free_) owned_free_(owned_);
+  owned_ = nullptr;
+  owned_bytes_ = 0;
+  owned_free_ = nullptr;
+}
 
 size_t TensorImpl::HostBytes() const {
   size_t n = DataTypeBytes(spec_.datatype_);
@@ -215,12 +225,27 @@ size_t TensorImpl::HostBytes() const {
 void TensorImpl::EnsureHostBuffer() {
   if (user_ptr_) return;
   size_t n = HostBytes();
-  if (owned_.size() != n) owned_.assign(n, 0);
+  if (owned_bytes_ == n && (owned_ || n == 0)) return;
+  ReleaseOwned();
+  if (n == 0) return;
+  const bool io = (spec_.attr_ & (TensorAttribute::INPUT | TensorAttribute::OUTPUT)) != 0;
+  if (io && g_host_alloc && g_host_free) {
+    owned_ = static_cast<uint8_t*>(g_host_alloc(n));
+    if (owned_) owned_free_ = g_host_free;
+  }
+  if (!owned_) {
+    owned_ = static_cast<uint8_t*>(std::malloc(n));
+    owned_free_ = std::free;
+  }
+  if (owned_) {
+    owned_bytes_ = n;
+    std::memset(owned_, 0, n);
+  }
 }
 
 uint8_t* TensorImpl::HostData() {
   if (user_ptr_) return user_ptr_;
-  return owned_.empty() ? nullptr : owned_.data();
+  return owned_;
 }
 
 bool TensorImpl::CopyDataToTensor(const void* data, uint32_t size_in_bytes) {

@@ -485,6 +485,21 @@ std::unique_ptr<Executor> CreateExecutor() {
   return std::unique_ptr<Executor>(new HipExecutor());
 }
 
+// Host images of INPUT / OUTPUT tensors in page-locked memory (falls back to ordinary memory without a GPU).
+namespace {
+void* PinnedAlloc(size_t bytes) {
+  void* p = nullptr;
+  return tvx_host_malloc(&p, bytes) == TVX_OK ? p : nullptr;
+}
+void PinnedFree(void* p) { (void)tvx_host_free(p); }
+struct OfferPinnedMemory {
+  OfferPinnedMemory() {
+    g_host_alloc = PinnedAlloc;
+    g_host_free = PinnedFree;
+  }
+} g_offer_pinned_memory;
+}  // namespace
+
 }  // namespace vx
 }  // namespace tim
 

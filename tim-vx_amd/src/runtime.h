@@ -129,7 +129,12 @@ class TensorImpl : public Tensor {
   GraphImpl* graph_;
   uint32_t id_;
   TensorSpec spec_;
-  std::vector<uint8_t> owned_;
+  // The tensor's own host image: page-locked memory for INPUT / OUTPUT tensors when the executor offers
+  // it (g_host_alloc), ordinary memory otherwise.
+  uint8_t* owned_ = nullptr;
+  size_t owned_bytes_ = 0;
+  void (*owned_free_)(void*) = nullptr;
+  void ReleaseOwned();
   uint8_t* user_ptr_ = nullptr;  // CreateIOTensor(spec, ptr) / SwapHandle
   bool host_dirty_ = false;      // host image newer than the device copy
   int8_t is_scalar_ = 0;
@@ -152,6 +157,9 @@ class Executor {
   virtual bool Execute(GraphImpl* graph) = 0;
 };
 std::unique_ptr<Executor> CreateExecutor();
+// Host memory the executor can copy from / to fastest (null: none on offer). Set by the executor's module.
+extern void* (*g_host_alloc)(size_t bytes);
+extern void (*g_host_free)(void* p);
 
 class ContextImpl : public Context {
  public:
