@@ -40,10 +40,12 @@ struct ImArgs {
   int zws, out_zp, lo, hi;
   int out_stride;        // epilogue staging row stride in bytes (odd number of dwords)
   int off_a, off_w, off_sx, off_rq, off_bias;  // LDS carve-up
-  // The window, one word per reduction index: c | dy << 8 | dx << 16 | 1 << 24, zero past the end.
-  // It travels in the kernel arguments so that the (wavefront-uniform) reads of it are scalar loads
-  // of memory nothing can write; a table in global memory is read per lane, one round trip a tap.
+  // The window, per reduction index: dy | dx << 8 | 1 << 16 (zero past the end) and the input offset
+  // c * H * W + dy * W + dx. They travel in the kernel arguments so that the (wavefront-uniform) reads
+  // are scalar loads of memory nothing can write; a table in global memory is read per lane, one round
+  // trip a tap.
   int taps[64];
+  int offs[64];
 };
 
 template <int OT, int RQ>
@@ -85,20 +87,27 @@ __global__ void __launch_bounds__(kThreads) ConvIm2colKernel(ImArgs a) {
     const int ih0 = oh * a.sh - a.pad_t, iw0 = ow * a.sw - a.pad_l;
     const uint8_t* img = a.x + static_cast<size_t>(n) * a.C * a.H * a.W;
     const int origin = ih0 * a.W + iw0;  // may be negative; only added to offsets of taps inside the image
-    const int plane = a.H * a.W;
+    // Which window rows / columns (offsets 0..31 from the window's origin) lie inside the image, as bit
+    // masks: a tap's validity is then two shifts and an AND instead of two additions and two compares.
+    auto span_mask = [](int first, int extent) {  // bits d with 0 <= first + d < extent, d in 0..31
+      const int lo = max(0, -first), hi = min(32, extent - first);
+      const int n = hi - lo;
+      return n <= 0 ? 0u : ((n >= 32 ? 0xffffffffu : ((1u << n) - 1u)) << lo);
+    };
+    const uint32_t row_ok = span_mask(ih0, a.H), col_ok = span_mask(iw0, a.W);
     for (int k0 = 0; k0 < a.kp; k0 += 16) {
       int b[16];
-      bool inside[16], real[16];
+      bool inside[16];
+      int fill[16];
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
-        const int t = a.taps[k0 + j];
-        const int c = t & 0xff, dy = (t >> 8) & 0xff, dx = (t >> 16) & 0xff;
-        real[j] = (t >> 24) != 0;
+        const int t = a.taps[k0 + j];  // scalar: dy | dx << 8 | real << 16
+        const int dy = t & 0xff, dx = (t >> 8) & 0xff;
+        const uint32_t real = 0u - static_cast<uint32_t>(t >> 16);  // all ones or zero
+        fill[j] = a.pad_fill & static_cast<int>(real);
         // bitwise, not short-circuit: no branch may stand between the loads
-        inside[j] = real[j] & (static_cast<unsigned>(ih0 + dy) < static_cast<unsigned>(a.H)) &
-                    (static_cast<unsigned>(iw0 + dx) < static_cast<unsigned>(a.W));
-        const int off = c * plane + dy * a.W + dx;  // scalar arithmetic
-        b[j] = img[static_cast<uint32_t>(inside[j] ? origin + off : 0)];  // uniform base + 32-bit lane offset
+        inside[j] = ((row_ok >> dy) & (col_ok >> dx) & real & 1u) != 0;
+        b[j] = img[static_cast<uint32_t>(inside[j] ? origin + a.offs[k0 + j] : 0)];  // uniform base + 32-bit lane offset
       }
       __builtin_amdgcn_sched_barrier(0);  // all sixteen loads travel together
       int dw[4];
@@ -108,8 +117,8 @@ __global__ void __launch_bounds__(kThreads) ConvIm2colKernel(ImArgs a) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int j = q * 4 + e;
-          const int byte = inside[j] ? (b[j] ^ a.xor_mask) : (real[j] ? a.pad_fill : 0);
-          v |= (byte & 0xff) << (8 * e);
+          const int byte = inside[j] ? (b[j] ^ a.xor_mask) : fill[j];  // both below 256
+          v |= byte << (8 * e);
         }
         dw[q] = v;
         sx = __builtin_amdgcn_sdot4(v, 0x01010101, sx, false);
@@ -268,12 +277,13 @@ int ConvIm2colSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, co
   std::vector<int32_t> rqt;
   const int rq = BuildRequantRecords(op->h_mult, op->h_shift, a.OC, a.oct, d->out_zp, &rqt,
                                      AccumulatorBound(static_cast<uint64_t>(K), bias_host, a.OC));
-  if (d->k_h * d->dilation_h > 255 || d->k_w * d->dilation_w > 255) return TVX_E_UNSUPPORTED;  // dy, dx in a byte
+  if ((d->k_h - 1) * d->dilation_h > 31 || (d->k_w - 1) * d->dilation_w > 31) return TVX_E_UNSUPPORTED;  // window offsets index 32-bit masks
   for (int k = 0; k < K; ++k) {
     const int c = k / taps, t = k % taps;
     const int dy = (t / static_cast<int>(d->k_w)) * static_cast<int>(d->dilation_h);
     const int dx = (t % static_cast<int>(d->k_w)) * static_cast<int>(d->dilation_w);
-    a.taps[k] = c | dy << 8 | dx << 16 | 1 << 24;
+    a.taps[k] = dy | dx << 8 | 1 << 16;
+    a.offs[k] = c * a.H * a.W + dy * a.W + dx;
   }
   int s = op->packed.Upload(packed.data(), packed.size());
   if (s == TVX_OK) s = op->aux.Upload(biasf.data(), biasf.size() * 4);
