@@ -164,6 +164,23 @@ def test_eltwise_quantized(oracle, dtype):
     assert np.allclose(sm_got, sm_want, rtol=1e-4, atol=1e-7)
 
 
+@pytest.mark.parametrize("c", [1, 3, 4, 5, 16, 17, 64, 65, 1000, 1001, 1024, 1025, 3000])
+def test_softmax_group_sizes(oracle, c):
+    # every lanes-per-group choice of the register-resident kernel, its upper limit and the strided
+    # kernel past it; a row count that leaves the last wavefront partly empty
+    rng = np.random.default_rng(c)
+    rows = 37
+    x = rand_q(rng, rows * c, 0)
+    want = oracle.softmax(0, x, c, 0.7, (0.05, 131))
+    got = TC.gpu_softmax(0, x, c, 0.7, (0.05, 131))
+    assert np.allclose(got, want, rtol=1e-4, atol=1e-9)
+    assert np.allclose(got.reshape(rows, c).sum(axis=1), 1.0, atol=1e-5)
+    f = (rng.standard_normal(rows * c) * 3).astype(np.float32)
+    for beta in (1.0, -0.5):
+        want = oracle.softmax(3, f, c, beta, (1.0, 0))
+        assert np.allclose(TC.gpu_softmax(3, f, c, beta, (1.0, 0)), want, rtol=1e-4, atol=1e-9)
+
+
 def test_eltwise_float(oracle):
     rng = np.random.default_rng(3)
     a = (rng.standard_normal(5000) * 4).astype(np.float32)

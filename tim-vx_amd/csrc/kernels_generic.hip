@@ -584,7 +584,7 @@ template <typename T, bool QUANT>
 __global__ void __launch_bounds__(kBlock)
 SoftmaxKernel(int c, uint64_t rows, uint64_t inner, float beta, float scale, int zp, const T* __restrict__ x,
               float* __restrict__ y) {
-  // one thread per (row, inner position); the c elements of its group are `inner` apart
+  // any axis: one thread per (row, inner position); the c elements of its group are `inner` apart
   const uint64_t t = static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x;
   if (t >= rows * inner) return;
   const uint64_t base = (t / inner) * c * inner + t % inner;
@@ -607,10 +607,86 @@ SoftmaxKernel(int c, uint64_t rows, uint64_t inner, float beta, float scale, int
   for (int i = 0; i < c; ++i) yp[i * inner] = yp[i * inner] / sum;
 }
 
+// Contiguous groups of at most 64 * kSmVals elements: G lanes share a group and keep its
+// elements in registers between the three passes (maximum, exponentials and their sum,
+// division), so that the group is read once and written once.
+constexpr int kSmVals = 16;
+
+template <typename T, bool QUANT, int G>
+__global__ void __launch_bounds__(kBlock)
+SoftmaxRowKernel(int c, uint64_t rows, float beta, float scale, int zp, const T* __restrict__ x,
+                 float* __restrict__ y) {
+  const uint64_t row = (static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x) / G;
+  const int lane = threadIdx.x % G;
+  // lanes past the last row stay for the shuffles and touch no memory
+  const int live = row < rows ? c : 0;
+  const T* xp = x + row * c;
+  float* yp = y + row * c;
+  float v[kSmVals];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < kSmVals; ++j) {
+    const int i = lane + j * G;
+    v[j] = -INFINITY;
+    if (i < live) {
+      if constexpr (QUANT) v[j] = scale * static_cast<float>(static_cast<int>(xp[i]) - zp);
+      else v[j] = ToFloat(xp[i]);
+    }
+    mx = v[j] > mx ? v[j] : mx;
+  }
+#pragma unroll
+  for (int o = G / 2; o; o >>= 1) {
+    const float other = __shfl_xor(mx, o, 64);
+    mx = other > mx ? other : mx;
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < kSmVals; ++j) {
+    const int i = lane + j * G;
+    v[j] = i < live ? expf(beta * (v[j] - mx)) : 0.f;
+    sum += v[j];
+  }
+#pragma unroll
+  for (int o = G / 2; o; o >>= 1) sum += __shfl_xor(sum, o, 64);
+#pragma unroll
+  for (int j = 0; j < kSmVals; ++j) {
+    const int i = lane + j * G;
+    if (i < live) yp[i] = v[j] / sum;
+  }
+}
+
+template <typename T, bool QUANT>
+static void LaunchSoftmaxRows(const tvx_softmax_desc& d, int zp, float scale, const void* in0, float* y,
+                              hipStream_t st) {
+  const int c = static_cast<int>(d.channels);
+  const T* x = static_cast<const T*>(in0);
+  const dim3 block(kBlock);
+  // the fewest lanes that leave at most four elements to each, 64 from there on
+  const int g = c <= 4 ? 1 : (c <= 16 ? 4 : (c <= 64 ? 16 : 64));
+  const dim3 grid(Blocks(d.rows * g));
+  switch (g) {
+    case 1: hipLaunchKernelGGL((SoftmaxRowKernel<T, QUANT, 1>), grid, block, 0, st, c, d.rows, d.beta, scale, zp, x, y); break;
+    case 4: hipLaunchKernelGGL((SoftmaxRowKernel<T, QUANT, 4>), grid, block, 0, st, c, d.rows, d.beta, scale, zp, x, y); break;
+    case 16: hipLaunchKernelGGL((SoftmaxRowKernel<T, QUANT, 16>), grid, block, 0, st, c, d.rows, d.beta, scale, zp, x, y); break;
+    default: hipLaunchKernelGGL((SoftmaxRowKernel<T, QUANT, 64>), grid, block, 0, st, c, d.rows, d.beta, scale, zp, x, y);
+  }
+}
+
 int SoftmaxRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
   const tvx_softmax_desc& d = op->sm;
   if (!d.rows) return TVX_OK;
   const uint64_t inner = d.inner ? d.inner : 1;
+  if (inner == 1 && d.channels <= 64u * kSmVals) {
+    float* yr = static_cast<float*>(out);
+    switch (d.in_dtype) {
+      case TVX_U8: LaunchSoftmaxRows<uint8_t, true>(d, d.in_zp, d.in_scale, in0, yr, st); break;
+      case TVX_I8: LaunchSoftmaxRows<int8_t, true>(d, d.in_zp, d.in_scale, in0, yr, st); break;
+      case TVX_F32: LaunchSoftmaxRows<float, false>(d, 0, 1.f, in0, yr, st); break;
+      default: LaunchSoftmaxRows<__half, false>(d, 0, 1.f, in0, yr, st);
+    }
+    TVX_HIP_CHECK(hipGetLastError());
+    return TVX_OK;
+  }
   const dim3 grid(Blocks(d.rows * inner)), block(kBlock);
   float* y = static_cast<float*>(out);
   const int c = static_cast<int>(d.channels);
