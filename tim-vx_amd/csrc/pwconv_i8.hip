@@ -45,7 +45,8 @@ struct PwArgs {
   int ksteps;            // cp / 32
   int pix_stride;        // LDS bytes per pixel: cp + 16 (an odd number of 16-byte chunks)
   int oc_tiles;          // ceil(OC / 32)
-  int tiles_per_wg;      // output tiles one workgroup walks (grid.y covers the rest)
+  int tiles_per_wg;      // output tiles one workgroup walks
+  int tile_groups;       // workgroups that share a pixel tile (oc_tiles / tiles_per_wg, rounded up)
   int xor_mask;          // 0x80808080 for uint8 activations
   int neg_zws4;          // -(weight zero point, int8 domain) in all four bytes
   int out_zp, lo, hi;
@@ -106,12 +107,24 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((P
   constexpr int kRowBytes = 32 * PT;  // staged bytes per output row
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = NW == 1 ? 0 : __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int q_base = blockIdx.x * kPix;
+  // Workgroups go to the eight XCDs round-robin in launch order and each XCD has its own L2:
+  // renumber them so that an XCD gets a contiguous run of (pixel tile, output-tile group) pairs,
+  // pixel tiles in order and the groups of one pixel tile next to each other. A 32-pixel row
+  // segment is a quarter of a cache line and neighbouring pixel tiles take the other quarters;
+  // spread over four XCDs, every line would cross the fabric four times.
+  int wg = blockIdx.x;
+  {
+    const int per = gridDim.x >> 3, rem = gridDim.x & 7, xcd = wg & 7;
+    wg = xcd * per + min(xcd, rem) + (wg >> 3);
+  }
+  const int pix_tile = static_cast<int>(static_cast<uint32_t>(wg) / static_cast<uint32_t>(a.tile_groups));
+  const int tile_group = wg - pix_tile * a.tile_groups;
+  const int q_base = pix_tile * kPix;
   int8_t* xl = lds;
   int8_t* stage = lds + kPix * a.pix_stride + wave * kStageBytes;
 
   // ---- work items of this wavefront: (output tile, pixel part) ---------------------------
-  const int t_begin = blockIdx.y * a.tiles_per_wg;
+  const int t_begin = tile_group * a.tiles_per_wg;
   const int t_end = min(t_begin + a.tiles_per_wg, a.oc_tiles);
   // wavefront w takes items w, w + NW, ...; with kParts | NW its pixel part never changes
   const int part = wave % kParts;
@@ -127,6 +140,11 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((P
   v4i nf[kRing];
 #pragma unroll
   for (int j = 0; j < kRing; ++j) nf[j] = *frag_ptr(n_tiles > 0 ? tile0 : 0, min(j, a.ksteps - 1));
+  // The folded bias and the requantization record of a tile travel with its first fragments: asked
+  // for inside a tile's own computation they would each be a round trip that also waits for the
+  // previous tile's stores (loads and stores complete in issue order).
+  int nb = a.biasf[(n_tiles > 0 ? tile0 : 0) * 32 + (lane & 31)];
+  v4i nq = a.rq[(n_tiles > 0 ? tile0 : 0) * 32 + (lane & 31)];
 
   // ---- activations of the 128 pixels, all channels: global (pixel-innermost) -> LDS
   {
@@ -241,8 +259,10 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((P
       for (int r = 0; r < 16; ++r) accz[i][r] = 0;
   }
   int tile = tile0;
+  v4i q;
   auto init_acc = [&]() {
-    const int b = a.biasf[tile * 32 + frag_row];
+    const int b = nb;
+    q = nq;
 #pragma unroll
     for (int i = 0; i < PT; ++i)
 #pragma unroll
@@ -275,8 +295,6 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((P
         }
       }
     }
-    const int oc = tile * 32 + frag_row;
-    const v4i q = a.rq[oc];
     const int lo = a.lo, hi = a.hi;
 #pragma unroll
     for (int i = 0; i < PT; ++i)
@@ -372,6 +390,8 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((P
     const int next_tile = tile + tile_step < t_end ? tile + tile_step : tile;
 #pragma unroll
     for (int j = 0; j < kRing; ++j) nf[j] = *frag_ptr(next_tile, min(j, a.ksteps - 1));
+    nb = a.biasf[next_tile * 32 + frag_row];
+    nq = a.rq[next_tile * 32 + frag_row];
     epilogue();
   }
 }
@@ -512,6 +532,8 @@ int PwConvSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const 
   int gy = static_cast<int>(std::min<long long>(quads, std::max<long long>(1, want_wgs / gx)));
   a.tiles_per_wg = std::min(((quads + gy - 1) / gy) * nw, a.oc_tiles);
   gy = (a.oc_tiles + a.tiles_per_wg - 1) / a.tiles_per_wg;
+  a.tile_groups = gy;
+  if (gx * gy > 0x7fffffffll) return TVX_E_UNSUPPORTED;
   // fewer output tiles than wavefronts: split the pixels of a tile over wavefronts instead
   const int pt = kp == 32 ? 1 : (nw == 1 ? 4 : (a.tiles_per_wg >= 4 ? 4 : (a.tiles_per_wg >= 2 ? 2 : 1)));
 
@@ -554,7 +576,7 @@ int PwConvSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const 
   plan.gran = (a.HW % 16 == 0) ? 16 : ((a.HW % 4 == 0) ? 4 : 1);
   plan.zp = zws != 0;
   plan.rq = rq;
-  plan.grid = dim3(static_cast<unsigned>(gx), static_cast<unsigned>(gy));
+  plan.grid = dim3(static_cast<unsigned>(gx * gy));
   s = Dispatch(&plan, a, nullptr, true);
   if (s != TVX_OK) return s;
   op->host_blob.assign(reinterpret_cast<const uint8_t*>(&plan), reinterpret_cast<const uint8_t*>(&plan) + sizeof(plan));
