@@ -333,7 +333,7 @@ def test_conv2d_igemm_shapes(oracle, gi, mode):
 
 PW_GRID = [
     # (n, c, h, w, oc): 1x1 stride 1; HW % 16 == 0, % 4 == 0 and odd sizes; channel tails;
-    # few and many output tiles; a tile that straddles images
+    # few and many output tiles; a tile that straddles images; images of fewer than four pixels
     (2, 32, 16, 16, 64),
     (3, 16, 14, 14, 96),
     (5, 24, 7, 7, 144),
@@ -343,6 +343,10 @@ PW_GRID = [
     (2, 576, 14, 14, 96),
     (1, 40, 20, 13, 33),
     (2, 130, 6, 6, 200),
+    (4, 33, 1, 1, 40),
+    (3, 8, 1, 3, 9),
+    (2, 70, 2, 1, 5),
+    (1, 2, 1, 2, 3),
 ]
 
 

@@ -40,7 +40,10 @@ struct PwArgs {
   const int32_t* biasf;  // bias + per-channel zero-point terms
   const v4i* rq;         // per channel requantization record
   int C, OC, HW;
-  int Q;                 // batch * HW (< 2^31 - 256: flat pixel indices are 32-bit)
+  int HWp;               // pixels per image on the flat pixel axis: HW, rounded up to 4 when HW % 4 != 0,
+                         // so that a 4-pixel group never straddles two images (the padding pixels are
+                         // computed and dropped)
+  int Q;                 // batch * HWp (< 2^31 - 256: flat pixel indices are 32-bit)
   int cp;                // channels padded to 32
   int ksteps;            // cp / 32
   int pix_stride;        // LDS bytes per pixel: cp + 16 (an odd number of 16-byte chunks)
@@ -149,59 +152,50 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((P
   // ---- activations of the 128 pixels, all channels: global (pixel-innermost) -> LDS
   {
     // A thread takes a group of 4 consecutive flat pixels and 16 channels per pass: 16 dword
-    // loads in flight, 4x4 byte transposes, four 16-byte LDS stores. With GRAN 1 a group may
-    // start at any byte (the dword loads are then unaligned, which global memory allows) and
-    // may straddle two images or the end of the batch.
+    // loads in flight, 4x4 byte transposes, four 16-byte LDS stores.
     constexpr int kQuads = KP / 4;
     const int pq = tid % kQuads, cg0 = tid / kQuads;  // 4-pixel group, first 16-channel group
     const int q0 = q_base + pq * 4;
     const bool live = q0 < a.Q;
-    const int n = live ? static_cast<int>(static_cast<uint32_t>(q0) / static_cast<uint32_t>(a.HW)) : 0;
-    const int p = live ? static_cast<int>(q0 - n * a.HW) : 0;
-    const bool whole = GRAN >= 4 ? live : (q0 + 3 < a.Q && p + 3 < a.HW);
+    const int n = live ? static_cast<int>(static_cast<uint32_t>(q0) / static_cast<uint32_t>(a.HWp)) : 0;
+    const int p = live ? static_cast<int>(q0 - n * a.HWp) : 0;
+    // GRAN 1: the last group of an image holds fewer than four of its pixels
+    const bool whole = GRAN >= 4 ? live : (live && p + 3 < a.HW);
     const uint8_t* src = a.x + (static_cast<size_t>(n) * a.C) * a.HW + p;
-    // GRAN 1, group straddling two images (or the end of the batch): its first k pixels end
-    // image n, the rest start image n + 1. Both parts are fetched as unaligned dwords - the
-    // second one shifted so that its bytes land in lanes k..3 - and merged with a byte mask.
-    // The bytes such a dword reads outside its own row belong to neighbouring rows of the
-    // tensor, except behind the very last row, which is therefore read byte by byte.
-    const int k_first = GRAN == 1 && live && !whole ? a.HW - p : 4;
-    const uint32_t mask_first = k_first >= 4 ? 0xffffffffu : ((1u << (8 * k_first)) - 1u);
-    const bool has_second = GRAN == 1 && live && !whole && q0 + k_first < a.Q;
-    const uint8_t* src2 = has_second ? a.x + (static_cast<size_t>(n + 1) * a.C) * a.HW - k_first : src;
     // Every load below is unconditional - a load under a per-lane condition becomes a branch
     // and a full wait, sixteen round trips instead of one: lanes and channels with nothing to
     // fetch read a valid address (channel clamped, src at the tensor base) and are masked.
-    // The last row of the tensor must not be read past its end: there the dword is fetched
-    // 4 - k bytes early and shifted down.
-    const bool last_image = GRAN == 1 && live && !whole && static_cast<long long>(n + 1) * a.HW >= a.Q;
-    const int back = last_image ? 4 - k_first : 0;
-    const bool any_split = GRAN == 1 && __any(live && !whole);
+    // With GRAN 1 a group may start at any byte (the dword loads are then unaligned, which
+    // global memory allows), and the dword of an image's last group reaches past the end of its
+    // row into the next row of the tensor; only behind the very last row there is nothing:
+    // there the dword is fetched 4 - k bytes early and shifted down.
+    const bool last_row_tail = GRAN == 1 && live && !whole && static_cast<long long>(n + 1) * a.HWp >= a.Q;
+    const int back = last_row_tail ? 4 - (a.HW - p) : 0;
+    // lanes with nothing to fetch stay on the first dword of the tensor: with images of fewer than
+    // four pixels a dword at a later row of the first image could end behind a one-image tensor
+    const size_t row_stride = (GRAN == 1 && !live) ? 0 : static_cast<size_t>(a.HW);
     for (int cg = cg0; cg < a.cp / 16; cg += kThreads / kQuads) {
       uint32_t raw[16];
 #pragma unroll
       for (int j = 0; j < 16; ++j) {
         const int c = cg * 16 + j;
-        const uint8_t* row = src + static_cast<size_t>(min(c, a.C - 1)) * a.HW;
-        uint32_t v;
+        const uint8_t* row = src + static_cast<size_t>(min(c, a.C - 1)) * row_stride;
         if (GRAN >= 4) {
-          v = *reinterpret_cast<const uint32_t*>(row);
+          raw[j] = *reinterpret_cast<const uint32_t*>(row);
         } else {
-          const int bk = c == a.C - 1 ? back : 0;
-          __builtin_memcpy(&v, row - bk, 4);
-          v >>= 8 * bk;
+          const int bk = c >= a.C - 1 ? back : 0;  // padding channels re-read the last one
+          __builtin_memcpy(&raw[j], row - bk, 4);
         }
-        raw[j] = (live && c < a.C) ? v ^ a.xor_mask : 0u;
       }
-      if (any_split) {
+      // all sixteen loads are issued before the first one is used: left to itself the scheduler
+      // sometimes pairs every load with its use, sixteen round trips instead of one
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int j = 0; j < 16; ++j) {
-          const int c = cg * 16 + j;
-          uint32_t v;
-          __builtin_memcpy(&v, src2 + static_cast<size_t>(min(c, a.C - 1)) * a.HW, 4);
-          v = (has_second && c < a.C) ? v ^ a.xor_mask : 0u;
-          raw[j] = (raw[j] & mask_first) | (v & ~mask_first);
-        }
+      for (int j = 0; j < 16; ++j) {
+        const int c = cg * 16 + j;
+        uint32_t v = raw[j];
+        if (GRAN == 1) v >>= 8 * (c >= a.C - 1 ? back : 0);
+        raw[j] = (live && c < a.C) ? v ^ a.xor_mask : 0u;
       }
       uint32_t t[4][4];
 #pragma unroll
@@ -221,26 +215,24 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((P
   // ---- where this lane's output groups live (the same for every output tile) -----
   // Copy-out mapping of a staged row of kRowBytes pixels: GRAN 16: lane -> 16-pixel chunk
   // lane % (kRowBytes/16); GRAN 4 and 1: 4-pixel group lane % (kRowBytes/4), which with
-  // GRAN 1 may be unaligned or straddle two images (then stored byte by byte).
+  // GRAN 1 may be unaligned or an image's short last group (then stored byte by byte).
   constexpr int kUnit = GRAN == 16 ? 16 : 4;
   constexpr int kPerRow = kRowBytes / kUnit;
   constexpr int kRowsPerIter = 64 / kPerRow;
   const int px_in_row = (lane % kPerRow) * kUnit;
   const int oq0 = q_base + part * kRowBytes + px_in_row;
   const bool out_live = oq0 < a.Q;
-  const int on = out_live ? static_cast<int>(static_cast<uint32_t>(oq0) / static_cast<uint32_t>(a.HW)) : 0;
-  const int op0 = out_live ? static_cast<int>(oq0 - on * a.HW) : 0;
+  const int on = out_live ? static_cast<int>(static_cast<uint32_t>(oq0) / static_cast<uint32_t>(a.HWp)) : 0;
+  const int op0 = out_live ? static_cast<int>(oq0 - on * a.HWp) : 0;
   const size_t out_off = static_cast<size_t>(on) * a.OC * a.HW + static_cast<size_t>(op0);
-  const bool out_whole = GRAN >= 4 ? out_live : (oq0 + 3 < a.Q && op0 + 3 < a.HW);
+  const bool out_whole = GRAN >= 4 ? out_live : (out_live && op0 + 3 < a.HW);
   size_t out_px_off[4] = {0, 0, 0, 0};
   bool out_px_live[4] = {false, false, false, false};
   if (GRAN == 1 && out_live && !out_whole) {
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const int qe = oq0 + e;
-      out_px_live[e] = qe < a.Q;
-      const int ne = out_px_live[e] ? static_cast<int>(static_cast<uint32_t>(qe) / static_cast<uint32_t>(a.HW)) : 0;
-      out_px_off[e] = static_cast<size_t>(ne) * a.OC * a.HW + static_cast<size_t>(qe - ne * a.HW);
+      out_px_live[e] = op0 + e < a.HW;
+      out_px_off[e] = out_off + e;
     }
   }
 
@@ -476,19 +468,21 @@ int PwConvSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const 
   a.C = d->in_c;
   a.OC = d->out_c;
   const uint64_t hw = static_cast<uint64_t>(d->in_w) * d->in_h;
-  if (hw >= (1ull << 30) || hw < 4) return TVX_E_UNSUPPORTED;  // a 4-pixel group spans at most two images
+  if (hw >= (1ull << 30) || hw * d->in_c * d->batch < 4) return TVX_E_UNSUPPORTED;  // the input is read as dwords
   a.HW = static_cast<int>(hw);
-  if (hw * d->batch >= (1ull << 31) - 256) return TVX_E_UNSUPPORTED;
-  a.Q = static_cast<int>(hw * d->batch);
+  const uint64_t hwp = (hw + 3) / 4 * 4;
+  a.HWp = static_cast<int>(hwp);
+  if (hwp * d->batch >= (1ull << 31) - 256) return TVX_E_UNSUPPORTED;
+  a.Q = static_cast<int>(hwp * d->batch);
   a.cp = RoundUp(a.C, 32);
   a.ksteps = a.cp / 32;
   a.pix_stride = a.cp + 16;
   a.oc_tiles = (a.OC + 31) / 32;
   // few pixels in the whole batch: 32-pixel workgroups, four times as many
   int kp = a.Q < 128 * 1024 ? 32 : 128;
-  // a shallow input (its tile is loaded in one or two passes by a single wavefront): one
+  // a shallow input (a single wavefront loads its tile in one pass, or two of a 128-pixel tile): one
   // wavefront per workgroup, no barrier, many tiles in flight per CU
-  int nw = a.cp / 16 <= (kp == 128 ? 4 : 16) ? 1 : 4;
+  int nw = a.cp / 16 <= (kp == 128 ? 4 : 8) ? 1 : 4;
   if (const char* f = getenv("TVX_PWCONV_SHAPE")) {  // tuning aid: "<pixels per workgroup>,<wavefronts>"
     int fk = 0, fn = 0;
     if (sscanf(f, "%d,%d", &fk, &fn) == 2 && (fk == 32 || fk == 128) && (fn == 1 || fn == 4)) { kp = fk; nw = fn; }
