@@ -50,6 +50,7 @@ struct PwArgs {
   int oc_tiles;          // ceil(OC / 32)
   int tiles_per_wg;      // output tiles one workgroup walks
   int tile_groups;       // workgroups that share a pixel tile (oc_tiles / tiles_per_wg, rounded up)
+  int xcd_runs;          // renumber the workgroups so that each XCD gets a contiguous run of them
   int xor_mask;          // 0x80808080 for uint8 activations
   int neg_zws4;          // -(weight zero point, int8 domain) in all four bytes
   int out_zp, lo, hi;
@@ -116,7 +117,7 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((P
   // segment is a quarter of a cache line and neighbouring pixel tiles take the other quarters;
   // spread over four XCDs, every line would cross the fabric four times.
   int wg = blockIdx.x;
-  {
+  if (a.xcd_runs) {
     const int per = gridDim.x >> 3, rem = gridDim.x & 7, xcd = wg & 7;
     wg = xcd * per + min(xcd, rem) + (wg >> 3);
   }
@@ -527,6 +528,10 @@ int PwConvSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const 
   a.tiles_per_wg = std::min(((quads + gy - 1) / gy) * nw, a.oc_tiles);
   gy = (a.oc_tiles + a.tiles_per_wg - 1) / a.tiles_per_wg;
   a.tile_groups = gy;
+  // pixel tiles that are whole cache lines of every channel row and have a single workgroup each
+  // share nothing: they keep the launch order, which spreads the stream over all memory channels
+  a.xcd_runs = (kp % 128 != 0 || a.HW % 128 != 0 || gy > 1) ? 1 : 0;
+  if (const char* f = getenv("TVX_PWCONV_XCD_RUNS")) a.xcd_runs = atoi(f) != 0;  // tuning aid
   if (gx * gy > 0x7fffffffll) return TVX_E_UNSUPPORTED;
   // fewer output tiles than wavefronts: split the pixels of a tile over wavefronts instead
   const int pt = kp == 32 ? 1 : (nw == 1 ? 4 : (a.tiles_per_wg >= 4 ? 4 : (a.tiles_per_wg >= 2 ? 2 : 1)));
