@@ -142,13 +142,13 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
 
 struct Plan {
   DwArgs a;
-  int stride, pad_l, boxsum, rq, rows_per_thread;
+  int stride, pad_l, boxsum, rq, rows_per_thread, threads;
   dim3 grid;
 };
 
 template <int S, int PL, bool BOXSUM, int RPT>
 void LaunchRq(const Plan* p, const DwArgs& a, hipStream_t st) {
-  const dim3 block(kThreads);
+  const dim3 block(p->threads);
   if (p->rq == kRqFastNoTie) hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqFastNoTie, RPT>), p->grid, block, 0, st, a);
   else if (p->rq == kRqFast) hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqFast, RPT>), p->grid, block, 0, st, a);
   else hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqGeneric, RPT>), p->grid, block, 0, st, a);
@@ -271,11 +271,20 @@ int DwConv3x3Setup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   a.pad_t = d->pad_top; a.pad_l = d->pad_left;
   a.ow4 = ow4;
   a.lpr_shift = lpr_shift;
-  a.rg_per_block = kThreads >> lpr_shift;
   // tall planes at stride 1: eight output rows per thread (a third of the workgroups to dispatch,
   // ten input rows read for eight instead of six for four)
-  const int rpt = S == 1 && d->out_h >= 96 ? 8 : 4;
+  int rpt = S == 1 && d->out_h >= 96 ? 8 : 4;
+  if (const char* f = getenv("TVX_DWCONV_ROWS")) {  // tuning aid: output rows per thread
+    if (atoi(f) == 4 || (atoi(f) == 8 && S == 1)) rpt = atoi(f);
+  }
   const int row_groups = (static_cast<int>(d->out_h) + rpt - 1) / rpt;
+  // a workgroup is as many wavefronts as a plane's row groups fill, four at most: wavefronts
+  // without rows would be dispatched only to leave at once
+  p.threads = std::min(kThreads, ((row_groups << lpr_shift) + 63) / 64 * 64);
+  if (const char* f = getenv("TVX_DWCONV_THREADS")) {  // tuning aid
+    if (atoi(f) == 64 || atoi(f) == 128 || atoi(f) == 192 || atoi(f) == 256) p.threads = std::max(atoi(f), 1 << lpr_shift);
+  }
+  a.rg_per_block = p.threads >> lpr_shift;
   a.xor_mask = x_u8 ? static_cast<int>(0x80808080u) : 0;
   a.pad_fill = static_cast<int>(static_cast<uint32_t>(zxs & 0xff) * 0x01010101u);
   a.zws = zws; a.out_zp = d->out_zp; a.lo = op->act_lo; a.hi = op->act_hi;

@@ -218,8 +218,7 @@ int DwPlanesRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t
 // two or three dwords of each input row behind them, cuts the windows with v_alignbyte,
 // multiplies with v_dot4 against the packed kernel rows and stores its bytes straight to
 // the output tensor (unaligned dword stores are legal on global memory; rows of width 14 or
-// 7 need them). Index arithmetic uses 24-bit multiplies and reciprocals (full-rate
-// instructions; the 32-bit integer multiply issues at a quarter of the rate).
+// 7 need them). Index arithmetic uses 24-bit multiplies and reciprocals, no divisions.
 struct DwrArgs {
   const uint8_t* x;
   uint8_t* y;
