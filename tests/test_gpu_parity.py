@@ -593,7 +593,7 @@ def test_conv2d_im2col(oracle, gi, mode):
     assert 0.02 < np.mean((want > want.min()) & (want < want.max())), "saturated test data"
 
 
-@pytest.mark.parametrize("side,n", [(16, 2), (14, 3), (7, 5), (5, 1)], ids=lambda v: str(v))   # hw % 16 == 0, % 4 == 0, odd
+@pytest.mark.parametrize("side,n", [(16, 2), (14, 3), (7, 5), (5, 1), (3, 2), (1, 6)], ids=lambda v: str(v))   # hw % 16 == 0, % 4 == 0, odd, below 4
 @pytest.mark.parametrize("mode", ["u8", "i8pc"])
 @pytest.mark.parametrize("conv_operand", [1, 2])
 def test_pointwise_conv_with_fused_add(oracle, side, n, mode, conv_operand):
