@@ -148,6 +148,25 @@ def test_pool2d_random(oracle, pi, ptype, dtype):
         assert np.allclose(got.astype(np.float32), want.astype(np.float32), rtol=FLOAT_RTOL, atol=1e-3)
 
 
+@pytest.mark.parametrize("shape", [(7, 7, 1280, 3), (2, 2, 5, 1), (5, 3, 9, 2), (17, 19, 6, 2), (33, 31, 3, 1)], ids=str)
+@pytest.mark.parametrize("ptype", [1, 3])
+@pytest.mark.parametrize("dtype", [0, 1])
+def test_global_average_pool(oracle, shape, ptype, dtype):
+    """Quantized average over the whole plane: its own kernel (4, 16 or 64 lanes per plane, planes that do
+    not end on a dword), the oracle's arithmetic."""
+    w, h, c, n = shape
+    rng = np.random.default_rng(w * 100 + h + dtype)
+    x = rand_q(rng, w * h * c * n, dtype)
+    kws = dict(in_shape=list(shape), out_shape=[1, 1, c, n], ksize=[w, h], stride=[1, 1], pad_left=0, pad_top=0,
+               pool_type=ptype, dtype=dtype)
+    zp = 7 if dtype else 120  # near the mean of the data, so that the finer output scale does not saturate
+    for in_q, out_q in (((0.1, zp), (0.1, zp)), ((0.1, zp), (0.013, -2 if dtype else 9))):
+        want = oracle.pool2d(x, in_q=in_q, out_q=out_q, **kws)
+        got = TC.gpu_pool2d(x, in_q=in_q, out_q=out_q, want_kernel="avgpool_plane_i8", **kws)
+        assert np.array_equal(got, want)
+        assert out_q[0] != in_q[0] or len(np.unique(want)) > 2
+
+
 @pytest.mark.parametrize("dtype", [0, 1])
 def test_eltwise_quantized(oracle, dtype):
     rng = np.random.default_rng(dtype)

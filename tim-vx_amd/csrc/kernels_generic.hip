@@ -378,6 +378,56 @@ PoolFloatKernel(PoolArgs a, const T* __restrict__ x, T* __restrict__ y, uint64_t
   FromFloat(r, &y[idx]);
 }
 
+// Quantized average over a whole plane (global average pooling): L lanes share a plane, read it
+// as dwords (the last one ending with the plane), sum the bytes with dot4 against ones and add
+// up across the lanes; the result is formed exactly as in the kernel above.
+template <typename T, int L>
+__global__ void __launch_bounds__(kBlock)
+PoolPlaneAvgKernel(PoolArgs a, const T* __restrict__ x, T* __restrict__ y, uint64_t planes) {
+  const uint64_t plane = (static_cast<uint64_t>(blockIdx.x) * kBlock + threadIdx.x) / L;
+  const int lane = threadIdx.x % L;
+  const int hw = a.in_w * a.in_h;
+  const int n_dw = plane < planes ? (hw + 3) / 4 : 0;  // lanes past the last plane stay for the shuffles
+  const uint8_t* xp = reinterpret_cast<const uint8_t*>(x) + plane * hw;
+  int sum = 0;
+  for (int i = lane; i < n_dw; i += L) {
+    const int at = min(4 * i, hw - 4);
+    uint32_t v;
+    __builtin_memcpy(&v, xp + at, 4);
+    v >>= 8 * (4 * i - at);  // the bytes in front of a short last dword were counted already
+    if constexpr (std::is_signed<T>::value) sum = __builtin_amdgcn_sdot4(static_cast<int>(v), 0x01010101, sum, false);
+    else sum = static_cast<int>(__builtin_amdgcn_udot4(v, 0x01010101u, static_cast<uint32_t>(sum), false));
+  }
+#pragma unroll
+  for (int o = L / 2; o; o >>= 1) sum += __shfl_xor(sum, o, 64);
+  if (lane != 0 || plane >= planes) return;
+  const int64_t total = static_cast<int64_t>(sum) - static_cast<int64_t>(hw) * a.in_zp;
+  int64_t r = static_cast<int64_t>(rint(static_cast<double>(total) * a.ratio / static_cast<double>(hw)));
+  r += a.out_zp;
+  r = r < a.qmin ? a.qmin : (r > a.qmax ? a.qmax : r);
+  y[plane] = static_cast<T>(r);
+}
+
+template <typename T>
+static void LaunchPoolPlaneAvg(const PoolArgs& a, const void* in0, void* out, uint64_t planes, hipStream_t st) {
+  const int n_dw = (a.in_w * a.in_h + 3) / 4;
+  const T* x = static_cast<const T*>(in0);
+  T* y = static_cast<T*>(out);
+  const dim3 block(kBlock);
+  if (n_dw <= 4) hipLaunchKernelGGL((PoolPlaneAvgKernel<T, 4>), dim3(Blocks(planes * 4)), block, 0, st, a, x, y, planes);
+  else if (n_dw <= 16) hipLaunchKernelGGL((PoolPlaneAvgKernel<T, 16>), dim3(Blocks(planes * 16)), block, 0, st, a, x, y, planes);
+  else hipLaunchKernelGGL((PoolPlaneAvgKernel<T, 64>), dim3(Blocks(planes * 64)), block, 0, st, a, x, y, planes);
+}
+
+// does the window of a quantized average pooling cover exactly the whole, unpadded plane?
+static bool IsPlaneAverage(const tvx_op* op) {
+  const tvx_pool2d_desc& d = op->pool;
+  const uint64_t hw = static_cast<uint64_t>(d.in_w) * d.in_h;
+  return op->quantized && (d.pool_type == TVX_POOL_AVG || d.pool_type == TVX_POOL_AVG_ANDROID) &&
+         d.k_w == d.in_w && d.k_h == d.in_h && d.pad_left == 0 && d.pad_top == 0 && d.out_w == 1 && d.out_h == 1 &&
+         hw >= 4 && hw <= (1u << 22);  // the byte sum of a plane stays below 2^31
+}
+
 int PoolGenericRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
   const tvx_pool2d_desc& d = op->pool;
   PoolArgs a{static_cast<int>(d.in_w), static_cast<int>(d.in_h), static_cast<int>(d.out_w),
@@ -388,6 +438,12 @@ int PoolGenericRun(tvx_op* op, const void* in0, const void*, void* out, hipStrea
              op->geo[0], op->geo[1],
              op->quantized ? static_cast<double>(d.in_scale) / static_cast<double>(d.out_scale) : 1.0};
   const uint64_t total = static_cast<uint64_t>(d.out_w) * d.out_h * d.channels * d.batch;
+  if (IsPlaneAverage(op)) {
+    if (d.dtype == TVX_U8) LaunchPoolPlaneAvg<uint8_t>(a, in0, out, total, st);
+    else LaunchPoolPlaneAvg<int8_t>(a, in0, out, total, st);
+    TVX_HIP_CHECK(hipGetLastError());
+    return TVX_OK;
+  }
   const dim3 grid(Blocks(total)), block(kBlock);
   switch (d.dtype) {
     case TVX_U8:
@@ -863,7 +919,7 @@ int PoolGenericSetup(tvx_op* op) {
     if (s != TVX_OK) return s;
   }
   op->run = PoolGenericRun;
-  op->kernel_name = "pool2d_generic";
+  op->kernel_name = IsPlaneAverage(op) ? "avgpool_plane_i8" : "pool2d_generic";
   return TVX_OK;
 }
 
