@@ -597,6 +597,8 @@ IM2COL_GRID = [
     dict(n=1, c=7, h=20, w=20, oc=100, kh=3, kw=3, stride=[1, 1], dil=[2, 2], pad=[2, 2, 2, 2], mult=0),  # K = 63, dilated, 4 channel tiles
     dict(n=5, c=2, h=9, w=7, oc=5, kh=1, kw=3, stride=[1, 1], dil=[1, 1], pad=[1, 1, 0, 0], mult=0),      # tiny, hw % 4 != 0
     dict(n=2, c=3, h=64, w=64, oc=64, kh=3, kw=3, stride=[1, 1], dil=[1, 1], pad=[1, 1, 1, 1], mult=0),   # several workgroups per image
+    dict(n=1, c=5, h=10, w=6, oc=40, kh=2, kw=3, stride=[1, 1], dil=[1, 3], pad=[2, 2, 1, 1], mult=0),    # rows as dwords that begin two bytes in front of the tensor / end behind it
+    dict(n=1, c=1, h=1, w=4, oc=3, kh=1, kw=3, stride=[1, 1], dil=[1, 1], pad=[2, 2, 0, 0], mult=0),      # a four-byte tensor
 ]
 
 

@@ -44,11 +44,16 @@ struct ImArgs {
   // c * H * W + dy * W + dx. They travel in the kernel arguments so that the (wavefront-uniform) reads
   // are scalar loads of memory nothing can write; a table in global memory is read per lane, one round
   // trip a tap.
+  // In row mode (kernels three taps wide, unit dilation along the row) entry r stands for a whole
+  // kernel row of a channel: dy | 1 << 16 and c * H * W + dy * W; the three taps are one dword load.
   int taps[64];
   int offs[64];
+  int rows;              // row mode: C * Kh
+  int total_bytes;       // row mode: size of the input tensor (< 2^31)
 };
 
-template <int OT, int RQ>
+// KW: 0 = any window, one byte load per tap; 3 = row mode
+template <int OT, int RQ, int KW>
 __global__ void __launch_bounds__(kThreads) ConvIm2colKernel(ImArgs a) {
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -95,6 +100,62 @@ __global__ void __launch_bounds__(kThreads) ConvIm2colKernel(ImArgs a) {
       return n <= 0 ? 0u : ((n >= 32 ? 0xffffffffu : ((1u << n) - 1u)) << lo);
     };
     const uint32_t row_ok = span_mask(ih0, a.H), col_ok = span_mask(iw0, a.W);
+    if constexpr (KW == 3) {
+      // Row mode: byte loads cost the L1 a tag lookup for every few lanes, and those lookups bound the
+      // gather; the three taps of a kernel row are adjacent bytes, so one (unaligned) dword fetches
+      // them. The dword may begin in front of the tensor (left padding of its first row) or end behind
+      // it: it is moved inside by up to three bytes and shifted back. A row with no tap inside the
+      // image reads the tensor's first dword and is not used.
+      constexpr int kMaxRows = 64 / 3;
+      const int img_at = n * (a.C * a.H * a.W) + origin;
+      auto place = [&](int r, bool* row_in, int* moved) {  // -> byte index of the row's dword in the tensor
+        const int t = a.taps[r];
+        *row_in = ((row_ok >> (t & 0xff)) & static_cast<uint32_t>(t >> 16) & 1u) != 0;
+        const bool any = *row_in & ((col_ok & 7u) != 0);
+        const int want = any ? img_at + a.offs[r] : 0;
+        const int at = min(max(want, 0), a.total_bytes - 4);
+        *moved = at - want;  // -3 .. 3
+        return at;
+      };
+      uint32_t v[kMaxRows];
+#pragma unroll
+      for (int r = 0; r < kMaxRows; ++r) {
+        v[r] = 0;
+        if (r < a.rows) {  // uniform
+          bool row_in;
+          int moved;
+          const int at = place(r, &row_in, &moved);
+          __builtin_memcpy(&v[r], a.x + static_cast<uint32_t>(at), 4);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);  // all loads travel together
+      int dw[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) dw[i] = 0;
+#pragma unroll
+      for (int r = 0; r < kMaxRows; ++r) {
+        if (r < a.rows) {
+          bool row_in;
+          int moved;
+          (void)place(r, &row_in, &moved);
+          const uint32_t got = moved >= 0 ? v[r] << (8 * moved) : v[r] >> (-8 * moved);
+#pragma unroll
+          for (int e = 0; e < 3; ++e) {
+            const bool inside = row_in & (((col_ok >> e) & 1u) != 0);
+            const int byte = inside ? static_cast<int>(((got >> (8 * e)) & 0xffu) ^ static_cast<uint32_t>(a.xor_mask)) : a.pad_fill;
+            const int k = r * 3 + e;
+            dw[k >> 2] |= byte << (8 * (k & 3));
+          }
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i) sx = __builtin_amdgcn_sdot4(dw[i], 0x01010101, sx, false);
+      for (int k0 = 0; k0 < a.kp; k0 += 16) {
+        const int i = k0 >> 2;
+        const v4i out = i == 0 ? v4i{dw[0], dw[1], dw[2], dw[3]} : (i == 4 ? v4i{dw[4], dw[5], dw[6], dw[7]} : (i == 8 ? v4i{dw[8], dw[9], dw[10], dw[11]} : v4i{dw[12], dw[13], dw[14], dw[15]}));
+        *reinterpret_cast<v4i*>(a_lds + tid * a.row_stride + k0) = out;
+      }
+    } else
     for (int k0 = 0; k0 < a.kp; k0 += 16) {
       int b[16];
       bool inside[16];
@@ -194,19 +255,26 @@ __global__ void __launch_bounds__(kThreads) ConvIm2colKernel(ImArgs a) {
 struct Plan {
   ImArgs a;
   int lds_bytes;
-  int ot, rq;
+  int ot, rq, row_mode;
   dim3 grid;
 };
 
-template <int OT>
+template <int OT, int KW>
 void LaunchRq(const Plan* plan, const ImArgs& a, hipStream_t st) {
   const dim3 block(kThreads);
   if (plan->rq == kRqFastNoTie)
-    hipLaunchKernelGGL((ConvIm2colKernel<OT, kRqFastNoTie>), plan->grid, block, plan->lds_bytes, st, a);
+    hipLaunchKernelGGL((ConvIm2colKernel<OT, kRqFastNoTie, KW>), plan->grid, block, plan->lds_bytes, st, a);
   else if (plan->rq == kRqFast)
-    hipLaunchKernelGGL((ConvIm2colKernel<OT, kRqFast>), plan->grid, block, plan->lds_bytes, st, a);
+    hipLaunchKernelGGL((ConvIm2colKernel<OT, kRqFast, KW>), plan->grid, block, plan->lds_bytes, st, a);
   else
-    hipLaunchKernelGGL((ConvIm2colKernel<OT, kRqGeneric>), plan->grid, block, plan->lds_bytes, st, a);
+    hipLaunchKernelGGL((ConvIm2colKernel<OT, kRqGeneric, KW>), plan->grid, block, plan->lds_bytes, st, a);
+}
+
+template <int KW>
+void LaunchOt(const Plan* plan, const ImArgs& a, hipStream_t st) {
+  if (plan->ot == 1) LaunchRq<1, KW>(plan, a, st);
+  else if (plan->ot == 2) LaunchRq<2, KW>(plan, a, st);
+  else LaunchRq<4, KW>(plan, a, st);
 }
 
 int ConvIm2colRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
@@ -214,9 +282,8 @@ int ConvIm2colRun(tvx_op* op, const void* in0, const void*, void* out, hipStream
   ImArgs a = plan->a;
   a.x = static_cast<const uint8_t*>(in0);
   a.y = static_cast<uint8_t*>(out);
-  if (plan->ot == 1) LaunchRq<1>(plan, a, st);
-  else if (plan->ot == 2) LaunchRq<2>(plan, a, st);
-  else LaunchRq<4>(plan, a, st);
+  if (plan->row_mode) LaunchOt<3>(plan, a, st);
+  else LaunchOt<0>(plan, a, st);
   TVX_HIP_CHECK(hipGetLastError());
   return TVX_OK;
 }
@@ -278,12 +345,26 @@ int ConvIm2colSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, co
   const int rq = BuildRequantRecords(op->h_mult, op->h_shift, a.OC, a.oct, d->out_zp, &rqt,
                                      AccumulatorBound(static_cast<uint64_t>(K), bias_host, a.OC));
   if ((d->k_h - 1) * d->dilation_h > 31 || (d->k_w - 1) * d->dilation_w > 31) return TVX_E_UNSUPPORTED;  // window offsets index 32-bit masks
-  for (int k = 0; k < K; ++k) {
-    const int c = k / taps, t = k % taps;
-    const int dy = (t / static_cast<int>(d->k_w)) * static_cast<int>(d->dilation_h);
-    const int dx = (t % static_cast<int>(d->k_w)) * static_cast<int>(d->dilation_w);
-    a.taps[k] = dy | dx << 8 | 1 << 16;
-    a.offs[k] = c * a.H * a.W + dy * a.W + dx;
+  const uint64_t total_bytes = static_cast<uint64_t>(d->batch) * d->in_c * d->in_h * d->in_w;
+  bool row_mode = d->k_w == 3 && d->dilation_w == 1 && total_bytes >= 4 && total_bytes < (1ull << 31);
+  if (const char* f = getenv("TVX_IM2COL_ROWS")) row_mode = row_mode && atoi(f) != 0;  // tuning aid
+  if (row_mode) {
+    a.rows = static_cast<int>(d->in_c * d->k_h);
+    a.total_bytes = static_cast<int>(total_bytes);
+    for (int r = 0; r < a.rows; ++r) {
+      const int c = r / static_cast<int>(d->k_h);
+      const int dy = (r % static_cast<int>(d->k_h)) * static_cast<int>(d->dilation_h);
+      a.taps[r] = dy | 1 << 16;
+      a.offs[r] = c * a.H * a.W + dy * a.W;
+    }
+  } else {
+    for (int k = 0; k < K; ++k) {
+      const int c = k / taps, t = k % taps;
+      const int dy = (t / static_cast<int>(d->k_w)) * static_cast<int>(d->dilation_h);
+      const int dx = (t % static_cast<int>(d->k_w)) * static_cast<int>(d->dilation_w);
+      a.taps[k] = dy | dx << 8 | 1 << 16;
+      a.offs[k] = c * a.H * a.W + dy * a.W + dx;
+    }
   }
   int s = op->packed.Upload(packed.data(), packed.size());
   if (s == TVX_OK) s = op->aux.Upload(biasf.data(), biasf.size() * 4);
@@ -298,6 +379,7 @@ int ConvIm2colSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, co
   plan.lds_bytes = lds_bytes;
   plan.ot = ot;
   plan.rq = rq;
+  plan.row_mode = row_mode ? 1 : 0;
   const int hw = a.OH * a.OW;
   plan.grid = dim3(static_cast<unsigned>((hw + kPixels - 1) / kPixels), static_cast<unsigned>(d->batch));
   op->host_blob.assign(reinterpret_cast<const uint8_t*>(&plan), reinterpret_cast<const uint8_t*>(&plan) + sizeof(plan));
