@@ -140,7 +140,7 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((P
   // are requested before the previous tile's epilogue (for the first tile: before the input
   // tile is built), so their latency hides behind work that does not need them.
   auto frag_ptr = [&](int t, int k) { return a.wpk + (static_cast<size_t>(t) * a.ksteps + k) * 64 + lane; };
-  constexpr int kRing = PT == 4 ? 2 : 4;  // fragments in flight; four pixel tiles leave room for two
+  constexpr int kRing = PT == 4 ? 2 : ((KP == 32 && NW == 4) ? 8 : 4);  // fragments in flight; four pixel tiles leave room for two, deep inputs (the 32-pixel, four-wavefront shape) take eight
   v4i nf[kRing];
 #pragma unroll
   for (int j = 0; j < kRing; ++j) nf[j] = *frag_ptr(n_tiles > 0 ? tile0 : 0, min(j, a.ksteps - 1));
