@@ -13,7 +13,7 @@
 //     private LDS patch and writes them itself - no workgroup barrier after the
 //     input tile is built, and every global store is a complete cache line;
 //   * weights are pre-packed in MFMA fragment order and stream global -> registers
-//     (1 KiB contiguous per wavefront load, prefetched up to four steps ahead, the
+//     (1 KiB contiguous per wavefront load, prefetched up to four (deep inputs: eight) steps ahead, the
 //     first ones of a tile during the previous tile's epilogue); they are small and live in L2.
 // Zero points: sum (x - zx)(w - zw) = sum xs ws - zws Sx - zxs Sw + C zxs zws with
 // xs, ws the operands moved to the signed int8 domain; the Sx term is one more MFMA
