@@ -155,21 +155,129 @@ def test_fc_restatement_vs_numpy(oracle):
     assert np.array_equal(got.astype(np.int64), want.ravel())
 
 
+def _f32(v):
+    """The exact rational value of a float32 number (scales travel as float32)."""
+    return Fraction(float(np.float32(v)))
+
+
+def _closed_form_activation(q, act, qmin, qmax, s_in, z_in, s_out, z_out, oracle):
+    """Textbook definition, exact: dequantize, clamp to [0, inf) or [0, 6] in the real domain, divide by the
+    output scale, round half to even, add the zero point, saturate. The only thing taken from the oracle is the
+    Q31 image of s_in / s_out (pinned on its own above): the real value is (q - z_in) * mult * 2^-shift output
+    quanta, six real units are 6 / s_out of them."""
+    mult, shift = oracle.quantize_multiplier(float(np.float32(s_in)) / float(np.float32(s_out)))
+    v = Fraction((int(q) - z_in) * mult, 2 ** shift)
+    if act in ("RELU", "RELU6"):
+        v = max(v, Fraction(0))
+    if act == "RELU6":
+        v = min(v, Fraction(6) / _f32(s_out))
+    return min(qmax, max(qmin, rne_fraction(v) + z_out))
+
+
+@pytest.mark.parametrize("dtype_name,z_in,z_out", [("U8", 117, 9), ("U8", 3, 131), ("I8", -11, -100), ("I8", 20, 5)])
+@pytest.mark.parametrize("s_in,s_out", [(0.07, 0.07), (0.05, 0.023), (0.023, 0.07), (0.11, 0.047), (0.5, 0.25),
+                                         (0.25, 0.5), (3.0, 4.0)])
+@pytest.mark.parametrize("act", ["RELU", "RELU6"])
+def test_activation_restatement_vs_closed_form(oracle, dtype_name, z_in, z_out, s_in, s_out, act):
+    # 6 / 0.07 = 85.71, 6 / 0.023 = 260.87, 6 / 0.047 = 127.66, 6 / 4 = 1.5 (a tie: half-even gives 2):
+    # floor instead of round-to-nearest, a bound at zero instead of the zero point, or clamping the rounded
+    # value to the wrong side of the requantization all change codes here. 0.25 -> 0.5 and 3 -> 4 put odd
+    # inputs on exact .5 ties.
+    u8 = dtype_name == "U8"
+    dt = oracle.U8 if u8 else oracle.I8
+    qmin, qmax = (0, 255) if u8 else (-128, 127)
+    q = np.arange(qmin, qmax + 1).astype(np.uint8 if u8 else np.int8)
+    got = oracle.activation(oracle.ACT_RELU if act == "RELU" else oracle.ACT_RELU6, dt, q,
+                            (s_in, z_in), (s_out, z_out))
+    want = [_closed_form_activation(v, act, qmin, qmax, s_in, z_in, s_out, z_out, oracle) for v in q]
+    assert got.astype(np.int64).tolist() == want
+    assert len(set(want)) > 2  # the case is not saturated flat
+
+
+def test_activation_ties_and_bounds_by_hand(oracle):
+    # s_in 0.25 -> s_out 0.5, zero points 10 -> 3: real = (q - 10) / 4, quanta = (q - 10) / 2
+    q = np.array([10, 11, 12, 13, 15, 9, 0, 34, 35, 36, 255], dtype=np.uint8)
+    # quanta:      0  .5   1  1.5 2.5 -.5 -5  12 12.5 13  122.5 ; six real units = 12 quanta
+    relu = oracle.activation(oracle.ACT_RELU, oracle.U8, q, (0.25, 10), (0.5, 3))
+    assert relu.tolist() == [3, 3, 4, 5, 5, 3, 3, 15, 15, 16, 125]      # .5 -> 0, 1.5 -> 2, 2.5 -> 2, 12.5 -> 12, 122.5 -> 122
+    relu6 = oracle.activation(oracle.ACT_RELU6, oracle.U8, q, (0.25, 10), (0.5, 3))
+    assert relu6.tolist() == [3, 3, 4, 5, 5, 3, 3, 15, 15, 15, 15]
+    # int8, negative zero point, upper bound beyond the type: 6 / 0.02 = 300 quanta -> saturates at 127
+    qi = np.array([-128, -101, -100, -99, 0, 127], dtype=np.int8)
+    r6 = oracle.activation(oracle.ACT_RELU6, oracle.I8, qi, (0.02, -100), (0.02, -100))
+    assert r6.tolist() == [-100, -100, -100, -99, 0, 127]
+    # upper bound inside the type with a non-integer quotient: 6 / 0.07 = 85.71 -> 86 quanta above the zero point
+    r6 = oracle.activation(oracle.ACT_RELU6, oracle.I8, qi, (0.07, -100), (0.07, -100))
+    assert r6.tolist() == [-100, -100, -100, -99, -14, -14]
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_fused_activation_on_conv_vs_closed_form(oracle, seed):
+    # the fused epilogue, output zero point != 0, checked through brute-force accumulators and exact rationals
+    rng = np.random.default_rng(500 + seed)
+    u8 = seed % 2 == 0
+    n, c, h, wd, oc = 1, 5, 6, 7, 4
+    qmin, qmax = (0, 255) if u8 else (-128, 127)
+    npdt = np.uint8 if u8 else np.int8
+    x = rng.integers(qmin, qmax + 1, (n, c, h, wd)).astype(npdt)
+    w = rng.integers(qmin, qmax + 1, (oc, c, 3, 3)).astype(npdt)
+    bias = rng.integers(-4096, 4097, oc).astype(np.int32)
+    zx, zw, zo = (128, 120, 17) if u8 else (-5, 0, -90)
+    s_in, s_w, s_out = 0.05, 0.01, [0.07, 0.023, 0.047, 0.11][seed]
+    acc = brute_conv(x.astype(np.int64) - zx, w.astype(np.int64) - zw, bias.astype(np.int64),
+                     [1, 1], [1, 1], 1, 1, wd, h, 0)
+    mult, shift = oracle.quantize_multiplier(float(np.float32(s_in)) * float(np.float32(s_w)) / float(np.float32(s_out)))
+    for act_name, act in (("RELU", oracle.ACT_RELU), ("RELU6", oracle.ACT_RELU6)):
+        want = []
+        for a in acc.ravel():
+            v = max(Fraction(int(a) * mult, 2 ** shift), Fraction(0))
+            if act_name == "RELU6":
+                v = min(v, Fraction(6) / _f32(s_out))
+            want.append(min(qmax, max(qmin, rne_fraction(v) + zo)))
+        dt = oracle.U8 if u8 else oracle.I8
+        got = oracle.conv2d(x.ravel(), w.ravel(), bias, in_shape=[wd, h, c, n], w_shape=[3, 3, c, oc],
+                            out_shape=[wd, h, oc, n], stride=[1, 1], dilation=[1, 1], pad_left=1, pad_top=1,
+                            multiplier=0, in_dtype=dt, w_dtype=dt, out_dtype=dt, in_q=(s_in, zx),
+                            w_q=(s_w, zw, None), out_q=(s_out, zo), act=act)
+        assert got.astype(np.int64).tolist() == want
+        assert min(want) == max(qmin, zo) and len(set(want)) > 3   # both the lower bound and the interior occur
+    # and the same on FullyConnected (int8 per-channel)
+    if not u8:
+        m, k, nn = 5, 19, 6
+        xf = rng.integers(-128, 128, (m, k)).astype(np.int8)
+        wf = rng.integers(-128, 128, (nn, k)).astype(np.int8)
+        bf = rng.integers(-3000, 3000, nn).astype(np.int32)
+        ws = np.exp(rng.uniform(np.log(0.001), np.log(0.02), nn)).astype(np.float32)
+        accf = (xf.astype(np.int64) - 4) @ wf.astype(np.int64).T + bf
+        got = oracle.fully_connected(xf.ravel(), wf.ravel(), bf, m=m, k=k, n=nn, in_dtype=oracle.I8, w_dtype=oracle.I8,
+                                     out_dtype=oracle.I8, in_q=(0.02, 4), w_q=(1.0, 0, ws), out_q=(0.047, -90),
+                                     act=oracle.ACT_RELU6)
+        want = np.zeros((m, nn), dtype=np.int64)
+        for j in range(nn):
+            mu, sh = oracle.quantize_multiplier(float(np.float32(0.02)) * float(ws[j]) / float(np.float32(0.047)))
+            for i in range(m):
+                v = min(max(Fraction(int(accf[i, j]) * mu, 2 ** sh), Fraction(0)), Fraction(6) / _f32(0.047))
+                want[i, j] = min(127, max(-128, rne_fraction(v) - 90))
+        assert np.array_equal(got.astype(np.int64), want.ravel())
+
+
 def test_fused_relu6_equals_conv_then_relu6_when_quant_is_shared(oracle):
+    # consistency of the two forms (each is pinned by closed form above): fusing is legal when the tensor
+    # between the operators and the output share their quantization
     rng = np.random.default_rng(13)
     n, c, h, wd, oc = 1, 8, 6, 6, 4
     x = rng.integers(0, 256, (n, c, h, wd)).astype(np.uint8)
     w = rng.integers(0, 256, (oc, c, 3, 3)).astype(np.uint8)
     bias = rng.integers(-4096, 4097, oc).astype(np.int32)
-    kw = dict(in_shape=[wd, h, c, n], w_shape=[3, 3, c, oc], out_shape=[wd, h, oc, n], stride=[1, 1],
-              dilation=[1, 1], pad_left=1, pad_top=1, multiplier=0, in_dtype=oracle.U8,
-              w_dtype=oracle.U8, out_dtype=oracle.U8, in_q=(0.05, 128), w_q=(0.01, 120, None),
-              out_q=(0.1, 0))
-    fused = oracle.conv2d(x.ravel(), w.ravel(), bias, act=oracle.ACT_RELU6, **kw)
-    plain = oracle.conv2d(x.ravel(), w.ravel(), bias, **kw)
-    two_step = oracle.activation(oracle.ACT_RELU6, oracle.U8, plain, (0.1, 0), (0.1, 0))
-    assert np.array_equal(fused, two_step)
-    assert fused.max() <= 60
+    for out_q in ((0.1, 0), (0.07, 23)):
+        kw = dict(in_shape=[wd, h, c, n], w_shape=[3, 3, c, oc], out_shape=[wd, h, oc, n], stride=[1, 1],
+                  dilation=[1, 1], pad_left=1, pad_top=1, multiplier=0, in_dtype=oracle.U8,
+                  w_dtype=oracle.U8, out_dtype=oracle.U8, in_q=(0.05, 128), w_q=(0.01, 120, None),
+                  out_q=out_q)
+        fused = oracle.conv2d(x.ravel(), w.ravel(), bias, act=oracle.ACT_RELU6, **kw)
+        plain = oracle.conv2d(x.ravel(), w.ravel(), bias, **kw)
+        two_step = oracle.activation(oracle.ACT_RELU6, oracle.U8, plain, out_q, out_q)
+        assert np.array_equal(fused, two_step)
 
 
 def test_pool_avg_divisors(oracle):
@@ -183,14 +291,75 @@ def test_pool_avg_divisors(oracle):
     assert np.allclose(android, [(1 + 2 + 4 + 5) / 4, (3 + 6) / 2, (7 + 8) / 2, 9])
 
 
-def test_quantized_add_and_softmax(oracle):
+def _pool_windows(xr, k, stride, pad, out_wh):
+    """In-bounds taps of every window of one plane xr[H][W] (plain Python)."""
+    H, W = xr.shape
+    for oh in range(out_wh[1]):
+        for ow in range(out_wh[0]):
+            taps = [int(xr[ih, iw])
+                    for ih in range(oh * stride[1] - pad[1], oh * stride[1] - pad[1] + k[1]) if 0 <= ih < H
+                    for iw in range(ow * stride[0] - pad[0], ow * stride[0] - pad[0] + k[0]) if 0 <= iw < W]
+            yield taps
+
+
+@pytest.mark.parametrize("dtype_name", ["U8", "I8"])
+@pytest.mark.parametrize("s_in,s_out", [(0.05, 0.05), (0.05, 0.023), (0.07, 0.11), (0.5, 0.25), (0.25, 0.5), (1.0, 1.0)])
+@pytest.mark.parametrize("pool", ["MAX", "AVG", "AVG_ANDROID"])
+def test_quantized_pool_requantization_is_exact(oracle, dtype_name, s_in, s_out, pool):
+    # in != out quantization, padded 3x3 stride-2 windows on 7x6 planes. MAX: the largest code, dequantized and
+    # requantized by the Q31 rule; averages: exact rational mean of (x - z_in) * s_in / s_out, half to even.
+    # (1.0 -> 1.0 and 0.25 -> 0.5 land sums on exact .5 ties.)
+    rng = np.random.default_rng(40 + 3 * (dtype_name == "U8") + ["MAX", "AVG", "AVG_ANDROID"].index(pool))
+    u8 = dtype_name == "U8"
+    qmin, qmax = (0, 255) if u8 else (-128, 127)
+    z_in, z_out = (101, 7) if u8 else (-9, 12)
+    W, H, C, N = 7, 6, 3, 2
+    k, stride, pad = [3, 3], [2, 2], [1, 1]
+    ow, oh = (W + 2 * pad[0] - k[0]) // stride[0] + 1, (H + 2 * pad[1] - k[1]) // stride[1] + 1
+    x = rng.integers(qmin, qmax + 1, (N * C, H, W)).astype(np.uint8 if u8 else np.int8)
+    got = oracle.pool2d(x.ravel(), in_shape=[W, H, C, N], out_shape=[ow, oh, C, N], ksize=k, stride=stride,
+                        pad_left=pad[0], pad_top=pad[1], pool_type=oracle.POOL[pool],
+                        dtype=oracle.U8 if u8 else oracle.I8, in_q=(s_in, z_in), out_q=(s_out, z_out))
+    ratio = _f32(s_in) / _f32(s_out)
+    mult, shift = oracle.quantize_multiplier(float(np.float32(s_in)) / float(np.float32(s_out)))
+    want, ties = [], 0
+    for p in range(N * C):
+        for taps in _pool_windows(x[p], k, stride, pad, (ow, oh)):
+            if pool == "MAX":
+                v = Fraction((max(taps) - z_in) * mult, 2 ** shift)
+            else:
+                div = k[0] * k[1] if pool == "AVG" else len(taps)
+                v = Fraction(sum(t - z_in for t in taps)) * ratio / div
+            ties += (v - (v.numerator // v.denominator)) == Fraction(1, 2)
+            want.append(min(qmax, max(qmin, rne_fraction(v) + z_out)))
+    assert got.astype(np.int64).tolist() == want
+    if pool == "AVG_ANDROID" and s_in == s_out:
+        assert ties > 0   # window sums over 4 / 6 taps hit .5 often: the tie rule is exercised
+
+
+def test_quantized_add_is_exact(oracle):
+    # exact rational value of (a - za) * sa / so + (b - zb) * sb / so with the float32 scales, half to even
     rng = np.random.default_rng(17)
-    a = rng.integers(0, 256, 1000).astype(np.uint8)
-    b = rng.integers(0, 256, 1000).astype(np.uint8)
-    got = oracle.add(oracle.U8, a, (0.03, 120), b, (0.05, 110), (0.07, 128))
-    real = (a.astype(np.float64) - 120) * 0.03 + (b.astype(np.float64) - 110) * 0.05
-    want = np.clip(np.rint(real / 0.07) + 128, 0, 255)
-    assert np.max(np.abs(got.astype(np.float64) - want)) <= 1  # float32 scales vs exact decimals
+    for dt_name, sa, za, sb, zb, so, zo in (("U8", 0.03, 120, 0.05, 110, 0.07, 128), ("I8", 0.011, -3, 0.2, 7, 0.09, -20),
+                                            ("U8", 0.5, 3, 0.25, 200, 1.0, 100), ("I8", 0.25, 1, 0.25, 0, 0.5, 0)):
+        u8 = dt_name == "U8"
+        qmin, qmax = (0, 255) if u8 else (-128, 127)
+        a = rng.integers(qmin, qmax + 1, 1500).astype(np.uint8 if u8 else np.int8)
+        b = rng.integers(qmin, qmax + 1, 1500).astype(np.uint8 if u8 else np.int8)
+        got = oracle.add(oracle.U8 if u8 else oracle.I8, a, (sa, za), b, (sb, zb), (so, zo))
+        ra, rb = _f32(sa) / _f32(so), _f32(sb) / _f32(so)
+        want, ties = [], 0
+        for p, q in zip(a.tolist(), b.tolist()):
+            v = (p - za) * ra + (q - zb) * rb
+            ties += (v - (v.numerator // v.denominator)) == Fraction(1, 2)
+            want.append(min(qmax, max(qmin, rne_fraction(v) + zo)))
+        assert got.astype(np.int64).tolist() == want
+        if so in (1.0, 0.5):
+            assert ties > 100  # power-of-two ratios: a quarter or half of the sums sit on .5
+
+
+def test_quantized_softmax(oracle):
+    rng = np.random.default_rng(17)
     x = rng.integers(0, 256, 40).astype(np.uint8)
     sm = oracle.softmax(oracle.U8, x, 10, 1.0, (0.1, 128))
     ref = np.exp((x.reshape(4, 10).astype(np.float64) - 128) * np.float32(0.1))
