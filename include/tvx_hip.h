@@ -265,17 +265,6 @@ int tvx_op_run3(tvx_op* op, const void* in0, const void* in1, const void* in2, v
 const char* tvx_op_kernel_name(const tvx_op* op);
 void tvx_op_destroy(tvx_op* op);
 
-/* ---- calibration (measurement aids; no counterpart in the reference) ------------ */
-/* Sustained rate of v_mfma_i32_32x32x32_i8 issued from registers on every CU, in
- * TOPS (2 ops per multiply-accumulate), over `launches` timed launches on the null
- * stream. random_operands = 0 multiplies zeros (the nominal clock), != 0 random bytes
- * (the clock the chip holds under the multipliers' switching power): the second
- * figure is what a real int8 GEMM on this device can approach. */
-int tvx_calibrate_mfma_i8(int random_operands, int launches, double* tops);
-/* Read + write bytes per second (GB/s, 1e9) of a plain streaming copy of `bytes`
- * (a multiple of 16), over `launches` timed launches on the null stream. */
-int tvx_calibrate_copy(size_t bytes, int launches, double* gb_per_s);
-
 #ifdef __cplusplus
 }
 #endif

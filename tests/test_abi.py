@@ -48,6 +48,41 @@ def test_descriptor_validation_needs_no_gpu(tvx):
     assert e.value.status == tvx.E_UNSUPPORTED
 
 
+def test_zero_points_outside_the_type_are_invalid(tvx):
+    """A zero point is a code of its tensor's type; checked before any device work."""
+    import numpy as np
+    d = tvx.Conv2dDesc()
+    d.in_w = d.in_h = d.out_w = d.out_h = 4
+    d.in_c = d.out_c = 16
+    d.batch = d.k_w = d.k_h = d.stride_w = d.stride_h = d.dilation_w = d.dilation_h = 1
+    d.in_dtype = d.w_dtype = d.out_dtype = tvx.U8
+    d.in_scale = d.w_scale = d.out_scale = 0.5
+    w = np.zeros(256, dtype=np.uint8)
+    for field, bad in (("in_zp", 256), ("w_zp", -1), ("out_zp", 300)):
+        setattr(d, field, bad)
+        with pytest.raises(tvx.TvxError) as e:
+            tvx.conv2d_create(d, w, None)
+        assert e.value.status == tvx.E_INVALID and "zero point" in str(e.value)
+        setattr(d, field, 0)
+    f = tvx.FcDesc()
+    f.m, f.k, f.n = 2, 16, 4
+    f.in_dtype = f.w_dtype = f.out_dtype = tvx.I8
+    f.in_scale = f.w_scale = f.out_scale = 0.5
+    f.out_zp = -129
+    with pytest.raises(tvx.TvxError) as e:
+        tvx.fully_connected_create(f, np.zeros(64, dtype=np.int8), None)
+    assert e.value.status == tvx.E_INVALID
+    p = tvx.Pool2dDesc()
+    p.in_w = p.in_h = p.out_w = p.out_h = 2
+    p.channels = p.batch = p.k_w = p.k_h = p.stride_w = p.stride_h = 1
+    p.dtype = tvx.U8
+    p.in_scale = p.out_scale = 1.0
+    p.in_zp = 256
+    with pytest.raises(tvx.TvxError) as e:
+        tvx.pool2d_create(p)
+    assert e.value.status == tvx.E_INVALID
+
+
 def test_compute_fails_loudly_without_a_gpu(tvx):
     if tvx.lib().tvx_device_count() > 0:
         pytest.skip("a GPU is present")

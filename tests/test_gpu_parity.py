@@ -388,6 +388,27 @@ def test_pointwise_conv_shapes(oracle, gi, mode, shape, monkeypatch):
     assert len(np.unique(want)) > 4
 
 
+@pytest.mark.parametrize("shape", ["128,1", "128,4", "32,1", "32,4"])
+@pytest.mark.parametrize("mode", ["u8", "i8pc", "u8pc"])
+@pytest.mark.parametrize("gi", [0, 2, 3, 4, 8])
+def test_pointwise_conv_walks_several_output_tiles_per_wavefront(oracle, gi, mode, shape, monkeypatch):
+    """One workgroup per pixel tile (the launch the heuristic picks when pixel tiles alone fill the chip, as in
+    a batch-64 network): every wavefront then walks several output tiles in sequence, re-using its input tile
+    and - with per-tensor uint8 weights whose zero point is not 128 - the zero-point sums it computed once."""
+    n, c, h, w, oc = PW_GRID[gi]
+    monkeypatch.setenv("TVX_PWCONV_SHAPE", shape)
+    monkeypatch.setenv("TVX_PWCONV_WGS", "1")
+    rng = np.random.default_rng(4100 + gi)
+    x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=oc, kh=1, kw=1, stride=[1, 1], dil=[1, 1],
+                              pad=[0, 0, 0, 0], mult=0, mode=mode)
+    assert kws["w_q"][2] is not None or kws["w_q"][1] != 128
+    for act in (0, 2):
+        want = oracle.conv2d(x, wt, b, act=act, **kws)
+        got = TC.gpu_conv2d(x, wt, b, act=act, want_kernel="pwconv_i8", **kws)
+        assert np.array_equal(got, want), int((got != want).sum())
+    assert len(np.unique(want)) > 4
+
+
 DW_GRID = [
     # (n, c, h, w, stride, pad[l,r,t,b])
     (2, 8, 16, 16, 1, [1, 1, 1, 1]),

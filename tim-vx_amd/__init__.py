@@ -123,8 +123,6 @@ def lib():
         L.tvx_convert_create.argtypes = [C.POINTER(ConvertDesc), C.POINTER(vp)]
         L.tvx_transpose_create.argtypes = [C.POINTER(TransposeDesc), C.POINTER(vp)]
         L.tvx_op_run.argtypes = [vp, vp, vp, vp, vp]
-        L.tvx_calibrate_mfma_i8.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_double)]
-        L.tvx_calibrate_copy.argtypes = [C.c_size_t, C.c_int, C.POINTER(C.c_double)]
         L.tvx_op_destroy.argtypes = [vp]
         L.tvx_op_destroy.restype = None
         _lib = L
@@ -232,16 +230,32 @@ def transpose_create(desc):
     return Op(h)
 
 
+_calib = None
+
+
+def _calibration_lib():
+    """libtvx_calibrate.so: the benchmark's device-calibration kernels (not part of the C ABI)."""
+    global _calib
+    if _calib is None:
+        L = C.CDLL(os.path.join(PKG_DIR, "lib", "libtvx_calibrate.so"))
+        L.tvx_calibrate_mfma_i8.argtypes = [C.c_int, C.c_int, C.POINTER(C.c_double)]
+        L.tvx_calibrate_copy.argtypes = [C.c_size_t, C.c_int, C.POINTER(C.c_double)]
+        _calib = L
+    return _calib
+
+
 def calibrate_mfma_i8(random_operands, launches=5):
     """Sustained int8 matrix-core rate of this GPU in TOPS (zeros: nominal clock; random
     operands: the clock held under the multipliers' switching power)."""
     v = C.c_double()
-    check(lib().tvx_calibrate_mfma_i8(int(bool(random_operands)), launches, C.byref(v)))
+    if _calibration_lib().tvx_calibrate_mfma_i8(int(bool(random_operands)), launches, C.byref(v)) != 0:
+        raise RuntimeError("tvx_calibrate_mfma_i8 failed")
     return v.value
 
 
 def calibrate_copy(nbytes=256 << 20, launches=10):
     """Read + write GB/s of a plain streaming device copy of `nbytes`."""
     v = C.c_double()
-    check(lib().tvx_calibrate_copy(nbytes, launches, C.byref(v)))
+    if _calibration_lib().tvx_calibrate_copy(nbytes, launches, C.byref(v)) != 0:
+        raise RuntimeError("tvx_calibrate_copy failed")
     return v.value

@@ -8,13 +8,24 @@
 //    figure is what any real int8 GEMM on this device can approach.
 //  * tvx_calibrate_copy: a plain 16-bytes-per-lane streaming copy, read + write bytes per
 //    second.
+//
+// Built as its own small library (libtvx_calibrate.so) for the benchmark: it is not part of
+// the operator library or of its C ABI. Both functions return 0, or -1 after printing the
+// reason to stderr.
 #include <cstdint>
 #include <vector>
 
-#include "tvx_internal.h"
+#include <hip/hip_runtime.h>
 
-namespace tvx {
+#include <cstdio>
+
 namespace {
+
+int Fail(const char* what) {
+  std::fprintf(stderr, "tvx_calibrate: %s\n", what);
+  return -1;
+}
+
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
@@ -61,7 +72,7 @@ template <typename F>
 int TimeLaunches(int launches, F launch, double* ms_per_launch) {
   hipEvent_t e0 = nullptr, e1 = nullptr;
   if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)
-    return SetError(TVX_E_DEVICE, "calibration: hipEventCreate failed");
+    return Fail("calibration: hipEventCreate failed");
   launch();
   hipError_t err = hipDeviceSynchronize();
   if (err == hipSuccess) err = hipEventRecord(e0, nullptr);
@@ -72,19 +83,17 @@ int TimeLaunches(int launches, F launch, double* ms_per_launch) {
   if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
   (void)hipEventDestroy(e0);
   (void)hipEventDestroy(e1);
-  if (err != hipSuccess || hipGetLastError() != hipSuccess) return SetError(TVX_E_DEVICE, "calibration: launch or timing failed");
+  if (err != hipSuccess || hipGetLastError() != hipSuccess) return Fail("calibration: launch or timing failed");
   *ms_per_launch = ms / launches;
-  return TVX_OK;
+  return 0;
 }
 
 }  // namespace
-}  // namespace tvx
 
 extern "C" int tvx_calibrate_mfma_i8(int random_operands, int launches, double* tops) {
-  using namespace tvx;
-  if (!tops || launches < 1 || launches > 1000) return SetError(TVX_E_INVALID, "tvx_calibrate_mfma_i8: bad argument");
+  if (!tops || launches < 1 || launches > 1000) return Fail("tvx_calibrate_mfma_i8: bad argument");
   hipDeviceProp_t prop;
-  if (hipGetDeviceProperties(&prop, 0) != hipSuccess) return SetError(TVX_E_DEVICE, "tvx_calibrate_mfma_i8: no GPU");
+  if (hipGetDeviceProperties(&prop, 0) != hipSuccess) return Fail("tvx_calibrate_mfma_i8: no GPU");
   const int wgs = prop.multiProcessorCount, iters = 500;
   std::vector<uint32_t> host(4096, 0u);
   if (random_operands) {
@@ -97,44 +106,43 @@ extern "C" int tvx_calibrate_mfma_i8(int random_operands, int launches, double* 
   void *ops = nullptr, *sink = nullptr;
   if (hipMalloc(&ops, host.size() * 4) != hipSuccess || hipMalloc(&sink, static_cast<size_t>(wgs) * 256 * 4) != hipSuccess) {
     (void)hipFree(ops);
-    return SetError(TVX_E_DEVICE, "tvx_calibrate_mfma_i8: allocation failed");
+    return Fail("tvx_calibrate_mfma_i8: allocation failed");
   }
-  int st = hipMemcpy(ops, host.data(), host.size() * 4, hipMemcpyHostToDevice) == hipSuccess ? TVX_OK
-                                                                                                : SetError(TVX_E_DEVICE, "tvx_calibrate_mfma_i8: upload failed");
+  int st = hipMemcpy(ops, host.data(), host.size() * 4, hipMemcpyHostToDevice) == hipSuccess ? 0
+                                                                                                : Fail("tvx_calibrate_mfma_i8: upload failed");
   double ms = 0;
-  if (st == TVX_OK)
+  if (st == 0)
     st = TimeLaunches(launches, [&] {
       hipLaunchKernelGGL(MfmaRateKernel, dim3(wgs), dim3(256), 0, nullptr, static_cast<const v4i*>(ops), static_cast<int*>(sink), iters);
     }, &ms);
   (void)hipFree(ops);
   (void)hipFree(sink);
-  if (st != TVX_OK) return st;
+  if (st != 0) return st;
   const double ops_per_launch = 2.0 * 32 * 32 * 32 * kMfmaPerIter * iters * 4.0 * wgs;
   *tops = ops_per_launch / (ms * 1e-3) / 1e12;
-  return TVX_OK;
+  return 0;
 }
 
 extern "C" int tvx_calibrate_copy(size_t bytes, int launches, double* gb_per_s) {
-  using namespace tvx;
   if (!gb_per_s || launches < 1 || launches > 1000 || bytes < 4096 || (bytes & 15))
-    return SetError(TVX_E_INVALID, "tvx_calibrate_copy: bad argument");
+    return Fail("tvx_calibrate_copy: bad argument");
   hipDeviceProp_t prop;
-  if (hipGetDeviceProperties(&prop, 0) != hipSuccess) return SetError(TVX_E_DEVICE, "tvx_calibrate_copy: no GPU");
+  if (hipGetDeviceProperties(&prop, 0) != hipSuccess) return Fail("tvx_calibrate_copy: no GPU");
   void *src = nullptr, *dst = nullptr;
   if (hipMalloc(&src, bytes) != hipSuccess || hipMalloc(&dst, bytes) != hipSuccess) {
     (void)hipFree(src);
-    return SetError(TVX_E_DEVICE, "tvx_calibrate_copy: allocation failed");
+    return Fail("tvx_calibrate_copy: allocation failed");
   }
-  int st = hipMemset(src, 3, bytes) == hipSuccess ? TVX_OK : SetError(TVX_E_DEVICE, "tvx_calibrate_copy: memset failed");
+  int st = hipMemset(src, 3, bytes) == hipSuccess ? 0 : Fail("tvx_calibrate_copy: memset failed");
   double ms = 0;
   const int wgs = prop.multiProcessorCount * 8;
-  if (st == TVX_OK)
+  if (st == 0)
     st = TimeLaunches(launches, [&] {
       hipLaunchKernelGGL(CopyKernel, dim3(wgs), dim3(256), 0, nullptr, static_cast<const v4i*>(src), static_cast<v4i*>(dst), bytes / 16);
     }, &ms);
   (void)hipFree(src);
   (void)hipFree(dst);
-  if (st != TVX_OK) return st;
+  if (st != 0) return st;
   *gb_per_s = 2.0 * static_cast<double>(bytes) / (ms * 1e-3) / 1e9;
-  return TVX_OK;
+  return 0;
 }

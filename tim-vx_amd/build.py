@@ -52,6 +52,9 @@ def build_hip(verbose=False):
             raise RuntimeError("build step failed: " + " ".join(cmd))
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o",
           os.path.join(PKG_DIR, "lib", "libtvx_hip.so")] + objs, verbose)
+    # the benchmark's calibration kernels: a library of their own, outside the operator library's C ABI
+    _run([HIPCC] + HIP_FLAGS + ["-shared", os.path.join(PKG_DIR, "bench_aids", "calibrate.hip"), "-o",
+                               os.path.join(PKG_DIR, "lib", "libtvx_calibrate.so")], verbose)
 
 
 def build_runtime(verbose=False):

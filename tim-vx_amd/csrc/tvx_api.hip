@@ -156,6 +156,24 @@ static int CheckOperandTypes(int in, int w, int out, const char* what) {
   return TVX_OK;
 }
 
+// A zero point is a code of its tensor's type. The kernels' accumulator bounds (|x - zx|, |w - zw| <= 255)
+// and the 32-bit requantization records (out_zp << t) rely on it.
+static int CheckZeroPoint(int dtype, int32_t zp, const char* what, const char* which) {
+  if (!IsQuant(dtype)) return TVX_OK;
+  const int32_t lo = dtype == TVX_U8 ? 0 : -128, hi = dtype == TVX_U8 ? 255 : 127;
+  if (zp < lo || zp > hi)
+    return SetError(TVX_E_INVALID, "%s: %s zero point %d outside [%d, %d]", what, which, zp, lo, hi);
+  return TVX_OK;
+}
+
+static int CheckConvZeroPoints(int in_dtype, int32_t in_zp, int w_dtype, int32_t w_zp, bool per_channel,
+                               int out_dtype, int32_t out_zp, const char* what) {
+  int s = CheckZeroPoint(in_dtype, in_zp, what, "input");
+  if (s == TVX_OK && !per_channel) s = CheckZeroPoint(w_dtype, w_zp, what, "weight");
+  if (s == TVX_OK) s = CheckZeroPoint(out_dtype, out_zp, what, "output");
+  return s;
+}
+
 }  // namespace tvx
 
 using namespace tvx;
@@ -297,6 +315,8 @@ int tvx_conv2d_create(const tvx_conv2d_desc* d, const void* weights_host,
       static_cast<uint64_t>(d->out_h - 1) * d->stride_h >= static_cast<uint64_t>(d->in_h) + d->pad_top)
     return SetError(TVX_E_INVALID, "tvx_conv2d_create: output extent reaches past the input");
   int s = CheckOperandTypes(d->in_dtype, d->w_dtype, d->out_dtype, "tvx_conv2d_create");
+  if (s == TVX_OK) s = CheckConvZeroPoints(d->in_dtype, d->in_zp, d->w_dtype, d->w_zp, d->w_scales != nullptr,
+                                           d->out_dtype, d->out_zp, "tvx_conv2d_create");
   if (s != TVX_OK) return s;
   if ((s = NoGpu()) != TVX_OK) return s;
 
@@ -352,6 +372,11 @@ int tvx_conv2d_add_create(const tvx_conv2d_desc* d, const tvx_eltwise_desc* add,
   if (!d->in_w || !d->in_h || !d->in_c || !d->batch || !d->out_c)
     return SetError(TVX_E_INVALID, "tvx_conv2d_add_create: zero extent");
   int s = CheckOperandTypes(d->in_dtype, d->w_dtype, d->out_dtype, "tvx_conv2d_add_create");
+  if (s == TVX_OK) s = CheckConvZeroPoints(d->in_dtype, d->in_zp, d->w_dtype, d->w_zp, d->w_scales != nullptr,
+                                           d->out_dtype, d->out_zp, "tvx_conv2d_add_create");
+  if (s == TVX_OK) s = CheckZeroPoint(add->dtype, add->a_zp, "tvx_conv2d_add_create", "Add operand");
+  if (s == TVX_OK) s = CheckZeroPoint(add->dtype, add->b_zp, "tvx_conv2d_add_create", "Add operand");
+  if (s == TVX_OK) s = CheckZeroPoint(add->dtype, add->out_zp, "tvx_conv2d_add_create", "Add output");
   if (s != TVX_OK) return s;
   if ((s = NoGpu()) != TVX_OK) return s;
   tvx_op* op = new (std::nothrow) tvx_op();
@@ -395,6 +420,8 @@ int tvx_deconv2d_create(const tvx_conv2d_desc* d, const void* weights_host, cons
       static_cast<uint64_t>(d->out_h) + d->pad_top > static_cast<uint64_t>(d->in_h - 1) * d->stride_h + d->k_h + d->stride_h - 1)
     return SetError(TVX_E_INVALID, "tvx_deconv2d_create: output extent reaches past the last input window");
   int s = CheckOperandTypes(d->in_dtype, d->w_dtype, d->out_dtype, "tvx_deconv2d_create");
+  if (s == TVX_OK) s = CheckConvZeroPoints(d->in_dtype, d->in_zp, d->w_dtype, d->w_zp, d->w_scales != nullptr,
+                                           d->out_dtype, d->out_zp, "tvx_deconv2d_create");
   if (s != TVX_OK) return s;
   if ((s = NoGpu()) != TVX_OK) return s;
   tvx_op* op = new (std::nothrow) tvx_op();
@@ -430,6 +457,8 @@ int tvx_fully_connected_create(const tvx_fc_desc* d, const void* weights_host,
   *out = nullptr;
   if (!d->m || !d->k || !d->n) return SetError(TVX_E_INVALID, "tvx_fully_connected_create: zero extent");
   int s = CheckOperandTypes(d->in_dtype, d->w_dtype, d->out_dtype, "tvx_fully_connected_create");
+  if (s == TVX_OK) s = CheckConvZeroPoints(d->in_dtype, d->in_zp, d->w_dtype, d->w_zp, d->w_scales != nullptr,
+                                           d->out_dtype, d->out_zp, "tvx_fully_connected_create");
   if (s != TVX_OK) return s;
   if ((s = NoGpu()) != TVX_OK) return s;
   tvx_op* op = new (std::nothrow) tvx_op();
@@ -467,7 +496,9 @@ int tvx_pool2d_create(const tvx_pool2d_desc* d, tvx_op** out) {
   if (!ValidDtype(d->dtype)) return SetError(TVX_E_INVALID, "tvx_pool2d_create: unknown dtype");
   if (d->pool_type != TVX_POOL_MAX && d->pool_type != TVX_POOL_AVG && d->pool_type != TVX_POOL_AVG_ANDROID)
     return SetError(TVX_E_UNSUPPORTED, "tvx_pool2d_create: pool type %d", d->pool_type);
-  int s = NoGpu();
+  int s = CheckZeroPoint(d->dtype, d->in_zp, "tvx_pool2d_create", "input");
+  if (s == TVX_OK) s = CheckZeroPoint(d->dtype, d->out_zp, "tvx_pool2d_create", "output");
+  if (s == TVX_OK) s = NoGpu();
   if (s != TVX_OK) return s;
   tvx_op* op = new (std::nothrow) tvx_op();
   if (!op) return SetError(TVX_E_NOMEM, "tvx_pool2d_create: host allocation failed");
@@ -496,7 +527,10 @@ static int CreateSimple(int kind, const tvx_eltwise_desc* d, tvx_op** out, int (
   if (IsQuant(d->dtype) && (!(d->a_scale > 0.f) || !(d->out_scale > 0.f) ||
                             (kind == OP_ADD && !(d->b_scale > 0.f))))
     return SetError(TVX_E_INVALID, "%s: scales must be positive", what);
-  int s = NoGpu();
+  int s = CheckZeroPoint(d->dtype, d->a_zp, what, "input");
+  if (s == TVX_OK && kind == OP_ADD) s = CheckZeroPoint(d->dtype, d->b_zp, what, "second input");
+  if (s == TVX_OK) s = CheckZeroPoint(d->dtype, d->out_zp, what, "output");
+  if (s == TVX_OK) s = NoGpu();
   if (s != TVX_OK) return s;
   tvx_op* op = new (std::nothrow) tvx_op();
   if (!op) return SetError(TVX_E_NOMEM, "%s: host allocation failed", what);

@@ -59,6 +59,94 @@ def lenet_asymu8(weights, image, batch=1):
     return {"test": "lenet_asymu8_b%d" % batch, "tensors": T, "ops": P, "output": 16}
 
 
+def lenet_random(batch=1, seed=0x71):
+    """The same LeNet topology with seeded synthetic parameters: input uint8 uniform [0, 255] at
+    scale 1/255, zero point 0; weights uint8 uniform at scale 0.02 with a zero point drawn from
+    [100, 156] per tensor; int32 biases uniform in [-1024, 1024] at scale s_in * s_w. Activation
+    scales and zero points come from a calibration pass in floating point over the first images
+    of the batch (each layer's output range between its 0.1 % and 99.9 % quantiles, widened to hold
+    zero, mapped onto the 256 codes), so that no layer collapses or saturates; they are part of the description."""
+    rng = np.random.default_rng(seed)
+    b = batch
+    u8 = lambda n: rng.integers(0, 256, n, dtype=np.uint8)
+    s_w = 0.02
+    T, P = [], []
+    nb = min(b, 4)  # images of the calibration pass
+
+    def t(dtype, attr, shape, quant=None, data=None):
+        T.append(tensor(len(T), dtype, attr, shape, quant, data))
+        return T[-1]
+
+    def quantize(real, relu):
+        # the range always holds the real value 0: the zero point has to be one of the 256 codes
+        lo = 0.0 if relu else min(float(np.quantile(real, 0.001)), 0.0)
+        hi = max(float(np.quantile(real, 0.999)), 0.0)
+        s_out = float(np.float32(max(hi - lo, 1e-6) / 255.0))
+        zp = int(np.clip(np.rint(-lo / s_out), 0, 255))
+        codes = np.clip(np.rint(real / s_out) + zp, zp if relu else 0, 255)
+        return asym(s_out, zp), (codes - zp) * s_out
+
+    def layer(kind, x, real_in, w_shape, out_shape, relu=False, **attrs):
+        """real_in: the calibration images' activations as real numbers, [nb, C, H, W] or [nb, K]."""
+        s_in = x["quant"]["scales"][0]
+        oc = w_shape[-1]
+        w_zp = int(rng.integers(100, 157))
+        wq = u8(int(np.prod(w_shape)))
+        bq = rng.integers(-1024, 1025, oc).astype(np.int32)
+        w = t("UINT8", "CONSTANT", w_shape, asym(s_w, w_zp), wq)
+        bias = t("INT32", "CONSTANT", [oc], asym(float(np.float32(s_in) * np.float32(s_w)), 0), bq)
+        wr = (wq.astype(np.float64) - w_zp) * s_w
+        if kind == "CONV2D":
+            k = w_shape[0]
+            win = np.lib.stride_tricks.sliding_window_view(real_in, (k, k), axis=(2, 3))  # [n, c, oh, ow, k, k]
+            real = np.einsum("nchwyx,ocyx->nohw", win, wr.reshape(oc, w_shape[2], k, k))
+            real += (bq * s_in * s_w)[None, :, None, None]
+        else:
+            real = real_in.reshape(nb, -1) @ wr.reshape(oc, -1).T + bq * s_in * s_w
+        q, real = quantize(real, relu)
+        y = t("UINT8", "TRANSIENT", out_shape, q)
+        P.append(op(kind, [x["id"], w["id"], bias["id"]], [y["id"]], weights=oc, **attrs))
+        return y, real
+
+    def pool(x, real):
+        w_, h_, c_, _ = x["shape"]
+        y = t("UINT8", "TRANSIENT", [w_ // 2, h_ // 2, c_, b], x["quant"])
+        P.append(op("POOL", [x["id"]], [y["id"]], pad_type="NONE", pool_type="MAX", ksize=[2, 2], stride=[2, 2]))
+        return y, real.reshape(nb, c_, h_ // 2, 2, w_ // 2, 2).max(axis=(3, 5))
+
+    img = u8(28 * 28 * b)
+    x = t("UINT8", "INPUT", [28, 28, 1, b], asym(1.0 / 255.0, 0), img)
+    real = img[:nb * 784].reshape(nb, 1, 28, 28).astype(np.float64) / 255.0
+    h, real = layer("CONV2D", x, real, [5, 5, 1, 20], [24, 24, 20, b], pad_type="VALID", ksize=[5, 5])
+    h, real = pool(h, real)
+    h, real = layer("CONV2D", h, real, [5, 5, 20, 50], [8, 8, 50, b], pad_type="VALID", ksize=[5, 5])
+    h, real = pool(h, real)
+    h, real = layer("FCL", h, real, [800, 500], [500, b], relu=True, axis=2)
+    r = t("UINT8", "TRANSIENT", [500, b], h["quant"])
+    P.append(op("RELU", [h["id"]], [r["id"]]))
+    logits, real = layer("FCL", r, real, [500, 10], [10, b], axis=0)
+    out = t("FLOAT32", "OUTPUT", [10, b])
+    P.append(op("SOFTMAX", [logits["id"]], [out["id"]], beta=1.0, sm_axis=0))
+    return {"test": "lenet_random_b%d" % batch, "tensors": T, "ops": P, "output": out["id"],
+            "logits": logits["id"]}
+
+
+def cut_at(graph, tensor_id, name=None):
+    """The graph up to the operator that produces `tensor_id`, with that tensor as the OUTPUT."""
+    import copy
+    last = next(i for i, o in enumerate(graph["ops"]) if tensor_id in o["outputs"])
+    g = {k: v for k, v in graph.items() if k not in ("tensors", "ops")}
+    g["ops"] = copy.deepcopy(graph["ops"][:last + 1])
+    used = {i for o in g["ops"] for i in o["inputs"] + o["outputs"]}
+    g["tensors"] = [dict(t) for t in graph["tensors"] if t["id"] in used]
+    for t in g["tensors"]:
+        if t["id"] == tensor_id:
+            t["attr"] = "OUTPUT"
+    g["output"] = tensor_id
+    g["test"] = name or "%s_cut%d" % (graph["test"], tensor_id)
+    return g
+
+
 # (expansion, output channels, repeats, first stride) of the MobileNetV2 bottleneck stages
 _MBV2_STAGES = [(1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1),
                 (6, 160, 3, 2), (6, 320, 1, 1)]
