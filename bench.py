@@ -28,8 +28,8 @@ PEAK_HBM_GBS = 8000.0     # HBM3E, 8 TB/s
 SEED = 0x71
 
 
-def conv_cfg2(T, rng):
-    n, c, h, w, oc = 32, 64, 56, 56, 64
+def conv_cfg2(T, rng, batch=32):
+    n, c, h, w, oc = batch, 64, 56, 56, 64
     x = rng.integers(0, 256, n * c * h * w, dtype=np.uint8)
     wt = rng.integers(0, 256, oc * c * 9, dtype=np.uint8)
     b = rng.integers(-4096, 4097, oc).astype(np.int32)
@@ -49,7 +49,7 @@ def conv_cfg2(T, rng):
                       stride=[1, 1], dilation=[1, 1], pad_left=1, pad_top=1, multiplier=0,
                       in_dtype=0, w_dtype=0, out_dtype=0, in_q=(0.05, 128), w_q=(0.01, 120, None),
                       out_q=(0.1, 0), act=2)
-    return dict(name="conv2d_u8_3x3_64to64_56x56_b32_same_relu6", op=op, inputs=(x,), out_elems=n * oc * h * w,
+    return dict(name="conv2d_u8_3x3_64to64_56x56_b%d_same_relu6" % n, op=op, inputs=(x,), out_elems=n * oc * h * w,
                 out_dtype=np.uint8, ops=2 * macs, algo_bytes=algo_bytes, bound="mfma",
                 oracle=("conv2d", (x, wt, b), oracle_kws, n))
 

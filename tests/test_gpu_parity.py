@@ -313,10 +313,12 @@ def test_conv2d_cfg2_full_size(oracle):
                dilation=[1, 1], pad_left=1, pad_top=1, multiplier=0, in_dtype=0, w_dtype=0, out_dtype=0,
                in_q=(0.05, 128), w_q=(0.01, 120, None), out_q=(0.1, 0), act=2)
     want = oracle.conv2d(x, wt, b, **kws)
-    got = TC.gpu_conv2d(x, wt, b, want_kernel="conv2d_igemm_i8", **kws)
+    got = TC.gpu_conv2d(x, wt, b, want_kernel="conv2d_igemm_i8_persistent", **kws)
     assert np.array_equal(got, want)
     assert got.max() == 60 and len(np.unique(got)) == 61  # ReLU6 at scale 0.1: q in [0, 60]
 
+
+IGEMM_KERNELS = ("conv2d_igemm_i8", "conv2d_igemm_i8_persistent")
 
 IGEMM_GRID = [
     # (n, c, h, w, oc, kh, kw, stride, dil, pad[l,r,t,b])
@@ -345,8 +347,43 @@ def test_conv2d_igemm_shapes(oracle, gi, mode):
                               pad=pad, mult=0, mode=mode)
     want = oracle.conv2d(x, wt, b, act=1, **kws)
     pointwise = kh == 1 and kw == 1 and stride == [1, 1] and pad == [0, 0, 0, 0]
-    got = TC.gpu_conv2d(x, wt, b, act=1, want_kernel="pwconv_i8" if pointwise else "conv2d_igemm_i8", **kws)
+    got = TC.gpu_conv2d(x, wt, b, act=1, want_kernel="pwconv_i8" if pointwise else IGEMM_KERNELS, **kws)
     assert np.array_equal(got, want)
+    assert len(np.unique(want)) > 4
+
+
+PERSIST_GRID = [
+    # (n, c, h, w, oc, kh, kw, stride, dil, pad[l,r,t,b]): shapes of the persistent variant (weights in registers:
+    # 32 or 64 input channels under a 3x3 kernel, 33..64 output channels, width a multiple of 4)
+    (5, 64, 56, 56, 64, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),
+    (3, 32, 28, 28, 64, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),
+    (4, 64, 20, 24, 40, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),     # 40 output channels: the second channel tile is ragged
+    (3, 32, 17, 40, 33, 3, 3, [2, 2], [1, 1], [0, 1, 0, 1]),     # stride 2: five halo rows for two output rows
+    (2, 64, 14, 20, 64, 3, 3, [1, 1], [1, 1], [0, 0, 0, 0]),     # VALID: no padding columns, 18-pixel rows
+    (2, 64, 12, 12, 48, 3, 3, [1, 1], [2, 2], [2, 2, 2, 2]),     # dilation 2: five halo rows per output row
+    (9, 64, 8, 8, 64, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),       # whole images smaller than one tile
+    (2, 32, 9, 64, 64, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),      # 64 columns: the widest single patch row
+]
+
+
+@pytest.mark.parametrize("knobs", [{}, {"TVX_IGEMM_WGS": "8"}, {"TVX_IGEMM_WGS": "16", "TVX_IGEMM_TILE_ROWS": "2"},
+                                   {"TVX_IGEMM_WGS": "8", "TVX_IGEMM_TILE_ROWS": "1"}], ids=lambda k: "-".join(k.values()) or "default")
+@pytest.mark.parametrize("mode", ["u8", "i8pc", "u8pc"])
+@pytest.mark.parametrize("gi", range(len(PERSIST_GRID)))
+def test_conv2d_igemm_persistent(oracle, gi, mode, knobs, monkeypatch):
+    """The persistent variant with its default launch and with few workgroups / small tiles forced, so that
+    every workgroup walks many tiles through both halo buffers (tiles of one, two and more output rows)."""
+    n, c, h, w, oc, kh, kw, stride, dil, pad = PERSIST_GRID[gi]
+    monkeypatch.setenv("TVX_IGEMM_PERSIST", "1")   # also where the heuristic would take the one-tile-per-workgroup kernel
+    for k, v in knobs.items():
+        monkeypatch.setenv(k, v)
+    rng = np.random.default_rng(2500 + gi)
+    x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=oc, kh=kh, kw=kw, stride=stride, dil=dil,
+                              pad=pad, mult=0, mode=mode)
+    for act in (0, 2):
+        want = oracle.conv2d(x, wt, b, act=act, **kws)
+        got = TC.gpu_conv2d(x, wt, b, act=act, want_kernel="conv2d_igemm_i8_persistent", **kws)
+        assert np.array_equal(got, want), (int((got != want).sum()), np.flatnonzero(got != want)[:8])
     assert len(np.unique(want)) > 4
 
 

@@ -43,8 +43,10 @@ CONV_TIE_CASES = [
     # need accumulators of 2^10 .. 2^14 and are rare: those cases are sized for a few dozen of them)
     ("pwconv_i8", dict(n=2, c=32, h=16, w=16, oc=64, k=1, stride=1, pad=0, mult=0), (15, 7)),
     ("pwconv_i8", dict(n=8, c=96, h=14, w=14, oc=160, k=1, stride=1, pad=0, mult=0), None),
-    ("conv2d_igemm_i8", dict(n=2, c=32, h=28, w=28, oc=64, k=3, stride=1, pad=1, mult=0), (15, 7)),
+    ("conv2d_igemm_i8_persistent", dict(n=2, c=32, h=28, w=28, oc=64, k=3, stride=1, pad=1, mult=0), (15, 7)),
+    ("conv2d_igemm_i8", dict(n=2, c=48, h=28, w=28, oc=96, k=3, stride=1, pad=1, mult=0), (15, 7)),
     ("conv2d_igemm_i8", dict(n=8, c=64, h=28, w=28, oc=80, k=3, stride=1, pad=1, mult=0), None),
+    ("conv2d_igemm_i8_persistent", dict(n=10, c=64, h=28, w=28, oc=64, k=3, stride=1, pad=1, mult=0), None),
     ("conv2d_im2col_i8", dict(n=3, c=3, h=33, w=31, oc=32, k=3, stride=2, pad=1, mult=0), (15, 7)),
     ("conv2d_im2col_i8", dict(n=12, c=1, h=28, w=28, oc=20, k=5, stride=1, pad=0, mult=0), None),
     ("dwconv3x3_i8", dict(n=2, c=8, h=16, w=16, oc=8, k=3, stride=1, pad=1, mult=1), (15, 7)),
@@ -56,10 +58,12 @@ CONV_TIE_CASES = [
 
 @pytest.mark.parametrize("mode", ["u8", "i8pc"])
 @pytest.mark.parametrize("ci", range(len(CONV_TIE_CASES)))
-def test_conv_epilogues_round_ties_to_even(oracle, ci, mode):
+def test_conv_epilogues_round_ties_to_even(oracle, ci, mode, monkeypatch):
     import torch
     import torch.nn.functional as F
     kernel, g, amp = CONV_TIE_CASES[ci]
+    if kernel.endswith("_persistent"):
+        monkeypatch.setenv("TVX_IGEMM_PERSIST", "1")
     rng = np.random.default_rng(9000 + ci)
     u8 = mode == "u8"
     n, c, h, w, oc, k, stride, pad, dm = (g[key] for key in ("n", "c", "h", "w", "oc", "k", "stride", "pad", "mult"))

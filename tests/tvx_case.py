@@ -98,7 +98,7 @@ def gpu_conv2d(x, w, bias, *, in_shape, w_shape, out_shape, stride, dilation, pa
     d.activation = act
     op = (T.deconv2d_create if transposed else T.conv2d_create)(d, w if const_weights else None, bias)
     if want_kernel is not None:
-        assert op.kernel_name == want_kernel, op.kernel_name
+        assert op.kernel_name in ((want_kernel,) if isinstance(want_kernel, str) else want_kernel), op.kernel_name
     import torch
     xd = to_device(x)
     wd = None if const_weights else to_device(w)

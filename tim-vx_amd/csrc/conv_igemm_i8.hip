@@ -20,6 +20,7 @@
 // four pixels per dword, stage [oc][pixel] in LDS, copy out as contiguous
 // runs of the WHCN output.
 #include <algorithm>
+#include <cstdlib>
 #include <type_traits>
 
 #include "variants.h"
@@ -56,7 +57,24 @@ struct ConvArgs {
   int w_chunks;          // 16-byte chunks of one channel block's weights
   int w4_blocks;         // ceil(W / 64): blocks of 16 four-column patches per channel row
   int off_w, off_halo, off_sx, off_tap, off_rq, off_bias;  // LDS carve-up
+  // persistent variant only
+  int total_tiles;       // batch * tiles_per_image
+  int halo_bytes;        // one of the two halo buffers
+  int off_out;           // epilogue staging tile
+  int tap_off[40];       // halo byte offset of k-step ks (both fragment halves lie in one tap: + 16 * half)
+#ifdef TVX_CONV_TIMESTAMPS
+  unsigned long long* ts;  // profiling build only: [workgroup][wavefront][64] wall-clock samples
+#endif
 };
+
+#ifdef TVX_CONV_TIMESTAMPS
+#define TVX_TS(slot)                                                                                         \
+  do {                                                                                                       \
+    if (a.ts && lane == 0 && (slot) < 64) a.ts[(static_cast<size_t>(blockIdx.x) * 4 + wave) * 64 + (slot)] = wall_clock64(); \
+  } while (0)
+#else
+#define TVX_TS(slot) do { } while (0)
+#endif
 
 __device__ __forceinline__ int FastDiv(int u, uint32_t magic) {
   return magic ? static_cast<int>(__umulhi(static_cast<uint32_t>(u), magic)) : u;
@@ -404,12 +422,328 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(O
   }
 }
 
+
+// ---- persistent variant ----------------------------------------------------------------
+// The same implicit GEMM for layers whose whole weight block fits the register file: every
+// wavefront keeps all KSTEPS x OT weight fragments of the operator in VGPRs for its whole life
+// (they reach the CU once per workgroup, by DMA into LDS, and are read into registers from
+// there; afterwards no weight travels through LDS and one 1 KiB activation fragment read feeds
+// OT MFMAs), and a workgroup walks many pixel tiles. While a tile is being multiplied the next
+// tile's input rows are pulled into L2 by loads whose results nobody reads; behind the tile's
+// epilogue they are loaded for real (the accumulators' registers are free then), transposed and
+// stored into the second halo buffer. Two such workgroups share a CU and drift out of phase, so
+// that one's requantization and stores run under the other's MFMA loop. Needs W % 4 == 0, all
+// input channels in one reduction group with an even number of 16-byte chunks, at most six halo
+// rows per tile and one (4 columns x 4 channels) patch per thread.
+constexpr int kPersistRows = 6;  // most halo rows of a tile
+
+// Behind a tile's epilogue its successor's halo rows go through registers in PHASES batches of NBP rows.
+template <int KSTEPS, int OT, int RQ, bool ZP, int NBP, int PHASES>
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
+ConvPersistKernel(ConvArgs a) {
+  extern __shared__ __attribute__((aligned(16))) int8_t lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int frag_row = lane & 31, frag_half = lane >> 5;
+  const int hw = a.OH * a.OW;
+
+  // ---- this workgroup's tiles: an XCD gets a contiguous run of tiles (neighbouring tiles of an
+  // image share halo rows and meet in that XCD's L2); inside the run the XCD's workgroups
+  // interleave, so that at any time they work on neighbours.
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
+  const int t_first = static_cast<int>(static_cast<long long>(a.total_tiles) * xcd / 8);
+  const int t_end = static_cast<int>(static_cast<long long>(a.total_tiles) * (xcd + 1) / 8);
+  int t = t_first + slot;
+  if (t >= t_end) return;
+
+  int8_t* out_tile = lds + a.off_out;
+  int* sx_lds = reinterpret_cast<int*>(lds + a.off_sx) + wave * 32;  // wavefront-private
+  v4i* rq_lds = reinterpret_cast<v4i*>(lds + a.off_rq);
+  int* bias_lds = reinterpret_cast<int*>(lds + a.off_bias);
+
+  // ---- this thread's patch of the halo tile: 4 input columns x 4 channels, every halo row ------
+  const size_t plane = static_cast<size_t>(a.H) * a.W;
+  const uint32_t plane32 = static_cast<uint32_t>(plane);
+  const int w4n = a.W / 4, c4n = a.cp / 4;
+  const int row_bytes = a.iwt * a.pix_stride;
+  const int blk = tid >> 6, in_blk = tid & 63;
+  const int w4 = (blk % a.w4_blocks) * 16 + (in_blk & 15);
+  const int c4 = (blk / a.w4_blocks) * 4 + (in_blk >> 4);
+  const bool has_patch = w4 < w4n && c4 < c4n;
+  const int pc = c4 * 4;
+  const int hc = a.pad_l + w4 * 4;
+  const int dst0 = __mul24(hc, a.pix_stride) + pc;
+  const int ncols = min(4, a.iwt - hc);
+  uint32_t ch_off[4];  // byte offset of the patch's four channel rows inside an image
+#pragma unroll
+  for (int j = 0; j < 4; ++j) ch_off[j] = has_patch ? static_cast<uint32_t>(pc + j) * plane32 + static_cast<uint32_t>(w4 * 4) : 0u;
+  const int xm = a.xor_mask;
+
+  auto tile_geometry = [&](int tile_index, int* n, int* p0, int* p_end, int* r0, int* ih0, int* rows_needed) {
+    const int img = tile_index / a.tiles_per_image;
+    const int tl = tile_index - img * a.tiles_per_image;
+    *n = img;
+    *p0 = tl * a.P;
+    *p_end = min(*p0 + a.P, hw);
+    *r0 = *p0 / a.OW;
+    const int r1 = (*p_end - 1) / a.OW;
+    *ih0 = *r0 * a.sh - a.pad_t;
+    *rows_needed = (r1 - *r0) * a.sh + (a.kh - 1) * a.dh + 1;
+  };
+  // address of halo row b of a tile (wavefront-uniform); rows outside the image read row 0 and are replaced later
+  auto row_pointer = [&](int n, int ih0, int rows_needed, int b) {
+    const int ih = ih0 + b;
+    const bool inside = b < rows_needed && ih >= 0 && ih < a.H;
+    return a.x + static_cast<size_t>(n) * a.C * plane + __umul24(static_cast<uint32_t>(inside ? ih : 0), static_cast<uint32_t>(a.W));
+  };
+  // all loads of a tile's patch at once
+  auto issue_loads = [&](int (&d)[NBP][4], int tile_index, int row_begin) {
+    int n, p0, p_end, r0, ih0, rows_needed;
+    tile_geometry(tile_index, &n, &p0, &p_end, &r0, &ih0, &rows_needed);
+#pragma unroll
+    for (int b = 0; b < NBP; ++b) {
+      const uint8_t* row = row_pointer(n, ih0, rows_needed, row_begin + b);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) d[b][j] = *reinterpret_cast<const int*>(row + ch_off[j]);
+    }
+  };
+  // The same loads with nobody waiting for them: they bring the rows into L2 while the matrix cores work. All
+  // write one register, which stays allocated (it is an operand of every one of them and of the wait below)
+  // until they have landed.
+  int landing = 0;
+  auto pull_into_l2 = [&](int tile_index) {
+    int n, p0, p_end, r0, ih0, rows_needed;
+    tile_geometry(tile_index, &n, &p0, &p_end, &r0, &ih0, &rows_needed);
+#pragma unroll
+    for (int b = 0; b < NBP * PHASES; ++b) {
+      const uint8_t* row = row_pointer(n, ih0, rows_needed, b);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        asm volatile("global_load_dword %0, %1, %2" : "+v"(landing) : "v"(ch_off[j]), "s"(row) : "memory");
+    }
+  };
+  // masks, 4 x 4 byte transposes, stores into halo buffer `halo`
+  auto store_halo = [&](const int (&d)[NBP][4], int tile_index, int8_t* halo, int row_begin) {
+    int n, p0, p_end, r0, ih0, rows_needed;
+    tile_geometry(tile_index, &n, &p0, &p_end, &r0, &ih0, &rows_needed);
+    if (has_patch) {
+#pragma unroll
+      for (int b = 0; b < NBP; ++b) {
+        if (row_begin + b >= rows_needed) continue;
+        const int ih = ih0 + row_begin + b;
+        const int keep = (ih >= 0 && ih < a.H) ? -1 : 0;
+        int e[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) e[j] = ((d[b][j] ^ xm) & keep) | (a.pad_fill & ~keep);
+        const int lo01 = __builtin_amdgcn_perm(e[1], e[0], 0x05010400);
+        const int hi01 = __builtin_amdgcn_perm(e[1], e[0], 0x07030602);
+        const int lo23 = __builtin_amdgcn_perm(e[3], e[2], 0x05010400);
+        const int hi23 = __builtin_amdgcn_perm(e[3], e[2], 0x07030602);
+        int px[4];
+        px[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100);
+        px[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302);
+        px[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100);
+        px[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302);
+        int8_t* dst = halo + dst0 + __mul24(row_begin + b, row_bytes);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (i < ncols) *reinterpret_cast<int*>(dst + __mul24(i, a.pix_stride)) = px[i];
+      }
+    }
+  };
+  auto store_pad_columns = [&](int tile_index, int8_t* halo) {
+    int n, p0, p_end, r0, ih0, rows_needed;
+    tile_geometry(tile_index, &n, &p0, &p_end, &r0, &ih0, &rows_needed);
+    const int right0 = a.pad_l + a.W;
+    const int pad_cols = a.pad_l + max(a.iwt - right0, 0);
+    const int units = rows_needed * pad_cols * a.cpc;
+    const v4i fill = v4i{a.pad_fill, a.pad_fill, a.pad_fill, a.pad_fill};
+    for (int u = tid; u < units; u += kThreads) {
+      const int cell = u / a.cpc, c = (u - cell * a.cpc) * 16;
+      const int hr = cell / pad_cols, pcol = cell - hr * pad_cols;
+      const int col = pcol < a.pad_l ? pcol : right0 + (pcol - a.pad_l);
+      *reinterpret_cast<v4i*>(halo + (hr * a.iwt + col) * a.pix_stride + c) = fill;
+    }
+  };
+  // Barriers here wait for this wavefront's LDS traffic only: __syncthreads() would also wait for
+  // the global stores of the tile just copied out.
+  auto lds_barrier = [] { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+  TVX_TS(0);
+  // ---- prologue: the first tile's rows on their way, the weights by DMA into the (still empty) staging tile and halo buffers,
+  // from there into every wavefront's registers; then the rows into the first halo buffer ----
+  int d0[PHASES][NBP][4];
+#pragma unroll
+  for (int ph = 0; ph < PHASES; ++ph)
+    if (has_patch) issue_loads(d0[ph], t, ph * NBP);
+  for (int i = wave * 64; i < a.w_chunks; i += kThreads)
+    __builtin_amdgcn_global_load_lds(
+        (const __attribute__((address_space(1))) void*)(a.w + static_cast<size_t>(i + lane) * 16),
+        (__attribute__((address_space(3))) void*)(lds + a.off_out + i * 16), 16, 0, 0);
+  if (tid < 32 * OT) {
+    rq_lds[tid] = a.rq[tid];
+    bias_lds[tid] = a.biasf[tid];
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the DMA has landed (and the rows have arrived)
+  lds_barrier();
+  v4i wr[KSTEPS][OT];
+  {
+    const int8_t* w_row = lds + a.off_out + frag_row * a.kstride + frag_half * 16;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks)
+#pragma unroll
+      for (int j = 0; j < OT; ++j) wr[ks][j] = *reinterpret_cast<const v4i*>(w_row + j * 32 * a.kstride + ks * 32);
+  }
+  lds_barrier();  // every wavefront has its weights: the buffers are free
+#pragma unroll
+  for (int ph = 0; ph < PHASES; ++ph) store_halo(d0[ph], t, lds + a.off_halo, ph * NBP);
+  store_pad_columns(t, lds + a.off_halo);
+  lds_barrier();
+  TVX_TS(1);
+
+  int buf = 0;
+  int ts_it = 0;
+  (void)ts_it;
+  for (; t < t_end; t += per_xcd) {
+    const int tn = t + per_xcd;
+    const bool has_next = tn < t_end;
+    if (has_next && has_patch) pull_into_l2(tn);
+    int n, p0, p_end, r0, ih0, rows_needed;
+    tile_geometry(t, &n, &p0, &p_end, &r0, &ih0, &rows_needed);
+    const int8_t* halo = lds + a.off_halo + buf * a.halo_bytes;
+    TVX_TS(2 + ts_it * 8);
+
+    // ---- one 32-pixel MFMA tile at a time: reduction, then requantization into the staging tile ----
+#pragma unroll
+    for (int i = 0; i < kMaxPtw; ++i) {
+      const int pt = wave + 4 * i;
+      if (pt < a.PT && p0 + pt * 32 < p_end) {
+        const int p = min(p0 + pt * 32 + frag_row, p_end - 1);  // rows past the tile's end recompute its last pixel
+        const int oh = p / a.OW, ow = p - oh * a.OW;
+        const int8_t* frag = halo + ((oh - r0) * a.sh * a.iwt + ow * a.sw) * a.pix_stride + frag_half * 16;
+        v16i acc[OT];
+#pragma unroll
+        for (int j = 0; j < OT; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[j][r] = 0;
+        int sx = 0;
+        // fragments RING - 1 k-steps ahead: LDS latency, not bandwidth, is what the loop would wait for
+        constexpr int RING = ZP ? 3 : 4;  // (the pixel sums' registers cost the zero-point form one stage)
+        v4i fa[RING];
+#pragma unroll
+        for (int q = 0; q < RING - 1; ++q)
+          if (q < KSTEPS) fa[q] = *reinterpret_cast<const v4i*>(frag + a.tap_off[q]);
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+          if (ks + RING - 1 < KSTEPS) fa[(ks + RING - 1) % RING] = *reinterpret_cast<const v4i*>(frag + a.tap_off[ks + RING - 1]);
+          const v4i f = fa[ks % RING];
+          if (ZP) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) sx = __builtin_amdgcn_sdot4(f[q], 0x01010101, sx, false);
+          }
+#pragma unroll
+          for (int j = 0; j < OT; ++j) acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f, wr[ks][j], acc[j], 0, 0, 0);
+        }
+        if (i == 0) TVX_TS(3 + ts_it * 8);
+        if (ZP) {
+          sx += __shfl_xor(sx, 32);
+          __builtin_amdgcn_wave_barrier();
+          if (frag_half == 0) sx_lds[frag_row] = a.zws * sx;
+          __builtin_amdgcn_wave_barrier();
+        }
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int pl = pt * 32 + 8 * g + 4 * frag_half;
+          v4i s4 = v4i{0, 0, 0, 0};
+          if (ZP) s4 = *reinterpret_cast<const v4i*>(sx_lds + 8 * g + 4 * frag_half);
+#pragma unroll
+          for (int j = 0; j < OT; ++j) {
+            const int ocl = j * 32 + frag_row;
+            const v4i rq = rq_lds[ocl];
+            const int bias = bias_lds[ocl];
+            int r4[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              r4[e] = Requant8<RQ>(acc[j][g * 4 + e] + (bias - s4[e]), rq, a.out_zp, a.lo, a.hi);
+            *reinterpret_cast<uint32_t*>(out_tile + ocl * a.out_stride + pl) = PackBytes(r4[0], r4[1], r4[2], r4[3]);
+          }
+        }
+        if (ZP) __builtin_amdgcn_wave_barrier();  // the sums are read before the next MFMA tile's are written
+      }
+      TVX_TS(4 + i + ts_it * 8);
+    }
+    // ---- the next tile's rows: L2 -> registers -> the other halo buffer ----
+    if (has_next) {
+      int8_t* halo_next = lds + a.off_halo + (buf ^ 1) * a.halo_bytes;
+      if (has_patch) asm volatile("s_waitcnt vmcnt(0)" : "+v"(landing)::"memory");
+#pragma unroll
+      for (int ph = 0; ph < PHASES; ++ph) {
+        int d[NBP][4];
+        if (has_patch) issue_loads(d, tn, ph * NBP);
+        store_halo(d, tn, halo_next, ph * NBP);
+      }
+      store_pad_columns(tn, halo_next);
+    }
+    TVX_TS(6 + ts_it * 8);
+    lds_barrier();  // staging tile complete, next halo complete
+    TVX_TS(7 + ts_it * 8);
+    // ---- copy out: contiguous runs of the WHCN output ----
+    {
+      const int valid = p_end - p0;
+      const int oc_n = min(a.oct, a.OC);
+      uint8_t* ybase = a.y + static_cast<size_t>(n) * a.OC * hw + p0;
+      if ((((hw | p0 | valid) & 15) | (reinterpret_cast<uintptr_t>(a.y) & 15)) == 0) {
+        // 16 bytes per lane, four output-channel rows per wavefront instruction
+        const int chunk = lane & 15, chunks = valid >> 4;
+        for (int o = wave * 4 + (lane >> 4); o < oc_n; o += 16) {
+          if (chunk < chunks) {
+            const int* src = reinterpret_cast<const int*>(out_tile + o * a.out_stride + chunk * 16);
+            const v4i v = v4i{src[0], src[1], src[2], src[3]};
+            *reinterpret_cast<v4i*>(ybase + static_cast<size_t>(o) * hw + chunk * 16) = v;
+          }
+        }
+      } else {
+        const int per_row = valid >> 2;  // p0 and hw are multiples of 4: whole dwords
+        for (int o = wave; o < oc_n; o += 4)
+          for (int dwi = lane; dwi < per_row; dwi += 64)
+            *reinterpret_cast<uint32_t*>(ybase + static_cast<size_t>(o) * hw + dwi * 4) =
+                *reinterpret_cast<const uint32_t*>(out_tile + o * a.out_stride + dwi * 4);
+      }
+    }
+    TVX_TS(8 + ts_it * 8);
+    lds_barrier();  // everyone has read the staging tile before the next tile's results go in
+    TVX_TS(9 + ts_it * 8);
+    ++ts_it;
+    buf ^= 1;
+  }
+  asm volatile("" ::"v"(landing));
+}
+
 struct Plan {
   ConvArgs a;
   int lds_bytes;
   int ot, rq;
   dim3 grid;
+  int persist_ksteps;  // 0: one tile per workgroup (ConvIgemmKernel); else the persistent variant
+  bool zp, small;
 };
+
+typedef void (*PersistFn)(ConvArgs);
+// The persistent variant exists for these reduction lengths (k-steps of 32 bytes) with two output-channel tiles.
+template <int KSTEPS, int NBP, int PHASES>
+PersistFn PersistKernelOf(int rq, bool zp) {
+  if (rq == kRqFastNoTie)
+    return zp ? ConvPersistKernel<KSTEPS, 2, kRqFastNoTie, true, NBP, PHASES> : ConvPersistKernel<KSTEPS, 2, kRqFastNoTie, false, NBP, PHASES>;
+  return zp ? ConvPersistKernel<KSTEPS, 2, kRqFast, true, NBP, PHASES> : ConvPersistKernel<KSTEPS, 2, kRqFast, false, NBP, PHASES>;
+}
+// small: tiles of at most four halo rows (two batches of two rows); else two batches of three
+PersistFn PersistKernel(int ksteps, int rq, bool zp, bool small) {
+  if (rq == kRqGeneric) return nullptr;
+  switch (ksteps) {
+    case 9: return small ? PersistKernelOf<9, 2, 2>(rq, zp) : PersistKernelOf<9, 3, 2>(rq, zp);
+    case 18: return small ? PersistKernelOf<18, 2, 2>(rq, zp) : PersistKernelOf<18, 3, 2>(rq, zp);
+  }
+  return nullptr;
+}
 
 template <int OT>
 void LaunchRq(const Plan* plan, const ConvArgs& a, hipStream_t st) {
@@ -422,12 +756,25 @@ void LaunchRq(const Plan* plan, const ConvArgs& a, hipStream_t st) {
     hipLaunchKernelGGL((ConvIgemmKernel<OT, kRqGeneric>), plan->grid, block, plan->lds_bytes, st, a);
 }
 
+#ifdef TVX_CONV_TIMESTAMPS
+unsigned long long* g_ts = nullptr;
+constexpr size_t kTsBytes = 1024 * 4 * 64 * 8;
+#endif
+
 int ConvIgemmRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
   const Plan* plan = reinterpret_cast<const Plan*>(op->host_blob.data());
   ConvArgs a = plan->a;
   a.x = static_cast<const uint8_t*>(in0);
   a.y = static_cast<uint8_t*>(out);
-  if (plan->ot == 1) LaunchRq<1>(plan, a, st);
+#ifdef TVX_CONV_TIMESTAMPS
+  if (!g_ts) { (void)hipMalloc(&g_ts, kTsBytes); (void)hipMemset(g_ts, 0, kTsBytes); }
+  a.ts = g_ts;
+#endif
+  if (plan->persist_ksteps) {
+    if (reinterpret_cast<uintptr_t>(in0) & 3 || reinterpret_cast<uintptr_t>(out) & 3)
+      return SetError(TVX_E_INVALID, "conv2d_igemm_i8: tensors must be 4-byte aligned");
+    hipLaunchKernelGGL(PersistKernel(plan->persist_ksteps, plan->rq, plan->zp, plan->small), plan->grid, dim3(kThreads), plan->lds_bytes, st, a);
+  } else if (plan->ot == 1) LaunchRq<1>(plan, a, st);
   else if (plan->ot == 2) LaunchRq<2>(plan, a, st);
   else LaunchRq<4>(plan, a, st);
   TVX_HIP_CHECK(hipGetLastError());
@@ -447,6 +794,13 @@ hipError_t AllowLds(int bytes) {
 }
 
 }  // namespace
+
+#ifdef TVX_CONV_TIMESTAMPS
+extern "C" int tvx_debug_conv_timestamps(void* host, size_t bytes) {
+  if (!g_ts) return -1;
+  return hipMemcpy(host, g_ts, bytes < kTsBytes ? bytes : kTsBytes, hipMemcpyDeviceToHost) == hipSuccess ? 0 : -1;
+}
+#endif
 
 // Claims dense quantized convolutions with constant weights whose weight block
 // and halo tile fit the CU's LDS.
@@ -607,10 +961,80 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   plan.lds_bytes = lds_bytes;
   plan.ot = ot;
   plan.rq = rq;
+  plan.persist_ksteps = 0;
+  plan.zp = zws != 0;
+  plan.small = false;
   plan.grid = dim3(static_cast<unsigned>(d->batch * a.tiles_per_image), static_cast<unsigned>(oc_blocks));
+
+  // ---- the persistent variant, where it applies ------------------------------------------------
+  do {
+    if (const char* f = getenv("TVX_IGEMM_PERSIST")) if (atoi(f) == 0) break;  // tuning aid
+    if (a.groups != 1 || a.cp != a.C || (a.cpc & 1) || oc_blocks != 1 || ot != 2 || (a.W & 3)) break;  // two output-channel tiles
+    const int ksteps = taps * a.cpc / 2;
+    if (!PersistKernel(ksteps, rq, plan.zp, false) || ksteps > 40) break;
+    if (a.w4_blocks * ((a.cp / 4 + 3) / 4) > kThreads / 64) break;  // one patch per thread
+    // pixel tile: whole output rows, at most six halo rows and 256 pixels; as many tiles as keep a few in
+    // every workgroup's queue
+    int want_rows = 0;
+    if (const char* f = getenv("TVX_IGEMM_TILE_ROWS")) want_rows = atoi(f);  // tuning aid
+    int rows = 0;
+    if ((a.OH * a.OW) & 3) break;  // the copy-out writes whole dwords
+    for (int r = 1; r <= a.OH; ++r) {
+      if ((r - 1) * a.sh + (a.kh - 1) * a.dh + 1 > kPersistRows || r * a.OW > 256) break;
+      if (r * a.OW & 3) continue;
+      rows = r;
+      if (r == want_rows) break;
+    }
+    if (rows == 0) break;
+    ConvArgs pa = a;
+    pa.P = rows * a.OW;
+    pa.PT = (pa.P + 31) / 32;
+    pa.tiles_per_image = (a.OH + rows - 1) / rows;
+    pa.iht = (rows - 1) * a.sh + (a.kh - 1) * a.dh + 1;
+    plan.small = pa.iht <= 4;
+    PersistFn fn = PersistKernel(ksteps, rq, plan.zp, plan.small);
+    pa.out_stride = ((pa.PT * 32 / 4) | 1) * 4;
+    const uint64_t total = static_cast<uint64_t>(d->batch) * pa.tiles_per_image;
+    if (total > 0x7fffffffull) break;
+    pa.total_tiles = static_cast<int>(total);
+    pa.oct = 64;
+    pa.halo_bytes = RoundUp(pa.iht * pa.iwt * pa.pix_stride + 64, 16);
+    pa.off_sx = 0;
+    pa.off_rq = 512;
+    pa.off_bias = pa.off_rq + 64 * 16;
+    pa.off_out = pa.off_bias + 64 * 4;
+    pa.off_halo = pa.off_out + RoundUp(pa.oct * pa.out_stride, 16);
+    // (the weights pass through the staging tile and the halo buffers on their way into the registers)
+    const int plds = std::max(pa.off_halo + 2 * pa.halo_bytes, pa.off_out + pa.w_chunks * 16);
+    if (plds > 80 * 1024) break;  // two workgroups per CU
+    for (int ks = 0; ks < ksteps; ++ks) pa.tap_off[ks] = tapt[ks * 4];  // chunk 2 * ks (chunk 2 * ks + 1 follows it)
+    bool halves_adjacent = true;
+    for (int ks = 0; ks < ksteps; ++ks) halves_adjacent = halves_adjacent && tapt[ks * 4 + 2] == tapt[ks * 4] + 16;
+    if (!halves_adjacent) break;
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, plds) != hipSuccess) {
+      (void)hipGetLastError();
+      break;
+    }
+    hipDeviceProp_t prop;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) break;
+    int wgs = 2 * prop.multiProcessorCount;
+    // Few tiles: one tile per workgroup on as many CUs as there are tiles is as fast, and the prologue above
+    // (the weights into every wavefront's registers) is not free.
+    bool forced = false;
+    if (const char* f = getenv("TVX_IGEMM_PERSIST")) forced = atoi(f) > 0;  // tuning aid
+    if (pa.total_tiles < wgs * 3 / 4 && !forced && !getenv("TVX_IGEMM_WGS")) break;
+    if (const char* f = getenv("TVX_IGEMM_WGS")) wgs = std::max(8, atoi(f));  // tuning aid
+    wgs = std::min<int>(wgs, RoundUp(pa.total_tiles, 8));
+    wgs = std::max(8, wgs / 8 * 8);
+    plan.a = pa;
+    plan.lds_bytes = plds;
+    plan.persist_ksteps = ksteps;
+    plan.grid = dim3(static_cast<unsigned>(wgs));
+  } while (false);
   op->host_blob.assign(reinterpret_cast<const uint8_t*>(&plan), reinterpret_cast<const uint8_t*>(&plan) + sizeof(plan));
   op->run = ConvIgemmRun;
-  op->kernel_name = "conv2d_igemm_i8";
+  op->kernel_name = plan.persist_ksteps ? "conv2d_igemm_i8_persistent" : "conv2d_igemm_i8";
   return TVX_OK;
 }
 
