@@ -72,6 +72,14 @@ int tvx_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, void* strea
 int tvx_stream_create(void** stream);
 int tvx_stream_destroy(void* stream);
 int tvx_stream_synchronize(void* stream);
+/* Device-side time stamps on a stream, for per-node timing: what an OpenVX application reads back with
+ * vxQueryNode(node, VX_NODE_PERFORMANCE, &vx_perf_t)
+ * (prebuilt-sdk/x86_64_linux/include/VX/vx_types.h:1008,1692-1701). tvx_event_elapsed_ms needs both
+ * events reached (synchronize the stream first). */
+int tvx_event_create(void** event);
+int tvx_event_destroy(void* event);
+int tvx_event_record(void* event, void* stream);
+int tvx_event_elapsed_ms(void* start, void* stop, float* ms);
 
 /* ---- requantization (host side, no GPU needed) ---------------------------- */
 /* real multiplier m (= s_in * s_w / s_out in double) -> mult * 2^-shift with

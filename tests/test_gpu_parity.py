@@ -148,6 +148,54 @@ def test_pool2d_random(oracle, pi, ptype, dtype):
         assert np.allclose(got.astype(np.float32), want.astype(np.float32), rtol=FLOAT_RTOL, atol=1e-3)
 
 
+POOL_ROWS = [
+    # in_shape {W, H, C, N}, ksize, stride, pad {l, r, t, b}: windows two or three taps wide (pool2d_rows_i8)
+    dict(in_shape=[24, 24, 20, 5], ksize=[2, 2], stride=[2, 2], pad=[0, 0, 0, 0]),      # LeNet: several planes per workgroup
+    dict(in_shape=[8, 8, 50, 3], ksize=[2, 2], stride=[2, 2], pad=[0, 0, 0, 0]),
+    dict(in_shape=[112, 112, 8, 2], ksize=[3, 3], stride=[2, 2], pad=[0, 1, 0, 1]),    # SAME at stride 2: right / bottom padding
+    dict(in_shape=[112, 112, 6, 1], ksize=[3, 3], stride=[2, 2], pad=[1, 1, 1, 1]),
+    dict(in_shape=[13, 9, 5, 2], ksize=[3, 3], stride=[2, 2], pad=[1, 1, 0, 1]),        # odd widths: planes that do not start on a dword
+    dict(in_shape=[10, 10, 3, 1], ksize=[3, 2], stride=[1, 3], pad=[1, 0, 1, 1]),
+    dict(in_shape=[15, 7, 9, 3], ksize=[2, 5], stride=[1, 2], pad=[1, 1, 2, 2]),        # tall window, output width not a multiple of 4
+    dict(in_shape=[230, 190, 2, 2], ksize=[3, 3], stride=[2, 2], pad=[1, 1, 1, 1]),     # planes in several row bands
+    dict(in_shape=[301, 77, 3, 1], ksize=[2, 2], stride=[1, 1], pad=[0, 1, 0, 1]),
+    dict(in_shape=[5, 4, 70, 4], ksize=[3, 3], stride=[1, 1], pad=[2, 2, 2, 2]),        # more padding than image in places
+    dict(in_shape=[3, 3, 5, 2], ksize=[2, 2], stride=[2, 2], pad=[1, 1, 1, 1]),
+]
+
+
+@pytest.mark.parametrize("dtype", [0, 1])
+@pytest.mark.parametrize("ptype", [0, 1, 3])
+@pytest.mark.parametrize("pi", range(len(POOL_ROWS)))
+def test_pool2d_rows(oracle, pi, ptype, dtype):
+    p = POOL_ROWS[pi]
+    rng = np.random.default_rng(600 + pi * 10 + ptype)
+    w, h, c, n = p["in_shape"]
+    out_w = (w + p["pad"][0] + p["pad"][1] - p["ksize"][0]) // p["stride"][0] + 1
+    out_h = (h + p["pad"][2] + p["pad"][3] - p["ksize"][1]) // p["stride"][1] + 1
+    kws = dict(in_shape=p["in_shape"], out_shape=[out_w, out_h, c, n], ksize=p["ksize"],
+               stride=p["stride"], pad_left=p["pad"][0], pad_top=p["pad"][2], pool_type=ptype, dtype=dtype)
+    x = rand_q(rng, w * h * c * n, dtype)
+    zi = 7 if dtype else 120
+    for in_q, out_q in (((0.1, zi), (0.1, zi)), ((0.1, zi), (0.07, -2 if dtype else 9)), ((0.5, zi), (0.25, zi))):
+        want = oracle.pool2d(x, in_q=in_q, out_q=out_q, **kws)
+        got = TC.gpu_pool2d(x, in_q=in_q, out_q=out_q, want_kernel="pool2d_rows_i8", **kws)
+        assert np.array_equal(got, want), (int((got != want).sum()), np.flatnonzero(got != want)[:8])
+    assert len(np.unique(want)) > 4
+
+
+def test_pool2d_full_size_max_3x3_stride2(oracle):
+    """3x3 stride 2 MAX on 112x112x64 at batch 32 (25.7 MB in, 6.4 MB out): whole output against the oracle."""
+    rng = np.random.default_rng(0x74)
+    w, h, c, n = 112, 112, 64, 32
+    x = rng.integers(0, 256, w * h * c * n, dtype=np.uint8)
+    kws = dict(in_shape=[w, h, c, n], out_shape=[56, 56, c, n], ksize=[3, 3], stride=[2, 2], pad_left=0, pad_top=0,
+               pool_type=0, dtype=0, in_q=(0.05, 3), out_q=(0.05, 3))
+    want = oracle.pool2d(x, **kws)
+    got = TC.gpu_pool2d(x, want_kernel="pool2d_rows_i8", **kws)
+    assert np.array_equal(got, want)
+
+
 @pytest.mark.parametrize("shape", [(7, 7, 1280, 3), (2, 2, 5, 1), (5, 3, 9, 2), (17, 19, 6, 2), (33, 31, 3, 1)], ids=str)
 @pytest.mark.parametrize("ptype", [1, 3])
 @pytest.mark.parametrize("dtype", [0, 1])

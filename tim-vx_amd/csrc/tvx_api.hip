@@ -273,6 +273,31 @@ int tvx_stream_synchronize(void* stream) {
   return TVX_OK;
 }
 
+int tvx_event_create(void** event) {
+  if (!event) return SetError(TVX_E_INVALID, "tvx_event_create: null result pointer");
+  hipEvent_t e = nullptr;
+  TVX_HIP_CHECK(hipEventCreate(&e));
+  *event = e;
+  return TVX_OK;
+}
+
+int tvx_event_destroy(void* event) {
+  if (event) TVX_HIP_CHECK(hipEventDestroy(static_cast<hipEvent_t>(event)));
+  return TVX_OK;
+}
+
+int tvx_event_record(void* event, void* stream) {
+  if (!event) return SetError(TVX_E_INVALID, "tvx_event_record: null event");
+  TVX_HIP_CHECK(hipEventRecord(static_cast<hipEvent_t>(event), static_cast<hipStream_t>(stream)));
+  return TVX_OK;
+}
+
+int tvx_event_elapsed_ms(void* start, void* stop, float* ms) {
+  if (!start || !stop || !ms) return SetError(TVX_E_INVALID, "tvx_event_elapsed_ms: null argument");
+  TVX_HIP_CHECK(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+  return TVX_OK;
+}
+
 int tvx_quantize_multiplier(double m, int32_t* mult, int32_t* shift) {
   if (!mult || !shift) return SetError(TVX_E_INVALID, "tvx_quantize_multiplier: null pointer");
   QuantizeMultiplier(m, mult, shift);

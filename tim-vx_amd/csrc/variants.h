@@ -46,6 +46,8 @@ bool PackDepthwise3x3(int C, const void* w_host, bool w_u8, const void* bias_hos
 int ConvGenericSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 int FcGenericSetup(tvx_op*, const tvx_fc_desc*, const void*, const void*);
 int PoolGenericSetup(tvx_op*);
+// quantized pooling, windows two or three taps wide, planes staged through LDS (pool2d_i8.hip)
+int PoolRowsSetup(tvx_op*);
 int TransposeSetup(tvx_op*);
 int ConvertSetup(tvx_op*);
 

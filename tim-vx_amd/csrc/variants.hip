@@ -14,7 +14,7 @@ const std::vector<FcSetupFn>& FcVariants() {
 }
 
 const std::vector<SimpleSetupFn>& PoolVariants() {
-  static const std::vector<SimpleSetupFn> v = {PoolGenericSetup};
+  static const std::vector<SimpleSetupFn> v = {PoolRowsSetup, PoolGenericSetup};
   return v;
 }
 

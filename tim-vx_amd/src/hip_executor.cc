@@ -17,6 +17,8 @@
 #include <map>
 
 #include "runtime.h"
+#include <utility>
+
 #include "tvx_hip.h"
 
 namespace tim {
@@ -24,6 +26,8 @@ namespace vx {
 namespace {
 
 double g_last_device_ms = 0.0;
+// Per-operator device time of the most recent Graph::Run() (TVX_RUNTIME_PROFILE=ops): name and microseconds.
+std::vector<std::pair<std::string, double>> g_last_op_us;
 
 int DtypeCode(DataType t) {
   switch (t) {
@@ -197,7 +201,19 @@ class HipExecutor : public Executor {
       if (tvx_stream_synchronize(stream_) != TVX_OK) return Fail("sync");
       t0 = std::chrono::steady_clock::now();
     }
+    // TVX_RUNTIME_PROFILE=ops: a time stamp on the stream in front of every operator and behind the last
+    // (what vxQueryNode(VX_NODE_PERFORMANCE) reports per node in the reference's driver)
+    if (profile_ops_ && events_.size() != steps_.size() + 1) {
+      while (events_.size() < steps_.size() + 1) {
+        void* e = nullptr;
+        if (tvx_event_create(&e) != TVX_OK) return Fail("event");
+        events_.push_back(e);
+      }
+    }
+    size_t step_index = 0;
     for (auto& s : steps_) {
+      if (profile_ops_ && tvx_event_record(events_[step_index], stream_) != TVX_OK) return Fail("event");
+      ++step_index;
       const int st = tvx_op_run3(s.op, dev_[s.in0], s.in1 ? dev_[s.in1] : nullptr, s.in2 ? dev_[s.in2] : nullptr,
                                  dev_[s.out], stream_);
       if (st != TVX_OK) {
@@ -205,9 +221,18 @@ class HipExecutor : public Executor {
         return false;
       }
     }
+    if (profile_ops_ && tvx_event_record(events_[steps_.size()], stream_) != TVX_OK) return Fail("event");
     if (profile_) {
       if (tvx_stream_synchronize(stream_) != TVX_OK) return Fail("sync");
       g_last_device_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+    }
+    if (profile_ops_) {
+      g_last_op_us.clear();
+      for (size_t i = 0; i < steps_.size(); ++i) {
+        float ms = 0.f;
+        if (tvx_event_elapsed_ms(events_[i], events_[i + 1], &ms) != TVX_OK) return Fail("event");
+        g_last_op_us.emplace_back(steps_[i].name, static_cast<double>(ms) * 1e3);
+      }
     }
     for (auto& t : graph->outputs_tensor_) {
       TensorImpl* ti = static_cast<TensorImpl*>(t.get());
@@ -474,6 +499,8 @@ class HipExecutor : public Executor {
 
   void* stream_ = nullptr;
   bool profile_ = std::getenv("TVX_RUNTIME_PROFILE") != nullptr;
+  bool profile_ops_ = profile_ && std::string(std::getenv("TVX_RUNTIME_PROFILE")) == "ops";
+  std::vector<void*> events_;
   std::vector<Step> steps_;
   std::map<TensorImpl*, void*> dev_;    // tensor -> device pointer (possibly an alias)
   std::map<TensorImpl*, void*> owned_;  // tensors that own their buffer
@@ -506,3 +533,9 @@ struct OfferPinnedMemory {
 // Milliseconds the operator sequence of the most recent Graph::Run() took on the
 // device (0 unless TVX_RUNTIME_PROFILE is set). No counterpart in the reference.
 extern "C" double tvx_runtime_last_device_ms(void) { return tim::vx::g_last_device_ms; }
+// Operators of the most recent Graph::Run() with their device time (TVX_RUNTIME_PROFILE=ops): count, then
+// name and microseconds of operator i. No counterpart in the reference's API (its driver keeps such numbers
+// per vx_node).
+extern "C" int tvx_runtime_last_op_count(void) { return static_cast<int>(tim::vx::g_last_op_us.size()); }
+extern "C" const char* tvx_runtime_last_op_name(int i) { return tim::vx::g_last_op_us[static_cast<size_t>(i)].first.c_str(); }
+extern "C" double tvx_runtime_last_op_us(int i) { return tim::vx::g_last_op_us[static_cast<size_t>(i)].second; }

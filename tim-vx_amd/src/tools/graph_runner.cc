@@ -17,7 +17,8 @@
 //   bench <warmup> <iters>    time Graph::Run() (after a `run`)
 //   end
 // For every `run` one line goes to stdout: "ok <name> <offset> <bytes>" or
-// "fail <name> <stage>"; for every `bench`: "bench <name> <ms per Run> <ms per Run, device part>".
+// "fail <name> <stage>"; for every `bench`: "bench <name> <ms per Run> <ms per Run, device part>" and, with
+// TVX_RUNTIME_PROFILE=ops in the environment, "opbench <name> <index> <operator> <microseconds>" per operator.
 #include <algorithm>
 #include <memory>
 #include <chrono>
@@ -39,6 +40,9 @@
 #include "tim/vx/tensor.h"
 
 extern "C" double tvx_runtime_last_device_ms(void);
+extern "C" int tvx_runtime_last_op_count(void);
+extern "C" const char* tvx_runtime_last_op_name(int i);
+extern "C" double tvx_runtime_last_op_us(int i);
 
 using namespace tim::vx;
 
@@ -363,15 +367,24 @@ int main(int argc, char** argv) {
       };
       for (int i = 0; i < warmup; ++i) { feed(); graph->Run(); }
       double dev_ms = 0;
+      std::vector<double> op_us;
       auto t0 = std::chrono::steady_clock::now();
       for (int i = 0; i < iters; ++i) {
         feed();
         graph->Run();
         dev_ms += tvx_runtime_last_device_ms();
+        const int n_ops = tvx_runtime_last_op_count();  // only with TVX_RUNTIME_PROFILE=ops
+        op_us.resize(static_cast<size_t>(n_ops), 0.0);
+        for (int o = 0; o < n_ops; ++o) op_us[static_cast<size_t>(o)] += tvx_runtime_last_op_us(o);
       }
       auto t1 = std::chrono::steady_clock::now();
       std::printf("bench %s %.6f %.6f\n", name.c_str(),
                   std::chrono::duration<double, std::milli>(t1 - t0).count() / iters, dev_ms / iters);
+      for (size_t o = 0; o < op_us.size(); ++o) {
+        std::string op_name = tvx_runtime_last_op_name(static_cast<int>(o));
+        for (char& c : op_name) if (c == ' ') c = '_';
+        std::printf("opbench %s %zu %s %.3f\n", name.c_str(), o, op_name.c_str(), op_us[o] / iters);
+      }
       std::fflush(stdout);
     } else if (rec == "end") {
       graph.reset();
