@@ -167,6 +167,44 @@ def pool_global_avg(T, rng):
     return pool_workload(T, rng, "avgpool7x7_u8_7x7x1280_b64", [7, 7, 1280, 64], 7, 7, T.POOL_AVG)
 
 
+def dwpw_cfg3(T, rng):
+    """The depthwise 3x3 and the pointwise convolution behind it as one operator: the 112x112x32 tensor between them
+    stays on the chip (38.54 MB of compulsory traffic instead of 64.2 MB for the two operators)."""
+    import ctypes as C
+    n, c, h, w, oc = 32, 32, 112, 112, 64
+    x = rng.integers(-128, 128, n * c * h * w, dtype=np.int8)
+    wd = rng.integers(-128, 128, c * 9, dtype=np.int8)
+    bd = rng.integers(-4096, 4097, c).astype(np.int32)
+    sd = np.exp(rng.uniform(np.log(0.002), np.log(0.05), c)).astype(np.float32)
+    wp = rng.integers(-128, 128, oc * c, dtype=np.int8)
+    bp = rng.integers(-4096, 4097, oc).astype(np.int32)
+    sp = np.exp(rng.uniform(np.log(0.002), np.log(0.05), oc)).astype(np.float32)
+    d = T.Conv2dDesc()
+    d.in_w, d.in_h, d.in_c, d.batch = w, h, c, n
+    d.k_w = d.k_h = 3
+    d.out_w, d.out_h, d.out_c = w, h, c
+    d.stride_w = d.stride_h = d.dilation_w = d.dilation_h = 1
+    d.pad_left = d.pad_top = 1
+    d.multiplier = 1
+    d.in_dtype = d.w_dtype = d.out_dtype = T.I8
+    d.in_scale, d.in_zp = 0.03, 0
+    d.w_scales = sd.ctypes.data_as(C.POINTER(C.c_float))
+    d.out_scale, d.out_zp = 0.08, 0
+    p = T.Conv2dDesc()
+    p.in_w, p.in_h, p.in_c, p.batch = w, h, c, n
+    p.k_w = p.k_h = 1
+    p.out_w, p.out_h, p.out_c = w, h, oc
+    p.stride_w = p.stride_h = p.dilation_w = p.dilation_h = 1
+    p.in_dtype = p.w_dtype = p.out_dtype = T.I8
+    p.in_scale, p.in_zp = 0.08, 0
+    p.w_scales = sp.ctypes.data_as(C.POINTER(C.c_float))
+    p.out_scale, p.out_zp, p.activation = 0.05, 0, T.ACT_RELU6
+    op = T.conv2d_dw_pw_create(d, wd, bd, p, wp, bp)
+    return dict(name="depthwise3x3_then_pointwise1x1_i8_per_channel_112x112x32to64_b32_relu6", op=op, inputs=(x,),
+                out_elems=n * oc * h * w, out_dtype=np.int8, ops=2 * n * h * w * c * (9 + oc),
+                algo_bytes=x.size + n * oc * h * w + wd.size + wp.size + 4 * (c + oc), bound="hbm", oracle=None)
+
+
 def time_workload(wl, steps, warmup, ring_bytes=0):
     """Returns (wall ms per step over exactly `steps` steps, mean kernel ms per launch). With ring_bytes the
     launches rotate over as many copies of the input and output tensors as make up that many bytes, so that
@@ -216,7 +254,7 @@ def time_workload(wl, steps, warmup, ring_bytes=0):
 
 KERNEL_SOURCES = {"conv2d_igemm_i8": "conv_igemm_i8.hip", "conv2d_igemm_i8_persistent": "conv_igemm_i8.hip",
                   "fc_mfma_i8_256x256x128": "fc_mfma_i8.hip", "fc_mfma_f16_256x256x64": "fc_mfma_i8.hip",
-                  "dwconv3x3_i8": "dwconv3x3_i8.hip", "pwconv_i8": "pwconv_i8.hip", "pool2d_rows_i8": "pool2d_i8.hip"}
+                  "dwconv3x3_i8": "dwconv3x3_i8.hip", "pwconv_i8": "pwconv_i8.hip", "dwconv3x3_pwconv_i8": "dwpw_i8.hip", "pool2d_rows_i8": "pool2d_i8.hip"}
 
 
 def kernel_source_sha256(kernel_name):
@@ -385,7 +423,7 @@ def main():
         line["roofline"]["traffic_stale"] = True
     if not args.no_extra:
         extra = {}
-        for make in (fc_cfg5, fc_cfg5_f16, dw_cfg3a, pw_cfg3b, conv_cfg2_b256, pool_3x3_s2, pool_lenet_b256, pool_global_avg):
+        for make in (fc_cfg5, fc_cfg5_f16, dw_cfg3a, pw_cfg3b, dwpw_cfg3, conv_cfg2_b256, pool_3x3_s2, pool_lenet_b256, pool_global_avg):
             w2 = make(T, rng)
             steps2 = max(5, min(args.steps, 50))
             wall2, k2 = time_workload(w2, steps2, min(args.warmup, 5))

@@ -214,6 +214,21 @@ int tvx_softmax_create(const tvx_softmax_desc* desc, tvx_op** op);
 int tvx_conv2d_add_create(const tvx_conv2d_desc* conv, const tvx_eltwise_desc* add, int conv_operand,
                           const void* weights_host, const void* bias_host, tvx_op** op);
 
+/* ---- depthwise 3x3 Conv2d + the 1x1 Conv2d it only feeds, in one kernel ------------------- */
+/* Two nodes of the reference's graph (vxConvolutionLayer twice: kernel/vx/convolutional.c:504-582, the
+ * first through the "depthwise_conv2d" backend) whose intermediate tensor has no other reader: the closed
+ * driver merges such layers when it verifies the graph (src/tim/vx/internal/src/vsi_nn_graph.c:1591-1603).
+ * The result is, bit for bit, what the two operators give one after the other - the depthwise result is
+ * quantized to its own tensor (dw->out_scale / out_zp, clamped by dw->activation) before the pointwise
+ * convolution reads it - but that tensor never reaches memory. `dw` and `pw` describe the two convolutions
+ * as for tvx_conv2d_create (pw's input is dw's output: same shape, type and quantization); `add` (may be
+ * NULL) is a residual Add behind the pointwise convolution as in tvx_conv2d_add_create, its other operand
+ * going in as in1 of tvx_op_run. Returns TVX_E_UNSUPPORTED when no kernel fuses this pair (the caller
+ * then creates the operators one by one). */
+int tvx_conv2d_dw_pw_create(const tvx_conv2d_desc* dw, const void* dw_weights_host, const void* dw_bias_host,
+                            const tvx_conv2d_desc* pw, const void* pw_weights_host, const void* pw_bias_host,
+                            const tvx_eltwise_desc* add, int conv_operand, tvx_op** op);
+
 /* ---- DeConv2d (transposed convolution) ----------------------------------------------- */
 /* Replaces vxDeconvolutionLayer (src/tim/vx/ops/deconv.cc:45-79,
  * src/tim/vx/internal/src/ops/vsi_nn_op_deconvolution.c:217-218,398-497). Same descriptor as

@@ -114,6 +114,8 @@ def lib():
         L.tvx_conv2d_create.argtypes = [C.POINTER(Conv2dDesc), vp, vp, C.POINTER(vp)]
         L.tvx_conv2d_add_create.argtypes = [C.POINTER(Conv2dDesc), C.POINTER(EltwiseDesc), C.c_int, vp, vp, C.POINTER(vp)]
         L.tvx_deconv2d_create.argtypes = [C.POINTER(Conv2dDesc), vp, vp, C.POINTER(vp)]
+        L.tvx_conv2d_dw_pw_create.argtypes = [C.POINTER(Conv2dDesc), vp, vp, C.POINTER(Conv2dDesc), vp, vp,
+                                              C.POINTER(EltwiseDesc), C.c_int, C.POINTER(vp)]
         L.tvx_fully_connected_create.argtypes = [C.POINTER(FcDesc), vp, vp, C.POINTER(vp)]
         L.tvx_pool2d_create.argtypes = [C.POINTER(Pool2dDesc), C.POINTER(vp)]
         L.tvx_activation_create.argtypes = [C.POINTER(EltwiseDesc), C.POINTER(vp)]
@@ -179,6 +181,14 @@ def conv2d_add_create(desc, add_desc, conv_operand, weights, bias=None):
     h = C.c_void_p()
     check(lib().tvx_conv2d_add_create(C.byref(desc), C.byref(add_desc), conv_operand, _host_ptr(weights),
                                       _host_ptr(bias), C.byref(h)))
+    return Op(h)
+
+
+def conv2d_dw_pw_create(dw_desc, dw_weights, dw_bias, pw_desc, pw_weights, pw_bias, add_desc=None, conv_operand=0):
+    h = C.c_void_p()
+    check(lib().tvx_conv2d_dw_pw_create(C.byref(dw_desc), _host_ptr(dw_weights), _host_ptr(dw_bias),
+                                        C.byref(pw_desc), _host_ptr(pw_weights), _host_ptr(pw_bias),
+                                        C.byref(add_desc) if add_desc is not None else None, conv_operand, C.byref(h)))
     return Op(h)
 
 

@@ -426,6 +426,66 @@ int tvx_conv2d_add_create(const tvx_conv2d_desc* d, const tvx_eltwise_desc* add,
   return TVX_OK;
 }
 
+int tvx_conv2d_dw_pw_create(const tvx_conv2d_desc* dw, const void* dw_w, const void* dw_b,
+                            const tvx_conv2d_desc* pw, const void* pw_w, const void* pw_b,
+                            const tvx_eltwise_desc* add, int conv_operand, tvx_op** out) {
+  if (!dw || !pw || !out) return SetError(TVX_E_INVALID, "tvx_conv2d_dw_pw_create: null argument");
+  *out = nullptr;
+  if (add && conv_operand != 1 && conv_operand != 2)
+    return SetError(TVX_E_INVALID, "tvx_conv2d_dw_pw_create: conv_operand must be 1 or 2");
+  if (!IsQuant(dw->in_dtype) || !IsQuant(dw->out_dtype) || !IsQuant(pw->out_dtype) || !dw_w || !pw_w)
+    return SetError(TVX_E_UNSUPPORTED, "tvx_conv2d_dw_pw_create: quantized tensors and constant weights only");
+  if (!dw->in_w || !dw->in_h || !dw->in_c || !dw->batch || !dw->out_w || !dw->out_h || !pw->out_c)
+    return SetError(TVX_E_INVALID, "tvx_conv2d_dw_pw_create: zero extent");
+  if (dw->multiplier < 1 || dw->out_c != dw->in_c * static_cast<uint32_t>(dw->multiplier))
+    return SetError(TVX_E_INVALID, "tvx_conv2d_dw_pw_create: the first convolution must be depthwise");
+  int s = CheckOperandTypes(dw->in_dtype, dw->w_dtype, dw->out_dtype, "tvx_conv2d_dw_pw_create");
+  if (s == TVX_OK) s = CheckOperandTypes(pw->in_dtype, pw->w_dtype, pw->out_dtype, "tvx_conv2d_dw_pw_create");
+  if (s == TVX_OK) s = CheckConvZeroPoints(dw->in_dtype, dw->in_zp, dw->w_dtype, dw->w_zp, dw->w_scales != nullptr,
+                                           dw->out_dtype, dw->out_zp, "tvx_conv2d_dw_pw_create");
+  if (s == TVX_OK) s = CheckConvZeroPoints(pw->in_dtype, pw->in_zp, pw->w_dtype, pw->w_zp, pw->w_scales != nullptr,
+                                           pw->out_dtype, pw->out_zp, "tvx_conv2d_dw_pw_create");
+  if (s != TVX_OK) return s;
+  if (add) {
+    if (add->dtype != pw->out_dtype || !(add->a_scale > 0.f) || !(add->b_scale > 0.f) || !(add->out_scale > 0.f))
+      return SetError(TVX_E_UNSUPPORTED, "tvx_conv2d_dw_pw_create: the Add must be of the convolution's output type");
+    const float conv_scale = conv_operand == 1 ? add->a_scale : add->b_scale;
+    const int32_t conv_zp = conv_operand == 1 ? add->a_zp : add->b_zp;
+    if (conv_scale != pw->out_scale || conv_zp != pw->out_zp)
+      return SetError(TVX_E_INVALID, "tvx_conv2d_dw_pw_create: the Add's operand %d is not quantized like the convolution's output", conv_operand);
+    s = CheckZeroPoint(add->dtype, add->a_zp, "tvx_conv2d_dw_pw_create", "Add operand");
+    if (s == TVX_OK) s = CheckZeroPoint(add->dtype, add->b_zp, "tvx_conv2d_dw_pw_create", "Add operand");
+    if (s == TVX_OK) s = CheckZeroPoint(add->dtype, add->out_zp, "tvx_conv2d_dw_pw_create", "Add output");
+    if (s != TVX_OK) return s;
+  }
+  if ((s = NoGpu()) != TVX_OK) return s;
+  tvx_op* op = new (std::nothrow) tvx_op();
+  if (!op) return SetError(TVX_E_NOMEM, "tvx_conv2d_dw_pw_create: host allocation failed");
+  op->kind = OP_CONV2D;
+  op->conv = *pw;
+  op->conv.w_scales = nullptr;
+  if (add) {
+    op->elt = *add;
+    op->fused_add = conv_operand;
+  }
+  op->quantized = true;
+  op->has_const_weights = true;
+  op->w_zp = pw->w_scales ? 0 : pw->w_zp;
+  std::vector<int32_t> dw_mult, dw_shift;
+  int32_t dw_lo = 0, dw_hi = 0;
+  s = BuildRequantTables(pw->out_c, pw->in_scale, pw->w_scale, pw->w_scales, pw->out_scale, &op->h_mult, &op->h_shift);
+  if (s == TVX_OK) s = BuildRequantTables(dw->out_c, dw->in_scale, dw->w_scale, dw->w_scales, dw->out_scale, &dw_mult, &dw_shift);
+  ActRange(pw->out_dtype, pw->out_scale, pw->out_zp, pw->activation, &op->act_lo, &op->act_hi);
+  ActRange(dw->out_dtype, dw->out_scale, dw->out_zp, dw->activation, &dw_lo, &dw_hi);
+  if (s == TVX_OK) s = DwPwSetup(op, dw, dw_w, dw_b, dw_mult, dw_shift, dw_lo, dw_hi, pw, pw_w, pw_b);
+  if (s != TVX_OK) {
+    delete op;
+    return s == TVX_E_UNSUPPORTED ? SetError(TVX_E_UNSUPPORTED, "tvx_conv2d_dw_pw_create: no fused kernel for this pair") : s;
+  }
+  *out = op;
+  return TVX_OK;
+}
+
 int tvx_deconv2d_create(const tvx_conv2d_desc* d, const void* weights_host, const void* bias_host,
                         tvx_op** out) {
   if (!d || !out) return SetError(TVX_E_INVALID, "tvx_deconv2d_create: null argument");

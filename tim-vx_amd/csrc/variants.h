@@ -42,6 +42,11 @@ int DwPlanesSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 bool PackDepthwise3x3(int C, const void* w_host, bool w_u8, const void* bias_host, int zxs, int zws,
                       bool all_or_none, std::vector<int32_t>* wpk, std::vector<int32_t>* biasf);
 
+// depthwise 3x3 + pointwise convolution in one kernel (dwpw_i8.hip); `op` carries the pointwise half
+int DwPwSetup(tvx_op* op, const tvx_conv2d_desc* dw, const void* dw_w, const void* dw_b,
+              const std::vector<int32_t>& dw_mult, const std::vector<int32_t>& dw_shift, int dw_lo, int dw_hi,
+              const tvx_conv2d_desc* pw, const void* pw_w, const void* pw_b);
+
 // generic (kernels_generic.hip)
 int ConvGenericSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 int FcGenericSetup(tvx_op*, const tvx_fc_desc*, const void*, const void*);

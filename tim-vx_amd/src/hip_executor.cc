@@ -62,6 +62,7 @@ class HipExecutor : public Executor {
  public:
   ~HipExecutor() override {
     for (auto& s : steps_) tvx_op_destroy(s.op);
+    for (void* e : events_) (void)tvx_event_destroy(e);
     for (auto& kv : owned_) tvx_free(kv.second);
     if (stream_) tvx_stream_destroy(stream_);
   }
@@ -94,10 +95,10 @@ class HipExecutor : public Executor {
     // Add's other operand being there before the convolution runs, may become one operator
     struct AddFusion { Operation* add; int conv_operand; };
     std::map<Operation*, AddFusion> fused_add;  // convolution -> the Add folded into it
+    std::map<Tensor*, size_t> produced_at;  // position of the operator that writes a tensor
+    for (size_t i = 0; i < graph->sorted_ops_.size(); ++i)
+      for (auto& t : graph->sorted_ops_[i]->impl()->outputs_tensor_) produced_at[t.get()] = i;
     if (!std::getenv("TVX_NO_RESIDUAL_FUSION")) {  // tuning aid: keep the Adds as operators of their own
-      std::map<Tensor*, size_t> produced_at;  // position of the operator that writes a tensor
-      for (size_t i = 0; i < graph->sorted_ops_.size(); ++i)
-        for (auto& t : graph->sorted_ops_[i]->impl()->outputs_tensor_) produced_at[t.get()] = i;
       for (size_t i = 0; i < graph->sorted_ops_.size(); ++i) {
         Operation* add = graph->sorted_ops_[i];
         OpImpl* aim = add->impl().get();
@@ -116,6 +117,33 @@ class HipExecutor : public Executor {
           fused_add[conv] = AddFusion{add, k + 1};
           break;
         }
+      }
+    }
+    // ---- depthwise -> pointwise plan: a depthwise convolution (with the activation folded into it) whose
+    // TRANSIENT result only feeds a 1x1 convolution may become one operator with it
+    std::map<Operation*, Operation*> fused_dwpw;  // depthwise convolution -> the pointwise one folded into it
+    if (!std::getenv("TVX_NO_DWPW_FUSION")) {  // tuning aid: keep the two convolutions apart
+      for (Operation* op : graph->sorted_ops_) {
+        OpImpl* im = op->impl().get();
+        if (im->kind_ != OpKind::CONV2D || im->attrs_.multiplier != 1 || im->attrs_.conv_1d || fused_add.count(op)) continue;
+        auto fa = fused_act.find(op);
+        auto mid = fa != fused_act.end() ? fa->second->impl()->outputs_tensor_[0] : im->outputs_tensor_[0];
+        if (!(mid->GetSpec().attr_ & TensorAttribute::TRANSIENT)) continue;
+        auto consumers = graph->GetConsumersOp(mid);
+        if (consumers.size() != 1) continue;
+        OpImpl* pim = consumers[0]->impl().get();
+        if (pim->kind_ != OpKind::CONV2D || pim->attrs_.multiplier != 0 || pim->attrs_.conv_1d ||
+            pim->inputs_tensor_[0] != mid)
+          continue;
+        // the merged operator runs where the depthwise convolution stands: a residual operand of the pointwise
+        // convolution's Add has to exist by then
+        auto pad = fused_add.find(consumers[0].get());
+        if (pad != fused_add.end()) {
+          auto other = pad->second.add->impl()->inputs_tensor_[pad->second.conv_operand == 1 ? 1 : 0];
+          auto oit = produced_at.find(other.get());
+          if (oit != produced_at.end() && oit->second >= produced_at[im->outputs_tensor_[0].get()]) continue;
+        }
+        fused_dwpw[op] = consumers[0].get();
       }
     }
     // ---- device storage: one buffer per tensor, Reshape outputs alias their input --
@@ -150,6 +178,29 @@ class HipExecutor : public Executor {
       bool ok = true;
       switch (im->kind_) {
         case OpKind::CONV2D: {
+          auto fd = fused_dwpw.find(op);
+          if (fd != fused_dwpw.end()) {
+            Operation* pw = fd->second;
+            OpImpl* pim = pw->impl().get();
+            int pw_act = TVX_ACT_NONE;
+            TensorImpl* pw_out = static_cast<TensorImpl*>(pim->outputs_tensor_[0].get());
+            auto pf = fused_act.find(pw);
+            if (pf != fused_act.end()) {
+              OpImpl* pa = pf->second->impl().get();
+              pw_act = pa->kind_ == OpKind::RELU ? TVX_ACT_RELU : TVX_ACT_RELU6;
+              pw_out = static_cast<TensorImpl*>(pa->outputs_tensor_[0].get());
+            }
+            auto pad = fused_add.find(pw);
+            bool both = false;
+            ok = AddDwPw(im, out, act, pim, pw_out, pw_act, pad != fused_add.end() ? pad->second.add->impl().get() : nullptr,
+                         pad != fused_add.end() ? pad->second.conv_operand : 0, &both);
+            if (!ok) break;
+            if (both) {
+              skipped[pw] = true;  // (the activation folded into it is skipped already)
+              if (pad != fused_add.end()) skipped[pad->second.add] = true;
+              break;
+            }
+          }
           auto fa = fused_add.find(op);
           bool fused = false;
           if (fa != fused_add.end()) {
@@ -287,12 +338,10 @@ class HipExecutor : public Executor {
   // With add_im: tries the Conv2d + Add operator (conv_operand: which operand of the Add the convolution is);
   // *fused says whether it exists for this convolution - if not, nothing has been added and the caller goes on
   // with the two operators.
-  bool AddConv(OpImpl* im, TensorImpl* out, int act, bool transposed = false, OpImpl* add_im = nullptr,
-               int conv_operand = 0, bool* fused = nullptr) {
+  // The convolution `im` writing `out` (its own output tensor or that of the activation folded into it) as a descriptor.
+  static tvx_conv2d_desc ConvDesc(OpImpl* im, TensorImpl* out, int act, bool transposed) {
     TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
     TensorImpl* w = static_cast<TensorImpl*>(im->inputs_tensor_[1].get());
-    TensorImpl* b = im->inputs_tensor_.size() > 2 && !im->inputs_tensor_[2]->IsPlaceHolder()
-                        ? static_cast<TensorImpl*>(im->inputs_tensor_[2].get()) : nullptr;
     const OpAttrs& a = im->attrs_;
     ShapeType xs = x->spec_.shape_, ws = w->spec_.shape_, os = out->spec_.shape_;
     if (a.conv_1d) {  // {W, C, N} tensors viewed as {W, 1, C, N}; only the kernel extents of `ws` are read
@@ -316,6 +365,66 @@ class HipExecutor : public Executor {
     WeightQuant(w->spec_, &d.w_scale, &d.w_zp, &d.w_scales);
     d.out_scale = ScaleOf(out->spec_); d.out_zp = ZpOf(out->spec_);
     d.activation = act;
+    return d;
+  }
+
+  static bool AddDesc(OpImpl* add_im, tvx_eltwise_desc* e) {
+    TensorImpl* a0 = static_cast<TensorImpl*>(add_im->inputs_tensor_[0].get());
+    TensorImpl* a1 = static_cast<TensorImpl*>(add_im->inputs_tensor_[1].get());
+    TensorImpl* sum = static_cast<TensorImpl*>(add_im->outputs_tensor_[0].get());
+    if (a0->spec_.datatype_ != a1->spec_.datatype_ || a0->spec_.datatype_ != sum->spec_.datatype_ ||
+        a0->spec_.shape_ != a1->spec_.shape_)
+      return false;
+    *e = tvx_eltwise_desc{};
+    e->count = static_cast<uint64_t>(sum->spec_.GetElementNum());
+    e->dtype = DtypeCode(sum->spec_.datatype_);
+    e->a_scale = ScaleOf(a0->spec_); e->a_zp = ZpOf(a0->spec_);
+    e->b_scale = ScaleOf(a1->spec_); e->b_zp = ZpOf(a1->spec_);
+    e->out_scale = ScaleOf(sum->spec_); e->out_zp = ZpOf(sum->spec_);
+    return true;
+  }
+
+  // A depthwise convolution and the pointwise convolution that alone reads its result as one operator
+  // (tvx_conv2d_dw_pw_create), the pointwise one possibly with the residual Add behind it. *fused says whether a
+  // kernel took the pair; if not, the caller adds the operators one by one.
+  bool AddDwPw(OpImpl* dw_im, TensorImpl* dw_out, int dw_act, OpImpl* pw_im, TensorImpl* pw_out, int pw_act,
+               OpImpl* add_im, int conv_operand, bool* fused) {
+    *fused = false;
+    auto constant = [](OpImpl* im, TensorImpl** w, TensorImpl** b) {
+      *w = static_cast<TensorImpl*>(im->inputs_tensor_[1].get());
+      *b = im->inputs_tensor_.size() > 2 && !im->inputs_tensor_[2]->IsPlaceHolder()
+               ? static_cast<TensorImpl*>(im->inputs_tensor_[2].get()) : nullptr;
+      return (*w)->IsConstTensor() && (*w)->HostData() && (!*b || ((*b)->IsConstTensor() && (*b)->HostData()));
+    };
+    TensorImpl *dw_w, *dw_b, *pw_w, *pw_b;
+    if (!constant(dw_im, &dw_w, &dw_b) || !constant(pw_im, &pw_w, &pw_b)) return true;
+    const tvx_conv2d_desc dw = ConvDesc(dw_im, dw_out, dw_act, false);
+    const tvx_conv2d_desc pw = ConvDesc(pw_im, pw_out, pw_act, false);
+    tvx_eltwise_desc e{};
+    if (add_im && !AddDesc(add_im, &e)) return true;
+    tvx_op* op = nullptr;
+    const int st = tvx_conv2d_dw_pw_create(&dw, dw_w->HostData(), dw_b ? dw_b->HostData() : nullptr, &pw, pw_w->HostData(),
+                                           pw_b ? pw_b->HostData() : nullptr, add_im ? &e : nullptr, conv_operand, &op);
+    if (st == TVX_E_UNSUPPORTED) return true;
+    if (st != TVX_OK) return Fail("tvx_conv2d_dw_pw_create");
+    *fused = true;
+    TensorImpl* x = static_cast<TensorImpl*>(dw_im->inputs_tensor_[0].get());
+    if (add_im) {
+      TensorImpl* other = static_cast<TensorImpl*>(add_im->inputs_tensor_[conv_operand == 1 ? 1 : 0].get());
+      Push(op, dw_im, x, other, static_cast<TensorImpl*>(add_im->outputs_tensor_[0].get()));
+    } else {
+      Push(op, dw_im, x, nullptr, pw_out);
+    }
+    return true;
+  }
+
+  bool AddConv(OpImpl* im, TensorImpl* out, int act, bool transposed = false, OpImpl* add_im = nullptr,
+               int conv_operand = 0, bool* fused = nullptr) {
+    TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
+    TensorImpl* w = static_cast<TensorImpl*>(im->inputs_tensor_[1].get());
+    TensorImpl* b = im->inputs_tensor_.size() > 2 && !im->inputs_tensor_[2]->IsPlaceHolder()
+                        ? static_cast<TensorImpl*>(im->inputs_tensor_[2].get()) : nullptr;
+    tvx_conv2d_desc d = ConvDesc(im, out, act, transposed);
     // a bias that is not a constant is read at run time, which the kernels with packed weights
     // cannot do: weights and bias then both go in as operands of the generic kernel
     const bool bias_at_run = b && !b->IsConstTensor();
@@ -326,15 +435,8 @@ class HipExecutor : public Executor {
       TensorImpl* a0 = static_cast<TensorImpl*>(add_im->inputs_tensor_[0].get());
       TensorImpl* a1 = static_cast<TensorImpl*>(add_im->inputs_tensor_[1].get());
       TensorImpl* sum = static_cast<TensorImpl*>(add_im->outputs_tensor_[0].get());
-      if (!const_w || a0->spec_.datatype_ != a1->spec_.datatype_ || a0->spec_.datatype_ != sum->spec_.datatype_ ||
-          a0->spec_.shape_ != a1->spec_.shape_)
-        return true;
       tvx_eltwise_desc e{};
-      e.count = static_cast<uint64_t>(sum->spec_.GetElementNum());
-      e.dtype = DtypeCode(sum->spec_.datatype_);
-      e.a_scale = ScaleOf(a0->spec_); e.a_zp = ZpOf(a0->spec_);
-      e.b_scale = ScaleOf(a1->spec_); e.b_zp = ZpOf(a1->spec_);
-      e.out_scale = ScaleOf(sum->spec_); e.out_zp = ZpOf(sum->spec_);
+      if (!const_w || !AddDesc(add_im, &e)) return true;
       const int st = tvx_conv2d_add_create(&d, &e, conv_operand, w->HostData(), b ? b->HostData() : nullptr, &op);
       if (st == TVX_E_UNSUPPORTED) return true;
       if (st != TVX_OK) return Fail("tvx_conv2d_add_create");
