@@ -292,3 +292,80 @@ def test_mobilenet_v2_graph_bit_exact(tmp_path, oracle, batch, res):
     # the ten residual Adds ride on the projection convolutions in front of them: no Add kernel in the plan
     plan = [l for l in log.splitlines() if "uid" in l and "->" in l]
     assert sum("pwconv_add_i8" in l for l in plan) == 10 and not any("ADD" in l for l in plan), plan
+
+
+def _pool_graph(name, in_shape, out_shape, pool_type, form, ksize, stride, dt="UINT8", in_q=(0.5, 12), out_q=(0.5, 12)):
+    rng = np.random.default_rng(len(name))
+    lo, hi = (0, 256) if dt == "UINT8" else (-128, 128)
+    x = rng.integers(lo, hi, int(np.prod(in_shape))).astype(np.uint8 if dt == "UINT8" else np.int8)
+    ts = [GF.tensor(0, dt, "INPUT", in_shape, GF.asym(*in_q), x),
+          GF.tensor(1, dt, "OUTPUT", out_shape, GF.asym(*out_q))]
+    ops = [GF.op("POOL", [0], [1], pool_type=pool_type, pool_1d=form, ksize=ksize, stride=stride)]
+    return {"test": name, "tensors": ts, "ops": ops, "output": 1}
+
+
+@pytest.mark.gpu
+def test_pool2d_global_and_adaptive_constructors(tmp_path, oracle):
+    """Pool2d's two constructors that take sizes instead of a window (include/tim/vx/ops/pool2d.h:87-99,
+    src/tim/vx/ops/pool2d.cc:62-93): global pooling (window = stride = input size) and adaptive pooling
+    (stride = floor(in / out), window = in - (out - 1) * stride). The runner calls the constructors; the
+    expectation is the oracle's pooling over the window those rules give, written out here."""
+    cases, wants = [], []
+    for pool_type in ("MAX", "AVG"):
+        g = _pool_graph("global_" + pool_type, [7, 5, 24, 3], [1, 1, 24, 3], pool_type, "global", [7, 5], [7, 5],
+                        out_q=(0.75, 3))
+        cases.append(g)
+        e = copy.deepcopy(g)
+        e["ops"][0]["attrs"].update(pool_1d=False, ksize=[7, 5], stride=[7, 5])
+        wants.append(oracle.run_graph(e))
+        for (iw, ih), (ow, oh) in (((12, 10), (4, 3)), ((9, 9), (2, 2)), ((16, 8), (16, 8))):
+            g = _pool_graph("adaptive_%s_%dx%d_to_%dx%d" % (pool_type, iw, ih, ow, oh), [iw, ih, 8, 2], [ow, oh, 8, 2],
+                            pool_type, "adaptive", [iw, ih], [ow, oh], dt="INT8", in_q=(0.1, -4), out_q=(0.13, 2))
+            cases.append(g)
+            sw, sh = iw // ow, ih // oh
+            e = copy.deepcopy(g)
+            e["ops"][0]["attrs"].update(pool_1d=False, ksize=[iw - (ow - 1) * sw, ih - (oh - 1) * sh], stride=[sw, sh])
+            wants.append(oracle.run_graph(e))
+    res, info, log = GF.run_graphs(cases, str(tmp_path))
+    for c, got, want in zip(cases, res, wants):
+        assert got is not None, (c["test"], info.get(c["test"]), log[-1500:])
+        assert np.array_equal(got, want), c["test"]
+    assert all(len(np.unique(w)) > 4 for w in wants)
+
+
+@pytest.mark.gpu
+def test_operators_arrive_through_clone(tmp_path, oracle):
+    """Operation::Clone (include/tim/vx/operation.h:46): every operator of the sample network and of a graph
+    with the sized Pool2d constructors is created in a second graph and cloned into the one that runs; the
+    clone must carry every attribute (pads, strides, multiplier, weights, axis, the pooling window)."""
+    w, x = _lenet_data()
+    g = GRAPHS.lenet_asymu8(w, x)
+    g["test"] = "lenet_cloned"
+    g["clone"] = True
+    p = _pool_graph("adaptive_cloned", [12, 10, 8, 2], [4, 3, 8, 2], "AVG", "adaptive", [12, 10], [4, 3])
+    p["clone"] = True
+    e = copy.deepcopy(p)
+    e["ops"][0]["attrs"].update(pool_1d=False, ksize=[12 - 3 * 3, 10 - 2 * 3], stride=[3, 3])
+    m = GRAPHS.mobilenet_v2(batch=1, res=32)
+    m["test"] = "mobilenet_cloned"
+    m["clone"] = True
+    res, info, log = GF.run_graphs([g, p, m], str(tmp_path))
+    assert all(r is not None for r in res), (info, log[-1500:])
+    assert np.array_equal(res[0], oracle.run_graph(g))
+    assert np.array_equal(res[1], oracle.run_graph(e))
+    assert np.array_equal(res[2], oracle.run_graph(m))
+
+
+def test_compile_option_carries_the_device(tmp_path):
+    """CompileOption::setDeviceId / getDeviceId (include/tim/vx/compile_option.h:45-48; the graph hands the
+    index to the driver at src/tim/vx/graph.cc:345-348): a graph created for a GPU the machine does not have
+    must not compile; index 0 is the GPU this runtime drives."""
+    g = _pool_graph("device_7", [4, 4, 8, 1], [2, 2, 8, 1], "MAX", False, [2, 2], [2, 2])
+    g["device"] = 7
+    ok = _pool_graph("device_0", [4, 4, 8, 1], [2, 2, 8, 1], "MAX", False, [2, 2], [2, 2])
+    ok["device"] = 0
+    res, info, log = GF.run_graphs([g, ok], str(tmp_path))
+    assert res[0] is None and info["device_7"]["fail"] == "compile"
+    if _has_gpu():
+        assert "compiled for device 7" in log
+        assert res[1] is not None

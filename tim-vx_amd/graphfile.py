@@ -43,6 +43,11 @@ _DEFAULT_ATTRS = {"pad_type": "AUTO", "pad": [0, 0, 0, 0], "stride": [1, 1], "di
                   "layout": "ANY", "kernel_layout": "ANY", "output_padding": [0, 0]}
 
 
+# "pool_1d": False / True, or the Pool2d constructor to call: "global" (ksize = input size) or "adaptive"
+# (ksize = input size, stride = output size)
+_POOL_FORM = {False: 0, True: 1, 0: 0, 1: 1, "global": 2, "adaptive": 3}
+
+
 def op(kind, inputs, outputs, **attrs):
     a = dict(_DEFAULT_ATTRS)
     a.update(attrs)
@@ -70,6 +75,10 @@ def write_graphs(graphs, txt_path, blob_path, bench=None):
                 txt.write("handles\n")
             if g.get("platform"):
                 txt.write("platform\n")
+            if g.get("device") is not None:
+                txt.write("device %d\n" % g["device"])
+            if g.get("clone"):
+                txt.write("clone\n")
             for t in g["tensors"]:
                 raw = tensor_bytes(t)
                 q = t["quant"]
@@ -84,7 +93,7 @@ def write_graphs(graphs, txt_path, blob_path, bench=None):
                 a.update(o["attrs"])
                 f = ["op", o["kind"], len(o["inputs"])] + list(o["inputs"]) + [len(o["outputs"])] + list(o["outputs"])
                 f += [a["pad_type"]] + list(a["pad"]) + list(a["stride"]) + list(a["dilation"]) + list(a["ksize"])
-                f += [a["multiplier"], a["weights"], a["pool_type"], a["round_type"], int(bool(a["pool_1d"])),
+                f += [a["multiplier"], a["weights"], a["pool_type"], a["round_type"], _POOL_FORM[a["pool_1d"]],
                       a["axis"], "%.9g" % a["beta"], a["sm_axis"], len(a["new_shape"])] + list(a["new_shape"]) + [a["groups"], int(bool(a["conv_1d"]))]
                 f += [len(a["perm"])] + list(a["perm"]) + [a["layout"], a["kernel_layout"]] + list(a["output_padding"])
                 txt.write(" ".join(str(x) for x in f) + "\n")

@@ -174,6 +174,11 @@ class CompileOption {
   ~CompileOption() {}
   bool isRelaxMode() const;
   bool setRelaxMode(bool enable = false);
+  // The GPU a graph compiles for (platform::IDevice::device_id_t, the index IDevice::Enumerate() numbers devices
+  // by; reference: compile_option.h:45-48, consumed at graph.cc:345-348). A graph whose index names no GPU of the
+  // machine does not compile.
+  void setDeviceId(uint32_t device);
+  uint32_t getDeviceId();
   static CompileOption DefaultOptions;
 
  private:

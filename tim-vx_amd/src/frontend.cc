@@ -131,6 +131,7 @@ bool Quantization::operator==(const Quantization& o) const {
 // ---------------------------------------------------------------------------
 struct CompileOptionImpl {
   bool relax_mode = false;
+  uint32_t device_id = 0;
 };
 CompileOption::CompileOption() : impl_(std::make_shared<CompileOptionImpl>()) {}
 bool CompileOption::isRelaxMode() const { return impl_->relax_mode; }
@@ -138,6 +139,8 @@ bool CompileOption::setRelaxMode(bool enable) {
   impl_->relax_mode = enable;
   return true;
 }
+void CompileOption::setDeviceId(uint32_t device) { impl_->device_id = device; }
+uint32_t CompileOption::getDeviceId() { return impl_->device_id; }
 CompileOption CompileOption::DefaultOptions;
 
 // ---------------------------------------------------------------------------

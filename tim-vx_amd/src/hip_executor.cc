@@ -72,6 +72,13 @@ class HipExecutor : public Executor {
       VSILOGE("no GPU: this runtime has no CPU execution path");
       return false;
     }
+    // the device the graph was compiled for (reference: graph.cc:345-348, VX_GRAPH_DEVICE_INDEX_VIV): this runtime
+    // drives the process's current GPU, index 0
+    const uint32_t device = graph->options_.getDeviceId();
+    if (device >= static_cast<uint32_t>(tvx_device_count()) || device != 0) {
+      VSILOGE("graph compiled for device %u: this runtime runs on device 0 of %d", device, tvx_device_count());
+      return false;
+    }
     if (tvx_stream_create(&stream_) != TVX_OK) return Fail("stream");
     // ---- activation fusion plan ------------------------------------------------
     std::map<Operation*, Operation*> fused_act;  // producer -> activation folded into it

@@ -34,7 +34,10 @@ class ExecutableImpl : public NativeExecutable {
       : source_(source) {
     executor_ = executor;
     context_ = executor->Contex();
-    nb_graph_ = context_->CreateGraph();
+    // (reference: native.cc:300-303 - the executable's graph is compiled for the executor's device)
+    CompileOption option;
+    option.setDeviceId(executor->Device()->Id());
+    nb_graph_ = context_->CreateGraph(option);
   }
   void SetInput(const std::shared_ptr<ITensorHandle>& th) override { input_handles_.push_back(th); }
   void SetOutput(const std::shared_ptr<ITensorHandle>& th) override { output_handles_.push_back(th); }

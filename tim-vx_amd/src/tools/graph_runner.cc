@@ -11,7 +11,11 @@
 //   op <KIND> <n_in> <ids..> <n_out> <ids..> <pad_type> <pl> <pr> <pt> <pb> <sw> <sh> <dw> <dh>
 //      <kw> <kh> <multiplier> <weights> <pool_type> <round_type> <pool_1d> <axis> <beta> <sm_axis>
 //      <n_shape> <shape..> <groups> <conv_1d>
-//       id -1 = the graph's placeholder tensor (no bias)
+//       id -1 = the graph's placeholder tensor (no bias); <pool_1d>: 0 = Pool2d by pad / pad type, 1 = Pool1d,
+//       2 = Pool2d's global-pooling constructor (<kw> <kh> = input size), 3 = its adaptive constructor
+//       (<kw> <kh> = input size, <sw> <sh> = output size)
+//   device <index>            (before the tensors) the graph is created with CompileOption::setDeviceId(index)
+//   clone                     operators are created in a second graph and arrive through Operation::Clone()
 //   run <tensor id>           compile (first time) + run; append the tensor to out.bin
 //   feed <tensor id> <off> <len>   an INPUT tensor takes these blob bytes from the next run on
 //   bench <warmup> <iters>    time Graph::Run() (after a `run`)
@@ -123,7 +127,8 @@ int main(int argc, char** argv) {
   std::shared_ptr<Graph> graph, source_graph;
   std::map<int, Pending> tensors;
   std::string name, line;
-  bool compiled = false, compile_ok = false, use_handles = false, use_platform = false;
+  bool compiled = false, compile_ok = false, use_handles = false, use_platform = false, use_clone = false;
+  std::shared_ptr<Graph> donor;  // with `clone`: operators are created here and Clone()d into the graph
   std::shared_ptr<platform::IExecutor> executor;
   std::shared_ptr<platform::IExecutable> executable;
   std::vector<std::unique_ptr<std::vector<char>>> handle_bufs;
@@ -140,12 +145,26 @@ int main(int argc, char** argv) {
       use_handles = false;
       handle_bufs.clear();
       use_platform = false;
+      use_clone = false;
+      donor.reset();
       executable.reset();
       executor.reset();
     } else if (rec == "platform") {
       // the graph runs as an executable of the platform API: device -> executor -> Compile(graph),
       // tensor handles allocated by the executable for every graph input / output, Submit + Trigger
       use_platform = true;
+    } else if (rec == "device") {
+      // the graph is created with a CompileOption that names the GPU it compiles for
+      uint32_t id = 0;
+      ss >> id;
+      CompileOption option;
+      option.setDeviceId(id);
+      if (option.getDeviceId() != id) { std::fprintf(stderr, "CompileOption lost the device id\n"); return 2; }
+      graph = context->CreateGraph(option);
+    } else if (rec == "clone") {
+      // every operator is created in a second graph and arrives in this one through Operation::Clone()
+      use_clone = true;
+      donor = context->CreateGraph();
     } else if (rec == "handles") {
       // graph inputs and outputs live in buffers of the caller (Graph::CreateIOTensor), are handed over
       // with FlushCacheForHandle / InvalidateCacheForHandle and exchanged with SwapHandle between runs
@@ -217,6 +236,8 @@ int main(int argc, char** argv) {
       const DataLayout layout = ParseLayout(layout_s, DataLayout::WHCN), klayout = ParseLayout(klayout_s, DataLayout::WHIcOc);
       const RoundType rnd = round_type == "CEILING" ? RoundType::CEILING : RoundType::FLOOR;
       std::shared_ptr<Operation> op;
+      std::shared_ptr<Graph> target = graph;
+      if (use_clone) graph = donor;
       if (kind == "CONV2D" && conv_1d) {
         op = graph->CreateOperation<ops::Conv1d>(weights, ParsePad(pad_type), ksize[0], stride[0], dil[0],
                                                  std::array<uint32_t, 2>{pad[0], pad[1]}, multiplier);
@@ -230,9 +251,13 @@ int main(int argc, char** argv) {
       } else if (kind == "FCL") {
         op = graph->CreateOperation<ops::FullyConnected>(static_cast<uint32_t>(axis), static_cast<uint32_t>(weights));
       } else if (kind == "POOL") {
-        if (pool_1d) {
+        if (pool_1d == 1) {
           op = graph->CreateOperation<ops::Pool1d>(ParsePool(pool_type), std::array<uint32_t, 2>{pad[0], pad[1]},
                                                    ksize[0], stride[0], rnd);
+        } else if (pool_1d == 2) {  // the global-pooling constructor: ksize carries the input size
+          op = graph->CreateOperation<ops::Pool2d>(ParsePool(pool_type), ksize, rnd, layout);
+        } else if (pool_1d == 3) {  // the adaptive constructor: ksize = input size, stride = output size
+          op = graph->CreateOperation<ops::Pool2d>(ParsePool(pool_type), ksize, stride, rnd, layout);
         } else if (ParsePad(pad_type) == PadType::AUTO) {
           op = graph->CreateOperation<ops::Pool2d>(ParsePool(pool_type), pad, ksize, stride, rnd, layout);
         } else {
@@ -258,6 +283,10 @@ int main(int argc, char** argv) {
       } else {
         std::fprintf(stderr, "unknown op kind %s\n", kind.c_str());
         return 2;
+      }
+      if (use_clone) {
+        graph = target;
+        op = op->Clone(graph);
       }
       op->BindInputs(ins).BindOutputs(outs);
     } else if (rec == "infer") {
