@@ -60,6 +60,48 @@ def conv_cfg2_b256(T, rng):
     return conv_cfg2(T, rng, batch=256)
 
 
+def conv_f16(T, rng):
+    """The headline convolution's shape in float16 (float32 accumulation)."""
+    n, c, h, w, oc = 32, 64, 56, 56, 64
+    x = rng.standard_normal(n * c * h * w, dtype=np.float32).astype(np.float16)
+    wt = (rng.standard_normal(oc * c * 9, dtype=np.float32) * 0.05).astype(np.float16)
+    b = rng.standard_normal(oc).astype(np.float32)
+    d = T.Conv2dDesc()
+    d.in_w, d.in_h, d.in_c, d.batch = w, h, c, n
+    d.k_w = d.k_h = 3
+    d.out_w, d.out_h, d.out_c = w, h, oc
+    d.stride_w = d.stride_h = d.dilation_w = d.dilation_h = 1
+    d.pad_left = d.pad_top = 1
+    d.in_dtype = d.w_dtype = d.out_dtype = T.F16
+    d.activation = T.ACT_RELU6
+    op = T.conv2d_create(d, wt, b)
+    return dict(name="conv2d_f16_3x3_64to64_56x56_b32_same_relu6", op=op, inputs=(x,), out_elems=n * oc * h * w,
+                out_dtype=np.float16, ops=2 * n * h * w * oc * c * 9, algo_bytes=2 * (x.size + n * oc * h * w + wt.size) + 4 * oc,
+                bound="mfma", peak=PEAK_F16_TFLOPS, oracle=None)
+
+
+def conv_grouped(T, rng):
+    """A grouped convolution (4 groups of 32 -> 32 channels, 3x3, 28x28, batch 32), u8 per-tensor."""
+    n, c, h, w, oc, groups = 32, 128, 28, 28, 128, 4
+    x = rng.integers(0, 256, n * c * h * w, dtype=np.uint8)
+    wt = rng.integers(0, 256, oc * (c // groups) * 9, dtype=np.uint8)
+    b = rng.integers(-4096, 4097, oc).astype(np.int32)
+    d = T.Conv2dDesc()
+    d.in_w, d.in_h, d.in_c, d.batch = w, h, c, n
+    d.k_w = d.k_h = 3
+    d.out_w, d.out_h, d.out_c = w, h, oc
+    d.stride_w = d.stride_h = d.dilation_w = d.dilation_h = 1
+    d.pad_left = d.pad_top = 1
+    d.groups = groups
+    d.in_dtype = d.w_dtype = d.out_dtype = T.U8
+    d.in_scale, d.in_zp, d.w_scale, d.w_zp = 0.05, 128, 0.01, 120
+    d.out_scale, d.out_zp, d.activation = 0.1, 0, T.ACT_RELU6
+    op = T.conv2d_create(d, wt, b)
+    return dict(name="grouped_conv2d_u8_3x3_4x32to32_28x28_b32_same_relu6", op=op, inputs=(x,),
+                out_elems=n * oc * h * w, out_dtype=np.uint8, ops=2 * n * h * w * oc * (c // groups) * 9,
+                algo_bytes=x.size + n * oc * h * w + wt.size + 4 * oc, bound="mfma", oracle=None)
+
+
 def fc_cfg5(T, rng):
     m, k, n = 8192, 4096, 4096
     x = rng.integers(-128, 128, m * k, dtype=np.int8)

@@ -554,6 +554,56 @@ def test_grouped_conv2d(oracle, gi, mode):
         assert np.array_equal(TC.gpu_conv2d(x, wt, b, **dw), got)
 
 
+GEMM_GRID = [
+    # (n, c, oc, groups, h, w, kh, kw, stride, dil, pad[l,r,t,b]): groups worth a matrix tile (at least 8 output
+    # channels and 32 window bytes each), one and two 32-channel tiles per workgroup, ragged last tiles, pixel
+    # counts that are no multiple of four (element stores) and of 128 (ragged pixel tile), dilation, strides
+    (2, 32, 48, 2, 13, 11, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),
+    (2, 64, 256, 4, 16, 16, 3, 3, [2, 2], [1, 1], [0, 1, 0, 1]),
+    (1, 40, 40, 2, 15, 14, 5, 5, [1, 1], [2, 2], [4, 4, 4, 4]),
+    (3, 48, 200, 2, 12, 20, 3, 1, [1, 2], [1, 1], [0, 0, 1, 1]),
+    (2, 36, 27, 3, 9, 9, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),
+    (1, 40, 72, 1, 24, 24, 1, 1, [1, 1], [1, 1], [0, 0, 0, 0]),
+]
+
+
+@pytest.mark.parametrize("mode", ["u8", "i8pc", "u8pc", "f16"])
+@pytest.mark.parametrize("gi", range(len(GEMM_GRID)))
+def test_conv2d_gemm(oracle, gi, mode):
+    """conv2d_gemm_i8 / conv2d_gemm_f16: windows gathered into LDS, MFMA over 64-byte chunks of the reduction."""
+    n, c, oc, groups, h, w, kh, kw, stride, dil, pad = GEMM_GRID[gi]
+    rng = np.random.default_rng(7300 + gi)
+    x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=oc, kh=kh, kw=kw, stride=stride, dil=dil,
+                              pad=pad, mult=0, mode=mode, groups=groups if groups > 1 else 0)
+    quant = mode != "f16"
+    if quant and groups == 1 and kh == 1 and kw == 1:
+        pytest.skip("the pointwise kernel takes the quantized 1x1 case")
+    for act in (0, 2):
+        want = oracle.conv2d(x, wt, b, act=act, **kws)
+        got = TC.gpu_conv2d(x, wt, b, act=act, want_kernel="conv2d_gemm_i8" if quant else "conv2d_gemm_f16", **kws)
+        if quant:
+            assert np.array_equal(got, want), int((got != want).sum())
+        else:
+            assert np.allclose(got.astype(np.float32), want.astype(np.float32), rtol=FLOAT_RTOL, atol=2e-2)
+    assert len(np.unique(want)) > 4
+
+
+def test_conv2d_gemm_f16_matches_float32_arithmetic(oracle):
+    """The float16 kernel accumulates in float32 and rounds once: against a float64 convolution of the same
+    float16 operands the error stays within one float16 rounding of the result (plus the accumulation's)."""
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(7400)
+    n, c, oc, h, w = 2, 48, 64, 20, 20
+    x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=oc, kh=3, kw=3, stride=[1, 1], dil=[1, 1],
+                              pad=[1, 1, 1, 1], mult=0, mode="f16")
+    got = TC.gpu_conv2d(x, wt, b, want_kernel="conv2d_gemm_f16", **kws).astype(np.float64)
+    ref = F.conv2d(torch.from_numpy(x.astype(np.float64).reshape(n, c, h, w)),
+                   torch.from_numpy(wt.astype(np.float64).reshape(oc, c, 3, 3)),
+                   torch.from_numpy(b.astype(np.float64)), padding=1).numpy().reshape(-1)
+    assert np.all(np.abs(got - ref) <= np.abs(ref) * 2.0 ** -10 + 2e-3)
+
+
 DWP_GRID = [
     # (n, c, h, w, kh, kw, stride, dil, pad[l,r,t,b]): widths 14 / 7 / odd, 5x5 and 1x3 kernels,
     # dilation, asymmetric padding, a plane count that leaves a ragged last workgroup

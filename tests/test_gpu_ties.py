@@ -47,6 +47,8 @@ CONV_TIE_CASES = [
     ("conv2d_igemm_i8", dict(n=2, c=48, h=28, w=28, oc=96, k=3, stride=1, pad=1, mult=0), (15, 7)),
     ("conv2d_igemm_i8", dict(n=8, c=64, h=28, w=28, oc=80, k=3, stride=1, pad=1, mult=0), None),
     ("conv2d_igemm_i8_persistent", dict(n=10, c=64, h=28, w=28, oc=64, k=3, stride=1, pad=1, mult=0), None),
+    ("conv2d_gemm_i8", dict(n=2, c=40, h=16, w=16, oc=40, k=3, stride=1, pad=1, mult=0, groups=2), (15, 7)),
+    ("conv2d_gemm_i8", dict(n=16, c=48, h=48, w=48, oc=48, k=3, stride=2, pad=1, mult=0, groups=2), None),
     ("conv2d_im2col_i8", dict(n=3, c=3, h=33, w=31, oc=32, k=3, stride=2, pad=1, mult=0), (15, 7)),
     ("conv2d_im2col_i8", dict(n=12, c=1, h=28, w=28, oc=20, k=5, stride=1, pad=0, mult=0), None),
     ("dwconv3x3_i8", dict(n=2, c=8, h=16, w=16, oc=8, k=3, stride=1, pad=1, mult=1), (15, 7)),
@@ -67,7 +69,8 @@ def test_conv_epilogues_round_ties_to_even(oracle, ci, mode, monkeypatch):
     rng = np.random.default_rng(9000 + ci)
     u8 = mode == "u8"
     n, c, h, w, oc, k, stride, pad, dm = (g[key] for key in ("n", "c", "h", "w", "oc", "k", "stride", "pad", "mult"))
-    icg = 1 if dm else c
+    groups = g.get("groups", 0)
+    icg = 1 if dm else c // max(groups, 1)
     zx, zw, zo = (128, 120, 101) if u8 else (-3, 0, 7)
     ax, aw = amp if amp else (None, None)
     x, wt = _operands(rng, u8, ax, aw, n * c * h * w, oc * icg * k * k, zx, zw)
@@ -76,7 +79,7 @@ def test_conv_epilogues_round_ties_to_even(oracle, ci, mode, monkeypatch):
     acc = F.conv2d(torch.from_numpy(x.reshape(n, c, h, w).astype(np.float64) - zx),
                    torch.from_numpy(wt.reshape(oc, icg, k, k).astype(np.float64) - zw),
                    torch.from_numpy(b.astype(np.float64)), stride=stride, padding=pad,
-                   groups=c if dm else 1).numpy().astype(np.int64)
+                   groups=c if dm else max(groups, 1)).numpy().astype(np.int64)
     e = max(3, int(np.round(np.log2(max(acc.std(), 1.0) / 12.0))))   # ~12 output codes of spread
     m = _multipliers(not u8, oc, e)
     out_h, out_w = acc.shape[2], acc.shape[3]
@@ -84,6 +87,8 @@ def test_conv_epilogues_round_ties_to_even(oracle, ci, mode, monkeypatch):
                stride=[stride, stride], dilation=[1, 1], pad_left=pad, pad_top=pad, multiplier=dm,
                in_dtype=0 if u8 else 1, w_dtype=0 if u8 else 1, out_dtype=0 if u8 else 1, in_q=(0.5, zx),
                w_q=(float(2 * m[0]), zw, None) if u8 else (1.0, 0, (2 * m).astype(np.float32)), out_q=(1.0, zo))
+    if groups:
+        kws["groups"] = groups
     qlo, qhi = (0, 255) if u8 else (-128, 127)
     ties = sum(_count_ties(oracle, acc[:, ch], float(m[ch]), qlo, qhi, zo) for ch in range(oc))
     assert ties >= 10, (ties, e)

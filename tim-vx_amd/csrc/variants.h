@@ -47,6 +47,9 @@ int DwPwSetup(tvx_op* op, const tvx_conv2d_desc* dw, const void* dw_w, const voi
               const std::vector<int32_t>& dw_mult, const std::vector<int32_t>& dw_shift, int dw_lo, int dw_hi,
               const tvx_conv2d_desc* pw, const void* pw_w, const void* pw_b);
 
+// convolution as a GEMM over gathered windows: grouped, dilated, float16 (conv_gemm.hip)
+int ConvGemmSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
+
 // generic (kernels_generic.hip)
 int ConvGenericSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 int FcGenericSetup(tvx_op*, const tvx_fc_desc*, const void*, const void*);
