@@ -296,7 +296,8 @@ def time_workload(wl, steps, warmup, ring_bytes=0):
 
 KERNEL_SOURCES = {"conv2d_igemm_i8": "conv_igemm_i8.hip", "conv2d_igemm_i8_persistent": "conv_igemm_i8.hip",
                   "fc_mfma_i8_256x256x128": "fc_mfma_i8.hip", "fc_mfma_f16_256x256x64": "fc_mfma_i8.hip",
-                  "dwconv3x3_i8": "dwconv3x3_i8.hip", "pwconv_i8": "pwconv_i8.hip", "dwconv3x3_pwconv_i8": "dwpw_i8.hip", "pool2d_rows_i8": "pool2d_i8.hip"}
+                  "dwconv3x3_i8": "dwconv3x3_i8.hip", "pwconv_i8": "pwconv_i8.hip", "dwconv3x3_pwconv_i8": "dwpw_i8.hip", "pool2d_rows_i8": "pool2d_i8.hip",
+                  "conv2d_gemm_i8": "conv_gemm.hip", "conv2d_gemm_f16": "conv_gemm.hip"}
 
 
 def kernel_source_sha256(kernel_name):
@@ -465,7 +466,8 @@ def main():
         line["roofline"]["traffic_stale"] = True
     if not args.no_extra:
         extra = {}
-        for make in (fc_cfg5, fc_cfg5_f16, dw_cfg3a, pw_cfg3b, dwpw_cfg3, conv_cfg2_b256, pool_3x3_s2, pool_lenet_b256, pool_global_avg):
+        for make in (fc_cfg5, fc_cfg5_f16, dw_cfg3a, pw_cfg3b, dwpw_cfg3, conv_cfg2_b256, conv_f16, conv_grouped, pool_3x3_s2,
+                     pool_lenet_b256, pool_global_avg):
             w2 = make(T, rng)
             steps2 = max(5, min(args.steps, 50))
             wall2, k2 = time_workload(w2, steps2, min(args.warmup, 5))

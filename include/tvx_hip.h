@@ -229,6 +229,23 @@ int tvx_conv2d_dw_pw_create(const tvx_conv2d_desc* dw, const void* dw_weights_ho
                             const tvx_conv2d_desc* pw, const void* pw_weights_host, const void* pw_bias_host,
                             const tvx_eltwise_desc* add, int conv_operand, tvx_op** op);
 
+/* ---- an inverted-residual block: 1x1 Conv2d, depthwise 3x3 Conv2d, 1x1 Conv2d (+ Add) in one kernel ---- */
+/* Three (four) nodes of the reference's graph (vxConvolutionLayer: kernel/vx/convolutional.c:504-582, and
+ * vxTensorAdd behind them) whose two intermediate tensors have no other reader - the chain the closed driver
+ * merges at verification (src/tim/vx/internal/src/vsi_nn_graph.c:1591-1603). The result is, bit for bit,
+ * what the operators give one after the other: each intermediate is quantized to its own tensor (out_scale /
+ * out_zp, clamped by the stage's activation) before the next stage reads it, but neither reaches memory.
+ * `expand`, `dw` and `project` describe the convolutions as for tvx_conv2d_create (each stage's input is the
+ * previous stage's output); `add` (may be NULL) is the residual Add behind the projection as in
+ * tvx_conv2d_add_create, its other operand going in as in1 of tvx_op_run. Returns TVX_E_UNSUPPORTED when no
+ * kernel fuses this block (the kernel covers feature maps 28, 14 or 7 columns wide, SAME depthwise padding,
+ * at most 160 input and 320 output channels, and by default claims only the 14-column stride-1 blocks, where
+ * it is faster than the three launches; the caller then creates the operators one by one). */
+int tvx_mbconv_create(const tvx_conv2d_desc* expand, const void* expand_weights_host, const void* expand_bias_host,
+                      const tvx_conv2d_desc* dw, const void* dw_weights_host, const void* dw_bias_host,
+                      const tvx_conv2d_desc* project, const void* project_weights_host, const void* project_bias_host,
+                      const tvx_eltwise_desc* add, int conv_operand, tvx_op** op);
+
 /* ---- DeConv2d (transposed convolution) ----------------------------------------------- */
 /* Replaces vxDeconvolutionLayer (src/tim/vx/ops/deconv.cc:45-79,
  * src/tim/vx/internal/src/ops/vsi_nn_op_deconvolution.c:217-218,398-497). Same descriptor as

@@ -116,6 +116,8 @@ def lib():
         L.tvx_deconv2d_create.argtypes = [C.POINTER(Conv2dDesc), vp, vp, C.POINTER(vp)]
         L.tvx_conv2d_dw_pw_create.argtypes = [C.POINTER(Conv2dDesc), vp, vp, C.POINTER(Conv2dDesc), vp, vp,
                                               C.POINTER(EltwiseDesc), C.c_int, C.POINTER(vp)]
+        L.tvx_mbconv_create.argtypes = [C.POINTER(Conv2dDesc), vp, vp, C.POINTER(Conv2dDesc), vp, vp, C.POINTER(Conv2dDesc), vp, vp,
+                                        C.POINTER(EltwiseDesc), C.c_int, C.POINTER(vp)]
         L.tvx_fully_connected_create.argtypes = [C.POINTER(FcDesc), vp, vp, C.POINTER(vp)]
         L.tvx_pool2d_create.argtypes = [C.POINTER(Pool2dDesc), C.POINTER(vp)]
         L.tvx_activation_create.argtypes = [C.POINTER(EltwiseDesc), C.POINTER(vp)]
@@ -189,6 +191,16 @@ def conv2d_dw_pw_create(dw_desc, dw_weights, dw_bias, pw_desc, pw_weights, pw_bi
     check(lib().tvx_conv2d_dw_pw_create(C.byref(dw_desc), _host_ptr(dw_weights), _host_ptr(dw_bias),
                                         C.byref(pw_desc), _host_ptr(pw_weights), _host_ptr(pw_bias),
                                         C.byref(add_desc) if add_desc is not None else None, conv_operand, C.byref(h)))
+    return Op(h)
+
+
+def mbconv_create(expand, expand_w, expand_b, dw, dw_w, dw_b, project, project_w, project_b, add_desc=None, conv_operand=0):
+    """1x1 expansion, depthwise 3x3 and 1x1 projection (+ residual Add) as one operator."""
+    h = C.c_void_p()
+    check(lib().tvx_mbconv_create(C.byref(expand), _host_ptr(expand_w), _host_ptr(expand_b),
+                                  C.byref(dw), _host_ptr(dw_w), _host_ptr(dw_b),
+                                  C.byref(project), _host_ptr(project_w), _host_ptr(project_b),
+                                  C.byref(add_desc) if add_desc is not None else None, conv_operand, C.byref(h)))
     return Op(h)
 
 

@@ -486,6 +486,72 @@ int tvx_conv2d_dw_pw_create(const tvx_conv2d_desc* dw, const void* dw_w, const v
   return TVX_OK;
 }
 
+int tvx_mbconv_create(const tvx_conv2d_desc* expand, const void* expand_w, const void* expand_b,
+                      const tvx_conv2d_desc* dw, const void* dw_w, const void* dw_b,
+                      const tvx_conv2d_desc* project, const void* project_w, const void* project_b,
+                      const tvx_eltwise_desc* add, int conv_operand, tvx_op** out) {
+  static const char* const fn = "tvx_mbconv_create";
+  if (!expand || !dw || !project || !out) return SetError(TVX_E_INVALID, "%s: null argument", fn);
+  *out = nullptr;
+  if (add && conv_operand != 1 && conv_operand != 2) return SetError(TVX_E_INVALID, "%s: conv_operand must be 1 or 2", fn);
+  const tvx_conv2d_desc* stages[3] = {expand, dw, project};
+  const void* weights[3] = {expand_w, dw_w, project_w};
+  for (int i = 0; i < 3; ++i) {
+    const tvx_conv2d_desc* d = stages[i];
+    if (!IsQuant(d->in_dtype) || !IsQuant(d->out_dtype) || !weights[i])
+      return SetError(TVX_E_UNSUPPORTED, "%s: quantized tensors and constant weights only", fn);
+    if (!d->in_w || !d->in_h || !d->in_c || !d->batch || !d->out_w || !d->out_h || !d->out_c)
+      return SetError(TVX_E_INVALID, "%s: zero extent", fn);
+    int s = CheckOperandTypes(d->in_dtype, d->w_dtype, d->out_dtype, fn);
+    if (s == TVX_OK) s = CheckConvZeroPoints(d->in_dtype, d->in_zp, d->w_dtype, d->w_zp, d->w_scales != nullptr, d->out_dtype, d->out_zp, fn);
+    if (s != TVX_OK) return s;
+  }
+  if (dw->multiplier != 1 || dw->out_c != dw->in_c)
+    return SetError(TVX_E_INVALID, "%s: the second convolution must be depthwise with multiplier 1", fn);
+  if (add) {
+    if (add->dtype != project->out_dtype || !(add->a_scale > 0.f) || !(add->b_scale > 0.f) || !(add->out_scale > 0.f))
+      return SetError(TVX_E_UNSUPPORTED, "%s: the Add must be of the block's output type", fn);
+    const float conv_scale = conv_operand == 1 ? add->a_scale : add->b_scale;
+    const int32_t conv_zp = conv_operand == 1 ? add->a_zp : add->b_zp;
+    if (conv_scale != project->out_scale || conv_zp != project->out_zp)
+      return SetError(TVX_E_INVALID, "%s: the Add's operand %d is not quantized like the projection's output", fn, conv_operand);
+    int s = CheckZeroPoint(add->dtype, add->a_zp, fn, "Add operand");
+    if (s == TVX_OK) s = CheckZeroPoint(add->dtype, add->b_zp, fn, "Add operand");
+    if (s == TVX_OK) s = CheckZeroPoint(add->dtype, add->out_zp, fn, "Add output");
+    if (s != TVX_OK) return s;
+  }
+  int s = NoGpu();
+  if (s != TVX_OK) return s;
+  tvx_op* op = new (std::nothrow) tvx_op();
+  if (!op) return SetError(TVX_E_NOMEM, "%s: host allocation failed", fn);
+  op->kind = OP_CONV2D;
+  op->conv = *project;
+  op->conv.w_scales = nullptr;
+  if (add) {
+    op->elt = *add;
+    op->fused_add = conv_operand;
+  }
+  op->quantized = true;
+  op->has_const_weights = true;
+  op->w_zp = project->w_scales ? 0 : project->w_zp;
+  std::vector<int32_t> mult[2], shift[2];
+  MbStage st[2] = {{expand, expand_w, expand_b, &mult[0], &shift[0], 0, 0}, {dw, dw_w, dw_b, &mult[1], &shift[1], 0, 0}};
+  s = BuildRequantTables(project->out_c, project->in_scale, project->w_scale, project->w_scales, project->out_scale, &op->h_mult, &op->h_shift);
+  ActRange(project->out_dtype, project->out_scale, project->out_zp, project->activation, &op->act_lo, &op->act_hi);
+  for (int i = 0; i < 2 && s == TVX_OK; ++i) {
+    const tvx_conv2d_desc* d = st[i].desc;
+    s = BuildRequantTables(d->out_c, d->in_scale, d->w_scale, d->w_scales, d->out_scale, &mult[i], &shift[i]);
+    ActRange(d->out_dtype, d->out_scale, d->out_zp, d->activation, &st[i].lo, &st[i].hi);
+  }
+  if (s == TVX_OK) s = MbConvSetup(op, st[0], st[1], project, project_w, project_b);
+  if (s != TVX_OK) {
+    delete op;
+    return s == TVX_E_UNSUPPORTED ? SetError(TVX_E_UNSUPPORTED, "%s: no fused kernel for this block", fn) : s;
+  }
+  *out = op;
+  return TVX_OK;
+}
+
 int tvx_deconv2d_create(const tvx_conv2d_desc* d, const void* weights_host, const void* bias_host,
                         tvx_op** out) {
   if (!d || !out) return SetError(TVX_E_INVALID, "tvx_deconv2d_create: null argument");

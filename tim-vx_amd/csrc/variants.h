@@ -47,6 +47,19 @@ int DwPwSetup(tvx_op* op, const tvx_conv2d_desc* dw, const void* dw_w, const voi
               const std::vector<int32_t>& dw_mult, const std::vector<int32_t>& dw_shift, int dw_lo, int dw_hi,
               const tvx_conv2d_desc* pw, const void* pw_w, const void* pw_b);
 
+// an inverted-residual block - 1x1 expansion, depthwise 3x3, 1x1 projection (+ Add) - in one kernel (mbconv_i8.hip);
+// `op` carries the projection, the two stages in front of it come with their own tables
+struct MbStage {
+  const tvx_conv2d_desc* desc;
+  const void* w;
+  const void* b;
+  const std::vector<int32_t>* mult;
+  const std::vector<int32_t>* shift;
+  int32_t lo, hi;  // output clamp incl. the stage's activation
+};
+int MbConvSetup(tvx_op* op, const MbStage& expand, const MbStage& depthwise, const tvx_conv2d_desc* project,
+                const void* project_w, const void* project_b);
+
 // convolution as a GEMM over gathered windows: grouped, dilated, float16 (conv_gemm.hip)
 int ConvGemmSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 

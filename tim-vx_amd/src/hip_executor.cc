@@ -153,6 +153,31 @@ class HipExecutor : public Executor {
         fused_dwpw[op] = consumers[0].get();
       }
     }
+    // ---- inverted-residual plan: a 1x1 convolution (with its activation) whose TRANSIENT result only feeds the
+    // depthwise convolution of such a pair may become one operator with both
+    std::map<Operation*, Operation*> fused_block;  // expansion -> the depthwise convolution behind it
+    if (!std::getenv("TVX_NO_BLOCK_FUSION")) {  // tuning aid
+      for (Operation* op : graph->sorted_ops_) {
+        OpImpl* im = op->impl().get();
+        if (im->kind_ != OpKind::CONV2D || im->attrs_.multiplier != 0 || im->attrs_.conv_1d || fused_add.count(op)) continue;
+        auto fa = fused_act.find(op);
+        auto mid = fa != fused_act.end() ? fa->second->impl()->outputs_tensor_[0] : im->outputs_tensor_[0];
+        if (!(mid->GetSpec().attr_ & TensorAttribute::TRANSIENT)) continue;
+        auto consumers = graph->GetConsumersOp(mid);
+        if (consumers.size() != 1) continue;
+        Operation* dw = consumers[0].get();
+        auto fd = fused_dwpw.find(dw);
+        if (fd == fused_dwpw.end() || dw->impl()->inputs_tensor_[0] != mid) continue;
+        // the merged operator runs where the expansion stands: the residual operand has to exist by then
+        auto pad = fused_add.find(fd->second);
+        if (pad != fused_add.end()) {
+          auto other = pad->second.add->impl()->inputs_tensor_[pad->second.conv_operand == 1 ? 1 : 0];
+          auto oit = produced_at.find(other.get());
+          if (oit != produced_at.end() && oit->second >= produced_at[im->outputs_tensor_[0].get()]) continue;
+        }
+        fused_block[op] = dw;
+      }
+    }
     // ---- device storage: one buffer per tensor, Reshape outputs alias their input --
     for (Operation* op : graph->sorted_ops_) {
       OpImpl* im = op->impl().get();
@@ -185,6 +210,38 @@ class HipExecutor : public Executor {
       bool ok = true;
       switch (im->kind_) {
         case OpKind::CONV2D: {
+          // folded activation and output tensor of a convolution of the plan
+          auto folded = [&](Operation* c, int* c_act) {
+            *c_act = TVX_ACT_NONE;
+            TensorImpl* c_out = static_cast<TensorImpl*>(c->impl()->outputs_tensor_[0].get());
+            auto cf = fused_act.find(c);
+            if (cf != fused_act.end()) {
+              OpImpl* ca = cf->second->impl().get();
+              *c_act = ca->kind_ == OpKind::RELU ? TVX_ACT_RELU : TVX_ACT_RELU6;
+              c_out = static_cast<TensorImpl*>(ca->outputs_tensor_[0].get());
+            }
+            return c_out;
+          };
+          auto fb = fused_block.find(op);
+          if (fb != fused_block.end()) {
+            Operation* dw = fb->second;
+            Operation* pw = fused_dwpw[dw];
+            int dw_act, pw_act;
+            TensorImpl* dw_out = folded(dw, &dw_act);
+            TensorImpl* pw_out = folded(pw, &pw_act);
+            auto pad = fused_add.find(pw);
+            bool all = false;
+            ok = AddBlock(im, out, act, dw->impl().get(), dw_out, dw_act, pw->impl().get(), pw_out, pw_act,
+                          pad != fused_add.end() ? pad->second.add->impl().get() : nullptr,
+                          pad != fused_add.end() ? pad->second.conv_operand : 0, &all);
+            if (!ok) break;
+            if (all) {
+              skipped[dw] = true;  // (the activations folded into the three are skipped already)
+              skipped[pw] = true;
+              if (pad != fused_add.end()) skipped[pad->second.add] = true;
+              break;
+            }
+          }
           auto fd = fused_dwpw.find(op);
           if (fd != fused_dwpw.end()) {
             Operation* pw = fd->second;
@@ -388,6 +445,42 @@ class HipExecutor : public Executor {
     e->a_scale = ScaleOf(a0->spec_); e->a_zp = ZpOf(a0->spec_);
     e->b_scale = ScaleOf(a1->spec_); e->b_zp = ZpOf(a1->spec_);
     e->out_scale = ScaleOf(sum->spec_); e->out_zp = ZpOf(sum->spec_);
+    return true;
+  }
+
+  // Expansion, depthwise convolution and projection (+ residual Add) as one operator (tvx_mbconv_create). *fused
+  // says whether a kernel took the block; if not, nothing has been added and the caller goes on operator by operator.
+  bool AddBlock(OpImpl* ex_im, TensorImpl* ex_out, int ex_act, OpImpl* dw_im, TensorImpl* dw_out, int dw_act,
+                OpImpl* pw_im, TensorImpl* pw_out, int pw_act, OpImpl* add_im, int conv_operand, bool* fused) {
+    *fused = false;
+    TensorImpl* w[3];
+    TensorImpl* b[3];
+    OpImpl* ims[3] = {ex_im, dw_im, pw_im};
+    for (int i = 0; i < 3; ++i) {
+      w[i] = static_cast<TensorImpl*>(ims[i]->inputs_tensor_[1].get());
+      b[i] = ims[i]->inputs_tensor_.size() > 2 && !ims[i]->inputs_tensor_[2]->IsPlaceHolder()
+                 ? static_cast<TensorImpl*>(ims[i]->inputs_tensor_[2].get()) : nullptr;
+      if (!w[i]->IsConstTensor() || !w[i]->HostData() || (b[i] && (!b[i]->IsConstTensor() || !b[i]->HostData()))) return true;
+    }
+    const tvx_conv2d_desc ex = ConvDesc(ex_im, ex_out, ex_act, false);
+    const tvx_conv2d_desc dw = ConvDesc(dw_im, dw_out, dw_act, false);
+    const tvx_conv2d_desc pw = ConvDesc(pw_im, pw_out, pw_act, false);
+    tvx_eltwise_desc e{};
+    if (add_im && !AddDesc(add_im, &e)) return true;
+    tvx_op* op = nullptr;
+    const int st = tvx_mbconv_create(&ex, w[0]->HostData(), b[0] ? b[0]->HostData() : nullptr, &dw, w[1]->HostData(),
+                                     b[1] ? b[1]->HostData() : nullptr, &pw, w[2]->HostData(),
+                                     b[2] ? b[2]->HostData() : nullptr, add_im ? &e : nullptr, conv_operand, &op);
+    if (st == TVX_E_UNSUPPORTED) return true;
+    if (st != TVX_OK) return Fail("tvx_mbconv_create");
+    *fused = true;
+    TensorImpl* x = static_cast<TensorImpl*>(ex_im->inputs_tensor_[0].get());
+    if (add_im) {
+      TensorImpl* other = static_cast<TensorImpl*>(add_im->inputs_tensor_[conv_operand == 1 ? 1 : 0].get());
+      Push(op, ex_im, x, other, static_cast<TensorImpl*>(add_im->outputs_tensor_[0].get()));
+    } else {
+      Push(op, ex_im, x, nullptr, pw_out);
+    }
     return true;
   }
 
