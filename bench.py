@@ -494,6 +494,9 @@ def main():
             "mfma_i8_tops_zero_operands": round(T.calibrate_mfma_i8(False), 0),
             "mfma_i8_tops_random_operands": round(T.calibrate_mfma_i8(True), 0),
             "copy_read_plus_write_gbs": round(T.calibrate_copy(), 0),
+            # the same copy kernel on the depthwise workload's bytes (12.8 MB in, 12.8 MB out), launched back to
+            # back in place: what a launch of that size can reach with the per-launch floor under it
+            "copy_12p8MB_read_plus_write_gbs": round(T.calibrate_copy(12845056, 50), 0),
         }
         line["extra"] = extra
     print(json.dumps(line))
