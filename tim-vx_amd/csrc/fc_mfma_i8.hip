@@ -211,7 +211,8 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   // up in the memory pipeline with the wavefront waiting behind them). The weight registers
   // of this k-step are refilled (for k-tile kt + 3) only after the MFMAs that read them
   // were issued.
-  auto k_step = [&](int kt, int kk, v4i* fx, v4i* w_slot, int kt_max) {
+  auto k_step = [&](auto prefetch, int kt, int kk, v4i* fx, v4i* w_slot, int kt_max) {
+    constexpr bool kPrefetch = decltype(prefetch)::value;
     if (X_U8) {
 #pragma unroll
       for (int t = 0; t < 8; ++t) fx[t] ^= static_cast<int>(0x80808080);
@@ -228,11 +229,11 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
 #pragma unroll
       for (int mb = 0; mb < 8; ++mb) {
         acc[nb][mb] = Mfma(w_slot[nb * 4 + kk], fx[mb], acc[nb][mb]);
-        if (mb == 3) {
+        if (kPrefetch && mb == 3) {
           dma_piece(kt + 3, kk * 2 + nb);
           __builtin_amdgcn_sched_barrier(0);
         }
-        if (mb == 7) {
+        if (kPrefetch && mb == 7) {
           __builtin_amdgcn_sched_barrier(0);
           w_piece(kt + 3, nb, kk, w_slot[nb * 4 + kk], kt_max);
           __builtin_amdgcn_sched_barrier(0);
@@ -248,29 +249,35 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   // - the activations and weights of k-tile kt + 1 - has landed.
   const int kt_max = k_tiles_padded(a.K) - 1;
   v4i fxa[8], fxb[8];
-  auto k_tile = [&](int kt, v4i* w_slot) {
+  // `prefetch`: the k-tile issues its share of k-tile kt + 3 (all rounds but the last, which is peeled off so that
+  // no fetch is in flight when the loop ends: registers named by an unfinished fetch would otherwise have to be
+  // kept out of the epilogue's hands). `in_flight`: memory operations that may still be on their way at the
+  // barrier (28 while prefetching; 16, 0, 0 in the last round). `last`: no fragments of a next k-tile.
+  auto k_tile = [&](auto prefetch, auto in_flight, auto last, int kt, v4i* w_slot) {
     load_frags(kt, 1, fxb);
     asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
-    k_step(kt, 0, fxa, w_slot, kt_max);
+    k_step(prefetch, kt, 0, fxa, w_slot, kt_max);
     __builtin_amdgcn_sched_barrier(0);
     load_frags(kt, 2, fxa);
     asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
-    k_step(kt, 1, fxb, w_slot, kt_max);
+    k_step(prefetch, kt, 1, fxb, w_slot, kt_max);
     __builtin_amdgcn_sched_barrier(0);
     load_frags(kt, 3, fxb);
     asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
-    k_step(kt, 2, fxa, w_slot, kt_max);
+    k_step(prefetch, kt, 2, fxa, w_slot, kt_max);
     __builtin_amdgcn_sched_barrier(0);
-    asm volatile("s_waitcnt vmcnt(28) lgkmcnt(0)" ::: "memory");
+    if constexpr (decltype(in_flight)::value == 28) asm volatile("s_waitcnt vmcnt(28) lgkmcnt(0)" ::: "memory");
+    else if constexpr (decltype(in_flight)::value == 16) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     // the bare barrier: __syncthreads() adds a fence that waits for every memory operation in
     // flight - the whole prefetch - at every k-tile
     __builtin_amdgcn_s_barrier();
-    load_frags(kt + 1, 0, fxa);
+    if constexpr (!decltype(last)::value) load_frags(kt + 1, 0, fxa);
     __builtin_amdgcn_sched_barrier(0);
-    k_step(kt, 3, fxb, w_slot, kt_max);
+    k_step(prefetch, kt, 3, fxb, w_slot, kt_max);
     __builtin_amdgcn_sched_barrier(0);
   };
   // prologue: k-tiles 0, 1, 2 in the order every later k-tile uses (8 x (activation piece,
@@ -291,24 +298,22 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   load_frags(0, 0, fxa);
   // the loop runs whole rounds of three k-tiles (the weight slots are named registers); the
   // packed weights are zero-padded to that count and the activations past K read zeros
-  for (int kt = 0; kt <= kt_max; kt += 3) {
-    k_tile(kt, wr[0]);
-    k_tile(kt + 1, wr[1]);
-    k_tile(kt + 2, wr[2]);
+  {
+    using std::integral_constant;
+    const integral_constant<bool, true> yes;
+    const integral_constant<bool, false> no;
+    int kt = 0;
+    for (; kt + 3 <= kt_max; kt += 3) {
+      k_tile(yes, integral_constant<int, 28>(), no, kt, wr[0]);
+      k_tile(yes, integral_constant<int, 28>(), no, kt + 1, wr[1]);
+      k_tile(yes, integral_constant<int, 28>(), no, kt + 2, wr[2]);
+    }
+    // the last round: its k-tiles were fetched by the round before (or the prologue); nothing new is fetched
+    k_tile(no, integral_constant<int, 16>(), no, kt, wr[0]);
+    k_tile(no, integral_constant<int, 0>(), no, kt + 1, wr[1]);
+    k_tile(no, integral_constant<int, 0>(), yes, kt + 2, wr[2]);
   }
-  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // nothing may land in the epilogue's staging tile
-  // The last round's prefetches target registers whose values nobody reads. To the compiler
-  // such registers are free the moment the fetch is "done" (it cannot see that the data is
-  // still on its way) and it would move epilogue arithmetic into them above the wait. Naming
-  // them as operands after the wait keeps them occupied until everything has landed.
-#define TVX_KEEP8(v) \
-  asm volatile("" : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]))
-  TVX_KEEP8(wr[0]);
-  TVX_KEEP8(wr[1]);
-  TVX_KEEP8(wr[2]);
-  TVX_KEEP8(fxa);
-  TVX_KEEP8(fxb);
-#undef TVX_KEEP8
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // (nothing is in flight here; the staging tile is about to be written)
   __syncthreads();  // the epilogue reuses the LDS
 
   // ---- epilogue ---------------------------------------------------------------
@@ -324,6 +329,7 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
       if (round) __syncthreads();
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
+        __builtin_amdgcn_sched_barrier(0);  // (one feature quad at a time, as below)
         const int n = n0 + wave * 64 + round * 32 + 8 * g + 4 * frag_half;
         float b4[4];
 #pragma unroll
@@ -372,6 +378,8 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
     for (int nb = 0; nb < 2; ++nb) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
+        // (one feature quad at a time: hoisting the table reads of all eight quads costs more registers than there are)
+        __builtin_amdgcn_sched_barrier(0);
         const int nl = wave * 64 + nb * 32 + 8 * g + 4 * frag_half;
         const int n = n0 + nl;
         int b4[4];
