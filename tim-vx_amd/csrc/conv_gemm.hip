@@ -4,8 +4,9 @@
 // those (reference: src/tim/vx/internal/src/ops/vsi_nn_op_conv2d.c:35-118, vsi_nn_op_grouped_conv2d.c).
 //
 // A workgroup owns 128 consecutive output pixels of one image and 32 or 64 output channels of one group.
-// The reduction runs over (channel, ky, kx) in chunks of 64 bytes per pixel row: every thread gathers half
-// a chunk of one pixel's window into registers (the next chunk's loads are in flight under the MFMAs),
+// The reduction runs tap by tap (a tap's channels padded to whole half-chunks) in chunks of 64 bytes per pixel
+// row: every thread gathers half a chunk - 32 bytes of one tap, walking the channel planes from one base
+// address under one validity test - into registers (the next chunk's loads are in flight under the MFMAs),
 // the chunk lands in LDS as [pixel][k], the weights - packed at creation into the very LDS image - are
 // copied beside it, and each wavefront multiplies its 32 pixels with all the workgroup's channels
 // (v_mfma_i32_32x32x32_i8 / v_mfma_f32_32x32x16_f16: both read 16 bytes per lane and step 32 bytes of a row).
@@ -36,7 +37,7 @@ struct GemmArgs {
   const uint8_t* x;
   uint8_t* y;
   const uint8_t* wpk;    // [group][channel tile][chunk][32 * OT rows][64 bytes]
-  const int2* tab;       // per k of a group, padded to whole chunks: {element offset, dy | dx << 8 | valid << 16}
+  const int2* tab;       // per half-chunk (32 bytes of one tap's channels): {element offset of its first channel at the tap, dy | dx << 8 | real channels << 16}
   const int32_t* biasf;  // quantized: bias with the zero-point terms folded in, per padded output channel
   const float* biasfl;   // float16: the bias
   const tvx_v4i* rq;
@@ -103,28 +104,32 @@ __global__ void __launch_bounds__(kThreads) ConvGemmKernel(GemmArgs a) {
   const int origin = ih0 * a.W + iw0;  // may be negative: only added to offsets of taps inside the image
   const uint8_t* wsrc = a.wpk + (static_cast<size_t>(group) * a.tiles_per_group + tile) * a.chunks * (OT * 32 * kChunkBytes);
 
+  // The reduction runs tap by tap, a tap's channels padded to whole half-chunks: the 32 bytes a thread gathers
+  // belong to one tap (one validity test, one base address) and walk the channel planes.
   uint32_t g[8];  // the 32 bytes of this thread's pixel row and chunk half
+  const int plane_i = a.H * a.W;
   auto gather = [&](int chunk) {
-    const int2* t = a.tab + (chunk * 2 + half) * kPerHalf;
+    const int2 e = a.tab[chunk * 2 + half];  // (the same for the whole wavefront)
+    const int dy = e.y & 0xff, dx = (e.y >> 8) & 0xff;
+    const int nreal = e.y >> 16;              // real channels in this half-chunk (the rest is padding)
+    const bool inside = p_live && static_cast<unsigned>(ih0 + dy) < static_cast<unsigned>(a.H) &&
+                        static_cast<unsigned>(iw0 + dx) < static_cast<unsigned>(a.W);
+    const int base = inside ? origin + e.x : 0;  // (outside: any readable element, masked below)
 #pragma unroll
     for (int i = 0; i < kPerHalf; i += 4 / ESZ) {
       uint32_t word = 0;
 #pragma unroll
       for (int j = 0; j < 4 / ESZ; ++j) {
-        const int2 e = t[i + j];  // (the same for the whole wavefront)
-        const int dy = e.y & 0xff, dx = (e.y >> 8) & 0xff;
-        const bool real = (e.y >> 16) != 0;
-        const bool inside = static_cast<unsigned>(ih0 + dy) < static_cast<unsigned>(a.H) &&
-                            static_cast<unsigned>(iw0 + dx) < static_cast<unsigned>(a.W);
+        const int c = max(0, min(i + j, nreal - 1));  // (padding channels re-read a real one, masked below)
         uint32_t v;
         if (F16) {
-          v = 0;
-          if (real && inside && p_live) v = reinterpret_cast<const uint16_t*>(xg)[origin + e.x];
+          v = reinterpret_cast<const uint16_t*>(xg)[base + c * plane_i];
+          if (!inside || i + j >= nreal) v = 0;
           word |= v << (16 * j);
         } else {
-          v = static_cast<uint32_t>(a.pad_fill4) & 0xff;
-          if (real && inside && p_live) v = xg[origin + e.x] ^ (static_cast<uint32_t>(a.xor_mask4) & 0xff);
-          if (!real || !p_live) v = 0;
+          v = xg[base + c * plane_i] ^ (static_cast<uint32_t>(a.xor_mask4) & 0xff);
+          if (!inside) v = static_cast<uint32_t>(a.pad_fill4) & 0xff;
+          if (i + j >= nreal || !p_live) v = 0;
           word |= v << (8 * j);
         }
       }
@@ -271,7 +276,10 @@ int ConvGemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, cons
   if (in_elems >= (1ull << 31) || hw >= (1ull << 31) || d->batch > 65535) return TVX_E_UNSUPPORTED;
   const int K = static_cast<int>(K64);
   const int kc = kChunkBytes / esz;  // window elements per chunk
-  const int chunks = (K + kc - 1) / kc;
+  const int kh = kc / 2;             // ... per half-chunk: what one thread gathers, all of one tap
+  const int cpt = (icg + kh - 1) / kh * kh;  // a tap's channels, padded to whole half-chunks
+  const int halves = taps * cpt / kh;
+  const int chunks = (halves + 1) / 2;
   const int ot = ocg <= 32 ? 1 : 2;
   const int tiles = (ocg + 32 * ot - 1) / (32 * ot);
   if (static_cast<uint64_t>(groups) * tiles > 65535) return TVX_E_UNSUPPORTED;
@@ -284,14 +292,15 @@ int ConvGemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, cons
   a.act = d->activation;
   a.aligned4 = hw % 4 == 0;
 
-  // ---- the window table: element offset and tap position of every k, the same for all groups ----
-  std::vector<int32_t> tab(static_cast<size_t>(chunks) * kc * 2, 0);
-  for (int k = 0; k < K; ++k) {
-    const int c = k / taps, t = k % taps;
+  // ---- the window table, the same for all groups: per half-chunk its tap and first channel ----
+  std::vector<int32_t> tab(static_cast<size_t>(chunks) * 2 * 2, 0);
+  for (int h = 0; h < halves; ++h) {
+    const int t = h * kh / cpt, c0 = h * kh % cpt;
     const int dy = (t / static_cast<int>(d->k_w)) * static_cast<int>(d->dilation_h);
     const int dx = (t % static_cast<int>(d->k_w)) * static_cast<int>(d->dilation_w);
-    tab[2 * k] = c * a.H * a.W + dy * a.W + dx;
-    tab[2 * k + 1] = dy | dx << 8 | 1 << 16;
+    const int nreal = std::max(0, std::min(kh, icg - c0));
+    tab[2 * h] = c0 * a.H * a.W + dy * a.W + dx;
+    tab[2 * h + 1] = dy | dx << 8 | nreal << 16;
   }
 
   // ---- weights [oc][c][ky][kx] -> per group, channel tile and chunk the LDS image [32 * OT rows][64 bytes] ----
@@ -313,9 +322,10 @@ int ConvGemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, cons
       const int tile = ocl / rows, r = ocl % rows;
       const size_t slot = (static_cast<size_t>(g) * tiles + tile) * rows + r;
       int64_t sw = 0;
-      for (int k = 0; k < K; ++k) {
-        const size_t at = (((static_cast<size_t>(g) * tiles + tile) * chunks + k / kc) * rows + r) * kChunkBytes +
-                          static_cast<size_t>(k % kc) * esz;
+      for (int k = 0; k < K; ++k) {  // the weight tensor's own order: [oc][c][ky][kx]
+        const int kp = (k % taps) * cpt + k / taps;  // position in the tap-major, channel-padded reduction
+        const size_t at = (((static_cast<size_t>(g) * tiles + tile) * chunks + kp / kc) * rows + r) * kChunkBytes +
+                          static_cast<size_t>(kp % kc) * esz;
         if (f16) {
           std::memcpy(&packed[at], src + (static_cast<size_t>(oc) * K + k) * 2, 2);
         } else {
