@@ -147,6 +147,8 @@ def run_graphs(graphs, workdir, bench=None, timeout=600, env=None):
             info.setdefault(f[1], {}).update(run_ms=float(f[2]), device_ms=float(f[3]))
         elif f[0] == "opbench":  # per-operator device time (env TVX_RUNTIME_PROFILE=ops)
             info.setdefault(f[1], {}).setdefault("ops_us", []).append((f[3], float(f[4])))
+            if len(f) > 5:  # the bytes of the operator's operands and result
+                info[f[1]].setdefault("ops_bytes", []).append(int(f[5]))
     cursor = {}
     for g in graphs:
         name = g["test"].replace(" ", "_")

@@ -28,6 +28,7 @@ namespace {
 double g_last_device_ms = 0.0;
 // Per-operator device time of the most recent Graph::Run() (TVX_RUNTIME_PROFILE=ops): name and microseconds.
 std::vector<std::pair<std::string, double>> g_last_op_us;
+std::vector<uint64_t> g_last_op_bytes;
 
 int DtypeCode(DataType t) {
   switch (t) {
@@ -56,6 +57,7 @@ struct Step {
   TensorImpl* in2 = nullptr;  // run-time bias
   TensorImpl* out = nullptr;
   std::string name;
+  uint64_t bytes = 0;  // tensor bytes the step has to move: its operands and its result
 };
 
 class HipExecutor : public Executor {
@@ -343,10 +345,12 @@ class HipExecutor : public Executor {
     }
     if (profile_ops_) {
       g_last_op_us.clear();
+      g_last_op_bytes.clear();
       for (size_t i = 0; i < steps_.size(); ++i) {
         float ms = 0.f;
         if (tvx_event_elapsed_ms(events_[i], events_[i + 1], &ms) != TVX_OK) return Fail("event");
         g_last_op_us.emplace_back(steps_[i].name, static_cast<double>(ms) * 1e3);
+        g_last_op_bytes.push_back(steps_[i].bytes);
       }
     }
     for (auto& t : graph->outputs_tensor_) {
@@ -382,6 +386,8 @@ class HipExecutor : public Executor {
     s.in2 = in2;
     s.out = out;
     s.name = std::string(OpKindName(im->kind_)) + " (" + tvx_op_kernel_name(op) + ")";
+    for (TensorImpl* t : {in0, in1, in2, out})
+      if (t) s.bytes += t->HostBytes();
     VSILOGI("uid %u -> %s", im->uid_, s.name.c_str());
     steps_.push_back(s);
   }
@@ -741,3 +747,4 @@ extern "C" double tvx_runtime_last_device_ms(void) { return tim::vx::g_last_devi
 extern "C" int tvx_runtime_last_op_count(void) { return static_cast<int>(tim::vx::g_last_op_us.size()); }
 extern "C" const char* tvx_runtime_last_op_name(int i) { return tim::vx::g_last_op_us[static_cast<size_t>(i)].first.c_str(); }
 extern "C" double tvx_runtime_last_op_us(int i) { return tim::vx::g_last_op_us[static_cast<size_t>(i)].second; }
+extern "C" unsigned long long tvx_runtime_last_op_bytes(int i) { return tim::vx::g_last_op_bytes[static_cast<size_t>(i)]; }

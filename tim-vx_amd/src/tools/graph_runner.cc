@@ -22,7 +22,7 @@
 //   end
 // For every `run` one line goes to stdout: "ok <name> <offset> <bytes>" or
 // "fail <name> <stage>"; for every `bench`: "bench <name> <ms per Run> <ms per Run, device part>" and, with
-// TVX_RUNTIME_PROFILE=ops in the environment, "opbench <name> <index> <operator> <microseconds>" per operator.
+// TVX_RUNTIME_PROFILE=ops in the environment, "opbench <name> <index> <operator> <microseconds> <operand + result bytes>" per operator.
 #include <algorithm>
 #include <memory>
 #include <chrono>
@@ -47,6 +47,7 @@ extern "C" double tvx_runtime_last_device_ms(void);
 extern "C" int tvx_runtime_last_op_count(void);
 extern "C" const char* tvx_runtime_last_op_name(int i);
 extern "C" double tvx_runtime_last_op_us(int i);
+extern "C" unsigned long long tvx_runtime_last_op_bytes(int i);
 
 using namespace tim::vx;
 
@@ -412,7 +413,8 @@ int main(int argc, char** argv) {
       for (size_t o = 0; o < op_us.size(); ++o) {
         std::string op_name = tvx_runtime_last_op_name(static_cast<int>(o));
         for (char& c : op_name) if (c == ' ') c = '_';
-        std::printf("opbench %s %zu %s %.3f\n", name.c_str(), o, op_name.c_str(), op_us[o] / iters);
+        std::printf("opbench %s %zu %s %.3f %llu\n", name.c_str(), o, op_name.c_str(), op_us[o] / iters,
+                    tvx_runtime_last_op_bytes(static_cast<int>(o)));
       }
       std::fflush(stdout);
     } else if (rec == "end") {
