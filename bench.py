@@ -297,7 +297,8 @@ def time_workload(wl, steps, warmup, ring_bytes=0):
 KERNEL_SOURCES = {"conv2d_igemm_i8": "conv_igemm_i8.hip", "conv2d_igemm_i8_persistent": "conv_igemm_i8.hip",
                   "fc_mfma_i8_256x256x128": "fc_mfma_i8.hip", "fc_mfma_f16_256x256x64": "fc_mfma_i8.hip",
                   "dwconv3x3_i8": "dwconv3x3_i8.hip", "pwconv_i8": "pwconv_i8.hip", "dwconv3x3_pwconv_i8": "dwpw_i8.hip", "pool2d_rows_i8": "pool2d_i8.hip",
-                  "conv2d_gemm_i8": "conv_gemm.hip", "conv2d_gemm_f16": "conv_gemm.hip"}
+                  "conv2d_gemm_i8": "conv_gemm.hip", "conv2d_gemm_f16": "conv_gemm.hip",
+                  "avgpool_plane_i8": "kernels_generic.hip"}
 
 
 def kernel_source_sha256(kernel_name):
@@ -441,7 +442,7 @@ def main():
         """Measured HBM bytes per launch of this kernel on this workload (profiles/traffic.json), or None. The
         record carries the hash of the kernel's source file at the time of the measurement: when the source has
         changed since, the figure is still reported but flagged (stderr and `traffic_stale`)."""
-        rec = tmap.get(w["op"].kernel_name, {})
+        rec = tmap.get(w["op"].kernel_name + "|" + w["name"]) or tmap.get(w["op"].kernel_name, {})
         if rec.get("workload") != w["name"]:
             return None
         if rec.get("source_sha256") != kernel_source_sha256(w["op"].kernel_name):
