@@ -320,45 +320,51 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   // A lane holds activation row mb * 32 + lane % 32 and, per accumulator quad g, the four
   // consecutive features 8 g + 4 (lane / 32) + 0..3 of its wavefront's blocks 2 w, 2 w + 1.
   if constexpr (F16) {
-    // ---- float16: bias, activation clamp, round; the 256 x 256 x 2-byte tile is staged in
-    // two rounds, round r taking feature block r of every wavefront (128 columns, 64 KiB + padding)
+    // ---- float16: bias, activation clamp, round; the 256 x 256 x 2-byte tile is staged in two rounds of 128
+    // columns (64 KiB + padding): round r stages both feature blocks of wavefronts 2 r and 2 r + 1, so that a
+    // staged row is 256 contiguous output bytes - two whole lines (halves of a line written in different
+    // rounds cost half as many bytes again at the memory)
     constexpr int kHalfStride = 128 * 2 + 16;  // bytes per staged row: 128 halves + padding
     int8_t* out_tile = lds;
 #pragma unroll
     for (int round = 0; round < 2; ++round) {
       if (round) __syncthreads();
+      if ((wave >> 1) == round) {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        __builtin_amdgcn_sched_barrier(0);  // (one feature quad at a time, as below)
-        const int n = n0 + wave * 64 + round * 32 + 8 * g + 4 * frag_half;
-        float b4[4];
+        for (int nb = 0; nb < 2; ++nb) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) b4[q] = reinterpret_cast<const float*>(lds + kTabOffset)[n - n0 + q];
-        const int col = wave * 32 + 8 * g + 4 * frag_half;  // staged column (halves)
+          for (int g = 0; g < 4; ++g) {
+            __builtin_amdgcn_sched_barrier(0);  // (one feature quad at a time, as below)
+            const int nl = wave * 64 + nb * 32 + 8 * g + 4 * frag_half;  // feature within the tile
+            float b4[4];
 #pragma unroll
-        for (int mb = 0; mb < 8; ++mb) {
-          const int ml = mb * 32 + frag_row;
-          _Float16 h[4];
+            for (int q = 0; q < 4; ++q) b4[q] = reinterpret_cast<const float*>(lds + kTabOffset)[nl + q];
+            const int col = nl - round * 128;  // staged column (halves)
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            float v = acc[round][mb][g * 4 + q] + b4[q];
-            v = fminf(fmaxf(v, a.flo), a.fhi);
-            h[q] = static_cast<_Float16>(v);
+            for (int mb = 0; mb < 8; ++mb) {
+              const int ml = mb * 32 + frag_row;
+              _Float16 h[4];
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                float v = acc[nb][mb][g * 4 + q] + b4[q];
+                v = fminf(fmaxf(v, a.flo), a.fhi);
+                h[q] = static_cast<_Float16>(v);
+              }
+              uint2 pk;
+              __builtin_memcpy(&pk, h, 8);
+              *reinterpret_cast<uint2*>(out_tile + ml * kHalfStride + col * 2) = pk;
+            }
           }
-          uint2 pk;
-          __builtin_memcpy(&pk, h, 8);
-          *reinterpret_cast<uint2*>(out_tile + ml * kHalfStride + col * 2) = pk;
         }
       }
       __syncthreads();
-      // staged columns [32 w, 32 w + 32) are features [64 w + 32 round, + 32) of the tile; 8 halves per chunk
+      // a staged row holds features [128 round, 128 round + 128) of the tile: 16 chunks of 8 halves
       const bool vec_ok = (a.N & 7) == 0;
       for (int c = tid; c < TM * 16; c += kThreads) {
         const int ml = c >> 4, ch = c & 15;
-        const int wcol = ch >> 2, in_w = (ch & 3) * 8;
-        const int m = m0 + ml, n = n0 + wcol * 64 + round * 32 + in_w;
+        const int m = m0 + ml, n = n0 + round * 128 + ch * 8;
         if (m >= a.M || n >= a.N) continue;
-        const int8_t* src = out_tile + ml * kHalfStride + (wcol * 32 + in_w) * 2;
+        const int8_t* src = out_tile + ml * kHalfStride + ch * 16;
         int8_t* dst = a.y + (static_cast<size_t>(m) * a.N + n) * 2;
         if (vec_ok) {
           *reinterpret_cast<v4i*>(dst) = *reinterpret_cast<const v4i*>(src);
