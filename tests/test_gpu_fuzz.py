@@ -65,6 +65,44 @@ def test_conv2d_sweep(oracle, tvx):
         assert seen[k] >= 5, seen
 
 
+def test_grouped_and_float16_conv2d_sweep(oracle):
+    """Random grouped convolutions (quantized, bit for bit) and float16 convolutions (1e-2) on the GEMM-over-windows
+    kernels: group counts 2-4, channel counts per group around the 32-channel tile edges, any kernel / stride /
+    dilation / padding, pixel counts that leave ragged tiles."""
+    rng = np.random.default_rng(0x6E)
+    seen = collections.Counter()
+    for i in range(90):
+        kh, kw = (int(rng.choice([1, 2, 3, 5])), int(rng.choice([1, 3, 5]))) if rng.random() < 0.4 else (3, 3)
+        s = [int(rng.choice([1, 1, 2])), int(rng.choice([1, 1, 2]))]
+        d = [int(rng.choice([1, 1, 1, 2])), int(rng.choice([1, 1, 1, 2]))]
+        pad = [int(min(rng.integers(0, 3), (kw - 1) * d[0])) for _ in range(2)] + \
+              [int(min(rng.integers(0, 3), (kh - 1) * d[1])) for _ in range(2)]
+        h = int(rng.integers((kh - 1) * d[1] + 1, 26))
+        w = int(rng.integers((kw - 1) * d[0] + 1, 26))
+        f16 = i % 3 == 2
+        groups = 1 if f16 and rng.random() < 0.5 else int(rng.integers(2, 5))
+        icg = int(rng.choice([4, 8, 12, 16, 20, 31, 32, 33, 48]))
+        ocg = int(rng.choice([8, 9, 16, 31, 32, 33, 40, 64, 70]))
+        if icg * kh * kw * (2 if f16 else 1) < 32:
+            icg = 32
+        mode = "f16" if f16 else str(rng.choice(["u8", "i8pc", "u8pc"]))
+        x, wt, b, kws = conv_case(rng, n=int(rng.integers(1, 4)), c=groups * icg, h=h, w=w, oc=groups * ocg, kh=kh, kw=kw,
+                                  stride=s, dil=d, pad=pad, mult=0, mode=mode, groups=groups if groups > 1 else 0)
+        if min(kws["out_shape"][:2]) < 1:
+            continue
+        act = int(rng.integers(0, 3))
+        want = oracle.conv2d(x, wt, b, act=act, **kws)
+        T = TC.tvx()
+        got = TC.gpu_conv2d(x, wt, b, act=act, **kws)
+        if f16:
+            assert np.allclose(got.astype(np.float32), want.astype(np.float32), rtol=1e-2, atol=2e-2), (i, kws)
+            seen["f16"] += 1
+        else:
+            assert np.array_equal(got, want), (i, kws["in_shape"], kws["w_shape"], groups, mode, act, int((got != want).sum()))
+            seen["q"] += 1
+    assert seen["f16"] >= 20 and seen["q"] >= 40, seen
+
+
 def _run_conv(tvx, x, wt, b, act, kws, kernel_out):
     """gpu_conv2d, also reporting which kernel ran."""
     import ctypes as C
