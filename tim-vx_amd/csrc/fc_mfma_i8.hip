@@ -47,7 +47,8 @@ constexpr int kThreads = 256;
 constexpr int kTileBytes = TM * TK;             // 32 KiB per activation tile
 constexpr int kStages = 4;                      // activation tiles in LDS (a power of two)
 constexpr int kTabOffset = kStages * kTileBytes;  // behind the stages: the tile's epilogue tables
-constexpr int kLdsBytes = kTabOffset + TN * 4 + TN * 16;  // folded bias (or fp32 bias), requantization records
+constexpr int kRowsumOffset = kTabOffset + TN * 4 + TN * 16;  // behind the folded bias (or fp32 bias) and the requantization records
+constexpr int kLdsBytes = kRowsumOffset + TM * 4;  // the activation rows' sums, exchanged between the wavefronts
 // k-tiles of the packed weights: whole rounds of three (the kernel's weight slots)
 __host__ __device__ constexpr int k_tiles_padded(int k_bytes) { return ((k_bytes + TK - 1) / TK + 2) / 3 * 3; }
 constexpr int kOutStride = TN + 16;             // epilogue staging row stride (bytes)
@@ -83,6 +84,7 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);
 
   // Workgroups are dealt round-robin to the 8 XCDs; give each XCD a contiguous
   // run of tiles so that neighbours in its L2 share operand panels.
@@ -134,9 +136,17 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   const bool k_tail = (a.K % TK) != 0;
   // piece i of k-tile kt into its stage; tiles past the last one and reduction bytes past K
   // read the zero source (0x80 before the re-bias of uint8 activations) and meet zero weights
-  auto dma_piece = [&](int kt, int i) {
-    int8_t* dst = lds + (kt & (kStages - 1)) * kTileBytes + wave * 64 * TK + i * 1024;
+  auto dma_piece = [&](auto whole, int kt, int i) {
+    int8_t* dst = lds + (kt & (kStages - 1)) * kTileBytes + wave_s * 64 * TK + i * 1024;
     const int k0 = kt * TK;
+    if constexpr (decltype(whole)::value) {
+      // a k-tile that lies inside K: a scalar base (tensor + k0) and the lane's 32-bit offset, no address arithmetic
+      // on the vector unit
+      const int8_t* base = a.x + k0;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + off_x[i]),
+                                       (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+      return;
+    }
     // branch-free: the address is blended from the two candidates with a mask
     const bool past = (kt >= k_tiles) | (k_tail & (k0 + dma_chunk[i & 1] * 16 >= a.K));
     const uintptr_t real = reinterpret_cast<uintptr_t>(a.x) + (off_x[i] + static_cast<uint32_t>(k0));
@@ -153,16 +163,17 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   // Wavefront w owns feature blocks 2 w and 2 w + 1 of the tile's eight and every
   // activation row, so no fragment is fetched twice. Three k-tiles of fragments are
   // resident; slot kt % 3 is refilled for k-tile kt + 3 as its k-steps retire.
-  const int8_t* wp[2];
+  const int8_t* wp[2];  // (wavefront-uniform: the lane's 16 bytes are the load's vector offset)
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb)
-    wp[nb] = a.w + (static_cast<size_t>(n0 / 32 + wave * 2 + nb) * (k_tiles_padded(a.K) * 4)) * 1024 + lane * 16;
+    wp[nb] = a.w + (static_cast<size_t>(n0 / 32 + wave_s * 2 + nb) * (k_tiles_padded(a.K) * 4)) * 1024;
+  const uint32_t lane16 = lane * 16;
   v4i wr[3][8];  // [slot][nb * 4 + k-step]
 #define TVX_W_LOAD(dst, ptr, off) \
-  asm volatile("global_load_dwordx4 %0, %1, off offset:%2" : "=v"(dst) : "v"(ptr), "n"(off))
-  // fragment (nb, kk) of k-tile kt; k-tiles past the padded count do not exist: re-read the last
-  auto w_piece = [&](int kt, int nb, int kk, v4i& dst, int kt_max) {
-    const int8_t* ptr = wp[nb] + static_cast<size_t>(min(kt, kt_max)) * 4096;
+  asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(dst) : "v"(lane16), "s"(ptr), "n"(off))
+  // fragment (nb, kk) of k-tile kt (callers stay below the padded count of k-tiles)
+  auto w_piece = [&](int kt, int nb, int kk, v4i& dst) {
+    const int8_t* ptr = wp[nb] + static_cast<size_t>(kt) * 4096;
     if (kk == 0) TVX_W_LOAD(dst, ptr, 0);
     else if (kk == 1) TVX_W_LOAD(dst, ptr, 1024);
     else if (kk == 2) TVX_W_LOAD(dst, ptr, 2048);
@@ -177,7 +188,7 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
     for (int j = 0; j < 8; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-  int rowsum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  int rowsum[8] = {0, 0, 0, 0, 0, 0, 0, 0};  // per piece of this wavefront's share of the activation tile (see the in-place pass below)
 
   const int frag_row = lane & 31;   // row inside a 32-row MFMA tile
   const int frag_half = lane >> 5;  // which 16-byte half of a 32-byte k-step
@@ -194,51 +205,111 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
     frag_x[kk] = lds_base + frag_row * TK + (((kk * 2 + frag_half) ^ row7) << 4);
 #define TVX_DS_READ(dst, addr, off) \
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
-  auto load_frags = [&](int kt, int kk, v4i* fx) {
+  // fragment t (activation rows 32 t ..) of k-step kk of k-tile kt
+  auto load_frag = [&](int kt, int kk, v4i* fx, int t) {
     const uint32_t ax = frag_x[kk] + (kt & (kStages - 1)) * kTileBytes;
-    TVX_DS_READ(fx[0], ax, 0);
-    TVX_DS_READ(fx[1], ax, 32 * TK);
-    TVX_DS_READ(fx[2], ax, 64 * TK);
-    TVX_DS_READ(fx[3], ax, 96 * TK);
-    TVX_DS_READ(fx[4], ax, 128 * TK);
-    TVX_DS_READ(fx[5], ax, 160 * TK);
-    TVX_DS_READ(fx[6], ax, 192 * TK);
-    TVX_DS_READ(fx[7], ax, 224 * TK);
+    if (t == 0) TVX_DS_READ(fx[0], ax, 0);
+    else if (t == 1) TVX_DS_READ(fx[1], ax, 32 * TK);
+    else if (t == 2) TVX_DS_READ(fx[2], ax, 64 * TK);
+    else if (t == 3) TVX_DS_READ(fx[3], ax, 96 * TK);
+    else if (t == 4) TVX_DS_READ(fx[4], ax, 128 * TK);
+    else if (t == 5) TVX_DS_READ(fx[5], ax, 160 * TK);
+    else if (t == 6) TVX_DS_READ(fx[6], ax, 192 * TK);
+    else TVX_DS_READ(fx[7], ax, 224 * TK);
   };
 #undef TVX_DS_READ
-  // One k-step: 16 MFMAs with the four memory operations of this k-step's share of the
-  // prefetch spread between them, one every fourth MFMA (issued in a burst they would queue
-  // up in the memory pipeline with the wavefront waiting behind them). The weight registers
-  // of this k-step are refilled (for k-tile kt + 3) only after the MFMAs that read them
-  // were issued.
-  auto k_step = [&](auto prefetch, int kt, int kk, v4i* fx, v4i* w_slot, int kt_max) {
-    constexpr bool kPrefetch = decltype(prefetch)::value;
-    if (X_U8) {
-#pragma unroll
-      for (int t = 0; t < 8; ++t) fx[t] ^= static_cast<int>(0x80808080);
-    }
+  // ---- uint8 activations and row sums: one pass over the tile in LDS ---------------------
+  // The MFMA is signed, so uint8 activations are re-biased (x ^ 0x80 = x - 128 as int8), and a uniform
+  // weight zero point needs the sum of every activation row. Both are vector-unit work, and a wavefront's
+  // vector instructions do not overlap its own MFMAs (measured: each costs its full issue time on top of
+  // the MFMA time). Done on the fragments, the four wavefronts - which all read every row - would each do
+  // all of it; done once on the tile in LDS it is a quarter: every wavefront rewrites the 64 rows it
+  // fetched itself (eight pieces of 1 KiB, a lane's 16 bytes of one row each), one k-tile ahead of the
+  // MFMAs, spread over the first three k-steps. The barrier that publishes k-tile kt + 1 also publishes
+  // its rewritten form.
+  constexpr bool kInPlace = X_U8 || ROWSUM;
+  const uint32_t own_x = lds_base + wave * 64 * TK + lane * 16;
+#define TVX_DS_READ(dst, addr, off) \
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
+#define TVX_DS_WRITE(addr, src, off) \
+  asm volatile("ds_write_b128 %0, %1 offset:%2" : : "v"(addr), "v"(src), "n"(off))
+  auto piece_read = [&](int kt, int i, v4i& t) {
+    const uint32_t ax = own_x + (kt & (kStages - 1)) * kTileBytes;
+    if (i == 0) TVX_DS_READ(t, ax, 0);
+    else if (i == 1) TVX_DS_READ(t, ax, 1024);
+    else if (i == 2) TVX_DS_READ(t, ax, 2048);
+    else if (i == 3) TVX_DS_READ(t, ax, 3072);
+    else if (i == 4) TVX_DS_READ(t, ax, 4096);
+    else if (i == 5) TVX_DS_READ(t, ax, 5120);
+    else if (i == 6) TVX_DS_READ(t, ax, 6144);
+    else TVX_DS_READ(t, ax, 7168);
+  };
+  auto piece_finish = [&](int kt, int i, v4i& t) {
+    if (X_U8) t ^= static_cast<int>(0x80808080);
     if (ROWSUM) {
 #pragma unroll
-      for (int t = 0; t < 8; ++t)
-#pragma unroll
-        for (int q = 0; q < 4; ++q)
-          rowsum[t] = __builtin_amdgcn_sdot4(fx[t][q], 0x01010101, rowsum[t], false);
+      for (int q = 0; q < 4; ++q) rowsum[i] = __builtin_amdgcn_sdot4(t[q], 0x01010101, rowsum[i], false);
     }
+    if (X_U8) {
+      const uint32_t ax = own_x + (kt & (kStages - 1)) * kTileBytes;
+      if (i == 0) TVX_DS_WRITE(ax, t, 0);
+      else if (i == 1) TVX_DS_WRITE(ax, t, 1024);
+      else if (i == 2) TVX_DS_WRITE(ax, t, 2048);
+      else if (i == 3) TVX_DS_WRITE(ax, t, 3072);
+      else if (i == 4) TVX_DS_WRITE(ax, t, 4096);
+      else if (i == 5) TVX_DS_WRITE(ax, t, 5120);
+      else if (i == 6) TVX_DS_WRITE(ax, t, 6144);
+      else TVX_DS_WRITE(ax, t, 7168);
+    }
+  };
+#undef TVX_DS_READ
+#undef TVX_DS_WRITE
+  v4i pc[3];  // pieces on their way through the pass
+  // One k-step: 16 MFMAs of 32 cycles each, and everything else the k-step has to issue dealt out
+  // between them, a few instructions at a time (the compiler, left to itself, gathers them into two
+  // runs per k-step; memory instructions issued in a burst queue up with the wavefront waiting behind
+  // them). Pair p multiplies activation block p with the wavefront's two weight fragments; behind its
+  // MFMAs go: the LDS reads of the next k-step's fragments (two per pair, all eight issued by the
+  // middle of the k-step), this k-step's share of the in-place pass over the next k-tile (three
+  // pieces in k-steps 0 and 1, two in k-step 2: read behind pair 2, finished behind pairs 6 and 7),
+  // and the k-step's four memory operations of the prefetch - the weight registers are refilled
+  // (for k-tile kt + 3) right after the last MFMA that reads them.
+  auto k_step = [&](auto prefetch, auto whole, auto fetch_next, auto in_place, auto newer, int kt, int kk, v4i* fx,
+                    v4i* w_slot, int next_kt, int next_kk, v4i* fx_next) {
+    constexpr bool kPrefetch = decltype(prefetch)::value;
+    constexpr bool kNext = decltype(fetch_next)::value;
+    constexpr bool kPass = kInPlace && decltype(in_place)::value;
+    const int first = kk * 3, pieces = kk < 2 ? 3 : (kk == 2 ? 2 : 0);
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb) {
+    for (int mb = 0; mb < 8; ++mb) {
+      acc[0][mb] = Mfma(w_slot[kk], fx[mb], acc[0][mb]);
+      if (kNext && mb < 4) load_frag(next_kt, next_kk, fx_next, 2 * mb);
+      if (kPass && mb == 2) {
+        // this wavefront's own pieces of k-tile kt + 1 have landed when at most the newest 16 memory
+        // operations (or, in the last round, none) are still on their way
+        if (kk == 0) {
+          if constexpr (decltype(newer)::value != 0) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+          else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
 #pragma unroll
-      for (int mb = 0; mb < 8; ++mb) {
-        acc[nb][mb] = Mfma(w_slot[nb * 4 + kk], fx[mb], acc[nb][mb]);
-        if (kPrefetch && mb == 3) {
-          dma_piece(kt + 3, kk * 2 + nb);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        if (kPrefetch && mb == 7) {
-          __builtin_amdgcn_sched_barrier(0);
-          w_piece(kt + 3, nb, kk, w_slot[nb * 4 + kk], kt_max);
-          __builtin_amdgcn_sched_barrier(0);
-        }
+        for (int j = 0; j < 3; ++j)
+          if (j < pieces) piece_read(kt + 1, first + j, pc[j]);
       }
+      if (kPrefetch && mb == 4) dma_piece(whole, kt + 3, kk * 2);
+      if (kPass && mb == 6 && pieces > 0) {
+        // (the pieces are operands of the wait: nothing that uses them may be moved in front of it)
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(pc[0]), "+v"(pc[1]), "+v"(pc[2])::"memory");
+        piece_finish(kt + 1, first, pc[0]);
+      }
+      if (kPass && mb == 7 && pieces > 2) piece_finish(kt + 1, first + 2, pc[2]);
+      if (kPrefetch && mb == 7) w_piece(kt + 3, 0, kk, w_slot[kk]);
+      __builtin_amdgcn_sched_barrier(0);
+      acc[1][mb] = Mfma(w_slot[4 + kk], fx[mb], acc[1][mb]);
+      if (kNext && mb < 4) load_frag(next_kt, next_kk, fx_next, 2 * mb + 1);
+      if (kPrefetch && mb == 5) dma_piece(whole, kt + 3, kk * 2 + 1);
+      if (kPass && mb == 6 && pieces > 1) piece_finish(kt + 1, first + 1, pc[1]);
+      if (kPrefetch && mb == 7) w_piece(kt + 3, 1, kk, w_slot[4 + kk]);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
   // k-tile kt with its weight slot: the fragments of k-step kk + 1 are fetched while step kk
@@ -247,38 +318,31 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   // issues 16 memory operations in the same order; "at most 28 in flight" at the barrier
   // (12 of this k-tile, 16 of the one before) means that everything issued two k-tiles ago
   // - the activations and weights of k-tile kt + 1 - has landed.
-  const int kt_max = k_tiles_padded(a.K) - 1;
   v4i fxa[8], fxb[8];
   // `prefetch`: the k-tile issues its share of k-tile kt + 3 (all rounds but the last, which is peeled off so that
   // no fetch is in flight when the loop ends: registers named by an unfinished fetch would otherwise have to be
   // kept out of the epilogue's hands). `in_flight`: memory operations that may still be on their way at the
   // barrier (28 while prefetching; 16, 0, 0 in the last round). `last`: no fragments of a next k-tile.
-  auto k_tile = [&](auto prefetch, auto in_flight, auto last, int kt, v4i* w_slot) {
-    load_frags(kt, 1, fxb);
-    asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
+  auto k_tile = [&](auto prefetch, auto whole, auto in_flight, auto last, int kt, v4i* w_slot) {
+    const std::integral_constant<bool, true> yes;
+    const std::integral_constant<bool, !decltype(last)::value> unless_last;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the fragments of k-step 0
     __builtin_amdgcn_sched_barrier(0);
-    k_step(prefetch, kt, 0, fxa, w_slot, kt_max);
+    k_step(prefetch, whole, yes, unless_last, in_flight, kt, 0, fxa, w_slot, kt, 1, fxb);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
-    load_frags(kt, 2, fxa);
-    asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
+    k_step(prefetch, whole, yes, unless_last, in_flight, kt, 1, fxb, w_slot, kt, 2, fxa);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
-    k_step(prefetch, kt, 1, fxb, w_slot, kt_max);
-    __builtin_amdgcn_sched_barrier(0);
-    load_frags(kt, 3, fxb);
-    asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-    k_step(prefetch, kt, 2, fxa, w_slot, kt_max);
-    __builtin_amdgcn_sched_barrier(0);
+    k_step(prefetch, whole, yes, unless_last, in_flight, kt, 2, fxa, w_slot, kt, 3, fxb);
     if constexpr (decltype(in_flight)::value == 28) asm volatile("s_waitcnt vmcnt(28) lgkmcnt(0)" ::: "memory");
     else if constexpr (decltype(in_flight)::value == 16) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     // the bare barrier: __syncthreads() adds a fence that waits for every memory operation in
     // flight - the whole prefetch - at every k-tile
     __builtin_amdgcn_s_barrier();
-    if constexpr (!decltype(last)::value) load_frags(kt + 1, 0, fxa);
     __builtin_amdgcn_sched_barrier(0);
-    k_step(prefetch, kt, 3, fxb, w_slot, kt_max);
-    __builtin_amdgcn_sched_barrier(0);
+    k_step(prefetch, whole, unless_last, unless_last, in_flight, kt, 3, fxb, w_slot, kt + 1, 0, fxa);
   };
   // prologue: k-tiles 0, 1, 2 in the order every later k-tile uses (8 x (activation piece,
   // weight fragment)), so that the in-flight counts line up from the first barrier on
@@ -288,14 +352,28 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
     for (int kk = 0; kk < 4; ++kk)
 #pragma unroll
       for (int nb = 0; nb < 2; ++nb) {
-        dma_piece(t, kk * 2 + nb);
+        dma_piece(std::integral_constant<bool, false>(), t, kk * 2 + nb);
         __builtin_amdgcn_sched_barrier(0);
-        w_piece(t, nb, kk, wr[t][nb * 4 + kk], kt_max);
+        w_piece(t, nb, kk, wr[t][nb * 4 + kk]);
         __builtin_amdgcn_sched_barrier(0);
       }
   asm volatile("s_waitcnt vmcnt(32)" ::: "memory");  // k-tile 0 has landed
+  if (kInPlace) {
+    // the in-place pass over k-tile 0 (every later k-tile gets it while the one before multiplies)
+#pragma unroll
+    for (int i = 0; i < 8; i += 2) {
+      piece_read(0, i, pc[0]);
+      piece_read(0, i + 1, pc[1]);
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(pc[0]), "+v"(pc[1])::"memory");
+      piece_finish(0, i, pc[0]);
+      piece_finish(0, i + 1, pc[1]);
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
   __builtin_amdgcn_s_barrier();
-  load_frags(0, 0, fxa);
+#pragma unroll
+  for (int t = 0; t < 8; ++t) load_frag(0, 0, fxa, t);
+  const int kt_max = k_tiles_padded(a.K) - 1;
   // the loop runs whole rounds of three k-tiles (the weight slots are named registers); the
   // packed weights are zero-padded to that count and the activations past K read zeros
   {
@@ -303,17 +381,35 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
     const integral_constant<bool, true> yes;
     const integral_constant<bool, false> no;
     int kt = 0;
+    // rounds whose prefetch (k-tiles kt + 3 .. kt + 5) lies inside K, then those that reach past it
+    const int whole_tiles = a.K / TK;
+    for (; kt + 6 <= whole_tiles; kt += 3) {
+      k_tile(yes, yes, integral_constant<int, 28>(), no, kt, wr[0]);
+      k_tile(yes, yes, integral_constant<int, 28>(), no, kt + 1, wr[1]);
+      k_tile(yes, yes, integral_constant<int, 28>(), no, kt + 2, wr[2]);
+    }
     for (; kt + 3 <= kt_max; kt += 3) {
-      k_tile(yes, integral_constant<int, 28>(), no, kt, wr[0]);
-      k_tile(yes, integral_constant<int, 28>(), no, kt + 1, wr[1]);
-      k_tile(yes, integral_constant<int, 28>(), no, kt + 2, wr[2]);
+      k_tile(yes, no, integral_constant<int, 28>(), no, kt, wr[0]);
+      k_tile(yes, no, integral_constant<int, 28>(), no, kt + 1, wr[1]);
+      k_tile(yes, no, integral_constant<int, 28>(), no, kt + 2, wr[2]);
     }
     // the last round: its k-tiles were fetched by the round before (or the prologue); nothing new is fetched
-    k_tile(no, integral_constant<int, 16>(), no, kt, wr[0]);
-    k_tile(no, integral_constant<int, 0>(), no, kt + 1, wr[1]);
-    k_tile(no, integral_constant<int, 0>(), yes, kt + 2, wr[2]);
+    k_tile(no, no, integral_constant<int, 16>(), no, kt, wr[0]);
+    k_tile(no, no, integral_constant<int, 0>(), no, kt + 1, wr[1]);
+    k_tile(no, no, integral_constant<int, 0>(), yes, kt + 2, wr[2]);
   }
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // (nothing is in flight here; the staging tile is about to be written)
+  if (ROWSUM) {
+    // piece i holds rows 64 w + 8 i + lane / 8, a lane its 16 bytes of every k-tile: eight lanes make a row
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      int sum = rowsum[i];
+      sum += __shfl_xor(sum, 1);
+      sum += __shfl_xor(sum, 2);
+      sum += __shfl_xor(sum, 4);
+      if ((lane & 7) == 0) reinterpret_cast<int*>(lds + kRowsumOffset)[wave * 64 + i * 8 + (lane >> 3)] = sum;
+    }
+  }
   __syncthreads();  // the epilogue reuses the LDS
 
   // ---- epilogue ---------------------------------------------------------------
@@ -375,10 +471,10 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
       }
     }
   } else {
-    if (ROWSUM) {
+    int zp_term[8];  // weight zero point x row sum, per activation block of this lane's row
 #pragma unroll
-      for (int t = 0; t < 8; ++t) rowsum[t] += __shfl_xor(rowsum[t], 32);
-    }
+    for (int t = 0; t < 8; ++t)
+      zp_term[t] = ROWSUM ? a.zws * reinterpret_cast<const int*>(lds + kRowsumOffset)[t * 32 + frag_row] : 0;
     int8_t* out_tile = lds;  // TM rows x kOutStride bytes (the loop's last barrier freed the LDS)
 #pragma unroll
     for (int nb = 0; nb < 2; ++nb) {
@@ -401,7 +497,7 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
             int v = acc[nb][mb][g * 4 + q] + b4[q];
-            if (ROWSUM) v -= a.zws * rowsum[mb];
+            if (ROWSUM) v -= zp_term[mb];
             r4[q] = Requant8<RQ>(v, q4[q], a.out_zp, a.lo, a.hi);
           }
           *reinterpret_cast<uint32_t*>(out_tile + ml * kOutStride + nl) = PackBytes(r4[0], r4[1], r4[2], r4[3]);
