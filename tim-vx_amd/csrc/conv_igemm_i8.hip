@@ -620,11 +620,14 @@ ConvPersistKernel(ConvArgs a) {
         const int p = min(p0 + pt * 32 + frag_row, p_end - 1);  // rows past the tile's end recompute its last pixel
         const int oh = p / a.OW, ow = p - oh * a.OW;
         const int8_t* frag = halo + ((oh - r0) * a.sh * a.iwt + ow * a.sw) * a.pix_stride + frag_half * 16;
+        // a lane's accumulators belong to one output channel per tile: they start from its folded bias
         v16i acc[OT];
 #pragma unroll
-        for (int j = 0; j < OT; ++j)
+        for (int j = 0; j < OT; ++j) {
+          const int bias = bias_lds[j * 32 + frag_row];
 #pragma unroll
-          for (int r = 0; r < 16; ++r) acc[j][r] = 0;
+          for (int r = 0; r < 16; ++r) acc[j][r] = bias;
+        }
         int sx = 0;
         // fragments RING - 1 k-steps ahead: LDS latency, not bandwidth, is what the loop would wait for
         constexpr int RING = ZP ? 3 : 4;  // (the pixel sums' registers cost the zero-point form one stage)
@@ -659,11 +662,10 @@ ConvPersistKernel(ConvArgs a) {
           for (int j = 0; j < OT; ++j) {
             const int ocl = j * 32 + frag_row;
             const v4i rq = rq_lds[ocl];
-            const int bias = bias_lds[ocl];
             int r4[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-              r4[e] = Requant8<RQ>(acc[j][g * 4 + e] + (bias - s4[e]), rq, a.out_zp, a.lo, a.hi);
+              r4[e] = Requant8<RQ>(ZP ? acc[j][g * 4 + e] - s4[e] : acc[j][g * 4 + e], rq, a.out_zp, a.lo, a.hi);
             *reinterpret_cast<uint32_t*>(out_tile + ocl * a.out_stride + pl) = PackBytes(r4[0], r4[1], r4[2], r4[3]);
           }
         }

@@ -113,6 +113,7 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
       reinterpret_cast<tvx_v4i*>(lds + kTabOffset + TN * 4)[tid] = a.rq[n0 + tid];
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the in-flight counts below start from zero
+    if constexpr (!F16) __syncthreads();  // the accumulators start from the folded bias
   }
   // ---- activations: global -> LDS DMA ---------------------------------------------
   // One wave instruction moves 64 x 16 bytes into 1 KiB of consecutive LDS: 8
@@ -181,13 +182,23 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   };
 #undef TVX_W_LOAD
 
-  acc_t acc[2][8];  // [feature block][activation block]
+  // [feature block][activation block]; a lane holds, per accumulator quad g, features 8 g + 4 (lane / 32) + 0..3 of its
+  // wavefront's blocks. The integer accumulators start from the folded bias: one addition less per output in the epilogue.
+  acc_t acc[2][8];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 8; ++j)
+    for (int g = 0; g < 4; ++g) {
+      int b4[4] = {0, 0, 0, 0};
+      if constexpr (!F16) {
+        const v4i t = *reinterpret_cast<const v4i*>(lds + kTabOffset + (wave * 64 + i * 32 + 8 * g + 4 * (lane >> 5)) * 4);
+        b4[0] = t[0], b4[1] = t[1], b4[2] = t[2], b4[3] = t[3];
+      }
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) acc[i][j][g * 4 + q] = b4[q];
+    }
   int rowsum[8] = {0, 0, 0, 0, 0, 0, 0, 0};  // per piece of this wavefront's share of the activation tile (see the in-place pass below)
 
   const int frag_row = lane & 31;   // row inside a 32-row MFMA tile
@@ -484,9 +495,6 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
         __builtin_amdgcn_sched_barrier(0);
         const int nl = wave * 64 + nb * 32 + 8 * g + 4 * frag_half;
         const int n = n0 + nl;
-        int b4[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) b4[q] = reinterpret_cast<const int*>(lds + kTabOffset)[nl + q];
         tvx_v4i q4[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) q4[q] = reinterpret_cast<const tvx_v4i*>(lds + kTabOffset + TN * 4)[nl + q];
@@ -496,7 +504,7 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
           int r4[4];
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            int v = acc[nb][mb][g * 4 + q] + b4[q];
+            int v = acc[nb][mb][g * 4 + q];  // (bias included: the accumulators started from it)
             if (ROWSUM) v -= zp_term[mb];
             r4[q] = Requant8<RQ>(v, q4[q], a.out_zp, a.lo, a.hi);
           }
