@@ -293,6 +293,24 @@ def test_fully_connected_mfma_edges(oracle, mode, shape, kernel):
     assert len(np.unique(want)) > 4
 
 
+def test_fully_connected_full_size_uint8_asymmetric(oracle):
+    """M=8192, K=4096, N=4096 uint8 with a uniform weight zero point: the variant whose activations are re-biased
+    and summed per row inside the kernel, one k-tile ahead of the multiplications, over all 32 k-tiles and both
+    tiles of a CU. A seeded sample of rows against the oracle, every tile row covered."""
+    m, k, n = 8192, 4096, 4096
+    rng = np.random.default_rng(0x76)
+    x = rng.integers(0, 256, m * k, dtype=np.uint8)
+    w = rng.integers(0, 256, n * k, dtype=np.uint8)
+    b = rng.integers(-16384, 16385, n).astype(np.int32)
+    kws = dict(k=k, n=n, in_dtype=0, w_dtype=0, out_dtype=0, in_q=(0.02, 121), w_q=(0.01, 131, None),
+               out_q=(1.2, 128))
+    got = TC.gpu_fully_connected(x, w, b, m=m, want_kernel="fc_mfma_i8_256x256x128", **kws).reshape(m, n)
+    rows = np.sort(np.concatenate([np.arange(32) * 256 + rng.integers(0, 256, 32), rng.choice(m, 16, replace=False)]))
+    want = oracle.fully_connected(np.ascontiguousarray(x.reshape(m, k)[rows]).ravel(), w, b, m=len(rows), **kws)
+    assert np.array_equal(got[rows], want.reshape(len(rows), n))
+    assert len(np.unique(got)) > 100
+
+
 def test_fully_connected_full_size_int8_per_channel(oracle):
     """M=8192, K=4096, N=4096 int8 per-channel: the whole problem on the GPU, a
     seeded sample of 48 rows recomputed by the oracle, plus linearity in the bias."""
