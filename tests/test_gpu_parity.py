@@ -582,6 +582,16 @@ GEMM_GRID = [
     (3, 48, 200, 2, 12, 20, 3, 1, [1, 2], [1, 1], [0, 0, 1, 1]),
     (2, 36, 27, 3, 9, 9, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),
     (1, 40, 72, 1, 24, 24, 1, 1, [1, 1], [1, 1], [0, 0, 0, 0]),
+    # unit column stride and output rows of whole pixel quads (the gather by quads): windows that leave the image
+    # on the left and right by 1, 2 and 3 columns, the narrowest row (4 columns: every load is clamped), groups
+    # whose channels do not fill a chunk half, row stride 2, as much padding as the window reaches
+    (2, 32, 48, 2, 12, 16, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),
+    (1, 24, 24, 3, 10, 12, 3, 3, [1, 1], [2, 2], [2, 2, 2, 2]),
+    (2, 64, 64, 2, 8, 4, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),
+    (1, 80, 40, 2, 9, 8, 3, 3, [1, 1], [3, 3], [3, 3, 3, 3]),
+    (2, 36, 96, 3, 15, 20, 3, 5, [1, 2], [1, 1], [2, 2, 1, 1]),
+    (1, 32, 32, 2, 6, 10, 3, 3, [1, 1], [1, 1], [2, 2, 2, 2]),
+    (1, 64, 64, 2, 35, 32, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),
 ]
 
 

@@ -5,10 +5,11 @@
 //
 // A workgroup owns 128 consecutive output pixels of one image and 32 or 64 output channels of one group.
 // The reduction runs tap by tap (a tap's channels padded to whole half-chunks) in chunks of 64 bytes per pixel
-// row: every thread gathers half a chunk - 32 bytes of one tap, walking the channel planes from one base
-// address under one validity test - into registers (the next chunk's loads are in flight under the MFMAs),
-// the chunk lands in LDS as [pixel][k], the weights - packed at creation into the very LDS image - are
-// copied beside it, and each wavefront multiplies its 32 pixels with all the workgroup's channels
+// row: every thread gathers its share of half a chunk - 32 bytes per pixel of one tap's channel planes, by pixel
+// quads where rows allow it (four pixels x 8 channels from 8 loads, transposed in registers), else by elements
+// (one pixel x 32 channels) - into registers (the next chunk's loads are in flight under the MFMAs),
+// the chunk lands in LDS as [pixel][k], the weights - packed at creation into the very LDS image and fetched
+// a chunk ahead like the activations - are copied beside it, and each wavefront multiplies its 32 pixels with all the workgroup's channels
 // (v_mfma_i32_32x32x32_i8 / v_mfma_f32_32x32x16_f16: both read 16 bytes per lane and step 32 bytes of a row).
 // Quantized tensors: activations and weights go to the signed domain (u8 ^ 0x80), padding holds the input's
 // zero point, the weights' zero point is a second MFMA against a constant vector, everything constant is
@@ -78,8 +79,8 @@ __device__ __forceinline__ void StoreFour(const GemmArgs& a, uint8_t* y, size_t 
   }
 }
 
-// OT: 32-channel tiles of a workgroup (1 or 2).
-template <bool F16, int OT>
+// OT: 32-channel tiles of a workgroup (1 or 2). QUAD: the gather by pixel quads (see below) instead of by elements.
+template <bool F16, int OT, bool QUAD>
 __global__ void __launch_bounds__(kThreads) ConvGemmKernel(GemmArgs a) {
   __shared__ __attribute__((aligned(16))) uint8_t a_lds[kPixels * kRowStride];
   __shared__ __attribute__((aligned(16))) uint8_t b_lds[OT * 32 * kRowStride];
@@ -137,6 +138,104 @@ __global__ void __launch_bounds__(kThreads) ConvGemmKernel(GemmArgs a) {
     }
   };
 
+  // ---- the gather by pixel quads (unit column stride, output rows of whole quads) -------------------
+  // Four consecutive output pixels of a row read four consecutive input columns at every tap: a thread owns one
+  // quad and 8 (float16: 4) channels of its chunk half, loads per channel the 4 (8) bytes under the quad - one
+  // unaligned load instead of four element loads, clamped into the row and shifted back into place at the
+  // image's left and right edges -, transposes the channel x pixel block in registers and writes 8 bytes per
+  // pixel into the LDS image. Per chunk: 8 (4) loads and ~45 vector instructions, against 32 (16) loads and ~200.
+  constexpr int kQuadCh = F16 ? 4 : 8;  // channels of a thread
+  const int q = lane & 31;
+  const int cg = (wave & 1) * 2 + (lane >> 5);
+  const int pq = p0 + 4 * q;
+  const bool q_live = pq < hw;
+  const int q_oh = pq / a.OW, q_ow = pq - q_oh * a.OW;
+  const int q_ih0 = q_oh * a.sh - a.pad_t, q_iw0 = q_ow - a.pad_l;
+  const int q_origin = q_ih0 * a.W + q_iw0;
+  int q_shift = 0, q_s = 0, q_n = 0;  // of the chunk in flight: columns clamped away, first column, real channels from this thread's first
+  bool q_row = false;
+  auto gather_quad = [&](int chunk) {
+    const int2 e = a.tab[chunk * 2 + half];
+    const int dy = e.y & 0xff, dx = (e.y >> 8) & 0xff;
+    const int nreal = e.y >> 16;
+    q_row = q_live && static_cast<unsigned>(q_ih0 + dy) < static_cast<unsigned>(a.H);
+    q_s = q_iw0 + dx;
+    q_shift = q_s - max(0, min(q_s, a.W - 4));
+    q_n = nreal - cg * kQuadCh;
+    const int base = q_row ? q_origin + e.x - q_shift : 0;  // (rows outside the image: any readable place, replaced below)
+#pragma unroll
+    for (int j = 0; j < kQuadCh; ++j) {
+      const int c = max(0, min(cg * kQuadCh + j, nreal - 1));  // (padding channels re-read a real one, masked below)
+      if (F16) {
+        uint2 v;
+        __builtin_memcpy(&v, xg + (static_cast<size_t>(base) + static_cast<size_t>(c) * plane_i) * 2, 8);
+        g[2 * j] = v.x;
+        g[2 * j + 1] = v.y;
+      } else {
+        uint32_t v;
+        __builtin_memcpy(&v, xg + base + static_cast<size_t>(c) * plane_i, 4);
+        g[j] = v;
+      }
+    }
+  };
+  // the chunk in the registers -> the LDS image [pixel][k]
+  auto commit_quad = [&] {
+    uint32_t out[4][2];  // per pixel of the quad: this thread's 8 bytes
+    bool ok[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ok[i] = q_row && static_cast<unsigned>(q_s + i) < static_cast<unsigned>(a.W);
+    if (F16) {
+      // byte k of the shifted pair = byte (k + 2 shift) mod 8 of the eight loaded (added per byte, no carries: at most 7 + 7)
+      const uint32_t turn = static_cast<uint32_t>((2 * q_shift) & 7) * 0x01010101u;
+      const uint32_t sel0 = (0x03020100u + turn) & 0x07070707u;
+      const uint32_t sel1 = (0x07060504u + turn) & 0x07070707u;
+      uint32_t lo[4], hi[4];  // per channel: pixels 0, 1 and 2, 3
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        lo[j] = __builtin_amdgcn_perm(g[2 * j + 1], g[2 * j], sel0);
+        hi[j] = __builtin_amdgcn_perm(g[2 * j + 1], g[2 * j], sel1);
+      }
+      const uint32_t m0 = q_n >= 2 ? ~0u : (q_n == 1 ? 0xffffu : 0u), m1 = q_n >= 4 ? ~0u : (q_n == 3 ? 0xffffu : 0u);
+      out[0][0] = __builtin_amdgcn_perm(lo[1], lo[0], 0x05040100) & m0;
+      out[0][1] = __builtin_amdgcn_perm(lo[3], lo[2], 0x05040100) & m1;
+      out[1][0] = __builtin_amdgcn_perm(lo[1], lo[0], 0x07060302) & m0;
+      out[1][1] = __builtin_amdgcn_perm(lo[3], lo[2], 0x07060302) & m1;
+      out[2][0] = __builtin_amdgcn_perm(hi[1], hi[0], 0x05040100) & m0;
+      out[2][1] = __builtin_amdgcn_perm(hi[3], hi[2], 0x05040100) & m1;
+      out[3][0] = __builtin_amdgcn_perm(hi[1], hi[0], 0x07060302) & m0;
+      out[3][1] = __builtin_amdgcn_perm(hi[3], hi[2], 0x07060302) & m1;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (!ok[i]) out[i][0] = out[i][1] = 0;
+    } else {
+      // pixel i = byte (i + shift) mod 4 of the four loaded (added per byte, no carries: at most 3 + 3)
+      const uint32_t sel = (0x03020100u + static_cast<uint32_t>(q_shift & 3) * 0x01010101u) & 0x03030303u;
+      uint32_t e8[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) e8[j] = __builtin_amdgcn_perm(g[j], g[j], sel) ^ static_cast<uint32_t>(a.xor_mask4);
+      const int na = max(0, min(q_n, 4)), nb = max(0, min(q_n - 4, 4));
+      const uint32_t ma = na >= 4 ? ~0u : (1u << (8 * na)) - 1u, mb = nb >= 4 ? ~0u : (1u << (8 * nb)) - 1u;
+      const uint32_t pad = q_live ? static_cast<uint32_t>(a.pad_fill4) : 0u;
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const uint32_t lo01 = __builtin_amdgcn_perm(e8[4 * b + 1], e8[4 * b], 0x05010400);
+        const uint32_t hi01 = __builtin_amdgcn_perm(e8[4 * b + 1], e8[4 * b], 0x07030602);
+        const uint32_t lo23 = __builtin_amdgcn_perm(e8[4 * b + 3], e8[4 * b + 2], 0x05010400);
+        const uint32_t hi23 = __builtin_amdgcn_perm(e8[4 * b + 3], e8[4 * b + 2], 0x07030602);
+        out[0][b] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100);
+        out[1][b] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302);
+        out[2][b] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100);
+        out[3][b] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302);
+        const uint32_t m = b ? mb : ma;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) out[i][b] = (ok[i] ? out[i][b] : pad) & m;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      *reinterpret_cast<uint2*>(a_lds + (4 * q + i) * kRowStride + half * 32 + cg * 8) = make_uint2(out[i][0], out[i][1]);
+  };
+
   const int row = lane & 31, fh = lane >> 5;
   v16i acc_i[OT];
   v16f acc_f[OT];
@@ -149,20 +248,33 @@ __global__ void __launch_bounds__(kThreads) ConvGemmKernel(GemmArgs a) {
     }
   const v4i fz = {a.neg_zws4, a.neg_zws4, a.neg_zws4, a.neg_zws4};
 
-  gather(0);
+  // the weights of a chunk travel like its activations: into registers under the MFMAs of the chunk before
+  uint4 w16 = make_uint4(0, 0, 0, 0);
+  auto fetch_weights = [&](int chunk) {
+    if (tid < OT * 128)
+      w16 = *reinterpret_cast<const uint4*>(wsrc + static_cast<size_t>(chunk) * (OT * 32 * kChunkBytes) + tid * 16);
+  };
+  if (QUAD) gather_quad(0);
+  else gather(0);
+  fetch_weights(0);
   for (int chunk = 0; chunk < a.chunks; ++chunk) {
-    // registers -> LDS, weights global -> LDS
+    // registers -> LDS
     {
-      uint8_t* dst = a_lds + px * kRowStride + half * 32;
-      *reinterpret_cast<uint4*>(dst) = make_uint4(g[0], g[1], g[2], g[3]);
-      *reinterpret_cast<uint4*>(dst + 16) = make_uint4(g[4], g[5], g[6], g[7]);
-      if (tid < OT * 128) {
-        const uint4 w16 = *reinterpret_cast<const uint4*>(wsrc + static_cast<size_t>(chunk) * (OT * 32 * kChunkBytes) + tid * 16);
-        *reinterpret_cast<uint4*>(b_lds + (tid >> 2) * kRowStride + (tid & 3) * 16) = w16;
+      if (QUAD) {
+        commit_quad();
+      } else {
+        uint8_t* dst = a_lds + px * kRowStride + half * 32;
+        *reinterpret_cast<uint4*>(dst) = make_uint4(g[0], g[1], g[2], g[3]);
+        *reinterpret_cast<uint4*>(dst + 16) = make_uint4(g[4], g[5], g[6], g[7]);
       }
+      if (tid < OT * 128) *reinterpret_cast<uint4*>(b_lds + (tid >> 2) * kRowStride + (tid & 3) * 16) = w16;
     }
     __syncthreads();
-    if (chunk + 1 < a.chunks) gather(chunk + 1);
+    if (chunk + 1 < a.chunks) {
+      if (QUAD) gather_quad(chunk + 1);
+      else gather(chunk + 1);
+      fetch_weights(chunk + 1);
+    }
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
       const uint8_t* ap = a_lds + (wave * 32 + row) * kRowStride + ks * 32 + fh * 16;
@@ -232,6 +344,7 @@ struct Plan {
   dim3 grid;
   int ot;
   bool f16;
+  bool quad;  // unit column stride, output rows of whole pixel quads, at least four input columns
 };
 
 int ConvGemmRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
@@ -243,13 +356,16 @@ int ConvGemmRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t
   a.aligned4 = a.aligned4 && (reinterpret_cast<uintptr_t>(out) & need) == 0;
   if (plan->f16 && ((reinterpret_cast<uintptr_t>(in0) | reinterpret_cast<uintptr_t>(out)) & 1))
     return SetError(TVX_E_INVALID, "conv2d_gemm_f16: tensors must be 2-byte aligned");
+  const dim3 block(kThreads);
+#define TVX_LAUNCH(F, O, Q) hipLaunchKernelGGL((ConvGemmKernel<F, O, Q>), plan->grid, block, 0, st, a)
   if (plan->f16) {
-    if (plan->ot == 2) hipLaunchKernelGGL((ConvGemmKernel<true, 2>), plan->grid, dim3(kThreads), 0, st, a);
-    else hipLaunchKernelGGL((ConvGemmKernel<true, 1>), plan->grid, dim3(kThreads), 0, st, a);
+    if (plan->quad) { if (plan->ot == 2) TVX_LAUNCH(true, 2, true); else TVX_LAUNCH(true, 1, true); }
+    else { if (plan->ot == 2) TVX_LAUNCH(true, 2, false); else TVX_LAUNCH(true, 1, false); }
   } else {
-    if (plan->ot == 2) hipLaunchKernelGGL((ConvGemmKernel<false, 2>), plan->grid, dim3(kThreads), 0, st, a);
-    else hipLaunchKernelGGL((ConvGemmKernel<false, 1>), plan->grid, dim3(kThreads), 0, st, a);
+    if (plan->quad) { if (plan->ot == 2) TVX_LAUNCH(false, 2, true); else TVX_LAUNCH(false, 1, true); }
+    else { if (plan->ot == 2) TVX_LAUNCH(false, 2, false); else TVX_LAUNCH(false, 1, false); }
   }
+#undef TVX_LAUNCH
   TVX_HIP_CHECK(hipGetLastError());
   return TVX_OK;
 }
@@ -371,6 +487,8 @@ int ConvGemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, cons
   plan.grid = dim3(static_cast<unsigned>((hw + kPixels - 1) / kPixels), static_cast<unsigned>(groups * tiles), d->batch);
   plan.ot = ot;
   plan.f16 = f16;
+  plan.quad = d->stride_w == 1 && d->out_w % 4 == 0 && d->in_w >= 4;
+  if (const char* f = getenv("TVX_CONV_GEMM_QUAD")) plan.quad = plan.quad && atoi(f) != 0;  // tuning aid: 0 = the gather by elements
   op->host_blob.resize(sizeof(Plan));
   std::memcpy(op->host_blob.data(), &plan, sizeof(Plan));
   op->run = ConvGemmRun;
