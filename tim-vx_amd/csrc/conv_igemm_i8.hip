@@ -645,6 +645,9 @@ ConvPersistKernel(ConvArgs a) {
           }
 #pragma unroll
           for (int j = 0; j < OT; ++j) acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f, wr[ks][j], acc[j], 0, 0, 0);
+          // a k-step's instructions stay in their k-step: the scheduler otherwise pulls the pixel sums of the fragment
+          // just requested in front of the MFMAs on the older ones, and every k-step waits out a whole LDS round trip
+          __builtin_amdgcn_sched_barrier(0);
         }
         if (i == 0) TVX_TS(3 + ts_it * 8);
         if (ZP) {
