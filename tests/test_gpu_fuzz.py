@@ -156,6 +156,34 @@ def test_fully_connected_sweep(oracle):
         assert np.array_equal(got, want), (i, m, k, n, mode, act)
 
 
+def test_fully_connected_tiled_sweep(oracle):
+    """The 256 x 256 tile kernel (more than 2^18 outputs): ragged last tiles in both directions, reductions from
+    one 16-byte chunk to nine k-tiles with every tail, uint8 and int8 activations with and without a uniform weight
+    zero point (re-bias and row sums inside the kernel), per-channel weights."""
+    rng = np.random.default_rng(0xFD)
+    for i in range(24):
+        m, n = int(rng.integers(513, 1100)), int(rng.integers(513, 1100))
+        k = 16 * int(rng.integers(1, 80))
+        mode = str(rng.choice(["u8", "i8pc", "u8pc", "i8zp"]))
+        in_dt = 0 if mode.startswith("u8") else 1
+        w_dt = 0 if mode == "u8" else 1
+        x, w = rand_q(rng, m * k, in_dt), rand_q(rng, n * k, w_dt)
+        b = rng.integers(-16384, 16385, n).astype(np.int32)
+        if mode == "u8":
+            wq = (0.01, int(rng.integers(100, 157)), None)
+        elif mode == "i8zp":
+            wq = (0.01, int(rng.integers(-20, 21)), None)
+        else:
+            wq = (1.0, 0, np.exp(rng.uniform(np.log(0.001), np.log(0.02), n)).astype(np.float32))
+        kws = dict(m=m, k=k, n=n, in_dtype=in_dt, w_dtype=w_dt, out_dtype=in_dt,
+                   in_q=(0.02, int(rng.integers(100, 157)) if in_dt == 0 else int(rng.integers(-9, 10))), w_q=wq,
+                   out_q=(float(np.float32(0.02 * 0.01 * 40 * np.sqrt(k))), 5 if in_dt == 0 else -3))
+        act = int(rng.integers(0, 3))
+        want = oracle.fully_connected(x, w, b, act=act, **kws)
+        got = TC.gpu_fully_connected(x, w, b, act=act, want_kernel="fc_mfma_i8_256x256x128", **kws)
+        assert np.array_equal(got, want), (i, m, k, n, mode, act, int((got != want).sum()))
+
+
 def test_pool2d_sweep(oracle):
     rng = np.random.default_rng(0xB0)
     for i in range(80):
