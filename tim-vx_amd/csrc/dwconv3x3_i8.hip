@@ -41,14 +41,6 @@ struct DwArgs {
   int xor_mask, pad_fill, zws, out_zp, lo, hi;
 };
 
-// bytes [idx, idx + 4) of the little-endian byte array formed by arr[0], arr[1], ...
-template <int IDX, int N>
-__device__ __forceinline__ int Window(const int (&arr)[N]) {
-  constexpr int d = IDX / 4, sh = IDX % 4;
-  static_assert(d + (sh ? 1 : 0) < N, "window outside the loaded dwords");
-  if (sh == 0) return arr[d];
-  return __builtin_amdgcn_alignbyte(arr[d + 1], arr[d], sh);
-}
 
 
 // S = stride (1 or 2, both directions), PL = left padding (0 or 1)

@@ -64,65 +64,6 @@ struct DwPwArgs {
   int add_za, add_zb, add_zo, add_lo, add_hi;
 };
 
-// Four accumulators of one channel requantized together. `ties` (wave-uniform: a kernel argument) tells whether any
-// accumulator of the operator can land on an exact .5: only then is the round-half-even fix-up executed.
-__device__ __forceinline__ void Requant8x4(const int (&v)[4], const v4i& q, int zp, int lo, int hi, int ties,
-                                           int (&out)[4]) {
-  int h[4], r[4];
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    h[e] = __mulhi(v[e], q[0]);
-    r[e] = (h[e] + q[2]) >> q[1];
-  }
-  if (ties) {
-    const int half = 1 << (q[1] - 1);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const bool tie = ((h[e] & (2 * half - 1)) == half) && ((v[e] & q[3]) == 0);
-      if (tie && ((r[e] - zp) & 1)) --r[e];
-    }
-  }
-#pragma unroll
-  for (int e = 0; e < 4; ++e) out[e] = Med3(r[e], lo, hi);
-}
-
-__device__ __forceinline__ uint32_t AddResidual4(const DwPwArgs& a, uint32_t t4, uint32_t r4) {
-  int out[4];
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    int t = (t4 >> (8 * e)) & 0xff, r = (r4 >> (8 * e)) & 0xff;
-    if (a.add_signed) {
-      t = static_cast<int8_t>(t);
-      r = static_cast<int8_t>(r);
-    }
-    const int av = a.add_mode == 1 ? t : r, bv = a.add_mode == 1 ? r : t;
-    const double tb = __dmul_rn(static_cast<double>(bv - a.add_zb), a.add_rb);
-    const double s = fma(static_cast<double>(av - a.add_za), a.add_ra, tb);
-    out[e] = Med3(static_cast<int>(rint(s)) + a.add_zo, a.add_lo, a.add_hi);
-  }
-  return PackBytes(out[0], out[1], out[2], out[3]);
-}
-
-__device__ __forceinline__ void Transpose4x4(const uint32_t in[4], uint32_t out[4]) {
-  const uint32_t ab_lo = __builtin_amdgcn_perm(in[1], in[0], 0x05010400);
-  const uint32_t ab_hi = __builtin_amdgcn_perm(in[1], in[0], 0x07030602);
-  const uint32_t cd_lo = __builtin_amdgcn_perm(in[3], in[2], 0x05010400);
-  const uint32_t cd_hi = __builtin_amdgcn_perm(in[3], in[2], 0x07030602);
-  out[0] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x05040100);
-  out[1] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x07060302);
-  out[2] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x05040100);
-  out[3] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x07060302);
-}
-
-// bytes [idx, idx + 4) of the little-endian byte array formed by arr[0], arr[1], ...
-template <int IDX, int N>
-__device__ __forceinline__ int Window(const int (&arr)[N]) {
-  constexpr int d = IDX / 4, sh = IDX % 4;
-  static_assert(d + (sh ? 1 : 0) < N, "window outside the loaded dwords");
-  if (sh == 0) return arr[d];
-  return __builtin_amdgcn_alignbyte(arr[d + 1], arr[d], sh);
-}
-
 // Four columns x RPT output rows of one depthwise channel plane, in two steps so that the loads of several
 // channels can be in flight together; S = stride, PL = left padding.
 template <int S, int RPT>

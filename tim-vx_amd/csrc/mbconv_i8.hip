@@ -79,52 +79,6 @@ struct MbArgs {
 #define TVX_TS(slot) do { } while (0)
 #endif
 
-__device__ __forceinline__ void Requant8x4(const int (&v)[4], const v4i& q, int zp, int lo, int hi, int ties, int (&out)[4]) {
-  int h[4], r[4];
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    h[e] = __mulhi(v[e], q[0]);
-    r[e] = (h[e] + q[2]) >> q[1];
-  }
-  if (ties) {  // (wave-uniform) some accumulator of the operator can land on an exact .5: round half to even
-    const int half = 1 << (q[1] - 1);
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const bool tie = ((h[e] & (2 * half - 1)) == half) && ((v[e] & q[3]) == 0);
-      if (tie && ((r[e] - zp) & 1)) --r[e];
-    }
-  }
-#pragma unroll
-  for (int e = 0; e < 4; ++e) out[e] = Med3(r[e], lo, hi);
-}
-
-__device__ __forceinline__ int AddResidual1(const MbArgs& a, int t, int r) {
-  if (a.add_signed) {
-    t = static_cast<int8_t>(t);
-    r = static_cast<int8_t>(r);
-  }
-  const int av = a.add_mode == 1 ? t : r, bv = a.add_mode == 1 ? r : t;
-  const double tb = __dmul_rn(static_cast<double>(bv - a.add_zb), a.add_rb);
-  const double s = fma(static_cast<double>(av - a.add_za), a.add_ra, tb);
-  return Med3(static_cast<int>(rint(s)) + a.add_zo, a.add_lo, a.add_hi);
-}
-
-__device__ __forceinline__ uint32_t AddResidual4(const MbArgs& a, uint32_t t4, uint32_t r4) {
-  int out[4];
-#pragma unroll
-  for (int e = 0; e < 4; ++e) out[e] = AddResidual1(a, (t4 >> (8 * e)) & 0xff, (r4 >> (8 * e)) & 0xff);
-  return PackBytes(out[0], out[1], out[2], out[3]);
-}
-
-// bytes [IDX, IDX + 4) of the little-endian byte array formed by arr[0], arr[1], ...
-template <int IDX, int N>
-__device__ __forceinline__ int Window(const int (&arr)[N]) {
-  constexpr int d = IDX / 4, sh = IDX % 4;
-  static_assert(d + (sh ? 1 : 0) < N, "window outside the row registers");
-  if (sh == 0) return arr[d];
-  return __builtin_amdgcn_alignbyte(arr[d + 1], arr[d], sh);
-}
-
 // Window of output column J of a depthwise row: W input columns, stride S, SAME padding (one column left at
 // stride 1, none at stride 2); byte 0 of `row` is the column under the first output's leftmost tap. Columns past
 // the row's end recompute the last one (nobody stores them).

@@ -63,35 +63,6 @@ struct PwArgs {
   int add_za, add_zb, add_zo, add_lo, add_hi;
 };
 
-// Four output bytes of the convolution and the four residual bytes at the same place -> four sums.
-__device__ __forceinline__ uint32_t AddResidual4(const PwArgs& a, uint32_t t4, uint32_t r4) {
-  int out[4];
-#pragma unroll
-  for (int e = 0; e < 4; ++e) {
-    int t = (t4 >> (8 * e)) & 0xff, r = (r4 >> (8 * e)) & 0xff;
-    if (a.add_signed) {
-      t = static_cast<int8_t>(t);
-      r = static_cast<int8_t>(r);
-    }
-    const int av = a.add_mode == 1 ? t : r, bv = a.add_mode == 1 ? r : t;
-    const double tb = __dmul_rn(static_cast<double>(bv - a.add_zb), a.add_rb);
-    const double s = fma(static_cast<double>(av - a.add_za), a.add_ra, tb);
-    out[e] = Med3(static_cast<int>(rint(s)) + a.add_zo, a.add_lo, a.add_hi);
-  }
-  return PackBytes(out[0], out[1], out[2], out[3]);
-}
-
-// 4 dwords = 4 channels x 4 pixels (pixel in the byte lanes) -> 4 dwords = 4 pixels x 4 channels.
-__device__ __forceinline__ void Transpose4x4(const uint32_t in[4], uint32_t out[4]) {
-  const uint32_t ab_lo = __builtin_amdgcn_perm(in[1], in[0], 0x05010400);  // a0 b0 a1 b1
-  const uint32_t ab_hi = __builtin_amdgcn_perm(in[1], in[0], 0x07030602);  // a2 b2 a3 b3
-  const uint32_t cd_lo = __builtin_amdgcn_perm(in[3], in[2], 0x05010400);
-  const uint32_t cd_hi = __builtin_amdgcn_perm(in[3], in[2], 0x07030602);
-  out[0] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x05040100);  // a0 b0 c0 d0
-  out[1] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x07060302);  // a1 b1 c1 d1
-  out[2] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x05040100);
-  out[3] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x07060302);
-}
 
 // KP: flat pixels per workgroup: 128, or 32 when the whole batch has few pixels and more,
 //     smaller workgroups are needed to fill the chip.

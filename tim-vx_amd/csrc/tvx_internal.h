@@ -138,6 +138,73 @@ __device__ __forceinline__ int Requant8(int v, const tvx_v4i& q, int zp, int lo,
   return Med3(r, lo, hi);
 }
 
+// Four accumulators of one channel requantized together (the 32-bit record forms). `ties` (wave-uniform: a kernel
+// argument) tells whether any accumulator of the operator can land on an exact .5: only then is the round-half-even
+// fix-up executed.
+__device__ __forceinline__ void Requant8x4(const int (&v)[4], const tvx_v4i& q, int zp, int lo, int hi, int ties,
+                                           int (&out)[4]) {
+  int h[4], r[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    h[e] = __mulhi(v[e], q[0]);
+    r[e] = (h[e] + q[2]) >> q[1];
+  }
+  if (ties) {
+    const int half = 1 << (q[1] - 1);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const bool tie = ((h[e] & (2 * half - 1)) == half) && ((v[e] & q[3]) == 0);
+      if (tie && ((r[e] - zp) & 1)) --r[e];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) out[e] = Med3(r[e], lo, hi);
+}
+
+// The quantized Add fused behind a convolution: one code of the convolution's result (t) and one of the residual
+// (r) -> the code of their sum, in the arithmetic of the stand-alone Add. `Args` carries add_mode (1: a = t, b = r;
+// 2: a = r, b = t), add_signed, the zero points add_za / add_zb / add_zo, the ratios add_ra / add_rb and the clamp.
+template <class Args>
+__device__ __forceinline__ int AddResidual1(const Args& a, int t, int r) {
+  if (a.add_signed) {
+    t = static_cast<int8_t>(t);
+    r = static_cast<int8_t>(r);
+  }
+  const int av = a.add_mode == 1 ? t : r, bv = a.add_mode == 1 ? r : t;
+  const double tb = __dmul_rn(static_cast<double>(bv - a.add_zb), a.add_rb);
+  const double s = fma(static_cast<double>(av - a.add_za), a.add_ra, tb);
+  return Med3(static_cast<int>(rint(s)) + a.add_zo, a.add_lo, a.add_hi);
+}
+// ... on four codes in the bytes of a dword
+template <class Args>
+__device__ __forceinline__ uint32_t AddResidual4(const Args& a, uint32_t t4, uint32_t r4) {
+  int out[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) out[e] = AddResidual1(a, static_cast<int>((t4 >> (8 * e)) & 0xff), static_cast<int>((r4 >> (8 * e)) & 0xff));
+  return PackBytes(out[0], out[1], out[2], out[3]);
+}
+
+// 4 dwords = 4 channels x 4 pixels (pixel in the byte lanes) -> 4 dwords = 4 pixels x 4 channels.
+__device__ __forceinline__ void Transpose4x4(const uint32_t in[4], uint32_t out[4]) {
+  const uint32_t ab_lo = __builtin_amdgcn_perm(in[1], in[0], 0x05010400);  // a0 b0 a1 b1
+  const uint32_t ab_hi = __builtin_amdgcn_perm(in[1], in[0], 0x07030602);  // a2 b2 a3 b3
+  const uint32_t cd_lo = __builtin_amdgcn_perm(in[3], in[2], 0x05010400);
+  const uint32_t cd_hi = __builtin_amdgcn_perm(in[3], in[2], 0x07030602);
+  out[0] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x05040100);  // a0 b0 c0 d0
+  out[1] = __builtin_amdgcn_perm(cd_lo, ab_lo, 0x07060302);
+  out[2] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x05040100);
+  out[3] = __builtin_amdgcn_perm(cd_hi, ab_hi, 0x07060302);
+}
+
+// bytes [IDX, IDX + 4) of the little-endian byte array formed by arr[0], arr[1], ...
+template <int IDX, int N>
+__device__ __forceinline__ int Window(const int (&arr)[N]) {
+  constexpr int d = IDX / 4, sh = IDX % 4;
+  static_assert(d + (sh ? 1 : 0) < N, "window outside the loaded dwords");
+  if (sh == 0) return arr[d];
+  return __builtin_amdgcn_alignbyte(arr[d + 1], arr[d], sh);
+}
+
 // ---- host helpers ------------------------------------------------------------
 // Builds the records above for `alloc` channels (the first `channels` from the
 // operator's mult/shift tables, the rest neutral) and returns the flavour.
