@@ -60,6 +60,7 @@ struct ConvArgs {
   // persistent variant only
   int total_tiles;       // batch * tiles_per_image
   int halo_bytes;        // one of the two halo buffers
+  int off_halo1;         // the second halo buffer (persistent variant: the staging tile lies between the two)
   int off_out;           // epilogue staging tile
   int tap_off[40];       // halo byte offset of k-step ks (both fragment halves lie in one tap: + 16 * half)
 #ifdef TVX_CONV_TIMESTAMPS
@@ -569,8 +570,10 @@ ConvPersistKernel(ConvArgs a) {
   auto lds_barrier = [] { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
   TVX_TS(0);
-  // ---- prologue: the first tile's rows on their way, the weights by DMA into the (still empty) staging tile and halo buffers,
-  // from there into every wavefront's registers; then the rows into the first halo buffer ----
+  // ---- prologue: the first tile's rows on their way, the weights by DMA into the (still empty) staging tile and second
+  // halo buffer, which lie side by side; from there into every wavefront's registers - 288 KB per CU through LDS,
+  // a microsecond of LDS bandwidth with the vector units idle - while the rows are transposed into the first halo
+  // buffer - vector work with LDS nearly idle: half of the weight reads are issued in front of each half of the rows ----
   int d0[PHASES][NBP][4];
 #pragma unroll
   for (int ph = 0; ph < PHASES; ++ph)
@@ -588,16 +591,20 @@ ConvPersistKernel(ConvArgs a) {
   v4i wr[KSTEPS][OT];
   {
     const int8_t* w_row = lds + a.off_out + frag_row * a.kstride + frag_half * 16;
+    constexpr int kPerPhase = (KSTEPS + PHASES - 1) / PHASES;
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks)
+    for (int ph = 0; ph < PHASES; ++ph) {
 #pragma unroll
-      for (int j = 0; j < OT; ++j) wr[ks][j] = *reinterpret_cast<const v4i*>(w_row + j * 32 * a.kstride + ks * 32);
+      for (int ks = ph * kPerPhase; ks < (ph + 1) * kPerPhase; ++ks)
+        if (ks < KSTEPS) {
+#pragma unroll
+          for (int j = 0; j < OT; ++j) wr[ks][j] = *reinterpret_cast<const v4i*>(w_row + j * 32 * a.kstride + ks * 32);
+        }
+      store_halo(d0[ph], t, lds + a.off_halo, ph * NBP);
+    }
   }
-  lds_barrier();  // every wavefront has its weights: the buffers are free
-#pragma unroll
-  for (int ph = 0; ph < PHASES; ++ph) store_halo(d0[ph], t, lds + a.off_halo, ph * NBP);
   store_pad_columns(t, lds + a.off_halo);
-  lds_barrier();
+  lds_barrier();  // the first halo tile is complete, every wavefront has its weights: staging tile and second buffer are free
   TVX_TS(1);
 
   int buf = 0;
@@ -609,7 +616,7 @@ ConvPersistKernel(ConvArgs a) {
     if (has_next && has_patch) pull_into_l2(tn);
     int n, p0, p_end, r0, ih0, rows_needed;
     tile_geometry(t, &n, &p0, &p_end, &r0, &ih0, &rows_needed);
-    const int8_t* halo = lds + a.off_halo + buf * a.halo_bytes;
+    const int8_t* halo = lds + (buf ? a.off_halo1 : a.off_halo);
     TVX_TS(2 + ts_it * 8);
 
     // ---- one 32-pixel MFMA tile at a time: reduction, then requantization into the staging tile ----
@@ -678,7 +685,7 @@ ConvPersistKernel(ConvArgs a) {
     }
     // ---- the next tile's rows: L2 -> registers -> the other halo buffer ----
     if (has_next) {
-      int8_t* halo_next = lds + a.off_halo + (buf ^ 1) * a.halo_bytes;
+      int8_t* halo_next = lds + (buf ? a.off_halo : a.off_halo1);
       if (has_patch) asm volatile("s_waitcnt vmcnt(0)" : "+v"(landing)::"memory");
 #pragma unroll
       for (int ph = 0; ph < PHASES; ++ph) {
@@ -1007,10 +1014,12 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
     pa.off_sx = 0;
     pa.off_rq = 512;
     pa.off_bias = pa.off_rq + 64 * 16;
-    pa.off_out = pa.off_bias + 64 * 4;
-    pa.off_halo = pa.off_out + RoundUp(pa.oct * pa.out_stride, 16);
+    // first halo buffer | staging tile | second halo buffer: the weights' DMA lands in the last two
+    pa.off_halo = pa.off_bias + 64 * 4;
+    pa.off_out = pa.off_halo + pa.halo_bytes;
+    pa.off_halo1 = pa.off_out + RoundUp(pa.oct * pa.out_stride, 16);
     // (the weights pass through the staging tile and the halo buffers on their way into the registers)
-    const int plds = std::max(pa.off_halo + 2 * pa.halo_bytes, pa.off_out + pa.w_chunks * 16);
+    const int plds = std::max(pa.off_halo1 + pa.halo_bytes, pa.off_out + pa.w_chunks * 16);
     if (plds > 80 * 1024) break;  // two workgroups per CU
     for (int ks = 0; ks < ksteps; ++ks) pa.tap_off[ks] = tapt[ks * 4];  // chunk 2 * ks (chunk 2 * ks + 1 follows it)
     bool halves_adjacent = true;
