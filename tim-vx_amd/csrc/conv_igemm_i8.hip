@@ -663,6 +663,13 @@ ConvPersistKernel(ConvArgs a) {
           if (frag_half == 0) sx_lds[frag_row] = a.zws * sx;
           __builtin_amdgcn_wave_barrier();
         }
+        // the lane's requantization records, read before the first store into the staging tile (behind a store the
+        // compiler has to read them again, and each read is a round trip the wavefront waits out)
+        // (not in the tie-testing form, whose extra temporaries leave no registers for them)
+        constexpr bool kRecordsAhead = RQ != kRqFast;
+        v4i rqj[OT];
+#pragma unroll
+        for (int j = 0; j < OT; ++j) rqj[j] = kRecordsAhead ? rq_lds[j * 32 + frag_row] : v4i{0, 0, 0, 0};
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
           const int pl = pt * 32 + 8 * g + 4 * frag_half;
@@ -671,7 +678,7 @@ ConvPersistKernel(ConvArgs a) {
 #pragma unroll
           for (int j = 0; j < OT; ++j) {
             const int ocl = j * 32 + frag_row;
-            const v4i rq = rq_lds[ocl];
+            const v4i rq = kRecordsAhead ? rqj[j] : rq_lds[ocl];
             int r4[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e)
