@@ -121,6 +121,25 @@ def fc_cfg5(T, rng):
                 bound="mfma", oracle=None)
 
 
+def fc_cfg5_u8(T, rng):
+    """The same shape with uint8 activations and uint8 weights under a uniform zero point: the operand kinds of
+    the reference's own quantized tests (the kernel re-biases the activations and sums their rows on its way)."""
+    m, k, n = 8192, 4096, 4096
+    x = rng.integers(0, 256, m * k, dtype=np.uint8)
+    wt = rng.integers(0, 256, n * k, dtype=np.uint8)
+    b = rng.integers(-16384, 16385, n).astype(np.int32)
+    d = T.FcDesc()
+    d.m, d.k, d.n = m, k, n
+    d.in_dtype = d.w_dtype = d.out_dtype = T.U8
+    d.in_scale, d.in_zp = 0.02, 121
+    d.w_scale, d.w_zp = 0.01, 131
+    d.out_scale, d.out_zp = 1.2, 128
+    op = T.fully_connected_create(d, wt, b)
+    return dict(name="fc_u8_asymmetric_m8192_k4096_n4096", op=op, inputs=(x,), out_elems=m * n,
+                out_dtype=np.uint8, ops=2 * m * k * n, algo_bytes=m * k + n * k + m * n + 4 * n,
+                bound="mfma", oracle=None)
+
+
 def fc_cfg5_f16(T, rng):
     m, k, n = 8192, 4096, 4096
     x = rng.standard_normal(m * k, dtype=np.float32).astype(np.float16)
@@ -467,7 +486,7 @@ def main():
         line["roofline"]["traffic_stale"] = True
     if not args.no_extra:
         extra = {}
-        for make in (fc_cfg5, fc_cfg5_f16, dw_cfg3a, pw_cfg3b, dwpw_cfg3, conv_cfg2_b256, conv_f16, conv_grouped, pool_3x3_s2,
+        for make in (fc_cfg5, fc_cfg5_u8, fc_cfg5_f16, dw_cfg3a, pw_cfg3b, dwpw_cfg3, conv_cfg2_b256, conv_f16, conv_grouped, pool_3x3_s2,
                      pool_lenet_b256, pool_global_avg):
             w2 = make(T, rng)
             steps2 = max(5, min(args.steps, 50))
