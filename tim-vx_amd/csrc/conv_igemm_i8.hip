@@ -831,10 +831,7 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   a.dh = d->dilation_h; a.dw = d->dilation_w; a.pad_t = d->pad_top; a.pad_l = d->pad_left;
   const int taps = a.kh * a.kw;
   const int oc_pad = RoundUp(a.OC, 32);
-  const int ot = oc_pad <= 32 ? 1 : (oc_pad <= 64 ? 2 : 4);
-  a.oct = 32 * ot;
-  const int oc_blocks = (oc_pad + a.oct - 1) / a.oct;
-  const int oc_alloc = oc_blocks * a.oct;
+  int ot = oc_pad <= 32 ? 1 : (oc_pad <= 64 ? 2 : 4);
   // pixel tile: the multiple of 32 (<= 256) wasting the fewest MFMA rows
   const int hw = a.OH * a.OW;
   int best_p = 32;
@@ -844,6 +841,40 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
     const double eff = static_cast<double>(hw) / (static_cast<double>(tiles) * p);
     if (eff > best_eff + 1e-9) { best_eff = eff; best_p = p; }
   }
+  // Few pixels and many channels (256 -> 256 on 14 x 14, batch 32: 64 such workgroups on 256 CUs): when that
+  // choice fills less than half of the chip's workgroup slots, trade tile size for workgroups. A workgroup's
+  // critical path is modelled as its MFMA blocks per wavefront (32-pixel tiles / 4 wavefronts x 32-channel
+  // tiles) plus two blocks' worth of loads and barriers, the launch as that times the rounds the workgroups
+  // need on two slots per CU; ties go to the larger tiles (fewer halo copies).
+  {
+    int cus = 256;
+    hipDeviceProp_t prop;
+    int dev = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
+    const long long slots = 2ll * cus;
+    auto workgroups = [&](int ot_, int p_) {
+      return static_cast<long long>(d->batch) * ((hw + p_ - 1) / p_) * ((oc_pad + 32 * ot_ - 1) / (32 * ot_));
+    };
+    if (ot == 4 && workgroups(ot, best_p) < slots / 2) {  // (up to 64 output channels the choice above also decides the persistent variant)
+      auto cost = [&](int ot_, int p_) {
+        const long long rounds = (workgroups(ot_, p_) + slots - 1) / slots;
+        return rounds * (((p_ / 32 + 3) / 4) * ot_ + 2);
+      };
+      long long best_cost = cost(ot, best_p);
+      const int ot_max = ot;
+      for (int ot_ = ot_max; ot_ >= 1; ot_ /= 2)
+        for (int p_ = 256; p_ >= 32; p_ -= 32) {
+          if (p_ - 32 >= hw) continue;  // (a tile larger than the image needs)
+          const long long c = cost(ot_, p_);
+          if (c < best_cost) { best_cost = c; ot = ot_; best_p = p_; }
+        }
+    }
+  }
+  if (const char* f = getenv("TVX_IGEMM_OT")) { const int v = atoi(f); if ((v == 1 || v == 2 || v == 4) && 32 * v <= std::max(oc_pad, 32) * 2) ot = v; }  // tuning aid
+  if (const char* f = getenv("TVX_IGEMM_P")) { const int v = atoi(f); if (v >= 32 && v <= 256 && v % 32 == 0) best_p = v; }  // tuning aid
+  a.oct = 32 * ot;
+  const int oc_blocks = (oc_pad + a.oct - 1) / a.oct;
+  const int oc_alloc = oc_blocks * a.oct;
   a.P = best_p;
   a.PT = a.P / 32;
   a.tiles_per_image = (hw + a.P - 1) / a.P;
