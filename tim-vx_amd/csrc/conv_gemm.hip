@@ -107,10 +107,21 @@ __global__ void __launch_bounds__(kThreads) ConvGemmKernel(GemmArgs a) {
 
   // The reduction runs tap by tap, a tap's channels padded to whole half-chunks: the 32 bytes a thread gathers
   // belong to one tap (one validity test, one base address) and walk the channel planes.
+  // The window table's entry of this wavefront's half of a chunk (the same for all its lanes), read through the
+  // constant address space: a scalar load. As a vector load the compiler waits for it with every load in flight
+  // counted - the whole round trip in front of every chunk's gather.
+  auto table_entry = [&](int chunk) {
+    const __attribute__((address_space(4))) int* tab4 =
+        reinterpret_cast<const __attribute__((address_space(4))) int*>(reinterpret_cast<uintptr_t>(a.tab));
+    int2 e;
+    e.x = tab4[(chunk * 2 + half) * 2];
+    e.y = tab4[(chunk * 2 + half) * 2 + 1];
+    return e;
+  };
   uint32_t g[8];  // the 32 bytes of this thread's pixel row and chunk half
   const int plane_i = a.H * a.W;
   auto gather = [&](int chunk) {
-    const int2 e = a.tab[chunk * 2 + half];  // (the same for the whole wavefront)
+    const int2 e = table_entry(chunk);
     const int dy = e.y & 0xff, dx = (e.y >> 8) & 0xff;
     const int nreal = e.y >> 16;              // real channels in this half-chunk (the rest is padding)
     const bool inside = p_live && static_cast<unsigned>(ih0 + dy) < static_cast<unsigned>(a.H) &&
@@ -155,7 +166,7 @@ __global__ void __launch_bounds__(kThreads) ConvGemmKernel(GemmArgs a) {
   int q_shift = 0, q_s = 0, q_n = 0;  // of the chunk in flight: columns clamped away, first column, real channels from this thread's first
   bool q_row = false;
   auto gather_quad = [&](int chunk) {
-    const int2 e = a.tab[chunk * 2 + half];
+    const int2 e = table_entry(chunk);
     const int dy = e.y & 0xff, dx = (e.y >> 8) & 0xff;
     const int nreal = e.y >> 16;
     q_row = q_live && static_cast<unsigned>(q_ih0 + dy) < static_cast<unsigned>(a.H);
