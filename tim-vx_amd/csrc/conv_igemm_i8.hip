@@ -61,6 +61,7 @@ struct ConvArgs {
   int total_tiles;       // batch * tiles_per_image
   int halo_bytes;        // one of the two halo buffers
   int off_halo1;         // the second halo buffer (persistent variant: the staging tile lies between the two)
+  uint32_t magic_ow;     // persistent variant: ceil(2^32 / OW), exact for every pixel index of an image (the host checks)
   int off_out;           // epilogue staging tile
   int tap_off[40];       // halo byte offset of k-step ks (both fragment halves lie in one tap: + 16 * half)
 #ifdef TVX_CONV_TIMESTAMPS
@@ -625,7 +626,7 @@ ConvPersistKernel(ConvArgs a) {
       const int pt = wave + 4 * i;
       if (pt < a.PT && p0 + pt * 32 < p_end) {
         const int p = min(p0 + pt * 32 + frag_row, p_end - 1);  // rows past the tile's end recompute its last pixel
-        const int oh = p / a.OW, ow = p - oh * a.OW;
+        const int oh = static_cast<int>(__umulhi(static_cast<uint32_t>(p), a.magic_ow)), ow = p - oh * a.OW;  // p / OW
         const int8_t* frag = halo + ((oh - r0) * a.sh * a.iwt + ow * a.sw) * a.pix_stride + frag_half * 16;
         // a lane's accumulators belong to one output channel per tile: they start from its folded bias
         v16i acc[OT];
@@ -1037,6 +1038,9 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
     }
     if (rows == 0) break;
     ConvArgs pa = a;
+    // the reciprocal the kernel divides pixel indices by the row length with: exact while p * OW < 2^32
+    if (a.OW < 2 || static_cast<uint64_t>(a.OH) * a.OW * a.OW >= (uint64_t{1} << 32)) break;
+    pa.magic_ow = static_cast<uint32_t>(((uint64_t{1} << 32) + a.OW - 1) / a.OW);
     pa.P = rows * a.OW;
     pa.PT = (pa.P + 31) / 32;
     pa.tiles_per_image = (a.OH + rows - 1) / rows;
