@@ -62,6 +62,8 @@ struct ConvArgs {
   int halo_bytes;        // one of the two halo buffers
   int off_halo1;         // the second halo buffer (persistent variant: the staging tile lies between the two)
   uint32_t magic_ow;     // persistent variant: ceil(2^32 / OW), exact for every pixel index of an image (the host checks)
+  uint32_t magic_tpi;    // ... ceil(2^32 / tiles_per_image), exact for every tile index (0: one tile per image)
+  int rows;              // ... output rows of a tile
   int off_out;           // epilogue staging tile
   int tap_off[40];       // halo byte offset of k-step ks (both fragment halves lie in one tap: + 16 * half)
 #ifdef TVX_CONV_TIMESTAMPS
@@ -481,13 +483,13 @@ ConvPersistKernel(ConvArgs a) {
   const int xm = a.xor_mask;
 
   auto tile_geometry = [&](int tile_index, int* n, int* p0, int* p_end, int* r0, int* ih0, int* rows_needed) {
-    const int img = tile_index / a.tiles_per_image;
+    const int img = a.magic_tpi ? static_cast<int>(__umulhi(static_cast<uint32_t>(tile_index), a.magic_tpi)) : tile_index;
     const int tl = tile_index - img * a.tiles_per_image;
     *n = img;
     *p0 = tl * a.P;
     *p_end = min(*p0 + a.P, hw);
-    *r0 = *p0 / a.OW;
-    const int r1 = (*p_end - 1) / a.OW;
+    *r0 = tl * a.rows;  // (tiles are whole output rows)
+    const int r1 = min(*r0 + a.rows, a.OH) - 1;
     *ih0 = *r0 * a.sh - a.pad_t;
     *rows_needed = (r1 - *r0) * a.sh + (a.kh - 1) * a.dh + 1;
   };
@@ -1044,6 +1046,9 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
     pa.P = rows * a.OW;
     pa.PT = (pa.P + 31) / 32;
     pa.tiles_per_image = (a.OH + rows - 1) / rows;
+    pa.rows = rows;
+    if (static_cast<uint64_t>(d->batch) * pa.tiles_per_image * pa.tiles_per_image >= (uint64_t{1} << 32)) break;
+    pa.magic_tpi = pa.tiles_per_image > 1 ? static_cast<uint32_t>(((uint64_t{1} << 32) + pa.tiles_per_image - 1) / pa.tiles_per_image) : 0u;
     pa.iht = (rows - 1) * a.sh + (a.kh - 1) * a.dh + 1;
     plan.small = pa.iht <= 4;
     PersistFn fn = PersistKernel(ksteps, rq, plan.zp, plan.small);
