@@ -64,6 +64,7 @@ struct ConvArgs {
   uint32_t magic_ow;     // persistent variant: ceil(2^32 / OW), exact for every pixel index of an image (the host checks)
   uint32_t magic_tpi;    // ... ceil(2^32 / tiles_per_image), exact for every tile index (0: one tile per image)
   int rows;              // ... output rows of a tile
+  uint32_t blk_col, blk_chan;  // ... per wavefront w (byte w): w % w4_blocks and w / w4_blocks
   int off_out;           // epilogue staging tile
   int tap_off[40];       // halo byte offset of k-step ks (both fragment halves lie in one tap: + 16 * half)
 #ifdef TVX_CONV_TIMESTAMPS
@@ -470,8 +471,8 @@ ConvPersistKernel(ConvArgs a) {
   const int w4n = a.W / 4, c4n = a.cp / 4;
   const int row_bytes = a.iwt * a.pix_stride;
   const int blk = tid >> 6, in_blk = tid & 63;
-  const int w4 = (blk % a.w4_blocks) * 16 + (in_blk & 15);
-  const int c4 = (blk / a.w4_blocks) * 4 + (in_blk >> 4);
+  const int w4 = static_cast<int>((a.blk_col >> (8 * blk)) & 0xff) * 16 + (in_blk & 15);
+  const int c4 = static_cast<int>((a.blk_chan >> (8 * blk)) & 0xff) * 4 + (in_blk >> 4);
   const bool has_patch = w4 < w4n && c4 < c4n;
   const int pc = c4 * 4;
   const int hc = a.pad_l + w4 * 4;
@@ -1047,6 +1048,11 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
     pa.PT = (pa.P + 31) / 32;
     pa.tiles_per_image = (a.OH + rows - 1) / rows;
     pa.rows = rows;
+    pa.blk_col = pa.blk_chan = 0;
+    for (int wv = 0; wv < kThreads / 64; ++wv) {
+      pa.blk_col |= static_cast<uint32_t>(wv % pa.w4_blocks) << (8 * wv);
+      pa.blk_chan |= static_cast<uint32_t>(wv / pa.w4_blocks) << (8 * wv);
+    }
     if (static_cast<uint64_t>(d->batch) * pa.tiles_per_image * pa.tiles_per_image >= (uint64_t{1} << 32)) break;
     pa.magic_tpi = pa.tiles_per_image > 1 ? static_cast<uint32_t>(((uint64_t{1} << 32) + pa.tiles_per_image - 1) / pa.tiles_per_image) : 0u;
     pa.iht = (rows - 1) * a.sh + (a.kh - 1) * a.dh + 1;
