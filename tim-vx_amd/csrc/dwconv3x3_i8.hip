@@ -45,30 +45,33 @@ struct DwArgs {
 
 // S = stride (1 or 2, both directions), PL = left padding (0 or 1)
 // RPT: output rows a thread produces (more rows: fewer, fatter workgroups and fewer halo rows re-read)
-template <int S, int PL, bool BOXSUM, int RQ, int RPT>
+// CW: output columns a thread produces, 4 or 8 (8: one 64-bit load per input row, twice the bytes in flight
+// per lane; stride 1 only, rows and pointers multiples of eight bytes)
+template <int S, int PL, bool BOXSUM, int RQ, int RPT, int CW = 4>
 __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
-  const int plane = blockIdx.x;
-  const int c = plane % a.C;
+  // grid: (channel, image, block of row groups) - the channel comes without a division
+  const int c = blockIdx.x;
+  const int plane = blockIdx.y * a.C + c;
   const int tid = threadIdx.x;
   const int rgl = tid >> a.lpr_shift;
   const int w4 = tid & ((1 << a.lpr_shift) - 1);
-  const int oh0 = (blockIdx.y * a.rg_per_block + rgl) * RPT;
+  const int oh0 = (blockIdx.z * a.rg_per_block + rgl) * RPT;
+  // the channel's constants (scalar loads: the channel is the same for the whole workgroup)
+  const int wk0 = a.wpk[c * 4 + 0], wk1 = a.wpk[c * 4 + 1], wk2 = a.wpk[c * 4 + 2];
+  const bool box = BOXSUM && a.wpk[c * 4 + 3] != 0;  // a uniform branch, taken by few channels
+  const int bias = a.biasf[c];
+  const tvx_v4i q = a.rq[c];
   if (oh0 >= a.OH) return;  // whole rows of lanes leave together: neighbours stay consistent
 
   const uint8_t* xp = a.x + static_cast<size_t>(plane) * a.H * a.W;
   uint8_t* yp = a.y + static_cast<size_t>(plane) * a.OH * a.OW;
-  const int wk0 = a.wpk[c * 4 + 0], wk1 = a.wpk[c * 4 + 1], wk2 = a.wpk[c * 4 + 2];
-  // the channel is the same for the whole workgroup: a uniform branch, taken by few channels
-  const bool box = BOXSUM && __builtin_amdgcn_readfirstlane(a.wpk[c * 4 + 3]) != 0;
-  const int bias = a.biasf[c];
-  const tvx_v4i q = a.rq[c];
   const int in_dwords = a.W / 4;
 
   // input dwords under this thread's four outputs: S of them, starting at S * w4;
   // the byte array of a row is {left neighbour, own dwords, right neighbour}
-  constexpr int kOwn = S;
+  constexpr int kOwn = S * CW / 4;
   constexpr int kRows = S * (RPT - 1) + 3;  // input rows behind the thread's output rows
-  const int d0 = S * w4;
+  const int d0 = kOwn * w4;
   const int ih0 = oh0 * S - a.pad_t;
   const bool has_left = w4 > 0;                      // else: left of the image
   const bool has_right = d0 + kOwn < in_dwords;      // else: right of the image
@@ -81,25 +84,74 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
     const int ih = ih0 + r;
     const bool inside = ih >= 0 && ih < a.H;
     const int* row = reinterpret_cast<const int*>(xp + static_cast<size_t>(inside ? ih : 0) * a.W);
-    const int keep_row = inside ? -1 : 0;
+    if constexpr (CW == 8) {
+      // (rows are whole 8-byte units here: a lane's unit lies inside the row or wholly past it)
+      const int2 v2 = *reinterpret_cast<const int2*>(row + min(d0, in_dwords - 2));
+      raw[r][1] = v2.x;
+      raw[r][2] = v2.y;
+    } else {
+#pragma unroll
+      for (int i = 0; i < kOwn; ++i) raw[r][1 + i] = row[min(d0 + i, in_dwords - 1)];
+    }
+  }
+  // The channel's constants are needed from here on: their (scalar) loads are in flight together with the rows.
+  // Left to the compiler they are requested where they are first used, behind the wait for the rows - a second
+  // round trip.
+  asm volatile("" ::"s"(wk0), "s"(wk1), "s"(wk2), "s"(bias), "s"(q[0]), "s"(q[1]), "s"(q[2]), "s"(q[3]));
+#pragma unroll
+  for (int r = 0; r < kRows; ++r) {
+    const int ih = ih0 + r;
+    const int keep_row = (ih >= 0 && ih < a.H) ? -1 : 0;
 #pragma unroll
     for (int i = 0; i < kOwn; ++i) {
-      const int d = d0 + i;
-      const int keep = d < in_dwords ? keep_row : 0;
+      const int keep = d0 + i < in_dwords ? keep_row : 0;
       // mask arithmetic, not a select: a select on the loaded value would be compiled into a
       // branch around the load, and then the loads would be waited for one at a time
-      const int v = row[min(d, in_dwords - 1)];
-      raw[r][1 + i] = ((v ^ a.xor_mask) & keep) | (a.pad_fill & ~keep);
+      raw[r][1 + i] = ((raw[r][1 + i] ^ a.xor_mask) & keep) | (a.pad_fill & ~keep);
     }
   }
 #pragma unroll
   for (int r = 0; r < kRows; ++r) {
-    // lane l - 1 holds the dwords to the left, lane l + 1 those to the right (wave_shr:1, wave_shl:1)
-    const int l = __builtin_amdgcn_update_dpp(a.pad_fill, raw[r][kOwn], 0x138, 0xf, 0xf, false);
-    const int rr = __builtin_amdgcn_update_dpp(a.pad_fill, raw[r][1], 0x130, 0xf, 0xf, false);
+    // lane l - 1 holds the dwords to the left, lane l + 1 those to the right (wave_shr:1, wave_shl:1); the
+    // wavefront's first / last lane, which has no such neighbour, is the first / last lane of an image row
+    // and takes the padding below
+    const int l = __builtin_amdgcn_mov_dpp(raw[r][kOwn], 0x138, 0xf, 0xf, true);
+    const int rr = __builtin_amdgcn_mov_dpp(raw[r][1], 0x130, 0xf, 0xf, true);
     raw[r][0] = has_left ? l : a.pad_fill;
     raw[r][kOwn + 1] = has_right ? rr : a.pad_fill;
   }
+  if (w4 >= a.ow4) return;  // lanes that only fed their neighbour
+  if constexpr (CW == 8) {
+    // windows are cut per output row (three input rows x eight windows live at a time)
+#pragma unroll
+    for (int o = 0; o < RPT; ++o) {
+      if (oh0 + o >= a.OH) break;
+      int res[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        int win3[3];
+#pragma unroll
+        for (int r = 0; r < 3; ++r) {
+          const int (&rw)[kOwn + 2] = raw[o + r];
+          win3[r] = i == 0 ? Window<4 + 0 - PL>(rw) : i == 1 ? Window<4 + 1 - PL>(rw) : i == 2 ? Window<4 + 2 - PL>(rw)
+                  : i == 3 ? Window<4 + 3 - PL>(rw) : i == 4 ? Window<4 + 4 - PL>(rw) : i == 5 ? Window<4 + 5 - PL>(rw)
+                  : i == 6 ? Window<4 + 6 - PL>(rw) : Window<4 + 7 - PL>(rw);
+        }
+        int acc = Dot4Add(win3[0], wk0, bias);
+        acc = __builtin_amdgcn_sdot4(win3[1], wk1, acc, false);
+        acc = __builtin_amdgcn_sdot4(win3[2], wk2, acc, false);
+        if (BOXSUM && box) {
+          int sx = __builtin_amdgcn_sdot4(win3[0], 0x00010101, 0, false);
+          sx = __builtin_amdgcn_sdot4(win3[1], 0x00010101, sx, false);
+          sx = __builtin_amdgcn_sdot4(win3[2], 0x00010101, sx, false);
+          acc -= a.zws * sx;
+        }
+        res[i] = Requant8<RQ>(acc, q, a.out_zp, a.lo, a.hi);
+      }
+      *reinterpret_cast<uint2*>(yp + static_cast<size_t>(oh0 + o) * a.OW + w4 * 8) =
+          make_uint2(PackBytes(res[0], res[1], res[2], res[3]), PackBytes(res[4], res[5], res[6], res[7]));
+    }
+  } else {
   int win[kRows][4];
 #pragma unroll
   for (int r = 0; r < kRows; ++r) {
@@ -109,15 +161,13 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
     win[r][2] = Window<4 + S * 2 - PL>(raw[r]);
     win[r][3] = Window<4 + S * 3 - PL>(raw[r]);
   }
-  if (w4 >= a.ow4) return;  // lanes that only fed their neighbour
 #pragma unroll
   for (int o = 0; o < RPT; ++o) {
     if (oh0 + o >= a.OH) break;
-    uint32_t packed = 0;
+    int res[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      int acc = bias;
-      acc = __builtin_amdgcn_sdot4(win[S * o][i], wk0, acc, false);
+      int acc = Dot4Add(win[S * o][i], wk0, bias);
       acc = __builtin_amdgcn_sdot4(win[S * o + 1][i], wk1, acc, false);
       acc = __builtin_amdgcn_sdot4(win[S * o + 2][i], wk2, acc, false);
       if (BOXSUM && box) {
@@ -126,35 +176,44 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
         sx = __builtin_amdgcn_sdot4(win[S * o + 2][i], 0x00010101, sx, false);
         acc -= a.zws * sx;
       }
-      packed |= static_cast<uint32_t>(Requant8<RQ>(acc, q, a.out_zp, a.lo, a.hi) & 0xff) << (8 * i);
+      res[i] = Requant8<RQ>(acc, q, a.out_zp, a.lo, a.hi);
     }
-    *reinterpret_cast<uint32_t*>(yp + static_cast<size_t>(oh0 + o) * a.OW + w4 * 4) = packed;
+    *reinterpret_cast<uint32_t*>(yp + static_cast<size_t>(oh0 + o) * a.OW + w4 * 4) = PackBytes(res[0], res[1], res[2], res[3]);
+  }
   }
 }
 
-struct Plan {
-  DwArgs a;
-  int stride, pad_l, boxsum, rq, rows_per_thread, threads;
+// Launch geometry for one patch width.
+struct Shape {
+  int ow4, lpr_shift, rg_per_block, threads, rows_per_thread;
   dim3 grid;
 };
 
-template <int S, int PL, bool BOXSUM, int RPT>
-void LaunchRq(const Plan* p, const DwArgs& a, hipStream_t st) {
-  const dim3 block(p->threads);
-  if (p->rq == kRqFastNoTie) hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqFastNoTie, RPT>), p->grid, block, 0, st, a);
-  else if (p->rq == kRqFast) hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqFast, RPT>), p->grid, block, 0, st, a);
-  else hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqGeneric, RPT>), p->grid, block, 0, st, a);
+struct Plan {
+  DwArgs a;
+  int stride, pad_l, boxsum, rq;
+  int cols;         // output columns per thread of the preferred form: 4 or 8
+  Shape shape;      // ... its geometry
+  Shape fallback;   // four columns per thread: taken when the 8-column form is preferred but a pointer is not 8-byte aligned
+};
+
+template <int S, int PL, bool BOXSUM, int RPT, int CW>
+void LaunchRq(const Plan* p, const Shape& sh, const DwArgs& a, hipStream_t st) {
+  const dim3 block(sh.threads);
+  if (p->rq == kRqFastNoTie) hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqFastNoTie, RPT, CW>), sh.grid, block, 0, st, a);
+  else if (p->rq == kRqFast) hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqFast, RPT, CW>), sh.grid, block, 0, st, a);
+  else hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqGeneric, RPT, CW>), sh.grid, block, 0, st, a);
 }
 
-template <int S, int PL>
-void LaunchBox(const Plan* p, const DwArgs& a, hipStream_t st) {
+template <int S, int PL, int CW>
+void LaunchBox(const Plan* p, const Shape& sh, const DwArgs& a, hipStream_t st) {
   // eight rows per thread only exist for stride 1 (chosen for tall planes)
-  if (S == 1 && p->rows_per_thread == 8) {
-    if (p->boxsum) LaunchRq<1, PL, true, 8>(p, a, st);
-    else LaunchRq<1, PL, false, 8>(p, a, st);
+  if (S == 1 && sh.rows_per_thread == 8) {
+    if (p->boxsum) LaunchRq<1, PL, true, 8, CW>(p, sh, a, st);
+    else LaunchRq<1, PL, false, 8, CW>(p, sh, a, st);
   } else {
-    if (p->boxsum) LaunchRq<S, PL, true, 4>(p, a, st);
-    else LaunchRq<S, PL, false, 4>(p, a, st);
+    if (p->boxsum) LaunchRq<S, PL, true, 4, CW>(p, sh, a, st);
+    else LaunchRq<S, PL, false, 4, CW>(p, sh, a, st);
   }
 }
 
@@ -163,10 +222,19 @@ int DwRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
   DwArgs a = p->a;
   a.x = static_cast<const uint8_t*>(in0);
   a.y = static_cast<uint8_t*>(out);
+  const bool wide = p->cols == 8 && ((reinterpret_cast<uintptr_t>(in0) | reinterpret_cast<uintptr_t>(out)) & 7) == 0;
+  const Shape& sh = wide ? p->shape : (p->cols == 8 ? p->fallback : p->shape);
+  a.ow4 = sh.ow4;
+  a.lpr_shift = sh.lpr_shift;
+  a.rg_per_block = sh.rg_per_block;
   if (p->stride == 1) {
-    if (p->pad_l) LaunchBox<1, 1>(p, a, st); else LaunchBox<1, 0>(p, a, st);
+    if (wide) {
+      if (p->pad_l) LaunchBox<1, 1, 8>(p, sh, a, st); else LaunchBox<1, 0, 8>(p, sh, a, st);
+    } else {
+      if (p->pad_l) LaunchBox<1, 1, 4>(p, sh, a, st); else LaunchBox<1, 0, 4>(p, sh, a, st);
+    }
   } else {
-    if (p->pad_l) LaunchBox<2, 1>(p, a, st); else LaunchBox<2, 0>(p, a, st);
+    if (p->pad_l) LaunchBox<2, 1, 4>(p, sh, a, st); else LaunchBox<2, 0, 4>(p, sh, a, st);
   }
   TVX_HIP_CHECK(hipGetLastError());
   return TVX_OK;
@@ -232,13 +300,16 @@ int DwConv3x3Setup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   if (d->stride_w != d->stride_h || (d->stride_w != 1 && d->stride_w != 2)) return TVX_E_UNSUPPORTED;
   if (d->pad_left > 1 || (d->in_w & 3) || (d->out_w & 3)) return TVX_E_UNSUPPORTED;
   const int S = d->stride_w;
-  const int ow4 = d->out_w / 4;
   // an image row takes a power-of-two number of lanes (at most a wavefront) that covers both its
-  // output dwords and its input dwords
-  const int in_dw = d->in_w / 4;
-  int lpr_shift = 0;
-  while ((1 << lpr_shift) < ow4 || S * (1 << lpr_shift) < in_dw) ++lpr_shift;
-  if (lpr_shift > 6) return TVX_E_UNSUPPORTED;
+  // output patches and the input dwords behind them
+  auto lanes_shift = [&](int cols) {
+    const int out_patches = d->out_w / cols, own = S * cols / 4, in_dw = d->in_w / 4;
+    int shift = 0;
+    while ((1 << shift) < out_patches || own * (1 << shift) < in_dw) ++shift;
+    return shift;
+  };
+  if (lanes_shift(4) > 6) return TVX_E_UNSUPPORTED;
+  if (d->batch > 65535 || (d->out_h + 3) / 4 > 65535) return TVX_E_UNSUPPORTED;  // (grid.y, grid.z)
   // every output's window must end inside {own dwords, right neighbour}
   if (static_cast<uint32_t>((d->out_w - 1) * S + 2) >= d->in_w + d->pad_left + 4) return TVX_E_UNSUPPORTED;
   const bool x_u8 = d->in_dtype == TVX_U8, w_u8 = d->w_dtype == TVX_U8;
@@ -261,27 +332,41 @@ int DwConv3x3Setup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   a.rq = op->aux2.as<tvx_v4i>();
   a.C = C; a.H = d->in_h; a.W = d->in_w; a.OH = d->out_h; a.OW = d->out_w;
   a.pad_t = d->pad_top; a.pad_l = d->pad_left;
-  a.ow4 = ow4;
-  a.lpr_shift = lpr_shift;
-  // tall planes at stride 1: eight output rows per thread (a third of the workgroups to dispatch,
-  // ten input rows read for eight instead of six for four)
-  int rpt = S == 1 && d->out_h >= 96 ? 8 : 4;
-  if (const char* f = getenv("TVX_DWCONV_ROWS")) {  // tuning aid: output rows per thread
-    if (atoi(f) == 4 || (atoi(f) == 8 && S == 1)) rpt = atoi(f);
+  // Eight columns per thread (stride 1, rows that are whole 8-byte units): one 64-bit load per input row and lane.
+  int cols = (S == 1 && (d->in_w & 7) == 0 && (d->out_w & 7) == 0) ? 8 : 4;
+  if (const char* f = getenv("TVX_DWCONV_COLS")) {  // tuning aid: output columns per thread
+    if (atoi(f) == 4) cols = 4;
   }
-  const int row_groups = (static_cast<int>(d->out_h) + rpt - 1) / rpt;
-  // a workgroup is as many wavefronts as a plane's row groups fill, four at most: wavefronts
-  // without rows would be dispatched only to leave at once
-  p.threads = std::min(kThreads, ((row_groups << lpr_shift) + 63) / 64 * 64);
-  if (const char* f = getenv("TVX_DWCONV_THREADS")) {  // tuning aid
-    if (atoi(f) == 64 || atoi(f) == 128 || atoi(f) == 192 || atoi(f) == 256) p.threads = std::max(atoi(f), 1 << lpr_shift);
-  }
-  a.rg_per_block = p.threads >> lpr_shift;
+  auto shape_for = [&](int cw) {
+    Shape sh{};
+    sh.ow4 = d->out_w / cw;
+    sh.lpr_shift = lanes_shift(cw);
+    // tall planes at stride 1: eight output rows per thread (a third of the workgroups to dispatch,
+    // ten input rows read for eight instead of six for four)
+    // (with eight columns per thread four rows measure faster: the patch is already 32 outputs)
+    int rpt = S == 1 && cw == 4 && d->out_h >= 96 ? 8 : 4;
+    if (const char* f = getenv("TVX_DWCONV_ROWS")) {  // tuning aid: output rows per thread
+      if (atoi(f) == 4 || (atoi(f) == 8 && S == 1)) rpt = atoi(f);
+    }
+    sh.rows_per_thread = rpt;
+    const int row_groups = (static_cast<int>(d->out_h) + rpt - 1) / rpt;
+    // a workgroup is as many wavefronts as a plane's row groups fill, four at most: wavefronts
+    // without rows would be dispatched only to leave at once
+    sh.threads = std::min(kThreads, ((row_groups << sh.lpr_shift) + 63) / 64 * 64);
+    if (const char* f = getenv("TVX_DWCONV_THREADS")) {  // tuning aid
+      if (atoi(f) == 64 || atoi(f) == 128 || atoi(f) == 192 || atoi(f) == 256) sh.threads = std::max(atoi(f), 1 << sh.lpr_shift);
+    }
+    sh.rg_per_block = sh.threads >> sh.lpr_shift;
+    sh.grid = dim3(C, d->batch, (row_groups + sh.rg_per_block - 1) / sh.rg_per_block);
+    return sh;
+  };
+  p.cols = cols;
+  p.shape = shape_for(cols);
+  p.fallback = shape_for(4);
   a.xor_mask = x_u8 ? static_cast<int>(0x80808080u) : 0;
   a.pad_fill = static_cast<int>(static_cast<uint32_t>(zxs & 0xff) * 0x01010101u);
   a.zws = zws; a.out_zp = d->out_zp; a.lo = op->act_lo; a.hi = op->act_hi;
-  p.stride = S; p.pad_l = d->pad_left; p.boxsum = any_box; p.rq = rq; p.rows_per_thread = rpt;
-  p.grid = dim3(d->batch * C, (row_groups + a.rg_per_block - 1) / a.rg_per_block);
+  p.stride = S; p.pad_l = d->pad_left; p.boxsum = any_box; p.rq = rq;
   op->host_blob.assign(reinterpret_cast<const uint8_t*>(&p), reinterpret_cast<const uint8_t*>(&p) + sizeof(p));
   op->run = DwRun;
   op->kernel_name = "dwconv3x3_i8";

@@ -345,9 +345,9 @@ __global__ void __launch_bounds__(kThreads) DwRowsKernel(DwrArgs a) {
       int r4[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        int acc = t0[3];
+        int acc = Dot4Add(static_cast<int>(win[orow * S][j]), t0[0], t0[3]);
 #pragma unroll
-        for (int ky = 0; ky < 3; ++ky) acc = __builtin_amdgcn_sdot4(static_cast<int>(win[orow * S + ky][j]), t0[ky], acc, false);
+        for (int ky = 1; ky < 3; ++ky) acc = __builtin_amdgcn_sdot4(static_cast<int>(win[orow * S + ky][j]), t0[ky], acc, false);
         if (BOXSUM) {
           int sx = 0;
 #pragma unroll

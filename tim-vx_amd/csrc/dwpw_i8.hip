@@ -130,8 +130,9 @@ __device__ __forceinline__ void PatchCompute(const DwPwArgs& a, const ChannelCon
   }
 #pragma unroll
   for (int r = 0; r < kRows; ++r) {
-    const int l = __builtin_amdgcn_update_dpp(a.dw_pad_fill, raw[r][kOwn], 0x138, 0xf, 0xf, false);
-    const int rr = __builtin_amdgcn_update_dpp(a.dw_pad_fill, raw[r][1], 0x130, 0xf, 0xf, false);
+    // (the wavefront's first / last lane has no such neighbour; it is the first / last lane of an image row and takes the padding)
+    const int l = __builtin_amdgcn_mov_dpp(raw[r][kOwn], 0x138, 0xf, 0xf, true);
+    const int rr = __builtin_amdgcn_mov_dpp(raw[r][1], 0x130, 0xf, 0xf, true);
     raw[r][0] = has_left ? l : a.dw_pad_fill;
     raw[r][kOwn + 1] = has_right ? rr : a.dw_pad_fill;
   }
@@ -148,8 +149,7 @@ __device__ __forceinline__ void PatchCompute(const DwPwArgs& a, const ChannelCon
     int accs[4], outs[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      int acc = bias;
-      acc = __builtin_amdgcn_sdot4(win[0][i], wk0, acc, false);
+      int acc = Dot4Add(win[0][i], wk0, bias);
       acc = __builtin_amdgcn_sdot4(win[1][i], wk1, acc, false);
       acc = __builtin_amdgcn_sdot4(win[2][i], wk2, acc, false);
       if (box) {

@@ -91,8 +91,7 @@ __device__ __forceinline__ int WindowOf(const int (&row)[(W + 5) / 4 + 1]) {
 template <int W, int S, int J>
 __device__ __forceinline__ int DwOne(const MbArgs& a, const int (&rows)[3][(W + 5) / 4 + 1], const v4i& k) {
   const int w0 = WindowOf<W, S, J>(rows[0]), w1 = WindowOf<W, S, J>(rows[1]), w2 = WindowOf<W, S, J>(rows[2]);
-  int v = k[3];
-  v = __builtin_amdgcn_sdot4(w0, k[0], v, false);
+  int v = Dot4Add(w0, k[0], k[3]);
   v = __builtin_amdgcn_sdot4(w1, k[1], v, false);
   v = __builtin_amdgcn_sdot4(w2, k[2], v, false);
   if (a.dw_box) {  // (wave-uniform) weights packed unshifted: their zero point times the window sum

@@ -118,6 +118,14 @@ __device__ __forceinline__ int Med3(int v, int lo, int hi) {
   return r;
 }
 
+// a . b (four signed bytes each) + c into a new register: the three-address form. The builtin becomes the
+// two-address v_dot4c, which needs a copy of c in front of it whenever c stays live (a bias shared by many outputs).
+__device__ __forceinline__ int Dot4Add(int a, int b, int c) {
+  int r;
+  asm("v_dot4_i32_i8 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
 // The low bytes of four ints as one dword (a in byte 0).
 __device__ __forceinline__ uint32_t PackBytes(int a, int b, int c, int d) {
   const uint32_t ab = __builtin_amdgcn_perm(static_cast<uint32_t>(b), static_cast<uint32_t>(a), 0x0c0c0400);
