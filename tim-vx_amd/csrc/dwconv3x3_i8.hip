@@ -79,19 +79,22 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
   // all loads of the thread are issued before the first use; a lane beyond the row's last
   // output still fetches its dwords when they exist (its left neighbour needs them)
   int raw[kRows][kOwn + 2];
+  // (a row outside the image reads the nearest row inside and is replaced below; offsets inside a plane fit 32 bits:
+  // one scalar base + one vector offset per load, no 64-bit vector arithmetic)
+  const uint32_t col_off = static_cast<uint32_t>(CW == 8 ? min(d0, in_dwords - 2) : 0) * 4u;
 #pragma unroll
   for (int r = 0; r < kRows; ++r) {
-    const int ih = ih0 + r;
-    const bool inside = ih >= 0 && ih < a.H;
-    const int* row = reinterpret_cast<const int*>(xp + static_cast<size_t>(inside ? ih : 0) * a.W);
+    const int ihc = min(max(ih0 + r, 0), a.H - 1);
+    const uint32_t row_off = __umul24(static_cast<uint32_t>(ihc), static_cast<uint32_t>(a.W));
     if constexpr (CW == 8) {
       // (rows are whole 8-byte units here: a lane's unit lies inside the row or wholly past it)
-      const int2 v2 = *reinterpret_cast<const int2*>(row + min(d0, in_dwords - 2));
+      const int2 v2 = *reinterpret_cast<const int2*>(xp + (row_off + col_off));
       raw[r][1] = v2.x;
       raw[r][2] = v2.y;
     } else {
 #pragma unroll
-      for (int i = 0; i < kOwn; ++i) raw[r][1 + i] = row[min(d0 + i, in_dwords - 1)];
+      for (int i = 0; i < kOwn; ++i)
+        raw[r][1 + i] = *reinterpret_cast<const int*>(xp + (row_off + static_cast<uint32_t>(min(d0 + i, in_dwords - 1)) * 4u));
     }
   }
   // The channel's constants are needed from here on: their (scalar) loads are in flight together with the rows.
@@ -101,7 +104,7 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
 #pragma unroll
   for (int r = 0; r < kRows; ++r) {
     const int ih = ih0 + r;
-    const int keep_row = (ih >= 0 && ih < a.H) ? -1 : 0;
+    const int keep_row = min(max(ih, 0), a.H - 1) == ih ? -1 : 0;
 #pragma unroll
     for (int i = 0; i < kOwn; ++i) {
       const int keep = d0 + i < in_dwords ? keep_row : 0;
@@ -310,6 +313,7 @@ int DwConv3x3Setup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   };
   if (lanes_shift(4) > 6) return TVX_E_UNSUPPORTED;
   if (d->batch > 65535 || (d->out_h + 3) / 4 > 65535) return TVX_E_UNSUPPORTED;  // (grid.y, grid.z)
+  if (d->in_h >= (1u << 24) || static_cast<uint64_t>(d->in_h) * d->in_w >= (1ull << 31)) return TVX_E_UNSUPPORTED;  // (32-bit offsets inside a plane)
   // every output's window must end inside {own dwords, right neighbour}
   if (static_cast<uint32_t>((d->out_w - 1) * S + 2) >= d->in_w + d->pad_left + 4) return TVX_E_UNSUPPORTED;
   const bool x_u8 = d->in_dtype == TVX_U8, w_u8 = d->w_dtype == TVX_U8;
