@@ -124,6 +124,12 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
     raw[r][kOwn + 1] = has_right ? rr : a.pad_fill;
   }
   if (w4 >= a.ow4) return;  // lanes that only fed their neighbour
+  // Uniform operands that the instructions below take from vector registers (the three-address dot product, the
+  // clamp) get one copy for all output rows: each row is a block of its own behind the bounds test, and the
+  // compiler would copy them again in every block.
+  int bias_v = bias, wk0_v = wk0, lo_v = a.lo, hi_v = a.hi;
+  asm volatile("" : "+v"(bias_v), "+v"(wk0_v), "+v"(lo_v), "+v"(hi_v));
+  uint8_t* const yrow = yp;  // (uniform base; offsets inside a plane fit 32 bits)
   if constexpr (CW == 8) {
     // windows are cut per output row (three input rows x eight windows live at a time)
 #pragma unroll
@@ -140,7 +146,7 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
                   : i == 3 ? Window<4 + 3 - PL>(rw) : i == 4 ? Window<4 + 4 - PL>(rw) : i == 5 ? Window<4 + 5 - PL>(rw)
                   : i == 6 ? Window<4 + 6 - PL>(rw) : Window<4 + 7 - PL>(rw);
         }
-        int acc = Dot4Add(win3[0], wk0, bias);
+        int acc = Dot4Add(win3[0], wk0_v, bias_v);
         acc = __builtin_amdgcn_sdot4(win3[1], wk1, acc, false);
         acc = __builtin_amdgcn_sdot4(win3[2], wk2, acc, false);
         if (BOXSUM && box) {
@@ -149,9 +155,9 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
           sx = __builtin_amdgcn_sdot4(win3[2], 0x00010101, sx, false);
           acc -= a.zws * sx;
         }
-        res[i] = Requant8<RQ>(acc, q, a.out_zp, a.lo, a.hi);
+        res[i] = Requant8<RQ>(acc, q, a.out_zp, lo_v, hi_v);
       }
-      *reinterpret_cast<uint2*>(yp + static_cast<size_t>(oh0 + o) * a.OW + w4 * 8) =
+      *reinterpret_cast<uint2*>(yrow + (__umul24(static_cast<uint32_t>(oh0 + o), static_cast<uint32_t>(a.OW)) + static_cast<uint32_t>(w4) * 8u)) =
           make_uint2(PackBytes(res[0], res[1], res[2], res[3]), PackBytes(res[4], res[5], res[6], res[7]));
     }
   } else {
@@ -170,7 +176,7 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
     int res[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      int acc = Dot4Add(win[S * o][i], wk0, bias);
+      int acc = Dot4Add(win[S * o][i], wk0_v, bias_v);
       acc = __builtin_amdgcn_sdot4(win[S * o + 1][i], wk1, acc, false);
       acc = __builtin_amdgcn_sdot4(win[S * o + 2][i], wk2, acc, false);
       if (BOXSUM && box) {
@@ -179,9 +185,10 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
         sx = __builtin_amdgcn_sdot4(win[S * o + 2][i], 0x00010101, sx, false);
         acc -= a.zws * sx;
       }
-      res[i] = Requant8<RQ>(acc, q, a.out_zp, a.lo, a.hi);
+      res[i] = Requant8<RQ>(acc, q, a.out_zp, lo_v, hi_v);
     }
-    *reinterpret_cast<uint32_t*>(yp + static_cast<size_t>(oh0 + o) * a.OW + w4 * 4) = PackBytes(res[0], res[1], res[2], res[3]);
+    *reinterpret_cast<uint32_t*>(yrow + (__umul24(static_cast<uint32_t>(oh0 + o), static_cast<uint32_t>(a.OW)) + static_cast<uint32_t>(w4) * 4u)) =
+        PackBytes(res[0], res[1], res[2], res[3]);
   }
   }
 }
