@@ -512,6 +512,35 @@ def test_pointwise_conv_walks_several_output_tiles_per_wavefront(oracle, gi, mod
     assert len(np.unique(want)) > 4
 
 
+STREAM_GRID = [
+    # (n, c, h, w, oc): shallow inputs, pixel groups of sixteen inside one image
+    (3, 32, 16, 48, 64),    # 18 pixel tiles, whole output tiles
+    (2, 24, 20, 36, 40),    # padded input channels, a partial output tile, a ragged last pixel tile (1440 pixels)
+    (5, 7, 4, 12, 100),     # 48-pixel images: pixel tiles straddle images; four output tiles
+    (1, 16, 8, 16, 33),     # one pixel tile
+]
+
+
+@pytest.mark.parametrize("tiles", [1, 2, 5])
+@pytest.mark.parametrize("mode", ["u8", "i8pc", "u8pc"])
+@pytest.mark.parametrize("gi", range(len(STREAM_GRID)))
+def test_pointwise_conv_streaming_form(oracle, gi, mode, tiles, monkeypatch):
+    """The form for shallow inputs in which a wavefront walks several pixel tiles with the next tile's rows in
+    flight: forced onto small cases (it is chosen from 2048 pixel tiles up), 1, 2 and 5 tiles per wavefront."""
+    n, c, h, w, oc = STREAM_GRID[gi]
+    monkeypatch.setenv("TVX_PWCONV_STREAM_MIN_TILES", "1")
+    monkeypatch.setenv("TVX_PWCONV_STREAM", str(tiles))
+    monkeypatch.setenv("TVX_PWCONV_SHAPE", "128,1")
+    rng = np.random.default_rng(4300 + gi)
+    x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=oc, kh=1, kw=1, stride=[1, 1], dil=[1, 1],
+                              pad=[0, 0, 0, 0], mult=0, mode=mode)
+    for act in (0, 2):
+        want = oracle.conv2d(x, wt, b, act=act, **kws)
+        got = TC.gpu_conv2d(x, wt, b, act=act, want_kernel="pwconv_i8_stream", **kws)
+        assert np.array_equal(got, want), int((got != want).sum())
+    assert len(np.unique(want)) > 4
+
+
 DW_GRID = [
     # (n, c, h, w, stride, pad[l,r,t,b])
     (2, 8, 16, 16, 1, [1, 1, 1, 1]),
@@ -691,7 +720,7 @@ def test_depthwise_then_pointwise_full_size(oracle):
               dilation=[1, 1], pad_left=0, pad_top=0, multiplier=0, in_dtype=1, w_dtype=1, out_dtype=1,
               in_q=(0.08, 0), w_q=(1.0, 0, sp), out_q=(0.05, 0), act=2)
     out_want = oracle.conv2d(mid, wp, bp, **kp)
-    out = TC.gpu_conv2d(mid, wp, bp, want_kernel="pwconv_i8", **kp)
+    out = TC.gpu_conv2d(mid, wp, bp, want_kernel=("pwconv_i8", "pwconv_i8_stream"), **kp)
     assert np.array_equal(out, out_want)
     assert out.min() == 0 and out.max() == 120  # ReLU6 at scale 0.05
 

@@ -360,10 +360,128 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((P
   }
 }
 
+
+// ---- shallow inputs (at most 32 channels), large pixel counts: one wavefront streams pixel tiles ----------------
+// The general kernel gives every 128-pixel tile a wavefront of its own, and with a few thousand tiles all of them are
+// resident at once: the whole launch loads, then computes, then stores, and memory idles while the vector units work.
+// Here a wavefront walks several pixel tiles; the sixteen dwords of its next tile are requested before the present
+// tile is multiplied and requantized, so that loads, vector work and stores of different tiles overlap. With one
+// k-step per output tile the operand fragments of a pixel tile are read from LDS once and kept for all output tiles.
+// Pixel groups of sixteen stay inside one image (HW % 16 == 0), no fused Add.
+constexpr int kStreamPix = 128;
+template <bool ZP, int RQ>
+__global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2))) PwStreamKernel(PwArgs a) {
+  extern __shared__ __attribute__((aligned(16))) int8_t lds[];
+  const int lane = threadIdx.x;
+  int8_t* xl = lds;                                 // [128 pixels][pix_stride]
+  int8_t* stage = lds + kStreamPix * a.pix_stride;  // [32 channels][kStageStride]
+  const int n_pix_tiles = (a.Q + kStreamPix - 1) / kStreamPix;
+  // an XCD gets a contiguous run of pixel tiles (the grid is a multiple of eight workgroups)
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
+  const int t_first = static_cast<int>(static_cast<long long>(n_pix_tiles) * xcd / 8);
+  const int t_end = static_cast<int>(static_cast<long long>(n_pix_tiles) * (xcd + 1) / 8);
+  int pt = t_first + slot;
+  if (pt >= t_end) return;
+
+  const int pq = lane & 31, cg = lane >> 5;  // this lane's 4-pixel group and 16-channel group of the input tile
+  const uint32_t hw = static_cast<uint32_t>(a.HW);
+  const uint32_t last_row = static_cast<uint32_t>(a.C - 1) * hw;
+  auto request = [&](int tile, uint32_t (&raw)[16]) {
+    const int q0 = tile * kStreamPix + pq * 4;
+    const bool live = q0 < a.Q;
+    const uint32_t n = live ? static_cast<uint32_t>(q0) / hw : 0u;
+    const uint32_t p = live ? static_cast<uint32_t>(q0) - n * hw : 0u;
+    const uint32_t at0 = n * static_cast<uint32_t>(a.C) * hw + p;
+#pragma unroll
+    for (int j = 0; j < 16; ++j)  // channel min(c, C - 1); unconditional loads, masked when they are used
+      raw[j] = *reinterpret_cast<const uint32_t*>(a.x + (at0 + min(static_cast<uint32_t>(cg * 16 + j) * hw, last_row)));
+  };
+  auto commit = [&](int tile, uint32_t (&raw)[16]) {
+    const bool live = tile * kStreamPix + pq * 4 < a.Q;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) raw[j] = (live && cg * 16 + j < a.C) ? raw[j] ^ a.xor_mask : 0u;
+    uint32_t t[4][4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) Transpose4x4(raw + 4 * b, t[b]);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const v4i v = {static_cast<int>(t[0][e]), static_cast<int>(t[1][e]), static_cast<int>(t[2][e]), static_cast<int>(t[3][e])};
+      *reinterpret_cast<v4i*>(xl + (pq * 4 + e) * a.pix_stride + cg * 16) = v;
+    }
+  };
+
+  const int frag_row = lane & 31, frag_half = lane >> 5;
+  const int px_in_row = (lane & 7) * 16, row0 = lane >> 3;  // copy-out: 16-pixel chunk lane % 8 of staged rows lane / 8 + 8 i
+  const v4i fz = {a.neg_zws4, a.neg_zws4, a.neg_zws4, a.neg_zws4};
+  const int lo = a.lo, hi = a.hi;
+
+  uint32_t raw[16];
+  request(pt, raw);
+  // the first output tile's weights and tables travel with the first rows
+  v4i nf = a.wpk[lane];
+  int nb = a.biasf[frag_row];
+  v4i nq = a.rq[frag_row];
+  for (; pt < t_end; pt += per_xcd) {
+    commit(pt, raw);
+    const int next_pt = pt + per_xcd;
+    if (next_pt < t_end) request(next_pt, raw);  // in flight until the next round's commit
+    __builtin_amdgcn_wave_barrier();
+    v4i fx[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      fx[i] = *reinterpret_cast<const v4i*>(xl + (i * 32 + frag_row) * a.pix_stride + frag_half * 16);
+    // where this lane's output chunks live
+    const int oq0 = pt * kStreamPix + px_in_row;
+    const bool out_live = oq0 < a.Q;
+    const uint32_t on = out_live ? static_cast<uint32_t>(oq0) / hw : 0u;
+    const uint32_t op0 = out_live ? static_cast<uint32_t>(oq0) - on * hw : 0u;
+    const size_t out_off = static_cast<size_t>(on) * a.OC * a.HW + op0;
+    for (int tile = 0; tile < a.oc_tiles; ++tile) {
+      const v4i fw = nf, q = nq;
+      v16i acc[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][r] = nb;
+      const int next_tile = tile + 1 < a.oc_tiles ? tile + 1 : 0;  // (the next pixel tile starts at output tile 0 again)
+      nf = a.wpk[next_tile * 64 + lane];
+      nb = a.biasf[next_tile * 32 + frag_row];
+      nq = a.rq[next_tile * 32 + frag_row];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fx[i], fw, acc[i], 0, 0, 0);
+        if (ZP) acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fx[i], fz, acc[i], 0, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          int v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = Requant8<RQ>(acc[i][g * 4 + e], q, a.out_zp, lo, hi);
+          *reinterpret_cast<uint32_t*>(stage + frag_row * kStageStride + i * 32 + 8 * g + 4 * frag_half) = PackBytes(v[0], v[1], v[2], v[3]);
+        }
+      __builtin_amdgcn_wave_barrier();
+      const int rows = min(32, a.OC - tile * 32);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int row = row0 + 8 * i;
+        const int8_t* sp = stage + row * kStageStride + px_in_row;
+        const uint2 lo8 = *reinterpret_cast<const uint2*>(sp);
+        const uint2 hi8 = *reinterpret_cast<const uint2*>(sp + 8);
+        if (row < rows && out_live)
+          *reinterpret_cast<uint4*>(a.y + (out_off + (static_cast<size_t>(tile) * 32 + row) * a.HW)) = make_uint4(lo8.x, lo8.y, hi8.x, hi8.y);
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+}
+
 struct Plan {
   PwArgs a;
   int lds_bytes, kp, nw, pt, gran, zp, rq;
   dim3 grid;
+  int stream_wgs;  // > 0: PwStreamKernel with that many workgroups
 };
 
 template <int KP, int NW, int PT, int GRAN, bool ZP, int RQ>
@@ -399,7 +517,21 @@ int DispatchGran(const Plan* plan, const PwArgs& a, hipStream_t st, bool configu
   return DispatchZp<KP, NW, PT, 1>(plan, a, st, configure);
 }
 
+template <bool ZP>
+int LaunchStream(const Plan* plan, const PwArgs& a, hipStream_t st) {
+  const dim3 grid(plan->stream_wgs), block(64);
+  const int lds = kStreamPix * a.pix_stride + kStageBytes;
+  if (plan->rq == kRqFastNoTie) hipLaunchKernelGGL((PwStreamKernel<ZP, kRqFastNoTie>), grid, block, lds, st, a);
+  else if (plan->rq == kRqFast) hipLaunchKernelGGL((PwStreamKernel<ZP, kRqFast>), grid, block, lds, st, a);
+  else hipLaunchKernelGGL((PwStreamKernel<ZP, kRqGeneric>), grid, block, lds, st, a);
+  return TVX_OK;
+}
+
 int Dispatch(const Plan* plan, const PwArgs& a, hipStream_t st, bool configure) {
+  if (plan->stream_wgs > 0) {
+    if (configure) return TVX_OK;  // (a few KiB of LDS: no attribute to set)
+    return plan->zp ? LaunchStream<true>(plan, a, st) : LaunchStream<false>(plan, a, st);
+  }
   if (plan->kp == 32) {
     if (plan->nw == 1) return DispatchGran<32, 1, 1>(plan, a, st, configure);
     return DispatchGran<32, 4, 1>(plan, a, st, configure);
@@ -547,11 +679,25 @@ int PwConvSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const 
   plan.zp = zws != 0;
   plan.rq = rq;
   plan.grid = dim3(static_cast<unsigned>(gx * gy));
+  // Shallow inputs with thousands of pixel tiles: wavefronts that stream several tiles each (see PwStreamKernel).
+  plan.stream_wgs = 0;
+  {
+    int tiles_per_wave = 2;
+    if (const char* f = getenv("TVX_PWCONV_STREAM")) tiles_per_wave = atoi(f);  // tuning aid: pixel tiles per wavefront, 0 = off
+    const long long pix_tiles = (static_cast<long long>(a.Q) + kStreamPix - 1) / kStreamPix;
+    long long min_tiles = 2048;
+    if (const char* f = getenv("TVX_PWCONV_STREAM_MIN_TILES")) min_tiles = atoll(f);  // tuning / test aid
+    if (tiles_per_wave > 0 && !op->fused_add && a.cp == 32 && plan.gran == 16 && kp == 128 && nw == 1 && pix_tiles >= min_tiles &&
+        hw * d->in_c * d->batch < (1ull << 32) - 16) {
+      const long long wgs = (pix_tiles + tiles_per_wave - 1) / tiles_per_wave;
+      plan.stream_wgs = static_cast<int>(std::min<long long>((wgs + 7) / 8 * 8, 1 << 20));
+    }
+  }
   s = Dispatch(&plan, a, nullptr, true);
   if (s != TVX_OK) return s;
   op->host_blob.assign(reinterpret_cast<const uint8_t*>(&plan), reinterpret_cast<const uint8_t*>(&plan) + sizeof(plan));
   op->run = PwConvRun;
-  op->kernel_name = op->fused_add ? "pwconv_add_i8" : "pwconv_i8";
+  op->kernel_name = op->fused_add ? "pwconv_add_i8" : (plan.stream_wgs > 0 ? "pwconv_i8_stream" : "pwconv_i8");
   return TVX_OK;
 }
 
