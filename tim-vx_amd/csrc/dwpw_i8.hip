@@ -73,19 +73,21 @@ struct PatchShape {
 };
 
 template <int S, int RPT>
-__device__ __forceinline__ void PatchLoad(const DwPwArgs& a, const uint8_t* xp, int w4, int oh0,
+__device__ __forceinline__ void PatchLoad(const DwPwArgs& a, const uint8_t* xn, uint32_t plane_off, int w4, int oh0,
                                           int (&raw)[PatchShape<S, RPT>::kRows][PatchShape<S, RPT>::kOwn + 2]) {
   constexpr int kOwn = PatchShape<S, RPT>::kOwn, kRows = PatchShape<S, RPT>::kRows;
   const int in_dwords = a.W / 4;
   const int d0 = S * w4;
   const int ih0 = oh0 * S - a.pad_t;
+  // xn: the image (uniform), plane_off: the channel plane inside it; offsets inside an image fit 32 bits (checked at
+  // creation): one scalar base + one vector offset per load. Rows outside the image read the nearest row inside.
 #pragma unroll
   for (int r = 0; r < kRows; ++r) {
-    const int ih = ih0 + r;
-    const bool inside = ih >= 0 && ih < a.H;
-    const int* row = reinterpret_cast<const int*>(xp + static_cast<size_t>(inside ? ih : 0) * a.W);
+    const int ihc = min(max(ih0 + r, 0), a.H - 1);
+    const uint32_t row_off = plane_off + __umul24(static_cast<uint32_t>(ihc), static_cast<uint32_t>(a.W));
 #pragma unroll
-    for (int i = 0; i < kOwn; ++i) raw[r][1 + i] = row[min(d0 + i, in_dwords - 1)];  // unconditional: masked later
+    for (int i = 0; i < kOwn; ++i)  // unconditional: masked later
+      raw[r][1 + i] = *reinterpret_cast<const int*>(xn + (row_off + static_cast<uint32_t>(min(d0 + i, in_dwords - 1)) * 4u));
   }
 }
 
@@ -215,6 +217,7 @@ __global__ void __launch_bounds__(kThreads) DwPwKernel(DwPwArgs a) {
     const int w4 = tid & ((1 << a.lpr_shift) - 1);
     const int per_pass = kThreads >> a.lpr_shift;
     const size_t plane = static_cast<size_t>(a.H) * a.W;
+    const uint32_t plane32 = static_cast<uint32_t>(plane);
     const uint8_t* xn = a.x + static_cast<size_t>(n) * a.C * plane;
     for (int c0 = tid >> a.lpr_shift; c0 < a.C; c0 += per_pass * kBatch) {
       int raw[kBatch][kRows][kOwn + 2];
@@ -222,7 +225,7 @@ __global__ void __launch_bounds__(kThreads) DwPwKernel(DwPwArgs a) {
 #pragma unroll
       for (int b = 0; b < kBatch; ++b) {
         const int c = min(c0 + b * per_pass, a.C - 1);
-        PatchLoad<S, RPT>(a, xn + static_cast<size_t>(c) * plane, w4, oh0, raw[b]);
+        PatchLoad<S, RPT>(a, xn, static_cast<uint32_t>(c) * plane32, w4, oh0, raw[b]);
         consts[b] = LoadChannelConsts(a, c);
       }
 #pragma unroll
@@ -419,7 +422,7 @@ int DwPwSetup(tvx_op* op, const tvx_conv2d_desc* dw, const void* dw_w, const voi
   }
   if (!rpt) return TVX_E_UNSUPPORTED;
   const uint64_t tiles = static_cast<uint64_t>(dw->batch) * (dw->out_h / rpt);
-  if (tiles > 0x7fffffffull || static_cast<uint64_t>(dw->in_h) * dw->in_w >= (1ull << 31)) return TVX_E_UNSUPPORTED;
+  if (tiles > 0x7fffffffull || static_cast<uint64_t>(dw->in_h) * dw->in_w * dw->in_c >= (1ull << 32) - 16 || dw->in_h >= (1u << 24)) return TVX_E_UNSUPPORTED;  // (32-bit offsets inside an image)
 
   DwPwArgs a{};
   const int C = dw->in_c;
