@@ -526,7 +526,7 @@ STREAM_GRID = [
 @pytest.mark.parametrize("gi", range(len(STREAM_GRID)))
 def test_pointwise_conv_streaming_form(oracle, gi, mode, tiles, monkeypatch):
     """The form for shallow inputs in which a wavefront walks several pixel tiles with the next tile's rows in
-    flight: forced onto small cases (it is chosen from 2048 pixel tiles up), 1, 2 and 5 tiles per wavefront."""
+    flight: forced onto small cases (it is chosen from 1024 pixel tiles up), 1, 2 and 5 tiles per wavefront."""
     n, c, h, w, oc = STREAM_GRID[gi]
     monkeypatch.setenv("TVX_PWCONV_STREAM_MIN_TILES", "1")
     monkeypatch.setenv("TVX_PWCONV_STREAM", str(tiles))

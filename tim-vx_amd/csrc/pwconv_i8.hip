@@ -682,10 +682,12 @@ int PwConvSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const 
   // Shallow inputs with thousands of pixel tiles: wavefronts that stream several tiles each (see PwStreamKernel).
   plan.stream_wgs = 0;
   {
-    int tiles_per_wave = 2;
-    if (const char* f = getenv("TVX_PWCONV_STREAM")) tiles_per_wave = atoi(f);  // tuning aid: pixel tiles per wavefront, 0 = off
     const long long pix_tiles = (static_cast<long long>(a.Q) + kStreamPix - 1) / kStreamPix;
-    long long min_tiles = 2048;
+    // two tiles per wavefront once that still leaves two wavefronts per SIMD; below that one tile each (the form's
+    // leaner per-tile code is then what it has to offer; from 1024 tiles up it measures faster than the general kernel)
+    int tiles_per_wave = pix_tiles >= 4096 ? 2 : 1;
+    if (const char* f = getenv("TVX_PWCONV_STREAM")) tiles_per_wave = atoi(f);  // tuning aid: pixel tiles per wavefront, 0 = off
+    long long min_tiles = 1024;
     if (const char* f = getenv("TVX_PWCONV_STREAM_MIN_TILES")) min_tiles = atoll(f);  // tuning / test aid
     if (tiles_per_wave > 0 && !op->fused_add && a.cp == 32 && plan.gran == 16 && kp == 128 && nw == 1 && pix_tiles >= min_tiles &&
         hw * d->in_c * d->batch < (1ull << 32) - 16) {
