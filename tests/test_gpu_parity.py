@@ -549,6 +549,10 @@ DW_GRID = [
     (2, 6, 16, 24, 2, [1, 1, 1, 1]),
     (1, 3, 10, 8, 1, [0, 0, 0, 0]),
     (1, 7, 33, 40, 1, [1, 1, 2, 2]),
+    # rows of whole 8-byte units at stride 1: eight columns per thread
+    (2, 4, 12, 16, 1, [0, 2, 0, 2]),     # no left padding
+    (1, 3, 100, 24, 1, [1, 1, 1, 1]),    # three patches on four lanes, a tall plane (several workgroups per plane)
+    (2, 5, 7, 64, 1, [1, 1, 1, 1]),      # eight patches per row, fewer rows than a patch is tall in the last group
 ]
 
 
@@ -564,6 +568,33 @@ def test_depthwise3x3_shapes(oracle, gi, mode):
         want = oracle.conv2d(x, wt, b, act=act, **kws)
         got = TC.gpu_conv2d(x, wt, b, act=act, want_kernel="dwconv3x3_i8" if fast else "dwconv_planes_i8", **kws)
         assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("gi", [0, 6, 7, 8])
+def test_depthwise3x3_four_columns_per_thread_on_wide_rows(oracle, gi, monkeypatch):
+    """The four-column form on shapes that would take the eight-column one (it is what runs there when a tensor
+    is not 8-byte aligned)."""
+    n, c, h, w, s, pad = DW_GRID[gi]
+    monkeypatch.setenv("TVX_DWCONV_COLS", "4")
+    rng = np.random.default_rng(3100 + gi)
+    x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=0, kh=3, kw=3, stride=[s, s], dil=[1, 1],
+                              pad=pad, mult=1, mode="u8")
+    want = oracle.conv2d(x, wt, b, act=2, **kws)
+    got = TC.gpu_conv2d(x, wt, b, act=2, want_kernel="dwconv3x3_i8", **kws)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("gi", [0, 6, 8])
+def test_depthwise3x3_tensors_off_the_eight_byte_grid(oracle, gi):
+    """Tensors that start four bytes into their allocations: the operator planned for 64-bit row loads has to
+    take its four-column form at run time."""
+    n, c, h, w, s, pad = DW_GRID[gi]
+    rng = np.random.default_rng(3200 + gi)
+    x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=0, kh=3, kw=3, stride=[s, s], dil=[1, 1],
+                              pad=pad, mult=1, mode="u8")
+    want = oracle.conv2d(x, wt, b, act=0, **kws)
+    got = TC.gpu_conv2d(x, wt, b, act=0, want_kernel="dwconv3x3_i8", misalign=4, **kws)
+    assert np.array_equal(got, want)
     assert len(np.unique(want)) > 4
 
 

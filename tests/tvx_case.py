@@ -80,7 +80,8 @@ def _wq(desc, w_q, keep):
 
 def gpu_conv2d(x, w, bias, *, in_shape, w_shape, out_shape, stride, dilation, pad_left, pad_top,
                multiplier, in_dtype, w_dtype, out_dtype, in_q=(1.0, 0), w_q=(1.0, 0, None),
-               out_q=(1.0, 0), act=0, const_weights=True, want_kernel=None, groups=0, transposed=False):
+               out_q=(1.0, 0), act=0, const_weights=True, want_kernel=None, groups=0, transposed=False, misalign=0):
+    """misalign: byte offset of the activation and result tensors from their (256-byte aligned) allocations."""
     T = tvx()
     d = T.Conv2dDesc()
     d.groups = groups
@@ -103,6 +104,11 @@ def gpu_conv2d(x, w, bias, *, in_shape, w_shape, out_shape, stride, dilation, pa
     xd = to_device(x)
     wd = None if const_weights else to_device(w)
     yd = device_out(np.prod(out_shape), NP_OF[out_dtype])
+    if misalign:
+        assert x.dtype.itemsize == 1 and NP_OF[out_dtype]().itemsize == 1
+        xd = to_device(np.concatenate([np.zeros(misalign, x.dtype), x.reshape(-1)]))[misalign:]
+        yd = device_out(np.prod(out_shape) + misalign, NP_OF[out_dtype])[misalign:]
+        assert xd.data_ptr() % 256 == misalign and yd.data_ptr() % 256 == misalign
     op.run(xd, wd, yd)
     torch.cuda.synchronize()
     out = yd.cpu().numpy()
