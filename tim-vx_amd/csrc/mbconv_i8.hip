@@ -130,9 +130,10 @@ struct DwRow {
 
 // W: columns of the input; S: stride of the depthwise convolution; MO: 32-pixel tiles of a band's output;
 // NTMAX: most 32-channel output tiles; ADD: residual Add behind the projection.
-// (the register budget follows the accumulators: three wavefronts per SIMD with two output tiles, two with five)
+// (the register budget follows the accumulators: two wavefronts per SIMD up to five output tiles - three with two
+// tiles, 168 registers, spill 36 bytes per lane and measure slower -, one beyond)
 template <int W, int S, int MO, int NTMAX, bool ADD>
-__global__ void __launch_bounds__(kThreads, (MO * NTMAX <= 2 ? 3 : (MO * NTMAX <= 5 ? 2 : 1))) MbConvKernel(MbArgs a) {
+__global__ void __launch_bounds__(kThreads, (MO * NTMAX <= 5 ? 2 : 1)) MbConvKernel(MbArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
   constexpr int PL = S == 1 ? 1 : 0;               // left (and top) padding of the depthwise convolution
   constexpr int OW = (W + S - 1) / S;
