@@ -297,8 +297,9 @@ def run_case(case):
         x, w = ins[0], ins[1]
         s, z, _ = _q(x["quant"])
         so, zo, _ = _q(out["quant"])
-        return conv2d(arr[0], arr[1], arr[2] if len(ins) > 2 else None, in_shape=x["shape"], w_shape=w["shape"],
-                      out_shape=out["shape"], stride=a["stride"], dilation=[1, 1], pad_left=a["pad"][0],
+        xs, wsh, osh = _conv_shapes(a, x["shape"], w["shape"], out["shape"])  # DeConv1d: rows of height one
+        return conv2d(arr[0], arr[1], arr[2] if len(ins) > 2 else None, in_shape=xs, w_shape=wsh,
+                      out_shape=osh, stride=a["stride"], dilation=[1, 1], pad_left=a["pad"][0],
                       pad_top=a["pad"][2], multiplier=0, groups=a.get("groups", 0), in_dtype=DTYPE_CODE[x["dtype"]],
                       w_dtype=DTYPE_CODE[w["dtype"]], out_dtype=DTYPE_CODE[out["dtype"]], in_q=(s, z),
                       w_q=_q(w["quant"]), out_q=(so, zo), transposed=True)

@@ -27,6 +27,8 @@ SOURCES = {
     "depthwise_conv": "src/tim/vx/ops/depthwiseConv_test.cc",
     "grouped_conv2d": "src/tim/vx/ops/groupedconv2d_test.cc",
     "conv1d": "src/tim/vx/ops/conv1d_test.cc",
+    "grouped_conv1d": "src/tim/vx/ops/groupedconv1d_test.cc",
+    "deconv1d": ("src/tim/vx/ops/deconv1d_test.cc", ["DeConv1d"]),  # (the file's other suite needs LeakyRelu)
     "fullyconnected": "src/tim/vx/ops/fullyconnected_test.cc",
     "max_pool": "src/tim/vx/ops/max_pool_test.cc",
     "avg_pool": "src/tim/vx/ops/avg_pool_test.cc",

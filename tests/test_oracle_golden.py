@@ -10,15 +10,15 @@ CASES = TC.all_cases()
 
 def test_fixture_inventory():
     # 24 conv2d tests (one of them loops over 66 input sizes), 16 depthwise, 3 grouped, 3 one-dimensional,
-    # 2 fully-connected, 3 max-pool, 8 avg-pool, 6 softmax, 2 transpose, 3 DataConvert, 4 layout-inference source graphs, 2 DeConv2d; the two int16 dynamic-fixed-point
+    # 2 fully-connected, 3 max-pool, 8 avg-pool, 6 softmax, 2 transpose, 3 DataConvert, 4 layout-inference source graphs, 2 DeConv2d, 2 GroupedConv1d, 3 DeConv1d (the file's fourth test needs LeakyRelu); the two int16 dynamic-fixed-point
     # conv tests of the reference are outside this path and not recorded.
     per_file = {}
     for n, c in CASES:
         per_file.setdefault(n, set()).add(c["test"])
     assert {k: len(v) for k, v in per_file.items()} == {
         "conv2d": 24, "depthwise_conv": 16, "grouped_conv2d": 3, "conv1d": 3, "fullyconnected": 2, "max_pool": 3, "avg_pool": 8, "softmax": 6,
-        "transpose": 2, "dataconvert": 3, "layout_inference": 4, "deconv2d": 2}
-    assert len(CASES) == 141
+        "transpose": 2, "dataconvert": 3, "layout_inference": 4, "deconv2d": 2, "grouped_conv1d": 2, "deconv1d": 3}
+    assert len(CASES) == 146
 
 
 @pytest.mark.parametrize("item", CASES, ids=TC.case_id)

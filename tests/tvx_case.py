@@ -12,7 +12,7 @@ import tvx_oracle as O
 HERE = os.path.dirname(os.path.abspath(__file__))
 GOLDEN_FILES = ["conv2d", "depthwise_conv", "grouped_conv2d", "conv1d", "fullyconnected", "max_pool", "avg_pool", "softmax",
                 "transpose", "dataconvert", "layout_inference",
-                "deconv2d"]
+                "deconv2d", "grouped_conv1d", "deconv1d"]
 
 
 def load_cases(name):
@@ -267,8 +267,9 @@ def run_case_gpu(case):
         x, w = ins[0], ins[1]
         s, z, _ = O._q(x["quant"])
         so, zo, _ = O._q(out["quant"])
-        return gpu_conv2d(arr[0], arr[1], arr[2] if len(ins) > 2 else None, in_shape=x["shape"], w_shape=w["shape"],
-                          out_shape=out["shape"], stride=a["stride"], dilation=[1, 1], pad_left=a["pad"][0],
+        xs, wsh, osh = O._conv_shapes(a, x["shape"], w["shape"], out["shape"])  # DeConv1d: rows of height one
+        return gpu_conv2d(arr[0], arr[1], arr[2] if len(ins) > 2 else None, in_shape=xs, w_shape=wsh,
+                          out_shape=osh, stride=a["stride"], dilation=[1, 1], pad_left=a["pad"][0],
                           pad_top=a["pad"][2], multiplier=0, groups=a.get("groups", 0), in_dtype=code[x["dtype"]],
                           w_dtype=code[w["dtype"]], out_dtype=code[out["dtype"]], in_q=(s, z),
                           w_q=O._q(w["quant"]), out_q=(so, zo), const_weights=(w["attr"] == "CONSTANT"),

@@ -96,6 +96,33 @@ class Conv1d : public BuiltinOp {
                            int32_t input_idx) override;
 };
 
+// Grouped 1-D convolution: the grouped operator on {W, C, N} tensors, weight {Kw, Ic / groups, Oc}.
+// reference: include/tim/vx/ops/groupedconv1d.h:56-80, src/tim/vx/ops/groupedconv1d.cc:34-66
+class GroupedConv1d : public BuiltinOp {
+ public:
+  GroupedConv1d(Graph* graph, PadType padding, std::array<uint32_t, 2> pad, uint32_t stride, uint32_t dilation,
+                uint32_t group, DataLayout input_layout = DataLayout::WCN,
+                DataLayout kernel_layout = DataLayout::WIcOc);
+  GroupedConv1d(Graph* graph, PadType padding, const uint32_t stride, const uint32_t dilation, uint32_t group,
+                DataLayout input_layout = DataLayout::WCN, DataLayout kernel_layout = DataLayout::WIcOc);
+
+  DataLayout KernelDataLayout() { return kernel_layout_; }
+  std::shared_ptr<Operation> Clone(
+      std::shared_ptr<Graph>& graph) const override;
+
+ protected:
+  const PadType padding_;
+  const std::array<uint32_t, 2> pad_;
+  const uint32_t stride_;
+  const uint32_t dilation_;
+  const uint32_t group_;
+  const DataLayout kernel_layout_;
+
+ private:
+  void OnBindInputPostProc(const std::shared_ptr<Tensor>& tensor,
+                           int32_t input_idx) override;
+};
+
 // Grouped 2-D convolution: output channel block j (Oc / groups channels) reads input
 // channel block j (Ic / groups channels); weight {Kw, Kh, Ic / groups, Oc}, optional bias {Oc}.
 // reference: include/tim/vx/ops/groupedconv2d.h:56-82, src/tim/vx/ops/groupedconv2d.cc
@@ -287,6 +314,40 @@ class DeConv2d : public BuiltinOp {
   const std::array<uint32_t, 2> stride_;
   const std::array<uint32_t, 2> output_padding_;
   const std::array<uint32_t, 4> pad_;
+  const uint32_t group_;
+  const DataLayout kernel_layout_;
+};
+
+// Transposed 1-D convolution: DeConv2d on {W, C, N} tensors, weight {Kw, Ic / groups, Oc} (the 2-D operator on rows
+// of height one, as ovxlib reshapes it: src/tim/vx/internal/src/ops/vsi_nn_op_deconvolution1d.c:62-72).
+// reference: include/tim/vx/ops/deconv1d.h:53-90, src/tim/vx/ops/deconv1d.cc:36-98
+class DeConv1d : public BuiltinOp {
+ public:
+  DeConv1d(Graph* graph, PadType pad_type, uint32_t stride, uint32_t output_padding, uint32_t group = 1,
+           DataLayout input_layout = DataLayout::WHCN, DataLayout kernel_layout = DataLayout::WHIcOc);
+  DeConv1d(Graph* graph, const std::array<uint32_t, 2>& pad, uint32_t stride, uint32_t output_padding,
+           uint32_t group = 1, DataLayout input_layout = DataLayout::WHCN,
+           DataLayout kernel_layout = DataLayout::WHIcOc);
+  DeConv1d(Graph* graph, int32_t oc_count_, PadType pad_type, uint32_t ksize, uint32_t stride,
+           uint32_t output_padding);
+  DeConv1d(Graph* graph, int32_t oc_count_, PadType pad_type, uint32_t ksize, uint32_t stride,
+           uint32_t output_padding, const std::array<uint32_t, 2>& pad, uint32_t group = 1);
+  DeConv1d(Graph* graph, PadType pad_type, uint32_t stride, uint32_t output_padding,
+           const std::array<uint32_t, 2>& pad, uint32_t group, DataLayout input_layout,
+           DataLayout kernel_layout);
+
+  DataLayout KernelDataLayout() { return kernel_layout_; }
+  std::shared_ptr<Operation> Clone(
+      std::shared_ptr<Graph>& graph) const override;
+
+ protected:
+  void OnBindInputPostProc(const std::shared_ptr<Tensor>& tensor, int32_t input_idx) override;
+  const uint32_t oc_count_;
+  const PadType pad_type_;
+  const uint32_t ksize_;
+  const uint32_t stride_;
+  const uint32_t output_padding_;
+  const std::array<uint32_t, 2> pad_;
   const uint32_t group_;
   const DataLayout kernel_layout_;
 };

@@ -807,6 +807,38 @@ void Conv1d::OnBindInputPostProc(const std::shared_ptr<Tensor>& tensor, int32_t)
   PromoteHalfBias(this, impl_.get(), tensor);
 }
 
+// ---- GroupedConv1d (reference: src/tim/vx/ops/groupedconv1d.cc:34-66) -------
+GroupedConv1d::GroupedConv1d(Graph* graph, PadType padding, const uint32_t stride, const uint32_t dilation,
+                             uint32_t group, DataLayout input_layout, DataLayout kernel_layout)
+    : GroupedConv1d(graph, padding, {0, 0}, stride, dilation, group, input_layout, kernel_layout) {}
+
+GroupedConv1d::GroupedConv1d(Graph* graph, PadType padding, std::array<uint32_t, 2> pad, uint32_t stride,
+                             uint32_t dilation, uint32_t group, DataLayout input_layout, DataLayout kernel_layout)
+    : BuiltinOp(graph, K(OpKind::CONV2D), 0, 0, input_layout),
+      padding_(padding), pad_(pad), stride_(stride), dilation_(dilation), group_(group),
+      kernel_layout_(kernel_layout) {
+  OpAttrs& a = impl_->attrs_;
+  a.kernel_layout = kernel_layout_;
+  a.conv_1d = true;
+  a.pad_type = padding_ == PadType::NONE ? PadType::AUTO : padding_;
+  a.pad[0] = pad_[0];
+  a.pad[1] = pad_[1];
+  a.stride[0] = stride_;
+  a.stride[1] = 1;
+  a.dilation[0] = dilation_;
+  a.dilation[1] = 1;
+  a.groups = static_cast<int32_t>(group_);
+}
+
+std::shared_ptr<Operation> GroupedConv1d::Clone(std::shared_ptr<Graph>& graph) const {
+  return graph->CreateOperation<GroupedConv1d>(padding_, pad_, stride_, dilation_, group_, impl_->layout_,
+                                               kernel_layout_);
+}
+
+void GroupedConv1d::OnBindInputPostProc(const std::shared_ptr<Tensor>& tensor, int32_t) {
+  PromoteHalfBias(this, impl_.get(), tensor);
+}
+
 // ---- GroupedConv2d ----------------------------------------------------------
 // The same operator kind as Conv2d with a group count (the reference has a kind of its own,
 // VSI_NN_OP_GROUPED_CONV2D, whose setup splits into per-group convolutions:
@@ -1063,6 +1095,51 @@ std::shared_ptr<Operation> DeConv2d::Clone(std::shared_ptr<Graph>& graph) const 
 }
 
 void DeConv2d::OnBindInputPostProc(const std::shared_ptr<Tensor>& tensor, int32_t) {
+  PromoteHalfBias(this, impl_.get(), tensor);
+}
+
+// ---- DeConv1d (reference: src/tim/vx/ops/deconv1d.cc:36-98) ------------------------------------
+DeConv1d::DeConv1d(Graph* graph, PadType pad_type, uint32_t stride, uint32_t output_padding, uint32_t group,
+                   DataLayout input_layout, DataLayout kernel_layout)
+    : DeConv1d(graph, pad_type, stride, output_padding, {0, 0}, group, input_layout, kernel_layout) {}
+
+DeConv1d::DeConv1d(Graph* graph, const std::array<uint32_t, 2>& pad, uint32_t stride, uint32_t output_padding,
+                   uint32_t group, DataLayout input_layout, DataLayout kernel_layout)
+    : DeConv1d(graph, PadType::AUTO, stride, output_padding, pad, group, input_layout, kernel_layout) {}
+
+DeConv1d::DeConv1d(Graph* graph, int32_t, PadType pad_type, uint32_t, uint32_t stride, uint32_t output_padding)
+    : DeConv1d(graph, pad_type, stride, output_padding, {0, 0}, 1, DataLayout::WHCN, DataLayout::WHIcOc) {}
+
+DeConv1d::DeConv1d(Graph* graph, int32_t, PadType pad_type, uint32_t, uint32_t stride, uint32_t output_padding,
+                   const std::array<uint32_t, 2>& pad, uint32_t group)
+    : DeConv1d(graph, pad_type, stride, output_padding, pad, group, DataLayout::WHCN, DataLayout::WHIcOc) {}
+
+// (as in the reference, the channel count and kernel size arguments are not forwarded: the weight tensor has them)
+DeConv1d::DeConv1d(Graph* graph, PadType pad_type, uint32_t stride, uint32_t output_padding,
+                   const std::array<uint32_t, 2>& pad, uint32_t group, DataLayout input_layout,
+                   DataLayout kernel_layout)
+    : BuiltinOp(graph, K(OpKind::DECONV2D), 0, 0, input_layout),
+      oc_count_(0), pad_type_(pad_type), ksize_(0), stride_(stride), output_padding_(output_padding), pad_(pad),
+      group_(group), kernel_layout_(kernel_layout) {
+  OpAttrs& a = impl_->attrs_;
+  a.kernel_layout = kernel_layout_;
+  a.conv_1d = true;
+  a.pad_type = PadType::AUTO;  // the explicit pads size the output (vsi_nn_op_deconvolution1d.c:250-259)
+  a.pad[0] = pad_[0];
+  a.pad[1] = pad_[1];
+  a.stride[0] = stride_;
+  a.stride[1] = 1;
+  a.output_padding[0] = output_padding_;
+  a.output_padding[1] = 0;
+  a.groups = static_cast<int32_t>(group_);
+}
+
+std::shared_ptr<Operation> DeConv1d::Clone(std::shared_ptr<Graph>& graph) const {
+  return graph->CreateOperation<DeConv1d>(pad_type_, stride_, output_padding_, pad_, group_, impl_->layout_,
+                                          kernel_layout_);
+}
+
+void DeConv1d::OnBindInputPostProc(const std::shared_ptr<Tensor>& tensor, int32_t) {
   PromoteHalfBias(this, impl_.get(), tensor);
 }
 

@@ -210,6 +210,23 @@ bool SetupConv(OpImpl* op) {
       ComputeFilterSize(xs[0], ws[0], &a.pad[0], a.stride[0], a.dilation[0], RoundType::FLOOR),
       ComputeFilterSize(xs[1], ws[1], &a.pad[2], a.stride[1], a.dilation[1], RoundType::FLOOR),
       oc, xs[3]};
+  // A declared output that is longer than the pads make it reads padding behind the input's end: the reference
+  // hands the declared size to the driver as it is (its GroupedConv1d "PaddingTest": a two-column input under a
+  // three-tap VALID kernel with two declared output columns, golden = the window sliding over trailing zeros).
+  {
+    const ShapeType& have = y->spec_.shape_;
+    const size_t rank = one_d ? 3 : 4;
+    if (have.size() == rank) {
+      const uint32_t declared[2] = {have[0], one_d ? 1u : have[1]};
+      for (int i = 0; i < 2; ++i) {
+        if (declared[i] <= out[i]) continue;
+        const uint64_t reach = static_cast<uint64_t>(declared[i] - 1) * a.stride[i] + static_cast<uint64_t>(ws[i] - 1) * a.dilation[i] + 1;
+        const uint64_t span = static_cast<uint64_t>(xs[i]) + a.pad[2 * i] + a.pad[2 * i + 1];
+        if (reach > span) a.pad[2 * i + 1] += static_cast<uint32_t>(reach - span);
+        out[i] = declared[i];
+      }
+    }
+  }
   if (out[0] == 0 || out[1] == 0) {
     VSILOGE("CONV2D: empty output");
     return false;
@@ -228,14 +245,21 @@ bool SetupDeconv(OpImpl* op) {
   TensorImpl* b = op->inputs_tensor_.size() > 2 && !op->inputs_tensor_[2]->IsPlaceHolder()
                       ? Impl(op->inputs_tensor_[2]) : nullptr;
   TensorImpl* y = Impl(op->outputs_tensor_[0]);
-  if (op->layout_ != DataLayout::WHCN && op->layout_ != DataLayout::ANY) {
-    VSILOGE("DECONV2D: only WHCN activations are supported");
+  const bool one_d = op->attrs_.conv_1d;
+  if (op->layout_ != DataLayout::WHCN && op->layout_ != DataLayout::ANY && !(one_d && op->layout_ == DataLayout::WCN)) {
+    VSILOGE("DECONV2D: only WHCN (1-D: WCN) activations are supported");
     return false;
   }
-  const ShapeType &xs = x->spec_.shape_, &ws = w->spec_.shape_;
-  if (xs.size() != 4 || ws.size() != 4) {
-    VSILOGE("DECONV2D: input and weight must be 4-D");
+  // DeConv1d: {W, C, N} x {Kw, Ic, Oc} is the 2-D operator on {W, 1, C, N} x {Kw, 1, Ic, Oc}
+  // (src/tim/vx/internal/src/ops/vsi_nn_op_deconvolution1d.c:62-72 reshapes the weight the same way)
+  ShapeType xs = x->spec_.shape_, ws = w->spec_.shape_;
+  if (one_d ? (xs.size() != 3 || ws.size() != 3) : (xs.size() != 4 || ws.size() != 4)) {
+    VSILOGE("%s", one_d ? "DECONV1D: input and weight must be 3-D" : "DECONV2D: input and weight must be 4-D");
     return false;
+  }
+  if (one_d) {
+    xs = {xs[0], 1, xs[1], xs[2]};
+    ws = {ws[0], 1, ws[1], ws[2]};
   }
   if (!BiasScaleConsistent(x->spec_, w->spec_, b ? &b->spec_ : nullptr)) return false;
   if (!WeightPairSupported(x->spec_, w->spec_)) {
@@ -272,6 +296,7 @@ bool SetupDeconv(OpImpl* op) {
     VSILOGE("DECONV2D: empty output");
     return false;
   }
+  if (one_d) return AssignShape(y, ShapeType{static_cast<uint32_t>(ow), oc, xs[3]}, "DECONV1D", 1);
   return AssignShape(y, ShapeType{static_cast<uint32_t>(ow), static_cast<uint32_t>(oh), oc, xs[3]}, "DECONV2D", 2);
 }
 

@@ -279,7 +279,8 @@ struct Walk {
           new_ins.push_back(t->IsPlaceHolder() ? dst->CreateTensorPlaceHolder() : InLayout(t, Identity(RankOf(t))));
         const size_t out_rank = im->kind_ == OpKind::FCL ? 2
                                 : im->kind_ == OpKind::RESHAPE ? im->attrs_.new_shape.size()
-                                : im->kind_ == OpKind::TRANSPOSE ? im->attrs_.perm.size() : 4;
+                                : im->kind_ == OpKind::TRANSPOSE ? im->attrs_.perm.size()
+                                : im->attrs_.conv_1d ? 3 : 4;  // (DeConv1d: {W, C, N})
         out_pv = Identity(out_rank);
         clone = op->Clone(dst);
         break;

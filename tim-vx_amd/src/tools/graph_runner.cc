@@ -239,7 +239,14 @@ int main(int argc, char** argv) {
       std::shared_ptr<Operation> op;
       std::shared_ptr<Graph> target = graph;
       if (use_clone) graph = donor;
-      if (kind == "CONV2D" && conv_1d) {
+      if (kind == "CONV2D" && conv_1d && groups > 1) {
+        op = graph->CreateOperation<ops::GroupedConv1d>(ParsePad(pad_type), std::array<uint32_t, 2>{pad[0], pad[1]},
+                                                        stride[0], dil[0], static_cast<uint32_t>(groups));
+      } else if (kind == "DECONV2D" && conv_1d) {
+        op = graph->CreateOperation<ops::DeConv1d>(weights, ParsePad(pad_type), ksize[0], stride[0], out_pad[0],
+                                                   std::array<uint32_t, 2>{pad[0], pad[1]},
+                                                   static_cast<uint32_t>(groups > 0 ? groups : 1));
+      } else if (kind == "CONV2D" && conv_1d) {
         op = graph->CreateOperation<ops::Conv1d>(weights, ParsePad(pad_type), ksize[0], stride[0], dil[0],
                                                  std::array<uint32_t, 2>{pad[0], pad[1]}, multiplier);
       } else if (kind == "CONV2D" && groups > 1) {
