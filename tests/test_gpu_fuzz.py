@@ -206,3 +206,42 @@ def test_pool2d_sweep(oracle):
         want = oracle.pool2d(x, in_q=in_q, out_q=out_q, **kws)
         got = TC.gpu_pool2d(x, in_q=in_q, out_q=out_q, **kws)
         assert np.array_equal(got, want), (i, kws)
+
+
+def test_depthwise_eight_column_form_sweep(oracle):
+    """Stride-1 depthwise 3x3 on rows of whole 8-byte units (the form with 64-bit row loads): random plane sizes up
+    to several workgroups per plane, left / top padding 0 or 1, and tensors 0, 4 or 8 bytes off their allocations
+    (4: the four-column form has to take over at run time)."""
+    rng = np.random.default_rng(77)
+    for i in range(60):
+        n, c = int(rng.integers(1, 4)), int(rng.integers(1, 20))
+        h, w = int(rng.integers(3, 120)), 8 * int(rng.integers(1, 33))
+        pl, pt = int(rng.integers(0, 2)), int(rng.integers(0, 2))
+        mode = str(rng.choice(["u8", "i8pc", "u8pc"]))
+        x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=0, kh=3, kw=3, stride=[1, 1], dil=[1, 1],
+                                  pad=[pl, 2 - pl, pt, 2 - pt], mult=1, mode=mode)
+        act, mis = int(rng.integers(0, 3)), int(rng.choice([0, 0, 4, 8]))
+        want = oracle.conv2d(x, wt, b, act=act, **kws)
+        got = TC.gpu_conv2d(x, wt, b, act=act, want_kernel="dwconv3x3_i8", misalign=mis, **kws)
+        assert np.array_equal(got, want), (i, n, c, h, w, pl, pt, mode, act, mis, int((got != want).sum()))
+
+
+def test_pointwise_streaming_form_sweep(oracle, monkeypatch):
+    """The streaming pointwise form forced onto random small cases: 1 to 32 input channels, pixel counts that are
+    multiples of 16 in several ways, partial output tiles, 1 to 5 pixel tiles per wavefront."""
+    monkeypatch.setenv("TVX_PWCONV_STREAM_MIN_TILES", "1")
+    monkeypatch.setenv("TVX_PWCONV_SHAPE", "128,1")
+    rng = np.random.default_rng(78)
+    for i in range(60):
+        n, c, oc = int(rng.integers(1, 6)), int(rng.integers(1, 33)), int(rng.integers(1, 200))
+        w, h = 16, int(rng.integers(1, 40))
+        if rng.integers(0, 2):
+            w, h = 4 * int(rng.integers(1, 9)), 4 * int(rng.integers(1, 9))
+        monkeypatch.setenv("TVX_PWCONV_STREAM", str(int(rng.integers(1, 6))))
+        mode = str(rng.choice(["u8", "i8pc", "u8pc"]))
+        x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=oc, kh=1, kw=1, stride=[1, 1], dil=[1, 1],
+                                  pad=[0, 0, 0, 0], mult=0, mode=mode)
+        act = int(rng.integers(0, 3))
+        want = oracle.conv2d(x, wt, b, act=act, **kws)
+        got = TC.gpu_conv2d(x, wt, b, act=act, want_kernel="pwconv_i8_stream", **kws)
+        assert np.array_equal(got, want), (i, n, c, h, w, oc, mode, act, int((got != want).sum()))
