@@ -223,6 +223,8 @@ bool SetupConv(OpImpl* op) {
         const uint64_t reach = static_cast<uint64_t>(declared[i] - 1) * a.stride[i] + static_cast<uint64_t>(ws[i] - 1) * a.dilation[i] + 1;
         const uint64_t span = static_cast<uint64_t>(xs[i]) + a.pad[2 * i] + a.pad[2 * i + 1];
         if (reach > span) a.pad[2 * i + 1] += static_cast<uint32_t>(reach - span);
+        VSILOGW("%s: declared output dim %d = %u, the pads give %u; the last windows read padding behind the input",
+                one_d ? "CONV1D" : "CONV2D", i, declared[i], out[i]);
         out[i] = declared[i];
       }
     }
