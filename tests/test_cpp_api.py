@@ -132,6 +132,24 @@ def test_every_reference_golden_through_the_platform_api(tmp_path):
 
 
 @pytest.mark.gpu
+def test_every_reference_golden_through_clone(tmp_path):
+    """The same graphs with every operator created in a second graph and cloned into the one that runs
+    (Operation::Clone, include/tim/vx/operation.h:46): Conv2d, Conv1d, GroupedConv2d, GroupedConv1d, DeConv2d,
+    DeConv1d, FullyConnected, Pool2d, Softmax, Transpose and DataConvert each carry their attributes over."""
+    cases = [c for c in _named_cases() if not c.get("layout_inference")]
+    for c in cases:
+        c["clone"] = True
+    res, info, log = GF.run_graphs(cases, str(tmp_path))
+    bad = []
+    for c, out in zip(cases, res):
+        if out is None:
+            bad.append((c["test"], info.get(c["test"])))
+        elif not TC.matches(c, out):
+            bad.append((c["test"], out[:8], TC.golden_of(c)[:8]))
+    assert not bad, (bad[:5], log[-2000:])
+
+
+@pytest.mark.gpu
 def test_lenet_sample_graph(tmp_path, oracle):
     w, x = _lenet_data()
     g = GRAPHS.lenet_asymu8(w, x)
