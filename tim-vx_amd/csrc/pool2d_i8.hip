@@ -184,7 +184,44 @@ __global__ void __launch_bounds__(kThreads) PoolRowsKernel(PoolRowsArgs a) {
   }
   __syncthreads();
   // ---- the input rows: per plane one contiguous range, read as aligned dwords ---------------------
-  if (ih_hi > ih_lo) {
+  const uint32_t plane_bytes = static_cast<uint32_t>(a.H) * static_cast<uint32_t>(a.W);
+  if (ih_lo == 0 && ih_hi == a.H && (a.W & 3) == 0 && (a.pad_l & 3) == 0 && a.magic_plane != 0 &&
+      ((reinterpret_cast<uintptr_t>(a.x) + static_cast<size_t>(p0) * plane_bytes) & 15) == 0 && ((static_cast<size_t>(g_n) * plane_bytes) & 15) == 0) {
+    // Whole planes of whole dwords: the workgroup's planes are one contiguous range. It is read as 16-byte chunks
+    // in lane order, every thread's loads issued before the first is used - plane by plane (below) small planes
+    // cost one memory round trip each.
+    const uint32_t row_bytes = static_cast<uint32_t>(a.W);
+    const uint32_t n16 = static_cast<uint32_t>(g_n) * plane_bytes >> 4;
+    const v4i* src16 = reinterpret_cast<const v4i*>(a.x + static_cast<size_t>(p0) * plane_bytes);
+    uint8_t* dst0 = lds + (0 - ih_first) * a.pitch + a.pad_l;
+    auto put16 = [&](uint32_t i, const v4i& v) {
+      const uint32_t o = i << 4;
+      const uint32_t g = __umulhi(o, a.magic_plane);
+      const uint32_t po = o - g * plane_bytes;
+      uint32_t r = DivMagic(po, a.magic_w, row_bytes);
+      uint32_t c = po - r * row_bytes;
+      uint8_t* dst_plane = dst0 + g * plane_lds;
+      uint32_t gg = g;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        *reinterpret_cast<uint32_t*>(dst_plane + r * a.pitch + c) = static_cast<uint32_t>(v[q]);
+        c += 4;
+        if (c == row_bytes) {
+          c = 0;
+          if (++r == static_cast<uint32_t>(a.H)) { r = 0; ++gg; dst_plane = dst0 + gg * plane_lds; }  // (a chunk may run into the next plane)
+        }
+      }
+    };
+    constexpr int kInFlight = 4;
+    for (uint32_t i0 = tid; i0 < n16; i0 += kInFlight * kThreads) {
+      v4i v[kInFlight];
+#pragma unroll
+      for (int k = 0; k < kInFlight; ++k) v[k] = src16[min(i0 + k * kThreads, n16 - 1)];
+#pragma unroll
+      for (int k = 0; k < kInFlight; ++k)
+        if (i0 + k * kThreads < n16) put16(i0 + k * kThreads, v[k]);
+    }
+  } else if (ih_hi > ih_lo) {
     const uint32_t row_bytes = static_cast<uint32_t>(a.W);
     const uint32_t range = static_cast<uint32_t>(ih_hi - ih_lo) * row_bytes;  // bytes per plane
     for (int g = 0; g < g_n; ++g) {
@@ -425,6 +462,11 @@ int PoolRowsSetup(tvx_op* op) {
   a.magic_w = a.W <= 1 ? 0u : static_cast<uint32_t>(((uint64_t{1} << 32) + a.W - 1) / a.W);
   a.magic_ow4 = a.ow4 <= 1 ? 0u : static_cast<uint32_t>(((uint64_t{1} << 32) + a.ow4 - 1) / a.ow4);
   a.magic_oh = a.OH <= 1 ? 0u : static_cast<uint32_t>(((uint64_t{1} << 32) + a.OH - 1) / a.OH);
+  {
+    // plane index of a byte offset inside a workgroup's planes (offsets below G * plane bytes; exact while offset * plane bytes < 2^32)
+    const uint64_t pb = static_cast<uint64_t>(a.W) * a.H;
+    a.magic_plane = (pb > 1 && pb * pb * static_cast<uint64_t>(a.G) < (1ull << 32)) ? static_cast<uint32_t>(((uint64_t{1} << 32) + pb - 1) / pb) : 0u;
+  }
   // (a workgroup's items fit its LDS image, fewer than 2^14, and OH, ow4 < 2^15: the products stay below 2^32)
   // the byte offsets divided by W stay below 2^32 / W: a band holds at most rows_in * W < 2^30 bytes
   if (static_cast<uint64_t>(a.rows_in) * a.W * a.W >= (1ull << 32)) return TVX_E_UNSUPPORTED;
