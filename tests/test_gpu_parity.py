@@ -843,6 +843,12 @@ IM2COL_GRID = [
     dict(n=2, c=3, h=64, w=64, oc=64, kh=3, kw=3, stride=[1, 1], dil=[1, 1], pad=[1, 1, 1, 1], mult=0),   # several workgroups per image
     dict(n=1, c=5, h=10, w=6, oc=40, kh=2, kw=3, stride=[1, 1], dil=[1, 3], pad=[2, 2, 1, 1], mult=0),    # rows as dwords that begin two bytes in front of the tensor / end behind it
     dict(n=1, c=1, h=1, w=4, oc=3, kh=1, kw=3, stride=[1, 1], dil=[1, 1], pad=[2, 2, 0, 0], mult=0),      # a four-byte tensor
+    # kernel rows five taps wide: two dwords per row
+    dict(n=1, c=1, h=1, w=5, oc=4, kh=1, kw=5, stride=[1, 1], dil=[1, 1], pad=[2, 2, 0, 0], mult=0),      # a five-byte tensor: both dwords moved inside
+    dict(n=1, c=1, h=2, w=4, oc=3, kh=1, kw=5, stride=[1, 1], dil=[1, 1], pad=[2, 2, 0, 0], mult=0),      # eight bytes: the second dword of the last windows lies behind the tensor
+    dict(n=2, c=2, h=7, w=9, oc=33, kh=5, kw=5, stride=[1, 1], dil=[1, 1], pad=[2, 2, 2, 2], mult=0),     # SAME 5 x 5, K = 50, two channel tiles
+    dict(n=3, c=1, h=11, w=13, oc=7, kh=3, kw=5, stride=[2, 1], dil=[1, 1], pad=[1, 3, 1, 1], mult=0),    # uneven pads, strides
+    dict(n=1, c=4, h=6, w=6, oc=9, kh=3, kw=5, stride=[1, 1], dil=[2, 1], pad=[4, 4, 2, 2], mult=0),      # K = 60, left padding as wide as the window reaches
 ]
 
 

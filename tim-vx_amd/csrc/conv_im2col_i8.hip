@@ -44,15 +44,15 @@ struct ImArgs {
   // c * H * W + dy * W + dx. They travel in the kernel arguments so that the (wavefront-uniform) reads
   // are scalar loads of memory nothing can write; a table in global memory is read per lane, one round
   // trip a tap.
-  // In row mode (kernels three taps wide, unit dilation along the row) entry r stands for a whole
-  // kernel row of a channel: dy | 1 << 16 and c * H * W + dy * W; the three taps are one dword load.
+  // In row mode (kernels three or five taps wide, unit dilation along the row) entry r stands for a whole
+  // kernel row of a channel: dy | 1 << 16 and c * H * W + dy * W; the taps are one or two dword loads.
   int taps[64];
   int offs[64];
   int rows;              // row mode: C * Kh
   int total_bytes;       // row mode: size of the input tensor (< 2^31)
 };
 
-// KW: 0 = any window, one byte load per tap; 3 = row mode
+// KW: 0 = any window, one byte load per tap; 3 / 5 = row mode for kernels three / five taps wide
 template <int OT, int RQ, int KW>
 __global__ void __launch_bounds__(kThreads) ConvIm2colKernel(ImArgs a) {
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
@@ -100,32 +100,38 @@ __global__ void __launch_bounds__(kThreads) ConvIm2colKernel(ImArgs a) {
       return n <= 0 ? 0u : ((n >= 32 ? 0xffffffffu : ((1u << n) - 1u)) << lo);
     };
     const uint32_t row_ok = span_mask(ih0, a.H), col_ok = span_mask(iw0, a.W);
-    if constexpr (KW == 3) {
+    if constexpr (KW == 3 || KW == 5) {
       // Row mode: byte loads cost the L1 a tag lookup for every few lanes, and those lookups bound the
-      // gather; the three taps of a kernel row are adjacent bytes, so one (unaligned) dword fetches
-      // them. The dword may begin in front of the tensor (left padding of its first row) or end behind
-      // it: it is moved inside by up to three bytes and shifted back. A row with no tap inside the
-      // image reads the tensor's first dword and is not used.
-      constexpr int kMaxRows = 64 / 3;
+      // gather; the taps of a kernel row are adjacent bytes, so one (unaligned) dword fetches three of
+      // them, two dwords five. A dword may begin in front of the tensor (left padding of its first row)
+      // or end behind it: it is moved inside and shifted back. A row with no tap inside the image reads
+      // the tensor's first dword(s) and is not used.
+      constexpr int kMaxRows = 64 / KW;
+      constexpr uint32_t kColMask = (1u << KW) - 1u;
       const int img_at = n * (a.C * a.H * a.W) + origin;
-      auto place = [&](int r, bool* row_in, int* moved) {  // -> byte index of the row's dword in the tensor
+      auto place = [&](int r, int which, bool* row_in, int* moved) {  // -> byte index of the row's dword `which` in the tensor
         const int t = a.taps[r];
         *row_in = ((row_ok >> (t & 0xff)) & static_cast<uint32_t>(t >> 16) & 1u) != 0;
-        const bool any = *row_in & ((col_ok & 7u) != 0);
-        const int want = any ? img_at + a.offs[r] : 0;
+        const bool any = *row_in & ((col_ok & kColMask) != 0);
+        const int want = (any ? img_at + a.offs[r] : 0) + 4 * which;
         const int at = min(max(want, 0), a.total_bytes - 4);
-        *moved = at - want;  // -3 .. 3
+        *moved = at - want;  // first dword: -3 .. 3; second: -7 .. 0
         return at;
       };
-      uint32_t v[kMaxRows];
+      uint32_t v[kMaxRows], v2[KW == 5 ? kMaxRows : 1];
 #pragma unroll
       for (int r = 0; r < kMaxRows; ++r) {
         v[r] = 0;
+        if (KW == 5) v2[r] = 0;
         if (r < a.rows) {  // uniform
           bool row_in;
           int moved;
-          const int at = place(r, &row_in, &moved);
+          const int at = place(r, 0, &row_in, &moved);
           __builtin_memcpy(&v[r], a.x + static_cast<uint32_t>(at), 4);
+          if constexpr (KW == 5) {
+            const int at2 = place(r, 1, &row_in, &moved);
+            __builtin_memcpy(&v2[r], a.x + static_cast<uint32_t>(at2), 4);
+          }
         }
       }
       __builtin_amdgcn_sched_barrier(0);  // all loads travel together
@@ -137,13 +143,19 @@ __global__ void __launch_bounds__(kThreads) ConvIm2colKernel(ImArgs a) {
         if (r < a.rows) {
           bool row_in;
           int moved;
-          (void)place(r, &row_in, &moved);
+          (void)place(r, 0, &row_in, &moved);
           const uint32_t got = moved >= 0 ? v[r] << (8 * moved) : v[r] >> (-8 * moved);
+          uint32_t got2 = 0;  // (fifth tap: the second dword's first byte)
+          if constexpr (KW == 5) {
+            (void)place(r, 1, &row_in, &moved);
+            got2 = moved <= -4 ? 0u : v2[r] >> (-8 * moved);  // (moved by four bytes or more: the tap lies behind the tensor and is masked)
+          }
 #pragma unroll
-          for (int e = 0; e < 3; ++e) {
+          for (int e = 0; e < KW; ++e) {
             const bool inside = row_in & (((col_ok >> e) & 1u) != 0);
-            const int byte = inside ? static_cast<int>(((got >> (8 * e)) & 0xffu) ^ static_cast<uint32_t>(a.xor_mask)) : a.pad_fill;
-            const int k = r * 3 + e;
+            const uint32_t raw = e < 4 ? (got >> (8 * e)) & 0xffu : got2 & 0xffu;
+            const int byte = inside ? static_cast<int>(raw ^ static_cast<uint32_t>(a.xor_mask)) : a.pad_fill;
+            const int k = r * KW + e;
             dw[k >> 2] |= byte << (8 * (k & 3));
           }
         }
@@ -282,7 +294,8 @@ int ConvIm2colRun(tvx_op* op, const void* in0, const void*, void* out, hipStream
   ImArgs a = plan->a;
   a.x = static_cast<const uint8_t*>(in0);
   a.y = static_cast<uint8_t*>(out);
-  if (plan->row_mode) LaunchOt<3>(plan, a, st);
+  if (plan->row_mode == 5) LaunchOt<5>(plan, a, st);
+  else if (plan->row_mode) LaunchOt<3>(plan, a, st);
   else LaunchOt<0>(plan, a, st);
   TVX_HIP_CHECK(hipGetLastError());
   return TVX_OK;
@@ -346,7 +359,7 @@ int ConvIm2colSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, co
                                      AccumulatorBound(static_cast<uint64_t>(K), bias_host, a.OC));
   if ((d->k_h - 1) * d->dilation_h > 31 || (d->k_w - 1) * d->dilation_w > 31) return TVX_E_UNSUPPORTED;  // window offsets index 32-bit masks
   const uint64_t total_bytes = static_cast<uint64_t>(d->batch) * d->in_c * d->in_h * d->in_w;
-  bool row_mode = d->k_w == 3 && d->dilation_w == 1 && total_bytes >= 4 && total_bytes < (1ull << 31);
+  bool row_mode = (d->k_w == 3 || d->k_w == 5) && d->dilation_w == 1 && total_bytes >= 4 && total_bytes < (1ull << 31);
   if (const char* f = getenv("TVX_IM2COL_ROWS")) row_mode = row_mode && atoi(f) != 0;  // tuning aid
   if (row_mode) {
     a.rows = static_cast<int>(d->in_c * d->k_h);
@@ -379,7 +392,7 @@ int ConvIm2colSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, co
   plan.lds_bytes = lds_bytes;
   plan.ot = ot;
   plan.rq = rq;
-  plan.row_mode = row_mode ? 1 : 0;
+  plan.row_mode = row_mode ? static_cast<int>(d->k_w) : 0;  // 0, or the taps of a kernel row (3 / 5)
   const int hw = a.OH * a.OW;
   plan.grid = dim3(static_cast<unsigned>((hw + kPixels - 1) / kPixels), static_cast<unsigned>(d->batch));
   op->host_blob.assign(reinterpret_cast<const uint8_t*>(&plan), reinterpret_cast<const uint8_t*>(&plan) + sizeof(plan));
