@@ -379,12 +379,12 @@ def test_conv2d_cfg2_full_size(oracle):
                dilation=[1, 1], pad_left=1, pad_top=1, multiplier=0, in_dtype=0, w_dtype=0, out_dtype=0,
                in_q=(0.05, 128), w_q=(0.01, 120, None), out_q=(0.1, 0), act=2)
     want = oracle.conv2d(x, wt, b, **kws)
-    got = TC.gpu_conv2d(x, wt, b, want_kernel="conv2d_igemm_i8_persistent", **kws)
+    got = TC.gpu_conv2d(x, wt, b, want_kernel="conv2d_band_i8", **kws)
     assert np.array_equal(got, want)
     assert got.max() == 60 and len(np.unique(got)) == 61  # ReLU6 at scale 0.1: q in [0, 60]
 
 
-IGEMM_KERNELS = ("conv2d_igemm_i8", "conv2d_igemm_i8_persistent")
+IGEMM_KERNELS = ("conv2d_igemm_i8", "conv2d_igemm_i8_persistent", "conv2d_band_i8")
 
 IGEMM_GRID = [
     # (n, c, h, w, oc, kh, kw, stride, dil, pad[l,r,t,b])
@@ -441,6 +441,7 @@ def test_conv2d_igemm_persistent(oracle, gi, mode, knobs, monkeypatch):
     every workgroup walks many tiles through both halo buffers (tiles of one, two and more output rows)."""
     n, c, h, w, oc, kh, kw, stride, dil, pad = PERSIST_GRID[gi]
     monkeypatch.setenv("TVX_IGEMM_PERSIST", "1")   # also where the heuristic would take the one-tile-per-workgroup kernel
+    monkeypatch.setenv("TVX_CONV_BAND", "0")       # (the kernel that is asked first)
     for k, v in knobs.items():
         monkeypatch.setenv(k, v)
     rng = np.random.default_rng(2500 + gi)
@@ -449,6 +450,44 @@ def test_conv2d_igemm_persistent(oracle, gi, mode, knobs, monkeypatch):
     for act in (0, 2):
         want = oracle.conv2d(x, wt, b, act=act, **kws)
         got = TC.gpu_conv2d(x, wt, b, act=act, want_kernel="conv2d_igemm_i8_persistent", **kws)
+        assert np.array_equal(got, want), (int((got != want).sum()), np.flatnonzero(got != want)[:8])
+    assert len(np.unique(want)) > 4
+
+
+BAND_GRID = [
+    # (n, c, h, w, oc, kh, kw, stride, dil, pad[l,r,t,b]): shapes of the one-workgroup-per-CU kernel (weights in LDS:
+    # 32 or 64 input channels under a 3x3 kernel, 33..64 output channels, input and output rows of whole 8-byte units)
+    (5, 64, 56, 56, 64, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),
+    (3, 32, 28, 24, 64, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),
+    (4, 64, 20, 24, 40, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),     # 40 output channels: the second channel tile is ragged
+    (3, 32, 17, 32, 33, 3, 3, [2, 2], [1, 1], [0, 1, 0, 1]),     # stride 2
+    (2, 64, 16, 16, 48, 3, 3, [1, 1], [2, 2], [2, 2, 2, 2]),     # dilation 2: five halo rows per output row
+    (9, 64, 8, 8, 64, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),       # whole images smaller than one band
+    (2, 32, 9, 64, 64, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),      # 64 columns
+    (2, 64, 11, 16, 64, 3, 3, [1, 1], [1, 1], [1, 1, 0, 2]),     # all vertical padding below
+    (2, 64, 13, 16, 56, 3, 3, [1, 1], [1, 1], [0, 2, 1, 1]),     # all horizontal padding on the right
+    (3, 64, 23, 40, 64, 3, 3, [1, 1], [1, 1], [1, 1, 1, 1]),     # 23 rows: the last band of an image is short
+]
+
+
+@pytest.mark.parametrize("knobs", [{}, {"TVX_BAND_WGS": "8"}, {"TVX_BAND_WGS": "16", "TVX_BAND_ROWS": "2"},
+                                   {"TVX_BAND_WGS": "8", "TVX_BAND_ROWS": "1"}, {"TVX_BAND_ROWS": "3"}],
+                         ids=lambda k: "-".join(k.values()) or "default")
+@pytest.mark.parametrize("mode", ["u8", "i8pc", "u8pc"])
+@pytest.mark.parametrize("gi", range(len(BAND_GRID)))
+def test_conv2d_band(oracle, gi, mode, knobs, monkeypatch):
+    """The band kernel with its default launch and with few workgroups / short bands forced, so that every
+    workgroup walks many bands through both halo buffers (bands of one, two, three and more output rows)."""
+    n, c, h, w, oc, kh, kw, stride, dil, pad = BAND_GRID[gi]
+    monkeypatch.setenv("TVX_CONV_BAND", "1")   # also where few bands make the one-tile-per-workgroup kernel the choice
+    for k, v in knobs.items():
+        monkeypatch.setenv(k, v)
+    rng = np.random.default_rng(2600 + gi)
+    x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=oc, kh=kh, kw=kw, stride=stride, dil=dil,
+                              pad=pad, mult=0, mode=mode)
+    for act in (0, 2):
+        want = oracle.conv2d(x, wt, b, act=act, **kws)
+        got = TC.gpu_conv2d(x, wt, b, act=act, want_kernel="conv2d_band_i8", **kws)
         assert np.array_equal(got, want), (int((got != want).sum()), np.flatnonzero(got != want)[:8])
     assert len(np.unique(want)) > 4
 

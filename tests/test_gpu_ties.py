@@ -46,6 +46,8 @@ CONV_TIE_CASES = [
     ("pwconv_i8_stream", dict(n=2, c=32, h=16, w=16, oc=64, k=1, stride=1, pad=0, mult=0), (15, 7)),
     ("pwconv_i8_stream", dict(n=24, c=24, h=16, w=32, oc=72, k=1, stride=1, pad=0, mult=0), None),
     ("conv2d_igemm_i8_persistent", dict(n=2, c=32, h=28, w=28, oc=64, k=3, stride=1, pad=1, mult=0), (15, 7)),
+    ("conv2d_band_i8", dict(n=2, c=32, h=24, w=24, oc=64, k=3, stride=1, pad=1, mult=0), (15, 7)),
+    ("conv2d_band_i8", dict(n=10, c=64, h=28, w=24, oc=64, k=3, stride=1, pad=1, mult=0), None),
     ("conv2d_igemm_i8", dict(n=2, c=48, h=28, w=28, oc=96, k=3, stride=1, pad=1, mult=0), (15, 7)),
     ("conv2d_igemm_i8", dict(n=8, c=64, h=28, w=28, oc=80, k=3, stride=1, pad=1, mult=0), None),
     ("conv2d_igemm_i8_persistent", dict(n=10, c=64, h=28, w=28, oc=64, k=3, stride=1, pad=1, mult=0), None),
@@ -68,6 +70,9 @@ def test_conv_epilogues_round_ties_to_even(oracle, ci, mode, monkeypatch):
     kernel, g, amp = CONV_TIE_CASES[ci]
     if kernel.endswith("_persistent"):
         monkeypatch.setenv("TVX_IGEMM_PERSIST", "1")
+        monkeypatch.setenv("TVX_CONV_BAND", "0")
+    if kernel == "conv2d_band_i8":
+        monkeypatch.setenv("TVX_CONV_BAND", "1")
     if kernel.endswith("_stream"):  # (the form is chosen from 1024 pixel tiles up)
         monkeypatch.setenv("TVX_PWCONV_STREAM_MIN_TILES", "1")
         monkeypatch.setenv("TVX_PWCONV_SHAPE", "128,1")

@@ -27,6 +27,8 @@ int FcMfmaSetup(tvx_op*, const tvx_fc_desc*, const void*, const void*);
 
 // int8 MFMA implicit-GEMM convolution (conv_igemm_i8.hip)
 int ConvIgemmSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
+// the same for layers whose weights and two halo tiles fit LDS: one sixteen-wavefront workgroup per CU (conv_band_i8.hip)
+int ConvBandSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 // Dense quantized conv whose whole window (C * Kh * Kw) is at most 64 bytes: im2col rows in LDS + MFMA.
 int ConvIm2colSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 
