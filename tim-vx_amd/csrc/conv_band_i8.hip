@@ -17,8 +17,9 @@
 //            a SIMD).
 //   multiply wavefront w owns the band's 32-pixel tile w and both 32-channel tiles: per
 //            k-step one A and two B fragment reads feed two v_mfma_i32_32x32x32_i8.
-//   epilogue requantization from the wavefront's own accumulators into a wavefront-private
-//            staging tile, from there 16 bytes per lane to the WHCN output: no second barrier.
+//   epilogue requantization from the wavefront's own accumulators; two lane swaps between the
+//            wavefront's halves (v_permlane32_swap) give every lane sixteen consecutive pixels
+//            of a channel, which go to the WHCN output as they are: no staging in LDS.
 #include <algorithm>
 #include <cstdlib>
 
@@ -32,121 +33,169 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int kBandThreads = 1024;
 constexpr int kBandWaves = kBandThreads / 64;
-constexpr int kStageStride = 40;  // bytes per channel row of a wavefront's staging tile (32 pixels + bank spread)
 
 struct BandArgs {
+  // what stands between a wavefront's start and its first loads comes first
   const uint8_t* x;
-  const int8_t* w;       // packed [64][kstride]
-  uint8_t* y;
-  const int32_t* biasf;  // bias + per-channel zero-point terms
-  const v4i* rq;         // per channel {mult, t, rounding constant, tie mask}
+  int total_tiles, tiles_per_xcd;
+  int tiles_per_image, gblocks, gpr, iwt_div;
+  uint32_t magic_tpi, magic_gblocks, magic_gpr, magic_iwt, magic_ow, magic_padcols;
+  int n_g8;              // 8-column groups of a band's halo rows
   int C, H, W, OC, OH, OW;
   int sh, sw, pad_t, pad_l, khe;  // khe: rows a kernel column spans, (kh - 1) * dh + 1
   int rows;              // output rows of a band
   int PT;                // 32-pixel tiles of a full band
-  int tiles_per_image, total_tiles;
-  uint32_t magic_tpi, magic_ow, magic_gpr, magic_gblocks;
-  int gpr;               // 8-column groups per input row
-  int n_g8;              // ... per band (all halo rows)
-  int gblocks;           // blocks of sixteen such groups
   int iwt, pix_stride;
+  const int8_t* w;       // packed [64][kstride]
+  uint8_t* y;
+  const int32_t* biasf;  // bias + per-channel zero-point terms
+  const v4i* rq;         // per channel {mult, t, rounding constant, tie mask}
   int kstride, w_chunks;
+  int row_step, col_step;  // halo bytes from a kernel row / column to the next
+  int s_row_step, s_col_step;  // ... sum-plane cells
   int xor_mask, pad_fill, zws, out_zp, lo, hi;
-  int halo_rows, pad_cols;
-  int off_sx, off_rq, off_bias, off_w, off_stage, off_halo0, off_halo1;
-  int tap_off[20];       // halo byte offset of k-step ks (its two 16-byte halves lie side by side)
+  int halo_rows, pad_cols, s_pad;  // s_pad: channel sum of a padding pixel
+  int off_sx, off_rq, off_bias, off_w, off_halo0, off_halo1, off_s, s_bytes;
 };
 
 // u / d by the host-made reciprocal ceil(2^32 / d); 0 stands for d = 1
 __device__ __forceinline__ int FastDiv(int u, uint32_t magic) {
-  return magic ? static_cast<int>(__umulhi(static_cast<uint32_t>(u), magic)) : u;
+  return static_cast<int>(__umulhi(static_cast<uint32_t>(u), magic)) + (magic == 0 ? u : 0);
 }
 
-template <int KSTEPS, int RQ, bool ZP>
+// (v >> t) into byte E of d (the other bytes stay): the shift writes its result where the packed dword wants it
+template <int E>
+__device__ __forceinline__ void ShiftIntoByte(uint32_t& d, int t, int v) {
+  if (E == 0) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:DWORD" : "=v"(d) : "v"(t), "v"(v));
+  if (E == 1) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(d) : "v"(t), "v"(v));
+  if (E == 2) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(d) : "v"(t), "v"(v));
+  if (E == 3) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(d) : "v"(t), "v"(v));
+}
+
+// KH x KW taps over CPC 16-channel chunks (an even number): a k-step is one tap's pair of chunks.
+template <int KH, int KW, int CPC, int RQ, bool ZP>
 __global__ void __launch_bounds__(kBandThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))
 ConvBandKernel(BandArgs a) {
+  constexpr int KSTEPS = KH * KW * CPC / 2;
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int frag_row = lane & 31, frag_half = lane >> 5;
-  const int hw = a.OH * a.OW;
 
   // An XCD gets a contiguous run of bands (neighbouring bands of an image share halo rows and meet in that
   // XCD's L2); inside the run the XCD's workgroups interleave.
-  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3, per_xcd = gridDim.x >> 3;
-  const int t_first = static_cast<int>(static_cast<long long>(a.total_tiles) * xcd / 8);
-  const int t_end = static_cast<int>(static_cast<long long>(a.total_tiles) * (xcd + 1) / 8);
-  int t = t_first + slot;
+  const int xcd = blockIdx.x & 7, per_xcd = gridDim.x >> 3;
+  int t = xcd * a.tiles_per_xcd + (blockIdx.x >> 3);
+  const int t_end = min((xcd + 1) * a.tiles_per_xcd, a.total_tiles);
   if (t >= t_end) return;
-
-  int* sx_lds = reinterpret_cast<int*>(lds + a.off_sx) + wave * 32;  // wavefront-private
-  const v4i* rq_lds = reinterpret_cast<const v4i*>(lds + a.off_rq);
-  const int* bias_lds = reinterpret_cast<const int*>(lds + a.off_bias);
-  int8_t* stage = lds + a.off_stage + wave * (32 * kStageStride);  // wavefront-private
 
   // ---- this thread's patch: 8 input columns x 4 channels of one halo row. Sixteen consecutive lanes read
   // 128 contiguous bytes of a channel plane, the next sixteen the next channel group.
-  const size_t plane = static_cast<size_t>(a.H) * a.W;
-  const uint32_t plane32 = static_cast<uint32_t>(plane);
+  const uint32_t plane32 = static_cast<uint32_t>(a.H * a.W);
   const int cb = FastDiv(wave, a.magic_gblocks);
-  const int gb = wave - cb * a.gblocks;
-  const int g8 = gb * 16 + (lane & 15);
+  const int g8 = (wave - cb * a.gblocks) * 16 + (lane & 15);
   const int c4 = cb * 4 + (lane >> 4);
   const bool has_patch = g8 < a.n_g8 && c4 * 4 < a.C;
   const int hr = has_patch ? FastDiv(g8, a.magic_gpr) : 0;
   const int col0 = has_patch ? (g8 - hr * a.gpr) * 8 : 0;
-  uint32_t ch_off[4];
+  const uint32_t ch_off = has_patch ? static_cast<uint32_t>(c4 * 4) * plane32 + static_cast<uint32_t>(col0) : 0u;
+  const int px0 = hr * a.iwt + a.pad_l + col0;  // the patch's first pixel in the halo tile
+  // With the i-th store every lane would write its i-th pixel: pixels 8 apart, i.e. one LDS bank for all column
+  // groups of a wavefront. The lanes therefore rotate their pixels by their column group (the loaded dwords'
+  // bytes are the pixels: a byte rotation in front of the transposes), and the i-th store writes pixel
+  // (i + rot) % 8: eight banks apart times four channel groups - every bank, twice.
+  const int rot = lane & 7;
+  int pxm[8];  // halo pixel of the i-th store
 #pragma unroll
-  for (int j = 0; j < 4; ++j) ch_off[j] = has_patch ? static_cast<uint32_t>(c4 * 4 + j) * plane32 + static_cast<uint32_t>(col0) : 0u;
-  const int dst0 = (hr * a.iwt + a.pad_l + col0) * a.pix_stride + c4 * 4;
+  for (int i = 0; i < 8; ++i) pxm[i] = px0 + ((i + rot) & 7);
+  // v_perm selectors of the rotation: byte k of the low dword is byte (k + rot) % 8 of the row, the high dword follows
+  const uint32_t sel_lo = (static_cast<uint32_t>(rot & 7) | static_cast<uint32_t>((rot + 1) & 7) << 8 |
+                           static_cast<uint32_t>((rot + 2) & 7) << 16 | static_cast<uint32_t>((rot + 3) & 7) << 24);
+  const uint32_t sel_hi = sel_lo ^ 0x04040404u;
+  const uint32_t image_bytes = static_cast<uint32_t>(a.C) * plane32;
 
-  auto tile_geometry = [&](int tile_index, int* n, int* tl) {
+  // Is this thread's halo row inside the image for band `tile_index`? (lanes hold different rows)
+  auto row_of = [&](int tile_index, int* n, bool* inside) {
     const int img = FastDiv(tile_index, a.magic_tpi);
-    *n = img;
-    *tl = tile_index - img * a.tiles_per_image;
-  };
-  // Is this thread's halo row inside the image for band `tl`? (wavefront-varying: lanes hold different rows)
-  auto row_of = [&](int tl, bool* inside) {
-    const int r0 = tl * a.rows;
+    const int r0 = (tile_index - img * a.tiles_per_image) * a.rows;
     const int rows_here = min(a.rows, a.OH - r0);
     const int ih = r0 * a.sh - a.pad_t + hr;
+    *n = img;
     *inside = hr < (rows_here - 1) * a.sh + a.khe && ih >= 0 && ih < a.H;
     return *inside ? ih : 0;  // rows outside read row 0 and are replaced by the zero point behind the load
   };
+  // The loads are inline assembly and are waited for by hand (loads_landed): the compiler's own wait insertion
+  // would also wait for the output stores issued in between. To the compiler d[] is defined here and next used
+  // by loads_landed, so it keeps the registers untouched in between.
   auto issue_loads = [&](int2 (&d)[4], int tile_index) {
-    int n, tl;
-    tile_geometry(tile_index, &n, &tl);
+    int n;
     bool inside;
-    const uint32_t row_off = __umul24(static_cast<uint32_t>(row_of(tl, &inside)), static_cast<uint32_t>(a.W));
-    const uint8_t* img = a.x + static_cast<size_t>(n) * a.C * plane;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) d[j] = *reinterpret_cast<const int2*>(img + (ch_off[j] + row_off));
-  };
-  auto store_halo = [&](const int2 (&d)[4], int tile_index, int8_t* halo) {
-    int n, tl;
-    tile_geometry(tile_index, &n, &tl);
-    bool inside;
-    (void)row_of(tl, &inside);
-    const int keep = inside ? -1 : 0;
-    uint32_t lo4[4], hi4[4], px[8];
+    const uint32_t row_off = __umul24(static_cast<uint32_t>(row_of(tile_index, &n, &inside)), static_cast<uint32_t>(a.W));
+    const uint8_t* img = a.x + static_cast<size_t>(static_cast<uint32_t>(n)) * image_bytes;
+    uint32_t off = ch_off + row_off;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      lo4[j] = static_cast<uint32_t>(((d[j].x ^ a.xor_mask) & keep) | (a.pad_fill & ~keep));
-      hi4[j] = static_cast<uint32_t>(((d[j].y ^ a.xor_mask) & keep) | (a.pad_fill & ~keep));
+      asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(d[j]) : "v"(off), "s"(img) : "memory");
+      off += plane32;
+    }
+  };
+  auto loads_landed = [](int2 (&d)[4]) {
+    asm volatile("s_waitcnt vmcnt(0)" : "+v"(d[0]), "+v"(d[1]), "+v"(d[2]), "+v"(d[3])::"memory");
+  };
+  // masks, two 4 x 4 byte transposes, eight dword stores; the patch's share of its pixels' channel sums goes
+  // into the sum plane `splane` by LDS atomics
+  auto store_halo = [&](const int2 (&d)[4], int tile_index, int8_t* halo, int* splane) {
+    int n;
+    bool inside;
+    (void)row_of(tile_index, &n, &inside);
+    uint32_t lo4[4], hi4[4], px[8];
+    // a band whose halo rows all lie inside the image (wavefront-uniform: most bands) needs no masks
+    const int tl = tile_index - n * a.tiles_per_image;
+    const int ih0 = tl * a.rows * a.sh - a.pad_t;
+    const bool all_inside = ih0 >= 0 && ih0 + a.halo_rows <= a.H && (tl + 1) * a.rows <= a.OH;
+    if (all_inside) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t lo = static_cast<uint32_t>(d[j].x ^ a.xor_mask), hi = static_cast<uint32_t>(d[j].y ^ a.xor_mask);
+        lo4[j] = __builtin_amdgcn_perm(hi, lo, sel_lo);
+        hi4[j] = __builtin_amdgcn_perm(hi, lo, sel_hi);
+      }
+    } else {
+      const int keep = inside ? -1 : 0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t lo = static_cast<uint32_t>(((d[j].x ^ a.xor_mask) & keep) | (a.pad_fill & ~keep));
+        const uint32_t hi = static_cast<uint32_t>(((d[j].y ^ a.xor_mask) & keep) | (a.pad_fill & ~keep));
+        lo4[j] = __builtin_amdgcn_perm(hi, lo, sel_lo);
+        hi4[j] = __builtin_amdgcn_perm(hi, lo, sel_hi);
+      }
     }
     Transpose4x4(lo4, px);
     Transpose4x4(hi4, px + 4);
     if (has_patch) {
-      int8_t* dst = halo + dst0;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) *reinterpret_cast<uint32_t*>(dst + i * a.pix_stride) = px[i];
+      for (int i = 0; i < 8; ++i) *reinterpret_cast<uint32_t*>(halo + c4 * 4 + __mul24(pxm[i], a.pix_stride)) = px[i];
+      if (ZP) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          __hip_atomic_fetch_add(splane + pxm[i], __builtin_amdgcn_sdot4(static_cast<int>(px[i]), 0x01010101, 0, false),
+                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
     }
   };
+  // The sum plane of the band after next starts from zero, its padding columns from the padding pixel's sum.
+  const int s_cells = a.halo_rows * a.iwt;
+  const int s_col = tid - FastDiv(tid, a.magic_iwt) * a.iwt_div;
+  const int s_init = (s_col < a.pad_l || s_col >= a.pad_l + a.W) ? a.s_pad : 0;
+  auto clear_sums = [&](int* splane) {
+    if (ZP && tid < s_cells) splane[tid] = s_init;
+  };
+  auto sum_plane = [&](int k) { return reinterpret_cast<int*>(lds + a.off_s + k * a.s_bytes); };
   auto lds_barrier = [] { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
   // ---- prologue: the first band's rows on their way, weights and tables by DMA, the padding columns of both
-  // halo buffers (no band ever writes them again) ----
-  int2 d0[4];
-  issue_loads(d0, t);
+  // halo buffers (no band ever writes them again), the sum planes' start values ----
+  int2 dn[4];
+  issue_loads(dn, t);
   {
     typedef const __attribute__((address_space(1))) void* gptr;
     typedef __attribute__((address_space(3))) void* lptr;
@@ -157,52 +206,78 @@ ConvBandKernel(BandArgs a) {
       __builtin_amdgcn_global_load_lds((gptr)(a.biasf + lane), (lptr)(lds + a.off_bias), 4, 0, 0);
     }
   }
+  clear_sums(sum_plane(0));
+  clear_sums(sum_plane(1));
   {
-    const int right0 = a.pad_l + a.W;
+    // padding cells (halo row, padding column, 16-channel chunk) of both buffers, one per thread and step
     const int cpc = a.C >> 4;
-    const int units = a.halo_rows * a.pad_cols * cpc;
+    const int per_buf = a.halo_rows * a.pad_cols * cpc;
     const v4i fill = v4i{a.pad_fill, a.pad_fill, a.pad_fill, a.pad_fill};
-    for (int u = tid; u < 2 * units; u += kBandThreads) {
-      const int b = u >= units ? 1 : 0, v = u - b * units;
-      const int cell = v / cpc, c = (v - cell * cpc) * 16;
-      const int r = cell / a.pad_cols, pcol = cell - r * a.pad_cols;
-      const int col = pcol < a.pad_l ? pcol : right0 + (pcol - a.pad_l);
-      *reinterpret_cast<v4i*>(lds + (b ? a.off_halo1 : a.off_halo0) + (r * a.iwt + col) * a.pix_stride + c) = fill;
+    for (int u = tid; u < 2 * per_buf; u += kBandThreads) {
+      const int b = u >= per_buf ? 1 : 0, v = u - b * per_buf;
+      const int chunk = v & (cpc - 1), cell = v >> (cpc == 4 ? 2 : 1);  // cpc is 2 or 4
+      const int r = FastDiv(cell, a.magic_padcols);
+      const int pcol = cell - r * a.pad_cols;
+      const int col = pcol < a.pad_l ? pcol : a.W + pcol;
+      *reinterpret_cast<v4i*>(lds + (b ? a.off_halo1 : a.off_halo0) + (r * a.iwt + col) * a.pix_stride + chunk * 16) = fill;
     }
   }
-  store_halo(d0, t, lds + a.off_halo0);
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the DMA has landed
+  lds_barrier();  // the sum planes hold their start values
+  // s_waitcnt vmcnt(0) as an instruction the compiler sees: it then knows that the DMA has landed (behind a wait in
+  // inline assembly it would go on protecting every later LDS read with a wait for all memory operations)
+  __builtin_amdgcn_s_waitcnt(0x0f70);
+  loads_landed(dn);
+  store_halo(dn, t, lds + a.off_halo0, sum_plane(0));
+  if (t + per_xcd < t_end) issue_loads(dn, t + per_xcd);
   lds_barrier();
 
-  int buf = 0;
+  // ---- the bands: multiply the present band; feed (the next band's rows into the other halo buffer, the loads of
+  // the band after it); requantize and store the present band; one barrier ----
+  const int hw = a.OH * a.OW;
+  int buf = 0, sk = 0;  // halo buffer and sum plane of the present band
   for (; t < t_end; t += per_xcd) {
     const int tn = t + per_xcd;
     const bool has_next = tn < t_end;
-    int2 dn[4];
-    if (has_next) issue_loads(dn, tn);
-    int n, tl;
-    tile_geometry(t, &n, &tl);
-    const int r0 = tl * a.rows;
+    const int img = FastDiv(t, a.magic_tpi);
+    const int r0 = (t - img * a.tiles_per_image) * a.rows;
     const int valid = min(a.rows, a.OH - r0) * a.OW;  // pixels of this band
-    const int8_t* halo = lds + (buf ? a.off_halo1 : a.off_halo0);
+    const bool mine = wave < a.PT && wave * 32 < valid;
+    int* sx_lds = reinterpret_cast<int*>(lds + a.off_sx) + wave * 32;  // wavefront-private
 
-    if (wave < a.PT && wave * 32 < valid) {
+    v16i acc[2];
+    if (mine) {
+      const int8_t* halo = lds + (buf ? a.off_halo1 : a.off_halo0);
       const int pl = min(wave * 32 + frag_row, valid - 1);  // rows past the band's end recompute its last pixel
       const int ohl = FastDiv(pl, a.magic_ow), ow = pl - ohl * a.OW;
-      const int8_t* frag = halo + (ohl * a.sh * a.iwt + ow * a.sw) * a.pix_stride + frag_half * 16;
+      const int hp = ohl * a.sh * a.iwt + ow * a.sw;  // the window's first halo pixel
+      const int8_t* frag = halo + hp * a.pix_stride + frag_half * 16;
       const int8_t* w_row = lds + a.off_w + frag_row * a.kstride + frag_half * 16;
-      v16i acc[2];
+      const int* bias_lds = reinterpret_cast<const int*>(lds + a.off_bias);
+      // The zero-point term of the wavefront's 32 pixels: window sums of the sum plane, times the weights' zero
+      // point (requested here, used behind the multiplication).
+      int st[KH * KW];
+      if (ZP) {
+        const int* sp = sum_plane(sk) + hp;
+#pragma unroll
+        for (int ky = 0; ky < KH; ++ky)
+#pragma unroll
+          for (int kx = 0; kx < KW; ++kx) st[ky * KW + kx] = sp[ky * a.s_row_step + kx * a.s_col_step];
+        int sx = 0;
+#pragma unroll
+        for (int i = 0; i < KH * KW; ++i) sx += st[i];
+        if (frag_half == 0) sx_lds[frag_row] = a.zws * sx;
+      }
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const int bias = bias_lds[j * 32 + frag_row];
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[j][r] = bias;
       }
-      int sx = 0;
       constexpr int RING = 3;
       v4i fa[RING], fb[RING][2];
       auto fetch = [&](int ks, int slot_) {
-        fa[slot_] = *reinterpret_cast<const v4i*>(frag + a.tap_off[ks]);
+        const int tap = ks * 2 / CPC, cc = ks * 2 % CPC;
+        fa[slot_] = *reinterpret_cast<const v4i*>(frag + ((tap / KW) * a.row_step + (tap % KW) * a.col_step + cc * 16));
 #pragma unroll
         for (int j = 0; j < 2; ++j) fb[slot_][j] = *reinterpret_cast<const v4i*>(w_row + j * 32 * a.kstride + ks * 32);
       };
@@ -212,79 +287,97 @@ ConvBandKernel(BandArgs a) {
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ++ks) {
         if (ks + RING - 1 < KSTEPS) fetch(ks + RING - 1, (ks + RING - 1) % RING);
-        const v4i f = fa[ks % RING];
-        if (ZP) {
 #pragma unroll
-          for (int q = 0; q < 4; ++q) sx = __builtin_amdgcn_sdot4(f[q], 0x01010101, sx, false);
-        }
-#pragma unroll
-        for (int j = 0; j < 2; ++j) acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f, fb[ks % RING][j], acc[j], 0, 0, 0);
+        for (int j = 0; j < 2; ++j) acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[ks % RING], fb[ks % RING][j], acc[j], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
       }
-      if (ZP) {
-        sx += __shfl_xor(sx, 32);
-        __builtin_amdgcn_wave_barrier();
-        if (frag_half == 0) sx_lds[frag_row] = a.zws * sx;
-        __builtin_amdgcn_wave_barrier();
-      }
-      // ---- requantize one 32-channel tile at a time into the wavefront's staging tile, copy it out ----
+    }
+    // ---- the next band's rows (loaded one band ago) into the other halo buffer; the loads of the band after it
+    // leave now; the sum plane of that band gets its start values ----
+    if (has_next) {
+      loads_landed(dn);
+      store_halo(dn, tn, lds + (buf ? a.off_halo0 : a.off_halo1), sum_plane(sk == 2 ? 0 : sk + 1));
+      if (tn + per_xcd < t_end) issue_loads(dn, tn + per_xcd);
+      clear_sums(sum_plane(sk == 0 ? 2 : sk - 1));
+    }
+    // ---- accumulators -> codes. A lane holds four pixels of a channel per accumulator quad; two lane swaps
+    // between the wavefront's halves turn four quads into sixteen consecutive pixels.
+    if (mine) {
+      const v4i* rq_lds = reinterpret_cast<const v4i*>(lds + a.off_rq);
       const int nvalid = min(32, valid - wave * 32);  // a multiple of 8
-      uint8_t* ytile = a.y + static_cast<size_t>(n) * a.OC * hw + static_cast<size_t>(r0) * a.OW + wave * 32;
+      uint8_t* ytile = a.y + (static_cast<size_t>(img) * a.OC * hw + static_cast<size_t>(r0) * a.OW + wave * 32);
+      v4i s4[4];
+      if (ZP) {
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int g = 0; g < 4; ++g) s4[g] = *reinterpret_cast<const v4i*>(sx_lds + 8 * g + 4 * frag_half);
+      }
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const v4i rq = rq_lds[j * 32 + frag_row];
+        const int lo_t = a.lo << rq[1], hi_t = (a.hi << rq[1]) | ((1 << rq[1]) - 1);
+        uint32_t quad[4];
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          v4i s4 = v4i{0, 0, 0, 0};
-          if (ZP) s4 = *reinterpret_cast<const v4i*>(sx_lds + 8 * g + 4 * frag_half);
-          int r4[4];
+          int v[4];
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            r4[e] = Requant8<RQ>(ZP ? acc[j][g * 4 + e] - s4[e] : acc[j][g * 4 + e], rq, a.out_zp, a.lo, a.hi);
-          *reinterpret_cast<uint32_t*>(stage + frag_row * kStageStride + 8 * g + 4 * frag_half) = PackBytes(r4[0], r4[1], r4[2], r4[3]);
+          for (int e = 0; e < 4; ++e) v[e] = ZP ? acc[j][g * 4 + e] - s4[g][e] : acc[j][g * 4 + e];
+          if (RQ == kRqFastNoTie) {
+            // clamp in front of the shift (bounds shifted up), the shift writes its byte of the dword
+            int u[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) u[e] = Med3(__mulhi(v[e], rq[0]) + rq[2], lo_t, hi_t);
+            ShiftIntoByte<0>(quad[g], rq[1], u[0]);
+            ShiftIntoByte<1>(quad[g], rq[1], u[1]);
+            ShiftIntoByte<2>(quad[g], rq[1], u[2]);
+            ShiftIntoByte<3>(quad[g], rq[1], u[3]);
+          } else {
+            int r4[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r4[e] = Requant8<RQ>(v[e], rq, a.out_zp, a.lo, a.hi);
+            quad[g] = PackBytes(r4[0], r4[1], r4[2], r4[3]);
+          }
         }
-        __builtin_amdgcn_wave_barrier();
-        // lane -> (channel lane / 2, 16-byte half lane % 2) of the 32 x 32 tile
-        const int ocl = lane >> 1, h16 = (lane & 1) * 16;
-        const int2 v0 = *reinterpret_cast<const int2*>(stage + ocl * kStageStride + h16);
-        const int2 v1 = *reinterpret_cast<const int2*>(stage + ocl * kStageStride + h16 + 8);
-        const int oc = j * 32 + ocl;
+        // quad g of the lower half: pixels 8g .. 8g+3, of the upper half: 8g+4 .. 8g+7. Behind the swaps a lower lane
+        // holds pixels 0 .. 15 of its channel, its partner in the upper half pixels 16 .. 31.
+        // (the builtin, not inline assembly: the compiler must know that the swap is a cross-lane operation, or it
+        // may move it into a divergent region, where the idle lanes' halves stay behind)
+        const auto s02 = __builtin_amdgcn_permlane32_swap(quad[0], quad[2], false, false);
+        const auto s13 = __builtin_amdgcn_permlane32_swap(quad[1], quad[3], false, false);
+        quad[0] = s02[0]; quad[2] = s02[1]; quad[1] = s13[0]; quad[3] = s13[1];
+        const int oc = j * 32 + frag_row, h16 = frag_half * 16;
         uint8_t* dst = ytile + static_cast<size_t>(oc) * hw + h16;
         if (oc < a.OC) {
-          if (h16 + 16 <= nvalid) *reinterpret_cast<v4i*>(dst) = v4i{v0.x, v0.y, v1.x, v1.y};
-          else if (h16 + 8 <= nvalid) *reinterpret_cast<int2*>(dst) = v0;
+          if (h16 + 16 <= nvalid) *reinterpret_cast<v4i*>(dst) = v4i{static_cast<int>(quad[0]), static_cast<int>(quad[2]), static_cast<int>(quad[1]), static_cast<int>(quad[3])};
+          else if (h16 + 8 <= nvalid) *reinterpret_cast<int2*>(dst) = int2{static_cast<int>(quad[0]), static_cast<int>(quad[2])};
         }
-        __builtin_amdgcn_wave_barrier();  // the staging tile is read before the next channel tile overwrites it
       }
     }
-    if (has_next) {
-      store_halo(dn, tn, lds + (buf ? a.off_halo0 : a.off_halo1));
-      lds_barrier();  // the next band's halo tile is complete; everyone is done reading the present one
-    }
+    if (has_next) lds_barrier();  // the next band's halo tile and sums are complete; everyone is done reading the present ones
     buf ^= 1;
+    sk = sk == 2 ? 0 : sk + 1;
   }
 }
 
 struct BandPlan {
   BandArgs a;
   int lds_bytes;
-  int ksteps, rq;
+  int kh, kw, cpc, rq;
   bool zp;
   unsigned grid;
 };
 
 typedef void (*BandFn)(BandArgs);
-template <int KSTEPS>
+template <int KH, int KW, int CPC>
 BandFn BandKernelOf(int rq, bool zp) {
-  if (rq == kRqFastNoTie) return zp ? ConvBandKernel<KSTEPS, kRqFastNoTie, true> : ConvBandKernel<KSTEPS, kRqFastNoTie, false>;
-  return zp ? ConvBandKernel<KSTEPS, kRqFast, true> : ConvBandKernel<KSTEPS, kRqFast, false>;
+  if (rq == kRqFastNoTie) return zp ? ConvBandKernel<KH, KW, CPC, kRqFastNoTie, true> : ConvBandKernel<KH, KW, CPC, kRqFastNoTie, false>;
+  return zp ? ConvBandKernel<KH, KW, CPC, kRqFast, true> : ConvBandKernel<KH, KW, CPC, kRqFast, false>;
 }
-BandFn BandKernel(int ksteps, int rq, bool zp) {
-  if (rq == kRqGeneric) return nullptr;
-  switch (ksteps) {
-    case 9: return BandKernelOf<9>(rq, zp);
-    case 18: return BandKernelOf<18>(rq, zp);
-  }
+// The kernel exists for 3 x 3 taps over 32 or 64 input channels.
+BandFn BandKernel(int kh, int kw, int cpc, int rq, bool zp) {
+  if (rq == kRqGeneric || kh != 3 || kw != 3) return nullptr;
+  if (cpc == 2) return BandKernelOf<3, 3, 2>(rq, zp);
+  if (cpc == 4) return BandKernelOf<3, 3, 4>(rq, zp);
   return nullptr;
 }
 
@@ -295,7 +388,7 @@ int ConvBandRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t
   a.y = static_cast<uint8_t*>(out);
   if (reinterpret_cast<uintptr_t>(in0) & 3 || reinterpret_cast<uintptr_t>(out) & 7)
     return SetError(TVX_E_INVALID, "conv2d_band_i8: the input must be 4-byte aligned, the output 8-byte aligned");
-  hipLaunchKernelGGL(BandKernel(plan->ksteps, plan->rq, plan->zp), dim3(plan->grid), dim3(kBandThreads), plan->lds_bytes, st, a);
+  hipLaunchKernelGGL(BandKernel(plan->kh, plan->kw, plan->cpc, plan->rq, plan->zp), dim3(plan->grid), dim3(kBandThreads), plan->lds_bytes, st, a);
   TVX_HIP_CHECK(hipGetLastError());
   return TVX_OK;
 }
@@ -336,6 +429,10 @@ int ConvBandSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, cons
   const int w_bytes = RoundUp(64 * a.kstride, 1024);
   a.w_chunks = w_bytes / 16;
   a.gpr = a.W / 8;
+  a.row_step = dh * a.iwt * a.pix_stride; a.col_step = dw * a.pix_stride;
+  a.s_row_step = dh * a.iwt; a.s_col_step = dw;
+  a.iwt_div = a.iwt;
+  if (a.pad_cols < 0) return TVX_E_UNSUPPORTED;
 
   const bool x_u8 = d->in_dtype == TVX_U8, w_u8 = d->w_dtype == TVX_U8;
   const int zxs = d->in_zp - (x_u8 ? 128 : 0);
@@ -345,11 +442,12 @@ int ConvBandSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, cons
   a.pad_fill = static_cast<int>(static_cast<uint32_t>(zxs & 0xff) * 0x01010101u);
   a.zws = zws;
   a.out_zp = d->out_zp; a.lo = op->act_lo; a.hi = op->act_hi;
+  a.s_pad = a.C * zxs;
 
   std::vector<int32_t> rqt;
   const int rq = BuildRequantRecords(op->h_mult, op->h_shift, a.OC, 64, d->out_zp, &rqt,
                                      AccumulatorBound(static_cast<uint64_t>(taps) * a.C, bias_host, a.OC));
-  BandFn fn = BandKernel(ksteps, rq, zws != 0);
+  BandFn fn = BandKernel(kh, kw, cpc, rq, zws != 0);
   if (!fn) return TVX_E_UNSUPPORTED;
 
   hipDeviceProp_t prop;
@@ -358,7 +456,7 @@ int ConvBandSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, cons
   const int cus = std::max(8, prop.multiProcessorCount / 8 * 8);
 
   // ---- rows of a band: what the loader (one patch per thread), the wavefronts (one 32-pixel tile each) and LDS
-  // allow; among those the choice that needs the fewest rounds of bands, each priced by its rows plus a fixed part
+  // allow; among those the choice that needs the fewest rounds of bands, each priced by its halo rows
   int best_rows = 0, best_lds = 0;
   long long best_cost = 0;
   int want_rows = 0;
@@ -370,11 +468,13 @@ int ConvBandSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, cons
     if (gblocks * (a.C / 16) > kBandWaves) break;
     if ((r * a.OW + 31) / 32 > kBandWaves) break;
     const int halo_bytes = RoundUp(halo_rows * a.iwt * a.pix_stride + 64, 16);
-    const int lds_bytes = kBandWaves * 128 + 64 * 16 + 64 * 4 + w_bytes + kBandWaves * 32 * kStageStride + 2 * halo_bytes;
+    const int s_bytes = RoundUp(halo_rows * a.iwt * 4, 16);
+    if (halo_rows * a.iwt > kBandThreads) break;  // a thread per cell gives the sum planes their start values
+    const int lds_bytes = kBandWaves * 128 + 64 * 16 + 64 * 4 + w_bytes + 2 * halo_bytes + 3 * s_bytes;
     if (lds_bytes > 160 * 1024) break;
     const long long tiles = static_cast<long long>(d->batch) * ((a.OH + r - 1) / r);
-    const long long cost = (tiles + cus - 1) / cus * (r + 2);
-    if (best_rows == 0 || cost <= best_cost || r == want_rows) { best_rows = r; best_cost = cost; best_lds = lds_bytes; }
+    const long long cost = (tiles + cus - 1) / cus * (r + 2);  // (a band costs its rows plus the halo's two; equal cost: the shorter band)
+    if (best_rows == 0 || cost < best_cost || r == want_rows) { best_rows = r; best_cost = cost; best_lds = lds_bytes; }
     if (r == want_rows) break;
   }
   if (best_rows == 0) return TVX_E_UNSUPPORTED;
@@ -390,29 +490,31 @@ int ConvBandSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, cons
   // a handful of bands cannot fill the chip this way: the one-tile-per-workgroup kernel spreads them wider
   if (a.total_tiles < cus * 3 / 4 && !forced) return TVX_E_UNSUPPORTED;
   if (!MagicExact(a.tiles_per_image, total) || !MagicExact(a.OW, static_cast<uint64_t>(a.rows) * a.OW) ||
-      !MagicExact(a.gpr, 1024) || !MagicExact(a.gblocks, kBandWaves))
+      !MagicExact(a.gpr, 1024) || !MagicExact(a.gblocks, kBandWaves) || !MagicExact(a.iwt, kBandThreads) ||
+      !MagicExact(std::max(a.pad_cols, 1), 2 * kBandThreads))
     return TVX_E_UNSUPPORTED;
+  a.tiles_per_xcd = (a.total_tiles + 7) / 8;
+  a.magic_iwt = Magic(a.iwt);
+  a.magic_padcols = Magic(std::max(a.pad_cols, 1));
   a.magic_tpi = Magic(a.tiles_per_image);
   a.magic_ow = Magic(a.OW);
   a.magic_gpr = Magic(a.gpr);
   a.magic_gblocks = Magic(a.gblocks);
   // the loader's 24-bit multiplies and 32-bit offsets inside one image
   if (static_cast<uint64_t>(a.H) * a.W >= (1ull << 24) || static_cast<uint64_t>(a.H) * a.W * a.C >= (1ull << 31)) return TVX_E_UNSUPPORTED;
+  if (a.halo_rows * a.iwt * a.pix_stride >= (1 << 23)) return TVX_E_UNSUPPORTED;
 
   const int halo_bytes = RoundUp(a.halo_rows * a.iwt * a.pix_stride + 64, 16);
   a.off_sx = 0;
   a.off_rq = kBandWaves * 128;
   a.off_bias = a.off_rq + 64 * 16;
   a.off_w = a.off_bias + 64 * 4;
-  a.off_stage = a.off_w + w_bytes;
-  a.off_halo0 = a.off_stage + kBandWaves * 32 * kStageStride;
+  a.off_halo0 = a.off_w + w_bytes;
   a.off_halo1 = a.off_halo0 + halo_bytes;
-  const int lds_bytes = a.off_halo1 + halo_bytes;
+  a.off_s = a.off_halo1 + halo_bytes;
+  a.s_bytes = RoundUp(a.halo_rows * a.iwt * 4, 16);
+  const int lds_bytes = a.off_s + 3 * a.s_bytes;
   if (lds_bytes != best_lds) return SetError(TVX_E_INVALID, "conv2d_band_i8: LDS plan mismatch (%d, %d)", lds_bytes, best_lds);
-  for (int ks = 0; ks < ksteps; ++ks) {
-    const int q = 2 * ks, tp = q / cpc, cc = q % cpc;  // chunk 2 * ks; cpc is even, so chunk 2 * ks + 1 is the same tap's next chunk
-    a.tap_off[ks] = ((tp / kw) * dh * a.iwt + (tp % kw) * dw) * a.pix_stride + cc * 16;
-  }
 
   // ---- pack weights [oc][(ky, kx, c)] int8 with zero padding, fold constants into the bias ----
   std::vector<int8_t> packed(static_cast<size_t>(w_bytes) + 1024, 0);
@@ -445,7 +547,7 @@ int ConvBandSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, cons
   BandPlan plan;
   plan.a = a;
   plan.lds_bytes = lds_bytes;
-  plan.ksteps = ksteps;
+  plan.kh = kh; plan.kw = kw; plan.cpc = cpc;
   plan.rq = rq;
   plan.zp = zws != 0;
   int wgs = cus;
