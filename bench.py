@@ -28,6 +28,31 @@ PEAK_HBM_GBS = 8000.0     # HBM3E, 8 TB/s
 SEED = 0x71
 
 
+def _same(a, b, float_tol=None):
+    if float_tol is None:
+        return bool(np.array_equal(a, b))
+    return bool(np.allclose(a.astype(np.float32), b.astype(np.float32), rtol=float_tol, atol=float_tol))
+
+
+def conv_check(x, wt, b, kws, batch, float_tol=None):
+    """The GPU result of the batch's first image against the CPU restatement of the same operator."""
+    def check(gpu_out):
+        import tvx_oracle as O
+        k1 = dict(kws, in_shape=kws["in_shape"][:3] + [1], out_shape=kws["out_shape"][:3] + [1])
+        ref = O.conv2d(np.ascontiguousarray(x[:x.size // batch]), wt, b, **k1)
+        return _same(ref, gpu_out[:ref.size], float_tol)
+    return check
+
+
+def fc_check(x, wt, b, kws, rows=32, float_tol=None):
+    """The first `rows` rows of the GPU result against the CPU restatement."""
+    def check(gpu_out):
+        import tvx_oracle as O
+        ref = O.fully_connected(np.ascontiguousarray(x[:rows * kws["k"]]), wt, b, **dict(kws, m=rows))
+        return _same(ref, gpu_out[:ref.size], float_tol)
+    return check
+
+
 def conv_cfg2(T, rng, batch=32):
     n, c, h, w, oc = batch, 64, 56, 56, 64
     x = rng.integers(0, 256, n * c * h * w, dtype=np.uint8)
@@ -51,7 +76,7 @@ def conv_cfg2(T, rng, batch=32):
                       out_q=(0.1, 0), act=2)
     return dict(name="conv2d_u8_3x3_64to64_56x56_b%d_same_relu6" % n, op=op, inputs=(x,), out_elems=n * oc * h * w,
                 out_dtype=np.uint8, ops=2 * macs, algo_bytes=algo_bytes, bound="mfma",
-                oracle=("conv2d", (x, wt, b), oracle_kws, n))
+                oracle=("conv2d", (x, wt, b), oracle_kws, n), check=conv_check(x, wt, b, oracle_kws, n))
 
 
 def conv_cfg2_b256(T, rng):
@@ -75,9 +100,11 @@ def conv_f16(T, rng):
     d.in_dtype = d.w_dtype = d.out_dtype = T.F16
     d.activation = T.ACT_RELU6
     op = T.conv2d_create(d, wt, b)
+    kws = dict(in_shape=[w, h, c, n], w_shape=[3, 3, c, oc], out_shape=[w, h, oc, n], stride=[1, 1], dilation=[1, 1],
+               pad_left=1, pad_top=1, multiplier=0, in_dtype=2, w_dtype=2, out_dtype=2, act=2)
     return dict(name="conv2d_f16_3x3_64to64_56x56_b32_same_relu6", op=op, inputs=(x,), out_elems=n * oc * h * w,
                 out_dtype=np.float16, ops=2 * n * h * w * oc * c * 9, algo_bytes=2 * (x.size + n * oc * h * w + wt.size) + 4 * oc,
-                bound="mfma", peak=PEAK_F16_TFLOPS, oracle=None)
+                bound="mfma", peak=PEAK_F16_TFLOPS, oracle=None, check=conv_check(x, wt, b, kws, n, float_tol=1e-2))
 
 
 def conv_grouped(T, rng):
@@ -99,7 +126,11 @@ def conv_grouped(T, rng):
     op = T.conv2d_create(d, wt, b)
     return dict(name="grouped_conv2d_u8_3x3_4x32to32_28x28_b32_same_relu6", op=op, inputs=(x,),
                 out_elems=n * oc * h * w, out_dtype=np.uint8, ops=2 * n * h * w * oc * (c // groups) * 9,
-                algo_bytes=x.size + n * oc * h * w + wt.size + 4 * oc, bound="mfma", oracle=None)
+                algo_bytes=x.size + n * oc * h * w + wt.size + 4 * oc, bound="mfma", oracle=None,
+                check=conv_check(x, wt, b, dict(in_shape=[w, h, c, n], w_shape=[3, 3, c // groups, oc], out_shape=[w, h, oc, n],
+                                                stride=[1, 1], dilation=[1, 1], pad_left=1, pad_top=1, multiplier=0, groups=groups,
+                                                in_dtype=0, w_dtype=0, out_dtype=0, in_q=(0.05, 128), w_q=(0.01, 120, None),
+                                                out_q=(0.1, 0), act=2), n))
 
 
 def fc_cfg5(T, rng):
@@ -118,7 +149,9 @@ def fc_cfg5(T, rng):
     op = T.fully_connected_create(d, wt, b)
     return dict(name="fc_i8_per_channel_m8192_k4096_n4096", op=op, inputs=(x,), out_elems=m * n,
                 out_dtype=np.int8, ops=2 * m * k * n, algo_bytes=m * k + n * k + m * n + 4 * n,
-                bound="mfma", oracle=None)
+                bound="mfma", oracle=None,
+                check=fc_check(x, wt, b, dict(k=k, n=n, in_dtype=1, w_dtype=1, out_dtype=1, in_q=(0.02, 0), w_q=(1.0, 0, ws),
+                                              out_q=(0.05, 0))))
 
 
 def fc_cfg5_u8(T, rng):
@@ -137,7 +170,9 @@ def fc_cfg5_u8(T, rng):
     op = T.fully_connected_create(d, wt, b)
     return dict(name="fc_u8_asymmetric_m8192_k4096_n4096", op=op, inputs=(x,), out_elems=m * n,
                 out_dtype=np.uint8, ops=2 * m * k * n, algo_bytes=m * k + n * k + m * n + 4 * n,
-                bound="mfma", oracle=None)
+                bound="mfma", oracle=None,
+                check=fc_check(x, wt, b, dict(k=k, n=n, in_dtype=0, w_dtype=0, out_dtype=0, in_q=(0.02, 121), w_q=(0.01, 131, None),
+                                              out_q=(1.2, 128))))
 
 
 def fc_cfg5_f16(T, rng):
@@ -151,7 +186,8 @@ def fc_cfg5_f16(T, rng):
     op = T.fully_connected_create(d, wt, b)
     return dict(name="fc_f16_m8192_k4096_n4096", op=op, inputs=(x,), out_elems=m * n,
                 out_dtype=np.float16, ops=2 * m * k * n, algo_bytes=2 * (m * k + n * k + m * n) + 4 * n,
-                bound="mfma", peak=PEAK_F16_TFLOPS, oracle=None)
+                bound="mfma", peak=PEAK_F16_TFLOPS, oracle=None,
+                check=fc_check(x, wt, b, dict(k=k, n=n, in_dtype=2, w_dtype=2, out_dtype=2), float_tol=1e-2))
 
 
 def dw_cfg3a(T, rng):
@@ -175,7 +211,10 @@ def dw_cfg3a(T, rng):
     op = T.conv2d_create(d, wt, b)
     return dict(name="depthwise3x3_i8_per_channel_112x112x32_b32", op=op, inputs=(x,), out_elems=x.size,
                 out_dtype=np.int8, ops=2 * x.size * 9, algo_bytes=2 * x.size + wt.size + 4 * c,
-                bound="hbm", oracle=None)
+                bound="hbm", oracle=None,
+                check=conv_check(x, wt, b, dict(in_shape=[w, h, c, n], w_shape=[3, 3, 1, c], out_shape=[w, h, c, n], stride=[1, 1],
+                                                dilation=[1, 1], pad_left=1, pad_top=1, multiplier=1, in_dtype=1, w_dtype=1,
+                                                out_dtype=1, in_q=(0.03, 0), w_q=(1.0, 0, ws), out_q=(0.08, 0)), n))
 
 
 def pw_cfg3b(T, rng):
@@ -197,7 +236,10 @@ def pw_cfg3b(T, rng):
     op = T.conv2d_create(d, wt, b)
     return dict(name="pointwise1x1_i8_per_channel_32to64_112x112_b32_relu6", op=op, inputs=(x,),
                 out_elems=n * oc * h * w, out_dtype=np.int8, ops=2 * n * h * w * c * oc,
-                algo_bytes=x.size + n * oc * h * w + wt.size + 4 * oc, bound="hbm", oracle=None)
+                algo_bytes=x.size + n * oc * h * w + wt.size + 4 * oc, bound="hbm", oracle=None,
+                check=conv_check(x, wt, b, dict(in_shape=[w, h, c, n], w_shape=[1, 1, c, oc], out_shape=[w, h, oc, n], stride=[1, 1],
+                                                dilation=[1, 1], pad_left=0, pad_top=0, multiplier=0, in_dtype=1, w_dtype=1,
+                                                out_dtype=1, in_q=(0.08, 0), w_q=(1.0, 0, ws), out_q=(0.05, 0), act=2), n))
 
 
 def pool_workload(T, rng, name, in_shape, k, stride, pool_type, dtype=0):
@@ -212,8 +254,14 @@ def pool_workload(T, rng, name, in_shape, k, stride, pool_type, dtype=0):
     d.pool_type, d.dtype = pool_type, dtype
     d.in_scale, d.in_zp, d.out_scale, d.out_zp = 0.05, 3, 0.05, 3
     op = T.pool2d_create(d)
+
+    def check(gpu_out):
+        import tvx_oracle as O
+        ref = O.pool2d(np.ascontiguousarray(x[:w * h * c]), in_shape=[w, h, c, 1], out_shape=[ow, oh, c, 1], ksize=[k, k],
+                       stride=[stride, stride], pad_left=0, pad_top=0, pool_type=pool_type, dtype=dtype, in_q=(0.05, 3), out_q=(0.05, 3))
+        return _same(ref, gpu_out[:ref.size])
     return dict(name=name, op=op, inputs=(x,), out_elems=ow * oh * c * n, out_dtype=np.uint8,
-                ops=w * h * c * n, algo_bytes=x.size + ow * oh * c * n, bound="hbm", oracle=None)
+                ops=w * h * c * n, algo_bytes=x.size + ow * oh * c * n, bound="hbm", oracle=None, check=check)
 
 
 def pool_lenet_b256(T, rng):
@@ -261,7 +309,16 @@ def dwpw_cfg3(T, rng):
     p.w_scales = sp.ctypes.data_as(C.POINTER(C.c_float))
     p.out_scale, p.out_zp, p.activation = 0.05, 0, T.ACT_RELU6
     op = T.conv2d_dw_pw_create(d, wd, bd, p, wp, bp)
-    return dict(name="depthwise3x3_then_pointwise1x1_i8_per_channel_112x112x32to64_b32_relu6", op=op, inputs=(x,),
+
+    def check(gpu_out):
+        import tvx_oracle as O
+        common = dict(stride=[1, 1], dilation=[1, 1], in_dtype=1, w_dtype=1, out_dtype=1)
+        mid = O.conv2d(np.ascontiguousarray(x[:c * h * w]), wd, bd, in_shape=[w, h, c, 1], w_shape=[3, 3, 1, c], out_shape=[w, h, c, 1],
+                       pad_left=1, pad_top=1, multiplier=1, in_q=(0.03, 0), w_q=(1.0, 0, sd), out_q=(0.08, 0), **common)
+        ref = O.conv2d(mid, wp, bp, in_shape=[w, h, c, 1], w_shape=[1, 1, c, oc], out_shape=[w, h, oc, 1], pad_left=0, pad_top=0,
+                       multiplier=0, in_q=(0.08, 0), w_q=(1.0, 0, sp), out_q=(0.05, 0), act=2, **common)
+        return _same(ref, gpu_out[:ref.size])
+    return dict(check=check, name="depthwise3x3_then_pointwise1x1_i8_per_channel_112x112x32to64_b32_relu6", op=op, inputs=(x,),
                 out_elems=n * oc * h * w, out_dtype=np.int8, ops=2 * n * h * w * c * (9 + oc),
                 algo_bytes=x.size + n * oc * h * w + wd.size + wp.size + 4 * (c + oc), bound="hbm", oracle=None)
 
@@ -491,7 +548,9 @@ def main():
             w2 = make(T, rng)
             steps2 = max(5, min(args.steps, 50))
             wall2, k2 = time_workload(w2, steps2, min(args.warmup, 5))
-            rec = dict(kernel=w2["op"].kernel_name, ms_per_step=round(wall2, 5),
+            # the first image (or rows) of the result against the CPU restatement, before any figure is reported
+            checked = w2["check"](w2["device_out"].cpu().numpy()) if w2.get("check") else None
+            rec = dict(kernel=w2["op"].kernel_name, parity_vs_oracle_on_sample=checked, ms_per_step=round(wall2, 5),
                        tops=round(w2["ops"] / (wall2 * 1e-3) / 1e12, 2),
                        gbs=round(w2["algo_bytes"] / (wall2 * 1e-3) / 1e9, 1),
                        roofline=dict(roofline(w2, k2, traffic_of(w2)), kernel_ms=round(k2, 5)))

@@ -410,6 +410,11 @@ typedef struct {
  * counts as real zeros, avg_pool_test.cc:428-455); AVG_ANDROID by the number
  * of in-bounds taps (avg_pool_test.cc:490-514). Quantized: operate on
  * (x - z_in), scale by s_in/s_out, round half to even, add z_out, saturate.
+ * L2 (src/tim/vx/type_utils.cc:99-100 -> VX_NN_POOLING_L2): the root of the
+ * mean of the squares, the mean taken over k_w*k_h like AVG's (padding counts
+ * as zeros); no reference test holds an L2 vector: the divisor is this
+ * restatement's choice (parity unpinned), the arithmetic is pinned by closed
+ * forms. Quantized: ratio * sqrt(sum (x - z_in)^2 / div) in double.
  */
 void tvxo_pool2d(const tvxo_pool_desc* d, const void* x, void* y) {
   const int quant = d->dtype == TVXO_U8 || d->dtype == TVXO_I8;
@@ -424,8 +429,8 @@ void tvxo_pool2d(const tvxo_pool_desc* d, const void* x, void* y) {
     for (int32_t oh = 0; oh < d->out_h; ++oh) {
       for (int32_t ow = 0; ow < d->out_w; ++ow) {
         int32_t cnt = 0, imax = INT32_MIN;
-        int64_t isum = 0;
-        float fmax = -INFINITY, fsum = 0.f;
+        int64_t isum = 0, isq = 0;
+        float fmax = -INFINITY, fsum = 0.f, fsq = 0.f;
         for (int32_t ky = 0; ky < d->k_h; ++ky) {
           const int32_t ih = oh * d->stride_h - d->pad_top + ky;
           if (ih < 0 || ih >= d->in_h) continue;
@@ -437,26 +442,31 @@ void tvxo_pool2d(const tvxo_pool_desc* d, const void* x, void* y) {
             if (quant) {
               int32_t v = load_q(x, d->dtype, xi) - d->in_zp;
               isum += v;
+              isq += (int64_t)v * v;
               if (v > imax) imax = v;
             } else {
               float v = load_f(x, d->dtype, xi);
               fsum += v;
+              fsq += v * v;
               if (v > fmax) fmax = v;
             }
           }
         }
         const int64_t yi = yb + (int64_t)oh * d->out_w + ow;
-        const int32_t div = d->pool_type == TVXO_POOL_AVG ? d->k_w * d->k_h : cnt;
+        const int32_t div = d->pool_type == TVXO_POOL_AVG || d->pool_type == TVXO_POOL_L2 ? d->k_w * d->k_h : cnt;
         if (quant) {
           int64_t r;
           if (d->pool_type == TVXO_POOL_MAX) {
             r = cnt ? tvxo_requant(imax, mult, shift) : 0;
+          } else if (d->pool_type == TVXO_POOL_L2) {
+            r = (int64_t)nearbyint(ratio * sqrt((double)isq / (double)div));
           } else {
             r = div ? (int64_t)nearbyint((double)isum * ratio / (double)div) : 0;
           }
           store_q(y, d->dtype, yi, clamp64(r + d->out_zp, qmin, qmax));
         } else {
           float r = d->pool_type == TVXO_POOL_MAX ? (cnt ? fmax : 0.f) : (div ? fsum / (float)div : 0.f);
+          if (d->pool_type == TVXO_POOL_L2) r = sqrtf(fsq / (float)div);
           store_f(y, d->dtype, yi, r);
         }
       }

@@ -173,6 +173,32 @@ def test_lenet_sample_graph(tmp_path, oracle):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("lock", [True, False], ids=["one_mutex", "concurrent"])
+def test_two_threads_build_compile_and_run_lenet(tmp_path, oracle, lock):
+    """Two threads, each with a context of its own, build, compile and run LeNet (batch 1 and batch 16): one after
+    the other under one mutex, as the reference's multi-thread sample does
+    (samples/multi_thread_test/multi_thread_test.cc:100,330-372), and without the mutex. Every thread's bytes must
+    be the single-threaded ones, bit for bit the oracle's."""
+    w, x = _lenet_data()
+    g = GRAPHS.lenet_asymu8(w, x)
+    logits = copy.deepcopy(g)  # cut before the softmax: the uint8 logits
+    logits["test"] = "lenet_logits"
+    logits["ops"] = logits["ops"][:-1]
+    logits["tensors"] = logits["tensors"][:-1]
+    logits["tensors"][15]["attr"] = "OUTPUT"
+    logits["output"] = 15
+    batched = GRAPHS.lenet_random(batch=16)
+    graphs = [g, logits, batched]
+    single, info, log = GF.run_graphs(graphs, str(tmp_path / "single"))
+    threaded, info_t, log_t = GF.run_graphs(graphs, str(tmp_path / "threads"), threads=2, lock=lock)
+    assert all(r is not None for r in single) and all(r is not None for r in threaded), (info, info_t, log_t[-2000:])
+    for a, b in zip(single, threaded):
+        assert np.array_equal(a, b)
+    assert np.array_equal(threaded[1], oracle.run_graph(logits))
+    assert int(np.argmax(threaded[0])) == 0
+
+
+@pytest.mark.gpu
 def test_transpose_feeds_a_convolution(tmp_path, oracle):
     """A channel-fastest {C, W, H, N} image brought to WHCN by Transpose{1, 2, 0, 3} (the permute
     layout inference puts in front of an NHWC model, src/tim/transform/layout_inference.cc), then a

@@ -125,7 +125,7 @@ POOLS = [
 
 
 @pytest.mark.parametrize("dtype", [0, 1, 2, 3])
-@pytest.mark.parametrize("ptype", [0, 1, 3])
+@pytest.mark.parametrize("ptype", [0, 1, 2, 3])   # MAX, AVG, L2, AVG_ANDROID
 @pytest.mark.parametrize("pi", range(len(POOLS)))
 def test_pool2d_random(oracle, pi, ptype, dtype):
     p = POOLS[pi]
@@ -182,6 +182,22 @@ def test_pool2d_rows(oracle, pi, ptype, dtype):
         got = TC.gpu_pool2d(x, in_q=in_q, out_q=out_q, want_kernel="pool2d_rows_i8", **kws)
         assert np.array_equal(got, want), (int((got != want).sum()), np.flatnonzero(got != want)[:8])
     assert len(np.unique(want)) > 4
+
+
+@pytest.mark.parametrize("band_kb", ["8", "33", "60"])
+def test_pool2d_rows_band_budgets(oracle, band_kb, monkeypatch):
+    """LDS budgets below and above what two images of the pipelined form may take (64 KiB together): where the
+    pipelined plan falls through, the plain plan's grid and LDS size must be the ones launched - every plane of
+    1024 plane groups written."""
+    monkeypatch.setenv("TVX_POOL_BAND_KB", band_kb)
+    rng = np.random.default_rng(650)
+    w, h, c, n = 24, 24, 64, 40   # 2560 planes: enough plane groups for the pipelined form at every budget
+    x = rng.integers(0, 256, w * h * c * n, dtype=np.uint8)
+    kws = dict(in_shape=[w, h, c, n], out_shape=[12, 12, c, n], ksize=[2, 2], stride=[2, 2], pad_left=0, pad_top=0,
+               pool_type=0, dtype=0, in_q=(0.1, 120), out_q=(0.1, 120))
+    want = oracle.pool2d(x, **kws)
+    got = TC.gpu_pool2d(x, want_kernel="pool2d_rows_i8", **kws)
+    assert np.array_equal(got, want), int((got != want).sum())
 
 
 def test_pool2d_full_size_max_3x3_stride2(oracle):

@@ -291,6 +291,68 @@ def test_pool_avg_divisors(oracle):
     assert np.allclose(android, [(1 + 2 + 4 + 5) / 4, (3 + 6) / 2, (7 + 8) / 2, 9])
 
 
+def test_pool_l2_closed_forms(oracle):
+    """L2 pooling = root of the mean of the squares over the window area. Pinned by cases with known answers: a
+    3-4 pair (sqrt(12.5)), a constant plane (its absolute value), a one-tap window (|x|), homogeneity (scaling the
+    input scales the result), padding that counts as zeros, and numpy on random planes."""
+    f32 = oracle.F32
+    l2 = oracle.POOL["L2"]
+    got = oracle.pool2d(np.array([3, 4], np.float32), in_shape=[2, 1, 1, 1], out_shape=[1, 1, 1, 1], ksize=[2, 1],
+                        stride=[1, 1], pad_left=0, pad_top=0, pool_type=l2, dtype=f32)
+    assert np.allclose(got, [np.sqrt(12.5)], rtol=1e-6)
+    x = np.full(5 * 4, -2.5, np.float32)
+    got = oracle.pool2d(x, in_shape=[5, 4, 1, 1], out_shape=[3, 2, 1, 1], ksize=[3, 3], stride=[1, 1], pad_left=0,
+                        pad_top=0, pool_type=l2, dtype=f32)
+    assert np.allclose(got, 2.5, rtol=1e-6)
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal(6 * 7 * 2).astype(np.float32)
+    one = oracle.pool2d(x, in_shape=[6, 7, 2, 1], out_shape=[6, 7, 2, 1], ksize=[1, 1], stride=[1, 1], pad_left=0,
+                        pad_top=0, pool_type=l2, dtype=f32)
+    assert np.allclose(one, np.abs(x), rtol=1e-6)
+    kw = dict(in_shape=[6, 7, 2, 1], out_shape=[3, 4, 2, 1], ksize=[3, 3], stride=[2, 2], pad_left=1, pad_top=1,
+              pool_type=l2, dtype=f32)
+    base = oracle.pool2d(x, **kw)
+    assert np.allclose(oracle.pool2d(-3 * x, **kw), 3 * base, rtol=1e-5)
+    # numpy: zero-padded plane, mean of squares over all nine taps
+    xp = np.pad(x.reshape(2, 7, 6).astype(np.float64), ((0, 0), (1, 1), (1, 1)))
+    want = np.array([[[np.sqrt(np.mean(xp[c, 2 * oh:2 * oh + 3, 2 * ow:2 * ow + 3] ** 2)) for ow in range(3)]
+                      for oh in range(4)] for c in range(2)])
+    assert np.allclose(base.reshape(2, 4, 3), want, rtol=1e-5)
+    # the corner window holds four real taps of nine: smaller than the mean over the taps alone
+    corner = x.reshape(2, 7, 6)[0, :2, :2].astype(np.float64)
+    assert np.isclose(base[0], np.sqrt((corner ** 2).sum() / 9), rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype_name", ["U8", "I8"])
+@pytest.mark.parametrize("s_in,s_out", [(0.05, 0.05), (0.05, 0.023), (0.5, 0.25), (1.0, 1.0)])
+def test_quantized_pool_l2_is_exact(oracle, dtype_name, s_in, s_out):
+    """Quantized L2 pooling against exact rational arithmetic: the code q with (q - 1/2)^2 <= V < (q + 1/2)^2 for
+    V = (s_in / s_out)^2 * sum (x - z_in)^2 / area - no square root is taken on this side."""
+    rng = np.random.default_rng(60 + (dtype_name == "U8"))
+    u8 = dtype_name == "U8"
+    qmin, qmax = (0, 255) if u8 else (-128, 127)
+    z_in, z_out = (101, 7) if u8 else (-9, -100)
+    W, H, C, N = 7, 6, 3, 2
+    k, stride, pad = [3, 3], [2, 2], [1, 1]
+    ow, oh = (W + 2 * pad[0] - k[0]) // stride[0] + 1, (H + 2 * pad[1] - k[1]) // stride[1] + 1
+    x = rng.integers(qmin, qmax + 1, (N * C, H, W)).astype(np.uint8 if u8 else np.int8)
+    got = oracle.pool2d(x.ravel(), in_shape=[W, H, C, N], out_shape=[ow, oh, C, N], ksize=k, stride=stride,
+                        pad_left=pad[0], pad_top=pad[1], pool_type=oracle.POOL["L2"],
+                        dtype=oracle.U8 if u8 else oracle.I8, in_q=(s_in, z_in), out_q=(s_out, z_out))
+    ratio = _f32(s_in) / _f32(s_out)
+    want = []
+    for p in range(N * C):
+        for taps in _pool_windows(x[p], k, stride, pad, (ow, oh)):
+            v4 = 4 * ratio * ratio * sum((t - z_in) ** 2 for t in taps) / (k[0] * k[1])   # (2 sqrt(V))^2
+            q = 0
+            while (2 * q + 1) ** 2 <= v4:   # smallest q with (2q + 1)^2 > 4V, i.e. sqrt(V) < q + 1/2
+                q += 1
+            assert (2 * q + 1) ** 2 != v4 and (q == 0 or (2 * q - 1) ** 2 != v4)   # (no exact tie in this data)
+            want.append(min(qmax, max(qmin, q + z_out)))
+    assert got.astype(np.int64).tolist() == want
+    assert len(set(want)) > 8
+
+
 def _pool_windows(xr, k, stride, pad, out_wh):
     """In-bounds taps of every window of one plane xr[H][W] (plain Python)."""
     H, W = xr.shape

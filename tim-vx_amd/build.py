@@ -68,7 +68,7 @@ def build_runtime(verbose=False):
          ["-L", os.path.join(PKG_DIR, "lib"), "-ltvx_hip", "-Wl,-rpath,$ORIGIN",
           "-o", os.path.join(PKG_DIR, "lib", "libtim-vx.so")], verbose)
     # the graph-file runner: an application of the public API, linked like any other
-    _run(["g++", "-std=c++17", "-O2", "-Wall", "-I", os.path.join(PKG_DIR, "include"),
+    _run(["g++", "-std=c++17", "-O2", "-Wall", "-pthread", "-I", os.path.join(PKG_DIR, "include"),
           os.path.join(PKG_DIR, "src", "tools", "graph_runner.cc"),
           "-L", os.path.join(PKG_DIR, "lib"), "-ltim-vx", "-ltvx_hip", "-Wl,-rpath,$ORIGIN",
           "-o", os.path.join(PKG_DIR, "lib", "tvx_graph_runner")], verbose)

@@ -67,19 +67,7 @@ struct ConvArgs {
   uint32_t blk_col, blk_chan;  // ... per wavefront w (byte w): w % w4_blocks and w / w4_blocks
   int off_out;           // epilogue staging tile
   int tap_off[40];       // halo byte offset of k-step ks (both fragment halves lie in one tap: + 16 * half)
-#ifdef TVX_CONV_TIMESTAMPS
-  unsigned long long* ts;  // profiling build only: [workgroup][wavefront][64] wall-clock samples
-#endif
 };
-
-#ifdef TVX_CONV_TIMESTAMPS
-#define TVX_TS(slot)                                                                                         \
-  do {                                                                                                       \
-    if (a.ts && lane == 0 && (slot) < 64) a.ts[(static_cast<size_t>(blockIdx.x) * 4 + wave) * 64 + (slot)] = wall_clock64(); \
-  } while (0)
-#else
-#define TVX_TS(slot) do { } while (0)
-#endif
 
 __device__ __forceinline__ int FastDiv(int u, uint32_t magic) {
   return magic ? static_cast<int>(__umulhi(static_cast<uint32_t>(u), magic)) : u;
@@ -427,7 +415,6 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(O
   }
 }
 
-
 // ---- persistent variant ----------------------------------------------------------------
 // The same implicit GEMM for layers whose whole weight block fits the register file: every
 // wavefront keeps all KSTEPS x OT weight fragments of the operator in VGPRs for its whole life
@@ -573,7 +560,6 @@ ConvPersistKernel(ConvArgs a) {
   // the global stores of the tile just copied out.
   auto lds_barrier = [] { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
-  TVX_TS(0);
   // ---- prologue: the first tile's rows on their way, the weights by DMA into the (still empty) staging tile and second
   // halo buffer, which lie side by side; from there into every wavefront's registers - 288 KB per CU through LDS,
   // a microsecond of LDS bandwidth with the vector units idle - while the rows are transposed into the first halo
@@ -609,11 +595,8 @@ ConvPersistKernel(ConvArgs a) {
   }
   store_pad_columns(t, lds + a.off_halo);
   lds_barrier();  // the first halo tile is complete, every wavefront has its weights: staging tile and second buffer are free
-  TVX_TS(1);
 
   int buf = 0;
-  int ts_it = 0;
-  (void)ts_it;
   for (; t < t_end; t += per_xcd) {
     const int tn = t + per_xcd;
     const bool has_next = tn < t_end;
@@ -621,7 +604,6 @@ ConvPersistKernel(ConvArgs a) {
     int n, p0, p_end, r0, ih0, rows_needed;
     tile_geometry(t, &n, &p0, &p_end, &r0, &ih0, &rows_needed);
     const int8_t* halo = lds + (buf ? a.off_halo1 : a.off_halo);
-    TVX_TS(2 + ts_it * 8);
 
     // ---- one 32-pixel MFMA tile at a time: reduction, then requantization into the staging tile ----
 #pragma unroll
@@ -660,7 +642,6 @@ ConvPersistKernel(ConvArgs a) {
           // just requested in front of the MFMAs on the older ones, and every k-step waits out a whole LDS round trip
           __builtin_amdgcn_sched_barrier(0);
         }
-        if (i == 0) TVX_TS(3 + ts_it * 8);
         if (ZP) {
           sx += __shfl_xor(sx, 32);
           __builtin_amdgcn_wave_barrier();
@@ -692,7 +673,6 @@ ConvPersistKernel(ConvArgs a) {
         }
         if (ZP) __builtin_amdgcn_wave_barrier();  // the sums are read before the next MFMA tile's are written
       }
-      TVX_TS(4 + i + ts_it * 8);
     }
     // ---- the next tile's rows: L2 -> registers -> the other halo buffer ----
     if (has_next) {
@@ -706,9 +686,7 @@ ConvPersistKernel(ConvArgs a) {
       }
       store_pad_columns(tn, halo_next);
     }
-    TVX_TS(6 + ts_it * 8);
     lds_barrier();  // staging tile complete, next halo complete
-    TVX_TS(7 + ts_it * 8);
     // ---- copy out: contiguous runs of the WHCN output ----
     {
       const int valid = p_end - p0;
@@ -732,10 +710,7 @@ ConvPersistKernel(ConvArgs a) {
                 *reinterpret_cast<const uint32_t*>(out_tile + o * a.out_stride + dwi * 4);
       }
     }
-    TVX_TS(8 + ts_it * 8);
     lds_barrier();  // everyone has read the staging tile before the next tile's results go in
-    TVX_TS(9 + ts_it * 8);
-    ++ts_it;
     buf ^= 1;
   }
   asm volatile("" ::"v"(landing));
@@ -779,20 +754,11 @@ void LaunchRq(const Plan* plan, const ConvArgs& a, hipStream_t st) {
     hipLaunchKernelGGL((ConvIgemmKernel<OT, kRqGeneric>), plan->grid, block, plan->lds_bytes, st, a);
 }
 
-#ifdef TVX_CONV_TIMESTAMPS
-unsigned long long* g_ts = nullptr;
-constexpr size_t kTsBytes = 1024 * 4 * 64 * 8;
-#endif
-
 int ConvIgemmRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
   const Plan* plan = reinterpret_cast<const Plan*>(op->host_blob.data());
   ConvArgs a = plan->a;
   a.x = static_cast<const uint8_t*>(in0);
   a.y = static_cast<uint8_t*>(out);
-#ifdef TVX_CONV_TIMESTAMPS
-  if (!g_ts) { (void)hipMalloc(&g_ts, kTsBytes); (void)hipMemset(g_ts, 0, kTsBytes); }
-  a.ts = g_ts;
-#endif
   if (plan->persist_ksteps) {
     if (reinterpret_cast<uintptr_t>(in0) & 3 || reinterpret_cast<uintptr_t>(out) & 3)
       return SetError(TVX_E_INVALID, "conv2d_igemm_i8: tensors must be 4-byte aligned");
@@ -817,13 +783,6 @@ hipError_t AllowLds(int bytes) {
 }
 
 }  // namespace
-
-#ifdef TVX_CONV_TIMESTAMPS
-extern "C" int tvx_debug_conv_timestamps(void* host, size_t bytes) {
-  if (!g_ts) return -1;
-  return hipMemcpy(host, g_ts, bytes < kTsBytes ? bytes : kTsBytes, hipMemcpyDeviceToHost) == hipSuccess ? 0 : -1;
-}
-#endif
 
 // Claims dense quantized convolutions with constant weights whose weight block
 // and halo tile fit the CU's LDS.

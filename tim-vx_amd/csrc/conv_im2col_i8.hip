@@ -115,7 +115,7 @@ __global__ void __launch_bounds__(kThreads) ConvIm2colKernel(ImArgs a) {
         const bool any = *row_in & ((col_ok & kColMask) != 0);
         const int want = (any ? img_at + a.offs[r] : 0) + 4 * which;
         const int at = min(max(want, 0), a.total_bytes - 4);
-        *moved = at - want;  // first dword: -3 .. 3; second: -7 .. 0
+        *moved = at - want;  // first dword: -3 .. 4; second: -7 .. 0
         return at;
       };
       uint32_t v[kMaxRows], v2[KW == 5 ? kMaxRows : 1];
@@ -144,7 +144,8 @@ __global__ void __launch_bounds__(kThreads) ConvIm2colKernel(ImArgs a) {
           bool row_in;
           int moved;
           (void)place(r, 0, &row_in, &moved);
-          const uint32_t got = moved >= 0 ? v[r] << (8 * moved) : v[r] >> (-8 * moved);
+          // (moved by a whole dword - a five-tap row four columns in front of the tensor: every tap is masked)
+          const uint32_t got = moved >= 4 ? 0u : (moved >= 0 ? v[r] << (8 * moved) : v[r] >> (-8 * moved));
           uint32_t got2 = 0;  // (fifth tap: the second dword's first byte)
           if constexpr (KW == 5) {
             (void)place(r, 1, &row_in, &moved);

@@ -320,7 +320,7 @@ PoolQuantKernel(PoolArgs a, const T* __restrict__ x, T* __restrict__ y, uint64_t
   const uint64_t plane = idx / (static_cast<uint64_t>(a.out_w) * a.out_h);
   const T* xp = x + plane * a.in_w * a.in_h;
   int cnt = 0, vmax = INT32_MIN;
-  int64_t sum = 0;
+  int64_t sum = 0, sq = 0;
   for (int ky = 0; ky < a.k_h; ++ky) {
     const int ih = oh * a.stride_h - a.pad_top + ky;
     if (ih < 0 || ih >= a.in_h) continue;
@@ -330,12 +330,16 @@ PoolQuantKernel(PoolArgs a, const T* __restrict__ x, T* __restrict__ y, uint64_t
       const int v = static_cast<int>(xp[ih * a.in_w + iw]) - a.in_zp;
       ++cnt;
       sum += v;
+      sq += static_cast<int64_t>(v) * v;
       vmax = v > vmax ? v : vmax;
     }
   }
   int64_t r = 0;
   if (a.type == TVX_POOL_MAX) {
     if (cnt) r = RequantRne(vmax, a.mult, a.shift);
+  } else if (a.type == TVX_POOL_L2) {
+    // root of the mean of the squares, the mean over the whole window (padding counts as zeros)
+    r = static_cast<int64_t>(rint(a.ratio * __dsqrt_rn(static_cast<double>(sq) / static_cast<double>(a.k_w * a.k_h))));
   } else {
     const int div = a.type == TVX_POOL_AVG ? a.k_w * a.k_h : cnt;
     if (div) r = static_cast<int64_t>(rint(static_cast<double>(sum) * a.ratio / static_cast<double>(div)));
@@ -355,7 +359,7 @@ PoolFloatKernel(PoolArgs a, const T* __restrict__ x, T* __restrict__ y, uint64_t
   const uint64_t plane = idx / (static_cast<uint64_t>(a.out_w) * a.out_h);
   const T* xp = x + plane * a.in_w * a.in_h;
   int cnt = 0;
-  float vmax = -INFINITY, sum = 0.f;
+  float vmax = -INFINITY, sum = 0.f, sq = 0.f;
   for (int ky = 0; ky < a.k_h; ++ky) {
     const int ih = oh * a.stride_h - a.pad_top + ky;
     if (ih < 0 || ih >= a.in_h) continue;
@@ -365,12 +369,15 @@ PoolFloatKernel(PoolArgs a, const T* __restrict__ x, T* __restrict__ y, uint64_t
       const float v = ToFloat(xp[ih * a.in_w + iw]);
       ++cnt;
       sum += v;
+      sq += v * v;
       vmax = v > vmax ? v : vmax;
     }
   }
   float r;
   if (a.type == TVX_POOL_MAX) {
     r = cnt ? vmax : 0.f;
+  } else if (a.type == TVX_POOL_L2) {
+    r = sqrtf(sq / static_cast<float>(a.k_w * a.k_h));
   } else {
     const int div = a.type == TVX_POOL_AVG ? a.k_w * a.k_h : cnt;
     r = div ? sum / static_cast<float>(div) : 0.f;

@@ -64,20 +64,7 @@ struct MbArgs {
   int add_mode, add_signed;
   int add_za, add_zb, add_zo, add_lo, add_hi;
   int aligned4;                    // output planes and bands are whole dwords: dword copy-out
-#ifdef TVX_MB_TIMESTAMPS
-  unsigned long long* ts;          // profiling build: [workgroup][wavefront][64] time stamps (100 MHz counter)
-#endif
 };
-
-#ifdef TVX_MB_TIMESTAMPS
-#define TVX_TS(slot)                                                                                         \
-  do {                                                                                                       \
-    if (a.ts && lane == 0 && (slot) < 64 && blockIdx.x < 1024)                                               \
-      a.ts[(static_cast<size_t>(blockIdx.x) * 4 + wave) * 64 + (slot)] = wall_clock64();                     \
-  } while (0)
-#else
-#define TVX_TS(slot) do { } while (0)
-#endif
 
 // Window of output column J of a depthwise row: W input columns, stride S, SAME padding (one column left at
 // stride 1, none at stride 2); byte 0 of `row` is the column under the first output's leftmost tap. Columns past
@@ -150,7 +137,6 @@ __global__ void __launch_bounds__(kThreads, (MO * NTMAX <= 5 ? 2 : 1)) MbConvKer
   uint8_t* e_w = lds + a.off_wave + wave * a.wave_bytes + 4;  // (+ 4: the byte in front of row 0 is read)
   uint8_t* m_w = lds + a.off_wave + wave * a.wave_bytes + 16 + 32 * a.ep;
 
-  TVX_TS(0);
   // ---- the band's input rows as the expansion's operand: xin[halo pixel][channel], signed bytes ----
   {
     const int slots = a.mh * 32;
@@ -178,7 +164,6 @@ __global__ void __launch_bounds__(kThreads, (MO * NTMAX <= 5 ? 2 : 1)) MbConvKer
     }
   }
   __syncthreads();
-  TVX_TS(1);
 
   const int frow = lane & 31, fh = lane >> 5;
   v16i acc_out[MO][NTMAX];
@@ -227,8 +212,6 @@ __global__ void __launch_bounds__(kThreads, (MO * NTMAX <= 5 ? 2 : 1)) MbConvKer
     v4i w2f[NTMAX];
 #pragma unroll
     for (int t = 0; t < NTMAX; ++t) w2f[t] = a.w2[(min(t, a.nt - 1) * a.chunks + chunk) * 64 + lane];
-    const int ts_it = (chunk - wave) >> 2;
-    TVX_TS(2 + ts_it * 4);
 
     // ---- expansion of every halo pixel for this chunk: e_w[channel][halo pixel], signed bytes; two halo tiles
     // at a time, so that one tile's MFMA chain runs under the other's ----
@@ -257,7 +240,6 @@ __global__ void __launch_bounds__(kThreads, (MO * NTMAX <= 5 ? 2 : 1)) MbConvKer
       if (two) expand_finish(acc1, mt1, cur.rq1);
     }
     __builtin_amdgcn_wave_barrier();
-    TVX_TS(3 + ts_it * 4);
 
     // ---- depthwise 3x3: lane = (channel, every second output row) -> m_w[output pixel][channel] ----
     for (int orr = fh; orr < rows_out; orr += 2) {
@@ -285,7 +267,6 @@ __global__ void __launch_bounds__(kThreads, (MO * NTMAX <= 5 ? 2 : 1)) MbConvKer
       DwRow<W, S, 0>::Run(a, rows, dk, rq2, m_w + orr * OW * kMStride, frow, ch < a.Cexp);
     }
     __builtin_amdgcn_wave_barrier();
-    TVX_TS(4 + ts_it * 4);
 
     // ---- this chunk's contribution to every output tile ----
 #pragma unroll
@@ -300,11 +281,8 @@ __global__ void __launch_bounds__(kThreads, (MO * NTMAX <= 5 ? 2 : 1)) MbConvKer
       }
     }
     __builtin_amdgcn_wave_barrier();
-    TVX_TS(5 + ts_it * 4);
   }
-  TVX_TS(44);
   __syncthreads();  // the walk's LDS areas are free from here
-  TVX_TS(45);
 
   // ---- the four partial projections meet, one output tile at a time; wavefront t % 4 owns tile t ----
   int* red = reinterpret_cast<int*>(lds + a.off_red);
@@ -397,7 +375,6 @@ __global__ void __launch_bounds__(kThreads, (MO * NTMAX <= 5 ? 2 : 1)) MbConvKer
         }
         __builtin_amdgcn_wave_barrier();
       }
-      TVX_TS(46 + t);
     }
   }
 }
@@ -432,18 +409,9 @@ MbFn Kernel(const Plan& p) {
   return p.a.add_mode ? KernelOf<true>(p.w, p.s, p.a.nt) : KernelOf<false>(p.w, p.s, p.a.nt);
 }
 
-#ifdef TVX_MB_TIMESTAMPS
-unsigned long long* g_ts = nullptr;
-constexpr size_t kTsBytes = 1024 * 4 * 64 * 8;
-#endif
-
 int MbConvRun(tvx_op* op, const void* in0, const void* in1, void* out, hipStream_t st) {
   const Plan* plan = reinterpret_cast<const Plan*>(op->host_blob.data());
   MbArgs a = plan->a;
-#ifdef TVX_MB_TIMESTAMPS
-  if (!g_ts) { (void)hipMalloc(&g_ts, kTsBytes); (void)hipMemset(g_ts, 0, kTsBytes); }
-  a.ts = g_ts;
-#endif
   a.x = static_cast<const uint8_t*>(in0);
   a.y = static_cast<uint8_t*>(out);
   a.res = static_cast<const uint8_t*>(in1);
@@ -486,17 +454,6 @@ bool Feeds(const tvx_conv2d_desc* a, const tvx_conv2d_desc* b) {
 }
 
 }  // namespace
-
-#ifdef TVX_MB_TIMESTAMPS
-// profiling build only: the time stamps of the most recent launches, then cleared
-extern "C" int tvx_debug_mb_timestamps(void* host, size_t bytes) {
-  if (!g_ts || bytes > kTsBytes) return -1;
-  if (hipDeviceSynchronize() != hipSuccess) return -1;
-  if (hipMemcpy(host, g_ts, bytes, hipMemcpyDeviceToHost) != hipSuccess) return -1;
-  (void)hipMemset(g_ts, 0, kTsBytes);
-  return 0;
-}
-#endif
 
 // `op` carries the projection (op->conv, its requantization tables in h_mult / h_shift, clamp, fused Add);
 // the expansion and the depthwise convolution come with their own tables. Declines (TVX_E_UNSUPPORTED) what

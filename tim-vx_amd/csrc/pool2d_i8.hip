@@ -412,7 +412,7 @@ int PoolRowsRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t
 // the vertical stride are free).
 int PoolRowsSetup(tvx_op* op) {
   const tvx_pool2d_desc& d = op->pool;
-  if (!op->quantized) return TVX_E_UNSUPPORTED;
+  if (!op->quantized || d.pool_type == TVX_POOL_L2) return TVX_E_UNSUPPORTED;  // (L2: the generic kernel)
   if ((d.k_w != 2 && d.k_w != 3) || (d.stride_w != 1 && d.stride_w != 2) || d.k_h > 16 || d.stride_h > 16)
     return TVX_E_UNSUPPORTED;
   if (d.pad_left >= d.k_w || d.pad_top >= d.k_h) return TVX_E_UNSUPPORTED;
@@ -450,7 +450,6 @@ int PoolRowsSetup(tvx_op* op) {
   while (a.G > 1 && (planes + a.G - 1) / a.G < 1024) a.G = (a.G + 1) / 2;
   const int lds_bytes = (a.G * plane_lds + 15) / 16 * 16 + 16;
   if (lds_bytes > 64 * 1024) return TVX_E_UNSUPPORTED;
-  const int plan_g = a.G, plan_rows_in = a.rows_in;
   const bool is_signed = d.dtype == TVX_I8;
   const int neutral = d.pool_type == TVX_POOL_MAX ? (is_signed ? 0x80 : 0x00) : (d.in_zp & 0xff);
   a.fill = static_cast<int>(static_cast<uint32_t>(neutral) * 0x01010101u);
@@ -490,23 +489,24 @@ int PoolRowsSetup(tvx_op* op) {
     pipelined = ((plane_bytes * g) & 15) == 0 && ((plane_bytes & 15) == 0 || planes % g == 0) &&
                 plane_bytes * g <= static_cast<uint64_t>(kChunks) * kThreads * 16 &&
                 plane_bytes * plane_bytes * g < (1ull << 32) && steps >= 512;
+    // the pipelined plan is worked out aside and taken over only if it stands: its two LDS images must fit 64 KiB
+    const int rows_in = std::max((a.OH - 1) * a.sh + a.kh, a.pad_t + a.H);  // every row of a plane is stored (with FLOOR rounding the last ones may lie below the last window)
+    const int lds2 = 2 * ((g * rows_in * a.pitch + 15) / 16 * 16) + 16;
+    if (pipelined && lds2 > 64 * 1024) pipelined = false;
     if (pipelined) {
-      a.G = g;
-      a.magic_plane = plane_bytes <= 1 ? 0u : static_cast<uint32_t>(((uint64_t{1} << 32) + plane_bytes - 1) / plane_bytes);
-      // every row of a plane is stored (with FLOOR rounding the last ones may lie below the last window)
-      a.rows_in = std::max((a.OH - 1) * a.sh + a.kh, a.pad_t + a.H);
       hipDeviceProp_t prop;
       int dev = 0;
       if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return SetError(TVX_E_DEVICE, "no device properties");
       int wg = 3 * prop.multiProcessorCount;
       if (const char* f = getenv("TVX_POOL_WGS")) wg = std::max(1, atoi(f));  // tuning aid
+      a.G = g;
+      a.magic_plane = plane_bytes <= 1 ? 0u : static_cast<uint32_t>(((uint64_t{1} << 32) + plane_bytes - 1) / plane_bytes);
+      a.rows_in = rows_in;
       plan.grid = dim3(static_cast<unsigned>(std::min<uint64_t>(steps, wg)));
-      plan.lds_bytes = 2 * ((a.G * a.rows_in * a.pitch + 15) / 16 * 16) + 16;
-      if (plan.lds_bytes > 64 * 1024) pipelined = false;
+      plan.lds_bytes = lds2;
     }
   }
   plan.pipelined = pipelined;
-  if (!pipelined) { a.G = plan_g; a.rows_in = plan_rows_in; }
   plan.a = a;
   if (!Kernel(&plan)) return TVX_E_UNSUPPORTED;
   op->host_blob.assign(reinterpret_cast<const uint8_t*>(&plan), reinterpret_cast<const uint8_t*>(&plan) + sizeof(plan));

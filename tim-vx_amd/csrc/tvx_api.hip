@@ -647,7 +647,7 @@ int tvx_pool2d_create(const tvx_pool2d_desc* d, tvx_op** out) {
       !d->k_h || !d->stride_w || !d->stride_h)
     return SetError(TVX_E_INVALID, "tvx_pool2d_create: zero extent or stride");
   if (!ValidDtype(d->dtype)) return SetError(TVX_E_INVALID, "tvx_pool2d_create: unknown dtype");
-  if (d->pool_type != TVX_POOL_MAX && d->pool_type != TVX_POOL_AVG && d->pool_type != TVX_POOL_AVG_ANDROID)
+  if (d->pool_type != TVX_POOL_MAX && d->pool_type != TVX_POOL_AVG && d->pool_type != TVX_POOL_AVG_ANDROID && d->pool_type != TVX_POOL_L2)
     return SetError(TVX_E_UNSUPPORTED, "tvx_pool2d_create: pool type %d", d->pool_type);
   int s = CheckZeroPoint(d->dtype, d->in_zp, "tvx_pool2d_create", "input");
   if (s == TVX_OK) s = CheckZeroPoint(d->dtype, d->out_zp, "tvx_pool2d_create", "output");

@@ -114,13 +114,15 @@ def write_graphs(graphs, txt_path, blob_path, bench=None):
             txt.write("end\n")
 
 
-def run_graphs(graphs, workdir, bench=None, timeout=600, env=None):
+def run_graphs(graphs, workdir, bench=None, timeout=600, env=None, threads=0, lock=True):
     """Returns (outputs, info, log): per graph the flat output array (None where the runtime
     refused the graph, the stage then in info[name]["fail"]); with `bench`, info[name] holds
     the milliseconds per Graph::Run() as "run_ms" (whole call, host copies included) and
     "device_ms" (the operator sequence alone); a graph with "reruns" (a list of {input tensor
     id: data}) is run again once per entry and info[name]["reruns"] lists those outputs; log is
-    what the runtime wrote to stderr."""
+    what the runtime wrote to stderr. With `threads` the runner processes the file in that many threads (one after
+    the other under one mutex, or all at once with lock=False), each from Context::Create() on; it fails unless all
+    threads produce the same bytes, and the first thread's results are returned."""
     if not os.path.exists(RUNNER):
         raise RuntimeError("%s is not built: run build.py" % RUNNER)
     os.makedirs(workdir, exist_ok=True)
@@ -128,10 +130,13 @@ def run_graphs(graphs, workdir, bench=None, timeout=600, env=None):
     write_graphs(graphs, txt, blob, bench)
     e = dict(os.environ)
     e.update(env or {})
-    p = subprocess.run([RUNNER, txt, blob, out], capture_output=True, text=True, timeout=timeout, env=e)
+    cmd = [RUNNER, txt, blob, out]
+    if threads:
+        cmd = [RUNNER, "--threads", str(threads)] + ([] if lock else ["--no-lock"]) + [txt, blob, out]
+    p = subprocess.run(cmd, capture_output=True, text=True, timeout=timeout, env=e)
     if p.returncode != 0:
         raise RuntimeError("tvx_graph_runner exit %d\n%s\n%s" % (p.returncode, p.stdout[-2000:], p.stderr[-4000:]))
-    raw = open(out, "rb").read()
+    raw = open(out + ".0" if threads else out, "rb").read()
     results, info = [], {}
     by_name = {}
     for line in p.stdout.splitlines():

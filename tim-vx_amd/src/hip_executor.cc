@@ -753,6 +753,13 @@ extern "C" double tvx_runtime_last_device_ms(void) { return tim::vx::g_last_devi
 // name and microseconds of operator i. No counterpart in the reference's API (its driver keeps such numbers
 // per vx_node).
 extern "C" int tvx_runtime_last_op_count(void) { return static_cast<int>(tim::vx::g_last_op_us.size()); }
-extern "C" const char* tvx_runtime_last_op_name(int i) { return tim::vx::g_last_op_us[static_cast<size_t>(i)].first.c_str(); }
-extern "C" double tvx_runtime_last_op_us(int i) { return tim::vx::g_last_op_us[static_cast<size_t>(i)].second; }
-extern "C" unsigned long long tvx_runtime_last_op_bytes(int i) { return tim::vx::g_last_op_bytes[static_cast<size_t>(i)]; }
+// (an index outside [0, count) answers with nothing / zero)
+extern "C" const char* tvx_runtime_last_op_name(int i) {
+  return i >= 0 && static_cast<size_t>(i) < tim::vx::g_last_op_us.size() ? tim::vx::g_last_op_us[static_cast<size_t>(i)].first.c_str() : nullptr;
+}
+extern "C" double tvx_runtime_last_op_us(int i) {
+  return i >= 0 && static_cast<size_t>(i) < tim::vx::g_last_op_us.size() ? tim::vx::g_last_op_us[static_cast<size_t>(i)].second : 0.0;
+}
+extern "C" unsigned long long tvx_runtime_last_op_bytes(int i) {
+  return i >= 0 && static_cast<size_t>(i) < tim::vx::g_last_op_bytes.size() ? tim::vx::g_last_op_bytes[static_cast<size_t>(i)] : 0ull;
+}

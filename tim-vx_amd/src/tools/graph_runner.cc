@@ -32,6 +32,8 @@
 #include <fstream>
 #include <iostream>
 #include <map>
+#include <mutex>
+#include <thread>
 #include <sstream>
 #include <string>
 #include <vector>
@@ -110,20 +112,73 @@ struct Pending {
 
 }  // namespace
 
+// Processes one graph file; result lines go to `log` (stdout for the plain invocation).
+static int RunFile(const char* graphs_path, const char* blob_path, const char* out_path, FILE* log);
+
+// With --threads N the file is processed by N threads, each from Context::Create() on, one after the other under one
+// mutex - the reference's multi-thread sample does the same with its LeNet
+// (samples/multi_thread_test/multi_thread_test.cc:330-372) - or, with --no-lock, all at once (a context per thread).
+// Thread i writes <out>.<i>; the results must be the same bytes and the same result lines.
+static int RunThreads(int n_threads, bool lock, const char* graphs_path, const char* blob_path, const char* out_path) {
+  std::mutex mutex;
+  std::vector<std::thread> threads;
+  std::vector<int> status(static_cast<size_t>(n_threads), -1);
+  std::vector<std::string> logs(static_cast<size_t>(n_threads)), outs(static_cast<size_t>(n_threads));
+  for (int i = 0; i < n_threads; ++i) {
+    outs[static_cast<size_t>(i)] = std::string(out_path) + "." + std::to_string(i);
+    threads.emplace_back([&, i]() {
+      std::unique_lock<std::mutex> guard(mutex, std::defer_lock);
+      if (lock) guard.lock();
+      char* text = nullptr;
+      size_t size = 0;
+      FILE* log = open_memstream(&text, &size);
+      status[static_cast<size_t>(i)] = RunFile(graphs_path, blob_path, outs[static_cast<size_t>(i)].c_str(), log);
+      std::fclose(log);
+      logs[static_cast<size_t>(i)].assign(text, size);
+      std::free(text);
+    });
+  }
+  for (auto& t : threads) t.join();
+  auto slurp = [](const std::string& path) {
+    std::ifstream f(path, std::ios::binary);
+    return std::string((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+  };
+  const std::string first = slurp(outs[0]);
+  bool same = status[0] == 0;
+  for (int i = 1; i < n_threads; ++i)
+    same = same && status[static_cast<size_t>(i)] == 0 && logs[static_cast<size_t>(i)] == logs[0] && slurp(outs[static_cast<size_t>(i)]) == first;
+  std::fputs(logs[0].c_str(), stdout);
+  std::printf("threads %d %s %zu\n", n_threads, same ? "identical" : "different", first.size());
+  return same ? 0 : 1;
+}
+
 int main(int argc, char** argv) {
+  setenv("TVX_RUNTIME_PROFILE", "1", 0);  // makes `bench` report the device part of Run()
+  if (argc >= 2 && std::string(argv[1]) == "--threads") {
+    const bool lock = !(argc >= 4 && std::string(argv[3]) == "--no-lock");
+    const int first = lock ? 3 : 4;
+    if (argc != first + 3) {
+      std::fprintf(stderr, "usage: tvx_graph_runner --threads N [--no-lock] graphs.txt blob.bin out.bin\n");
+      return 2;
+    }
+    return RunThreads(std::max(1, atoi(argv[2])), lock, argv[first], argv[first + 1], argv[first + 2]);
+  }
   if (argc != 4) {
-    std::fprintf(stderr, "usage: %s graphs.txt blob.bin out.bin\n", argv[0]);
+    std::fprintf(stderr, "usage: tvx_graph_runner graphs.txt blob.bin out.bin\n");
     return 2;
   }
-  std::ifstream txt(argv[1]);
-  std::ifstream blobf(argv[2], std::ios::binary);
+  return RunFile(argv[1], argv[2], argv[3], stdout);
+}
+
+static int RunFile(const char* graphs_path, const char* blob_path, const char* out_path, FILE* log) {
+  std::ifstream txt(graphs_path);
+  std::ifstream blobf(blob_path, std::ios::binary);
   if (!txt || !blobf) { std::fprintf(stderr, "cannot open inputs\n"); return 2; }
   std::vector<char> blob((std::istreambuf_iterator<char>(blobf)), std::istreambuf_iterator<char>());
-  FILE* out = std::fopen(argv[3], "wb");
-  if (!out) { std::fprintf(stderr, "cannot open %s\n", argv[3]); return 2; }
+  FILE* out = std::fopen(out_path, "wb");
+  if (!out) { std::fprintf(stderr, "cannot open %s\n", out_path); return 2; }
   size_t out_off = 0;
 
-  setenv("TVX_RUNTIME_PROFILE", "1", 0);  // makes `bench` report the device part of Run()
   auto context = Context::Create();
   std::shared_ptr<Graph> graph, source_graph;
   std::map<int, Pending> tensors;
@@ -371,13 +426,13 @@ int main(int argc, char** argv) {
         }
       }
       if (stage) {
-        std::printf("fail %s %s\n", name.c_str(), stage);
+        std::fprintf(log, "fail %s %s\n", name.c_str(), stage);
       } else {
         std::fwrite(result.data(), 1, result.size(), out);
-        std::printf("ok %s %zu %zu\n", name.c_str(), out_off, result.size());
+        std::fprintf(log, "ok %s %zu %zu\n", name.c_str(), out_off, result.size());
         out_off += result.size();
       }
-      std::fflush(stdout);
+      std::fflush(log);
     } else if (rec == "feed") {
       // the input tensor takes other bytes of the blob from the next `run` on
       int id;
@@ -394,7 +449,7 @@ int main(int argc, char** argv) {
     } else if (rec == "bench") {
       int warmup, iters;
       ss >> warmup >> iters;
-      if (!compile_ok) { std::printf("fail %s bench\n", name.c_str()); continue; }
+      if (!compile_ok) { std::fprintf(log, "fail %s bench\n", name.c_str()); continue; }
       // every iteration hands the inputs over again, as an application with new data would: the time per
       // Run() then holds the host -> device copy of the inputs as well as the download of the output
       auto feed = [&]() {
@@ -415,15 +470,16 @@ int main(int argc, char** argv) {
         for (int o = 0; o < n_ops; ++o) op_us[static_cast<size_t>(o)] += tvx_runtime_last_op_us(o);
       }
       auto t1 = std::chrono::steady_clock::now();
-      std::printf("bench %s %.6f %.6f\n", name.c_str(),
+      std::fprintf(log, "bench %s %.6f %.6f\n", name.c_str(),
                   std::chrono::duration<double, std::milli>(t1 - t0).count() / iters, dev_ms / iters);
       for (size_t o = 0; o < op_us.size(); ++o) {
-        std::string op_name = tvx_runtime_last_op_name(static_cast<int>(o));
+        const char* raw_name = tvx_runtime_last_op_name(static_cast<int>(o));
+        std::string op_name = raw_name ? raw_name : "?";
         for (char& c : op_name) if (c == ' ') c = '_';
-        std::printf("opbench %s %zu %s %.3f %llu\n", name.c_str(), o, op_name.c_str(), op_us[o] / iters,
+        std::fprintf(log, "opbench %s %zu %s %.3f %llu\n", name.c_str(), o, op_name.c_str(), op_us[o] / iters,
                     tvx_runtime_last_op_bytes(static_cast<int>(o)));
       }
-      std::fflush(stdout);
+      std::fflush(log);
     } else if (rec == "end") {
       graph.reset();
       source_graph.reset();
