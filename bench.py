@@ -564,6 +564,7 @@ def main():
             extra[w2["name"]] = rec
         if args.no_networks:
             line["extra"] = extra
+            line["children_at_exit"] = reap_children()
             print(json.dumps(line))
             return
         extra.update(network_extras(max(5, min(args.steps, 30)), 3))
@@ -578,7 +579,25 @@ def main():
             "copy_12p8MB_read_plus_write_gbs": round(T.calibrate_copy(12845056, 50), 0),
         }
         line["extra"] = extra
+    line["children_at_exit"] = reap_children()
     print(json.dumps(line))
+
+
+def reap_children():
+    """Nothing may outlive the benchmark: every child process this run started (the graph runner, a build step)
+    has been waited for; whatever is still there is ended and counted."""
+    try:
+        import psutil
+    except ImportError:
+        return None
+    left = psutil.Process().children(recursive=True)
+    for p in left:
+        try:
+            p.kill()
+        except psutil.Error:
+            pass
+    psutil.wait_procs(left, timeout=5)
+    return len(left)
 
 
 if __name__ == "__main__":

@@ -43,6 +43,38 @@ struct DwArgs {
 
 
 
+// (v >> t) into byte E of d (the other bytes stay): the shift writes its result where the packed dword wants it
+template <int E>
+__device__ __forceinline__ void ShiftIntoByte(uint32_t& d, int t, int v) {
+  if (E == 0) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:DWORD" : "=v"(d) : "v"(t), "v"(v));
+  if (E == 1) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(d) : "v"(t), "v"(v));
+  if (E == 2) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(d) : "v"(t), "v"(v));
+  if (E == 3) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(d) : "v"(t), "v"(v));
+}
+
+// Four accumulators of the channel -> four codes in one dword. Where no accumulator can land on a tie the clamp
+// comes in front of the shift (bounds shifted up: `lo_t`, `hi_t`), and the shift writes its byte of the dword: no
+// packing instructions.
+template <int RQ>
+__device__ __forceinline__ uint32_t Requant4(const int (&acc)[4], const tvx_v4i& q, int t_v, int lo_t, int hi_t, int out_zp,
+                                             int lo, int hi) {
+  if (RQ == kRqFastNoTie) {
+    int u[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) u[e] = Med3(__mulhi(acc[e], q[0]) + q[2], lo_t, hi_t);
+    uint32_t d;
+    ShiftIntoByte<0>(d, t_v, u[0]);
+    ShiftIntoByte<1>(d, t_v, u[1]);
+    ShiftIntoByte<2>(d, t_v, u[2]);
+    ShiftIntoByte<3>(d, t_v, u[3]);
+    return d;
+  }
+  int r[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) r[e] = Requant8<RQ>(acc[e], q, out_zp, lo, hi);
+  return PackBytes(r[0], r[1], r[2], r[3]);
+}
+
 // S = stride (1 or 2, both directions), PL = left padding (0 or 1)
 // RPT: output rows a thread produces (more rows: fewer, fatter workgroups and fewer halo rows re-read)
 // CW: output columns a thread produces, 4 or 8 (8: one 64-bit load per input row, twice the bytes in flight
@@ -101,17 +133,26 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
   // Left to the compiler they are requested where they are first used, behind the wait for the rows - a second
   // round trip.
   asm volatile("" ::"s"(wk0), "s"(wk1), "s"(wk2), "s"(bias), "s"(q[0]), "s"(q[1]), "s"(q[2]), "s"(q[3]));
+  // Wavefronts whose rows and dwords all lie inside the image (one vote: most of them) only re-bias their bytes.
+  const bool edge = ih0 < 0 || ih0 + kRows > a.H || d0 + kOwn > in_dwords;
+  if (__builtin_amdgcn_ballot_w64(edge) != 0) {
 #pragma unroll
-  for (int r = 0; r < kRows; ++r) {
-    const int ih = ih0 + r;
-    const int keep_row = min(max(ih, 0), a.H - 1) == ih ? -1 : 0;
+    for (int r = 0; r < kRows; ++r) {
+      const int ih = ih0 + r;
+      const int keep_row = min(max(ih, 0), a.H - 1) == ih ? -1 : 0;
 #pragma unroll
-    for (int i = 0; i < kOwn; ++i) {
-      const int keep = d0 + i < in_dwords ? keep_row : 0;
-      // mask arithmetic, not a select: a select on the loaded value would be compiled into a
-      // branch around the load, and then the loads would be waited for one at a time
-      raw[r][1 + i] = ((raw[r][1 + i] ^ a.xor_mask) & keep) | (a.pad_fill & ~keep);
+      for (int i = 0; i < kOwn; ++i) {
+        const int keep = d0 + i < in_dwords ? keep_row : 0;
+        // mask arithmetic, not a select: a select on the loaded value would be compiled into a
+        // branch around the load, and then the loads would be waited for one at a time
+        raw[r][1 + i] = ((raw[r][1 + i] ^ a.xor_mask) & keep) | (a.pad_fill & ~keep);
+      }
     }
+  } else if (a.xor_mask) {
+#pragma unroll
+    for (int r = 0; r < kRows; ++r)
+#pragma unroll
+      for (int i = 0; i < kOwn; ++i) raw[r][1 + i] ^= a.xor_mask;
   }
 #pragma unroll
   for (int r = 0; r < kRows; ++r) {
@@ -127,8 +168,10 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
   // Uniform operands that the instructions below take from vector registers (the three-address dot product, the
   // clamp) get one copy for all output rows: each row is a block of its own behind the bounds test, and the
   // compiler would copy them again in every block.
-  int bias_v = bias, wk0_v = wk0, lo_v = a.lo, hi_v = a.hi;
-  asm volatile("" : "+v"(bias_v), "+v"(wk0_v), "+v"(lo_v), "+v"(hi_v));
+  int bias_v = bias, wk0_v = wk0, lo_v = a.lo, hi_v = a.hi, t_v = q[1];
+  const int lo_t = a.lo << q[1];
+  int hi_t = (a.hi << q[1]) | ((1 << q[1]) - 1);
+  asm volatile("" : "+v"(bias_v), "+v"(wk0_v), "+v"(lo_v), "+v"(hi_v), "+v"(t_v), "+v"(hi_t));
   uint8_t* const yrow = yp;  // (uniform base; offsets inside a plane fit 32 bits)
   if constexpr (CW == 8) {
     // windows are cut per output row (three input rows x eight windows live at a time)
@@ -155,10 +198,11 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
           sx = __builtin_amdgcn_sdot4(win3[2], 0x00010101, sx, false);
           acc -= a.zws * sx;
         }
-        res[i] = Requant8<RQ>(acc, q, a.out_zp, lo_v, hi_v);
+        res[i] = acc;
       }
+      const int lo4[4] = {res[0], res[1], res[2], res[3]}, hi4[4] = {res[4], res[5], res[6], res[7]};
       *reinterpret_cast<uint2*>(yrow + (__umul24(static_cast<uint32_t>(oh0 + o), static_cast<uint32_t>(a.OW)) + static_cast<uint32_t>(w4) * 8u)) =
-          make_uint2(PackBytes(res[0], res[1], res[2], res[3]), PackBytes(res[4], res[5], res[6], res[7]));
+          make_uint2(Requant4<RQ>(lo4, q, t_v, lo_t, hi_t, a.out_zp, lo_v, hi_v), Requant4<RQ>(hi4, q, t_v, lo_t, hi_t, a.out_zp, lo_v, hi_v));
     }
   } else {
   int win[kRows][4];
@@ -185,10 +229,10 @@ __global__ void __launch_bounds__(kThreads) DwConv3x3Kernel(DwArgs a) {
         sx = __builtin_amdgcn_sdot4(win[S * o + 2][i], 0x00010101, sx, false);
         acc -= a.zws * sx;
       }
-      res[i] = Requant8<RQ>(acc, q, a.out_zp, lo_v, hi_v);
+      res[i] = acc;
     }
     *reinterpret_cast<uint32_t*>(yrow + (__umul24(static_cast<uint32_t>(oh0 + o), static_cast<uint32_t>(a.OW)) + static_cast<uint32_t>(w4) * 4u)) =
-        PackBytes(res[0], res[1], res[2], res[3]);
+        Requant4<RQ>(res, q, t_v, lo_t, hi_t, a.out_zp, lo_v, hi_v);
   }
   }
 }
@@ -202,6 +246,7 @@ struct Shape {
 struct Plan {
   DwArgs a;
   int stride, pad_l, boxsum, rq;
+  int lds_pad;      // dynamic LDS the launch asks for without using it: caps the workgroups a CU runs at a time
   int cols;         // output columns per thread of the preferred form: 4 or 8
   Shape shape;      // ... its geometry
   Shape fallback;   // four columns per thread: taken when the 8-column form is preferred but a pointer is not 8-byte aligned
@@ -210,9 +255,9 @@ struct Plan {
 template <int S, int PL, bool BOXSUM, int RPT, int CW>
 void LaunchRq(const Plan* p, const Shape& sh, const DwArgs& a, hipStream_t st) {
   const dim3 block(sh.threads);
-  if (p->rq == kRqFastNoTie) hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqFastNoTie, RPT, CW>), sh.grid, block, 0, st, a);
-  else if (p->rq == kRqFast) hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqFast, RPT, CW>), sh.grid, block, 0, st, a);
-  else hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqGeneric, RPT, CW>), sh.grid, block, 0, st, a);
+  if (p->rq == kRqFastNoTie) hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqFastNoTie, RPT, CW>), sh.grid, block, p->lds_pad, st, a);
+  else if (p->rq == kRqFast) hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqFast, RPT, CW>), sh.grid, block, p->lds_pad, st, a);
+  else hipLaunchKernelGGL((DwConv3x3Kernel<S, PL, BOXSUM, kRqGeneric, RPT, CW>), sh.grid, block, p->lds_pad, st, a);
 }
 
 template <int S, int PL, int CW>
@@ -371,6 +416,8 @@ int DwConv3x3Setup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
     sh.grid = dim3(C, d->batch, (row_groups + sh.rg_per_block - 1) / sh.rg_per_block);
     return sh;
   };
+  p.lds_pad = 0;
+  if (const char* f = getenv("TVX_DWCONV_LDS_KB")) p.lds_pad = std::max(0, std::min(64, atoi(f))) * 1024;  // tuning aid
   p.cols = cols;
   p.shape = shape_for(cols);
   p.fallback = shape_for(4);
