@@ -246,6 +246,30 @@ int tvx_mbconv_create(const tvx_conv2d_desc* expand, const void* expand_weights_
                       const tvx_conv2d_desc* project, const void* project_weights_host, const void* project_bias_host,
                       const tvx_eltwise_desc* add, int conv_operand, tvx_op** op);
 
+/* ---- Conv2d + the 2x2 / stride-2 max pooling it only feeds, in one kernel ------------------------------ */
+/* Two nodes of the reference's graph (vxConvolutionLayer: kernel/vx/convolutional.c:504-582, then
+ * vxPoolingLayer2: src/tim/vx/internal/src/ops/vsi_nn_op_pool.c:144-150) whose intermediate tensor has no
+ * other reader - LeNet's conv1 / pool1 and conv2 / pool2 (samples/lenet/lenet_asymu8.cc:248-272); the closed
+ * driver merges such layers when it verifies the graph (src/tim/vx/internal/src/vsi_nn_graph.c:1591-1603).
+ * The result is, bit for bit, what the two operators give one after the other (requantization is monotone, so
+ * the maximum of the four accumulators is requantized once). `conv` describes the convolution as for
+ * tvx_conv2d_create, `pool` the pooling as for tvx_pool2d_create: MAX, 2 x 2 window, stride 2, no padding,
+ * input = the convolution's output (even extents) with the same type and quantization on both sides.
+ * Returns TVX_E_UNSUPPORTED when no kernel fuses this pair (the caller then creates the two operators). */
+int tvx_conv2d_pool_create(const tvx_conv2d_desc* conv, const tvx_pool2d_desc* pool, const void* weights_host,
+                           const void* bias_host, tvx_op** op);
+
+/* ---- FullyConnected + the Softmax over its outputs, in one kernel -------------------------------------- */
+/* Two nodes of the reference's graph (vxFullyConnectedLayer: kernel/vx/convolutional.c:584-652, then
+ * vxSoftmaxLayer2: src/tim/vx/internal/src/kernel/vx/softmax_vx.c:88) - the classifier head of LeNet
+ * (samples/lenet/lenet_asymu8.cc:283-290): a quantized FullyConnected layer with at most 16 outputs whose
+ * codes only feed a Softmax along that axis. The result (fp32) is, bit for bit, what the two operators give
+ * one after the other. `fc` as for tvx_fully_connected_create (constant weights), `softmax` as for
+ * tvx_softmax_create with channels = fc->n, rows = fc->m, inner <= 1 and the FullyConnected output's type and
+ * quantization as its input's. Returns TVX_E_UNSUPPORTED otherwise (the caller then creates the two operators). */
+int tvx_fully_connected_softmax_create(const tvx_fc_desc* fc, const tvx_softmax_desc* softmax,
+                                       const void* weights_host, const void* bias_host, tvx_op** op);
+
 /* ---- DeConv2d (transposed convolution) ----------------------------------------------- */
 /* Replaces vxDeconvolutionLayer (src/tim/vx/ops/deconv.cc:45-79,
  * src/tim/vx/internal/src/ops/vsi_nn_op_deconvolution.c:217-218,398-497). Same descriptor as

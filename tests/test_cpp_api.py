@@ -169,7 +169,17 @@ def test_lenet_sample_graph(tmp_path, oracle):
     # FullyConnected + Relu through a single-consumer TRANSIENT tensor is fused: no separate
     # activation kernel appears in the plan
     plan = [l for l in log.splitlines() if "uid" in l and "->" in l]
-    assert plan and not any("RELU" in l for l in plan[:7]), plan
+    assert plan and not any("RELU" in l for l in plan), plan
+    # convolution + max pooling and FullyConnected + Softmax through such tensors run as one kernel each: the
+    # sample's nine operators are four launches (five where the graph ends with the logits)
+    kernels = [l.split("(")[-1].rstrip(")") for l in plan]
+    assert kernels[:4] == ["conv2d_im2col_maxpool_i8", "conv2d_igemm_maxpool_i8", "fc_generic", "fc_softmax_i8"], kernels
+    assert kernels[4:8] == ["conv2d_im2col_maxpool_i8", "conv2d_igemm_maxpool_i8", "fc_generic", "fc_generic"], kernels
+    assert len(kernels) == 12
+    # ... and give the bytes of the operators run one by one
+    apart, _, log2 = GF.run_graphs([g, batched], str(tmp_path / "apart"), env={"VSI_NN_LOG_LEVEL": "3", "TVX_NO_POOL_FUSION": "1"})
+    assert len([l for l in log2.splitlines() if "uid" in l and "->" in l]) == 14
+    assert np.array_equal(apart[0], res[0]) and np.array_equal(apart[1], res[2])
 
 
 @pytest.mark.gpu

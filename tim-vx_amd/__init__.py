@@ -118,6 +118,8 @@ def lib():
                                               C.POINTER(EltwiseDesc), C.c_int, C.POINTER(vp)]
         L.tvx_mbconv_create.argtypes = [C.POINTER(Conv2dDesc), vp, vp, C.POINTER(Conv2dDesc), vp, vp, C.POINTER(Conv2dDesc), vp, vp,
                                         C.POINTER(EltwiseDesc), C.c_int, C.POINTER(vp)]
+        L.tvx_conv2d_pool_create.argtypes = [C.POINTER(Conv2dDesc), C.POINTER(Pool2dDesc), vp, vp, C.POINTER(vp)]
+        L.tvx_fully_connected_softmax_create.argtypes = [C.POINTER(FcDesc), C.POINTER(SoftmaxDesc), vp, vp, C.POINTER(vp)]
         L.tvx_fully_connected_create.argtypes = [C.POINTER(FcDesc), vp, vp, C.POINTER(vp)]
         L.tvx_pool2d_create.argtypes = [C.POINTER(Pool2dDesc), C.POINTER(vp)]
         L.tvx_activation_create.argtypes = [C.POINTER(EltwiseDesc), C.POINTER(vp)]
@@ -201,6 +203,21 @@ def mbconv_create(expand, expand_w, expand_b, dw, dw_w, dw_b, project, project_w
                                   C.byref(dw), _host_ptr(dw_w), _host_ptr(dw_b),
                                   C.byref(project), _host_ptr(project_w), _host_ptr(project_b),
                                   C.byref(add_desc) if add_desc is not None else None, conv_operand, C.byref(h)))
+    return Op(h)
+
+
+def conv2d_pool_create(desc, pool_desc, weights, bias=None):
+    """A convolution and the 2x2 / stride-2 max pooling behind it as one operator."""
+    h = C.c_void_p()
+    check(lib().tvx_conv2d_pool_create(C.byref(desc), C.byref(pool_desc), _host_ptr(weights), _host_ptr(bias), C.byref(h)))
+    return Op(h)
+
+
+def fully_connected_softmax_create(desc, softmax_desc, weights, bias=None):
+    """A FullyConnected layer of at most 16 outputs and the Softmax over them as one operator (fp32 result)."""
+    h = C.c_void_p()
+    check(lib().tvx_fully_connected_softmax_create(C.byref(desc), C.byref(softmax_desc), _host_ptr(weights),
+                                                   _host_ptr(bias), C.byref(h)))
     return Op(h)
 
 

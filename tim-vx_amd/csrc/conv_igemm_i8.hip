@@ -66,6 +66,7 @@ struct ConvArgs {
   int rows;              // ... output rows of a tile
   uint32_t blk_col, blk_chan;  // ... per wavefront w (byte w): w % w4_blocks and w / w4_blocks
   int off_out;           // epilogue staging tile
+  int pool;              // one-tile-per-workgroup kernel: a 2 x 2 / stride-2 max pooling rides on the epilogue
   int tap_off[40];       // halo byte offset of k-step ks (both fragment halves lie in one tap: + 16 * half)
 };
 
@@ -103,8 +104,11 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(O
   const int hw = a.OH * a.OW;
   const int p0 = tile * a.P;
   const int p_end = min(p0 + a.P, hw);
-  const int r0 = p0 / a.OW;
-  const int r1 = (p_end - 1) / a.OW;
+  // With pooling the pixels run in pooling order: four consecutive ones are a 2 x 2 window (row-major), windows
+  // row-major over the pooled image - the four accumulators a lane holds per quad are one pooled pixel's candidates.
+  const int pool_w = a.OW >> 1;
+  const int r0 = a.pool ? 2 * ((p0 >> 2) / pool_w) : p0 / a.OW;
+  const int r1 = a.pool ? 2 * (((p_end - 1) >> 2) / pool_w) + 1 : (p_end - 1) / a.OW;
   const int ih0 = r0 * a.sh - a.pad_t;
   const int rows_needed = (r1 - r0) * a.sh + (a.kh - 1) * a.dh + 1;
 
@@ -145,7 +149,13 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(O
       n_ptw = i + 1;
       int p = p0 + pt * 32 + frag_row;
       p = min(p, hw - 1);
-      const int oh = p / a.OW, ow = p - oh * a.OW;
+      int oh = p / a.OW, ow = p - oh * a.OW;
+      if (a.pool) {
+        const int q = p >> 2, e = p & 3;
+        const int qh = q / pool_w, qw = q - qh * pool_w;
+        oh = 2 * qh + (e >> 1);
+        ow = 2 * qw + (e & 1);
+      }
       a_base[i] = ((oh - r0) * a.sh * a.iwt + ow * a.sw) * a.pix_stride;
     }
   }
@@ -391,6 +401,13 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(O
       for (int g = 0; g < 4; ++g) {
         const int pl = pt * 32 + 8 * g + 4 * frag_half;
         const v4i s4 = *reinterpret_cast<const v4i*>(sx_lds + pl);
+        if (a.pool) {
+          // requantization is monotone: the window's largest accumulator gives its largest code
+          const int m = max(max(acc[i][j][g * 4] - s4[0], acc[i][j][g * 4 + 1] - s4[1]),
+                            max(acc[i][j][g * 4 + 2] - s4[2], acc[i][j][g * 4 + 3] - s4[3]));
+          out_tile[ocl * a.out_stride + (pl >> 2)] = static_cast<int8_t>(Requant8<RQ>(m + bias, q, a.out_zp, lo, hi));
+          continue;
+        }
         int r4[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) r4[e] = Requant8<RQ>(acc[i][j][g * 4 + e] + (bias - s4[e]), q, a.out_zp, lo, hi);
@@ -399,19 +416,21 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(O
     }
   }
   __syncthreads();
-  const int valid = p_end - p0;
+  // what leaves: the tile's pixels, or its pooled pixels (a quarter as many)
+  const int valid = a.pool ? (p_end - p0) >> 2 : p_end - p0;
+  const int hw_y = a.pool ? hw >> 2 : hw;
   const int oc_n = min(a.oct, a.OC - oc0);
-  uint8_t* ybase = a.y + (static_cast<size_t>(n) * a.OC + oc0) * hw + p0;
-  if ((hw & 3) == 0) {
-    const int per_row = valid >> 2;  // p0 and hw are multiples of 4: whole dwords
+  uint8_t* ybase = a.y + (static_cast<size_t>(n) * a.OC + oc0) * hw_y + (a.pool ? p0 >> 2 : p0);
+  if ((hw_y & 3) == 0 && (valid & 3) == 0) {
+    const int per_row = valid >> 2;  // the tile's first pixel and the plane are multiples of 4: whole dwords
     for (int o = wave; o < oc_n; o += 4)
       for (int dwi = lane; dwi < per_row; dwi += 64)
-        *reinterpret_cast<uint32_t*>(ybase + static_cast<size_t>(o) * hw + dwi * 4) =
+        *reinterpret_cast<uint32_t*>(ybase + static_cast<size_t>(o) * hw_y + dwi * 4) =
             *reinterpret_cast<const uint32_t*>(out_tile + o * a.out_stride + dwi * 4);
   } else {
     for (int o = wave; o < oc_n; o += 4)
       for (int pi = lane; pi < valid; pi += 64)
-        ybase[static_cast<size_t>(o) * hw + pi] = static_cast<uint8_t>(out_tile[o * a.out_stride + pi]);
+        ybase[static_cast<size_t>(o) * hw_y + pi] = static_cast<uint8_t>(out_tile[o * a.out_stride + pi]);
   }
 }
 
@@ -842,10 +861,16 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   a.PT = a.P / 32;
   a.tiles_per_image = (hw + a.P - 1) / a.P;
   // halo extent: the most output rows any tile touches
+  a.pool = op->fused_pool;  // (the caller has checked the pooling: 2 x 2, stride 2, even output extents)
   int max_rows = 1;
   for (int t = 0; t < a.tiles_per_image; ++t) {
     const int p0 = t * a.P, pe = std::min(p0 + a.P, hw);
-    max_rows = std::max(max_rows, (pe - 1) / a.OW - p0 / a.OW + 1);
+    if (a.pool) {  // pixels in pooling order: pairs of rows
+      const int pw = a.OW / 2;
+      max_rows = std::max(max_rows, 2 * (((pe - 1) / 4) / pw - (p0 / 4) / pw + 1));
+    } else {
+      max_rows = std::max(max_rows, (pe - 1) / a.OW - p0 / a.OW + 1);
+    }
   }
   a.iht = (max_rows - 1) * a.sh + (a.kh - 1) * a.dh + 1;
   a.iwt = std::max((a.OW - 1) * a.sw + (a.kw - 1) * a.dw + 1, 1);
@@ -981,6 +1006,7 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
 
   // ---- the persistent variant, where it applies ------------------------------------------------
   do {
+    if (a.pool) break;  // the pooled epilogue exists in the one-tile-per-workgroup kernel
     if (const char* f = getenv("TVX_IGEMM_PERSIST")) if (atoi(f) == 0) break;  // tuning aid
     if (a.groups != 1 || a.cp != a.C || (a.cpc & 1) || oc_blocks != 1 || ot != 2 || (a.W & 3)) break;  // two output-channel tiles
     const int ksteps = taps * a.cpc / 2;
@@ -1060,7 +1086,7 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   } while (false);
   op->host_blob.assign(reinterpret_cast<const uint8_t*>(&plan), reinterpret_cast<const uint8_t*>(&plan) + sizeof(plan));
   op->run = ConvIgemmRun;
-  op->kernel_name = plan.persist_ksteps ? "conv2d_igemm_i8_persistent" : "conv2d_igemm_i8";
+  op->kernel_name = plan.persist_ksteps ? "conv2d_igemm_i8_persistent" : (a.pool ? "conv2d_igemm_maxpool_i8" : "conv2d_igemm_i8");
   return TVX_OK;
 }
 

@@ -50,6 +50,7 @@ struct ImArgs {
   int offs[64];
   int rows;              // row mode: C * Kh
   int total_bytes;       // row mode: size of the input tensor (< 2^31)
+  int pool;              // 1: a 2 x 2 / stride-2 max pooling rides on the epilogue (the result has OH / 2 x OW / 2 pixels)
 };
 
 // KW: 0 = any window, one byte load per tap; 3 / 5 = row mode for kernels three / five taps wide
@@ -88,7 +89,15 @@ __global__ void __launch_bounds__(kThreads) ConvIm2colKernel(ImArgs a) {
   int sx = 0;
   {
     const int p = min(p0 + tid, hw - 1);  // threads past the end redo the last pixel; nobody reads their row
-    const int oh = p / a.OW, ow = p - oh * a.OW;
+    int oh = p / a.OW, ow = p - oh * a.OW;
+    if (a.pool) {
+      // pixels in pooling order: four consecutive ones are a 2 x 2 window (row-major), windows row-major over
+      // the pooled image - the four accumulators a lane holds per quad then are one pooled pixel's candidates
+      const int q = p >> 2, e = p & 3, pw = a.OW >> 1;
+      const int qh = q / pw, qw = q - qh * pw;
+      oh = 2 * qh + (e >> 1);
+      ow = 2 * qw + (e & 1);
+    }
     const int ih0 = oh * a.sh - a.pad_t, iw0 = ow * a.sw - a.pad_l;
     const uint8_t* img = a.x + static_cast<size_t>(n) * a.C * a.H * a.W;
     const int origin = ih0 * a.W + iw0;  // may be negative; only added to offsets of taps inside the image
@@ -243,6 +252,13 @@ __global__ void __launch_bounds__(kThreads) ConvIm2colKernel(ImArgs a) {
       for (int g = 0; g < 4; ++g) {
         const int pl = pt * 32 + 8 * g + 4 * frag_half;
         const v4i s4 = *reinterpret_cast<const v4i*>(sx_lds + pl);
+        if (a.pool) {
+          // requantization is monotone: the window's largest accumulator gives its largest code
+          const int m = max(max(acc[i][j][g * 4] - s4[0], acc[i][j][g * 4 + 1] - s4[1]),
+                            max(acc[i][j][g * 4 + 2] - s4[2], acc[i][j][g * 4 + 3] - s4[3]));
+          out_tile[ocl * a.out_stride + (pl >> 2)] = static_cast<int8_t>(Requant8<RQ>(m + bias, q, a.out_zp, lo, hi));
+          continue;
+        }
         int r4[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) r4[e] = Requant8<RQ>(acc[i][j][g * 4 + e] + (bias - s4[e]), q, a.out_zp, lo, hi);
@@ -251,17 +267,19 @@ __global__ void __launch_bounds__(kThreads) ConvIm2colKernel(ImArgs a) {
     }
   }
   __syncthreads();
-  uint8_t* ybase = a.y + static_cast<size_t>(n) * a.OC * hw + p0;
-  if ((hw & 3) == 0) {
-    const int per_row = valid >> 2;  // p0 and hw are multiples of 4: whole dwords
+  // what leaves: the tile's pixels, or its pooled pixels (a quarter as many)
+  const int hw_y = a.pool ? hw >> 2 : hw, valid_y = a.pool ? valid >> 2 : valid;
+  uint8_t* ybase = a.y + static_cast<size_t>(n) * a.OC * hw_y + (a.pool ? p0 >> 2 : p0);
+  if ((hw_y & 3) == 0) {
+    const int per_row = valid_y >> 2;  // the tile's first pixel and the plane are multiples of 4: whole dwords
     for (int o = wave; o < a.OC; o += 4)
       for (int dwi = lane; dwi < per_row; dwi += 64)
-        *reinterpret_cast<uint32_t*>(ybase + static_cast<size_t>(o) * hw + dwi * 4) =
+        *reinterpret_cast<uint32_t*>(ybase + static_cast<size_t>(o) * hw_y + dwi * 4) =
             *reinterpret_cast<const uint32_t*>(out_tile + o * a.out_stride + dwi * 4);
   } else {
     for (int o = wave; o < a.OC; o += 4)
-      for (int pi = lane; pi < valid; pi += 64)
-        ybase[static_cast<size_t>(o) * hw + pi] = static_cast<uint8_t>(out_tile[o * a.out_stride + pi]);
+      for (int pi = lane; pi < valid_y; pi += 64)
+        ybase[static_cast<size_t>(o) * hw_y + pi] = static_cast<uint8_t>(out_tile[o * a.out_stride + pi]);
   }
 }
 
@@ -330,6 +348,7 @@ int ConvIm2colSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, co
   a.pad_fill = zxs & 0xff;
   a.zws = zws;
   a.out_zp = d->out_zp; a.lo = op->act_lo; a.hi = op->act_hi;
+  a.pool = op->fused_pool;  // (the caller has checked the pooling: 2 x 2, stride 2, even output extents)
   a.out_stride = ((kPixels / 4) | 1) * 4;
   // LDS: window sums and tables first; A rows + weights behind them are reused as the staging tile
   a.off_sx = 0;
@@ -398,7 +417,7 @@ int ConvIm2colSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, co
   plan.grid = dim3(static_cast<unsigned>((hw + kPixels - 1) / kPixels), static_cast<unsigned>(d->batch));
   op->host_blob.assign(reinterpret_cast<const uint8_t*>(&plan), reinterpret_cast<const uint8_t*>(&plan) + sizeof(plan));
   op->run = ConvIm2colRun;
-  op->kernel_name = "conv2d_im2col_i8";
+  op->kernel_name = op->fused_pool ? "conv2d_im2col_maxpool_i8" : "conv2d_im2col_i8";
   return TVX_OK;
 }
 

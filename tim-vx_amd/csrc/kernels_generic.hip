@@ -775,6 +775,114 @@ int SoftmaxRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t 
 }
 
 // ---------------------------------------------------------------------------
+// FullyConnected + Softmax over its (at most 16) outputs: one wavefront per input row. The lanes stride over K four
+// bytes at a time for every output (the row of x is loaded once), the partial sums meet in a butterfly, lane n
+// requantizes output n as the FullyConnected kernels do, and the Softmax runs across those lanes in the
+// arithmetic - and the order of additions - of SoftmaxRowKernel on the stored codes.
+// ---------------------------------------------------------------------------
+constexpr int kFcSmMaxN = 16;
+
+template <typename XT, typename WT>
+__global__ void __launch_bounds__(kBlock)
+FcSoftmaxKernel(FcArgs a, float beta, float sm_scale, const XT* __restrict__ x, const WT* __restrict__ w,
+                const int32_t* __restrict__ bias, const int32_t* __restrict__ mult,
+                const int32_t* __restrict__ shift, float* __restrict__ y) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+  if (row >= a.m) return;  // whole wavefronts
+  const XT* xp = x + static_cast<uint64_t>(row) * a.k;
+  // this lane's table entries travel with the rows
+  const int nl = min(lane, a.n - 1);
+  const int my_bias = bias ? bias[nl] : 0, my_mult = mult[nl], my_shift = shift[nl];
+  int32_t acc[kFcSmMaxN];
+#pragma unroll
+  for (int n = 0; n < kFcSmMaxN; ++n) acc[n] = 0;
+  const int k4 = a.k & ~3;
+  for (int k = lane * 4; k < k4; k += 256) {
+    uint32_t xv;
+    __builtin_memcpy(&xv, xp + k, 4);  // rows start at any byte: unaligned dwords
+    int32_t xe[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) xe[b] = static_cast<int32_t>(static_cast<XT>(xv >> (8 * b))) - a.in_zp;
+#pragma unroll
+    for (int n = 0; n < kFcSmMaxN; ++n) {
+      if (n < a.n) {  // uniform
+        uint32_t wv;
+        __builtin_memcpy(&wv, w + static_cast<uint64_t>(n) * a.k + k, 4);
+#pragma unroll
+        for (int b = 0; b < 4; ++b) acc[n] += xe[b] * (static_cast<int32_t>(static_cast<WT>(wv >> (8 * b))) - a.w_zp);
+      }
+    }
+  }
+  if (k4 + lane < a.k) {
+    const int32_t xe = static_cast<int32_t>(xp[k4 + lane]) - a.in_zp;
+#pragma unroll
+    for (int n = 0; n < kFcSmMaxN; ++n)
+      if (n < a.n) acc[n] += xe * (static_cast<int32_t>(w[static_cast<uint64_t>(n) * a.k + k4 + lane]) - a.w_zp);
+  }
+  int32_t mine = 0;  // output `lane` of the row
+#pragma unroll
+  for (int n = 0; n < kFcSmMaxN; ++n) {
+    if (n < a.n) {
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) acc[n] += __shfl_xor(acc[n], off);
+      if (lane == n) mine = acc[n];
+    }
+  }
+  const int code = RequantClamp(mine + my_bias, my_mult, my_shift, a.out_zp, a.lo, a.hi);
+  // ---- Softmax over lanes 0 .. n-1 ----
+  const bool live = lane < a.n;
+  const float v = live ? sm_scale * static_cast<float>(code - a.out_zp) : -INFINITY;
+  float mx = v;
+#pragma unroll
+  for (int o = 8; o; o >>= 1) {
+    const float other = __shfl_xor(mx, o, 64);
+    mx = other > mx ? other : mx;
+  }
+  const float e = live ? expf(beta * (v - mx)) : 0.f;
+  float ee[kFcSmMaxN];
+#pragma unroll
+  for (int i = 0; i < kFcSmMaxN; ++i) ee[i] = __shfl(e, i, 64);
+  float sum;
+  if (a.n <= 4) {  // SoftmaxRowKernel with one lane per row: in index order
+    sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sum += ee[i];
+  } else {  // ... with four lanes per row: lane l sums elements l, l + 4, ..., the lanes meet in a butterfly
+    float part[4];
+#pragma unroll
+    for (int l = 0; l < 4; ++l) {
+      part[l] = 0.f;
+#pragma unroll
+      for (int j = 0; j < kFcSmMaxN / 4; ++j) part[l] += ee[l + 4 * j];
+    }
+    sum = (part[0] + part[2]) + (part[1] + part[3]);
+  }
+  if (live) y[static_cast<uint64_t>(row) * a.n + lane] = e / sum;
+}
+
+int FcSoftmaxRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
+  const tvx_fc_desc& d = op->fc;
+  FcArgs a{static_cast<int>(d.m), static_cast<int>(d.k), static_cast<int>(d.n), d.in_zp, op->w_zp,
+           d.out_zp, op->act_lo, op->act_hi, d.activation};
+  const dim3 grid((d.m + kBlock / 64 - 1) / (kBlock / 64)), block(kBlock);
+  const int32_t* bias = op->bias.as<int32_t>();
+  const int32_t *mu = op->mult.as<int32_t>(), *sh = op->shift.as<int32_t>();
+  float* y = static_cast<float*>(out);
+  if (d.in_dtype == TVX_U8 && d.w_dtype == TVX_U8)
+    hipLaunchKernelGGL((FcSoftmaxKernel<uint8_t, uint8_t>), grid, block, 0, st, a, op->sm.beta, op->sm.in_scale,
+                       static_cast<const uint8_t*>(in0), op->weights.as<uint8_t>(), bias, mu, sh, y);
+  else if (d.in_dtype == TVX_U8)
+    hipLaunchKernelGGL((FcSoftmaxKernel<uint8_t, int8_t>), grid, block, 0, st, a, op->sm.beta, op->sm.in_scale,
+                       static_cast<const uint8_t*>(in0), op->weights.as<int8_t>(), bias, mu, sh, y);
+  else
+    hipLaunchKernelGGL((FcSoftmaxKernel<int8_t, int8_t>), grid, block, 0, st, a, op->sm.beta, op->sm.in_scale,
+                       static_cast<const int8_t*>(in0), op->weights.as<int8_t>(), bias, mu, sh, y);
+  TVX_HIP_CHECK(hipGetLastError());
+  return TVX_OK;
+}
+
+// ---------------------------------------------------------------------------
 // Transpose: one thread per output element; output dimension i walks input dimension perm[i]
 // ---------------------------------------------------------------------------
 struct TransposeArgs {
@@ -908,6 +1016,17 @@ int FcGenericSetup(tvx_op* op, const tvx_fc_desc* d, const void* w, const void* 
   if (s != TVX_OK) return s;
   op->run = FcGenericRun;
   op->kernel_name = "fc_generic";
+  return TVX_OK;
+}
+
+// FullyConnected + Softmax (the caller has checked that the Softmax reads the FullyConnected's codes along its outputs)
+int FcSoftmaxSetup(tvx_op* op, const tvx_fc_desc* d, const void* w, const void* b) {
+  if (!op->quantized || !w || d->n > static_cast<uint32_t>(kFcSmMaxN) || d->m > 0x7fffffffu / 64) return TVX_E_UNSUPPORTED;
+  if (d->in_dtype == TVX_I8 && d->w_dtype != TVX_I8) return TVX_E_UNSUPPORTED;
+  int s = UploadWeightsAndBias(op, w, static_cast<size_t>(d->k) * d->n, b, static_cast<size_t>(d->n) * 4);
+  if (s != TVX_OK) return s;
+  op->run = FcSoftmaxRun;
+  op->kernel_name = "fc_softmax_i8";
   return TVX_OK;
 }
 

@@ -321,10 +321,10 @@ static int NoGpu() {
   return TVX_OK;
 }
 
-int tvx_conv2d_create(const tvx_conv2d_desc* d, const void* weights_host,
-                      const void* bias_host, tvx_op** out) {
-  if (!d || !out) return SetError(TVX_E_INVALID, "tvx_conv2d_create: null argument");
-  *out = nullptr;
+// tvx_conv2d_create, and (fused_pool) the convolution half of tvx_conv2d_pool_create: then only the kernels with
+// a pooled epilogue are asked.
+static int CreateConv(const tvx_conv2d_desc* d, const void* weights_host, const void* bias_host, bool fused_pool,
+                      tvx_op** out) {
   if (!d->in_w || !d->in_h || !d->in_c || !d->batch || !d->k_w || !d->k_h || !d->out_w ||
       !d->out_h || !d->out_c || !d->stride_w || !d->stride_h || !d->dilation_w || !d->dilation_h)
     return SetError(TVX_E_INVALID, "tvx_conv2d_create: zero extent, stride or dilation");
@@ -349,6 +349,7 @@ int tvx_conv2d_create(const tvx_conv2d_desc* d, const void* weights_host,
   if (!op) return SetError(TVX_E_NOMEM, "tvx_conv2d_create: host allocation failed");
   op->kind = OP_CONV2D;
   op->conv = *d;
+  op->fused_pool = fused_pool ? 1 : 0;
   // one input channel per group is a depthwise convolution in other words: same weight image
   // ({k_w, k_h, 1, out_c} = {k_w, k_h, in_c * m, 1}), same channel map (oc / m), and the
   // depthwise kernels apply
@@ -371,13 +372,47 @@ int tvx_conv2d_create(const tvx_conv2d_desc* d, const void* weights_host,
     if (s != TVX_OK) { delete op; return s; }
   }
   s = TVX_E_UNSUPPORTED;
-  for (ConvSetupFn fn : ConvVariants()) {
-    s = fn(op, d, weights_host, bias_host);
-    if (s != TVX_E_UNSUPPORTED) break;
+  if (fused_pool) {
+    s = ConvIm2colSetup(op, d, weights_host, bias_host);
+    if (s == TVX_E_UNSUPPORTED) s = ConvIgemmSetup(op, d, weights_host, bias_host);
+  } else {
+    for (ConvSetupFn fn : ConvVariants()) {
+      s = fn(op, d, weights_host, bias_host);
+      if (s != TVX_E_UNSUPPORTED) break;
+    }
   }
   if (s != TVX_OK) { delete op; return s; }
   *out = op;
   return TVX_OK;
+}
+
+int tvx_conv2d_create(const tvx_conv2d_desc* d, const void* weights_host,
+                      const void* bias_host, tvx_op** out) {
+  if (!d || !out) return SetError(TVX_E_INVALID, "tvx_conv2d_create: null argument");
+  *out = nullptr;
+  return CreateConv(d, weights_host, bias_host, false, out);
+}
+
+int tvx_conv2d_pool_create(const tvx_conv2d_desc* d, const tvx_pool2d_desc* pool, const void* weights_host,
+                           const void* bias_host, tvx_op** out) {
+  if (!d || !pool || !out) return SetError(TVX_E_INVALID, "tvx_conv2d_pool_create: null argument");
+  *out = nullptr;
+  if (pool->in_w != d->out_w || pool->in_h != d->out_h || pool->channels != d->out_c || pool->batch != d->batch ||
+      pool->dtype != d->out_dtype)
+    return SetError(TVX_E_INVALID, "tvx_conv2d_pool_create: the pooling's input is not the convolution's output");
+  const bool fusable = IsQuant(d->in_dtype) && IsQuant(d->out_dtype) && weights_host && pool->pool_type == TVX_POOL_MAX &&
+                       pool->k_w == 2 && pool->k_h == 2 && pool->stride_w == 2 && pool->stride_h == 2 &&
+                       pool->pad_left == 0 && pool->pad_top == 0 && d->out_w % 2 == 0 && d->out_h % 2 == 0 &&
+                       pool->out_w == d->out_w / 2 && pool->out_h == d->out_h / 2 &&
+                       pool->in_scale == d->out_scale && pool->in_zp == d->out_zp &&
+                       pool->out_scale == d->out_scale && pool->out_zp == d->out_zp;
+  if (!fusable)
+    return SetError(TVX_E_UNSUPPORTED, "tvx_conv2d_pool_create: quantized convolution with constant weights and a 2 x 2 / stride-2 "
+                    "max pooling without padding that keeps the quantization are what is fused");
+  const int s = CreateConv(d, weights_host, bias_host, true, out);
+  if (s == TVX_E_UNSUPPORTED) return SetError(TVX_E_UNSUPPORTED, "tvx_conv2d_pool_create: no fused kernel for this convolution");
+  if (s == TVX_OK) (*out)->pool = *pool;
+  return s;
 }
 
 int tvx_conv2d_add_create(const tvx_conv2d_desc* d, const tvx_eltwise_desc* add, int conv_operand,
@@ -636,6 +671,44 @@ int tvx_fully_connected_create(const tvx_fc_desc* d, const void* weights_host,
     if (s != TVX_E_UNSUPPORTED) break;
   }
   if (s != TVX_OK) { delete op; return s; }
+  *out = op;
+  return TVX_OK;
+}
+
+int tvx_fully_connected_softmax_create(const tvx_fc_desc* d, const tvx_softmax_desc* sm, const void* weights_host,
+                                       const void* bias_host, tvx_op** out) {
+  if (!d || !sm || !out) return SetError(TVX_E_INVALID, "tvx_fully_connected_softmax_create: null argument");
+  *out = nullptr;
+  if (!d->m || !d->k || !d->n) return SetError(TVX_E_INVALID, "tvx_fully_connected_softmax_create: zero extent");
+  if (sm->channels != d->n || sm->rows != d->m || sm->inner > 1 || sm->in_dtype != d->out_dtype)
+    return SetError(TVX_E_INVALID, "tvx_fully_connected_softmax_create: the Softmax does not run along the FullyConnected's outputs");
+  if (!IsQuant(d->in_dtype) || !IsQuant(d->out_dtype) || !weights_host || sm->in_scale != d->out_scale || sm->in_zp != d->out_zp)
+    return SetError(TVX_E_UNSUPPORTED, "tvx_fully_connected_softmax_create: quantized tensors, constant weights and one quantization "
+                    "of the intermediate codes are what is fused");
+  int s = CheckOperandTypes(d->in_dtype, d->w_dtype, d->out_dtype, "tvx_fully_connected_softmax_create");
+  if (s == TVX_OK) s = CheckConvZeroPoints(d->in_dtype, d->in_zp, d->w_dtype, d->w_zp, d->w_scales != nullptr,
+                                           d->out_dtype, d->out_zp, "tvx_fully_connected_softmax_create");
+  if (s != TVX_OK) return s;
+  if ((s = NoGpu()) != TVX_OK) return s;
+  tvx_op* op = new (std::nothrow) tvx_op();
+  if (!op) return SetError(TVX_E_NOMEM, "tvx_fully_connected_softmax_create: host allocation failed");
+  op->kind = OP_FC;
+  op->fc = *d;
+  op->fc.w_scales = nullptr;
+  op->sm = *sm;
+  op->fused_softmax = 1;
+  op->quantized = true;
+  op->has_const_weights = true;
+  op->w_zp = d->w_scales ? 0 : d->w_zp;
+  s = BuildRequantTables(d->n, d->in_scale, d->w_scale, d->w_scales, d->out_scale, &op->h_mult, &op->h_shift);
+  if (s == TVX_OK) s = op->mult.Upload(op->h_mult.data(), op->h_mult.size() * 4);
+  if (s == TVX_OK) s = op->shift.Upload(op->h_shift.data(), op->h_shift.size() * 4);
+  ActRange(d->out_dtype, d->out_scale, d->out_zp, d->activation, &op->act_lo, &op->act_hi);
+  if (s == TVX_OK) s = FcSoftmaxSetup(op, d, weights_host, bias_host);
+  if (s != TVX_OK) {
+    delete op;
+    return s == TVX_E_UNSUPPORTED ? SetError(TVX_E_UNSUPPORTED, "tvx_fully_connected_softmax_create: no fused kernel for this layer") : s;
+  }
   *out = op;
   return TVX_OK;
 }

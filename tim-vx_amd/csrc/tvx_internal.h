@@ -48,6 +48,8 @@ struct tvx_op {
   int (*run)(tvx_op*, const void* in0, const void* in1, void* out, hipStream_t) = nullptr;
   const void* bias_at_run = nullptr;  // set by tvx_op_run3 for the duration of one enqueue
   int fused_add = 0;  // Conv2d + Add in one kernel: 1 = the convolution is the Add's first operand, 2 = its second (elt holds the Add)
+  int fused_pool = 0;  // Conv2d + 2x2 / stride-2 max pooling in one kernel: the result has a quarter of conv's output pixels
+  int fused_softmax = 0;  // FullyConnected + Softmax over its outputs in one kernel (sm holds the Softmax): fp32 result
 
   tvx_conv2d_desc conv{};
   tvx_fc_desc fc{};

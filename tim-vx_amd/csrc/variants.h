@@ -68,6 +68,8 @@ int ConvGemmSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 // generic (kernels_generic.hip)
 int ConvGenericSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 int FcGenericSetup(tvx_op*, const tvx_fc_desc*, const void*, const void*);
+// FullyConnected with at most 16 outputs + the Softmax over them, a wavefront per row (kernels_generic.hip)
+int FcSoftmaxSetup(tvx_op*, const tvx_fc_desc*, const void*, const void*);
 int PoolGenericSetup(tvx_op*);
 // quantized pooling, windows two or three taps wide, planes staged through LDS (pool2d_i8.hip)
 int PoolRowsSetup(tvx_op*);

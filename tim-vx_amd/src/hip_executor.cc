@@ -188,6 +188,28 @@ class HipExecutor : public Executor {
         fused_block[op] = dw;
       }
     }
+    // ---- convolution -> 2x2 max pooling, FullyConnected -> Softmax: a TRANSIENT result with that one reader may
+    // never reach memory (whether a kernel takes the pair is decided when the operators are created)
+    std::map<Operation*, Operation*> fused_pool, fused_softmax;
+    if (!std::getenv("TVX_NO_POOL_FUSION")) {  // tuning aid
+      for (Operation* op : graph->sorted_ops_) {
+        OpImpl* im = op->impl().get();
+        const bool conv = im->kind_ == OpKind::CONV2D && !im->attrs_.conv_1d && im->attrs_.multiplier == 0;
+        if (!conv && im->kind_ != OpKind::FCL) continue;
+        if (fused_add.count(op) || fused_dwpw.count(op) || fused_block.count(op)) continue;
+        auto fa = fused_act.find(op);
+        auto mid = fa != fused_act.end() ? fa->second->impl()->outputs_tensor_[0] : im->outputs_tensor_[0];
+        if (!(mid->GetSpec().attr_ & TensorAttribute::TRANSIENT)) continue;
+        auto consumers = graph->GetConsumersOp(mid);
+        if (consumers.size() != 1) continue;
+        OpImpl* next = consumers[0]->impl().get();
+        if (next->inputs_tensor_[0] != mid) continue;
+        if (conv && next->kind_ == OpKind::POOL && !next->attrs_.pool_1d) fused_pool[op] = consumers[0].get();
+        if (!conv && next->kind_ == OpKind::SOFTMAX) fused_softmax[op] = consumers[0].get();
+      }
+      // a pointwise convolution folded into the depthwise one in front of it is not there to take a pooling
+      for (auto& kv : fused_dwpw) fused_pool.erase(kv.second);
+    }
     // ---- device storage: one buffer per tensor, Reshape outputs alias their input --
     for (Operation* op : graph->sorted_ops_) {
       OpImpl* im = op->impl().get();
@@ -275,6 +297,16 @@ class HipExecutor : public Executor {
               break;
             }
           }
+          auto fp = fused_pool.find(op);
+          if (fp != fused_pool.end()) {
+            bool both = false;
+            ok = AddConvPool(im, out, act, fp->second->impl().get(), &both);
+            if (!ok) break;
+            if (both) {
+              skipped[fp->second] = true;
+              break;
+            }
+          }
           auto fa = fused_add.find(op);
           bool fused = false;
           if (fa != fused_add.end()) {
@@ -284,7 +316,16 @@ class HipExecutor : public Executor {
           if (ok && !fused) ok = AddConv(im, out, act);
           break;
         }
-        case OpKind::FCL: ok = AddFc(im, out, act); break;
+        case OpKind::FCL: {
+          bool both = false;
+          auto fs = fused_softmax.find(op);
+          if (fs != fused_softmax.end()) {
+            ok = AddFcSoftmax(im, out, act, fs->second->impl().get(), &both);
+            if (both) skipped[fs->second] = true;
+          }
+          if (ok && !both) ok = AddFc(im, out, act);
+          break;
+        }
         case OpKind::POOL: ok = AddPool(im, out); break;
         case OpKind::RELU: ok = AddActivation(im, out, TVX_ACT_RELU); break;
         case OpKind::RELU6: ok = AddActivation(im, out, TVX_ACT_RELU6); break;
@@ -565,11 +606,9 @@ class HipExecutor : public Executor {
     return true;
   }
 
-  bool AddFc(OpImpl* im, TensorImpl* out, int act) {
+  static tvx_fc_desc FcDesc(OpImpl* im, TensorImpl* out, int act) {
     TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
     TensorImpl* w = static_cast<TensorImpl*>(im->inputs_tensor_[1].get());
-    TensorImpl* b = im->inputs_tensor_.size() > 2 && !im->inputs_tensor_[2]->IsPlaceHolder()
-                        ? static_cast<TensorImpl*>(im->inputs_tensor_[2].get()) : nullptr;
     const ShapeType& xs = x->spec_.shape_;
     uint64_t k = 1, m = 1;
     for (uint32_t i = 0; i <= im->attrs_.axis; ++i) k *= xs[i];
@@ -585,6 +624,15 @@ class HipExecutor : public Executor {
     WeightQuant(w->spec_, &d.w_scale, &d.w_zp, &d.w_scales);
     d.out_scale = ScaleOf(out->spec_); d.out_zp = ZpOf(out->spec_);
     d.activation = act;
+    return d;
+  }
+
+  bool AddFc(OpImpl* im, TensorImpl* out, int act) {
+    TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
+    TensorImpl* w = static_cast<TensorImpl*>(im->inputs_tensor_[1].get());
+    TensorImpl* b = im->inputs_tensor_.size() > 2 && !im->inputs_tensor_[2]->IsPlaceHolder()
+                        ? static_cast<TensorImpl*>(im->inputs_tensor_[2].get()) : nullptr;
+    const tvx_fc_desc d = FcDesc(im, out, act);
     const bool bias_at_run = b && !b->IsConstTensor();  // as for Conv2d
     const bool const_w = w->IsConstTensor() && w->HostData() && !bias_at_run;
     tvx_op* op = nullptr;
@@ -594,8 +642,51 @@ class HipExecutor : public Executor {
     return true;
   }
 
-  bool AddPool(OpImpl* im, TensorImpl* out) {
+  // A FullyConnected layer and the Softmax that alone reads its codes as one operator (tvx_fully_connected_softmax_create).
+  // *fused says whether a kernel took the pair; if not, nothing has been added.
+  bool AddFcSoftmax(OpImpl* im, TensorImpl* out, int act, OpImpl* sm_im, bool* fused) {
+    *fused = false;
     TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
+    TensorImpl* w = static_cast<TensorImpl*>(im->inputs_tensor_[1].get());
+    TensorImpl* b = im->inputs_tensor_.size() > 2 && !im->inputs_tensor_[2]->IsPlaceHolder()
+                        ? static_cast<TensorImpl*>(im->inputs_tensor_[2].get()) : nullptr;
+    TensorImpl* y = static_cast<TensorImpl*>(sm_im->outputs_tensor_[0].get());
+    if (!w->IsConstTensor() || !w->HostData() || (b && (!b->IsConstTensor() || !b->HostData()))) return true;
+    tvx_softmax_desc sd{};
+    if (y->spec_.datatype_ != DataType::FLOAT32 || !SoftmaxDesc(sm_im, out, &sd)) return true;
+    const tvx_fc_desc d = FcDesc(im, out, act);
+    if (sd.inner > 1 || sd.channels != d.n || sd.rows != d.m) return true;
+    tvx_op* op = nullptr;
+    const int st = tvx_fully_connected_softmax_create(&d, &sd, w->HostData(), b ? b->HostData() : nullptr, &op);
+    if (st == TVX_E_UNSUPPORTED) return true;
+    if (st != TVX_OK) return Fail("tvx_fully_connected_softmax_create");
+    *fused = true;
+    Push(op, im, x, nullptr, y);
+    return true;
+  }
+
+  // A convolution and the pooling that alone reads its result as one operator (tvx_conv2d_pool_create).
+  bool AddConvPool(OpImpl* im, TensorImpl* out, int act, OpImpl* pool_im, bool* fused) {
+    *fused = false;
+    TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
+    TensorImpl* w = static_cast<TensorImpl*>(im->inputs_tensor_[1].get());
+    TensorImpl* b = im->inputs_tensor_.size() > 2 && !im->inputs_tensor_[2]->IsPlaceHolder()
+                        ? static_cast<TensorImpl*>(im->inputs_tensor_[2].get()) : nullptr;
+    TensorImpl* y = static_cast<TensorImpl*>(pool_im->outputs_tensor_[0].get());
+    if (!w->IsConstTensor() || !w->HostData() || (b && (!b->IsConstTensor() || !b->HostData()))) return true;
+    if (out->spec_.datatype_ != y->spec_.datatype_) return true;
+    const tvx_conv2d_desc d = ConvDesc(im, out, act, false);
+    const tvx_pool2d_desc pd = PoolDesc(pool_im, out, y);
+    tvx_op* op = nullptr;
+    const int st = tvx_conv2d_pool_create(&d, &pd, w->HostData(), b ? b->HostData() : nullptr, &op);
+    if (st == TVX_E_UNSUPPORTED || st == TVX_E_INVALID) return true;  // (a pooling the fused form does not describe)
+    if (st != TVX_OK) return Fail("tvx_conv2d_pool_create");
+    *fused = true;
+    Push(op, im, x, nullptr, y);
+    return true;
+  }
+
+  static tvx_pool2d_desc PoolDesc(OpImpl* im, TensorImpl* x, TensorImpl* out) {
     const OpAttrs& a = im->attrs_;
     const ShapeType &xs = x->spec_.shape_, &os = out->spec_.shape_;
     tvx_pool2d_desc d{};
@@ -614,6 +705,12 @@ class HipExecutor : public Executor {
     d.dtype = DtypeCode(x->spec_.datatype_);
     d.in_scale = ScaleOf(x->spec_); d.in_zp = ZpOf(x->spec_);
     d.out_scale = ScaleOf(out->spec_); d.out_zp = ZpOf(out->spec_);
+    return d;
+  }
+
+  bool AddPool(OpImpl* im, TensorImpl* out) {
+    TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
+    const tvx_pool2d_desc d = PoolDesc(im, x, out);
     tvx_op* op = nullptr;
     if (tvx_pool2d_create(&d, &op) != TVX_OK) return Fail("tvx_pool2d_create");
     Push(op, im, x, nullptr, out);
@@ -657,24 +754,32 @@ class HipExecutor : public Executor {
     return true;
   }
 
-  bool AddSoftmax(OpImpl* im, TensorImpl* out) {
-    TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
+  // The Softmax `im` over tensor x as a descriptor; false when its axis lies outside the tensor.
+  static bool SoftmaxDesc(OpImpl* im, TensorImpl* x, tvx_softmax_desc* d) {
     const ShapeType& xs = x->spec_.shape_;
     const int32_t rank = static_cast<int32_t>(xs.size());
     int32_t axis = im->attrs_.sm_axis;
     if (axis < 0) axis += rank;  // negative axes count from the slowest dimension
-    if (axis < 0 || axis >= rank || out->spec_.datatype_ != DataType::FLOAT32) {
-      VSILOGE("SOFTMAX: axis %d of a rank-%d tensor with a FLOAT32 output is what is implemented", im->attrs_.sm_axis, rank);
+    if (axis < 0 || axis >= rank) return false;
+    *d = tvx_softmax_desc{};
+    d->channels = xs[axis];
+    d->inner = 1;
+    for (int32_t i = 0; i < axis; ++i) d->inner *= xs[i];
+    d->rows = static_cast<uint64_t>(x->spec_.GetElementNum()) / (d->channels * d->inner);
+    d->beta = im->attrs_.beta;
+    d->in_dtype = DtypeCode(x->spec_.datatype_);
+    d->in_scale = ScaleOf(x->spec_); d->in_zp = ZpOf(x->spec_);
+    return true;
+  }
+
+  bool AddSoftmax(OpImpl* im, TensorImpl* out) {
+    TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
+    tvx_softmax_desc d{};
+    if (out->spec_.datatype_ != DataType::FLOAT32 || !SoftmaxDesc(im, x, &d)) {
+      VSILOGE("SOFTMAX: axis %d of a rank-%zu tensor with a FLOAT32 output is what is implemented", im->attrs_.sm_axis,
+              x->spec_.shape_.size());
       return false;
     }
-    tvx_softmax_desc d{};
-    d.channels = xs[axis];
-    d.inner = 1;
-    for (int32_t i = 0; i < axis; ++i) d.inner *= xs[i];
-    d.rows = static_cast<uint64_t>(x->spec_.GetElementNum()) / (d.channels * d.inner);
-    d.beta = im->attrs_.beta;
-    d.in_dtype = DtypeCode(x->spec_.datatype_);
-    d.in_scale = ScaleOf(x->spec_); d.in_zp = ZpOf(x->spec_);
     tvx_op* op = nullptr;
     if (tvx_softmax_create(&d, &op) != TVX_OK) return Fail("tvx_softmax_create");
     Push(op, im, x, nullptr, out);
