@@ -328,8 +328,9 @@ def test_fully_connected_full_size_uint8_asymmetric(oracle):
 
 
 def test_fully_connected_full_size_int8_per_channel(oracle):
-    """M=8192, K=4096, N=4096 int8 per-channel: the whole problem on the GPU, a
-    seeded sample of 48 rows recomputed by the oracle, plus linearity in the bias."""
+    """M=8192, K=4096, N=4096 int8 per-channel: the whole problem on the GPU, a seeded sample of 48 rows recomputed
+    by the oracle - one in every one of the 32 tile rows (all output columns: every tile of the launch is
+    touched) and 16 anywhere -, plus independence of the rows."""
     m, k, n = 8192, 4096, 4096
     rng = np.random.default_rng(0x75)
     x = rng.integers(-128, 128, m * k, dtype=np.int8)
@@ -339,7 +340,8 @@ def test_fully_connected_full_size_int8_per_channel(oracle):
     kws = dict(k=k, n=n, in_dtype=1, w_dtype=1, out_dtype=1, in_q=(0.02, 0), w_q=(1.0, 0, ws),
                out_q=(0.05, 0))
     got = TC.gpu_fully_connected(x, w, b, m=m, want_kernel="fc_mfma_i8_256x256x128", **kws).reshape(m, n)
-    rows = np.sort(rng.choice(m, 48, replace=False))
+    rows = np.unique(np.concatenate([np.arange(32) * 256 + rng.integers(0, 256, 32), rng.choice(m, 16, replace=False)]))
+    assert set(rows // 256) == set(range(32))
     want = oracle.fully_connected(np.ascontiguousarray(x.reshape(m, k)[rows]).ravel(), w, b, m=len(rows), **kws)
     assert np.array_equal(got[rows], want.reshape(len(rows), n))
     assert len(np.unique(got)) > 100

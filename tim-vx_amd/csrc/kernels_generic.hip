@@ -193,10 +193,25 @@ FcQuantKernel(FcArgs a, const XT* __restrict__ x, const WT* __restrict__ w,
   y[idx] = static_cast<XT>(RequantClamp(acc, mult[n], shift[n], a.out_zp, a.lo, a.hi));
 }
 
-// One wavefront per output: the lanes stride over K four bytes at a time (consecutive lanes
-// read consecutive dwords of both rows) and the partial sums meet in a butterfly. For the
-// small FullyConnected layers at the end of a network - a few thousand outputs with a long
-// reduction - where one thread per output would walk its row alone.
+// (x - zx) . (w - zw) over the sixteen bytes of two vectors
+template <typename XT, typename WT>
+__device__ __forceinline__ int32_t Dot16(const uint4& xv, const uint4& wv, int in_zp, int w_zp) {
+  const uint32_t xd[4] = {xv.x, xv.y, xv.z, xv.w}, wd[4] = {wv.x, wv.y, wv.z, wv.w};
+  int32_t acc = 0;
+#pragma unroll
+  for (int d = 0; d < 4; ++d)
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+      acc += (static_cast<int32_t>(static_cast<XT>(xd[d] >> (8 * b))) - in_zp) *
+             (static_cast<int32_t>(static_cast<WT>(wd[d] >> (8 * b))) - w_zp);
+  return acc;
+}
+
+// One wavefront per output: the lanes stride over K sixteen bytes at a time (consecutive lanes
+// read consecutive chunks of both rows; rows start at any byte, the loads are unaligned) and the
+// partial sums meet in a butterfly. For the small FullyConnected layers at the end of a network -
+// a few thousand outputs with a long reduction - where one thread per output would walk its row
+// alone. A row of up to 1024 bytes is one round trip to memory.
 template <typename XT, typename WT>
 __global__ void __launch_bounds__(kBlock)
 FcQuantWaveKernel(FcArgs a, const XT* __restrict__ x, const WT* __restrict__ w,
@@ -210,20 +225,15 @@ FcQuantWaveKernel(FcArgs a, const XT* __restrict__ x, const WT* __restrict__ w,
   const XT* xp = x + m * a.k;
   const WT* wp = w + static_cast<uint64_t>(n) * a.k;
   int32_t acc = 0;
-  const int k4 = a.k & ~3;
-  for (int k = lane * 4; k < k4; k += 256) {
-    uint32_t xv, wv;
-    __builtin_memcpy(&xv, xp + k, 4);  // rows start at any byte: unaligned dwords
-    __builtin_memcpy(&wv, wp + k, 4);
-#pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      const int32_t xe = static_cast<int32_t>(static_cast<XT>(xv >> (8 * b)));
-      const int32_t we = static_cast<int32_t>(static_cast<WT>(wv >> (8 * b)));
-      acc += (xe - a.in_zp) * (we - a.w_zp);
-    }
+  const int k16 = a.k & ~15;
+  for (int k = lane * 16; k < k16; k += 1024) {
+    uint4 xv, wv;
+    __builtin_memcpy(&xv, xp + k, 16);
+    __builtin_memcpy(&wv, wp + k, 16);
+    acc += Dot16<XT, WT>(xv, wv, a.in_zp, a.w_zp);
   }
-  if (k4 + lane < a.k)
-    acc += (static_cast<int32_t>(xp[k4 + lane]) - a.in_zp) * (static_cast<int32_t>(wp[k4 + lane]) - a.w_zp);
+  if (k16 + lane < a.k)
+    acc += (static_cast<int32_t>(xp[k16 + lane]) - a.in_zp) * (static_cast<int32_t>(wp[k16 + lane]) - a.w_zp);
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
   if (lane == 0) {
@@ -775,7 +785,7 @@ int SoftmaxRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t 
 }
 
 // ---------------------------------------------------------------------------
-// FullyConnected + Softmax over its (at most 16) outputs: one wavefront per input row. The lanes stride over K four
+// FullyConnected + Softmax over its (at most 16) outputs: one wavefront per input row. The lanes stride over K sixteen
 // bytes at a time for every output (the row of x is loaded once), the partial sums meet in a butterfly, lane n
 // requantizes output n as the FullyConnected kernels do, and the Softmax runs across those lanes in the
 // arithmetic - and the order of additions - of SoftmaxRowKernel on the stored codes.
@@ -794,41 +804,47 @@ FcSoftmaxKernel(FcArgs a, float beta, float sm_scale, const XT* __restrict__ x, 
   // this lane's table entries travel with the rows
   const int nl = min(lane, a.n - 1);
   const int my_bias = bias ? bias[nl] : 0, my_mult = mult[nl], my_shift = shift[nl];
+  // Sixteen bytes of the row and of every weight row per lane and step; the loads stand under no branch
+  // (outputs past the last read the last row again, lanes past the row's end read its start and add nothing),
+  // so that all of a step travel together: a row of up to 1024 bytes is one round trip to memory.
   int32_t acc[kFcSmMaxN];
 #pragma unroll
   for (int n = 0; n < kFcSmMaxN; ++n) acc[n] = 0;
-  const int k4 = a.k & ~3;
-  for (int k = lane * 4; k < k4; k += 256) {
-    uint32_t xv;
-    __builtin_memcpy(&xv, xp + k, 4);  // rows start at any byte: unaligned dwords
-    int32_t xe[4];
+  const int k16 = a.k & ~15;
+  for (int k0 = 0; k0 < k16; k0 += 1024) {
+    const int k = k0 + lane * 16;
+    const bool ok = k < k16;
+    const int kk = ok ? k : 0;
+    uint4 xv, wv[kFcSmMaxN];
+    __builtin_memcpy(&xv, xp + kk, 16);
 #pragma unroll
-    for (int b = 0; b < 4; ++b) xe[b] = static_cast<int32_t>(static_cast<XT>(xv >> (8 * b))) - a.in_zp;
+    for (int n = 0; n < kFcSmMaxN; ++n) __builtin_memcpy(&wv[n], w + static_cast<uint64_t>(min(n, a.n - 1)) * a.k + kk, 16);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int n = 0; n < kFcSmMaxN; ++n) {
-      if (n < a.n) {  // uniform
-        uint32_t wv;
-        __builtin_memcpy(&wv, w + static_cast<uint64_t>(n) * a.k + k, 4);
-#pragma unroll
-        for (int b = 0; b < 4; ++b) acc[n] += xe[b] * (static_cast<int32_t>(static_cast<WT>(wv >> (8 * b))) - a.w_zp);
-      }
+      const int32_t d = Dot16<XT, WT>(xv, wv[n], a.in_zp, a.w_zp);
+      acc[n] += ok ? d : 0;
     }
   }
-  if (k4 + lane < a.k) {
-    const int32_t xe = static_cast<int32_t>(xp[k4 + lane]) - a.in_zp;
+  {
+    const bool ok = k16 + lane < a.k;
+    const int kk = ok ? k16 + lane : 0;
+    const int32_t xe = static_cast<int32_t>(xp[kk]) - a.in_zp;
+    int32_t we[kFcSmMaxN];
 #pragma unroll
-    for (int n = 0; n < kFcSmMaxN; ++n)
-      if (n < a.n) acc[n] += xe * (static_cast<int32_t>(w[static_cast<uint64_t>(n) * a.k + k4 + lane]) - a.w_zp);
+    for (int n = 0; n < kFcSmMaxN; ++n) we[n] = static_cast<int32_t>(w[static_cast<uint64_t>(min(n, a.n - 1)) * a.k + kk]) - a.w_zp;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int n = 0; n < kFcSmMaxN; ++n) acc[n] += ok ? xe * we[n] : 0;
   }
   int32_t mine = 0;  // output `lane` of the row
 #pragma unroll
-  for (int n = 0; n < kFcSmMaxN; ++n) {
-    if (n < a.n) {
+  for (int off = 32; off > 0; off >>= 1)
 #pragma unroll
-      for (int off = 32; off > 0; off >>= 1) acc[n] += __shfl_xor(acc[n], off);
-      if (lane == n) mine = acc[n];
-    }
-  }
+    for (int n = 0; n < kFcSmMaxN; ++n) acc[n] += __shfl_xor(acc[n], off);
+#pragma unroll
+  for (int n = 0; n < kFcSmMaxN; ++n)
+    if (lane == n) mine = acc[n];
   const int code = RequantClamp(mine + my_bias, my_mult, my_shift, a.out_zp, a.lo, a.hi);
   // ---- Softmax over lanes 0 .. n-1 ----
   const bool live = lane < a.n;

@@ -11,8 +11,8 @@
 // (v_mfma_i32_32x32x32_i8, requantized into a wavefront-private [channel][pixel] image), depthwise stencil on
 // that image (signed dot4 over byte windows, requantized and transposed into the projection's operand), and
 // the chunk's contribution to every output channel accumulated in registers. No barrier inside the walk: a
-// wavefront only reads what it wrote. At the end the four partial projections meet in LDS, one output tile at
-// a time, and the tile's owner requantizes, adds the residual and stores.
+// wavefront only reads what it wrote. At the end the partial projections meet in LDS by integer atomics and
+// every wavefront requantizes, adds the residual to and stores its share of the outputs.
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
@@ -26,8 +26,8 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / 64;
 constexpr int kMStride = 48;      // bytes per pixel row of the projection operand (32 channels + 16: bank spread)
-constexpr int kStageStride = 40;  // bytes per staged output-channel row of 32 pixels
 constexpr int kMaxCinSteps = 5;   // 32-channel steps of the expansion's reduction (160 input channels)
 
 struct MbArgs {
@@ -51,7 +51,7 @@ struct MbArgs {
   int xs;                          // bytes per pixel row of the expansion operand
   int ep;                          // bytes per channel row of the expanded image
   int off_wave, wave_bytes;        // LDS: the wavefronts' private areas (expanded image, then projection operand)
-  int off_red, off_stage;          // LDS (reused after the walk): partial sums, the owners' staging rows
+  int off_red;                     // LDS: the projection's sums over all wavefronts, [tile][register][lane] (zeroed at the start)
   // quantization
   int x_xor;                       // 0x80 for uint8 input
   int zp1, neg_zws1_4;             // expansion weights' zero point as a second MFMA
@@ -137,45 +137,7 @@ __global__ void __launch_bounds__(kThreads, (MO * NTMAX <= 5 ? 2 : 1)) MbConvKer
   uint8_t* e_w = lds + a.off_wave + wave * a.wave_bytes + 4;  // (+ 4: the byte in front of row 0 is read)
   uint8_t* m_w = lds + a.off_wave + wave * a.wave_bytes + 16 + 32 * a.ep;
 
-  // ---- the band's input rows as the expansion's operand: xin[halo pixel][channel], signed bytes ----
-  {
-    const int slots = a.mh * 32;
-    const int cin_pad = a.cin_steps * 32;
-    const size_t plane = static_cast<size_t>(a.H) * W;
-    const uint8_t* xn = a.x + static_cast<size_t>(n) * a.Cin * plane;
-    // (sixteen loads in flight per thread: one at a time, every byte would wait out a memory round trip)
-    constexpr int kBatch = 16;
-    for (int it0 = tid; it0 < slots * cin_pad; it0 += kThreads * kBatch) {
-      uint8_t v[kBatch];
-      int at[kBatch];
-#pragma unroll
-      for (int u = 0; u < kBatch; ++u) {
-        const int it = it0 + u * kThreads;
-        const int c = it / slots, p = it - c * slots;  // pixels fastest: a channel's rows are consecutive bytes
-        const int row = p / W, col = p - row * W;
-        const int ih = ir0 + row;
-        const bool live = it < slots * cin_pad && p < hp && c < a.Cin && ih >= 0 && ih < a.H;
-        v[u] = live ? xn[c * plane + ih * W + col] : static_cast<uint8_t>(a.x_xor);
-        at[u] = it < slots * cin_pad ? p * a.xs + c : -1;
-      }
-#pragma unroll
-      for (int u = 0; u < kBatch; ++u)
-        if (at[u] >= 0) xin[at[u]] = v[u] ^ static_cast<uint8_t>(a.x_xor);
-    }
-  }
-  __syncthreads();
-
   const int frow = lane & 31, fh = lane >> 5;
-  v16i acc_out[MO][NTMAX];
-#pragma unroll
-  for (int mo = 0; mo < MO; ++mo)
-#pragma unroll
-    for (int t = 0; t < NTMAX; ++t)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc_out[mo][t][r] = 0;
-  const v4i fz1 = {a.neg_zws1_4, a.neg_zws1_4, a.neg_zws1_4, a.neg_zws1_4};
-  const v4i fz3 = {a.neg_zws3_4, a.neg_zws3_4, a.neg_zws3_4, a.neg_zws3_4};
-
   // The expansion's operands of the next chunk (fragments, the lane's bias and requantization record) are fetched
   // while this one is computed; what the later phases need is fetched at the chunk's start and has arrived by then.
   struct ExpandOperands {
@@ -190,6 +152,61 @@ __global__ void __launch_bounds__(kThreads, (MO * NTMAX <= 5 ? 2 : 1)) MbConvKer
     o.bias1 = a.b1[c * 32 + frow];
     o.rq1 = a.q1[c * 32 + frow];
   };
+  ExpandOperands next;
+  fetch(wave, next);  // (on its way while the input rows are loaded)
+
+  // ---- the band's input rows as the expansion's operand: xin[halo pixel][channel], signed bytes ----
+  // A channel's halo rows are consecutive bytes of its plane. A thread takes four of them for four channels (dwords
+  // at any byte offset where all sixteen bytes exist, else byte by byte with zeros for what lies outside the image,
+  // the band or the channels), transposes, and stores four pixels' channel quads.
+  {
+    const int quads = a.mh * 8;                        // pixel quads of the halo tiles
+    const int units = a.cin_steps * 8 * quads;         // x channel quads
+    const int plane = a.H * W;
+    const uint8_t* xn = a.x + static_cast<size_t>(n) * a.Cin * plane;
+    const int live_lo = max(0, -ir0) * W, live_hi = min(a.IR, a.H - ir0) * W;  // the live bytes of a channel's halo rows
+    const uint32_t xor4 = static_cast<uint32_t>(a.x_xor) * 0x01010101u;
+    for (int unit = tid; unit < units; unit += kThreads) {
+      const int c4 = unit / quads, p0 = (unit - c4 * quads) * 4;
+      const int c = c4 * 4;
+      const int at = ir0 * W + p0;                     // byte offset in the plane (negative above the image)
+      uint32_t d[4];
+      if (p0 >= live_lo && p0 + 4 <= live_hi && c + 4 <= a.Cin) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) __builtin_memcpy(&d[j], xn + (c + j) * plane + at, 4);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) d[j] ^= xor4;
+      } else {
+        uint8_t b[4][4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const bool live = p0 + e >= live_lo && p0 + e < live_hi && c + j < a.Cin;
+            b[j][e] = live ? static_cast<uint8_t>(xn[(c + j) * plane + at + e] ^ a.x_xor) : uint8_t{0};
+          }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) d[j] = b[j][0] | b[j][1] << 8 | b[j][2] << 16 | static_cast<uint32_t>(b[j][3]) << 24;
+      }
+      uint32_t px[4];
+      Transpose4x4(d, px);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) *reinterpret_cast<uint32_t*>(xin + (p0 + i) * a.xs + c) = px[i];
+    }
+  }
+  for (int i = tid; i < a.nt * MO * 256; i += kThreads) reinterpret_cast<v4i*>(lds + a.off_red)[i] = v4i{0, 0, 0, 0};
+  __syncthreads();
+
+  v16i acc_out[MO][NTMAX];
+#pragma unroll
+  for (int mo = 0; mo < MO; ++mo)
+#pragma unroll
+    for (int t = 0; t < NTMAX; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc_out[mo][t][r] = 0;
+  const v4i fz1 = {a.neg_zws1_4, a.neg_zws1_4, a.neg_zws1_4, a.neg_zws1_4};
+  const v4i fz3 = {a.neg_zws3_4, a.neg_zws3_4, a.neg_zws3_4, a.neg_zws3_4};
+
   // one halo tile of the chunk: accumulate, requantize, store as [channel][halo pixel]
   auto expand_finish = [&](const v16i& acc, int mt, const v4i& rq1) {
 #pragma unroll
@@ -201,12 +218,10 @@ __global__ void __launch_bounds__(kThreads, (MO * NTMAX <= 5 ? 2 : 1)) MbConvKer
           PackBytes(v[0], v[1], v[2], v[3]) ^ static_cast<uint32_t>(a.e_xor4);
     }
   };
-  ExpandOperands next;
-  fetch(wave, next);
-  for (int chunk = wave; chunk < a.chunks; chunk += 4) {
+  for (int chunk = wave; chunk < a.chunks; chunk += kWaves) {
     const int ch = chunk * 32 + frow;  // this lane's expanded channel, in all three phases
     const ExpandOperands cur = next;
-    fetch(chunk + 4, next);
+    fetch(chunk + kWaves, next);
     const v4i dk = a.dwk[ch];
     const v4i rq2 = a.q2[ch];
     v4i w2f[NTMAX];
@@ -282,99 +297,76 @@ __global__ void __launch_bounds__(kThreads, (MO * NTMAX <= 5 ? 2 : 1)) MbConvKer
     }
     __builtin_amdgcn_wave_barrier();
   }
-  __syncthreads();  // the walk's LDS areas are free from here
-
-  // ---- the four partial projections meet, one output tile at a time; wavefront t % 4 owns tile t ----
+  // ---- the wavefronts' partial projections meet in LDS (integer atomics on a zeroed image laid out like the
+  // accumulators: [tile][register][lane]); then every wavefront finishes its share of the (output tile, pixel tile,
+  // register quad) units: requantize, add the residual, store. A unit is four pixels of each of 32 channels.
   int* red = reinterpret_cast<int*>(lds + a.off_red);
-  uint8_t* stage = lds + a.off_stage + wave * (MO * 32 * kStageStride);
   const size_t out_plane = static_cast<size_t>(a.OH) * OW;
+  const int units = a.nt * MO * 4;
+  constexpr int kMaxUnits = (NTMAX * MO * 4 + kWaves - 1) / kWaves;
+  // what the units need from memory is requested first: the sums then form under these loads
+  int bias3[kMaxUnits];
+  v4i rq3[kMaxUnits];
+  uint32_t resv[kMaxUnits];
+  size_t at[kMaxUnits];
+  int px0[kMaxUnits];
 #pragma unroll
-  for (int t = 0; t < NTMAX; ++t) {
-    if (t < a.nt) {
-      const int owner = t & 3;
-      int* buf = red + (t & 1) * (3 * MO * 1024);
-      if (wave != owner) {
-        const int slot = wave - (wave > owner ? 1 : 0);
+  for (int i = 0; i < kMaxUnits; ++i) {
+    const int u = min(wave + i * kWaves, units - 1);
+    const int t = u / (MO * 4), mo = (u >> 2) % MO, gq = u & 3;
+    const int oc = t * 32 + frow;
+    bias3[i] = a.b3[oc];
+    rq3[i] = a.q3[oc];
+    px0[i] = mo * 32 + 8 * gq + 4 * fh;
+    at[i] = (static_cast<size_t>(n) * a.Cout + oc) * out_plane + static_cast<size_t>(or0) * OW + px0[i];
+    resv[i] = 0;
+    if (ADD && oc < a.Cout) {
+      if (a.aligned4) {
+        if (px0[i] < po) resv[i] = *reinterpret_cast<const uint32_t*>(a.res + at[i]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (px0[i] + e < po) resv[i] |= static_cast<uint32_t>(a.res[at[i] + e]) << (8 * e);
+      }
+    }
+  }
+  if (wave < a.chunks) {  // (a wavefront that walked no chunk has nothing to add)
+#pragma unroll
+    for (int t = 0; t < NTMAX; ++t)
+      if (t < a.nt) {
 #pragma unroll
         for (int mo = 0; mo < MO; ++mo)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) buf[((slot * MO + mo) * 16 + r) * 64 + lane] = acc_out[mo][t][r];
+          for (int r = 0; r < 16; ++r)
+            __hip_atomic_fetch_add(red + ((t * MO + mo) * 16 + r) * 64 + lane, acc_out[mo][t][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       }
-      __syncthreads();
-      if (wave == owner) {
-        const int oc = t * 32 + frow;
-        const int bias3 = a.b3[oc];
-        const v4i rq3 = a.q3[oc];
+  }
+  __syncthreads();
 #pragma unroll
-        for (int mo = 0; mo < MO; ++mo) {
+  for (int i = 0; i < kMaxUnits; ++i) {
+    const int u = wave + i * kWaves;
+    if (u >= units) break;
+    const int t = u / (MO * 4), gq = u & 3;
+    const int oc = t * 32 + frow;
+    int av[4], v[4];
 #pragma unroll
-          for (int gq = 0; gq < 4; ++gq) {
-            int av[4], v[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int r = gq * 4 + e;
-              av[e] = acc_out[mo][t][r] + bias3 + buf[((0 * MO + mo) * 16 + r) * 64 + lane] +
-                      buf[((1 * MO + mo) * 16 + r) * 64 + lane] + buf[((2 * MO + mo) * 16 + r) * 64 + lane];
-            }
-            Requant8x4(av, rq3, a.out_zp, a.lo, a.hi, a.ties3, v);
-            *reinterpret_cast<uint32_t*>(stage + (mo * 32 + frow) * kStageStride + 8 * gq + 4 * fh) =
-                PackBytes(v[0], v[1], v[2], v[3]);
-          }
-        }
-        __builtin_amdgcn_wave_barrier();
-        // copy-out: a channel's band is po consecutive bytes of its plane
-        const size_t base = (static_cast<size_t>(n) * a.Cout + static_cast<size_t>(t) * 32) * out_plane + static_cast<size_t>(or0) * OW;
-        const int rows_live = min(32, a.Cout - t * 32);
-        // (the residual operand's loads are issued together, ahead of the stores)
-        if (a.aligned4) {
-          // lane = (channel row lane >> 3 of eight, dword lane & 7 of a 32-pixel tile)
-          uint32_t resv[MO][4];
-          if (ADD) {
-#pragma unroll
-            for (int mo = 0; mo < MO; ++mo)
-#pragma unroll
-              for (int i = 0; i < 4; ++i) {
-                const int r = i * 8 + (lane >> 3), px = mo * 32 + (lane & 7) * 4;
-                resv[mo][i] = (r < rows_live && px < po)
-                                  ? *reinterpret_cast<const uint32_t*>(a.res + base + static_cast<size_t>(r) * out_plane + px) : 0u;
-              }
-          }
-#pragma unroll
-          for (int mo = 0; mo < MO; ++mo)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const int r = i * 8 + (lane >> 3), px = mo * 32 + (lane & 7) * 4;
-              if (r < rows_live && px < po) {
-                uint32_t o = *reinterpret_cast<const uint32_t*>(stage + (mo * 32 + r) * kStageStride + (lane & 7) * 4);
-                if (ADD) o = AddResidual4(a, o, resv[mo][i]);
-                *reinterpret_cast<uint32_t*>(a.y + base + static_cast<size_t>(r) * out_plane + px) = o;
-              }
-            }
-        } else {
-          // lane = (channel row lane >> 5 of two, pixel lane & 31)
-#pragma unroll
-          for (int mo = 0; mo < MO; ++mo) {
-            uint8_t resv[16];
-            if (ADD) {
-#pragma unroll
-              for (int i = 0; i < 16; ++i) {
-                const int r = i * 2 + (lane >> 5), px = mo * 32 + (lane & 31);
-                resv[i] = (r < rows_live && px < po) ? a.res[base + static_cast<size_t>(r) * out_plane + px] : uint8_t{0};
-              }
-            }
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-              const int r = i * 2 + (lane >> 5), px = mo * 32 + (lane & 31);
-              if (r < rows_live && px < po) {
-                int o = stage[(mo * 32 + r) * kStageStride + (lane & 31)];
-                if (ADD) o = AddResidual1(a, o, resv[i]);
-                a.y[base + static_cast<size_t>(r) * out_plane + px] = static_cast<uint8_t>(o);
-              }
-            }
-          }
-        }
-        __builtin_amdgcn_wave_barrier();
+    for (int e = 0; e < 4; ++e) av[e] = red[((u >> 2) * 16 + gq * 4 + e) * 64 + lane] + bias3[i];
+    Requant8x4(av, rq3[i], a.out_zp, a.lo, a.hi, a.ties3, v);
+    if (oc >= a.Cout) continue;
+    if (a.aligned4) {
+      if (px0[i] < po) {
+        uint32_t o = PackBytes(v[0], v[1], v[2], v[3]);
+        if (ADD) o = AddResidual4(a, o, resv[i]);
+        *reinterpret_cast<uint32_t*>(a.y + at[i]) = o;
       }
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (px0[i] + e < po) {
+          int o = v[e] & 0xff;
+          if (ADD) o = AddResidual1(a, o, static_cast<int>((resv[i] >> (8 * e)) & 0xff));
+          a.y[at[i] + e] = static_cast<uint8_t>(o);
+        }
     }
   }
 }
@@ -504,11 +496,8 @@ int MbConvSetup(tvx_op* op, const MbStage& ex, const MbStage& dw, const tvx_conv
   a.ep = mh * 32 + 4;
   a.off_wave = RoundUp(mh * 32 * a.xs, 16);
   a.wave_bytes = RoundUp(16 + 32 * a.ep + MO * 32 * kMStride, 16);
-  a.off_red = 0;
-  a.off_stage = 2 * 3 * MO * 4096;
-  const int walk_bytes = a.off_wave + 4 * a.wave_bytes;
-  const int tail_bytes = a.off_stage + 4 * MO * 32 * kStageStride;
-  plan.lds_bytes = std::max(walk_bytes, tail_bytes);
+  a.off_red = a.off_wave + kWaves * a.wave_bytes;
+  plan.lds_bytes = a.off_red + nt * MO * 4096;
   if (plan.lds_bytes > 160 * 1024) return TVX_E_UNSUPPORTED;
   const uint64_t grid = static_cast<uint64_t>(e->batch) * a.bands;
   if (grid > 0x7fffffffull) return TVX_E_UNSUPPORTED;
