@@ -198,7 +198,13 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(O
       const int patches = a.w4_blocks * ((c4n + 3) / 4) * 64;
       const uint32_t plane32 = static_cast<uint32_t>(plane);
       const int row_bytes = a.iwt * a.pix_stride;
-      for (int pi = tid; pi < patches; pi += kThreads) {
+      // Fewer patches than threads (small planes with few channels): the threads of a patch split its halo rows,
+      // so that the rows of a tile are one batch of loads - one memory round trip - instead of several.
+      const int row_groups = patches <= kThreads / 2 ? kThreads / patches : 1;  // (patches: 64 or 128 then)
+      const int rows_per_group = (rows_needed + row_groups - 1) / row_groups;
+      const int my_group = row_groups > 1 ? tid / patches : 0;
+      const int hr_begin = my_group * rows_per_group, hr_end = min(rows_needed, hr_begin + rows_per_group);
+      for (int pi = row_groups > 1 ? tid - my_group * patches : tid; pi < patches; pi += kThreads) {
         // patch index -> (column group, channel group): 16 consecutive lanes read 64
         // contiguous bytes of one channel row, the next 16 lanes the next channel group
         const int blk = pi >> 6, in_blk = pi & 63;
@@ -243,7 +249,7 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(O
 #pragma unroll
           for (int b = 0; b < NB; ++b) {
             const int ih = ih0 + hr0 + b;
-            const bool inside = hr0 + b < rows_needed && ih >= 0 && ih < a.H;
+            const bool inside = hr0 + b < hr_end && ih >= 0 && ih < a.H;
             const uint32_t row_off = __umul24(static_cast<uint32_t>(inside ? ih : 0), static_cast<uint32_t>(a.W));
 #pragma unroll
             for (int j = 0; j < 4; ++j) d[b][j] = *reinterpret_cast<const int*>(src_row[j] + row_off * row_mul[j]);
@@ -252,14 +258,14 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(O
 #pragma unroll
           for (int b = 0; b < NB; ++b) {
             const int ih = ih0 + hr0 + b;
-            const bool inside = hr0 + b < rows_needed && ih >= 0 && ih < a.H;
+            const bool inside = hr0 + b < hr_end && ih >= 0 && ih < a.H;
             const int keep = inside ? -1 : 0;
 #pragma unroll
             for (int j = 0; j < 4; ++j) d[b][j] = ((d[b][j] ^ xmask[j]) & keep) | (fill[j] & ~keep);
           }
 #pragma unroll
           for (int b = 0; b < NB; ++b) {
-            if (hr0 + b >= rows_needed) continue;
+            if (hr0 + b >= hr_end) continue;
             // 4 x 4 byte transpose: d[j] = 4 pixels of channel c+j  ->  px[i] = 4 channels of pixel i
             const int lo01 = __builtin_amdgcn_perm(d[b][1], d[b][0], 0x05010400);
             const int hi01 = __builtin_amdgcn_perm(d[b][1], d[b][0], 0x07030602);
@@ -276,8 +282,8 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(O
               if (i < ncols) *reinterpret_cast<int*>(dst + __mul24(i, a.pix_stride)) = px[i];
           }
         };
-        for (int hr0 = 0; hr0 < rows_needed;) {
-          const int left = rows_needed - hr0;
+        for (int hr0 = hr_begin; hr0 < hr_end;) {
+          const int left = hr_end - hr0;
           if (left > 6) {
             batch(std::integral_constant<int, 8>{}, hr0);
             hr0 += 8;
@@ -339,42 +345,49 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(O
       const int8_t* w_row = w_lds + frag_row * a.kstride + frag_half * 16;
       const int2* my_tap = tap_lds + frag_half;
 
-      auto load_ab = [&](v4i* fa, v4i* fb, int ks, int2 t) {
+      // NP: pixel tiles per wavefront - two, or one where the workgroup's tile has at most four (small planes: the
+      // second tile would multiply padding)
+      auto kloop = [&](auto np_tag) {
+        constexpr int NP = decltype(np_tag)::value;
+        auto load_ab = [&](v4i* fa, v4i* fb, int ks, int2 t) {
 #pragma unroll
-        for (int i = 0; i < kMaxPtw; ++i)
-          fa[i] = *reinterpret_cast<const v4i*>(halo + a_base[i] + t.x);
-        // one k-step past the end reads bytes that exist in LDS and are never used
+          for (int i = 0; i < NP; ++i)
+            fa[i] = *reinterpret_cast<const v4i*>(halo + a_base[i] + t.x);
+          // one k-step past the end reads bytes that exist in LDS and are never used
 #pragma unroll
-        for (int j = 0; j < OT; ++j)
-          fb[j] = *reinterpret_cast<const v4i*>(w_row + j * 32 * a.kstride + ks * 32);
-      };
-      auto step = [&](const v4i* fa, const v4i* fb, int ones) {
+          for (int j = 0; j < OT; ++j)
+            fb[j] = *reinterpret_cast<const v4i*>(w_row + j * 32 * a.kstride + ks * 32);
+        };
+        auto step = [&](const v4i* fa, const v4i* fb, int ones) {
 #pragma unroll
-        for (int i = 0; i < kMaxPtw; ++i)
+          for (int i = 0; i < NP; ++i)
 #pragma unroll
-          for (int q = 0; q < 4; ++q) sx[i] = __builtin_amdgcn_sdot4(fa[i][q], ones, sx[i], false);
+            for (int q = 0; q < 4; ++q) sx[i] = __builtin_amdgcn_sdot4(fa[i][q], ones, sx[i], false);
 #pragma unroll
-        for (int j = 0; j < OT; ++j)
+          for (int j = 0; j < OT; ++j)
 #pragma unroll
-          for (int i = 0; i < kMaxPtw; ++i)
-            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
-      };
+            for (int i = 0; i < NP; ++i)
+              acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        };
 
-      v4i fa0[kMaxPtw], fb0[OT], fa1[kMaxPtw], fb1[OT];
-      int2 t0 = my_tap[0], t1 = my_tap[2];  // the table has one spare k-step at its end
-      load_ab(fa0, fb0, 0, t0);
-      int ks = 0;
-      for (; ks + 1 < a.ksteps; ks += 2) {
-        const int2 t2 = my_tap[(ks + 2) * 2];
-        load_ab(fa1, fb1, ks + 1, t1);
-        step(fa0, fb0, t0.y);
-        const int2 t3 = my_tap[(ks + 3) * 2];
-        load_ab(fa0, fb0, ks + 2, t2);
-        step(fa1, fb1, t1.y);
-        t0 = t2;
-        t1 = t3;
-      }
-      if (ks < a.ksteps) step(fa0, fb0, t0.y);
+        v4i fa0[NP], fb0[OT], fa1[NP], fb1[OT];
+        int2 t0 = my_tap[0], t1 = my_tap[2];  // the table has one spare k-step at its end
+        load_ab(fa0, fb0, 0, t0);
+        int ks = 0;
+        for (; ks + 1 < a.ksteps; ks += 2) {
+          const int2 t2 = my_tap[(ks + 2) * 2];
+          load_ab(fa1, fb1, ks + 1, t1);
+          step(fa0, fb0, t0.y);
+          const int2 t3 = my_tap[(ks + 3) * 2];
+          load_ab(fa0, fb0, ks + 2, t2);
+          step(fa1, fb1, t1.y);
+          t0 = t2;
+          t1 = t3;
+        }
+        if (ks < a.ksteps) step(fa0, fb0, t0.y);
+      };
+      if (a.PT <= 4) kloop(std::integral_constant<int, 1>{});
+      else kloop(std::integral_constant<int, 2>{});
     }
 
   }
