@@ -63,15 +63,6 @@ __device__ __forceinline__ int FastDiv(int u, uint32_t magic) {
   return static_cast<int>(__umulhi(static_cast<uint32_t>(u), magic)) + (magic == 0 ? u : 0);
 }
 
-// (v >> t) into byte E of d (the other bytes stay): the shift writes its result where the packed dword wants it
-template <int E>
-__device__ __forceinline__ void ShiftIntoByte(uint32_t& d, int t, int v) {
-  if (E == 0) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:DWORD" : "=v"(d) : "v"(t), "v"(v));
-  if (E == 1) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(d) : "v"(t), "v"(v));
-  if (E == 2) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(d) : "v"(t), "v"(v));
-  if (E == 3) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(d) : "v"(t), "v"(v));
-}
-
 // KH x KW taps over CPC 16-channel chunks (an even number): a k-step is one tap's pair of chunks.
 template <int KH, int KW, int CPC, int RQ, bool ZP>
 __global__ void __launch_bounds__(kBandThreads) __attribute__((amdgpu_waves_per_eu(4, 4)))

@@ -43,15 +43,6 @@ struct DwArgs {
 
 
 
-// (v >> t) into byte E of d (the other bytes stay): the shift writes its result where the packed dword wants it
-template <int E>
-__device__ __forceinline__ void ShiftIntoByte(uint32_t& d, int t, int v) {
-  if (E == 0) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:DWORD" : "=v"(d) : "v"(t), "v"(v));
-  if (E == 1) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(d) : "v"(t), "v"(v));
-  if (E == 2) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(d) : "v"(t), "v"(v));
-  if (E == 3) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(d) : "v"(t), "v"(v));
-}
-
 // Four accumulators of the channel -> four codes in one dword. Where no accumulator can land on a tie the clamp
 // comes in front of the shift (bounds shifted up: `lo_t`, `hi_t`), and the shift writes its byte of the dword: no
 // packing instructions.

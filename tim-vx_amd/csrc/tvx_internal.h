@@ -135,6 +135,17 @@ __device__ __forceinline__ uint32_t PackBytes(int a, int b, int c, int d) {
   return __builtin_amdgcn_perm(cd, ab, 0x05040100);
 }
 
+// (v >> t) into byte E of d (the other bytes stay): the shift writes its result where the packed dword wants it.
+// With the clamp in front of the shift (bounds shifted up: lo << t and (hi << t) | ((1 << t) - 1)) a requantized
+// byte of the no-tie record form costs four instructions and no packing: high multiply, rounding constant, clamp, this.
+template <int E>
+__device__ __forceinline__ void ShiftIntoByte(uint32_t& d, int t, int v) {
+  if (E == 0) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:DWORD" : "=v"(d) : "v"(t), "v"(v));
+  if (E == 1) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(d) : "v"(t), "v"(v));
+  if (E == 2) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(d) : "v"(t), "v"(v));
+  if (E == 3) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(d) : "v"(t), "v"(v));
+}
+
 template <int RQ>
 __device__ __forceinline__ int Requant8(int v, const tvx_v4i& q, int zp, int lo, int hi) {
   if (RQ == kRqGeneric) return RequantClamp(v, q[0], q[1], zp, lo, hi);
