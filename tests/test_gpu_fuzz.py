@@ -245,3 +245,88 @@ def test_pointwise_streaming_form_sweep(oracle, monkeypatch):
         want = oracle.conv2d(x, wt, b, act=act, **kws)
         got = TC.gpu_conv2d(x, wt, b, act=act, want_kernel="pwconv_i8_stream", **kws)
         assert np.array_equal(got, want), (i, n, c, h, w, oc, mode, act, int((got != want).sum()))
+
+
+def test_conv2d_with_max_pool_sweep(oracle, tvx):
+    """Random convolutions with even output extents + the 2x2 / stride-2 max pooling behind them through
+    tvx_conv2d_pool_create, against the oracle's two operators; both fused kernels must be reached."""
+    import torch
+    from test_gpu_fused_small_nets import _descs
+    rng = np.random.default_rng(0x9001)
+    seen = collections.Counter()
+    done = 0
+    for i in range(400):
+        if done >= 120:
+            break
+        kh, kw = (int(rng.choice([1, 2, 3, 5])), int(rng.choice([1, 3, 5]))) if rng.random() < 0.5 else (3, 3)
+        s = [int(rng.choice([1, 1, 2])), int(rng.choice([1, 1, 2]))]
+        d = [int(rng.choice([1, 1, 1, 2])), int(rng.choice([1, 1, 1, 2]))]
+        pad = [int(min(rng.integers(0, 3), (kw - 1) * d[0])) for _ in range(2)] + \
+              [int(min(rng.integers(0, 3), (kh - 1) * d[1])) for _ in range(2)]
+        h = int(rng.integers((kh - 1) * d[1] + 2, 30))
+        w = int(rng.integers((kw - 1) * d[0] + 2, 30))
+        c = int(rng.choice([1, 2, 3, 4])) if rng.random() < 0.4 else int(rng.integers(5, 80))
+        cfg = dict(n=int(rng.integers(1, 4)), c=c, h=h, w=w, oc=int(rng.integers(1, 140)), kh=kh, kw=kw, stride=s, dil=d, pad=pad, mult=0)
+        mode = str(rng.choice(["u8", "i8pc", "u8pc"]))
+        act = int(rng.integers(0, 3))
+        x, wt, b, kws = conv_case(rng, mode=mode, **cfg)
+        ow, oh, oc, n = kws["out_shape"]
+        if ow < 2 or oh < 2 or ow % 2 or oh % 2:
+            continue
+        keep = []
+        dd, pp = _descs(tvx, kws, act, keep)
+        try:
+            op = tvx.conv2d_pool_create(dd, pp, wt, b)
+        except tvx.TvxError as e:
+            assert e.status == tvx.E_UNSUPPORTED, (i, cfg)
+            seen["declined"] += 1
+            continue
+        t = oracle.conv2d(x, wt, b, act=act, **kws)
+        want = oracle.pool2d(t, in_shape=[ow, oh, oc, n], out_shape=[ow // 2, oh // 2, oc, n], ksize=[2, 2], stride=[2, 2],
+                             pad_left=0, pad_top=0, pool_type=0, dtype=kws["out_dtype"], in_q=kws["out_q"], out_q=kws["out_q"])
+        seen[op.kernel_name] += 1
+        xd = TC.to_device(x)
+        yd = TC.device_out(want.size, TC.NP_OF[kws["out_dtype"]])
+        op.run(xd, None, yd)
+        torch.cuda.synchronize()
+        got = yd.cpu().numpy()
+        op.close()
+        assert np.array_equal(got, want), (i, cfg, mode, act, op.kernel_name, int((got != want).sum()))
+        done += 1
+    assert seen["conv2d_im2col_maxpool_i8"] >= 10 and seen["conv2d_igemm_maxpool_i8"] >= 30, seen
+
+
+def test_conv2d_band_sweep(oracle, tvx, monkeypatch):
+    """Random 3x3 convolutions of the shapes the one-workgroup-per-CU band kernel takes (32 or 64 input channels,
+    33..64 output channels, rows of whole 8-byte units, stride 1 or 2, any padding up to one), forced onto it at
+    small batches, with random band heights and grid sizes."""
+    rng = np.random.default_rng(0xBA2D)
+    ran = 0
+    for i in range(60):
+        st = int(rng.choice([1, 1, 2]))
+        w = 8 * int(rng.integers(1, 9))
+        if st == 2:
+            w = 16 * int(rng.integers(1, 5))
+        h = int(rng.integers(3, 40))
+        pad = [int(rng.integers(0, 2)) for _ in range(4)]
+        cfg = dict(n=int(rng.integers(1, 4)), c=int(rng.choice([32, 64])), h=h, w=w, oc=int(rng.integers(33, 65)), kh=3, kw=3,
+                   stride=[st, st], dil=[1, 1], pad=pad, mult=0)
+        mode = str(rng.choice(["u8", "i8pc", "u8pc"]))
+        act = int(rng.integers(0, 3))
+        x, wt, b, kws = conv_case(rng, mode=mode, **cfg)
+        if min(kws["out_shape"][:2]) < 1 or kws["out_shape"][0] % 8:
+            continue
+        monkeypatch.setenv("TVX_CONV_BAND", "1")
+        monkeypatch.setenv("TVX_BAND_WGS", str(int(rng.choice([8, 16, 64]))))
+        if rng.random() < 0.5:
+            monkeypatch.setenv("TVX_BAND_ROWS", str(int(rng.integers(1, 6))))
+        else:
+            monkeypatch.delenv("TVX_BAND_ROWS", raising=False)
+        want = oracle.conv2d(x, wt, b, act=act, **kws)
+        d_kernel = []
+        got = _run_conv(tvx, x, wt, b, act, kws, d_kernel)
+        if d_kernel[0] != "conv2d_band_i8":
+            continue
+        ran += 1
+        assert np.array_equal(got, want), (i, cfg, mode, act, int((got != want).sum()))
+    assert ran >= 25, ran
