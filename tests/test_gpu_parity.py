@@ -167,7 +167,8 @@ POOL_ROWS = [
 @pytest.mark.parametrize("dtype", [0, 1])
 @pytest.mark.parametrize("ptype", [0, 1, 3])
 @pytest.mark.parametrize("pi", range(len(POOL_ROWS)))
-def test_pool2d_rows(oracle, pi, ptype, dtype):
+def test_pool2d_rows(oracle, pi, ptype, dtype, monkeypatch):
+    monkeypatch.setenv("TVX_POOL_STENCIL", "0")   # (the register stencil would take the stride-2 MAX shapes of this grid)
     p = POOL_ROWS[pi]
     rng = np.random.default_rng(600 + pi * 10 + ptype)
     w, h, c, n = p["in_shape"]
@@ -190,6 +191,7 @@ def test_pool2d_rows_band_budgets(oracle, band_kb, monkeypatch):
     pipelined plan falls through, the plain plan's grid and LDS size must be the ones launched - every plane of
     1024 plane groups written."""
     monkeypatch.setenv("TVX_POOL_BAND_KB", band_kb)
+    monkeypatch.setenv("TVX_POOL_STENCIL", "0")
     rng = np.random.default_rng(650)
     w, h, c, n = 24, 24, 64, 40   # 2560 planes: enough plane groups for the pipelined form at every budget
     x = rng.integers(0, 256, w * h * c * n, dtype=np.uint8)
@@ -200,7 +202,7 @@ def test_pool2d_rows_band_budgets(oracle, band_kb, monkeypatch):
     assert np.array_equal(got, want), int((got != want).sum())
 
 
-def test_pool2d_full_size_max_3x3_stride2(oracle):
+def test_pool2d_full_size_max_3x3_stride2(oracle, monkeypatch):
     """3x3 stride 2 MAX on 112x112x64 at batch 32 (25.7 MB in, 6.4 MB out): whole output against the oracle."""
     rng = np.random.default_rng(0x74)
     w, h, c, n = 112, 112, 64, 32
@@ -208,8 +210,71 @@ def test_pool2d_full_size_max_3x3_stride2(oracle):
     kws = dict(in_shape=[w, h, c, n], out_shape=[56, 56, c, n], ksize=[3, 3], stride=[2, 2], pad_left=0, pad_top=0,
                pool_type=0, dtype=0, in_q=(0.05, 3), out_q=(0.05, 3))
     want = oracle.pool2d(x, **kws)
+    got = TC.gpu_pool2d(x, want_kernel="pool2d_stencil_i8", **kws)
+    assert np.array_equal(got, want)
+    monkeypatch.setenv("TVX_POOL_STENCIL", "0")
     got = TC.gpu_pool2d(x, want_kernel="pool2d_rows_i8", **kws)
     assert np.array_equal(got, want)
+
+
+POOL_STENCIL = [
+    # in_shape {W, H, C, N}, ksize, pad {l, r, t, b}: MAX pooling at stride 2 on rows of whole 8-byte units (pool2d_stencil_i8)
+    dict(in_shape=[112, 112, 6, 2], ksize=[3, 3], pad=[0, 1, 0, 1]),     # SAME at stride 2: the padding column and row behind
+    dict(in_shape=[112, 112, 5, 1], ksize=[3, 3], pad=[1, 1, 1, 1]),     # ... in front: the left neighbour's last column
+    dict(in_shape=[24, 24, 20, 5], ksize=[2, 2], pad=[0, 0, 0, 0]),      # LeNet
+    dict(in_shape=[8, 8, 50, 3], ksize=[2, 2], pad=[0, 0, 0, 0]),        # one lane per row
+    dict(in_shape=[56, 31, 7, 2], ksize=[3, 2], pad=[1, 0, 0, 0]),       # seven lanes per row (eight with the idle one), an odd height
+    dict(in_shape=[40, 13, 3, 3], ksize=[2, 3], pad=[1, 0, 1, 1]),       # two taps across with left padding, three down
+    dict(in_shape=[64, 9, 4, 2], ksize=[3, 3], pad=[0, 1, 1, 0]),        # row groups that end inside a thread's four rows
+    dict(in_shape=[512, 6, 2, 1], ksize=[3, 3], pad=[1, 0, 1, 0]),       # the widest row: a wavefront per image row
+    dict(in_shape=[16, 1100, 3, 1], ksize=[2, 2], pad=[0, 0, 1, 0]),     # tall planes: several workgroups per plane
+    dict(in_shape=[112, 112, 4, 2], ksize=[3, 3], pad=[0, 0, 0, 0]),     # VALID: 55 x 55, rows that end inside a lane's four outputs
+    dict(in_shape=[48, 20, 5, 2], ksize=[3, 2], pad=[0, 0, 1, 0]),       # 23 columns
+    dict(in_shape=[32, 11, 3, 2], ksize=[2, 2], pad=[0, 0, 0, 0], out_w=13),  # a declared output narrower than the input allows
+]
+
+
+@pytest.mark.parametrize("dtype", [0, 1])
+@pytest.mark.parametrize("pi", range(len(POOL_STENCIL)))
+def test_pool2d_stencil(oracle, pi, dtype):
+    """The register-stencil MAX pooling against the oracle, with equal quantization on both sides (the maximum is the
+    result), with a moved zero point and with a rescale (the generic requantization of the maximum)."""
+    p = POOL_STENCIL[pi]
+    rng = np.random.default_rng(900 + pi * 10 + dtype)
+    w, h, c, n = p["in_shape"]
+    out_w = p.get("out_w", (w + p["pad"][0] + p["pad"][1] - p["ksize"][0]) // 2 + 1)
+    out_h = (h + p["pad"][2] + p["pad"][3] - p["ksize"][1]) // 2 + 1
+    assert out_w <= w // 2
+    kws = dict(in_shape=p["in_shape"], out_shape=[out_w, out_h, c, n], ksize=p["ksize"], stride=[2, 2],
+               pad_left=p["pad"][0], pad_top=p["pad"][2], pool_type=0, dtype=dtype)
+    x = rand_q(rng, w * h * c * n, dtype)
+    # (low codes everywhere but in a few places: a padding tap that took part would show)
+    x = np.where(rng.random(x.size) < 0.7, x.min(), x).astype(x.dtype)
+    zi = 7 if dtype else 120
+    import torch
+    for in_q, out_q in (((0.1, zi), (0.1, zi)), ((0.1, zi), (0.1, zi + 5)), ((0.5, zi), (0.25, zi))):
+        want = oracle.pool2d(x, in_q=in_q, out_q=out_q, **kws)
+        T = TC.tvx()
+        d = T.Pool2dDesc()
+        d.in_w, d.in_h, d.channels, d.batch = p["in_shape"]
+        d.out_w, d.out_h = out_w, out_h
+        d.k_w, d.k_h = p["ksize"]
+        d.stride_w = d.stride_h = 2
+        d.pad_left, d.pad_top, d.pool_type, d.dtype = p["pad"][0], p["pad"][2], 0, dtype
+        d.in_scale, d.in_zp = in_q
+        d.out_scale, d.out_zp = out_q
+        op = T.pool2d_create(d)
+        assert op.kernel_name == "pool2d_stencil_i8", op.kernel_name
+        xd = TC.to_device(x)
+        yd = TC.device_out(want.size + 32, TC.NP_OF[dtype])
+        yd.fill_(99)
+        op.run(xd, None, yd)
+        torch.cuda.synchronize()
+        got = yd.cpu().numpy()
+        op.close()
+        assert np.array_equal(got[:want.size], want), (int((got[:want.size] != want).sum()), np.flatnonzero(got[:want.size] != want)[:8])
+        assert np.all(got[want.size:] == 99), "wrote past the tensor"
+    assert len(np.unique(want)) > 4
 
 
 @pytest.mark.parametrize("shape", [(7, 7, 1280, 3), (2, 2, 5, 1), (5, 3, 9, 2), (17, 19, 6, 2), (33, 31, 3, 1)], ids=str)

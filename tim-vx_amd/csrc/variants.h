@@ -73,6 +73,8 @@ int FcSoftmaxSetup(tvx_op*, const tvx_fc_desc*, const void*, const void*);
 int PoolGenericSetup(tvx_op*);
 // quantized pooling, windows two or three taps wide, planes staged through LDS (pool2d_i8.hip)
 int PoolRowsSetup(tvx_op*);
+// quantized MAX pooling at stride 2, windows of 2 or 3 taps, rows of whole 8-byte units: register stencil (pool2d_stencil_i8.hip)
+int PoolStencilSetup(tvx_op*);
 int TransposeSetup(tvx_op*);
 int ConvertSetup(tvx_op*);
 

@@ -14,7 +14,7 @@ const std::vector<FcSetupFn>& FcVariants() {
 }
 
 const std::vector<SimpleSetupFn>& PoolVariants() {
-  static const std::vector<SimpleSetupFn> v = {PoolRowsSetup, PoolGenericSetup};
+  static const std::vector<SimpleSetupFn> v = {PoolStencilSetup, PoolRowsSetup, PoolGenericSetup};
   return v;
 }
 
