@@ -16,6 +16,11 @@
 // the matrix cores, whose clock drops under random data, plus ~10 % for the barrier per
 // k-tile); prologue and epilogue of a tile cost ~9 us next to ~60 us of k-loop.
 //
+// Int8 activations with per-channel or zero-point-free weights also have a 128 x 256 form (MB = 4
+// activation blocks instead of 8): half the accumulators and two weight slots instead of three fit
+// two wavefronts per SIMD, i.e. two workgroups per CU, so that one tile's prologue, barriers and
+// epilogue run under the other's MFMAs. It is taken when there are 1024 such tiles and more.
+//
 // The MFMA "A" operand is the weight fragment and "B" the activation fragment,
 // so a lane ends up with one activation row m and, per accumulator quad, four
 // consecutive features n: four requantized bytes make one dword of the row-major
@@ -29,6 +34,7 @@
 // two lane halves also cover 32 bytes of a row, so tiles, DMA, swizzle and fragment
 // addresses are identical with K counted in bytes; accumulation is fp32, the
 // epilogue adds the fp32 bias, clamps for ReLU / ReLU6 and rounds to float16.
+#include <cstdlib>
 #include <cstring>
 #include <type_traits>
 
@@ -42,15 +48,24 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
-constexpr int TM = 256, TN = 256, TK = 128;
+constexpr int TN = 256, TK = 128;
 constexpr int kThreads = 256;
-constexpr int kTileBytes = TM * TK;             // 32 KiB per activation tile
 constexpr int kStages = 4;                      // activation tiles in LDS (a power of two)
-constexpr int kTabOffset = kStages * kTileBytes;  // behind the stages: the tile's epilogue tables
-constexpr int kRowsumOffset = kTabOffset + TN * 4 + TN * 16;  // behind the folded bias (or fp32 bias) and the requantization records
-constexpr int kLdsBytes = kRowsumOffset + TM * 4;  // the activation rows' sums, exchanged between the wavefronts
-// k-tiles of the packed weights: whole rounds of three (the kernel's weight slots)
-__host__ __device__ constexpr int k_tiles_padded(int k_bytes) { return ((k_bytes + TK - 1) / TK + 2) / 3 * 3; }
+// The tile's geometry by its count MB of 32-row activation blocks: 8 (256 rows, one workgroup per CU, three weight
+// slots) or 4 (128 rows, two workgroups per CU whose prologues, barriers and epilogues hide behind each other's
+// MFMAs, two weight slots: half the registers per wavefront).
+template <int MB>
+struct Geo {
+  static constexpr int TM = MB * 32;
+  static constexpr int kSlots = MB == 8 ? 3 : 2;            // k-tiles of weight fragments resident in registers = prefetch distance
+  static constexpr int kOps = MB + 8;                        // memory operations a wavefront issues per k-tile (DMA pieces + weight fragments)
+  static constexpr int kTileBytes = TM * TK;                 // per activation tile: 32 / 16 KiB
+  static constexpr int kTabOffset = kStages * kTileBytes;    // behind the stages: the tile's epilogue tables
+  static constexpr int kRowsumOffset = kTabOffset + TN * 4 + TN * 16;  // behind the folded bias (or fp32 bias) and the requantization records
+  static constexpr int kLdsBytes = kRowsumOffset + TM * 4;   // the activation rows' sums, exchanged between the wavefronts
+};
+// k-tiles of the packed weights: whole rounds of the kernel's weight slots
+__host__ __device__ constexpr int k_tiles_padded(int k_bytes, int slots) { return ((k_bytes + TK - 1) / TK + slots - 1) / slots * slots; }
 constexpr int kOutStride = TN + 16;             // epilogue staging row stride (bytes)
 
 struct FcArgs {
@@ -77,9 +92,17 @@ __device__ __forceinline__ v16f Mfma(const v4i& a, const v4i& b, const v16f& c) 
   return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
 }
 
-template <bool X_U8, bool ROWSUM, int RQ, bool F16 = false>
-__global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
+template <int MB, bool X_U8, bool ROWSUM, int RQ, bool F16 = false>
+__global__ void __launch_bounds__(kThreads, MB == 8 ? 1 : 2) FcMfmaKernel(FcArgs a) {
   typedef typename std::conditional<F16, v16f, v16i>::type acc_t;
+  typedef Geo<MB> G;
+  // The 128-row form holds 128 accumulator, 64 weight and 32 activation registers of the 256 a wavefront has at two
+  // per SIMD; the in-place pass of the uint8 / row-sum variants does not fit beside them, and a register the
+  // compiler spills while one of this kernel's hand-waited loads is still writing it would be saved too early.
+  static_assert(MB == 8 || (MB == 4 && !X_U8 && !ROWSUM && !F16), "128-row tiles: int8 activations without row sums only");
+  constexpr int TM = G::TM, S = G::kSlots, P = G::kOps;
+  constexpr int kTileBytes = G::kTileBytes, kTabOffset = G::kTabOffset, kRowsumOffset = G::kRowsumOffset;
+  constexpr int kWaveRows = TM / 4;  // activation rows a wavefront fetches (and rewrites in place)
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -122,11 +145,11 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   // l >> 3, a permutation inside one 128-byte line. A wavefront moves rows
   // [64 w, 64 w + 64) per k-tile (8 instructions).
   const int dma_row = lane >> 3;
-  uint32_t off_x[8];  // byte offsets from the tensor base (tensors are < 4 GiB)
+  uint32_t off_x[MB];  // byte offsets from the tensor base (tensors are < 4 GiB)
   int dma_chunk[2];   // source chunk of this lane for even / odd instructions
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int r = wave * 64 + i * 8 + dma_row;
+  for (int i = 0; i < MB; ++i) {
+    const int r = wave * kWaveRows + i * 8 + dma_row;
     // LDS slot (row r, position lane & 7) holds chunk (lane & 7) ^ ((r >> 1) & 7) of the row
     const int chunk = (lane & 7) ^ ((r >> 1) & 7);
     dma_chunk[i & 1] = chunk;
@@ -138,7 +161,7 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   // piece i of k-tile kt into its stage; tiles past the last one and reduction bytes past K
   // read the zero source (0x80 before the re-bias of uint8 activations) and meet zero weights
   auto dma_piece = [&](auto whole, int kt, int i) {
-    int8_t* dst = lds + (kt & (kStages - 1)) * kTileBytes + wave_s * 64 * TK + i * 1024;
+    int8_t* dst = lds + (kt & (kStages - 1)) * kTileBytes + wave_s * kWaveRows * TK + i * 1024;
     const int k0 = kt * TK;
     if constexpr (decltype(whole)::value) {
       // a k-tile that lies inside K: a scalar base (tensor + k0) and the lane's 32-bit offset, no address arithmetic
@@ -167,9 +190,9 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   const int8_t* wp[2];  // (wavefront-uniform: the lane's 16 bytes are the load's vector offset)
 #pragma unroll
   for (int nb = 0; nb < 2; ++nb)
-    wp[nb] = a.w + (static_cast<size_t>(n0 / 32 + wave_s * 2 + nb) * (k_tiles_padded(a.K) * 4)) * 1024;
+    wp[nb] = a.w + (static_cast<size_t>(n0 / 32 + wave_s * 2 + nb) * (k_tiles_padded(a.K, S) * 4)) * 1024;
   const uint32_t lane16 = lane * 16;
-  v4i wr[3][8];  // [slot][nb * 4 + k-step]
+  v4i wr[S][8];  // [slot][nb * 4 + k-step]
 #define TVX_W_LOAD(dst, ptr, off) \
   asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(dst) : "v"(lane16), "s"(ptr), "n"(off))
   // fragment (nb, kk) of k-tile kt (callers stay below the padded count of k-tiles)
@@ -184,7 +207,7 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
 
   // [feature block][activation block]; a lane holds, per accumulator quad g, features 8 g + 4 (lane / 32) + 0..3 of its
   // wavefront's blocks. The integer accumulators start from the folded bias: one addition less per output in the epilogue.
-  acc_t acc[2][8];
+  acc_t acc[2][MB];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
@@ -195,11 +218,11 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
         b4[0] = t[0], b4[1] = t[1], b4[2] = t[2], b4[3] = t[3];
       }
 #pragma unroll
-      for (int j = 0; j < 8; ++j)
+      for (int j = 0; j < MB; ++j)
 #pragma unroll
         for (int q = 0; q < 4; ++q) acc[i][j][g * 4 + q] = b4[q];
     }
-  int rowsum[8] = {0, 0, 0, 0, 0, 0, 0, 0};  // per piece of this wavefront's share of the activation tile (see the in-place pass below)
+  int rowsum[MB] = {};  // per piece of this wavefront's share of the activation tile (see the in-place pass below)
 
   const int frag_row = lane & 31;   // row inside a 32-row MFMA tile
   const int frag_half = lane >> 5;  // which 16-byte half of a 32-byte k-step
@@ -239,7 +262,7 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   // MFMAs, spread over the first three k-steps. The barrier that publishes k-tile kt + 1 also publishes
   // its rewritten form.
   constexpr bool kInPlace = X_U8 || ROWSUM;
-  const uint32_t own_x = lds_base + wave * 64 * TK + lane * 16;
+  const uint32_t own_x = lds_base + wave * kWaveRows * TK + lane * 16;
 #define TVX_DS_READ(dst, addr, off) \
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(dst) : "v"(addr), "n"(off))
 #define TVX_DS_WRITE(addr, src, off) \
@@ -290,36 +313,38 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
     constexpr bool kPrefetch = decltype(prefetch)::value;
     constexpr bool kNext = decltype(fetch_next)::value;
     constexpr bool kPass = kInPlace && decltype(in_place)::value;
-    const int first = kk * 3, pieces = kk < 2 ? 3 : (kk == 2 ? 2 : 0);
+    // MB = 8: pieces 0-2, 3-5, 6-7 in k-steps 0, 1, 2; MB = 4: pieces 0-1, 2, 3
+    const int first = MB == 8 ? kk * 3 : (kk == 0 ? 0 : kk + 1);
+    const int pieces = MB == 8 ? (kk < 2 ? 3 : (kk == 2 ? 2 : 0)) : (kk == 0 ? 2 : (kk < 3 ? 1 : 0));
 #pragma unroll
-    for (int mb = 0; mb < 8; ++mb) {
+    for (int mb = 0; mb < MB; ++mb) {
       acc[0][mb] = Mfma(w_slot[kk], fx[mb], acc[0][mb]);
-      if (kNext && mb < 4) load_frag(next_kt, next_kk, fx_next, 2 * mb);
-      if (kPass && mb == 2) {
-        // this wavefront's own pieces of k-tile kt + 1 have landed when at most the newest 16 memory
-        // operations (or, in the last round, none) are still on their way
+      if (kNext && mb < MB / 2) load_frag(next_kt, next_kk, fx_next, 2 * mb);
+      if (kPass && mb == MB / 4) {
+        // this wavefront's own pieces of k-tile kt + 1 have landed when at most the memory operations of the
+        // k-tiles behind it (one with three weight slots, none with two or in the last round) are still on their way
         if (kk == 0) {
-          if constexpr (decltype(newer)::value != 0) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+          if constexpr (decltype(newer)::value != 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((S - 2) * P) : "memory");
           else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
 #pragma unroll
         for (int j = 0; j < 3; ++j)
           if (j < pieces) piece_read(kt + 1, first + j, pc[j]);
       }
-      if (kPrefetch && mb == 4) dma_piece(whole, kt + 3, kk * 2);
-      if (kPass && mb == 6 && pieces > 0) {
+      if (kPrefetch && mb == MB / 2) dma_piece(whole, kt + S, MB == 8 ? kk * 2 : kk);
+      if (kPass && mb == MB - 2 && pieces > 0) {
         // (the pieces are operands of the wait: nothing that uses them may be moved in front of it)
         asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(pc[0]), "+v"(pc[1]), "+v"(pc[2])::"memory");
         piece_finish(kt + 1, first, pc[0]);
       }
-      if (kPass && mb == 7 && pieces > 2) piece_finish(kt + 1, first + 2, pc[2]);
-      if (kPrefetch && mb == 7) w_piece(kt + 3, 0, kk, w_slot[kk]);
+      if (kPass && mb == MB - 1 && pieces > 2) piece_finish(kt + 1, first + 2, pc[2]);
+      if (kPrefetch && mb == MB - 1) w_piece(kt + S, 0, kk, w_slot[kk]);
       __builtin_amdgcn_sched_barrier(0);
       acc[1][mb] = Mfma(w_slot[4 + kk], fx[mb], acc[1][mb]);
-      if (kNext && mb < 4) load_frag(next_kt, next_kk, fx_next, 2 * mb + 1);
-      if (kPrefetch && mb == 5) dma_piece(whole, kt + 3, kk * 2 + 1);
-      if (kPass && mb == 6 && pieces > 1) piece_finish(kt + 1, first + 1, pc[1]);
-      if (kPrefetch && mb == 7) w_piece(kt + 3, 1, kk, w_slot[4 + kk]);
+      if (kNext && mb < MB / 2) load_frag(next_kt, next_kk, fx_next, 2 * mb + 1);
+      if (MB == 8 && kPrefetch && mb == MB / 2 + 1) dma_piece(whole, kt + S, kk * 2 + 1);
+      if (kPass && mb == MB - 2 && pieces > 1) piece_finish(kt + 1, first + 1, pc[1]);
+      if (kPrefetch && mb == MB - 1) w_piece(kt + S, 1, kk, w_slot[4 + kk]);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -329,7 +354,7 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   // issues 16 memory operations in the same order; "at most 28 in flight" at the barrier
   // (12 of this k-tile, 16 of the one before) means that everything issued two k-tiles ago
   // - the activations and weights of k-tile kt + 1 - has landed.
-  v4i fxa[8], fxb[8];
+  v4i fxa[MB], fxb[MB];
   // `prefetch`: the k-tile issues its share of k-tile kt + 3 (all rounds but the last, which is peeled off so that
   // no fetch is in flight when the loop ends: registers named by an unfinished fetch would otherwise have to be
   // kept out of the epilogue's hands). `in_flight`: memory operations that may still be on their way at the
@@ -346,9 +371,7 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
     k_step(prefetch, whole, yes, unless_last, in_flight, kt, 2, fxa, w_slot, kt, 3, fxb);
-    if constexpr (decltype(in_flight)::value == 28) asm volatile("s_waitcnt vmcnt(28) lgkmcnt(0)" ::: "memory");
-    else if constexpr (decltype(in_flight)::value == 16) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(decltype(in_flight)::value) : "memory");
     // the bare barrier: __syncthreads() adds a fence that waits for every memory operation in
     // flight - the whole prefetch - at every k-tile
     __builtin_amdgcn_s_barrier();
@@ -358,21 +381,21 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   // prologue: k-tiles 0, 1, 2 in the order every later k-tile uses (8 x (activation piece,
   // weight fragment)), so that the in-flight counts line up from the first barrier on
 #pragma unroll
-  for (int t = 0; t < 3; ++t)
+  for (int t = 0; t < S; ++t)
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk)
 #pragma unroll
       for (int nb = 0; nb < 2; ++nb) {
-        dma_piece(std::integral_constant<bool, false>(), t, kk * 2 + nb);
+        if (MB == 8 || nb == 0) dma_piece(std::integral_constant<bool, false>(), t, MB == 8 ? kk * 2 + nb : kk);
         __builtin_amdgcn_sched_barrier(0);
         w_piece(t, nb, kk, wr[t][nb * 4 + kk]);
         __builtin_amdgcn_sched_barrier(0);
       }
-  asm volatile("s_waitcnt vmcnt(32)" ::: "memory");  // k-tile 0 has landed
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"((S - 1) * P) : "memory");  // k-tile 0 has landed
   if (kInPlace) {
     // the in-place pass over k-tile 0 (every later k-tile gets it while the one before multiplies)
 #pragma unroll
-    for (int i = 0; i < 8; i += 2) {
+    for (int i = 0; i < MB; i += 2) {
       piece_read(0, i, pc[0]);
       piece_read(0, i + 1, pc[1]);
       asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(pc[0]), "+v"(pc[1])::"memory");
@@ -383,8 +406,8 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
   }
   __builtin_amdgcn_s_barrier();
 #pragma unroll
-  for (int t = 0; t < 8; ++t) load_frag(0, 0, fxa, t);
-  const int kt_max = k_tiles_padded(a.K) - 1;
+  for (int t = 0; t < MB; ++t) load_frag(0, 0, fxa, t);
+  const int kt_max = k_tiles_padded(a.K, S) - 1;
   // the loop runs whole rounds of three k-tiles (the weight slots are named registers); the
   // packed weights are zero-padded to that count and the activations past K read zeros
   {
@@ -394,31 +417,39 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
     int kt = 0;
     // rounds whose prefetch (k-tiles kt + 3 .. kt + 5) lies inside K, then those that reach past it
     const int whole_tiles = a.K / TK;
-    for (; kt + 6 <= whole_tiles; kt += 3) {
-      k_tile(yes, yes, integral_constant<int, 28>(), no, kt, wr[0]);
-      k_tile(yes, yes, integral_constant<int, 28>(), no, kt + 1, wr[1]);
-      k_tile(yes, yes, integral_constant<int, 28>(), no, kt + 2, wr[2]);
+    // memory operations that may still be on their way at a k-tile's barrier when everything of k-tile kt + 1 has
+    // landed: the k-tiles between it and the one being fetched, and the three k-steps' worth of that one
+    const integral_constant<int, (S - 2) * P + 3 * P / 4> steady;
+    for (; kt + 2 * S <= whole_tiles; kt += S) {
+      k_tile(yes, yes, steady, no, kt, wr[0]);
+      k_tile(yes, yes, steady, no, kt + 1, wr[1]);
+      if constexpr (S == 3) k_tile(yes, yes, steady, no, kt + 2, wr[S - 1]);
     }
-    for (; kt + 3 <= kt_max; kt += 3) {
-      k_tile(yes, no, integral_constant<int, 28>(), no, kt, wr[0]);
-      k_tile(yes, no, integral_constant<int, 28>(), no, kt + 1, wr[1]);
-      k_tile(yes, no, integral_constant<int, 28>(), no, kt + 2, wr[2]);
+    for (; kt + S <= kt_max; kt += S) {
+      k_tile(yes, no, steady, no, kt, wr[0]);
+      k_tile(yes, no, steady, no, kt + 1, wr[1]);
+      if constexpr (S == 3) k_tile(yes, no, steady, no, kt + 2, wr[S - 1]);
     }
     // the last round: its k-tiles were fetched by the round before (or the prologue); nothing new is fetched
-    k_tile(no, no, integral_constant<int, 16>(), no, kt, wr[0]);
-    k_tile(no, no, integral_constant<int, 0>(), no, kt + 1, wr[1]);
-    k_tile(no, no, integral_constant<int, 0>(), yes, kt + 2, wr[2]);
+    if constexpr (S == 3) {
+      k_tile(no, no, integral_constant<int, P>(), no, kt, wr[0]);
+      k_tile(no, no, integral_constant<int, 0>(), no, kt + 1, wr[1]);
+      k_tile(no, no, integral_constant<int, 0>(), yes, kt + 2, wr[S - 1]);
+    } else {
+      k_tile(no, no, integral_constant<int, 0>(), no, kt, wr[0]);
+      k_tile(no, no, integral_constant<int, 0>(), yes, kt + 1, wr[1]);
+    }
   }
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");  // (nothing is in flight here; the staging tile is about to be written)
   if (ROWSUM) {
-    // piece i holds rows 64 w + 8 i + lane / 8, a lane its 16 bytes of every k-tile: eight lanes make a row
+    // piece i holds rows kWaveRows w + 8 i + lane / 8, a lane its 16 bytes of every k-tile: eight lanes make a row
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = 0; i < MB; ++i) {
       int sum = rowsum[i];
       sum += __shfl_xor(sum, 1);
       sum += __shfl_xor(sum, 2);
       sum += __shfl_xor(sum, 4);
-      if ((lane & 7) == 0) reinterpret_cast<int*>(lds + kRowsumOffset)[wave * 64 + i * 8 + (lane >> 3)] = sum;
+      if ((lane & 7) == 0) reinterpret_cast<int*>(lds + kRowsumOffset)[wave * kWaveRows + i * 8 + (lane >> 3)] = sum;
     }
   }
   __syncthreads();  // the epilogue reuses the LDS
@@ -448,7 +479,7 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
             for (int q = 0; q < 4; ++q) b4[q] = reinterpret_cast<const float*>(lds + kTabOffset)[nl + q];
             const int col = nl - round * 128;  // staged column (halves)
 #pragma unroll
-            for (int mb = 0; mb < 8; ++mb) {
+            for (int mb = 0; mb < MB; ++mb) {
               const int ml = mb * 32 + frag_row;
               _Float16 h[4];
 #pragma unroll
@@ -482,9 +513,9 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
       }
     }
   } else {
-    int zp_term[8];  // weight zero point x row sum, per activation block of this lane's row
+    int zp_term[MB];  // weight zero point x row sum, per activation block of this lane's row
 #pragma unroll
-    for (int t = 0; t < 8; ++t)
+    for (int t = 0; t < MB; ++t)
       zp_term[t] = ROWSUM ? a.zws * reinterpret_cast<const int*>(lds + kRowsumOffset)[t * 32 + frag_row] : 0;
     int8_t* out_tile = lds;  // TM rows x kOutStride bytes (the loop's last barrier freed the LDS)
 #pragma unroll
@@ -499,7 +530,7 @@ __global__ void __launch_bounds__(kThreads, 1) FcMfmaKernel(FcArgs a) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) q4[q] = reinterpret_cast<const tvx_v4i*>(lds + kTabOffset + TN * 4)[nl + q];
 #pragma unroll
-        for (int mb = 0; mb < 8; ++mb) {
+        for (int mb = 0; mb < MB; ++mb) {
           const int ml = mb * 32 + frag_row;
           int r4[4];
 #pragma unroll
@@ -622,23 +653,35 @@ void LaunchSmallRq(int rq, dim3 grid, hipStream_t st, const FcArgs& a) {
 // Few enough outputs that 256 x 256 tiles would leave most of the chip idle.
 bool UseSmallTiles(const tvx_fc_desc& d) { return static_cast<uint64_t>(d.m) * d.n <= (1u << 18); }
 
-template <bool X_U8, bool ROWSUM>
-void LaunchRq(int rq, dim3 grid, hipStream_t st, const FcArgs& a) {
-  const dim3 block(kThreads);
-  if (rq == kRqFastNoTie)
-    hipLaunchKernelGGL((FcMfmaKernel<X_U8, ROWSUM, kRqFastNoTie>), grid, block, kLdsBytes, st, a);
-  else if (rq == kRqFast)
-    hipLaunchKernelGGL((FcMfmaKernel<X_U8, ROWSUM, kRqFast>), grid, block, kLdsBytes, st, a);
-  else
-    hipLaunchKernelGGL((FcMfmaKernel<X_U8, ROWSUM, kRqGeneric>), grid, block, kLdsBytes, st, a);
+typedef void (*TileKernel)(FcArgs);
+template <int MB, bool X_U8, bool ROWSUM>
+TileKernel TileKernelOf(int rq) {
+  if (rq == kRqFastNoTie) return FcMfmaKernel<MB, X_U8, ROWSUM, kRqFastNoTie>;
+  if (rq == kRqFast) return FcMfmaKernel<MB, X_U8, ROWSUM, kRqFast>;
+  return FcMfmaKernel<MB, X_U8, ROWSUM, kRqGeneric>;
 }
+// mb: the tile's 32-row activation blocks (8, or 4 for int8 activations without row sums)
+TileKernel TileKernelOf(int mb, bool f16, bool x_u8, bool rowsum, int rq) {
+  if (f16) return FcMfmaKernel<8, false, false, kRqGeneric, true>;
+  if (x_u8 && rowsum) return TileKernelOf<8, true, true>(rq);
+  if (x_u8) return TileKernelOf<8, true, false>(rq);
+  if (rowsum) return TileKernelOf<8, false, true>(rq);
+  return mb == 8 ? TileKernelOf<8, false, false>(rq) : TileKernelOf<4, false, false>(rq);
+}
+int TileLdsBytes(int mb) { return mb == 8 ? Geo<8>::kLdsBytes : Geo<4>::kLdsBytes; }
+int TileSlots(int mb) { return mb == 8 ? Geo<8>::kSlots : Geo<4>::kSlots; }
 
-template <bool X_U8, bool ROWSUM>
-hipError_t AllowLds(int rq) {
-  const void* f = rq == kRqFastNoTie ? reinterpret_cast<const void*>(&FcMfmaKernel<X_U8, ROWSUM, kRqFastNoTie>)
-                  : (rq == kRqFast ? reinterpret_cast<const void*>(&FcMfmaKernel<X_U8, ROWSUM, kRqFast>)
-                                   : reinterpret_cast<const void*>(&FcMfmaKernel<X_U8, ROWSUM, kRqGeneric>));
-  return hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+// 128-row tiles (the variant that has them) where there are enough to give every CU two workgroups twice over;
+// TVX_FC_TILE_M=128|256 overrides (a test lever, read when the operator is created).
+int ChooseTileBlocks(uint32_t m, uint32_t n, bool plain_int8) {
+  if (!plain_int8) return 8;
+  int mb = static_cast<uint64_t>((m + 127) / 128) * ((n + TN - 1) / TN) >= 1024 ? 4 : 8;
+  if (const char* f = getenv("TVX_FC_TILE_M")) {
+    const int v = atoi(f);
+    if (v == 128) mb = 4;
+    if (v == 256) mb = 8;
+  }
+  return mb;
 }
 
 int FcMfmaRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t st) {
@@ -657,21 +700,22 @@ int FcMfmaRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t s
   a.out_zp = d.out_zp;
   a.lo = op->act_lo;
   a.hi = op->act_hi;
-  a.tiles_m = (a.M + TM - 1) / TM;
+  const int mb = op->geo[3];
+  a.tiles_m = (a.M + mb * 32 - 1) / (mb * 32);
   a.tiles_n = (a.N + TN - 1) / TN;
-  a.group_m = 4;
+  a.group_m = mb == 8 ? 4 : 8;  // panels of 1024 activation rows
   const dim3 grid(a.tiles_m * a.tiles_n);
+  const bool x_u8 = d.in_dtype == TVX_U8, rowsum = a.zws != 0;
+  const int rq = op->geo[1];
   if (op->geo[2]) {  // float16
     a.K = static_cast<int>(d.k) * 2;
     a.biasf32 = op->aux.as<float>();
     a.flo = d.activation == TVX_ACT_NONE ? -3.402823466e38f : 0.0f;
     a.fhi = d.activation == TVX_ACT_RELU6 ? 6.0f : 3.402823466e38f;
-    hipLaunchKernelGGL((FcMfmaKernel<false, false, kRqGeneric, true>), grid, dim3(kThreads), kLdsBytes, st, a);
+    hipLaunchKernelGGL(TileKernelOf(mb, true, false, false, rq), grid, dim3(kThreads), TileLdsBytes(mb), st, a);
     TVX_HIP_CHECK(hipGetLastError());
     return TVX_OK;
   }
-  const bool x_u8 = d.in_dtype == TVX_U8, rowsum = a.zws != 0;
-  const int rq = op->geo[1];
   if (UseSmallTiles(d)) {
     const dim3 small_grid(((a.M + 15) / 16) * ((a.N + 15) / 16));
     if (x_u8 && rowsum) LaunchSmallRq<true, true>(rq, small_grid, st, a);
@@ -681,10 +725,7 @@ int FcMfmaRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t s
     TVX_HIP_CHECK(hipGetLastError());
     return TVX_OK;
   }
-  if (x_u8 && rowsum) LaunchRq<true, true>(rq, grid, st, a);
-  else if (x_u8) LaunchRq<true, false>(rq, grid, st, a);
-  else if (rowsum) LaunchRq<false, true>(rq, grid, st, a);
-  else LaunchRq<false, false>(rq, grid, st, a);
+  hipLaunchKernelGGL(TileKernelOf(mb, false, x_u8, rowsum, rq), grid, dim3(kThreads), TileLdsBytes(mb), st, a);
   TVX_HIP_CHECK(hipGetLastError());
   return TVX_OK;
 }
@@ -694,10 +735,10 @@ int FcMfmaRun(tvx_op* op, const void* in0, const void*, void* out, hipStream_t s
 // Weights [N][k_bytes] (int8 domain or float16 bytes) -> MFMA-fragment order: for every block
 // of 32 features and every 32-byte k-step, 64 lanes x 16 bytes where lane l holds feature
 // 32 b + l % 32, bytes [32 ks + 16 (l / 32), + 16). Features are padded to the tile and the
-// reduction to whole rounds of three k-tiles, with zeros.
-static std::vector<int8_t> PackFragments(const int8_t* w, uint32_t n, uint32_t k_bytes) {
+// reduction to whole rounds of `slots` k-tiles (the kernel's weight slots), with zeros.
+static std::vector<int8_t> PackFragments(const int8_t* w, uint32_t n, uint32_t k_bytes, int slots) {
   const size_t n_blocks = (n + TN - 1) / TN * (TN / 32);
-  const size_t ksteps = static_cast<size_t>(k_tiles_padded(static_cast<int>(k_bytes))) * 4;
+  const size_t ksteps = static_cast<size_t>(k_tiles_padded(static_cast<int>(k_bytes), slots)) * 4;
   std::vector<int8_t> out(n_blocks * ksteps * 1024, 0);
   for (size_t b = 0; b < n_blocks; ++b)
     for (int r = 0; r < 32; ++r) {
@@ -721,18 +762,19 @@ static int FcMfmaSetupF16(tvx_op* op, const tvx_fc_desc* d, const void* w_host, 
   const uint32_t n_alloc = (d->n + TN - 1) / TN * TN;
   std::vector<float> bias(n_alloc, 0.0f);
   if (bias_host) std::memcpy(bias.data(), bias_host, sizeof(float) * d->n);
-  const std::vector<int8_t> frags = PackFragments(static_cast<const int8_t*>(w_host), d->n, d->k * 2);
+  const int mb = ChooseTileBlocks(d->m, d->n, false);
+  const std::vector<int8_t> frags = PackFragments(static_cast<const int8_t*>(w_host), d->n, d->k * 2, TileSlots(mb));
   int s = op->packed.Upload(frags.data(), frags.size());
   if (s == TVX_OK) s = op->aux.Upload(bias.data(), bias.size() * 4);
   std::vector<int8_t> zeros(256, 0);
   if (s == TVX_OK) s = op->aux3.Upload(zeros.data(), zeros.size());
   if (s != TVX_OK) return s;
-  const hipError_t e =
-      hipFuncSetAttribute(reinterpret_cast<const void*>(&FcMfmaKernel<false, false, kRqGeneric, true>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+  const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(TileKernelOf(mb, true, false, false, kRqGeneric)),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, TileLdsBytes(mb));
   if (e != hipSuccess)
-    return SetError(TVX_E_DEVICE, "hipFuncSetAttribute(dynamic LDS %d): %s", kLdsBytes, hipGetErrorString(e));
+    return SetError(TVX_E_DEVICE, "hipFuncSetAttribute(dynamic LDS %d): %s", TileLdsBytes(mb), hipGetErrorString(e));
   op->geo[2] = 1;
+  op->geo[3] = mb;
   op->run = FcMfmaRun;
   op->kernel_name = "fc_mfma_f16_256x256x64";
   return TVX_OK;
@@ -773,11 +815,12 @@ int FcMfmaSetup(tvx_op* op, const tvx_fc_desc* d, const void* w_host, const void
                                      static_cast<int>(n_alloc), d->out_zp, &rqt,
                                      AccumulatorBound(d->k, bias_host, d->n));
   // the tiled kernel reads fragment order, the small-tile kernel plain rows
+  const int mb = ChooseTileBlocks(d->m, d->n, d->in_dtype != TVX_U8 && zws == 0);
   int s;
   if (UseSmallTiles(*d)) {
     s = op->packed.Upload(ws.data(), wn);
   } else {
-    const std::vector<int8_t> frags = PackFragments(ws.data(), d->n, d->k);
+    const std::vector<int8_t> frags = PackFragments(ws.data(), d->n, d->k, TileSlots(mb));
     s = op->packed.Upload(frags.data(), frags.size());
   }
   if (s == TVX_OK) s = op->aux.Upload(biasf.data(), biasf.size() * 4);
@@ -787,14 +830,15 @@ int FcMfmaSetup(tvx_op* op, const tvx_fc_desc* d, const void* w_host, const void
   if (s == TVX_OK) s = op->aux3.Upload(zeros.data(), zeros.size());
   if (s != TVX_OK) return s;
   const bool x_u8 = d->in_dtype == TVX_U8, rowsum = zws != 0;
-  hipError_t e = x_u8 ? (rowsum ? AllowLds<true, true>(rq) : AllowLds<true, false>(rq))
-                      : (rowsum ? AllowLds<false, true>(rq) : AllowLds<false, false>(rq));
+  const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(TileKernelOf(mb, false, x_u8, rowsum, rq)),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, TileLdsBytes(mb));
   if (e != hipSuccess)
-    return SetError(TVX_E_DEVICE, "hipFuncSetAttribute(dynamic LDS %d): %s", kLdsBytes, hipGetErrorString(e));
+    return SetError(TVX_E_DEVICE, "hipFuncSetAttribute(dynamic LDS %d): %s", TileLdsBytes(mb), hipGetErrorString(e));
   op->geo[0] = zws;
   op->geo[1] = rq;
+  op->geo[3] = mb;
   op->run = FcMfmaRun;
-  op->kernel_name = UseSmallTiles(*d) ? "fc_mfma_i8_16x16_splitk" : "fc_mfma_i8_256x256x128";
+  op->kernel_name = UseSmallTiles(*d) ? "fc_mfma_i8_16x16_splitk" : (mb == 8 ? "fc_mfma_i8_256x256x128" : "fc_mfma_i8_128x256x128");
   return TVX_OK;
 }
 
