@@ -993,6 +993,11 @@ IM2COL_GRID = [
     dict(n=2, c=2, h=7, w=9, oc=33, kh=5, kw=5, stride=[1, 1], dil=[1, 1], pad=[2, 2, 2, 2], mult=0),     # SAME 5 x 5, K = 50, two channel tiles
     dict(n=3, c=1, h=11, w=13, oc=7, kh=3, kw=5, stride=[2, 1], dil=[1, 1], pad=[1, 3, 1, 1], mult=0),    # uneven pads, strides
     dict(n=1, c=4, h=6, w=6, oc=9, kh=3, kw=5, stride=[1, 1], dil=[2, 1], pad=[4, 4, 2, 2], mult=0),      # K = 60, left padding as wide as the window reaches
+    # wavefronts whose windows all lie inside the image's rows (no dword moved, the column border as one mask per
+    # thread) next to wavefronts on the first / last rows
+    dict(n=2, c=3, h=40, w=72, oc=32, kh=3, kw=3, stride=[2, 2], dil=[1, 1], pad=[1, 1, 1, 1], mult=0),
+    dict(n=2, c=1, h=40, w=44, oc=12, kh=5, kw=5, stride=[1, 1], dil=[1, 1], pad=[2, 2, 2, 2], mult=0),
+    dict(n=2, c=2, h=30, w=50, oc=16, kh=3, kw=3, stride=[1, 1], dil=[2, 1], pad=[0, 2, 2, 2], mult=0),   # dilated rows: window rows 0, 2, 4
 ]
 
 

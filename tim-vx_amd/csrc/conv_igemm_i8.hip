@@ -850,7 +850,11 @@ int ConvIgemmSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
     auto workgroups = [&](int ot_, int p_) {
       return static_cast<long long>(d->batch) * ((hw + p_ - 1) / p_) * ((oc_pad + 32 * ot_ - 1) / (32 * ot_));
     };
-    if (ot == 4 && workgroups(ot, best_p) < slots / 2) {  // (up to 64 output channels the choice above also decides the persistent variant)
+    // (up to 64 output channels the choice above also decides the persistent variant: there only a launch of a
+    // few workgroups - LeNet's second convolution at batch 1 is one - is re-cut)
+    const char* persist_lever = getenv("TVX_IGEMM_PERSIST");  // (forcing the persistent variant keeps its tile choice)
+    const bool tiny = ot < 4 && workgroups(ot, best_p) < cus / 8 && !(persist_lever && atoi(persist_lever) > 0);
+    if ((ot == 4 && workgroups(ot, best_p) < slots / 2) || tiny) {
       auto cost = [&](int ot_, int p_) {
         const long long rounds = (workgroups(ot_, p_) + slots - 1) / slots;
         return rounds * (((p_ / 32 + 3) / 4) * ot_ + 2);

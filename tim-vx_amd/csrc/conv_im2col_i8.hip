@@ -49,6 +49,7 @@ struct ImArgs {
   int taps[64];
   int offs[64];
   int rows;              // row mode: C * Kh
+  int rows_mask;         // row mode: the window rows in use (bit dy), all of them inside the image for most pixels
   int total_bytes;       // row mode: size of the input tensor (< 2^31)
   int pool;              // 1: a 2 x 2 / stride-2 max pooling rides on the epilogue (the result has OH / 2 x OW / 2 pixels)
 };
@@ -128,6 +129,52 @@ __global__ void __launch_bounds__(kThreads) ConvIm2colKernel(ImArgs a) {
         return at;
       };
       uint32_t v[kMaxRows], v2[KW == 5 ? kMaxRows : 1];
+      int dw[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) dw[i] = 0;
+      // Nearly every wavefront holds only pixels whose window rows all lie inside the image and whose dwords all
+      // lie inside the tensor (the exceptions: an image's first / last output rows under padding, the tensor's
+      // first and last bytes). There a row's dword sits where it is expected, nothing is moved or shifted back,
+      // and what is left of the border - the same one or two window columns outside the image in every row of a
+      // pixel - is one mask and one XOR pattern per thread: (dword & inside) ^ (re-bias where inside, the input
+      // zero point where not).
+      const int first_at = img_at + a.offs[0], last_at = img_at + a.offs[a.rows - 1] + (KW == 5 ? 4 : 0);
+      const bool plain = (row_ok & static_cast<uint32_t>(a.rows_mask)) == static_cast<uint32_t>(a.rows_mask) &&
+                         first_at >= 0 && last_at + 4 <= a.total_bytes;
+      if (__builtin_amdgcn_ballot_w64(!plain) == 0) {
+#pragma unroll
+        for (int r = 0; r < kMaxRows; ++r) {
+          v[r] = 0;
+          if (KW == 5) v2[r] = 0;
+          if (r < a.rows) {  // uniform
+            const uint32_t at = static_cast<uint32_t>(img_at + a.offs[r]);
+            __builtin_memcpy(&v[r], a.x + at, 4);
+            if constexpr (KW == 5) __builtin_memcpy(&v2[r], a.x + at + 4, 4);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);  // all loads travel together
+        uint32_t keep = 0, flip = 0, keep2 = 0, flip2 = 0;  // per window column: 0xff where inside; re-bias or zero point
+#pragma unroll
+        for (int e = 0; e < KW; ++e) {
+          const bool inside = ((col_ok >> e) & 1u) != 0;
+          const uint32_t k8 = inside ? 0xffu : 0u, f8 = static_cast<uint32_t>(inside ? a.xor_mask : a.pad_fill) & 0xffu;
+          if (e < 4) keep |= k8 << (8 * e), flip |= f8 << (8 * e);
+          else keep2 = k8, flip2 = f8;
+        }
+#pragma unroll
+        for (int r = 0; r < kMaxRows; ++r) {
+          if (r < a.rows) {
+            const int k = r * KW, i = k >> 2, pos = k & 3;  // (constants once unrolled)
+            const uint32_t row = (v[r] & keep) ^ flip;  // KW == 3: the fourth byte is masked away
+            dw[i] |= static_cast<int>(row << (8 * pos));
+            if (pos + (KW == 3 ? 3 : 4) > 4) dw[i + 1] |= static_cast<int>(row >> (8 * (4 - pos)));
+            if constexpr (KW == 5) {
+              const int k5 = k + 4;
+              dw[k5 >> 2] |= static_cast<int>(((v2[r] & keep2) ^ flip2) << (8 * (k5 & 3)));
+            }
+          }
+        }
+      } else {
 #pragma unroll
       for (int r = 0; r < kMaxRows; ++r) {
         v[r] = 0;
@@ -144,9 +191,6 @@ __global__ void __launch_bounds__(kThreads) ConvIm2colKernel(ImArgs a) {
         }
       }
       __builtin_amdgcn_sched_barrier(0);  // all loads travel together
-      int dw[16];
-#pragma unroll
-      for (int i = 0; i < 16; ++i) dw[i] = 0;
 #pragma unroll
       for (int r = 0; r < kMaxRows; ++r) {
         if (r < a.rows) {
@@ -169,6 +213,7 @@ __global__ void __launch_bounds__(kThreads) ConvIm2colKernel(ImArgs a) {
             dw[k >> 2] |= byte << (8 * (k & 3));
           }
         }
+      }
       }
 #pragma unroll
       for (int i = 0; i < 16; ++i) sx = __builtin_amdgcn_sdot4(dw[i], 0x01010101, sx, false);
@@ -389,6 +434,7 @@ int ConvIm2colSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, co
       const int dy = (r % static_cast<int>(d->k_h)) * static_cast<int>(d->dilation_h);
       a.taps[r] = dy | 1 << 16;
       a.offs[r] = c * a.H * a.W + dy * a.W;
+      a.rows_mask |= 1 << dy;
     }
   } else {
     for (int k = 0; k < K; ++k) {
