@@ -80,8 +80,10 @@ __device__ __forceinline__ void StoreFour(const GemmArgs& a, uint8_t* y, size_t 
 }
 
 // OT: 32-channel tiles of a workgroup (1 or 2). QUAD: the gather by pixel quads (see below) instead of by elements.
+// (two wavefronts per SIMD at least: within 256 registers the compiler keeps MFMA accumulators in ordinary vector
+// registers, where the epilogue reads them, instead of moving every value out of the accumulation registers first)
 template <bool F16, int OT, bool QUAD>
-__global__ void __launch_bounds__(kThreads) ConvGemmKernel(GemmArgs a) {
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) ConvGemmKernel(GemmArgs a) {
   __shared__ __attribute__((aligned(16))) uint8_t a_lds[kPixels * kRowStride];
   __shared__ __attribute__((aligned(16))) uint8_t b_lds[OT * 32 * kRowStride];
   constexpr int ESZ = F16 ? 2 : 1;

@@ -55,8 +55,10 @@ struct ImArgs {
 };
 
 // KW: 0 = any window, one byte load per tap; 3 / 5 = row mode for kernels three / five taps wide
+// (two wavefronts per SIMD at least: within 256 registers the compiler keeps MFMA accumulators in ordinary vector
+// registers, where the epilogue reads them, instead of moving every value out of the accumulation registers first)
 template <int OT, int RQ, int KW>
-__global__ void __launch_bounds__(kThreads) ConvIm2colKernel(ImArgs a) {
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) ConvIm2colKernel(ImArgs a) {
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n = blockIdx.y;

@@ -169,8 +169,10 @@ __device__ __forceinline__ void PatchCompute(const DwPwArgs& a, const ChannelCon
 
 // S: stride of the depthwise convolution (left padding 1 at stride 1, 0 at stride 2: SAME);
 // RPT: output rows of a tile.
+// (two wavefronts per SIMD at least: within 256 registers the compiler keeps MFMA accumulators in ordinary vector
+// registers, where the epilogue reads them, instead of moving every value out of the accumulation registers first)
 template <int S, int RPT, bool ADD>
-__global__ void __launch_bounds__(kThreads) DwPwKernel(DwPwArgs a) {
+__global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) DwPwKernel(DwPwArgs a) {
   extern __shared__ __attribute__((aligned(16))) int8_t lds[];
   constexpr int PL = S == 1 ? 1 : 0;
   const int tid = threadIdx.x, lane = tid & 63;
