@@ -156,8 +156,8 @@ def test_fully_connected_sweep(oracle):
         assert np.array_equal(got, want), (i, m, k, n, mode, act)
 
 
-def test_fully_connected_tiled_sweep(oracle):
-    """The 256 x 256 tile kernel (more than 2^18 outputs): ragged last tiles in both directions, reductions from
+def test_fully_connected_tiled_sweep(oracle, monkeypatch):
+    """The tiled kernel (more than 2^18 outputs), 256- and 128-row tiles in turn: ragged last tiles in both directions, reductions from
     one 16-byte chunk to nine k-tiles with every tail, uint8 and int8 activations with and without a uniform weight
     zero point (re-bias and row sums inside the kernel), per-channel weights."""
     rng = np.random.default_rng(0xFD)
@@ -180,8 +180,10 @@ def test_fully_connected_tiled_sweep(oracle):
                    out_q=(float(np.float32(0.02 * 0.01 * 40 * np.sqrt(k))), 5 if in_dt == 0 else -3))
         act = int(rng.integers(0, 3))
         want = oracle.fully_connected(x, w, b, act=act, **kws)
-        got = TC.gpu_fully_connected(x, w, b, act=act, want_kernel="fc_mfma_i8_256x256x128", **kws)
-        assert np.array_equal(got, want), (i, m, k, n, mode, act, int((got != want).sum()))
+        tile_m = "128" if i % 2 else "256"   # (its own choice here is 256: fewer than 1024 tiles)
+        monkeypatch.setenv("TVX_FC_TILE_M", tile_m)
+        got = TC.gpu_fully_connected(x, w, b, act=act, want_kernel="fc_mfma_i8_%sx256x128" % tile_m, **kws)
+        assert np.array_equal(got, want), (i, m, k, n, mode, act, tile_m, int((got != want).sum()))
 
 
 def test_pool2d_sweep(oracle):

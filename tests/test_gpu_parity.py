@@ -374,23 +374,32 @@ def test_fully_connected_mfma_edges(oracle, mode, shape, kernel):
     assert len(np.unique(want)) > 4
 
 
+@pytest.mark.parametrize("mode", ["i8pc", "u8", "u8pc", "i8zp"])
 @pytest.mark.parametrize("shape", [(600, 512, 528), (513, 144, 769), (1025, 16, 300), (130, 336, 2050), (385, 1040, 700)])
-def test_fully_connected_128_row_tiles(oracle, shape, monkeypatch):
-    """The 128 x 256 tile form of the int8 kernel (its own choice from 1024 tiles up) on small ragged shapes: M, N not
-    multiples of the tile, reductions of one 16-byte chunk, with a tail, of an odd and an even count of k-tiles
-    (its weight slots come in pairs). The same shapes on 256-row tiles give the same bytes."""
+def test_fully_connected_128_row_tiles(oracle, shape, mode, monkeypatch):
+    """The 128 x 256 tile form of the quantized kernel (its own choice from 1024 tiles up) on small ragged shapes: M, N
+    not multiples of the tile, reductions of one 16-byte chunk, with a tail, of an odd and an even count of k-tiles
+    (its weight slots come in pairs); int8 and uint8 activations, per-channel weights and a uniform weight zero point
+    (re-bias and row sums one piece at a time). The same shapes on 256-row tiles give the same bytes."""
     m, k, n = shape
     rng = np.random.default_rng(m * 7 + k + n)
-    x, w = rand_q(rng, m * k, 1), rand_q(rng, n * k, 1)
+    in_dt = 0 if mode.startswith("u8") else 1
+    w_dt = 0 if mode == "u8" else 1
+    x, w = rand_q(rng, m * k, in_dt), rand_q(rng, n * k, w_dt)
     b = rng.integers(-16384, 16385, n).astype(np.int32)
-    ws = np.exp(rng.uniform(np.log(0.001), np.log(0.02), n)).astype(np.float32)
-    kws = dict(m=m, k=k, n=n, in_dtype=1, w_dtype=1, out_dtype=1, in_q=(0.02, -2), w_q=(1.0, 0, ws),
-               out_q=(float(np.float32(0.02 * 0.01 * 40 * np.sqrt(k))), 3))
+    if mode == "u8":
+        wq = (0.01, 117, None)
+    elif mode == "i8zp":
+        wq = (0.01, -9, None)
+    else:
+        wq = (1.0, 0, np.exp(rng.uniform(np.log(0.001), np.log(0.02), n)).astype(np.float32))
+    kws = dict(m=m, k=k, n=n, in_dtype=in_dt, w_dtype=w_dt, out_dtype=in_dt, in_q=(0.02, 131 if in_dt == 0 else -2), w_q=wq,
+               out_q=(float(np.float32(0.02 * 0.01 * 40 * np.sqrt(k))), 5 if in_dt == 0 else 3))
     for act in (0, 1, 2):
         want = oracle.fully_connected(x, w, b, act=act, **kws)
         monkeypatch.setenv("TVX_FC_TILE_M", "128")
         got = TC.gpu_fully_connected(x, w, b, act=act, want_kernel="fc_mfma_i8_128x256x128", **kws)
-        assert np.array_equal(got, want), int((got != want).sum())
+        assert np.array_equal(got, want), (mode, act, int((got != want).sum()))
         monkeypatch.setenv("TVX_FC_TILE_M", "256")
         assert np.array_equal(TC.gpu_fully_connected(x, w, b, act=act, want_kernel="fc_mfma_i8_256x256x128", **kws), want)
     assert len(np.unique(want)) > 4
@@ -398,8 +407,8 @@ def test_fully_connected_128_row_tiles(oracle, shape, monkeypatch):
 
 def test_fully_connected_full_size_uint8_asymmetric(oracle):
     """M=8192, K=4096, N=4096 uint8 with a uniform weight zero point: the variant whose activations are re-biased
-    and summed per row inside the kernel, one k-tile ahead of the multiplications, over all 32 k-tiles and both
-    tiles of a CU. A seeded sample of rows against the oracle, every tile row covered."""
+    and summed per row inside the kernel, one k-tile ahead of the multiplications, over all 32 k-tiles, on 128-row
+    tiles (two workgroups per CU). A seeded sample of rows against the oracle, every one of the 64 tile rows covered."""
     m, k, n = 8192, 4096, 4096
     rng = np.random.default_rng(0x76)
     x = rng.integers(0, 256, m * k, dtype=np.uint8)
@@ -407,8 +416,8 @@ def test_fully_connected_full_size_uint8_asymmetric(oracle):
     b = rng.integers(-16384, 16385, n).astype(np.int32)
     kws = dict(k=k, n=n, in_dtype=0, w_dtype=0, out_dtype=0, in_q=(0.02, 121), w_q=(0.01, 131, None),
                out_q=(1.2, 128))
-    got = TC.gpu_fully_connected(x, w, b, m=m, want_kernel="fc_mfma_i8_256x256x128", **kws).reshape(m, n)
-    rows = np.sort(np.concatenate([np.arange(32) * 256 + rng.integers(0, 256, 32), rng.choice(m, 16, replace=False)]))
+    got = TC.gpu_fully_connected(x, w, b, m=m, want_kernel="fc_mfma_i8_128x256x128", **kws).reshape(m, n)
+    rows = np.sort(np.concatenate([np.arange(64) * 128 + rng.integers(0, 128, 64), rng.choice(m, 8, replace=False)]))
     want = oracle.fully_connected(np.ascontiguousarray(x.reshape(m, k)[rows]).ravel(), w, b, m=len(rows), **kws)
     assert np.array_equal(got[rows], want.reshape(len(rows), n))
     assert len(np.unique(got)) > 100

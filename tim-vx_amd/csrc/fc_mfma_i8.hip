@@ -16,10 +16,10 @@
 // the matrix cores, whose clock drops under random data, plus ~10 % for the barrier per
 // k-tile); prologue and epilogue of a tile cost ~9 us next to ~60 us of k-loop.
 //
-// Int8 activations with per-channel or zero-point-free weights also have a 128 x 256 form (MB = 4
-// activation blocks instead of 8): half the accumulators and two weight slots instead of three fit
-// two wavefronts per SIMD, i.e. two workgroups per CU, so that one tile's prologue, barriers and
-// epilogue run under the other's MFMAs. It is taken when there are 1024 such tiles and more.
+// The quantized variants also have a 128 x 256 form (MB = 4 activation blocks instead of 8): half
+// the accumulators and two weight slots instead of three fit two wavefronts per SIMD, i.e. two
+// workgroups per CU, so that one tile's prologue, barriers, in-place pass and epilogue run under
+// the other's MFMAs. It is taken when there are 1024 such tiles and more.
 //
 // The MFMA "A" operand is the weight fragment and "B" the activation fragment,
 // so a lane ends up with one activation row m and, per accumulator quad, four
@@ -97,9 +97,10 @@ __global__ void __launch_bounds__(kThreads, MB == 8 ? 1 : 2) FcMfmaKernel(FcArgs
   typedef typename std::conditional<F16, v16f, v16i>::type acc_t;
   typedef Geo<MB> G;
   // The 128-row form holds 128 accumulator, 64 weight and 32 activation registers of the 256 a wavefront has at two
-  // per SIMD; the in-place pass of the uint8 / row-sum variants does not fit beside them, and a register the
-  // compiler spills while one of this kernel's hand-waited loads is still writing it would be saved too early.
-  static_assert(MB == 8 || (MB == 4 && !X_U8 && !ROWSUM && !F16), "128-row tiles: int8 activations without row sums only");
+  // per SIMD; the in-place pass of the uint8 / row-sum variants fits beside them with one piece in flight at a time.
+  // (A register the compiler spilled while one of this kernel's hand-waited loads is still writing it would be saved
+  // too early: every variant must build without spills.)
+  static_assert(MB == 8 || (MB == 4 && !F16), "128-row tiles: the quantized variants only");
   constexpr int TM = G::TM, S = G::kSlots, P = G::kOps;
   constexpr int kTileBytes = G::kTileBytes, kTabOffset = G::kTabOffset, kRowsumOffset = G::kRowsumOffset;
   constexpr int kWaveRows = TM / 4;  // activation rows a wavefront fetches (and rewrites in place)
@@ -146,13 +147,13 @@ __global__ void __launch_bounds__(kThreads, MB == 8 ? 1 : 2) FcMfmaKernel(FcArgs
   // [64 w, 64 w + 64) per k-tile (8 instructions).
   const int dma_row = lane >> 3;
   uint32_t off_x[MB];  // byte offsets from the tensor base (tensors are < 4 GiB)
-  int dma_chunk[2];   // source chunk of this lane for even / odd instructions
+  // LDS slot (row r, position lane & 7) holds chunk (lane & 7) ^ ((r >> 1) & 7) of the row (a wavefront's rows begin
+  // at a multiple of 16: the chunk depends on the piece and the lane only)
+  auto dma_chunk = [&](int i) { return (lane & 7) ^ (((i * 8 + dma_row) >> 1) & 7); };
 #pragma unroll
   for (int i = 0; i < MB; ++i) {
     const int r = wave * kWaveRows + i * 8 + dma_row;
-    // LDS slot (row r, position lane & 7) holds chunk (lane & 7) ^ ((r >> 1) & 7) of the row
-    const int chunk = (lane & 7) ^ ((r >> 1) & 7);
-    dma_chunk[i & 1] = chunk;
+    const int chunk = dma_chunk(i);
     const int xm = min(m0 + r, a.M - 1);  // rows past the edge are computed and dropped
     off_x[i] = static_cast<uint32_t>(xm) * static_cast<uint32_t>(a.K) + chunk * 16;
   }
@@ -172,7 +173,7 @@ __global__ void __launch_bounds__(kThreads, MB == 8 ? 1 : 2) FcMfmaKernel(FcArgs
       return;
     }
     // branch-free: the address is blended from the two candidates with a mask
-    const bool past = (kt >= k_tiles) | (k_tail & (k0 + dma_chunk[i & 1] * 16 >= a.K));
+    const bool past = (kt >= k_tiles) | (k_tail & (k0 + dma_chunk(i) * 16 >= a.K));
     const uintptr_t real = reinterpret_cast<uintptr_t>(a.x) + (off_x[i] + static_cast<uint32_t>(k0));
     const uintptr_t zero = reinterpret_cast<uintptr_t>(a.zeros) + (X_U8 ? 128 : 0);
     const uintptr_t take_zero = past ? ~uintptr_t{0} : uintptr_t{0};
@@ -298,7 +299,7 @@ __global__ void __launch_bounds__(kThreads, MB == 8 ? 1 : 2) FcMfmaKernel(FcArgs
   };
 #undef TVX_DS_READ
 #undef TVX_DS_WRITE
-  v4i pc[3];  // pieces on their way through the pass
+  v4i pc[MB == 8 ? 3 : 1];  // pieces on their way through the pass (128 rows: one at a time)
   // One k-step: 16 MFMAs of 32 cycles each, and everything else the k-step has to issue dealt out
   // between them, a few instructions at a time (the compiler, left to itself, gathers them into two
   // runs per k-step; memory instructions issued in a burst queue up with the wavefront waiting behind
@@ -327,23 +328,42 @@ __global__ void __launch_bounds__(kThreads, MB == 8 ? 1 : 2) FcMfmaKernel(FcArgs
           if constexpr (decltype(newer)::value != 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"((S - 2) * P) : "memory");
           else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
+        if constexpr (MB == 8) {
 #pragma unroll
-        for (int j = 0; j < 3; ++j)
-          if (j < pieces) piece_read(kt + 1, first + j, pc[j]);
+          for (int j = 0; j < 3; ++j)
+            if (j < pieces) piece_read(kt + 1, first + j, pc[j]);
+        } else {
+          if (pieces > 0) piece_read(kt + 1, first, pc[0]);
+        }
       }
       if (kPrefetch && mb == MB / 2) dma_piece(whole, kt + S, MB == 8 ? kk * 2 : kk);
       if (kPass && mb == MB - 2 && pieces > 0) {
         // (the pieces are operands of the wait: nothing that uses them may be moved in front of it)
-        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(pc[0]), "+v"(pc[1]), "+v"(pc[2])::"memory");
-        piece_finish(kt + 1, first, pc[0]);
+        if constexpr (MB == 8) {
+          asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(pc[0]), "+v"(pc[1]), "+v"(pc[2])::"memory");
+          piece_finish(kt + 1, first, pc[0]);
+        } else {
+          asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(pc[0])::"memory");
+          piece_finish(kt + 1, first, pc[0]);
+          if (pieces > 1) piece_read(kt + 1, first + 1, pc[0]);  // (the second piece of k-step 0 follows through the same registers)
+        }
       }
-      if (kPass && mb == MB - 1 && pieces > 2) piece_finish(kt + 1, first + 2, pc[2]);
+      if constexpr (MB == 8) {
+        if (kPass && mb == MB - 1 && pieces > 2) piece_finish(kt + 1, first + 2, pc[2]);
+      } else {
+        if (kPass && mb == MB - 1 && pieces > 1) {
+          asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(pc[0])::"memory");
+          piece_finish(kt + 1, first + 1, pc[0]);
+        }
+      }
       if (kPrefetch && mb == MB - 1) w_piece(kt + S, 0, kk, w_slot[kk]);
       __builtin_amdgcn_sched_barrier(0);
       acc[1][mb] = Mfma(w_slot[4 + kk], fx[mb], acc[1][mb]);
       if (kNext && mb < MB / 2) load_frag(next_kt, next_kk, fx_next, 2 * mb + 1);
       if (MB == 8 && kPrefetch && mb == MB / 2 + 1) dma_piece(whole, kt + S, kk * 2 + 1);
-      if (kPass && mb == MB - 2 && pieces > 1) piece_finish(kt + 1, first + 1, pc[1]);
+      if constexpr (MB == 8) {
+        if (kPass && mb == MB - 2 && pieces > 1) piece_finish(kt + 1, first + 1, pc[1]);
+      }
       if (kPrefetch && mb == MB - 1) w_piece(kt + S, 1, kk, w_slot[4 + kk]);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -396,11 +416,20 @@ __global__ void __launch_bounds__(kThreads, MB == 8 ? 1 : 2) FcMfmaKernel(FcArgs
     // the in-place pass over k-tile 0 (every later k-tile gets it while the one before multiplies)
 #pragma unroll
     for (int i = 0; i < MB; i += 2) {
-      piece_read(0, i, pc[0]);
-      piece_read(0, i + 1, pc[1]);
-      asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(pc[0]), "+v"(pc[1])::"memory");
-      piece_finish(0, i, pc[0]);
-      piece_finish(0, i + 1, pc[1]);
+      if constexpr (MB == 8) {
+        piece_read(0, i, pc[0]);
+        piece_read(0, i + 1, pc[1]);
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(pc[0]), "+v"(pc[1])::"memory");
+        piece_finish(0, i, pc[0]);
+        piece_finish(0, i + 1, pc[1]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          piece_read(0, i + j, pc[0]);
+          asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(pc[0])::"memory");
+          piece_finish(0, i + j, pc[0]);
+        }
+      }
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   }
@@ -660,21 +689,21 @@ TileKernel TileKernelOf(int rq) {
   if (rq == kRqFast) return FcMfmaKernel<MB, X_U8, ROWSUM, kRqFast>;
   return FcMfmaKernel<MB, X_U8, ROWSUM, kRqGeneric>;
 }
-// mb: the tile's 32-row activation blocks (8, or 4 for int8 activations without row sums)
+// mb: the tile's 32-row activation blocks (8, or 4 for the quantized variants)
 TileKernel TileKernelOf(int mb, bool f16, bool x_u8, bool rowsum, int rq) {
   if (f16) return FcMfmaKernel<8, false, false, kRqGeneric, true>;
-  if (x_u8 && rowsum) return TileKernelOf<8, true, true>(rq);
-  if (x_u8) return TileKernelOf<8, true, false>(rq);
-  if (rowsum) return TileKernelOf<8, false, true>(rq);
+  if (x_u8 && rowsum) return mb == 8 ? TileKernelOf<8, true, true>(rq) : TileKernelOf<4, true, true>(rq);
+  if (x_u8) return mb == 8 ? TileKernelOf<8, true, false>(rq) : TileKernelOf<4, true, false>(rq);
+  if (rowsum) return mb == 8 ? TileKernelOf<8, false, true>(rq) : TileKernelOf<4, false, true>(rq);
   return mb == 8 ? TileKernelOf<8, false, false>(rq) : TileKernelOf<4, false, false>(rq);
 }
 int TileLdsBytes(int mb) { return mb == 8 ? Geo<8>::kLdsBytes : Geo<4>::kLdsBytes; }
 int TileSlots(int mb) { return mb == 8 ? Geo<8>::kSlots : Geo<4>::kSlots; }
 
-// 128-row tiles (the variant that has them) where there are enough to give every CU two workgroups twice over;
-// TVX_FC_TILE_M=128|256 overrides (a test lever, read when the operator is created).
-int ChooseTileBlocks(uint32_t m, uint32_t n, bool plain_int8) {
-  if (!plain_int8) return 8;
+// 128-row tiles (the quantized variants have them) where there are enough to give every CU two workgroups twice
+// over; TVX_FC_TILE_M=128|256 overrides (a test lever, read when the operator is created).
+int ChooseTileBlocks(uint32_t m, uint32_t n, bool quantized) {
+  if (!quantized) return 8;
   int mb = static_cast<uint64_t>((m + 127) / 128) * ((n + TN - 1) / TN) >= 1024 ? 4 : 8;
   if (const char* f = getenv("TVX_FC_TILE_M")) {
     const int v = atoi(f);
@@ -815,7 +844,7 @@ int FcMfmaSetup(tvx_op* op, const tvx_fc_desc* d, const void* w_host, const void
                                      static_cast<int>(n_alloc), d->out_zp, &rqt,
                                      AccumulatorBound(d->k, bias_host, d->n));
   // the tiled kernel reads fragment order, the small-tile kernel plain rows
-  const int mb = ChooseTileBlocks(d->m, d->n, d->in_dtype != TVX_U8 && zws == 0);
+  const int mb = ChooseTileBlocks(d->m, d->n, true);
   int s;
   if (UseSmallTiles(*d)) {
     s = op->packed.Upload(ws.data(), wn);
