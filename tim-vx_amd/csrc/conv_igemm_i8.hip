@@ -423,8 +423,8 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(O
         }
         int r4[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) r4[e] = Requant8<RQ>(acc[i][j][g * 4 + e] + (bias - s4[e]), q, a.out_zp, lo, hi);
-        *reinterpret_cast<uint32_t*>(out_tile + ocl * a.out_stride + pl) = PackBytes(r4[0], r4[1], r4[2], r4[3]);
+        for (int e = 0; e < 4; ++e) r4[e] = acc[i][j][g * 4 + e] + (bias - s4[e]);
+        *reinterpret_cast<uint32_t*>(out_tile + ocl * a.out_stride + pl) = RequantPack4<RQ>(r4, q, a.out_zp, lo, hi);
       }
     }
   }
@@ -699,8 +699,8 @@ ConvPersistKernel(ConvArgs a) {
             int r4[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-              r4[e] = Requant8<RQ>(ZP ? acc[j][g * 4 + e] - s4[e] : acc[j][g * 4 + e], rq, a.out_zp, a.lo, a.hi);
-            *reinterpret_cast<uint32_t*>(out_tile + ocl * a.out_stride + pl) = PackBytes(r4[0], r4[1], r4[2], r4[3]);
+              r4[e] = ZP ? acc[j][g * 4 + e] - s4[e] : acc[j][g * 4 + e];
+            *reinterpret_cast<uint32_t*>(out_tile + ocl * a.out_stride + pl) = RequantPack4<RQ>(r4, rq, a.out_zp, a.lo, a.hi);
           }
         }
         if (ZP) __builtin_amdgcn_wave_barrier();  // the sums are read before the next MFMA tile's are written

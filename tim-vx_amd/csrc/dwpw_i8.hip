@@ -148,7 +148,7 @@ __device__ __forceinline__ void PatchCompute(const DwPwArgs& a, const ChannelCon
       win[r][2] = Window<4 + S * 2 - PL>(raw[S * o + r]);
       win[r][3] = Window<4 + S * 3 - PL>(raw[S * o + r]);
     }
-    int accs[4], outs[4];
+    int accs[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       int acc = Dot4Add(win[0][i], wk0, bias);
@@ -162,8 +162,7 @@ __device__ __forceinline__ void PatchCompute(const DwPwArgs& a, const ChannelCon
       }
       accs[i] = acc;
     }
-    Requant8x4(accs, q, a.dw_out_zp, a.dw_lo, a.dw_hi, a.dw_ties, outs);
-    packed[o] = PackBytes(outs[0], outs[1], outs[2], outs[3]);
+    packed[o] = Requant8x4Pack(accs, q, a.dw_out_zp, a.dw_lo, a.dw_hi, a.dw_ties);
   }
 }
 
@@ -304,9 +303,7 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2
       for (int gq = 0; gq < 4; ++gq) {
         const int pl = 8 * gq + 4 * frag_half;
         const int av[4] = {acc[gq * 4], acc[gq * 4 + 1], acc[gq * 4 + 2], acc[gq * 4 + 3]};
-        int v[4];
-        Requant8x4(av, q, a.out_zp, a.lo, a.hi, a.pw_ties, v);
-        *reinterpret_cast<uint32_t*>(stage + frag_row * kStageStride + pl) = PackBytes(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<uint32_t*>(stage + frag_row * kStageStride + pl) = Requant8x4Pack(av, q, a.out_zp, a.lo, a.hi, a.pw_ties);
       }
       __builtin_amdgcn_wave_barrier();
       {

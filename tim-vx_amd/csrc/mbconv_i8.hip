@@ -212,10 +212,8 @@ __global__ void __launch_bounds__(kThreads, (MO * NTMAX <= 5 ? 2 : 1)) MbConvKer
 #pragma unroll
     for (int gq = 0; gq < 4; ++gq) {
       const int av[4] = {acc[gq * 4], acc[gq * 4 + 1], acc[gq * 4 + 2], acc[gq * 4 + 3]};
-      int v[4];
-      Requant8x4(av, rq1, a.e_zp, a.e_lo, a.e_hi, a.ties1, v);
       *reinterpret_cast<uint32_t*>(e_w + frow * a.ep + mt * 32 + 8 * gq + 4 * fh) =
-          PackBytes(v[0], v[1], v[2], v[3]) ^ static_cast<uint32_t>(a.e_xor4);
+          Requant8x4Pack(av, rq1, a.e_zp, a.e_lo, a.e_hi, a.ties1) ^ static_cast<uint32_t>(a.e_xor4);
     }
   };
   for (int chunk = wave; chunk < a.chunks; chunk += kWaves) {
@@ -348,14 +346,14 @@ __global__ void __launch_bounds__(kThreads, (MO * NTMAX <= 5 ? 2 : 1)) MbConvKer
     if (u >= units) break;
     const int t = u / (MO * 4), gq = u & 3;
     const int oc = t * 32 + frow;
-    int av[4], v[4];
+    int av[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) av[e] = red[((u >> 2) * 16 + gq * 4 + e) * 64 + lane] + bias3[i];
-    Requant8x4(av, rq3[i], a.out_zp, a.lo, a.hi, a.ties3, v);
+    const uint32_t codes = Requant8x4Pack(av, rq3[i], a.out_zp, a.lo, a.hi, a.ties3);
     if (oc >= a.Cout) continue;
     if (a.aligned4) {
       if (px0[i] < po) {
-        uint32_t o = PackBytes(v[0], v[1], v[2], v[3]);
+        uint32_t o = codes;
         if (ADD) o = AddResidual4(a, o, resv[i]);
         *reinterpret_cast<uint32_t*>(a.y + at[i]) = o;
       }
@@ -363,7 +361,7 @@ __global__ void __launch_bounds__(kThreads, (MO * NTMAX <= 5 ? 2 : 1)) MbConvKer
 #pragma unroll
       for (int e = 0; e < 4; ++e)
         if (px0[i] + e < po) {
-          int o = v[e] & 0xff;
+          int o = static_cast<int>((codes >> (8 * e)) & 0xff);
           if (ADD) o = AddResidual1(a, o, static_cast<int>((resv[i] >> (8 * e)) & 0xff));
           a.y[at[i] + e] = static_cast<uint8_t>(o);
         }

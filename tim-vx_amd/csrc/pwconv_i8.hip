@@ -267,9 +267,8 @@ __global__ void __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu((P
         const int pl = i * 32 + 8 * g + 4 * frag_half;
         int v[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          v[e] = Requant8<RQ>(acc[i][g * 4 + e] + (kSplitZp ? accz[i][g * 4 + e] : 0), q, a.out_zp, lo, hi);
-        *reinterpret_cast<uint32_t*>(stage + frag_row * kStageStride + pl) = PackBytes(v[0], v[1], v[2], v[3]);
+        for (int e = 0; e < 4; ++e) v[e] = acc[i][g * 4 + e] + (kSplitZp ? accz[i][g * 4 + e] : 0);
+        *reinterpret_cast<uint32_t*>(stage + frag_row * kStageStride + pl) = RequantPack4<RQ>(v, q, a.out_zp, lo, hi);
       }
     __builtin_amdgcn_wave_barrier();
     // copy-out: rows of the staging patch -> WHCN output
@@ -456,10 +455,8 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(2, 2)))
       for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          int v[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) v[e] = Requant8<RQ>(acc[i][g * 4 + e], q, a.out_zp, lo, hi);
-          *reinterpret_cast<uint32_t*>(stage + frag_row * kStageStride + i * 32 + 8 * g + 4 * frag_half) = PackBytes(v[0], v[1], v[2], v[3]);
+          const int v[4] = {acc[i][g * 4], acc[i][g * 4 + 1], acc[i][g * 4 + 2], acc[i][g * 4 + 3]};
+          *reinterpret_cast<uint32_t*>(stage + frag_row * kStageStride + i * 32 + 8 * g + 4 * frag_half) = RequantPack4<RQ>(v, q, a.out_zp, lo, hi);
         }
       __builtin_amdgcn_wave_barrier();
       const int rows = min(32, a.OC - tile * 32);

@@ -159,6 +159,29 @@ __device__ __forceinline__ int Requant8(int v, const tvx_v4i& q, int zp, int lo,
   return Med3(r, lo, hi);
 }
 
+// Four accumulators of one channel -> their four codes in one dword. Where no accumulator can land on a tie the clamp
+// comes in front of the shift (bounds shifted up; a loop over the channel's pixels hoists them) and the shift writes
+// its byte of the dword: four instructions a code - high multiply, rounding constant, clamp, shift - and no packing.
+template <int RQ>
+__device__ __forceinline__ uint32_t RequantPack4(const int (&v)[4], const tvx_v4i& q, int zp, int lo, int hi) {
+  if (RQ == kRqFastNoTie) {
+    const int lo_t = lo << q[1], hi_t = ((hi + 1) << q[1]) - 1;
+    int u[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) u[e] = Med3(__mulhi(v[e], q[0]) + q[2], lo_t, hi_t);
+    uint32_t d;
+    ShiftIntoByte<0>(d, q[1], u[0]);
+    ShiftIntoByte<1>(d, q[1], u[1]);
+    ShiftIntoByte<2>(d, q[1], u[2]);
+    ShiftIntoByte<3>(d, q[1], u[3]);
+    return d;
+  }
+  int r[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) r[e] = Requant8<RQ>(v[e], q, zp, lo, hi);
+  return PackBytes(r[0], r[1], r[2], r[3]);
+}
+
 // Four accumulators of one channel requantized together (the 32-bit record forms). `ties` (wave-uniform: a kernel
 // argument) tells whether any accumulator of the operator can land on an exact .5: only then is the round-half-even
 // fix-up executed.
@@ -180,6 +203,14 @@ __device__ __forceinline__ void Requant8x4(const int (&v)[4], const tvx_v4i& q, 
   }
 #pragma unroll
   for (int e = 0; e < 4; ++e) out[e] = Med3(r[e], lo, hi);
+}
+
+// ... and into one dword (`ties` as above: without ties the clamp-before-shift form, which needs no packing)
+__device__ __forceinline__ uint32_t Requant8x4Pack(const int (&v)[4], const tvx_v4i& q, int zp, int lo, int hi, int ties) {
+  if (!ties) return RequantPack4<kRqFastNoTie>(v, q, zp, lo, hi);
+  int out[4];
+  Requant8x4(v, q, zp, lo, hi, ties, out);
+  return PackBytes(out[0], out[1], out[2], out[3]);
 }
 
 // The quantized Add fused behind a convolution: one code of the convolution's result (t) and one of the residual
