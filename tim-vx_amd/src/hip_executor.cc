@@ -10,6 +10,7 @@
 // Execute() is vsi_nn_RunGraph -> vxProcessGraph (vsi_nn_graph.c:1605-1639):
 // inputs go host -> device, operators run in order on one stream, outputs come
 // back, and the call returns when everything is visible to the host.
+#include <atomic>
 #include <chrono>
 #include <cmath>
 #include <cstdlib>
@@ -26,6 +27,9 @@ namespace vx {
 namespace {
 
 double g_last_device_ms = 0.0;
+// Profiling of Graph::Run(): -1 follows TVX_RUNTIME_PROFILE in the environment (unset: off, "ops": per operator, anything
+// else: the operator sequence as a whole); 0 / 1 / 2 are set by tvx_runtime_set_profile().
+std::atomic<int> g_profile_mode{-1};
 // Per-operator device time of the most recent Graph::Run() (TVX_RUNTIME_PROFILE=ops): name and microseconds.
 std::vector<std::pair<std::string, double>> g_last_op_us;
 std::vector<uint64_t> g_last_op_bytes;
@@ -363,6 +367,8 @@ class HipExecutor : public Executor {
     // With TVX_RUNTIME_PROFILE set, the operator sequence is timed on its own
     // (uploads drained first), for tools that report device time per Run().
     std::chrono::steady_clock::time_point t0;
+    const int profile_mode = ProfileMode();
+    const bool profile_ = profile_mode >= 1, profile_ops_ = profile_mode == 2;
     if (profile_) {
       if (tvx_stream_synchronize(stream_) != TVX_OK) return Fail("sync");
       t0 = std::chrono::steady_clock::now();
@@ -819,8 +825,14 @@ class HipExecutor : public Executor {
   }
 
   void* stream_ = nullptr;
-  bool profile_ = std::getenv("TVX_RUNTIME_PROFILE") != nullptr;
-  bool profile_ops_ = profile_ && std::string(std::getenv("TVX_RUNTIME_PROFILE")) == "ops";
+  static int ProfileMode() {
+    static const int from_env = [] {
+      const char* e = std::getenv("TVX_RUNTIME_PROFILE");
+      return !e ? 0 : (std::string(e) == "ops" ? 2 : 1);
+    }();
+    const int m = g_profile_mode.load(std::memory_order_relaxed);
+    return m >= 0 ? m : from_env;
+  }
   std::vector<void*> events_;
   std::vector<Step> steps_;
   std::map<TensorImpl*, void*> dev_;    // tensor -> device pointer (possibly an alias)
@@ -854,6 +866,9 @@ struct OfferPinnedMemory {
 // Milliseconds the operator sequence of the most recent Graph::Run() took on the
 // device (0 unless TVX_RUNTIME_PROFILE is set). No counterpart in the reference.
 extern "C" double tvx_runtime_last_device_ms(void) { return tim::vx::g_last_device_ms; }
+// Profiling of the following Graph::Run() calls: 0 off (no synchronisation inside a Run() beyond its last one), 1 the
+// operator sequence as a whole, 2 per operator, -1 back to what TVX_RUNTIME_PROFILE says. No counterpart in the reference.
+extern "C" void tvx_runtime_set_profile(int mode) { tim::vx::g_profile_mode.store(mode < -1 || mode > 2 ? -1 : mode); }
 // Operators of the most recent Graph::Run() with their device time (TVX_RUNTIME_PROFILE=ops): count, then
 // name and microseconds of operator i. No counterpart in the reference's API (its driver keeps such numbers
 // per vx_node).

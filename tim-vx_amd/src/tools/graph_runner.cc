@@ -46,6 +46,7 @@
 #include "tim/vx/tensor.h"
 
 extern "C" double tvx_runtime_last_device_ms(void);
+extern "C" void tvx_runtime_set_profile(int mode);
 extern "C" int tvx_runtime_last_op_count(void);
 extern "C" const char* tvx_runtime_last_op_name(int i);
 extern "C" double tvx_runtime_last_op_us(int i);
@@ -153,7 +154,6 @@ static int RunThreads(int n_threads, bool lock, const char* graphs_path, const c
 }
 
 int main(int argc, char** argv) {
-  setenv("TVX_RUNTIME_PROFILE", "1", 0);  // makes `bench` report the device part of Run()
   if (argc >= 2 && std::string(argv[1]) == "--threads") {
     const bool lock = !(argc >= 4 && std::string(argv[3]) == "--no-lock");
     const int first = lock ? 3 : 4;
@@ -457,10 +457,18 @@ static int RunFile(const char* graphs_path, const char* blob_path, const char* o
           if (kv.second.is_input && kv.second.len && !kv.second.handle && !kv.second.th)
             kv.second.tensor->CopyDataToTensor(blob.data() + kv.second.off, static_cast<uint32_t>(kv.second.len));
       };
+      // two passes: Run() as an application calls it (no profiling: one synchronisation, at its end) for the time per
+      // Run(); then with the operator sequence timed on its own (a synchronisation in front of it and behind it)
+      tvx_runtime_set_profile(0);
+      for (int i = 0; i < warmup; ++i) { feed(); graph->Run(); }
+      auto t0 = std::chrono::steady_clock::now();
+      for (int i = 0; i < iters; ++i) { feed(); graph->Run(); }
+      auto t1 = std::chrono::steady_clock::now();
+      const char* env_profile = std::getenv("TVX_RUNTIME_PROFILE");
+      tvx_runtime_set_profile(env_profile && std::string(env_profile) == "ops" ? 2 : 1);
       for (int i = 0; i < warmup; ++i) { feed(); graph->Run(); }
       double dev_ms = 0;
       std::vector<double> op_us;
-      auto t0 = std::chrono::steady_clock::now();
       for (int i = 0; i < iters; ++i) {
         feed();
         graph->Run();
@@ -469,7 +477,7 @@ static int RunFile(const char* graphs_path, const char* blob_path, const char* o
         op_us.resize(static_cast<size_t>(n_ops), 0.0);
         for (int o = 0; o < n_ops; ++o) op_us[static_cast<size_t>(o)] += tvx_runtime_last_op_us(o);
       }
-      auto t1 = std::chrono::steady_clock::now();
+      tvx_runtime_set_profile(-1);
       std::fprintf(log, "bench %s %.6f %.6f\n", name.c_str(),
                   std::chrono::duration<double, std::milli>(t1 - t0).count() / iters, dev_ms / iters);
       for (size_t o = 0; o < op_us.size(); ++o) {
