@@ -332,3 +332,30 @@ def test_conv2d_band_sweep(oracle, tvx, monkeypatch):
         ran += 1
         assert np.array_equal(got, want), (i, cfg, mode, act, int((got != want).sum()))
     assert ran >= 25, ran
+
+
+def test_max_pool_register_stencil_sweep(oracle):
+    """Stride-2 max pooling with 2- and 3-tap windows on rows of whole 8-byte units (the register-stencil kernel): random
+    plane sizes from one lane to a whole wavefront per row and from one to hundreds of rows, pads 0 / 1 in front, output
+    widths from as wide as the input allows down to narrower declared ones (rows that end inside a lane's four outputs),
+    both code types, equal and different quantization on the two sides."""
+    rng = np.random.default_rng(0x57E)
+    for i in range(80):
+        w, h = 8 * int(rng.integers(1, 65)), int(rng.integers(2, 140 if i % 4 else 700))
+        kw, kh = int(rng.integers(2, 4)), int(rng.integers(2, 4))
+        pl, pt = int(rng.integers(0, 2)), int(rng.integers(0, 2))
+        pr, pb = int(rng.integers(0, 2)), int(rng.integers(0, 2))
+        out_w = min((w + pl + pr - kw) // 2 + 1, w // 2) - int(rng.integers(0, 3)) * int(rng.random() < 0.3)
+        out_h = (h + pt + pb - kh) // 2 + 1
+        if out_w < 1 or out_h < 1 or (out_h - 1) * 2 - pt > h - 1:
+            continue
+        c, n = int(rng.integers(1, 7)), int(rng.integers(1, 4))
+        dtype = int(rng.integers(0, 2))
+        kws = dict(in_shape=[w, h, c, n], out_shape=[out_w, out_h, c, n], ksize=[kw, kh], stride=[2, 2],
+                   pad_left=pl, pad_top=pt, pool_type=0, dtype=dtype)
+        x = rand_q(rng, w * h * c * n, dtype)
+        in_q = (0.1, 7)
+        out_q = (0.1, 7) if rng.random() < 0.6 else (0.07, 9 if dtype == 0 else -2)
+        want = oracle.pool2d(x, in_q=in_q, out_q=out_q, **kws)
+        got = TC.gpu_pool2d(x, in_q=in_q, out_q=out_q, want_kernel="pool2d_stencil_i8", **kws)
+        assert np.array_equal(got, want), (i, kws, out_q, int((got != want).sum()))
