@@ -313,6 +313,26 @@ typedef struct tvx_transpose_desc {
 
 int tvx_transpose_create(const tvx_transpose_desc* desc, tvx_op** op);
 
+/* ---- channel-blocked tensors ------------------------------------------------------------------- */
+/* A TRANSIENT tensor of the reference's graph has no host image (src/tim/vx/tensor.cc: its data can neither
+ * be written nor read by the application), so the order of its bytes is the runtime's own business, as it is
+ * the closed driver's. For one-byte codes on small planes (7 x 7: 49-byte rows that no load is aligned to) this
+ * library offers
+ *   byte ((c / 16) * P + p) * 16 + c % 16,  p = n * H * W + y * W + x,  P = N * H * W   (channels a multiple of 16)
+ * and operators between such tensors whose results are, code for code, those of the WHCN operators:
+ *  - tvx_conv2d_blocked_create: vxConvolutionLayer (kernel/vx/convolutional.c:504-582) for a 1x1 / stride-1 /
+ *    unpadded dense convolution (input and output channels multiples of 32), optionally with the same-shape Add
+ *    behind it (`add` / `conv_operand` as for tvx_conv2d_add_create, the other operand - blocked - as in1; NULL:
+ *    no Add), or for a depthwise 3x3 / stride-1 convolution (multiplier 1, `add` NULL); constant weights;
+ *  - tvx_pool2d_blocked_create: vxPoolingLayer2 (ops/vsi_nn_op_pool.c:144-150) averaging whole unpadded planes of
+ *    at most 256 pixels: blocked in, {1, 1, C, N} out in WHCN order (byte n * C + c);
+ *  - tvx_layout_create: WHCN -> blocked (to_blocked != 0) or back; no counterpart in the reference's API.
+ * TVX_E_UNSUPPORTED: no blocked kernel for this operator (the caller keeps the tensor in WHCN). */
+int tvx_conv2d_blocked_create(const tvx_conv2d_desc* conv, const tvx_eltwise_desc* add, int conv_operand,
+                              const void* weights_host, const void* bias_host, tvx_op** op);
+int tvx_pool2d_blocked_create(const tvx_pool2d_desc* desc, tvx_op** op);
+int tvx_layout_create(uint32_t w, uint32_t h, uint32_t c, uint32_t n, int to_blocked, tvx_op** op);
+
 /* ---- running / inspecting operators ---------------------------------------- */
 /* Enqueue one execution (the per-node share of vxProcessGraph).
  * in0: activation; in1: run-time weights (conv / FC created without constant

@@ -345,7 +345,7 @@ def test_mobilenet_v2_graph_bit_exact(tmp_path, oracle, batch, res):
     assert np.array_equal(out[0], ref), int((out[0] != ref).sum())
     # the ten residual Adds ride on the projection convolutions in front of them: no Add kernel in the plan
     plan = [l for l in log.splitlines() if "uid" in l and "->" in l]
-    assert sum("pwconv_add_i8" in l for l in plan) == 10 and not any("ADD" in l for l in plan), plan
+    assert sum("pwconv_add_i8" in l or "pwconv_add_blocked_i8" in l for l in plan) == 10 and not any("ADD" in l for l in plan), plan
 
 
 def _pool_graph(name, in_shape, out_shape, pool_type, form, ksize, stride, dt="UINT8", in_q=(0.5, 12), out_q=(0.5, 12)):

@@ -119,6 +119,9 @@ def lib():
         L.tvx_mbconv_create.argtypes = [C.POINTER(Conv2dDesc), vp, vp, C.POINTER(Conv2dDesc), vp, vp, C.POINTER(Conv2dDesc), vp, vp,
                                         C.POINTER(EltwiseDesc), C.c_int, C.POINTER(vp)]
         L.tvx_conv2d_pool_create.argtypes = [C.POINTER(Conv2dDesc), C.POINTER(Pool2dDesc), vp, vp, C.POINTER(vp)]
+        L.tvx_conv2d_blocked_create.argtypes = [C.POINTER(Conv2dDesc), C.POINTER(EltwiseDesc), C.c_int, vp, vp, C.POINTER(vp)]
+        L.tvx_pool2d_blocked_create.argtypes = [C.POINTER(Pool2dDesc), C.POINTER(vp)]
+        L.tvx_layout_create.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_int, C.POINTER(vp)]
         L.tvx_fully_connected_softmax_create.argtypes = [C.POINTER(FcDesc), C.POINTER(SoftmaxDesc), vp, vp, C.POINTER(vp)]
         L.tvx_fully_connected_create.argtypes = [C.POINTER(FcDesc), vp, vp, C.POINTER(vp)]
         L.tvx_pool2d_create.argtypes = [C.POINTER(Pool2dDesc), C.POINTER(vp)]
@@ -204,6 +207,28 @@ def mbconv_create(expand, expand_w, expand_b, dw, dw_w, dw_b, project, project_w
                                   C.byref(project), _host_ptr(project_w), _host_ptr(project_b),
                                   C.byref(add_desc) if add_desc is not None else None, conv_operand, C.byref(h)))
     return Op(h)
+
+
+def conv2d_blocked_create(desc, weights, bias=None, add_desc=None, conv_operand=0):
+    """A 1x1 (optionally + Add) or depthwise 3x3 convolution between channel-blocked tensors."""
+    h = C.c_void_p()
+    check(lib().tvx_conv2d_blocked_create(C.byref(desc), C.byref(add_desc) if add_desc is not None else None, conv_operand,
+                                          _host_ptr(weights), _host_ptr(bias), C.byref(h)))
+    return Op(h)
+
+
+def pool2d_blocked_create(desc):
+    """Whole-plane average pooling of a channel-blocked tensor."""
+    h = C.c_void_p()
+    check(lib().tvx_pool2d_blocked_create(C.byref(desc), C.byref(h)))
+    return Op(h)
+
+
+def layout_create(w, h, c, n, to_blocked):
+    """WHCN planes -> channel-blocked order (to_blocked) or back."""
+    hd = C.c_void_p()
+    check(lib().tvx_layout_create(w, h, c, n, 1 if to_blocked else 0, C.byref(hd)))
+    return Op(hd)
 
 
 def conv2d_pool_create(desc, pool_desc, weights, bias=None):

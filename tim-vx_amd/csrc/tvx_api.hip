@@ -461,6 +461,107 @@ int tvx_conv2d_add_create(const tvx_conv2d_desc* d, const tvx_eltwise_desc* add,
   return TVX_OK;
 }
 
+// ---- channel-blocked tensors (an order the runtime may give TRANSIENT tensors of small planes) ----
+int tvx_conv2d_blocked_create(const tvx_conv2d_desc* d, const tvx_eltwise_desc* add, int conv_operand,
+                              const void* weights_host, const void* bias_host, tvx_op** out) {
+  if (!d || !out) return SetError(TVX_E_INVALID, "tvx_conv2d_blocked_create: null argument");
+  *out = nullptr;
+  if (add && conv_operand != 1 && conv_operand != 2)
+    return SetError(TVX_E_INVALID, "tvx_conv2d_blocked_create: conv_operand must be 1 or 2");
+  if (!d->in_w || !d->in_h || !d->in_c || !d->batch || !d->k_w || !d->k_h || !d->out_w || !d->out_h || !d->out_c ||
+      !d->stride_w || !d->stride_h || !d->dilation_w || !d->dilation_h)
+    return SetError(TVX_E_INVALID, "tvx_conv2d_blocked_create: zero extent, stride or dilation");
+  if (static_cast<uint64_t>(d->out_w - 1) * d->stride_w >= static_cast<uint64_t>(d->in_w) + d->pad_left ||
+      static_cast<uint64_t>(d->out_h - 1) * d->stride_h >= static_cast<uint64_t>(d->in_h) + d->pad_top)
+    return SetError(TVX_E_INVALID, "tvx_conv2d_blocked_create: output extent reaches past the input");
+  if (!IsQuant(d->in_dtype) || !weights_host)
+    return SetError(TVX_E_UNSUPPORTED, "tvx_conv2d_blocked_create: quantized tensors and constant weights only");
+  int s = CheckOperandTypes(d->in_dtype, d->w_dtype, d->out_dtype, "tvx_conv2d_blocked_create");
+  if (s == TVX_OK) s = CheckConvZeroPoints(d->in_dtype, d->in_zp, d->w_dtype, d->w_zp, d->w_scales != nullptr,
+                                           d->out_dtype, d->out_zp, "tvx_conv2d_blocked_create");
+  if (s == TVX_OK && add) {
+    if (add->dtype != d->out_dtype || !(add->a_scale > 0.f) || !(add->b_scale > 0.f) || !(add->out_scale > 0.f))
+      return SetError(TVX_E_UNSUPPORTED, "tvx_conv2d_blocked_create: the Add must be quantized like the convolution's output type");
+    const float conv_scale = conv_operand == 1 ? add->a_scale : add->b_scale;
+    const int32_t conv_zp = conv_operand == 1 ? add->a_zp : add->b_zp;
+    if (conv_scale != d->out_scale || conv_zp != d->out_zp)
+      return SetError(TVX_E_INVALID, "tvx_conv2d_blocked_create: the Add's operand %d is not quantized like the convolution's output", conv_operand);
+    s = CheckZeroPoint(add->dtype, add->a_zp, "tvx_conv2d_blocked_create", "Add operand");
+    if (s == TVX_OK) s = CheckZeroPoint(add->dtype, add->b_zp, "tvx_conv2d_blocked_create", "Add operand");
+    if (s == TVX_OK) s = CheckZeroPoint(add->dtype, add->out_zp, "tvx_conv2d_blocked_create", "Add output");
+  }
+  if (s != TVX_OK) return s;
+  if ((s = NoGpu()) != TVX_OK) return s;
+  tvx_op* op = new (std::nothrow) tvx_op();
+  if (!op) return SetError(TVX_E_NOMEM, "tvx_conv2d_blocked_create: host allocation failed");
+  op->kind = OP_CONV2D;
+  op->conv = *d;
+  if (add) {
+    op->elt = *add;
+    op->fused_add = conv_operand;
+  }
+  const tvx_conv2d_desc norm = op->conv;
+  op->conv.w_scales = nullptr;
+  op->quantized = true;
+  op->has_const_weights = true;
+  op->w_zp = d->w_scales ? 0 : d->w_zp;
+  s = BuildRequantTables(d->out_c, d->in_scale, d->w_scale, d->w_scales, d->out_scale, &op->h_mult, &op->h_shift);
+  ActRange(d->out_dtype, d->out_scale, d->out_zp, d->activation, &op->act_lo, &op->act_hi);
+  if (s == TVX_OK) {
+    s = BlockedPwSetup(op, &norm, weights_host, bias_host);
+    if (s == TVX_E_UNSUPPORTED && !add) s = BlockedDwSetup(op, &norm, weights_host, bias_host);
+  }
+  if (s != TVX_OK) {
+    delete op;
+    return s == TVX_E_UNSUPPORTED ? SetError(TVX_E_UNSUPPORTED, "tvx_conv2d_blocked_create: no kernel for this convolution on blocked tensors") : s;
+  }
+  *out = op;
+  return TVX_OK;
+}
+
+int tvx_pool2d_blocked_create(const tvx_pool2d_desc* d, tvx_op** out) {
+  if (!d || !out) return SetError(TVX_E_INVALID, "tvx_pool2d_blocked_create: null argument");
+  *out = nullptr;
+  if (!d->in_w || !d->in_h || !d->channels || !d->batch || !d->out_w || !d->out_h || !d->k_w || !d->k_h || !d->stride_w || !d->stride_h)
+    return SetError(TVX_E_INVALID, "tvx_pool2d_blocked_create: zero extent or stride");
+  if (!IsQuant(d->dtype) || !(d->in_scale > 0.f) || !(d->out_scale > 0.f))
+    return SetError(TVX_E_UNSUPPORTED, "tvx_pool2d_blocked_create: quantized tensors with positive scales only");
+  int s = CheckZeroPoint(d->dtype, d->in_zp, "tvx_pool2d_blocked_create", "input");
+  if (s == TVX_OK) s = CheckZeroPoint(d->dtype, d->out_zp, "tvx_pool2d_blocked_create", "output");
+  if (s == TVX_OK) s = NoGpu();
+  if (s != TVX_OK) return s;
+  tvx_op* op = new (std::nothrow) tvx_op();
+  if (!op) return SetError(TVX_E_NOMEM, "tvx_pool2d_blocked_create: host allocation failed");
+  op->kind = OP_POOL2D;
+  op->pool = *d;
+  op->quantized = true;
+  s = BlockedAvgSetup(op);
+  if (s != TVX_OK) {
+    delete op;
+    return s == TVX_E_UNSUPPORTED ? SetError(TVX_E_UNSUPPORTED, "tvx_pool2d_blocked_create: whole-plane average pooling only") : s;
+  }
+  *out = op;
+  return TVX_OK;
+}
+
+int tvx_layout_create(uint32_t w, uint32_t h, uint32_t c, uint32_t n, int to_blocked, tvx_op** out) {
+  if (!out) return SetError(TVX_E_INVALID, "tvx_layout_create: null argument");
+  *out = nullptr;
+  if (!w || !h || !c || !n) return SetError(TVX_E_INVALID, "tvx_layout_create: zero extent");
+  int s = NoGpu();
+  if (s != TVX_OK) return s;
+  tvx_op* op = new (std::nothrow) tvx_op();
+  if (!op) return SetError(TVX_E_NOMEM, "tvx_layout_create: host allocation failed");
+  op->kind = OP_TRANSPOSE;
+  s = LayoutSetup(op, w, h, c, n, to_blocked ? 1 : 0);
+  if (s != TVX_OK) {
+    delete op;
+    return s == TVX_E_UNSUPPORTED ? SetError(TVX_E_UNSUPPORTED, "tvx_layout_create: channels must be a multiple of 16") : s;
+  }
+  *out = op;
+  return TVX_OK;
+}
+
 int tvx_conv2d_dw_pw_create(const tvx_conv2d_desc* dw, const void* dw_w, const void* dw_b,
                             const tvx_conv2d_desc* pw, const void* pw_w, const void* pw_b,
                             const tvx_eltwise_desc* add, int conv_operand, tvx_op** out) {

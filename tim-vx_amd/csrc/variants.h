@@ -38,6 +38,12 @@ int PwConvSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 // depthwise 3x3 stencil (dwconv3x3_i8.hip)
 int DwConv3x3Setup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 
+// convolutions, whole-plane average pooling and the layout change on channel-blocked tensors (blocked_i8.hip)
+int BlockedPwSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
+int BlockedDwSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
+int BlockedAvgSetup(tvx_op*);
+int LayoutSetup(tvx_op*, uint32_t w, uint32_t h, uint32_t c, uint32_t n, int to_blocked);
+
 // depthwise, any kernel / width, planes staged through LDS (dwconv_planes_i8.hip)
 int DwPlanesSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 // shared by the two depthwise 3x3 stencils (defined in dwconv3x3_i8.hip)

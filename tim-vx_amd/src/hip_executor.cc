@@ -60,6 +60,10 @@ struct Step {
   TensorImpl* in1 = nullptr;  // run-time weights / second Add operand
   TensorImpl* in2 = nullptr;  // run-time bias
   TensorImpl* out = nullptr;
+  // a channel-blocked copy of a tensor that stays in WHCN order for its other readers stands in for in0 / in1 / out
+  void* blocked_in0 = nullptr;
+  void* blocked_in1 = nullptr;
+  void* blocked_out = nullptr;
   std::string name;
   uint64_t bytes = 0;  // tensor bytes the step has to move: its operands and its result
 };
@@ -70,6 +74,7 @@ class HipExecutor : public Executor {
     for (auto& s : steps_) tvx_op_destroy(s.op);
     for (void* e : events_) (void)tvx_event_destroy(e);
     for (auto& kv : owned_) tvx_free(kv.second);
+    for (auto& kv : blocked_copy_) tvx_free(kv.second);
     if (stream_) tvx_stream_destroy(stream_);
   }
 
@@ -106,7 +111,6 @@ class HipExecutor : public Executor {
     }
     // ---- residual fusion plan: a convolution whose TRANSIENT result only feeds a same-type Add, the
     // Add's other operand being there before the convolution runs, may become one operator
-    struct AddFusion { Operation* add; int conv_operand; };
     std::map<Operation*, AddFusion> fused_add;  // convolution -> the Add folded into it
     std::map<Tensor*, size_t> produced_at;  // position of the operator that writes a tensor
     for (size_t i = 0; i < graph->sorted_ops_.size(); ++i)
@@ -214,6 +218,29 @@ class HipExecutor : public Executor {
       // a pointwise convolution folded into the depthwise one in front of it is not there to take a pooling
       for (auto& kv : fused_dwpw) fused_pool.erase(kv.second);
     }
+    // ---- channel-blocked plan: runs of convolutions over small planes between TRANSIENT tensors kept 16 channels to
+    // a unit; the operators of the plan are no longer there for the other fusions
+    std::map<Operation*, BlockedOp> blocked;
+    {
+      const char* lever = std::getenv("TVX_BLOCKED_LAYOUT");  // tuning aid: 0 keeps every tensor in WHCN order
+      if (!lever || std::atoi(lever) != 0) PlanBlocked(graph, fused_act, fused_add, &blocked);
+      for (auto it = fused_block.begin(); it != fused_block.end();) {
+        Operation* dw = it->second;
+        auto pair = fused_dwpw.find(dw);
+        const bool hit = blocked.count(it->first) || blocked.count(dw) || (pair != fused_dwpw.end() && blocked.count(pair->second));
+        it = hit ? fused_block.erase(it) : std::next(it);
+      }
+      for (auto it = fused_dwpw.begin(); it != fused_dwpw.end();) {
+        if (blocked.count(it->first) || blocked.count(it->second)) {
+          for (auto fb = fused_block.begin(); fb != fused_block.end();) fb = fb->second == it->first ? fused_block.erase(fb) : std::next(fb);
+          it = fused_dwpw.erase(it);
+        } else {
+          ++it;
+        }
+      }
+      for (auto it = fused_pool.begin(); it != fused_pool.end();)
+        it = blocked.count(it->first) || blocked.count(it->second) ? fused_pool.erase(it) : std::next(it);
+    }
     // ---- device storage: one buffer per tensor, Reshape outputs alias their input --
     for (Operation* op : graph->sorted_ops_) {
       OpImpl* im = op->impl().get();
@@ -234,6 +261,12 @@ class HipExecutor : public Executor {
       if (im->attrs_.overflow != OverflowPolicy::SATURATE || im->attrs_.rounding != RoundingPolicy::RTNE) {
         VSILOGE("%s: only SATURATE + RTNE rounding policy is implemented", OpKindName(im->kind_));
         return false;
+      }
+      auto planned = blocked.find(op);
+      if (planned != blocked.end()) {
+        if (!AddBlocked(im, &planned->second)) return false;
+        if (planned->second.add) skipped[planned->second.add] = true;
+        continue;
       }
       int act = TVX_ACT_NONE;
       TensorImpl* out = static_cast<TensorImpl*>(im->outputs_tensor_[0].get());
@@ -386,8 +419,9 @@ class HipExecutor : public Executor {
     for (auto& s : steps_) {
       if (profile_ops_ && tvx_event_record(events_[step_index], stream_) != TVX_OK) return Fail("event");
       ++step_index;
-      const int st = tvx_op_run3(s.op, dev_[s.in0], s.in1 ? dev_[s.in1] : nullptr, s.in2 ? dev_[s.in2] : nullptr,
-                                 dev_[s.out], stream_);
+      const int st = tvx_op_run3(s.op, s.blocked_in0 ? s.blocked_in0 : dev_[s.in0],
+                                 s.blocked_in1 ? s.blocked_in1 : (s.in1 ? dev_[s.in1] : nullptr),
+                                 s.in2 ? dev_[s.in2] : nullptr, s.blocked_out ? s.blocked_out : dev_[s.out], stream_);
       if (st != TVX_OK) {
         VSILOGE("%s failed: %s", s.name.c_str(), tvx_last_error());
         return false;
@@ -419,6 +453,19 @@ class HipExecutor : public Executor {
   }
 
  private:
+  struct AddFusion { Operation* add; int conv_operand; };  // conv_operand: 1 or 2, which operand of the Add the convolution is
+
+  // An operator of the channel-blocked plan.
+  struct BlockedOp {
+    tvx_op* op = nullptr;       // created when the plan is made; owned by steps_ once placed
+    TensorImpl* in0 = nullptr;
+    TensorImpl* res = nullptr;  // the other operand of the Add folded into a convolution
+    std::shared_ptr<Tensor> out;  // what it writes: its own output, its activation's or its Add's
+    Operation* add = nullptr;
+    bool pool = false;
+    bool convert[2] = {false, false};  // in0 / res come in WHCN order and need a blocked copy
+  };
+
   bool Fail(const char* what) {
     VSILOGE("%s: %s", what, tvx_last_error());
     return false;
@@ -576,6 +623,150 @@ class HipExecutor : public Executor {
     } else {
       Push(op, dw_im, x, nullptr, pw_out);
     }
+    return true;
+  }
+
+  // Channel-blocked plan. Planes of a few pixels (7 x 7 at the end of a MobileNet) make WHCN rows no 16-byte load is
+  // aligned to; 1x1 and depthwise 3x3 convolutions over them are faster between tensors kept 16 channels to a unit
+  // (tvx_conv2d_blocked_create). A TRANSIENT tensor has no host image, so its order in memory is this runtime's
+  // choice. An operator joins the plan if a blocked kernel takes it and every reader of its result is in the plan too;
+  // a tensor that comes in from outside gets a blocked copy, made by a step of its own (tvx_layout_create), and the
+  // plan ends at an average pooling over whole planes, whose result is one pixel per plane in WHCN order. A plan of
+  // fewer than three convolutions does not pay for the copy and is dropped.
+  void PlanBlocked(GraphImpl* graph, const std::map<Operation*, Operation*>& fused_act,
+                   const std::map<Operation*, AddFusion>& fused_add, std::map<Operation*, BlockedOp>* plan) {
+    constexpr uint64_t kMaxPlane = 64;  // pixels; larger planes have rows long enough for the WHCN kernels
+    std::map<Operation*, Operation*> add_owner;  // Add -> the convolution it is folded into
+    for (auto& kv : fused_add) add_owner[kv.second.add] = kv.first;
+    auto constant = [](OpImpl* im, TensorImpl** w, TensorImpl** b) {
+      *w = static_cast<TensorImpl*>(im->inputs_tensor_[1].get());
+      *b = im->inputs_tensor_.size() > 2 && !im->inputs_tensor_[2]->IsPlaceHolder()
+               ? static_cast<TensorImpl*>(im->inputs_tensor_[2].get()) : nullptr;
+      return (*w)->IsConstTensor() && (*w)->HostData() && (!*b || ((*b)->IsConstTensor() && (*b)->HostData()));
+    };
+    for (Operation* op : graph->sorted_ops_) {
+      OpImpl* im = op->impl().get();
+      if (im->attrs_.overflow != OverflowPolicy::SATURATE || im->attrs_.rounding != RoundingPolicy::RTNE) continue;
+      TensorImpl* x = static_cast<TensorImpl*>(im->inputs_tensor_[0].get());
+      const ShapeType& xs = x->spec_.shape_;
+      if (xs.size() != 4 || static_cast<uint64_t>(xs[0]) * xs[1] > kMaxPlane || !IsQuantSpec(x->spec_)) continue;
+      BlockedOp b;
+      b.in0 = x;
+      if (im->kind_ == OpKind::CONV2D && !im->attrs_.conv_1d) {
+        TensorImpl *w, *bias;
+        if (!constant(im, &w, &bias)) continue;
+        int act = TVX_ACT_NONE;
+        b.out = im->outputs_tensor_[0];
+        tvx_conv2d_desc d = ConvDesc(im, static_cast<TensorImpl*>(b.out.get()), act, false);
+        tvx_eltwise_desc e{};
+        int conv_operand = 0;
+        auto fa = fused_act.find(op);
+        auto fd = fused_add.find(op);
+        if (fa != fused_act.end()) {
+          OpImpl* a = fa->second->impl().get();
+          act = a->kind_ == OpKind::RELU ? TVX_ACT_RELU : TVX_ACT_RELU6;
+          b.out = a->outputs_tensor_[0];
+          d = ConvDesc(im, static_cast<TensorImpl*>(b.out.get()), act, false);
+        } else if (fd != fused_add.end()) {
+          OpImpl* a = fd->second.add->impl().get();
+          if (!AddDesc(a, &e)) continue;
+          conv_operand = fd->second.conv_operand;
+          b.add = fd->second.add;
+          b.res = static_cast<TensorImpl*>(a->inputs_tensor_[conv_operand == 1 ? 1 : 0].get());
+          b.out = a->outputs_tensor_[0];
+        }
+        if (!(b.out->GetSpec().attr_ & TensorAttribute::TRANSIENT)) continue;
+        if (tvx_conv2d_blocked_create(&d, b.add ? &e : nullptr, conv_operand, w->HostData(), bias ? bias->HostData() : nullptr,
+                                      &b.op) != TVX_OK)
+          continue;
+      } else if (im->kind_ == OpKind::POOL && !im->attrs_.pool_1d) {
+        b.pool = true;
+        b.out = im->outputs_tensor_[0];
+        const tvx_pool2d_desc d = PoolDesc(im, x, static_cast<TensorImpl*>(b.out.get()));
+        if (tvx_pool2d_blocked_create(&d, &b.op) != TVX_OK) continue;
+      } else {
+        continue;
+      }
+      (*plan)[op] = b;
+    }
+    // closure: what a convolution of the plan writes is blocked, so every reader has to be in the plan, as its input
+    // or as the residual operand of its Add; a pooling of the plan reads what a convolution of the plan wrote
+    for (bool changed = true; changed;) {
+      changed = false;
+      std::map<Tensor*, Operation*> written;  // blocked tensor -> the convolution of the plan that writes it
+      for (auto& kv : *plan)
+        if (!kv.second.pool) written[kv.second.out.get()] = kv.first;
+      for (auto it = plan->begin(); it != plan->end();) {
+        BlockedOp& b = it->second;
+        bool keep = true;
+        if (b.pool) {
+          keep = written.count(b.in0) != 0;
+        } else {
+          for (auto& reader : graph->GetConsumersOp(b.out)) {
+            auto r = plan->find(reader.get());
+            if (r != plan->end() && r->second.in0 == b.out.get()) continue;
+            auto owner = add_owner.find(reader.get());
+            if (owner != add_owner.end()) {
+              auto o = plan->find(owner->second);
+              if (o != plan->end() && o->second.add == reader.get() && o->second.res == b.out.get()) continue;
+            }
+            keep = false;
+            break;
+          }
+        }
+        if (keep) {
+          ++it;
+        } else {
+          tvx_op_destroy(b.op);
+          it = plan->erase(it);
+          changed = true;
+        }
+      }
+    }
+    size_t convolutions = 0;
+    std::map<Tensor*, Operation*> written;
+    for (auto& kv : *plan)
+      if (!kv.second.pool) {
+        written[kv.second.out.get()] = kv.first;
+        ++convolutions;
+      }
+    if (convolutions < 3) {
+      for (auto& kv : *plan) tvx_op_destroy(kv.second.op);
+      plan->clear();
+      return;
+    }
+    for (auto& kv : *plan) {
+      kv.second.convert[0] = !written.count(kv.second.in0);
+      kv.second.convert[1] = kv.second.res && !written.count(kv.second.res);
+    }
+  }
+
+  // Places an operator of the channel-blocked plan, behind the steps that make the blocked copies it reads.
+  bool AddBlocked(OpImpl* im, BlockedOp* b) {
+    void* copy[2] = {nullptr, nullptr};
+    TensorImpl* ins[2] = {b->in0, b->res};
+    for (int i = 0; i < 2; ++i) {
+      if (!ins[i] || !b->convert[i]) continue;
+      auto it = blocked_copy_.find(ins[i]);
+      if (it == blocked_copy_.end()) {
+        const ShapeType& s = ins[i]->spec_.shape_;
+        tvx_op* to_blocked = nullptr;
+        if (s.size() != 4 || tvx_layout_create(s[0], s[1], s[2], s[3], 1, &to_blocked) != TVX_OK) return Fail("tvx_layout_create");
+        void* p = nullptr;
+        if (tvx_malloc(&p, ins[i]->HostBytes()) != TVX_OK) {
+          tvx_op_destroy(to_blocked);
+          return Fail("device allocation");
+        }
+        it = blocked_copy_.emplace(ins[i], p).first;
+        Push(to_blocked, im, ins[i], nullptr, ins[i]);
+        steps_.back().blocked_out = p;
+      }
+      copy[i] = it->second;
+    }
+    Push(b->op, im, b->in0, b->res, static_cast<TensorImpl*>(b->out.get()));
+    steps_.back().blocked_in0 = copy[0];
+    steps_.back().blocked_in1 = copy[1];
+    b->op = nullptr;
     return true;
   }
 
@@ -837,6 +1028,7 @@ class HipExecutor : public Executor {
   std::vector<Step> steps_;
   std::map<TensorImpl*, void*> dev_;    // tensor -> device pointer (possibly an alias)
   std::map<TensorImpl*, void*> owned_;  // tensors that own their buffer
+  std::map<TensorImpl*, void*> blocked_copy_;  // WHCN tensor -> its channel-blocked copy, written by a step of the plan
 };
 
 }  // namespace
