@@ -70,12 +70,16 @@ PW_SHAPES = [
 ]
 
 
-@pytest.mark.parametrize("form", [None, (0, 1), (0, 2), (0, 4), (1, 1)], ids=str)
+@pytest.mark.parametrize("form", [None, (0, 1), (0, 2), (0, 4), (1, 1), "records"], ids=str)
 @pytest.mark.parametrize("mode", ["u8", "i8pc", "u8pc"])
 @pytest.mark.parametrize("shape", PW_SHAPES, ids=lambda s: "x".join(map(str, s)))
 def test_pointwise_conv_blocked(oracle, shape, mode, form, monkeypatch):
     n, c, side, oc = shape
-    if form is not None:   # (form, channel tiles per wavefront): every kernel shape on every problem
+    if form == "records":  # per-tensor quantization without the one-record-for-all-channels epilogue
+        if mode != "u8":
+            pytest.skip("per-channel scales never share a record")
+        monkeypatch.setenv("TVX_BLOCKED_UNIFORM_RQ", "0")
+    elif form is not None:   # (form, channel tiles per wavefront): every kernel shape on every problem
         monkeypatch.setenv("TVX_BLOCKED_PW_FORM", str(form[0]))
         monkeypatch.setenv("TVX_BLOCKED_PW_TILES", str(form[1]))
     rng = np.random.default_rng(c + oc + side)

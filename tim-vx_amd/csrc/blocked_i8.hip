@@ -25,6 +25,7 @@
 // Zero points and requantization are those of the WHCN kernels (pwconv_i8.hip, dwconv3x3_i8.hip, kernels_generic.hip).
 #include <algorithm>
 #include <cstdlib>
+#include <cstring>
 
 #include "variants.h"
 
@@ -78,6 +79,8 @@ struct BpArgs {
   int xor_mask;          // 0x80808080 for uint8 activations
   int neg_zws4;          // -(weight zero point, int8 domain) in all four bytes
   int out_zp, lo, hi;
+  int uni;               // one requantization record for every channel (per-tensor quantization): `u`, no record loads
+  tvx_v4i u;
   // the fused Add, as in pwconv_i8.hip (add_mode 0 = off, 1: a = convolution, b = residual, 2: the other way round)
   int add_mode, add_signed, add_za, add_zb, add_zo, add_lo, add_hi;
   double add_ra, add_rb;
@@ -157,10 +160,15 @@ __global__ void __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2
     for (int g = 0; g < 4; ++g) {
       const int oc = tile * 32 + 8 * g + 4 * h;
       const v4i b4 = *reinterpret_cast<const v4i*>(a.biasf + oc);
-      int r4[4];
+      if (a.uni) {  // (uniform)
+        const int v4[4] = {acc[j][4 * g] + b4[0], acc[j][4 * g + 1] + b4[1], acc[j][4 * g + 2] + b4[2], acc[j][4 * g + 3] + b4[3]};
+        quad[g] = RequantPack4<RQ>(v4, a.u, a.out_zp, a.lo, a.hi);
+      } else {
+        int r4[4];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) r4[e] = Requant8<RQ>(acc[j][4 * g + e] + b4[e], a.rq[oc + e], a.out_zp, a.lo, a.hi);
-      quad[g] = PackBytes(r4[0], r4[1], r4[2], r4[3]);
+        for (int e = 0; e < 4; ++e) r4[e] = Requant8<RQ>(acc[j][4 * g + e] + b4[e], a.rq[oc + e], a.out_zp, a.lo, a.hi);
+        quad[g] = PackBytes(r4[0], r4[1], r4[2], r4[3]);
+      }
     }
     // quad g of the lower half: channels 8 g .. 8 g + 3, of the upper half: 8 g + 4 .. 8 g + 7. Behind the swaps a lower
     // lane holds channels 0 .. 15 of the tile, its partner in the upper half channels 16 .. 31: one blocked unit each.
@@ -454,6 +462,11 @@ int BlockedPwSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, con
   a.wpk = op->packed.as<v4i>();
   a.biasf = op->aux.as<int32_t>();
   a.rq = op->aux2.as<tvx_v4i>();
+  a.uni = 1;
+  for (int oc = 1; oc < a.OC; ++oc)
+    if (std::memcmp(&rqt[4 * oc], &rqt[0], 16) != 0) a.uni = 0;
+  a.u = tvx_v4i{rqt[0], rqt[1], rqt[2], rqt[3]};
+  if (const char* f = getenv("TVX_BLOCKED_UNIFORM_RQ")) if (!atoi(f)) a.uni = 0;  // test lever: keeps the per-channel record loads
   plan.zp = zws != 0;
   // few output channels behind a long reduction: split the reduction over the workgroup; else four pixel tiles a workgroup
   const int pix_tiles = (a.P + 31) / 32;
