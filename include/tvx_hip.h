@@ -326,10 +326,14 @@ int tvx_transpose_create(const tvx_transpose_desc* desc, tvx_op** op);
  *    no Add), or for a depthwise 3x3 / stride-1 convolution (multiplier 1, `add` NULL); constant weights;
  *  - tvx_pool2d_blocked_create: vxPoolingLayer2 (ops/vsi_nn_op_pool.c:144-150) averaging whole unpadded planes of
  *    at most 256 pixels: blocked in, {1, 1, C, N} out in WHCN order (byte n * C + c);
+ *  - tvx_conv2d_to_blocked_create: the same vxConvolutionLayer for a depthwise 3x3 convolution (multiplier 1, stride 1
+ *    or 2, constant weights, channels a multiple of 16, planes that fit the LDS-staged kernel) that reads a WHCN tensor
+ *    and writes its result blocked: the way into a run of blocked operators without a copy;
  *  - tvx_layout_create: WHCN -> blocked (to_blocked != 0) or back; no counterpart in the reference's API.
  * TVX_E_UNSUPPORTED: no blocked kernel for this operator (the caller keeps the tensor in WHCN). */
 int tvx_conv2d_blocked_create(const tvx_conv2d_desc* conv, const tvx_eltwise_desc* add, int conv_operand,
                               const void* weights_host, const void* bias_host, tvx_op** op);
+int tvx_conv2d_to_blocked_create(const tvx_conv2d_desc* conv, const void* weights_host, const void* bias_host, tvx_op** op);
 int tvx_pool2d_blocked_create(const tvx_pool2d_desc* desc, tvx_op** op);
 int tvx_layout_create(uint32_t w, uint32_t h, uint32_t c, uint32_t n, int to_blocked, tvx_op** op);
 

@@ -191,3 +191,38 @@ def test_blocked_operators_decline_what_they_do_not_cover():
     with pytest.raises(T.TvxError) as err:   # 24 channels
         T.layout_create(7, 7, 24, 1, True)
     assert err.value.status == T.E_UNSUPPORTED
+
+
+@pytest.mark.parametrize("mode", ["u8", "i8pc", "u8pc"])
+@pytest.mark.parametrize("shape", [(3, 576, 14, 14, 2, [0, 1, 0, 1]), (2, 32, 7, 7, 1, [1, 1, 1, 1]), (1, 48, 9, 6, 2, [1, 1, 1, 1]),
+                                   (2, 16, 5, 13, 1, [1, 1, 1, 1]), (1, 64, 28, 28, 2, [0, 1, 0, 1])],
+                         ids=lambda s: "x".join(map(str, s[:5])))
+def test_depthwise_conv_writing_blocked(oracle, shape, mode):
+    """tvx_conv2d_to_blocked_create: WHCN in, blocked out - the way into a run of blocked operators."""
+    n, c, h, w, stride, pad = shape
+    rng = np.random.default_rng(c * 3 + h + stride)
+    x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=0, kh=3, kw=3, stride=[stride, stride], dil=[1, 1], pad=pad,
+                              mult=1, mode=mode)
+    T = TC.tvx()
+    ohw = kws["out_shape"][0] * kws["out_shape"][1]
+    for act in (0, 2):
+        want = oracle.conv2d(x, wt, b, act=act, **kws)
+        keep = []
+        op = T.conv2d_to_blocked_create(_conv_desc(T, kws, act, keep), wt, b)
+        assert op.kernel_name == "dwconv_planes_to_blocked_i8"
+        got = from_blocked(_run(op, x, want.size, kws["out_dtype"]), n, c, ohw)
+        assert np.array_equal(got, want), (shape, mode, act, np.flatnonzero(got != want)[:8])
+    assert len(np.unique(want)) > 4
+
+
+def test_conv2d_to_blocked_create_declines_other_convolutions():
+    T = TC.tvx()
+    rng = np.random.default_rng(6)
+    for kw in (dict(c=24, oc=0, kh=3, kw=3, mult=1, pad=[1, 1, 1, 1]),     # channels that do not fill 16-channel blocks
+               dict(c=32, oc=0, kh=5, kw=5, mult=1, pad=[2, 2, 2, 2]),     # another window
+               dict(c=32, oc=32, kh=1, kw=1, mult=0, pad=[0, 0, 0, 0])):  # not depthwise
+        x, wt, b, kws = conv_case(rng, n=1, h=7, w=7, stride=[1, 1], dil=[1, 1], mode="u8", **kw)
+        keep = []
+        with pytest.raises(T.TvxError) as err:
+            T.conv2d_to_blocked_create(_conv_desc(T, kws, 0, keep), wt, b)
+        assert err.value.status == T.E_UNSUPPORTED

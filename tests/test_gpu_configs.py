@@ -30,8 +30,10 @@ def test_mobilenet_v2_batch64_224_bit_exact(tmp_path, oracle):
     log = _check([g], tmp_path / "full", values, env={"VSI_NN_LOG_LEVEL": "3"})
     plan = [l for l in log.splitlines() if "uid" in l and "->" in l]
     assert sum("pwconv_add_i8" in l or "pwconv_add_blocked_i8" in l for l in plan) == 10, plan
-    # the 7 x 7 stage runs between channel-blocked tensors: one copy in, the whole-plane average out
-    assert sum("layout_to_blocked" in l for l in plan) == 1 and sum("_blocked_i8" in l for l in plan) == 12, plan
+    # the 7 x 7 stage runs between channel-blocked tensors: the stride-2 depthwise convolution in front writes the
+    # first of them (no copy), the whole-plane average leaves the stage
+    assert not any("layout_to_blocked" in l for l in plan) and sum("dwconv_planes_to_blocked_i8" in l for l in plan) == 1, plan
+    assert sum("_blocked_i8" in l for l in plan) == 13, plan
     # the network cut behind single operators: first convolution, expansions / depthwise / projections of every
     # resolution (112, 56, 28, 14, 7), residual Adds, the last 1x1 convolution
     cuts = []

@@ -120,6 +120,7 @@ def lib():
                                         C.POINTER(EltwiseDesc), C.c_int, C.POINTER(vp)]
         L.tvx_conv2d_pool_create.argtypes = [C.POINTER(Conv2dDesc), C.POINTER(Pool2dDesc), vp, vp, C.POINTER(vp)]
         L.tvx_conv2d_blocked_create.argtypes = [C.POINTER(Conv2dDesc), C.POINTER(EltwiseDesc), C.c_int, vp, vp, C.POINTER(vp)]
+        L.tvx_conv2d_to_blocked_create.argtypes = [C.POINTER(Conv2dDesc), vp, vp, C.POINTER(vp)]
         L.tvx_pool2d_blocked_create.argtypes = [C.POINTER(Pool2dDesc), C.POINTER(vp)]
         L.tvx_layout_create.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_int, C.POINTER(vp)]
         L.tvx_fully_connected_softmax_create.argtypes = [C.POINTER(FcDesc), C.POINTER(SoftmaxDesc), vp, vp, C.POINTER(vp)]
@@ -206,6 +207,13 @@ def mbconv_create(expand, expand_w, expand_b, dw, dw_w, dw_b, project, project_w
                                   C.byref(dw), _host_ptr(dw_w), _host_ptr(dw_b),
                                   C.byref(project), _host_ptr(project_w), _host_ptr(project_b),
                                   C.byref(add_desc) if add_desc is not None else None, conv_operand, C.byref(h)))
+    return Op(h)
+
+
+def conv2d_to_blocked_create(desc, weights, bias=None):
+    """A depthwise 3x3 convolution that reads a WHCN tensor and writes its result channel-blocked."""
+    h = C.c_void_p()
+    check(lib().tvx_conv2d_to_blocked_create(C.byref(desc), _host_ptr(weights), _host_ptr(bias), C.byref(h)))
     return Op(h)
 
 

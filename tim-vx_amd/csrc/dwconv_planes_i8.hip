@@ -232,6 +232,7 @@ struct DwrArgs {
   uint32_t m_c, m_plane4, m_pw4, m_ipp, m_ow4;  // reciprocals of C, ph*pw4, pw4, oh2*ow4, ow4
   int xor_mask, pad_fill, zws, out_zp, lo, hi;
   int off_tab;           // dword offset of the per-plane tables in LDS
+  int out_blocked, PO;   // the result goes out channel-blocked (byte ((c / 16) * PO + p) * 16 + c % 16, PO pixels in the batch)
 };
 
 constexpr int kCopyBatch = 8;  // input dwords a thread has in flight
@@ -357,7 +358,17 @@ __global__ void __launch_bounds__(kThreads) DwRowsKernel(DwrArgs a) {
         r4[j] = Requant8<RQ>(acc, rq, a.out_zp, lo, hi);
       }
       const uint32_t packed = PackBytes(r4[0], r4[1], r4[2], r4[3]);
-      if (oy + orow < a.OH) {
+      if (a.out_blocked) {  // (uniform) four pixels of one channel: four bytes sixteen apart
+        if (oy + orow < a.OH) {
+          const int pl = p0 + g;
+          const int img = DivMagic(pl, a.m_c), c = pl - __mul24(img, a.C);
+          const int pix = __mul24(img, hwo) + __mul24(oy + orow, a.OW) + 4 * q;
+          uint8_t* ob = a.y + (static_cast<size_t>(c >> 4) * a.PO + pix) * 16 + (c & 15);
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            if (j < n) ob[j * 16] = static_cast<uint8_t>(packed >> (8 * j));
+        }
+      } else if (oy + orow < a.OH) {
         uint8_t* orw = o + orow * a.OW;
         if (n == 4) {
           __builtin_memcpy(orw, &packed, 4);
@@ -470,11 +481,16 @@ int DwRowsSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, const 
   a.xor_mask = x_u8 ? static_cast<int>(0x80808080u) : 0;
   a.pad_fill = static_cast<int>(static_cast<uint32_t>(zxs & 0xff) * 0x01010101u);
   a.out_zp = d->out_zp; a.lo = op->act_lo; a.hi = op->act_hi;
+  if (op->out_blocked) {
+    if (C % 16 || d->batch * hwo * C >= (1ll << 31) || d->batch * hwo >= (1ll << 23)) return TVX_E_UNSUPPORTED;
+    a.out_blocked = 1;
+    a.PO = static_cast<int>(d->batch * hwo);
+  }
   p.stride = S;
   p.grid = static_cast<unsigned>(grid);
   op->host_blob.assign(reinterpret_cast<const uint8_t*>(&p), reinterpret_cast<const uint8_t*>(&p) + sizeof(p));
   op->run = DwRowsRun;
-  op->kernel_name = "dwconv_planes_i8";
+  op->kernel_name = op->out_blocked ? "dwconv_planes_to_blocked_i8" : "dwconv_planes_i8";
   return TVX_OK;
 }
 
@@ -486,7 +502,7 @@ int DwPlanesSetup(tvx_op* op, const tvx_conv2d_desc* d, const void* w_host, cons
   if (!op->quantized || !w_host || d->multiplier != 1) return TVX_E_UNSUPPORTED;
   {
     const int s = DwRowsSetup(op, d, w_host, bias_host);
-    if (s != TVX_E_UNSUPPORTED) return s;
+    if (s != TVX_E_UNSUPPORTED || op->out_blocked) return s;  // (only the dword form writes blocked results)
   }
   const uint64_t hwi = static_cast<uint64_t>(d->in_w) * d->in_h, hwo = static_cast<uint64_t>(d->out_w) * d->out_h;
   if (hwi == 0 || hwo == 0) return TVX_E_UNSUPPORTED;

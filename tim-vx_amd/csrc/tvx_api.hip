@@ -519,6 +519,43 @@ int tvx_conv2d_blocked_create(const tvx_conv2d_desc* d, const tvx_eltwise_desc* 
   return TVX_OK;
 }
 
+int tvx_conv2d_to_blocked_create(const tvx_conv2d_desc* d, const void* weights_host, const void* bias_host, tvx_op** out) {
+  static const char* const fn = "tvx_conv2d_to_blocked_create";
+  if (!d || !out) return SetError(TVX_E_INVALID, "%s: null argument", fn);
+  *out = nullptr;
+  if (!d->in_w || !d->in_h || !d->in_c || !d->batch || !d->k_w || !d->k_h || !d->out_w || !d->out_h || !d->out_c ||
+      !d->stride_w || !d->stride_h || !d->dilation_w || !d->dilation_h)
+    return SetError(TVX_E_INVALID, "%s: zero extent, stride or dilation", fn);
+  if (static_cast<uint64_t>(d->out_w - 1) * d->stride_w >= static_cast<uint64_t>(d->in_w) + d->pad_left ||
+      static_cast<uint64_t>(d->out_h - 1) * d->stride_h >= static_cast<uint64_t>(d->in_h) + d->pad_top)
+    return SetError(TVX_E_INVALID, "%s: output extent reaches past the input", fn);
+  if (!IsQuant(d->in_dtype) || !weights_host) return SetError(TVX_E_UNSUPPORTED, "%s: quantized tensors and constant weights only", fn);
+  if (d->multiplier != 1 || d->out_c != d->in_c) return SetError(TVX_E_UNSUPPORTED, "%s: depthwise convolutions with multiplier 1 only", fn);
+  int s = CheckOperandTypes(d->in_dtype, d->w_dtype, d->out_dtype, fn);
+  if (s == TVX_OK) s = CheckConvZeroPoints(d->in_dtype, d->in_zp, d->w_dtype, d->w_zp, d->w_scales != nullptr, d->out_dtype, d->out_zp, fn);
+  if (s != TVX_OK) return s;
+  if ((s = NoGpu()) != TVX_OK) return s;
+  tvx_op* op = new (std::nothrow) tvx_op();
+  if (!op) return SetError(TVX_E_NOMEM, "%s: host allocation failed", fn);
+  op->kind = OP_CONV2D;
+  op->conv = *d;
+  const tvx_conv2d_desc norm = op->conv;
+  op->conv.w_scales = nullptr;
+  op->quantized = true;
+  op->has_const_weights = true;
+  op->out_blocked = 1;
+  op->w_zp = d->w_scales ? 0 : d->w_zp;
+  s = BuildRequantTables(d->out_c, d->in_scale, d->w_scale, d->w_scales, d->out_scale, &op->h_mult, &op->h_shift);
+  ActRange(d->out_dtype, d->out_scale, d->out_zp, d->activation, &op->act_lo, &op->act_hi);
+  if (s == TVX_OK) s = DwPlanesSetup(op, &norm, weights_host, bias_host);
+  if (s != TVX_OK) {
+    delete op;
+    return s == TVX_E_UNSUPPORTED ? SetError(TVX_E_UNSUPPORTED, "%s: no kernel writes this convolution's result blocked", fn) : s;
+  }
+  *out = op;
+  return TVX_OK;
+}
+
 int tvx_pool2d_blocked_create(const tvx_pool2d_desc* d, tvx_op** out) {
   if (!d || !out) return SetError(TVX_E_INVALID, "tvx_pool2d_blocked_create: null argument");
   *out = nullptr;

@@ -50,6 +50,7 @@ struct tvx_op {
   int fused_add = 0;  // Conv2d + Add in one kernel: 1 = the convolution is the Add's first operand, 2 = its second (elt holds the Add)
   int fused_pool = 0;  // Conv2d + 2x2 / stride-2 max pooling in one kernel: the result has a quarter of conv's output pixels
   int fused_softmax = 0;  // FullyConnected + Softmax over its outputs in one kernel (sm holds the Softmax): fp32 result
+  int out_blocked = 0;  // the result is written channel-blocked (the input is WHCN): set before a variant is asked
 
   tvx_conv2d_desc conv{};
   tvx_fc_desc fc{};

@@ -220,18 +220,19 @@ class HipExecutor : public Executor {
     }
     // ---- channel-blocked plan: runs of convolutions over small planes between TRANSIENT tensors kept 16 channels to
     // a unit; the operators of the plan are no longer there for the other fusions
-    std::map<Operation*, BlockedOp> blocked;
+    std::map<Operation*, BlockedOp> blocked, blocked_writers;  // (writers: WHCN in, blocked out, in front of the plan)
     {
       const char* lever = std::getenv("TVX_BLOCKED_LAYOUT");  // tuning aid: 0 keeps every tensor in WHCN order
-      if (!lever || std::atoi(lever) != 0) PlanBlocked(graph, fused_act, fused_add, &blocked);
+      if (!lever || std::atoi(lever) != 0) PlanBlocked(graph, fused_act, fused_add, &blocked, &blocked_writers);
       for (auto it = fused_block.begin(); it != fused_block.end();) {
         Operation* dw = it->second;
         auto pair = fused_dwpw.find(dw);
-        const bool hit = blocked.count(it->first) || blocked.count(dw) || (pair != fused_dwpw.end() && blocked.count(pair->second));
+        const bool hit = blocked.count(it->first) || blocked.count(dw) || blocked_writers.count(dw) ||
+                         (pair != fused_dwpw.end() && blocked.count(pair->second));
         it = hit ? fused_block.erase(it) : std::next(it);
       }
       for (auto it = fused_dwpw.begin(); it != fused_dwpw.end();) {
-        if (blocked.count(it->first) || blocked.count(it->second)) {
+        if (blocked.count(it->first) || blocked.count(it->second) || blocked_writers.count(it->first)) {
           for (auto fb = fused_block.begin(); fb != fused_block.end();) fb = fb->second == it->first ? fused_block.erase(fb) : std::next(fb);
           it = fused_dwpw.erase(it);
         } else {
@@ -261,6 +262,11 @@ class HipExecutor : public Executor {
       if (im->attrs_.overflow != OverflowPolicy::SATURATE || im->attrs_.rounding != RoundingPolicy::RTNE) {
         VSILOGE("%s: only SATURATE + RTNE rounding policy is implemented", OpKindName(im->kind_));
         return false;
+      }
+      auto writer = blocked_writers.find(op);
+      if (writer != blocked_writers.end()) {
+        Push(writer->second.op, im, writer->second.in0, nullptr, static_cast<TensorImpl*>(writer->second.out.get()));
+        continue;
       }
       auto planned = blocked.find(op);
       if (planned != blocked.end()) {
@@ -634,7 +640,8 @@ class HipExecutor : public Executor {
   // plan ends at an average pooling over whole planes, whose result is one pixel per plane in WHCN order. A plan of
   // fewer than three convolutions does not pay for the copy and is dropped.
   void PlanBlocked(GraphImpl* graph, const std::map<Operation*, Operation*>& fused_act,
-                   const std::map<Operation*, AddFusion>& fused_add, std::map<Operation*, BlockedOp>* plan) {
+                   const std::map<Operation*, AddFusion>& fused_add, std::map<Operation*, BlockedOp>* plan,
+                   std::map<Operation*, BlockedOp>* writers) {
     // pixels of a plane; from 14 x 14 up the WHCN kernels and the block kernel are as fast or faster (MobileNetV2 at
     // batch 64: 19.5 us for the three blocked operators of a 64 -> 384 -> 64 block against 15.7 us)
     uint64_t kMaxPlane = 64;
@@ -741,6 +748,38 @@ class HipExecutor : public Executor {
     for (auto& kv : *plan) {
       kv.second.convert[0] = !written.count(kv.second.in0);
       kv.second.convert[1] = kv.second.res && !written.count(kv.second.res);
+    }
+    // a TRANSIENT tensor that enters the plan from a depthwise convolution and is read by nothing else: where a kernel
+    // can, that convolution writes it blocked itself (tvx_conv2d_to_blocked_create) and the copy falls away
+    if (std::getenv("TVX_NO_BLOCKED_WRITERS")) return;  // tuning aid
+    for (Operation* prod : graph->sorted_ops_) {
+      OpImpl* pim = prod->impl().get();
+      if (pim->kind_ != OpKind::CONV2D || pim->attrs_.conv_1d || pim->attrs_.multiplier != 1 || plan->count(prod) || fused_add.count(prod)) continue;
+      if (pim->attrs_.overflow != OverflowPolicy::SATURATE || pim->attrs_.rounding != RoundingPolicy::RTNE) continue;
+      int act = TVX_ACT_NONE;
+      std::shared_ptr<Tensor> out = pim->outputs_tensor_[0];
+      auto fa = fused_act.find(prod);
+      if (fa != fused_act.end()) {
+        OpImpl* a = fa->second->impl().get();
+        act = a->kind_ == OpKind::RELU ? TVX_ACT_RELU : TVX_ACT_RELU6;
+        out = a->outputs_tensor_[0];
+      }
+      if (!(out->GetSpec().attr_ & TensorAttribute::TRANSIENT)) continue;
+      auto readers = graph->GetConsumersOp(out);
+      bool all_in_plan = !readers.empty();
+      for (auto& r : readers) {
+        auto pr = plan->find(r.get());
+        all_in_plan = all_in_plan && pr != plan->end() && pr->second.in0 == out.get() && pr->second.convert[0] && pr->second.res != out.get();
+      }
+      TensorImpl *w, *bias;
+      if (!all_in_plan || !constant(pim, &w, &bias)) continue;
+      BlockedOp b;
+      b.in0 = static_cast<TensorImpl*>(pim->inputs_tensor_[0].get());
+      b.out = out;
+      const tvx_conv2d_desc d = ConvDesc(pim, static_cast<TensorImpl*>(out.get()), act, false);
+      if (tvx_conv2d_to_blocked_create(&d, w->HostData(), bias ? bias->HostData() : nullptr, &b.op) != TVX_OK) continue;
+      (*writers)[prod] = b;
+      for (auto& r : readers) (*plan)[r.get()].convert[0] = false;
     }
   }
 
