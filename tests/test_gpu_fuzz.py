@@ -359,3 +359,83 @@ def test_max_pool_register_stencil_sweep(oracle):
         want = oracle.pool2d(x, in_q=in_q, out_q=out_q, **kws)
         got = TC.gpu_pool2d(x, in_q=in_q, out_q=out_q, want_kernel="pool2d_stencil_i8", **kws)
         assert np.array_equal(got, want), (i, kws, out_q, int((got != want).sum()))
+
+
+def test_channel_blocked_operators_sweep(oracle):
+    """The operators between channel-blocked tensors on random shapes: pointwise convolutions (with and without the Add,
+    every kernel shape reached through the reduction length and the channel-tile count), depthwise 3x3 at stride 1 with
+    random pads, the depthwise kernel that reads WHCN and writes blocked (strides 1 and 2), the whole-plane average."""
+    from test_gpu_blocked import _conv_desc, _run, from_blocked, to_blocked
+    T = TC.tvx()
+    rng = np.random.default_rng(0xB10C)
+    seen = collections.Counter()
+    for i in range(90):
+        kind = ["pw", "pw_add", "dw", "dw_writer", "avg"][i % 5]
+        mode = str(rng.choice(["u8", "i8pc", "u8pc"]))
+        n = int(rng.integers(1, 5))
+        h, w = int(rng.integers(1, 12)), int(rng.integers(1, 12))
+        hw = h * w
+        act = int(rng.choice([0, 1, 2]))
+        keep = []
+        if kind in ("pw", "pw_add"):
+            c, oc = 32 * int(rng.integers(1, 18)), 32 * int(rng.integers(1, 14))
+            x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=oc, kh=1, kw=1, stride=[1, 1], dil=[1, 1], pad=[0, 0, 0, 0],
+                                      mult=0, mode=mode)
+            dt = kws["out_dtype"]
+            if kind == "pw":
+                want = oracle.conv2d(x, wt, b, act=act, **kws)
+                op = T.conv2d_blocked_create(_conv_desc(T, kws, act, keep), wt, b)
+                got = _run(op, to_blocked(x, n, c, hw), want.size, dt)
+            else:
+                operand = int(rng.integers(1, 3))
+                other = rand_q(rng, n * oc * hw, dt)
+                other_q, sum_q = (0.037, 121 if dt == 0 else -7), (float(np.float32(kws["out_q"][0] * 1.3)), 119 if dt == 0 else 5)
+                t = oracle.conv2d(x, wt, b, **kws)
+                a, aq, bb, bq = (t, kws["out_q"], other, other_q) if operand == 1 else (other, other_q, t, kws["out_q"])
+                want = oracle.add(dt, a, aq, bb, bq, sum_q)
+                e = T.EltwiseDesc()
+                e.count, e.dtype = want.size, dt
+                e.a_scale, e.a_zp = aq
+                e.b_scale, e.b_zp = bq
+                e.out_scale, e.out_zp = sum_q
+                op = T.conv2d_blocked_create(_conv_desc(T, kws, 0, keep), wt, b, add_desc=e, conv_operand=operand)
+                got = _run(op, to_blocked(x, n, c, hw), want.size, dt, other=to_blocked(other, n, oc, hw))
+            got = from_blocked(got, n, oc, hw)
+        elif kind == "dw":
+            c = 16 * int(rng.integers(1, 12))
+            pad = [int(rng.integers(0, 2)) for _ in range(4)]
+            if h + pad[2] + pad[3] < 3 or w + pad[0] + pad[1] < 3:
+                pad = [1, 1, 1, 1]
+            x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=0, kh=3, kw=3, stride=[1, 1], dil=[1, 1], pad=pad, mult=1, mode=mode)
+            want = oracle.conv2d(x, wt, b, act=act, **kws)
+            op = T.conv2d_blocked_create(_conv_desc(T, kws, act, keep), wt, b)
+            got = from_blocked(_run(op, to_blocked(x, n, c, hw), want.size, kws["out_dtype"]), n, c,
+                               kws["out_shape"][0] * kws["out_shape"][1])
+        elif kind == "dw_writer":
+            c, st = 16 * int(rng.integers(1, 8)), int(rng.choice([1, 2]))
+            h, w = int(rng.integers(3, 30)), int(rng.integers(4, 30))
+            pad = [1, 1, 1, 1] if st == 1 else [int(rng.integers(0, 2)), 1, int(rng.integers(0, 2)), 1]
+            x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=0, kh=3, kw=3, stride=[st, st], dil=[1, 1], pad=pad, mult=1, mode=mode)
+            want = oracle.conv2d(x, wt, b, act=act, **kws)
+            op = T.conv2d_to_blocked_create(_conv_desc(T, kws, act, keep), wt, b)
+            got = from_blocked(_run(op, x, want.size, kws["out_dtype"]), n, c, kws["out_shape"][0] * kws["out_shape"][1])
+        else:
+            c, dt = 16 * int(rng.integers(1, 40)), int(rng.integers(0, 2))
+            x = rand_q(rng, n * c * hw, dt)
+            in_q = (0.1, 7 if dt == 0 else -3)
+            out_q = in_q if rng.random() < 0.5 else (0.07, 9 if dt == 0 else 2)
+            kws = dict(in_shape=[w, h, c, n], out_shape=[1, 1, c, n], ksize=[w, h], stride=[1, 1], pad_left=0, pad_top=0,
+                       pool_type=int(rng.choice([1, 3])), dtype=dt)
+            want = oracle.pool2d(x, in_q=in_q, out_q=out_q, **kws)
+            d = T.Pool2dDesc()
+            d.in_w, d.in_h, d.channels, d.batch = w, h, c, n
+            d.out_w = d.out_h = 1
+            d.k_w, d.k_h, d.stride_w, d.stride_h = w, h, 1, 1
+            d.pool_type, d.dtype = kws["pool_type"], dt
+            d.in_scale, d.in_zp = in_q
+            d.out_scale, d.out_zp = out_q
+            op = T.pool2d_blocked_create(d)
+            got = _run(op, to_blocked(x, n, c, hw), want.size, dt)
+        seen[kind] += 1
+        assert np.array_equal(got, want), (i, kind, mode, n, h, w, int((got != want).sum()), np.flatnonzero(got != want)[:6])
+    assert min(seen.values()) == 18
