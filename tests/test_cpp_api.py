@@ -348,6 +348,36 @@ def test_mobilenet_v2_graph_bit_exact(tmp_path, oracle, batch, res):
     assert sum("pwconv_add_i8" in l or "pwconv_add_blocked_i8" in l for l in plan) == 10 and not any("ADD" in l for l in plan), plan
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("side,batch", [(7, 3), (5, 1), (8, 2)])
+def test_blocked_plan_with_a_copy_in(tmp_path, oracle, side, batch):
+    """A run of small-plane convolutions behind an INPUT tensor: the executor keeps its TRANSIENT tensors channel-blocked;
+    the input - read by the expansion and, as the residual, by the Add - is copied into that order once; the average
+    pooling leaves the plan. Bit for bit the WHCN plan's result."""
+    g = GRAPHS._Builder(side * 10 + batch)
+    x = g.new("UINT8", "INPUT", [side, side, 64, batch], GF.asym(0.05, 128),
+              g.rng.integers(0, 256, size=side * side * 64 * batch, dtype=np.uint8))
+    x["_rms"] = 74.0
+    h = g.conv(x, 192, 1, 1, "RELU6")
+    h = g.conv(h, 192, 3, 1, "RELU6", depthwise=True)
+    h = g.conv(h, 64, 1, 1, None)
+    h = g.add(x, h)
+    h = g.conv(h, 96, 1, 1, "RELU6")
+    out = g.new("UINT8", "OUTPUT", [1, 1, 96, batch], h["quant"])
+    g.ops.append(GF.op("POOL", [h["id"]], [out["id"]], pad_type="VALID", pool_type="AVG", ksize=[side, side], stride=[side, side]))
+    graph = {"test": "blocked_copy_in_%d_%d" % (side, batch), "tensors": g.tensors, "ops": g.ops, "output": out["id"]}
+    want = oracle.run_graph(graph)
+    assert len(np.unique(want)) > 8
+    got, info, log = GF.run_graphs([graph], str(tmp_path / "blocked"), env={"VSI_NN_LOG_LEVEL": "3"})
+    assert got[0] is not None, (info, log[-2000:])
+    assert np.array_equal(got[0], want), int((got[0] != want).sum())
+    plan = [l for l in log.splitlines() if "uid" in l and "->" in l]
+    assert sum("layout_to_blocked" in l for l in plan) == 1 and sum("_blocked_i8" in l for l in plan) == 5, plan
+    assert sum("pwconv_add_blocked_i8" in l for l in plan) == 1 and not any("ADD" in l for l in plan), plan
+    plain, info, log = GF.run_graphs([graph], str(tmp_path / "whcn"), env={"VSI_NN_LOG_LEVEL": "3", "TVX_BLOCKED_LAYOUT": "0"})
+    assert np.array_equal(plain[0], want) and "blocked" not in log
+
+
 def _pool_graph(name, in_shape, out_shape, pool_type, form, ksize, stride, dt="UINT8", in_q=(0.5, 12), out_q=(0.5, 12)):
     rng = np.random.default_rng(len(name))
     lo, hi = (0, 256) if dt == "UINT8" else (-128, 128)
