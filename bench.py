@@ -373,7 +373,7 @@ def time_workload(wl, steps, warmup, ring_bytes=0):
 KERNEL_SOURCES = {"conv2d_igemm_i8": "conv_igemm_i8.hip", "conv2d_igemm_i8_persistent": "conv_igemm_i8.hip", "conv2d_band_i8": "conv_band_i8.hip",
                   "fc_mfma_i8_256x256x128": "fc_mfma_i8.hip", "fc_mfma_i8_128x256x128": "fc_mfma_i8.hip", "fc_mfma_f16_256x256x64": "fc_mfma_i8.hip",
                   "dwconv3x3_i8": "dwconv3x3_i8.hip", "pwconv_i8": "pwconv_i8.hip", "pwconv_i8_stream": "pwconv_i8.hip", "dwconv3x3_pwconv_i8": "dwpw_i8.hip", "pool2d_rows_i8": "pool2d_i8.hip", "pool2d_stencil_i8": "pool2d_stencil_i8.hip",
-                  "conv2d_gemm_i8": "conv_gemm.hip", "conv2d_gemm_f16": "conv_gemm.hip",
+                  "conv2d_gemm_i8": "conv_gemm.hip", "conv2d_gemm_f16": "conv_gemm.hip", "conv2d_igemm_f16": "conv_igemm_f16.hip",
                   "avgpool_plane_i8": "kernels_generic.hip"}
 
 

@@ -829,20 +829,65 @@ def test_conv2d_gemm(oracle, gi, mode):
     assert len(np.unique(want)) > 4
 
 
-def test_conv2d_gemm_f16_matches_float32_arithmetic(oracle):
-    """The float16 kernel accumulates in float32 and rounds once: against a float64 convolution of the same
+@pytest.mark.parametrize("kernel", ["conv2d_gemm_f16", "conv2d_igemm_f16"])
+def test_conv2d_f16_kernels_match_float32_arithmetic(oracle, kernel, monkeypatch):
+    """The float16 kernels accumulate in float32 and round once: against a float64 convolution of the same
     float16 operands the error stays within one float16 rounding of the result (plus the accumulation's)."""
     import torch
     import torch.nn.functional as F
+    if kernel == "conv2d_gemm_f16":
+        monkeypatch.setenv("TVX_NO_CONV_IGEMM_F16", "1")
     rng = np.random.default_rng(7400)
     n, c, oc, h, w = 2, 48, 64, 20, 20
     x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=oc, kh=3, kw=3, stride=[1, 1], dil=[1, 1],
                               pad=[1, 1, 1, 1], mult=0, mode="f16")
-    got = TC.gpu_conv2d(x, wt, b, want_kernel="conv2d_gemm_f16", **kws).astype(np.float64)
+    got = TC.gpu_conv2d(x, wt, b, want_kernel=kernel, **kws).astype(np.float64)
     ref = F.conv2d(torch.from_numpy(x.astype(np.float64).reshape(n, c, h, w)),
                    torch.from_numpy(wt.astype(np.float64).reshape(oc, c, 3, 3)),
                    torch.from_numpy(b.astype(np.float64)), padding=1).numpy().reshape(-1)
     assert np.all(np.abs(got - ref) <= np.abs(ref) * 2.0 ** -10 + 2e-3)
+
+
+IGEMM_F16_GRID = [
+    # (n, c, oc, h, w, kh, kw, stride, pad[l,r,t,b]): the headline shape's layout in small; one and two channel tiles and a
+    # ragged third; 2 / 4 / 8 channel steps; pixel counts that are no multiple of 128 (ragged last tile) or of four
+    # (element stores); tiles that start in the middle of a row; strides 1 and 2; windows 1x1 .. 5x3; uneven pads
+    (2, 64, 64, 14, 14, 3, 3, 1, [1, 1, 1, 1]),
+    (1, 32, 40, 9, 10, 3, 3, 1, [1, 1, 1, 1]),
+    (2, 16, 100, 12, 20, 1, 1, 1, [0, 0, 0, 0]),
+    (1, 128, 32, 7, 6, 3, 3, 1, [1, 1, 1, 1]),
+    (2, 48, 64, 20, 20, 3, 3, 2, [0, 1, 0, 1]),
+    (1, 80, 48, 11, 14, 5, 3, 1, [2, 2, 1, 1]),
+    (3, 32, 33, 13, 16, 3, 3, 1, [0, 2, 2, 0]),
+    (1, 64, 64, 30, 56, 3, 3, 1, [1, 1, 1, 1]),
+    (2, 16, 16, 5, 2, 2, 2, 1, [1, 0, 0, 1]),
+    (1, 96, 70, 16, 12, 3, 3, 3, [1, 1, 1, 1]),
+]
+
+
+@pytest.mark.parametrize("pixel_tiles", [1, 2])
+@pytest.mark.parametrize("gi", range(len(IGEMM_F16_GRID)))
+def test_conv2d_igemm_f16(oracle, gi, pixel_tiles, monkeypatch):
+    """conv2d_igemm_f16 (halo rows transposed into LDS once, implicit GEMM on the matrix cores) against the oracle within
+    the float16 tolerance and, within float32 accumulation noise, against conv2d_gemm_f16 on the same operands."""
+    import os
+    n, c, oc, h, w, kh, kw, stride, pad = IGEMM_F16_GRID[gi]
+    monkeypatch.setenv("TVX_CONV_F16_PIXEL_TILES", str(pixel_tiles))   # 128- and 256-pixel workgroups
+    rng = np.random.default_rng(7600 + gi)
+    x, wt, b, kws = conv_case(rng, n=n, c=c, h=h, w=w, oc=oc, kh=kh, kw=kw, stride=[stride, stride], dil=[1, 1],
+                              pad=pad, mult=0, mode="f16")
+    for act in (0, 2):
+        want = oracle.conv2d(x, wt, b, act=act, **kws)
+        got = TC.gpu_conv2d(x, wt, b, act=act, want_kernel="conv2d_igemm_f16", **kws)
+        assert np.allclose(got.astype(np.float32), want.astype(np.float32), rtol=FLOAT_RTOL, atol=2e-2)
+        os.environ["TVX_NO_CONV_IGEMM_F16"] = "1"
+        try:
+            other = TC.gpu_conv2d(x, wt, b, act=act, want_kernel="conv2d_gemm_f16", **kws)
+        finally:
+            del os.environ["TVX_NO_CONV_IGEMM_F16"]
+        # two float32 accumulation orders of the same products, each rounded once to float16
+        assert np.allclose(got.astype(np.float32), other.astype(np.float32), rtol=2e-3, atol=2e-3)
+    assert len(np.unique(want)) > 4
 
 
 DWP_GRID = [

@@ -69,6 +69,8 @@ int MbConvSetup(tvx_op* op, const MbStage& expand, const MbStage& depthwise, con
                 const void* project_w, const void* project_b);
 
 // convolution as a GEMM over gathered windows: grouped, dilated, float16 (conv_gemm.hip)
+// dense float16 convolution, halo rows staged in LDS once (conv_igemm_f16.hip)
+int ConvIgemmF16Setup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 int ConvGemmSetup(tvx_op*, const tvx_conv2d_desc*, const void*, const void*);
 
 // generic (kernels_generic.hip)

@@ -4,7 +4,7 @@
 namespace tvx {
 
 const std::vector<ConvSetupFn>& ConvVariants() {
-  static const std::vector<ConvSetupFn> v = {DwConv3x3Setup, DwPlanesSetup, PwConvSetup, ConvIm2colSetup, ConvBandSetup, ConvIgemmSetup, ConvGemmSetup, ConvGenericSetup};
+  static const std::vector<ConvSetupFn> v = {DwConv3x3Setup, DwPlanesSetup, PwConvSetup, ConvIm2colSetup, ConvBandSetup, ConvIgemmSetup, ConvIgemmF16Setup, ConvGemmSetup, ConvGenericSetup};
   return v;
 }
 
